@@ -1,0 +1,314 @@
+/*
+ * CPU oracle for the quantized-Linear path.  TEST INFRASTRUCTURE ONLY: it is
+ * the checker the HIP kernels are compared against and the "port" CPU baseline
+ * that the benchmark times; nothing that ships calls into it.
+ *
+ * What it restates.  The reference's Linear layer is a plain float
+ * y = x @ W^T (+ b)  (astrai/model/components/linear.py:20-21, weight laid out
+ * [out_dim, in_dim] at linear.py:10).  The reference holds no quantized
+ * arithmetic, so the int8 / FP8 arithmetic below is the textbook symmetric
+ * absmax scheme, frozen here and implemented a second time in HIP:
+ *
+ *   int8, per row r of an [R, K] matrix, all in IEEE fp32:
+ *     amax_r = max_k |a_rk|;  s_r = amax_r / 127  (s_r = 1 when amax_r == 0)
+ *     q_rk   = clamp(rint(a_rk / s_r), -127, 127)      rint = half-to-even,
+ *                                                      '/' = true fp32 divide
+ *   accumulate: acc[m,n] = sum_k xq[m,k] * wq[n,k]  in int32 (exact)
+ *   epilogue:   y = (float(acc) * sx[m]) * sw[n] (+ bias[n]), each operation a
+ *               separately rounded fp32 op (no FMA), then one RNE cast.
+ *   FP8 (OCP e4m3fn, max 448), per tensor:
+ *     s = amax / 448 (s = 1 when amax == 0);  a8 = e4m3fn_rne(clamp(a/s, +-448))
+ *     acc in fp32, k ascending;  y = (acc * sx) * sw.
+ *
+ * Pinning status (tests/test_oracle_*.py):
+ *   oq_gemm_i8_i32        pinned: exact integer identity vs torch._int_mm and
+ *                         numpy int64 matmul, extreme +-127 cases.
+ *   oq_f32_to_e4m3fn      pinned: element-for-element vs torch's
+ *   oq_e4m3fn_to_f32      float8_e4m3fn cast over every code, every midpoint
+ *                         between codes and a dense random sweep.
+ *   oq_f32_to_bf16        pinned: vs torch's bfloat16 cast incl. ties.
+ *   oq_quant_rowwise_i8   pinned by mathematics: exact-rational brute force on
+ *                         small inputs (python fractions, correctly rounded
+ *                         divide, ties-to-even), constructed tie cases,
+ *                         invariants (max|q| = 127, zero rows, sign symmetry,
+ *                         |a - q s| <= s/2).  No reference vector exists for it:
+ *                         "parity unpinned" with respect to the reference.
+ *   oq_dequant_epilogue   pinned: vs numpy float32 elementwise arithmetic and,
+ *   oq_linear_w8a8        end to end, vs F.linear in fp32 (the reference's real
+ *                         path) within the quantisation-error bound.
+ *   oq_quant_tensor_fp8,  pinned through the cast above plus numpy float32
+ *   oq_linear_fp8         restatement; accumulation order makes the GEMM a
+ *                         tolerance (1e-2) comparison, never bit-exact.
+ *
+ * Build: gcc -O3 -march=native -fopenmp -ffp-contract=off -fno-fast-math
+ *        -shared -fPIC (oracle/build_oracle.py).  OpenMP only parallelises over
+ *        rows; every row's arithmetic is the scalar definition above.
+ */
+#include <math.h>
+#include <stdint.h>
+#include <string.h>
+#include <stdlib.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+int oq_num_threads(void) {
+#ifdef _OPENMP
+  return omp_get_max_threads();
+#else
+  return 1;
+#endif
+}
+
+void oq_set_num_threads(int n) {
+#ifdef _OPENMP
+  if (n > 0) omp_set_num_threads(n);
+#else
+  (void)n;
+#endif
+}
+
+/* ---------------------------------------------------------------- scalars */
+
+static inline float bits_to_f32(uint32_t u) {
+  float f;
+  memcpy(&f, &u, 4);
+  return f;
+}
+static inline uint32_t f32_to_bits(float f) {
+  uint32_t u;
+  memcpy(&u, &f, 4);
+  return u;
+}
+
+float oq_bf16_to_f32(uint16_t h) { return bits_to_f32((uint32_t)h << 16); }
+
+/* fp32 -> bf16, round to nearest even; NaN stays a quiet NaN. */
+uint16_t oq_f32_to_bf16(float f) {
+  uint32_t u = f32_to_bits(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
+  uint32_t lsb = (u >> 16) & 1u;
+  u += 0x7fffu + lsb;
+  return (uint16_t)(u >> 16);
+}
+
+/* OCP e4m3fn: 1 sign, 4 exponent (bias 7), 3 mantissa; no infinities; only
+ * S.1111.111 is NaN; largest finite 448 = 0x7e; subnormal step 2^-9. */
+float oq_e4m3fn_to_f32(uint8_t b) {
+  int sign = b >> 7, e = (b >> 3) & 0xf, m = b & 7;
+  float v;
+  if (e == 0xf && m == 7) return bits_to_f32(0x7fc00000u);
+  if (e == 0)
+    v = ldexpf((float)m, -9);
+  else
+    v = ldexpf((float)(8 + m), e - 10);
+  return sign ? -v : v;
+}
+
+/* fp32 -> e4m3fn, round to nearest even.  Finite inputs beyond the range
+ * saturate to +-448 and NaN gives 0x7f; callers clamp first, so saturation is
+ * never what a test depends on. */
+uint8_t oq_f32_to_e4m3fn(float f) {
+  uint32_t u = f32_to_bits(f);
+  uint8_t sign = (uint8_t)((u >> 24) & 0x80u);
+  uint32_t au = u & 0x7fffffffu;
+  if (au > 0x7f800000u) return (uint8_t)(sign | 0x7f);
+  float a = bits_to_f32(au);
+  if (a >= 464.0f) return (uint8_t)(sign | 0x7e); /* 464 = midpoint past 448 */
+  if (a < 0.015625f) {                            /* below 2^-6: subnormal grid 2^-9 */
+    float r = rintf(a * 512.0f);                  /* exact scaling, RNE */
+    return (uint8_t)(sign | (uint8_t)r);          /* r == 8 lands on 0x08 = 2^-6 */
+  }
+  int e;
+  float fr = frexpf(a, &e); /* a = fr * 2^e, fr in [0.5,1) */
+  /* a = (2 fr) * 2^(e-1); mantissa grid 1/8 on [1,2) */
+  float m = rintf(fr * 16.0f); /* in [8,16] */
+  int E = e - 1;
+  if (m == 16.0f) {
+    m = 8.0f;
+    E += 1;
+  }
+  int be = E + 7;
+  uint8_t code = (uint8_t)((be << 3) | ((int)m - 8));
+  if (code > 0x7e) code = 0x7e;
+  return (uint8_t)(sign | code);
+}
+
+/* ------------------------------------------------ int8 row-wise quantise */
+
+static void quant_row_f32(const float *a, int64_t K, int8_t *q, float *s_out) {
+  float amax = 0.0f;
+  for (int64_t k = 0; k < K; ++k) {
+    float v = fabsf(a[k]);
+    if (v > amax) amax = v;
+  }
+  float s = amax / 127.0f;
+  if (amax == 0.0f) s = 1.0f;
+  for (int64_t k = 0; k < K; ++k) {
+    float r = rintf(a[k] / s);
+    if (r > 127.0f) r = 127.0f;
+    if (r < -127.0f) r = -127.0f;
+    q[k] = (int8_t)r;
+  }
+  *s_out = s;
+}
+
+/* x: [M, K] fp32 with row stride ldx (elements); q: [M, K] contiguous. */
+void oq_quant_rowwise_i8_f32(const float *x, int64_t M, int64_t K, int64_t ldx,
+                             int8_t *q, float *scale) {
+#pragma omp parallel for schedule(static)
+  for (int64_t m = 0; m < M; ++m) quant_row_f32(x + m * ldx, K, q + m * K, scale + m);
+}
+
+/* Same with bf16 input: each element is widened to fp32 first (exact). */
+void oq_quant_rowwise_i8_bf16(const uint16_t *x, int64_t M, int64_t K, int64_t ldx,
+                              int8_t *q, float *scale) {
+#pragma omp parallel for schedule(static)
+  for (int64_t m = 0; m < M; ++m) {
+    float *tmp = (float *)malloc((size_t)K * sizeof(float));
+    for (int64_t k = 0; k < K; ++k) tmp[k] = oq_bf16_to_f32(x[m * ldx + k]);
+    quant_row_f32(tmp, K, q + m * K, scale + m);
+    free(tmp);
+  }
+}
+
+/* ------------------------------------------------------------- int8 GEMM */
+
+/* acc[m,n] = sum_k xq[m,k] * wq[n,k]; both operands K-contiguous, the layout
+ * of Linear.weight (linear.py:10). */
+void oq_gemm_i8_i32(const int8_t *xq, const int8_t *wq, int32_t *acc, int64_t M,
+                    int64_t N, int64_t K) {
+#pragma omp parallel for schedule(static)
+  for (int64_t m = 0; m < M; ++m) {
+    const int8_t *xr = xq + m * K;
+    for (int64_t n = 0; n < N; ++n) {
+      const int8_t *wr = wq + n * K;
+      int32_t s = 0;
+      for (int64_t k = 0; k < K; ++k) s += (int32_t)xr[k] * (int32_t)wr[k];
+      acc[m * N + n] = s;
+    }
+  }
+}
+
+/* y = (float(acc) * sx[m]) * sw[n] (+ bias[n]) in fp32, three separately
+ * rounded operations.  y_bf16 may be NULL; y_f32 may be NULL. */
+void oq_dequant_epilogue(const int32_t *acc, const float *sx, const float *sw,
+                         const float *bias, float *y_f32, uint16_t *y_bf16,
+                         int64_t M, int64_t N) {
+#pragma omp parallel for schedule(static)
+  for (int64_t m = 0; m < M; ++m) {
+    for (int64_t n = 0; n < N; ++n) {
+      volatile float t = (float)acc[m * N + n] * sx[m];
+      volatile float u = t * sw[n];
+      float y = u;
+      if (bias) {
+        volatile float w = u + bias[n];
+        y = w;
+      }
+      if (y_f32) y_f32[m * N + n] = y;
+      if (y_bf16) y_bf16[m * N + n] = oq_f32_to_bf16(y);
+    }
+  }
+}
+
+/* Whole W8A8 Linear from float inputs: quantise x per token, GEMM, epilogue.
+ * wq/sw are the already-quantised weight.  Scratch is allocated here. */
+void oq_linear_w8a8_f32(const float *x, const int8_t *wq, const float *sw,
+                        const float *bias, float *y_f32, uint16_t *y_bf16, int64_t M,
+                        int64_t N, int64_t K) {
+  int8_t *xq = (int8_t *)malloc((size_t)(M * K));
+  float *sx = (float *)malloc((size_t)M * sizeof(float));
+  int32_t *acc = (int32_t *)malloc((size_t)(M * N) * sizeof(int32_t));
+  oq_quant_rowwise_i8_f32(x, M, K, K, xq, sx);
+  oq_gemm_i8_i32(xq, wq, acc, M, N, K);
+  oq_dequant_epilogue(acc, sx, sw, bias, y_f32, y_bf16, M, N);
+  free(xq);
+  free(sx);
+  free(acc);
+}
+
+void oq_linear_w8a8_bf16(const uint16_t *x, const int8_t *wq, const float *sw,
+                         const float *bias, float *y_f32, uint16_t *y_bf16, int64_t M,
+                         int64_t N, int64_t K) {
+  int8_t *xq = (int8_t *)malloc((size_t)(M * K));
+  float *sx = (float *)malloc((size_t)M * sizeof(float));
+  int32_t *acc = (int32_t *)malloc((size_t)(M * N) * sizeof(int32_t));
+  oq_quant_rowwise_i8_bf16(x, M, K, K, xq, sx);
+  oq_gemm_i8_i32(xq, wq, acc, M, N, K);
+  oq_dequant_epilogue(acc, sx, sw, bias, y_f32, y_bf16, M, N);
+  free(xq);
+  free(sx);
+  free(acc);
+}
+
+/* -------------------------------------------------------------------- FP8 */
+
+static float amax_f32(const float *x, int64_t n) {
+  float amax = 0.0f;
+  for (int64_t i = 0; i < n; ++i) {
+    float v = fabsf(x[i]);
+    if (v > amax) amax = v;
+  }
+  return amax;
+}
+
+static void cast_fp8(const float *x, int64_t n, float s, uint8_t *q) {
+#pragma omp parallel for schedule(static)
+  for (int64_t i = 0; i < n; ++i) {
+    float v = x[i] / s;
+    if (v > 448.0f) v = 448.0f;
+    if (v < -448.0f) v = -448.0f;
+    q[i] = oq_f32_to_e4m3fn(v);
+  }
+}
+
+void oq_quant_tensor_fp8_f32(const float *x, int64_t numel, uint8_t *q, float *scale) {
+  float amax = amax_f32(x, numel);
+  float s = amax / 448.0f;
+  if (amax == 0.0f) s = 1.0f;
+  cast_fp8(x, numel, s, q);
+  *scale = s;
+}
+
+void oq_quant_tensor_fp8_bf16(const uint16_t *x, int64_t numel, uint8_t *q, float *scale) {
+  float *tmp = (float *)malloc((size_t)numel * sizeof(float));
+  for (int64_t i = 0; i < numel; ++i) tmp[i] = oq_bf16_to_f32(x[i]);
+  oq_quant_tensor_fp8_f32(tmp, numel, q, scale);
+  free(tmp);
+}
+
+/* y = (sum_k f(xq[m,k]) f(wq[n,k])) * sx * sw; fp32 accumulate, k ascending. */
+void oq_linear_fp8(const uint8_t *xq, float sx, const uint8_t *wq, float sw, float *y_f32,
+                   uint16_t *y_bf16, int64_t M, int64_t N, int64_t K) {
+  float lut[256];
+  for (int i = 0; i < 256; ++i) lut[i] = oq_e4m3fn_to_f32((uint8_t)i);
+#pragma omp parallel for schedule(static)
+  for (int64_t m = 0; m < M; ++m) {
+    float *xr = (float *)malloc((size_t)K * sizeof(float));
+    for (int64_t k = 0; k < K; ++k) xr[k] = lut[xq[m * K + k]];
+    for (int64_t n = 0; n < N; ++n) {
+      const uint8_t *wr = wq + n * K;
+      float s = 0.0f;
+      for (int64_t k = 0; k < K; ++k) s += xr[k] * lut[wr[k]];
+      volatile float t = s * sx;
+      volatile float u = t * sw;
+      float y = u;
+      if (y_f32) y_f32[m * N + n] = y;
+      if (y_bf16) y_bf16[m * N + n] = oq_f32_to_bf16(y);
+    }
+    free(xr);
+  }
+}
+
+/* Float reference of the Linear itself (linear.py:20-21): fp32, k ascending. */
+void oq_linear_f32(const float *x, const float *w, const float *bias, float *y, int64_t M,
+                   int64_t N, int64_t K) {
+#pragma omp parallel for schedule(static)
+  for (int64_t m = 0; m < M; ++m)
+    for (int64_t n = 0; n < N; ++n) {
+      double s = 0.0;
+      for (int64_t k = 0; k < K; ++k) s += (double)x[m * K + k] * (double)w[n * K + k];
+      if (bias) s += bias[n];
+      y[m * N + n] = (float)s;
+    }
+}

@@ -1,0 +1,109 @@
+/*
+ * astrai_q -- C ABI of the MI355X (gfx950) quantized-Linear path.
+ *
+ * The reference's Linear layer has no FFI: it is one Python call,
+ *   y = F.linear(x, weight, bias)      astrai/model/components/linear.py:20-21
+ * with weight laid out [out_dim, in_dim] (linear.py:10) and an optional bias
+ * [out_dim] (linear.py:11).  Every entry point below is a stage of the
+ * quantized replacement of that one call; each comment names the part of the
+ * reference call it stands in for.
+ *
+ * Conventions
+ *  - Every pointer is a DEVICE pointer owned by the caller.  The library never
+ *    allocates, frees or synchronises; work is queued on `stream` (a
+ *    hipStream_t passed as void*, NULL = the null stream).
+ *  - Matrices are row-major and contiguous unless a leading dimension is given.
+ *    K (the reduction length, Linear's in_dim) must be a multiple of 16 and
+ *    every matrix base 16-byte aligned.
+ *  - dtype codes: AQ_F32 = 0, AQ_BF16 = 1.
+ *  - Return value: 0 on success, a negative AQ_E_* for a rejected argument, or
+ *    a positive hipError_t from the launch.  aq_error_string() names either.
+ *  - Re-entrant: no global mutable state.  (The reference calls Linear from its
+ *    scheduler's daemon thread, astrai/inference/core/scheduler.py:191-196.)
+ */
+#ifndef ASTRAI_Q_H
+#define ASTRAI_Q_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define AQ_VERSION 100
+
+enum { AQ_F32 = 0, AQ_BF16 = 1 };
+
+enum {
+  AQ_OK = 0,
+  AQ_E_NULL = -1,      /* a required pointer is NULL                */
+  AQ_E_SHAPE = -2,     /* negative size, K not a multiple of 16 ... */
+  AQ_E_DTYPE = -3,     /* unknown dtype code                        */
+  AQ_E_ALIGN = -4,     /* pointer or leading dimension not 16-byte aligned */
+  AQ_E_WORKSPACE = -5, /* workspace too small                       */
+  AQ_E_RANGE = -6      /* size beyond what the kernels index        */
+};
+
+int aq_version(void);
+const char *aq_error_string(int code);
+
+/* Symmetric absmax int8 per row: scale[r] = amax_r / 127 (1 when the row is all
+ * zero), q = clamp(rint(x / scale), -127, 127), round-half-even, true divide.
+ * Used per token on the activation x of Linear.forward (linear.py:20) and, once
+ * and offline, per output channel on Linear.weight (linear.py:10).
+ * x: [M, K] of x_dtype with row stride ldx elements; q: [M, K]; scale: [M]. */
+int aq_quant_rowwise_i8(const void *x, int x_dtype, int64_t M, int64_t K, int64_t ldx,
+                        int8_t *q, float *scale, void *stream);
+
+/* Per-tensor FP8 (OCP e4m3fn): scale[0] = amax / 448 (1 when all zero),
+ * q = e4m3fn_rne(clamp(x / scale, -448, 448)).  Stands in for the operands of
+ * the same F.linear call (linear.py:21) in the FP8 variant.
+ * amax_ws: 4 bytes of device scratch the call overwrites. */
+int aq_quant_tensor_fp8(const void *x, int x_dtype, int64_t numel, uint8_t *q, float *scale,
+                        uint32_t *amax_ws, void *stream);
+
+/* acc[m, n] = sum_k xq[m, k] * wq[n, k], exact int32: the matrix product inside
+ * F.linear (linear.py:21) on int8 codes.  xq: [M, K], wq: [N, K], acc: [M, N]. */
+int aq_gemm_i8_i32(const int8_t *xq, const int8_t *wq, int32_t *acc, int64_t M, int64_t N,
+                   int64_t K, void *stream);
+
+/* The same product with the dequantising epilogue fused:
+ * y[m, n] = (float(acc) * sx[m]) * sw[n] (+ bias[n]), each step rounded to
+ * fp32, then one round-to-nearest-even cast to y_dtype.  Replaces the whole
+ * F.linear(x, weight, bias) of linear.py:21 for M > 16.
+ * bias may be NULL (the reference never constructs a Linear with bias=True). */
+int aq_linear_w8a8(const int8_t *xq, const float *sx, const int8_t *wq, const float *sw,
+                   const void *bias, int bias_dtype, void *y, int y_dtype, int64_t M,
+                   int64_t N, int64_t K, void *stream);
+
+/* Decode path, M <= 16 rows of x: quantises x per token on the fly, streams wq
+ * once and writes y in y_dtype; same arithmetic and results as
+ * aq_quant_rowwise_i8 followed by aq_linear_w8a8.  Replaces F.linear
+ * (linear.py:21) when the caller is the decode step (M = batch <= 16,
+ * astrai/inference/core/executor.py:59-94).
+ * ws: device scratch of at least aq_gemv_w8a8_workspace_bytes(M, K). */
+size_t aq_gemv_w8a8_workspace_bytes(int64_t M, int64_t K);
+int aq_gemv_w8a8_decode(const void *x, int x_dtype, const int8_t *wq, const float *sw,
+                        const void *bias, int bias_dtype, void *y, int y_dtype, int64_t M,
+                        int64_t N, int64_t K, void *ws, size_t ws_bytes, void *stream);
+
+/* The GEMV of the decode path on codes the caller already holds (for callers
+ * that quantise one activation once and feed several projections with it, as
+ * q/k/v_proj and up/gate share their input: astrai/model/components/
+ * attention.py:83-85, mlp.py:25).  xq: [M <= 16, K], sx: [M]. */
+int aq_gemv_w8a8_codes(const int8_t *xq, const float *sx, const int8_t *wq, const float *sw,
+                       const void *bias, int bias_dtype, void *y, int y_dtype, int64_t M,
+                       int64_t N, int64_t K, void *stream);
+
+/* FP8 Linear: y[m, n] = (sum_k f(xq[m,k]) * f(wq[n,k])) * sx[0] * sw[0] with
+ * fp32 accumulation, cast to y_dtype.  xq: [M, K], wq: [N, K] e4m3fn codes;
+ * sx, sw: device scalars written by aq_quant_tensor_fp8.  Replaces F.linear
+ * (linear.py:21) in the FP8 variant. */
+int aq_linear_fp8(const uint8_t *xq, const float *sx, const uint8_t *wq, const float *sw,
+                  void *y, int y_dtype, int64_t M, int64_t N, int64_t K, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ASTRAI_Q_H */

@@ -1,0 +1,58 @@
+"""ctypes binding of libastrai_q.so (the C ABI in include/astrai_q.h).
+
+The library is built in-tree by khaosz_amd/build.py.  There is no CPU
+fallback: if the shared object is missing, loading raises.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libastrai_q.so")
+
+AQ_F32, AQ_BF16 = 0, 1
+
+# every symbol include/astrai_q.h declares: name -> (restype, argtypes)
+_i64, _vp, _int, _sz = ctypes.c_int64, ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
+SYMBOLS = {
+    "aq_version": (_int, []),
+    "aq_error_string": (ctypes.c_char_p, [_int]),
+    "aq_quant_rowwise_i8": (_int, [_vp, _int, _i64, _i64, _i64, _vp, _vp, _vp]),
+    "aq_quant_tensor_fp8": (_int, [_vp, _int, _i64, _vp, _vp, _vp, _vp]),
+    "aq_gemm_i8_i32": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
+    "aq_linear_w8a8": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _vp, _int, _i64, _i64, _i64, _vp]),
+    "aq_gemv_w8a8_workspace_bytes": (_sz, [_i64, _i64]),
+    "aq_gemv_w8a8_decode": (_int, [_vp, _int, _vp, _vp, _vp, _int, _vp, _int, _i64, _i64, _i64, _vp, _sz, _vp]),
+    "aq_gemv_w8a8_codes": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _vp, _int, _i64, _i64, _i64, _vp]),
+    "aq_linear_fp8": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _vp]),
+}
+
+_lib = None
+
+
+def load() -> ctypes.CDLL:
+    """Load the HIP library; raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: build it with `python -m khaosz_amd.build` "
+            "(hipcc, --offload-arch=gfx950). There is no fallback path."
+        )
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in SYMBOLS.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def check(code: int, what: str) -> None:
+    """Reference convention: errors surface as Python exceptions
+    (e.g. astrai/parallel/module.py:34-37), never as return codes."""
+    if code != 0:
+        msg = load().aq_error_string(code).decode()
+        if code in (-2, -3, -4, -6):
+            raise ValueError(f"{what}: {msg} (code {code})")
+        raise RuntimeError(f"{what}: {msg} (code {code})")

@@ -1,0 +1,258 @@
+"""Host-side mirror of the reference's Linear module and its quantized drop-ins.
+
+``Linear`` keeps the reference's surface (astrai/model/components/linear.py:7-21):
+``Linear(in_dim, out_dim, bias=False)``, a ``weight [out_dim, in_dim]`` parameter,
+``bias [out_dim]`` or ``None``, ``forward(x[..., in_dim]) -> [..., out_dim]``.
+
+``QuantLinear`` and ``Fp8Linear`` subclass it, so ``isinstance(m, Linear)`` -- the
+test the reference uses to discover layers (astrai/model/components/lora.py:64,87)
+-- still holds, and they are swapped in with ``setattr(parent, child, new)`` the
+way ``inject_lora`` does (lora.py:74-106).  Their forward runs entirely in the HIP
+library; there is no CPU or eager fallback.
+"""
+from __future__ import annotations
+
+import logging
+import math
+from typing import Iterable, Optional, Set
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+from torch import Tensor
+
+from . import ops
+
+logger = logging.getLogger(__name__)
+
+
+class Linear(nn.Module):
+    """Float Linear with the reference's constructor, attributes and forward."""
+
+    def __init__(self, in_dim: int, out_dim: int, bias: bool = False):
+        super().__init__()
+        self.weight = nn.Parameter(torch.empty((out_dim, in_dim)))
+        self.bias = nn.Parameter(torch.zeros(out_dim)) if bias else None
+
+    @property
+    def in_dim(self) -> int:
+        return self.weight.shape[1]
+
+    @property
+    def out_dim(self) -> int:
+        return self.weight.shape[0]
+
+    def reset_parameters(self) -> None:
+        # same distributions as linear.py:13-18: U(-1/sqrt(in), 1/sqrt(in)) for both
+        bound = 1.0 / math.sqrt(self.weight.shape[1])
+        nn.init.kaiming_uniform_(self.weight, a=math.sqrt(5))
+        if self.bias is not None:
+            nn.init.uniform_(self.bias, -bound, bound)
+
+    def forward(self, x: Tensor) -> Tensor:
+        return F.linear(x, self.weight, self.bias)
+
+
+def _no_grad_guard(x: Tensor) -> None:
+    if torch.is_grad_enabled() and x.requires_grad:
+        raise RuntimeError("the quantized Linear is forward-only; call it under torch.no_grad()/inference_mode()")
+
+
+class QuantLinear(Linear):
+    """W8A8 Linear: per-channel int8 weight, per-token int8 activation.
+
+    Buffers: ``qweight int8 [out, in]``, ``w_scale float32 [out]``; ``bias`` stays a
+    parameter (or None).  ``weight`` reads back the dequantized float weight for
+    callers that inspect it (lora.py:34-38, transformer.py:95-96).  A float
+    ``<prefix>weight`` entry in a state dict is quantized on load, so float
+    checkpoints with the reference's key names (tests/module/test_lora.py:201-208)
+    still load.
+    """
+
+    DECODE_MAX_ROWS = 16
+
+    def __init__(self, in_dim: int, out_dim: int, bias: bool = False, device=None):
+        nn.Module.__init__(self)
+        self.register_buffer("qweight", torch.zeros((out_dim, in_dim), dtype=torch.int8, device=device))
+        self.register_buffer("w_scale", torch.ones((out_dim,), dtype=torch.float32, device=device))
+        self.bias = nn.Parameter(torch.zeros(out_dim, device=device), requires_grad=False) if bias else None
+        self._workspace: Optional[Tensor] = None
+
+    # -- construction -----------------------------------------------------
+    @classmethod
+    def from_linear(cls, base: nn.Module) -> "QuantLinear":
+        """Quantize ``base.weight`` per output channel on the GPU it lives on."""
+        w = base.weight.detach()
+        if not w.is_cuda:
+            raise RuntimeError("QuantLinear.from_linear needs the weight on the GPU (the quantizer is a HIP kernel)")
+        out_dim, in_dim = w.shape
+        q = cls(in_dim, out_dim, bias=base.bias is not None, device=w.device)
+        q.load_float_weight(w)
+        if base.bias is not None:
+            q.bias = nn.Parameter(base.bias.detach().clone(), requires_grad=False)
+        return q
+
+    def load_float_weight(self, w: Tensor) -> None:
+        if tuple(w.shape) != tuple(self.qweight.shape):
+            raise ValueError(f"weight shape {tuple(w.shape)} does not match {tuple(self.qweight.shape)}")
+        if w.dtype not in (torch.float32, torch.bfloat16):
+            w = w.float()
+        codes, scale = ops.quant_rowwise_i8(w.to(self.qweight.device))
+        self.qweight.copy_(codes)
+        self.w_scale.copy_(scale)
+
+    # -- the reference's attribute surface ----------------------------------
+    @property
+    def weight(self) -> Tensor:
+        return self.qweight.float() * self.w_scale[:, None]
+
+    @property
+    def in_dim(self) -> int:
+        return self.qweight.shape[1]
+
+    @property
+    def out_dim(self) -> int:
+        return self.qweight.shape[0]
+
+    def reset_parameters(self) -> None:
+        raise RuntimeError("QuantLinear holds quantized weights; initialise a float Linear and convert it")
+
+    def _load_from_state_dict(self, state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys,
+                              error_msgs):
+        key = prefix + "weight"
+        if key in state_dict and (prefix + "qweight") not in state_dict:
+            w = state_dict.pop(key)
+            try:
+                self.load_float_weight(w)
+            except (ValueError, RuntimeError) as e:
+                error_msgs.append(f"{key}: {e}")
+            state_dict[prefix + "qweight"] = self.qweight
+            state_dict[prefix + "w_scale"] = self.w_scale
+        super()._load_from_state_dict(state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys,
+                                      error_msgs)
+
+    # -- forward ----------------------------------------------------------------
+    def forward(self, x: Tensor) -> Tensor:
+        _no_grad_guard(x)
+        lead = x.shape[:-1]
+        x2 = x.reshape(-1, x.shape[-1])
+        M = x2.shape[0]
+        if x2.shape[1] != self.qweight.shape[1]:
+            raise ValueError(f"expected last dim {self.qweight.shape[1]}, got {x2.shape[1]}")
+        if x2.dtype not in (torch.float32, torch.bfloat16):
+            raise ValueError(f"activation dtype {x2.dtype} is not supported (float32 or bfloat16)")
+        if M <= self.DECODE_MAX_ROWS:
+            need = 16 * self.qweight.shape[1] + 512
+            ws = self._workspace
+            if ws is None or ws.device != x.device or ws.numel() < need:
+                ws = self._workspace = torch.empty((need,), dtype=torch.uint8, device=x.device)
+            y = ops.gemv_w8a8_decode(x2, self.qweight, self.w_scale, self.bias, out_dtype=x.dtype, workspace=ws)
+        else:
+            xq, sx = ops.quant_rowwise_i8(x2)
+            y = ops.linear_w8a8(xq, sx, self.qweight, self.w_scale, self.bias, out_dtype=x.dtype)
+        return y.reshape(*lead, self.qweight.shape[0])
+
+    def extra_repr(self) -> str:
+        return f"in_dim={self.in_dim}, out_dim={self.out_dim}, bias={self.bias is not None}, w8a8"
+
+
+class Fp8Linear(Linear):
+    """FP8 (OCP e4m3fn) Linear with per-tensor scales and fp32 accumulation."""
+
+    def __init__(self, in_dim: int, out_dim: int, bias: bool = False, device=None):
+        if bias:
+            raise ValueError("the FP8 path has no bias epilogue (the reference never builds a Linear with bias)")
+        nn.Module.__init__(self)
+        self.register_buffer("qweight", torch.zeros((out_dim, in_dim), dtype=torch.uint8, device=device))
+        self.register_buffer("w_scale", torch.ones((1,), dtype=torch.float32, device=device))
+        self.bias = None
+
+    @classmethod
+    def from_linear(cls, base: nn.Module) -> "Fp8Linear":
+        w = base.weight.detach()
+        if not w.is_cuda:
+            raise RuntimeError("Fp8Linear.from_linear needs the weight on the GPU (the quantizer is a HIP kernel)")
+        if base.bias is not None:
+            raise ValueError("the FP8 path has no bias epilogue")
+        q = cls(w.shape[1], w.shape[0], device=w.device)
+        if w.dtype not in (torch.float32, torch.bfloat16):
+            w = w.float()
+        codes, scale = ops.quant_tensor_fp8(w)
+        q.qweight.copy_(codes)
+        q.w_scale.copy_(scale)
+        return q
+
+    @property
+    def weight(self) -> Tensor:
+        return self.qweight.view(torch.float8_e4m3fn).float() * self.w_scale
+
+    @property
+    def in_dim(self) -> int:
+        return self.qweight.shape[1]
+
+    @property
+    def out_dim(self) -> int:
+        return self.qweight.shape[0]
+
+    def reset_parameters(self) -> None:
+        raise RuntimeError("Fp8Linear holds quantized weights; initialise a float Linear and convert it")
+
+    def forward(self, x: Tensor) -> Tensor:
+        _no_grad_guard(x)
+        lead = x.shape[:-1]
+        x2 = x.reshape(-1, x.shape[-1])
+        if x2.shape[1] != self.qweight.shape[1]:
+            raise ValueError(f"expected last dim {self.qweight.shape[1]}, got {x2.shape[1]}")
+        xq, sx = ops.quant_tensor_fp8(x2)
+        y = ops.linear_fp8(xq, sx, self.qweight, self.w_scale, out_dtype=x.dtype)
+        return y.reshape(*lead, self.qweight.shape[0])
+
+
+TARGET_MODULES_ATTN = {"q_proj", "k_proj", "v_proj", "o_proj"}
+TARGET_MODULES_FFN = {"up", "gate", "down"}
+
+
+def _is_float_linear(m: nn.Module, extra: Iterable[type]) -> bool:
+    if isinstance(m, (QuantLinear, Fp8Linear)):
+        return False
+    if isinstance(m, Linear) or isinstance(m, tuple(extra)):
+        return True
+    # the reference's own class, matched by identity of name and module so that
+    # this package never has to import it
+    t = type(m)
+    return t.__name__ == "Linear" and t.__module__ == "astrai.model.components.linear"
+
+
+def quantize_model(model: nn.Module, target_modules: Optional[Set[str]] = None, mode: str = "int8",
+                   linear_types: Iterable[type] = ()) -> int:
+    """Replace float Linear children by quantized ones, in place.
+
+    Walks ``named_modules`` and swaps by ``setattr`` exactly as ``inject_lora``
+    does (lora.py:85-94).  ``target_modules`` is a set of child names (default:
+    the attention and MLP projections); ``lm_head`` is never in the default set
+    because it may alias the embedding (astrai/model/transformer.py:95-96).
+    Returns the number of layers replaced.
+    """
+    if mode not in ("int8", "fp8"):
+        raise ValueError(f"mode must be 'int8' or 'fp8', got {mode!r}")
+    if target_modules is None:
+        target_modules = TARGET_MODULES_ATTN | TARGET_MODULES_FFN
+    cls = QuantLinear if mode == "int8" else Fp8Linear
+    replaced = 0
+    seen = []
+    for name, module in list(model.named_modules()):
+        if not _is_float_linear(module, linear_types):
+            continue
+        parent_name, _, child_name = name.rpartition(".")
+        seen.append(child_name)
+        if child_name not in target_modules:
+            continue
+        parent = model.get_submodule(parent_name) if parent_name else model
+        setattr(parent, child_name, cls.from_linear(module))
+        replaced += 1
+    if replaced == 0:
+        logger.warning("No Linear layers quantized. Available Linear child names: %s; target_modules: %s",
+                       sorted(set(seen)), sorted(target_modules))
+    else:
+        logger.info("Quantized %d Linear layers (%s)", replaced, mode)
+    return replaced

@@ -1,0 +1,230 @@
+"""Tensor-level operators over the C ABI.
+
+Each function takes torch tensors that already live on the GPU, checks layout
+the way the kernels assume it, and queues the work on torch's current HIP
+stream.  torch is used for device memory and streams only; all arithmetic is in
+libastrai_q.so.  Together these replace the single call
+``F.linear(x, weight, bias)`` of astrai/model/components/linear.py:21.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from . import _abi
+
+_DT = {torch.float32: _abi.AQ_F32, torch.bfloat16: _abi.AQ_BF16}
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _need_gpu(*ts: Optional[torch.Tensor]) -> None:
+    dev = None
+    for t in ts:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise RuntimeError("astrai_q operators run on the GPU only; got a CPU tensor (no CPU fallback exists)")
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise ValueError("all tensors must be on the same device")
+
+
+def _dt(t: torch.Tensor, what: str) -> int:
+    try:
+        return _DT[t.dtype]
+    except KeyError:
+        raise ValueError(f"{what}: dtype {t.dtype} is not supported (float32 or bfloat16)") from None
+
+
+def _rows(x: torch.Tensor, what: str) -> torch.Tensor:
+    """View [..., K] as a contiguous [M, K]."""
+    if x.dim() < 1:
+        raise ValueError(f"{what}: needs at least one dimension")
+    x2 = x.reshape(-1, x.shape[-1])
+    if not x2.is_contiguous():
+        x2 = x2.contiguous()
+    return x2
+
+
+def _check_k(K: int) -> None:
+    if K <= 0 or K % 16:
+        raise ValueError(f"in_dim (K) must be a positive multiple of 16, got {K}")
+
+
+def quant_rowwise_i8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Symmetric absmax int8 per row of ``x [..., K]`` -> (codes int8 [M, K], scale f32 [M])."""
+    _need_gpu(x)
+    x2 = _rows(x, "quant_rowwise_i8")
+    M, K = x2.shape
+    _check_k(K)
+    q = torch.empty((M, K), dtype=torch.int8, device=x.device)
+    s = torch.empty((M,), dtype=torch.float32, device=x.device)
+    if M:
+        with torch.cuda.device(x.device):
+            rc = _abi.load().aq_quant_rowwise_i8(x2.data_ptr(), _dt(x2, "x"), M, K, x2.stride(0), q.data_ptr(),
+                                                 s.data_ptr(), _stream(x))
+        _abi.check(rc, "aq_quant_rowwise_i8")
+    return q, s
+
+
+def quant_tensor_fp8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Per-tensor OCP e4m3fn -> (codes uint8 with x's shape, scale f32 [1])."""
+    _need_gpu(x)
+    xc = x.contiguous()
+    n = xc.numel()
+    if n % 16:
+        raise ValueError(f"numel must be a multiple of 16, got {n}")
+    q = torch.empty(xc.shape, dtype=torch.uint8, device=x.device)
+    s = torch.empty((1,), dtype=torch.float32, device=x.device)
+    ws = torch.empty((1,), dtype=torch.int32, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = _abi.load().aq_quant_tensor_fp8(xc.data_ptr(), _dt(xc, "x"), n, q.data_ptr(), s.data_ptr(),
+                                             ws.data_ptr(), _stream(x))
+    _abi.check(rc, "aq_quant_tensor_fp8")
+    return q, s
+
+
+def gemm_i8_i32(xq: torch.Tensor, wq: torch.Tensor) -> torch.Tensor:
+    """acc[m, n] = sum_k xq[m, k] * wq[n, k] in exact int32."""
+    _need_gpu(xq, wq)
+    if xq.dtype != torch.int8 or wq.dtype != torch.int8:
+        raise ValueError("gemm_i8_i32 takes int8 codes")
+    if xq.dim() != 2 or wq.dim() != 2 or xq.shape[1] != wq.shape[1]:
+        raise ValueError(f"shape mismatch: xq {tuple(xq.shape)} vs wq {tuple(wq.shape)}")
+    xq, wq = xq.contiguous(), wq.contiguous()
+    M, K = xq.shape
+    N = wq.shape[0]
+    _check_k(K)
+    acc = torch.empty((M, N), dtype=torch.int32, device=xq.device)
+    if M and N:
+        with torch.cuda.device(xq.device):
+            rc = _abi.load().aq_gemm_i8_i32(xq.data_ptr(), wq.data_ptr(), acc.data_ptr(), M, N, K, _stream(xq))
+        _abi.check(rc, "aq_gemm_i8_i32")
+    return acc
+
+
+def _bias_args(bias: Optional[torch.Tensor], N: int):
+    if bias is None:
+        return None, 0
+    if bias.dim() != 1 or bias.shape[0] != N:
+        raise ValueError(f"bias must have shape [{N}], got {tuple(bias.shape)}")
+    b = bias.contiguous()
+    return b, _dt(b, "bias")
+
+
+def linear_w8a8(xq, sx, wq, sw, bias=None, out_dtype=torch.bfloat16) -> torch.Tensor:
+    """MFMA GEMM with the fused epilogue y = (acc * sx[m]) * sw[n] (+ bias[n])."""
+    _need_gpu(xq, sx, wq, sw, bias)
+    if xq.dtype != torch.int8 or wq.dtype != torch.int8:
+        raise ValueError("linear_w8a8 takes int8 codes")
+    if xq.dim() != 2 or wq.dim() != 2 or xq.shape[1] != wq.shape[1]:
+        raise ValueError(f"shape mismatch: xq {tuple(xq.shape)} vs wq {tuple(wq.shape)}")
+    M, K = xq.shape
+    N = wq.shape[0]
+    _check_k(K)
+    if sx.dtype != torch.float32 or sw.dtype != torch.float32 or sx.numel() != M or sw.numel() != N:
+        raise ValueError("sx must be float32 [M] and sw float32 [N]")
+    if out_dtype not in _DT:
+        raise ValueError(f"out_dtype {out_dtype} is not supported")
+    xq, wq, sx, sw = xq.contiguous(), wq.contiguous(), sx.contiguous(), sw.contiguous()
+    b, bdt = _bias_args(bias, N)
+    y = torch.empty((M, N), dtype=out_dtype, device=xq.device)
+    if M and N:
+        with torch.cuda.device(xq.device):
+            rc = _abi.load().aq_linear_w8a8(xq.data_ptr(), sx.data_ptr(), wq.data_ptr(), sw.data_ptr(),
+                                            b.data_ptr() if b is not None else None, bdt, y.data_ptr(),
+                                            _DT[out_dtype], M, N, K, _stream(xq))
+        _abi.check(rc, "aq_linear_w8a8")
+    return y
+
+
+def gemv_w8a8_decode(x, wq, sw, bias=None, out_dtype=None, workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Decode path for at most 16 rows of ``x [M, K]``: fused per-token quantise + int8 GEMV + epilogue."""
+    _need_gpu(x, wq, sw, bias, workspace)
+    x2 = _rows(x, "gemv_w8a8_decode")
+    M, K = x2.shape
+    N = wq.shape[0]
+    if M > 16:
+        raise ValueError(f"the decode path takes at most 16 rows, got {M}")
+    if wq.dtype != torch.int8 or wq.dim() != 2 or wq.shape[1] != K:
+        raise ValueError(f"wq must be int8 [N, {K}], got {wq.dtype} {tuple(wq.shape)}")
+    _check_k(K)
+    if sw.dtype != torch.float32 or sw.numel() != N:
+        raise ValueError("sw must be float32 [N]")
+    out_dtype = out_dtype or x.dtype
+    if out_dtype not in _DT:
+        raise ValueError(f"out_dtype {out_dtype} is not supported")
+    wq, sw = wq.contiguous(), sw.contiguous()
+    b, bdt = _bias_args(bias, N)
+    lib = _abi.load()
+    need = lib.aq_gemv_w8a8_workspace_bytes(M, K)
+    if workspace is None:
+        workspace = torch.empty((max(need, 16),), dtype=torch.uint8, device=x.device)
+    elif workspace.numel() * workspace.element_size() < need:
+        raise ValueError(f"workspace holds {workspace.numel() * workspace.element_size()} bytes, {need} needed")
+    y = torch.empty((M, N), dtype=out_dtype, device=x.device)
+    if M and N:
+        with torch.cuda.device(x.device):
+            rc = lib.aq_gemv_w8a8_decode(x2.data_ptr(), _dt(x2, "x"), wq.data_ptr(), sw.data_ptr(),
+                                         b.data_ptr() if b is not None else None, bdt, y.data_ptr(), _DT[out_dtype],
+                                         M, N, K, workspace.data_ptr(), workspace.numel() * workspace.element_size(),
+                                         _stream(x))
+        _abi.check(rc, "aq_gemv_w8a8_decode")
+    return y
+
+
+def gemv_w8a8_codes(xq, sx, wq, sw, bias=None, out_dtype=torch.bfloat16) -> torch.Tensor:
+    """The decode GEMV on activation codes the caller already holds (at most 16 rows)."""
+    _need_gpu(xq, sx, wq, sw, bias)
+    if xq.dtype != torch.int8 or wq.dtype != torch.int8:
+        raise ValueError("gemv_w8a8_codes takes int8 codes")
+    if xq.dim() != 2 or wq.dim() != 2 or xq.shape[1] != wq.shape[1]:
+        raise ValueError(f"shape mismatch: xq {tuple(xq.shape)} vs wq {tuple(wq.shape)}")
+    M, K = xq.shape
+    N = wq.shape[0]
+    if M > 16:
+        raise ValueError(f"the decode path takes at most 16 rows, got {M}")
+    _check_k(K)
+    if sx.dtype != torch.float32 or sw.dtype != torch.float32 or sx.numel() != M or sw.numel() != N:
+        raise ValueError("sx must be float32 [M] and sw float32 [N]")
+    if out_dtype not in _DT:
+        raise ValueError(f"out_dtype {out_dtype} is not supported")
+    xq, wq, sx, sw = xq.contiguous(), wq.contiguous(), sx.contiguous(), sw.contiguous()
+    b, bdt = _bias_args(bias, N)
+    y = torch.empty((M, N), dtype=out_dtype, device=xq.device)
+    if M and N:
+        with torch.cuda.device(xq.device):
+            rc = _abi.load().aq_gemv_w8a8_codes(xq.data_ptr(), sx.data_ptr(), wq.data_ptr(), sw.data_ptr(),
+                                                b.data_ptr() if b is not None else None, bdt, y.data_ptr(),
+                                                _DT[out_dtype], M, N, K, _stream(xq))
+        _abi.check(rc, "aq_gemv_w8a8_codes")
+    return y
+
+
+def linear_fp8(xq, sx, wq, sw, out_dtype=torch.bfloat16) -> torch.Tensor:
+    """FP8 e4m3fn GEMM with fp32 accumulation: y = (acc * sx[0]) * sw[0]."""
+    _need_gpu(xq, sx, wq, sw)
+    if xq.dtype != torch.uint8 or wq.dtype != torch.uint8:
+        raise ValueError("linear_fp8 takes e4m3fn codes as uint8")
+    if xq.dim() != 2 or wq.dim() != 2 or xq.shape[1] != wq.shape[1]:
+        raise ValueError(f"shape mismatch: xq {tuple(xq.shape)} vs wq {tuple(wq.shape)}")
+    M, K = xq.shape
+    N = wq.shape[0]
+    _check_k(K)
+    if sx.dtype != torch.float32 or sw.dtype != torch.float32 or sx.numel() != 1 or sw.numel() != 1:
+        raise ValueError("sx and sw must be float32 device scalars")
+    if out_dtype not in _DT:
+        raise ValueError(f"out_dtype {out_dtype} is not supported")
+    xq, wq = xq.contiguous(), wq.contiguous()
+    y = torch.empty((M, N), dtype=out_dtype, device=xq.device)
+    if M and N:
+        with torch.cuda.device(xq.device):
+            rc = _abi.load().aq_linear_fp8(xq.data_ptr(), sx.data_ptr(), wq.data_ptr(), sw.data_ptr(), y.data_ptr(),
+                                           _DT[out_dtype], M, N, K, _stream(xq))
+        _abi.check(rc, "aq_linear_fp8")
+    return y

@@ -1,0 +1,383 @@
+"""GPU parity: the HIP kernels, called through the C ABI (ctypes, via
+khaosz_amd.ops), against the CPU oracle on the same seeded inputs.
+
+Bar: bit-exact for int8 codes, scales, int32 accumulators and (stronger than
+required) the dequantised int8-path outputs; FP8 codes bit-exact, FP8 GEMM
+outputs within rtol 1e-2 (the stated tolerance for bf16/FP8 outputs)."""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+from khaosz_amd import ops  # noqa: E402
+from khaosz_amd.linear import Fp8Linear, Linear, QuantLinear, quantize_model  # noqa: E402
+
+DEV = "cuda:0"
+
+
+def _say(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def bf16_bits(t: torch.Tensor) -> np.ndarray:
+    return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+def to_np(t: torch.Tensor) -> np.ndarray:
+    return t.detach().cpu().numpy()
+
+
+def make_x(M, K, seed, outlier_cols=0, outlier_gain=20.0):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(M, K, generator=g)
+    if outlier_cols:
+        cols = torch.randperm(K, generator=g)[:outlier_cols]
+        x[:, cols] *= outlier_gain
+    return x
+
+
+# ------------------------------------------------------------------ quantise
+
+ROW_SHAPES = [(1, 16), (7, 48), (5, 1040), (64, 2048), (9, 5632), (3, 8192 + 48), (130, 16384)]
+
+
+@pytest.mark.parametrize("M,K", ROW_SHAPES)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_quant_rowwise_bit_exact(oracle, M, K, dtype):
+    _say("quant_rowwise", M, K, dtype)
+    x = make_x(M, K, seed=M * 7 + K, outlier_cols=min(4, K // 8))
+    if M > 4:
+        x[1] = 0                      # all-zero row -> scale 1, codes 0
+        x[2] *= 1e-30                 # scale near the subnormal range
+        x[3] *= 1e30
+        x[4, :] = torch.arange(K) % 7 - 3  # small integers: many exact ratios / ties
+    xd = x.to(DEV, dtype)
+    q, s = ops.quant_rowwise_i8(xd)
+    if dtype == torch.bfloat16:
+        qo, so = oracle.c_quant_rowwise_i8(bf16_bits(xd), bf16_bits=True)
+    else:
+        qo, so = oracle.c_quant_rowwise_i8(to_np(xd))
+    assert np.array_equal(to_np(s).view(np.uint32), so.view(np.uint32))
+    assert np.array_equal(to_np(q), qo)
+
+
+def test_quant_rowwise_ties_and_strided_rows(oracle):
+    # amax 127 -> scale exactly 1: n + 0.5 inputs are exact ties (half-to-even)
+    row = torch.tensor([127.0, 0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 63.5, 64.5, 126.5, -126.5, 0.49999997,
+                        3.5, -3.5, 100.5, 101.5])
+    q, s = ops.quant_rowwise_i8(row[None].to(DEV))
+    assert s.item() == 1.0
+    assert to_np(q)[0].tolist() == [127, 0, 2, 2, 0, -2, -2, 64, 64, 126, -126, 0, 4, -4, 100, 102]
+    # rows taken out of a wider matrix: ldx > K
+    big = make_x(20, 96, seed=3).to(DEV)
+    view = big[:, :64]
+    from khaosz_amd import _abi
+    q2 = torch.empty((20, 64), dtype=torch.int8, device=DEV)
+    s2 = torch.empty((20,), dtype=torch.float32, device=DEV)
+    rc = _abi.load().aq_quant_rowwise_i8(view.data_ptr(), 0, 20, 64, 96, q2.data_ptr(), s2.data_ptr(),
+                                         torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    qo, so = oracle.c_quant_rowwise_i8(to_np(view.contiguous()))
+    assert np.array_equal(to_np(q2), qo) and np.array_equal(to_np(s2), so)
+
+
+def test_quant_rowwise_empty():
+    q, s = ops.quant_rowwise_i8(torch.empty((0, 32), device=DEV))
+    assert q.shape == (0, 32) and s.shape == (0,)
+
+
+# ---------------------------------------------------------------- int8 GEMM
+
+GEMM_SHAPES = [(1, 1, 16), (37, 91, 48), (17, 5, 2048), (256, 128, 128), (257, 129, 144), (300, 200, 2064),
+               (512, 384, 5632), (1000, 520, 1024)]
+
+
+def rand_codes(M, K, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(-127, 128, (M, K), generator=g, dtype=torch.int8)
+
+
+@pytest.mark.parametrize("M,N,K", GEMM_SHAPES)
+def test_gemm_i8_i32_bit_exact(oracle, M, N, K):
+    _say("gemm_i8_i32", M, N, K)
+    xq, wq = rand_codes(M, K, 1), rand_codes(N, K, 2)
+    acc = ops.gemm_i8_i32(xq.to(DEV), wq.to(DEV))
+    want = oracle.c_gemm_i8_i32(xq.numpy(), wq.numpy())
+    assert np.array_equal(to_np(acc), want)
+
+
+def test_gemm_i8_extremes(oracle):
+    K = 8192
+    xq = torch.full((40, K), 127, dtype=torch.int8)
+    wq = torch.full((33, K), -127, dtype=torch.int8)
+    wq[::2] = 127
+    acc = to_np(ops.gemm_i8_i32(xq.to(DEV), wq.to(DEV)))
+    assert np.all(acc[:, ::2] == K * 127 * 127) and np.all(acc[:, 1::2] == -K * 127 * 127)
+
+
+def test_gemm_i8_one_hot_pins_operand_order():
+    # xq has a single 1 at (m, k=m*3 % K); wq[n, k] = n*K + k small codes -> acc[m, n] = wq[n, k_m]
+    M, N, K = 70, 45, 64
+    xq = torch.zeros((M, K), dtype=torch.int8)
+    ks = (torch.arange(M) * 3) % K
+    xq[torch.arange(M), ks] = 1
+    wq = ((torch.arange(N)[:, None] * 5 + torch.arange(K)[None, :] * 3) % 251 - 125).to(torch.int8)
+    acc = to_np(ops.gemm_i8_i32(xq.to(DEV), wq.to(DEV)))
+    want = wq.numpy().astype(np.int32)[:, ks.numpy()].T
+    assert np.array_equal(acc, want)
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("bias_kind", ["none", "f32", "bf16"])
+def test_linear_w8a8_epilogue_bit_exact(oracle, out_dtype, bias_kind):
+    M, N, K = 150, 200, 512
+    _say("linear_w8a8", out_dtype, bias_kind)
+    x = make_x(M, K, 5, outlier_cols=3)
+    w = make_x(N, K, 6) * 0.02
+    xq, sx = oracle.c_quant_rowwise_i8(x.numpy())
+    wq, sw = oracle.c_quant_rowwise_i8(w.numpy())
+    bias = None
+    bias_np = None
+    if bias_kind != "none":
+        b = torch.randn(N, generator=torch.Generator().manual_seed(7)) * 0.01
+        bias = b.to(DEV, torch.float32 if bias_kind == "f32" else torch.bfloat16)
+        bias_np = to_np(bias.float())
+    y = ops.linear_w8a8(torch.from_numpy(xq).to(DEV), torch.from_numpy(sx).to(DEV), torch.from_numpy(wq).to(DEV),
+                        torch.from_numpy(sw).to(DEV), bias, out_dtype=out_dtype)
+    acc = oracle.c_gemm_i8_i32(xq, wq)
+    if out_dtype == torch.float32:
+        want = oracle.c_dequant_epilogue(acc, sx, sw, bias_np)
+        assert np.array_equal(to_np(y).view(np.uint32), want.view(np.uint32))
+    else:
+        want = oracle.c_dequant_epilogue(acc, sx, sw, bias_np, bf16_out=True)
+        assert np.array_equal(bf16_bits(y), want)
+
+
+# ------------------------------------------------------------------- decode
+
+@pytest.mark.parametrize("M", [1, 2, 3, 4, 5, 8, 11, 16])
+@pytest.mark.parametrize("N,K", [(8192, 2048), (50, 16), (130, 1040), (2048, 5632)])
+def test_gemv_decode_bit_exact(oracle, M, N, K):
+    _say("gemv", M, N, K)
+    x = make_x(M, K, 11 + M).to(torch.bfloat16)
+    w = make_x(N, K, 12) * 0.02
+    wq, sw = oracle.c_quant_rowwise_i8(w.numpy())
+    b = (torch.randn(N, generator=torch.Generator().manual_seed(13)) * 0.01)
+    for bias in (None, b):
+        y = ops.gemv_w8a8_decode(x.to(DEV), torch.from_numpy(wq).to(DEV), torch.from_numpy(sw).to(DEV),
+                                 None if bias is None else bias.to(DEV), out_dtype=torch.bfloat16)
+        want = oracle.c_linear_w8a8(bf16_bits(x), wq, sw, None if bias is None else bias.numpy(),
+                                    x_bf16_bits=True, bf16_out=True)
+        assert np.array_equal(bf16_bits(y), want)
+
+
+def test_gemv_f32_in_out_and_agrees_with_gemm_path(oracle):
+    M, N, K = 16, 1000, 2048
+    x = make_x(M, K, 21, outlier_cols=4)
+    w = make_x(N, K, 22) * 0.02
+    wq, sw = oracle.c_quant_rowwise_i8(w.numpy())
+    wqd, swd = torch.from_numpy(wq).to(DEV), torch.from_numpy(sw).to(DEV)
+    y = ops.gemv_w8a8_decode(x.to(DEV), wqd, swd, out_dtype=torch.float32)
+    want = oracle.c_linear_w8a8(x.numpy(), wq, sw)
+    assert np.array_equal(to_np(y).view(np.uint32), want.view(np.uint32))
+    xq, sx = ops.quant_rowwise_i8(x.to(DEV))
+    y2 = ops.linear_w8a8(xq, sx, wqd, swd, out_dtype=torch.float32)
+    assert torch.equal(y, y2)
+
+
+# ---------------------------------------------------------------------- FP8
+
+def test_quant_tensor_fp8_codes_bit_exact(oracle):
+    tab = oracle.np_e4m3fn_table()[:127].astype(np.float64)
+    mids = (tab[:-1] + tab[1:]) / 2
+    rng = np.random.default_rng(31)
+    base = np.concatenate([tab, -tab, mids, -mids, rng.uniform(-448, 448, 4096 - 506)]).astype(np.float32)
+    assert base.size == 4096
+    base[0] = 448.0  # amax == 448 -> scale exactly 1: inputs are cast as they are
+    x = torch.from_numpy(base)
+    q, s = ops.quant_tensor_fp8(x.to(DEV))
+    qo, so = oracle.c_quant_tensor_fp8(base)
+    assert s.item() == 1.0 == so
+    assert np.array_equal(to_np(q), qo)
+    # general scale, both input dtypes
+    for dtype in (torch.float32, torch.bfloat16):
+        xr = make_x(96, 512, 32).to(DEV, dtype)
+        q, s = ops.quant_tensor_fp8(xr)
+        if dtype == torch.bfloat16:
+            qo, so = oracle.c_quant_tensor_fp8(bf16_bits(xr), bf16_bits=True)
+        else:
+            qo, so = oracle.c_quant_tensor_fp8(to_np(xr))
+        assert np.float32(s.item()) == so
+        assert np.array_equal(to_np(q), qo)
+    q0, s0 = ops.quant_tensor_fp8(torch.zeros(4, 16, device=DEV))
+    assert s0.item() == 1.0 and not to_np(q0).any()
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 1, 16), (33, 70, 144), (256, 128, 1024), (300, 260, 2048), (64, 96, 8192)])
+def test_linear_fp8_within_tolerance(oracle, M, N, K):
+    _say("linear_fp8", M, N, K)
+    x = make_x(M, K, 41)
+    w = make_x(N, K, 42) * 0.02
+    xq, sx = oracle.c_quant_tensor_fp8(x.numpy())
+    wq, sw = oracle.c_quant_tensor_fp8(w.numpy())
+    args = (torch.from_numpy(xq).to(DEV), torch.tensor([sx], device=DEV), torch.from_numpy(wq).to(DEV),
+            torch.tensor([sw], device=DEV))
+    exact = oracle.np_linear_fp8(xq, sx, wq, sw)  # float64 accumulation of the decoded codes
+    rms = float(np.sqrt(np.mean(exact.astype(np.float64) ** 2)))
+    y32 = to_np(ops.linear_fp8(*args, out_dtype=torch.float32))
+    # fp32 accumulation: far inside the stated 1e-2; a wrong code table or a dropped k-slice is not
+    assert np.max(np.abs(y32 - exact)) <= 1e-4 * max(rms, 1e-30)
+    yb = to_np(ops.linear_fp8(*args, out_dtype=torch.bfloat16).float())
+    np.testing.assert_allclose(yb, exact, rtol=1e-2, atol=1e-2 * rms)  # stated tolerance: 1e-2 relative in bf16
+    yc = oracle.c_linear_fp8(xq, sx, wq, sw)
+    np.testing.assert_allclose(y32, yc, rtol=1e-2, atol=1e-4 * rms)
+
+
+def test_linear_fp8_one_hot_pins_operand_order(oracle):
+    M, N, K = 40, 35, 128
+    tab = oracle.np_e4m3fn_table()
+    xq = np.zeros((M, K), np.uint8)
+    ks = (np.arange(M) * 5) % K
+    xq[np.arange(M), ks] = 0x38  # 1.0
+    wq = ((np.arange(N)[:, None] * 7 + np.arange(K)[None, :] * 3) % 120).astype(np.uint8)
+    y = to_np(ops.linear_fp8(torch.from_numpy(xq).to(DEV), torch.tensor([1.0], device=DEV),
+                             torch.from_numpy(wq).to(DEV), torch.tensor([1.0], device=DEV), out_dtype=torch.float32))
+    assert np.array_equal(y, tab[wq][:, ks].T)
+
+
+# -------------------------------------------------------------- module level
+
+def test_config1_quant_linear_matches_oracle_and_float_reference(oracle):
+    """BASELINE config 1: X 64x2048 fp32 with 4 outlier columns x20, W 2048x2048 N(0, 0.02)."""
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(64, 2048, generator=g)
+    cols = torch.randperm(2048, generator=g)[:4]
+    x[:, cols] *= 20
+    w = torch.randn(2048, 2048, generator=g) * 0.02
+    lin = Linear(2048, 2048)
+    with torch.no_grad():
+        lin.weight.copy_(w)
+    lin = lin.to(DEV)
+    q = QuantLinear.from_linear(lin)
+    wq, sw = oracle.c_quant_rowwise_i8(w.numpy())
+    assert np.array_equal(to_np(q.qweight), wq) and np.array_equal(to_np(q.w_scale), sw)
+    with torch.inference_mode():
+        y = q(x.to(DEV))
+    want = oracle.c_linear_w8a8(x.numpy(), wq, sw)
+    assert np.array_equal(to_np(y).view(np.uint32), want.view(np.uint32))
+    ref = torch.nn.functional.linear(x, w).numpy()  # the reference's real path, linear.py:21
+    rel = np.linalg.norm(to_np(y) - ref) / np.linalg.norm(ref)
+    assert rel < 8e-2, rel
+
+
+def test_quant_linear_module_shapes_dispatch_and_state_dict(oracle):
+    torch.manual_seed(1)
+    lin = Linear(256, 192, bias=True)
+    lin.reset_parameters()
+    lin = lin.to(DEV)
+    q = QuantLinear.from_linear(lin)
+    assert isinstance(q, Linear)
+    x3 = torch.randn(2, 20, 256, device=DEV, dtype=torch.bfloat16)   # M = 40 -> MFMA path
+    xd = x3[:, :8].contiguous()                                       # M = 16 -> decode path
+    with torch.inference_mode():
+        y3 = q(x3)
+        yd = q(xd)
+    assert y3.shape == (2, 20, 192) and y3.dtype == torch.bfloat16
+    assert torch.equal(yd, y3[:, :8])  # per-token quantisation: both paths give identical rows
+    ref = torch.nn.functional.linear(x3.float(), lin.weight, lin.bias)
+    assert (y3.float() - ref).norm() / ref.norm() < 3e-2
+    # float checkpoints with the reference's key names load into the quantized module
+    q2 = QuantLinear(256, 192, bias=True, device=DEV)
+    q2.load_state_dict({"weight": lin.weight.detach(), "bias": lin.bias.detach()})
+    assert torch.equal(q2.qweight, q.qweight) and torch.equal(q2.w_scale, q.w_scale)
+    q3 = QuantLinear(256, 192, bias=True, device=DEV)
+    q3.load_state_dict(q.state_dict())
+    with torch.inference_mode():
+        assert torch.equal(q3(x3), y3)
+    with pytest.raises(RuntimeError, match="forward-only"):
+        q(torch.randn(4, 256, device=DEV, requires_grad=True))
+
+
+def test_quantize_model_on_gpu_preserves_outputs_within_quantisation_error():
+    import torch.nn as nn
+
+    class MLP(nn.Module):  # the reference's MLP shape: down(up(x) * silu(gate(x))), mlp.py:24-27
+        def __init__(self):
+            super().__init__()
+            self.up, self.gate, self.down = Linear(128, 352), Linear(128, 352), Linear(352, 128)
+
+        def forward(self, x):
+            return self.down(self.up(x) * torch.nn.functional.silu(self.gate(x)))
+
+    torch.manual_seed(2)
+    m = MLP()
+    for l in (m.up, m.gate, m.down):
+        l.reset_parameters()
+    m = m.to(DEV)
+    x = torch.randn(4, 33, 128, device=DEV)
+    with torch.inference_mode():
+        ref = m(x)
+        assert quantize_model(m) == 3
+        y = m(x)
+        assert (y - ref).norm() / ref.norm() < 5e-2
+        f = MLP().to(DEV)
+        f.load_state_dict({k: v for k, v in zip(["up.weight", "gate.weight", "down.weight"],
+                                                [m.up.weight, m.gate.weight, m.down.weight])})
+        assert quantize_model(f, mode="fp8") == 3 and isinstance(f.up, Fp8Linear)
+        yf = f(x)
+        assert (yf - ref).norm() / ref.norm() < 0.12
+
+
+# ------------------------------------------- full-size, size-independent checks
+
+def test_full_size_prefill_checksum_of_checksums(oracle):
+    """BASELINE config 3 at full size (M=4096, K=N=2048, 1 % outlier channels x10)."""
+    M, N, K = 4096, 2048, 2048
+    x = make_x(M, K, 51, outlier_cols=20, outlier_gain=10.0).to(torch.bfloat16).to(DEV)
+    w = (make_x(N, K, 52) * 0.02).to(DEV)
+    xq, sx = ops.quant_rowwise_i8(x)
+    wq, sw = ops.quant_rowwise_i8(w)
+    assert int(xq.abs().amax(1).min()) == 127 and int(wq.abs().amax(1).min()) == 127
+    acc = ops.gemm_i8_i32(xq, wq)
+    # sum over all outputs == dot of the column sums (exact in int64)
+    lhs = int(acc.sum(dtype=torch.int64))
+    rhs = int((xq.sum(0, dtype=torch.int64) * wq.sum(0, dtype=torch.int64)).sum())
+    assert lhs == rhs
+    # row / column checksums against int64 matvecs
+    ones_n = wq.sum(0, dtype=torch.int64).double()
+    assert torch.equal(acc.sum(1, dtype=torch.int64), (xq.double() @ ones_n).long())
+    ones_m = xq.sum(0, dtype=torch.int64).double()
+    assert torch.equal(acc.sum(0, dtype=torch.int64), (wq.double() @ ones_m).long())
+    # a slab of rows against the oracle, bit for bit, through the fused epilogue
+    bias = (torch.randn(N, generator=torch.Generator().manual_seed(53)) * 0.01).to(DEV)
+    y = ops.linear_w8a8(xq, sx, wq, sw, bias, out_dtype=torch.bfloat16)
+    rows = slice(1900, 2200)
+    want = oracle.c_dequant_epilogue(oracle.c_gemm_i8_i32(to_np(xq[rows]), to_np(wq)), to_np(sx[rows]), to_np(sw),
+                                     to_np(bias), bf16_out=True)
+    assert np.array_equal(bf16_bits(y[rows]), want)
+    # permuting the tokens permutes the output rows
+    perm = torch.randperm(M, generator=torch.Generator().manual_seed(54)).to(DEV)
+    y2 = ops.linear_w8a8(xq[perm].contiguous(), sx[perm].contiguous(), wq, sw, bias, out_dtype=torch.bfloat16)
+    assert torch.equal(y2, y[perm])
+
+
+def test_full_size_fp8_linearity_in_scales(oracle):
+    """BASELINE config 4 at full size (M=2048, K=8192, N=2048)."""
+    M, N, K = 2048, 2048, 8192
+    x = make_x(M, K, 61).to(torch.bfloat16).to(DEV)
+    w = (make_x(N, K, 62) * 0.02).to(DEV)
+    xq, sx = ops.quant_tensor_fp8(x)
+    wq, sw = ops.quant_tensor_fp8(w)
+    assert int(xq.max()) >= 0x7E or int((xq & 0x7F).max()) == 0x7E  # amax lands on 448
+    y = ops.linear_fp8(xq, sx, wq, sw, out_dtype=torch.float32)
+    y2 = ops.linear_fp8(xq, sx * 2, wq, sw * 4, out_dtype=torch.float32)
+    assert torch.equal(y2, y * 8)  # power-of-two scales commute with rounding
+    rows = slice(700, 740)
+    exact = oracle.np_linear_fp8(to_np(xq[rows]), sx.item(), to_np(wq), sw.item())
+    rms = float(np.sqrt(np.mean(exact.astype(np.float64) ** 2)))
+    assert np.max(np.abs(to_np(y[rows]) - exact)) <= 1e-4 * rms
+    ref = torch.nn.functional.linear(x[rows].float(), w)
+    assert ((y[rows] - ref).norm() / ref.norm()).item() < 0.06

@@ -17,6 +17,8 @@ SOURCES = ["abi.hip", "quant.hip", "gemm_mfma.hip", "gemv.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17",
+    # every fp32 operation rounds on its own (bit-exact parity with the CPU oracle)
+    "-ffp-contract=off",
     # packed-fp32 VALU forms are switched off for every kernel in this library
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",

@@ -5,6 +5,11 @@
 
 #include "../../include/astrai_q.h"
 
+// Results are compared bit for bit with a CPU restatement that rounds every
+// fp32 operation separately, so a*b+c must never be contracted into an FMA
+// (__fmul_rn / __fadd_rn are plain operators in HIP and do not prevent it).
+#pragma clang fp contract(off)
+
 #define AQ_WAVE 64
 
 typedef int v4i __attribute__((ext_vector_type(4)));

@@ -1,0 +1,323 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-Linear hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload decode|prefill|fp8]
+
+A "step" is one pass of the hot path over one batch of synthetic input that is
+already resident in HBM:
+
+  decode  (default; BASELINE configs[1], M=16)  x bf16 [16, 2048] -> per-token int8 quantise ->
+          int8 GEMV against W int8 [8192, 2048] -> dequant -> y bf16.  HBM-bound; value = GB/s of
+          algorithmic bytes N*K + 4N + 2MK + 2MN.  The weight rotates over 40 distinct buffers
+          (671 MB) so that no step finds its weight in the 256 MB last-level cache.
+  prefill (configs[2])  x bf16 [4096, 2048] -> per-token int8 quantise -> int8 MFMA GEMM against
+          W [2048, 2048] -> fused scale + bias -> y bf16.  value = TOPS of 2*M*N*K.
+  fp8     (configs[3])  x bf16 [2048, 8192], W [2048, 8192] e4m3, per-tensor scales.
+
+The K timed steps are captured once into a HIP graph and replayed, so the figure is the GPU's,
+not the Python launch loop's; the eager (un-captured) figure is reported beside it.  The
+dominant kernel of each workload is also timed on its own (same graph method) for the roofline
+object.  The CPU baseline is the C oracle (a scalar restatement, OpenMP over rows) on the same
+shapes, timed on the host in the same run.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+METRIC = "quantized-linear TOPS & HBM GB/s (% roofline), decode M=16 and prefill M=4096"
+PEAK_HBM_GBS = 8000.0        # MI355X HBM3E, published
+PEAK_INT8_TOPS = 5000.0      # dense int8 MFMA, published (no sparsity)
+PEAK_FP8_TFLOPS = 5000.0     # dense FP8 MFMA, published
+
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs,
+# scaled by a copy kernel of known size; None until such a run has been made for the workload.
+MEASURED_TRAFFIC = {"decode": None, "prefill": None, "fp8": None}
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="decode", choices=["decode", "prefill", "fp8"])
+    ap.add_argument("--m", type=int, default=16, help="decode rows (1..16)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="skip the secondary workloads")
+    return ap.parse_args()
+
+
+def graph_time_ms(torch, step, steps, warmup):
+    """Warm up eagerly, capture `steps` calls of step(i) into one HIP graph, replay it once
+    untimed, then time one replay with events on the launching stream.  Returns ms per step."""
+    for i in range(warmup):
+        step(i)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(g, stream=side):
+            for i in range(steps):
+                step(i)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    g.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    g.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / steps
+
+
+def eager_time_ms(torch, step, steps, warmup):
+    for i in range(warmup):
+        step(i)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for i in range(steps):
+        step(i)
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / steps
+
+
+def make_weights(torch, ops, N, K, nbuf, dev, seed, mode="int8"):
+    """nbuf independently drawn weights N(0, 0.02), quantised on the GPU by the library."""
+    g = torch.Generator(device=dev).manual_seed(seed)
+    out = []
+    for _ in range(nbuf):
+        w = torch.randn(N, K, generator=g, device=dev) * 0.02
+        out.append(ops.quant_rowwise_i8(w) if mode == "int8" else ops.quant_tensor_fp8(w))
+    return out
+
+
+def bench_decode(torch, ops, args, dev):
+    M, K, N = args.m, 2048, 8192
+    nbuf = 40
+    weights = make_weights(torch, ops, N, K, nbuf, dev, seed=1)
+    g = torch.Generator(device=dev).manual_seed(2)
+    x = torch.randn(M, K, generator=g, device=dev).to(torch.bfloat16)
+    ws = torch.empty((ops._abi.load().aq_gemv_w8a8_workspace_bytes(M, K),), dtype=torch.uint8, device=dev)
+    ys = [None]
+
+    def step(i):
+        wq, sw = weights[i % nbuf]
+        ys[0] = ops.gemv_w8a8_decode(x, wq, sw, None, out_dtype=torch.bfloat16, workspace=ws)
+
+    xq, sx = ops.quant_rowwise_i8(x)
+
+    def kernel_only(i):
+        wq, sw = weights[i % nbuf]
+        ys[0] = ops.gemv_w8a8_codes(xq, sx, wq, sw, None, out_dtype=torch.bfloat16)
+
+    def resident(i):  # same weight every step: served by the last-level cache
+        wq, sw = weights[0]
+        ys[0] = ops.gemv_w8a8_codes(xq, sx, wq, sw, None, out_dtype=torch.bfloat16)
+
+    bytes_alg = N * K + 4 * N + 2 * M * K + 2 * M * N
+    ms = graph_time_ms(torch, step, args.steps, args.warmup)
+    ms_eager = eager_time_ms(torch, step, args.steps, args.warmup)
+    ms_k = graph_time_ms(torch, kernel_only, args.steps, args.warmup)
+    ms_res = graph_time_ms(torch, resident, args.steps, args.warmup)
+    gbs = bytes_alg / (ms * 1e-3) / 1e9
+    gbs_k = bytes_alg / (ms_k * 1e-3) / 1e9
+    return {
+        "workload": f"decode_gemv_w8a8 M={M} K={K} N={N} bf16->int8 per-token, W int8 per-channel, bf16 out",
+        "value": gbs, "unit": "GB/s", "ms_per_step": ms, "eager_ms_per_step": ms_eager,
+        "bytes_per_step": bytes_alg, "dtype": "int8",
+        "roofline": {"bound": "hbm", "kernel": "gemv_w8a8_kernel", "achieved": gbs_k, "peak": PEAK_HBM_GBS,
+                     "unit": "GB/s", "frac": gbs_k / PEAK_HBM_GBS, "traffic": MEASURED_TRAFFIC["decode"],
+                     "kernel_us": ms_k * 1e3, "algorithmic_bytes": bytes_alg,
+                     "llc_resident_gbs": bytes_alg / (ms_res * 1e-3) / 1e9, "weight_buffers": nbuf},
+        "shape": (M, N, K),
+    }
+
+
+def bench_prefill(torch, ops, args, dev):
+    M, K, N = 4096, 2048, 2048
+    nbuf = 8
+    weights = make_weights(torch, ops, N, K, nbuf, dev, seed=3)
+    g = torch.Generator(device=dev).manual_seed(4)
+    xs = []
+    for _ in range(nbuf):
+        x = torch.randn(M, K, generator=g, device=dev)
+        cols = torch.randperm(K, generator=g, device=dev)[:20]  # 1 % outlier channels x10
+        x[:, cols] *= 10
+        xs.append(x.to(torch.bfloat16))
+    bias = (torch.randn(N, generator=g, device=dev) * 0.01)
+    ys = [None]
+
+    def step(i):
+        xq, sx = ops.quant_rowwise_i8(xs[i % nbuf])
+        wq, sw = weights[i % nbuf]
+        ys[0] = ops.linear_w8a8(xq, sx, wq, sw, bias, out_dtype=torch.bfloat16)
+
+    pre = [ops.quant_rowwise_i8(x) for x in xs]
+
+    def kernel_only(i):
+        xq, sx = pre[i % nbuf]
+        wq, sw = weights[i % nbuf]
+        ys[0] = ops.linear_w8a8(xq, sx, wq, sw, bias, out_dtype=torch.bfloat16)
+
+    def quant_only(i):
+        ys[0] = ops.quant_rowwise_i8(xs[i % nbuf])
+
+    ops_alg = 2.0 * M * N * K
+    steps = max(10, min(args.steps, 100))
+    ms = graph_time_ms(torch, step, steps, args.warmup)
+    ms_k = graph_time_ms(torch, kernel_only, steps, args.warmup)
+    ms_q = graph_time_ms(torch, quant_only, steps, args.warmup)
+    tops = ops_alg / (ms * 1e-3) / 1e12
+    tops_k = ops_alg / (ms_k * 1e-3) / 1e12
+    qbytes = 2 * M * K + M * K + 4 * M
+    return {
+        "workload": f"prefill_linear_w8a8 M={M} K={K} N={N} quantise + int8 MFMA GEMM + scale/bias epilogue, bf16 out",
+        "value": tops, "unit": "TOPS", "ms_per_step": ms, "ops_per_step": ops_alg, "dtype": "int8",
+        "roofline": {"bound": "mfma", "kernel": "gemm_kernel<int8,bf16>", "achieved": tops_k, "peak": PEAK_INT8_TOPS,
+                     "unit": "TOP/s", "frac": tops_k / PEAK_INT8_TOPS, "traffic": MEASURED_TRAFFIC["prefill"],
+                     "kernel_us": ms_k * 1e3, "algorithmic_ops": ops_alg},
+        "quantise_kernel": {"us": ms_q * 1e3, "gbs": qbytes / (ms_q * 1e-3) / 1e9, "frac_hbm": qbytes / (ms_q * 1e-3) / 1e9 / PEAK_HBM_GBS,
+                            "algorithmic_bytes": qbytes},
+        "shape": (M, N, K),
+    }
+
+
+def bench_fp8(torch, ops, args, dev):
+    M, K, N = 2048, 8192, 2048
+    nbuf = 4
+    weights = make_weights(torch, ops, N, K, nbuf, dev, seed=5, mode="fp8")
+    g = torch.Generator(device=dev).manual_seed(6)
+    xs = [torch.randn(M, K, generator=g, device=dev).to(torch.bfloat16) for _ in range(nbuf)]
+    ys = [None]
+
+    def step(i):
+        xq, sx = ops.quant_tensor_fp8(xs[i % nbuf])
+        wq, sw = weights[i % nbuf]
+        ys[0] = ops.linear_fp8(xq, sx, wq, sw, out_dtype=torch.bfloat16)
+
+    pre = [ops.quant_tensor_fp8(x) for x in xs]
+
+    def kernel_only(i):
+        xq, sx = pre[i % nbuf]
+        wq, sw = weights[i % nbuf]
+        ys[0] = ops.linear_fp8(xq, sx, wq, sw, out_dtype=torch.bfloat16)
+
+    flops = 2.0 * M * N * K
+    steps = max(10, min(args.steps, 50))
+    ms = graph_time_ms(torch, step, steps, args.warmup)
+    ms_k = graph_time_ms(torch, kernel_only, steps, args.warmup)
+    t = flops / (ms * 1e-3) / 1e12
+    tk = flops / (ms_k * 1e-3) / 1e12
+    return {
+        "workload": f"fp8_linear M={M} K={K} N={N} per-tensor e4m3 quantise + FP8 MFMA GEMM, bf16 out",
+        "value": t, "unit": "TFLOP/s", "ms_per_step": ms, "flops_per_step": flops, "dtype": "fp8_e4m3",
+        "roofline": {"bound": "mfma", "kernel": "gemm_kernel<fp8,bf16>", "achieved": tk, "peak": PEAK_FP8_TFLOPS,
+                     "unit": "TFLOP/s", "frac": tk / PEAK_FP8_TFLOPS, "traffic": MEASURED_TRAFFIC["fp8"],
+                     "kernel_us": ms_k * 1e3, "algorithmic_flops": flops},
+        "shape": (M, N, K),
+    }
+
+
+def cpu_baseline(workload, shape, unit, per_step):
+    """The C oracle on the same shape, on this host's cores.  Test infrastructure used as the
+    reported baseline only: it never feeds the GPU path."""
+    import numpy as np
+
+    from oracle import oracle
+
+    M, N, K = shape
+    rng = np.random.default_rng(0)
+    threads = oracle.c_num_threads()
+    if workload == "fp8":
+        Ms = 32  # bounded sample: 32 of the 2048 rows (scalar fp32 accumulation is slow)
+        x = rng.standard_normal((Ms, K)).astype(np.float32)
+        w = (rng.standard_normal((N, K)) * 0.02).astype(np.float32)
+        wq, sw = oracle.c_quant_tensor_fp8(w)
+        t0 = time.perf_counter()
+        xq, sx = oracle.c_quant_tensor_fp8(x)
+        oracle.c_linear_fp8(xq, sx, wq, sw, bf16_out=True)
+        dt = time.perf_counter() - t0
+        val = 2.0 * Ms * N * K / dt / 1e12
+        return {"value": val, "unit": unit, "cores": threads, "kind": "port",
+                "sample": f"one pass over {Ms} of {M} rows (same N, K), {dt:.2f} s"}
+    x = oracle.np_f32_to_bf16_bits(rng.standard_normal((M, K)).astype(np.float32))
+    w = (rng.standard_normal((N, K)) * 0.02).astype(np.float32)
+    wq, sw = oracle.c_quant_rowwise_i8(w)
+    bias = None if workload == "decode" else (rng.standard_normal(N) * 0.01).astype(np.float32)
+    oracle.c_linear_w8a8(x[: min(M, 64)], wq, sw, bias, x_bf16_bits=True, bf16_out=True)  # warm the threads
+    reps, t_total = 0, 0.0
+    budget = 6.0
+    while t_total < budget and reps < 400:
+        t0 = time.perf_counter()
+        oracle.c_linear_w8a8(x, wq, sw, bias, x_bf16_bits=True, bf16_out=True)
+        t_total += time.perf_counter() - t0
+        reps += 1
+    dt = t_total / reps
+    scale = 1e9 if unit == "GB/s" else 1e12
+    return {"value": per_step / dt / scale, "unit": unit, "cores": threads, "kind": "port",
+            "sample": f"{reps} full passes of the same shape (quantise + int8 GEMM + epilogue), {dt * 1e3:.2f} ms each"}
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU only: --gpus {args.gpus} is not supported in this build "
+              "(no collectives or sharding are part of it)", file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    from khaosz_amd import ops
+
+    ops._abi.load()  # fails loudly when the HIP library is missing
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    fns = {"decode": bench_decode, "prefill": bench_prefill, "fp8": bench_fp8}
+    with torch.inference_mode():
+        main_res = fns[args.workload](torch, ops, args, dev)
+        extra = {}
+        if not args.no_extra:
+            for name in ("decode", "prefill", "fp8"):
+                if name != args.workload:
+                    extra[name] = fns[name](torch, ops, args, dev)
+            if args.workload == "decode":
+                for m in (1, 4):
+                    a2 = argparse.Namespace(**vars(args))
+                    a2.m = m
+                    r = bench_decode(torch, ops, a2, dev)
+                    extra[f"decode_m{m}"] = r
+    per_step = main_res.get("bytes_per_step") or main_res.get("ops_per_step") or main_res.get("flops_per_step")
+    cpu = None
+    if not args.no_cpu:
+        cpu = cpu_baseline(args.workload, main_res["shape"], main_res["unit"], per_step)
+        if not args.no_extra and "prefill" in extra:
+            # one pass of the prefill shape as well, so both halves of the metric have a CPU figure
+            extra["prefill"]["cpu_baseline"] = cpu_baseline("prefill", extra["prefill"]["shape"], "TOPS",
+                                                            extra["prefill"]["ops_per_step"])
+    for r in [main_res, *extra.values()]:
+        r.pop("shape", None)
+    line = {
+        "metric": METRIC, "value": main_res["value"], "unit": main_res["unit"], "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": main_res["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": main_res["dtype"],
+        "data": "synthetic", "config": {"workload": main_res["workload"], "timing": "HIP graph replay of the timed steps",
+                                        "eager_ms_per_step": main_res.get("eager_ms_per_step")},
+        "roofline": main_res["roofline"], "cpu_baseline": cpu,
+        "also": {k: {kk: vv for kk, vv in v.items()} for k, v in extra.items()},
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

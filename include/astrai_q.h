@@ -103,6 +103,18 @@ int aq_gemv_w8a8_codes(const int8_t *xq, const float *sx, const int8_t *wq, cons
 int aq_linear_fp8(const uint8_t *xq, const float *sx, const uint8_t *wq, const float *sw,
                   void *y, int y_dtype, int64_t M, int64_t N, int64_t K, void *stream);
 
+/* ---- measurement probes: no counterpart in the reference, not on the Linear
+ * path.  They measure what this part's matrix cores and HBM deliver so that the
+ * benchmark can quote kernels against measured as well as published ceilings.
+ * aq_probe_mfma: `workgroups` x 4 wavefronts each issue iters x 8 independent
+ *   MFMAs; kind 0 = i32_32x32x32_i8 (65536 ops each), 1 = i32_16x16x64_i8
+ *   (32768 ops), 2 = f32_32x32x64 e4m3 (131072 flops).
+ * aq_probe_copy / aq_probe_read: grid-stride 16-byte streaming copy / read of
+ *   `bytes` (a multiple of 16). */
+int aq_probe_mfma(int kind, int workgroups, int iters, int *sink, void *stream);
+int aq_probe_copy(const void *src, void *dst, int64_t bytes, int workgroups, void *stream);
+int aq_probe_read(const void *src, int64_t bytes, int workgroups, int *sink, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

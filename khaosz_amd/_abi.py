@@ -7,7 +7,7 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libastrai_q.so")
+LIB_PATH = os.environ.get("ASTRAI_Q_LIB") or os.path.join(_HERE, "lib", "libastrai_q.so")
 
 AQ_F32, AQ_BF16 = 0, 1
 
@@ -24,6 +24,9 @@ SYMBOLS = {
     "aq_gemv_w8a8_decode": (_int, [_vp, _int, _vp, _vp, _vp, _int, _vp, _int, _i64, _i64, _i64, _vp, _sz, _vp]),
     "aq_gemv_w8a8_codes": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _vp, _int, _i64, _i64, _i64, _vp]),
     "aq_linear_fp8": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _vp]),
+    "aq_probe_mfma": (_int, [_int, _int, _int, _vp, _vp]),
+    "aq_probe_copy": (_int, [_vp, _vp, _i64, _int, _vp]),
+    "aq_probe_read": (_int, [_vp, _i64, _int, _vp, _vp]),
 }
 
 _lib = None

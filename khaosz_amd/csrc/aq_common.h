@@ -30,6 +30,16 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
   return r & 0xffffu;
 }
 
+// two fp32 -> packed bf16 pair (lo in bits 15:0) with the hardware converter
+// (v_cvt_pk_bf16_f32: round to nearest even, NaN stays NaN).
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  typedef float f2 __attribute__((ext_vector_type(2)));
+  typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+  const f2 v = {lo, hi};
+  const bf2 b = __builtin_convertvector(v, bf2);
+  return *reinterpret_cast<const uint32_t*>(&b);
+}
+
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, AQ_WAVE));

@@ -6,22 +6,32 @@
 //                                         B = weight codes     [N, K]
 // Both operands are K-contiguous, which is exactly the MFMA operand order
 // (each lane feeds 16 or 32 consecutive k of one row), so no transpose is ever
-// materialised.  A workgroup of 4 wavefronts owns a 256 x 128 tile of C; each
-// wavefront a 128 x 64 sub-tile held as 4 x 2 MFMA 32x32 accumulators (128
-// registers).  K is walked in 128-byte steps: global -> registers -> LDS with
-// two LDS stages, one barrier per step; rows are padded by 16 bytes so the
-// 16-byte fragment reads of 8 consecutive rows cover all 32 banks.
-// The epilogue is fused: int32 store, or dequantise (+bias) and cast.
+// materialised.  A workgroup of 8 wavefronts (two per SIMD) owns a 256 x 128
+// tile of C; each wavefront a 64 x 64 sub-tile held as 2 x 2 MFMA 32x32
+// accumulators.  K is walked in 128-byte steps through three LDS stages that
+// are filled by direct global->LDS loads (no register staging), with an XOR
+// permutation of 16-byte pieces that makes the fragment reads bank-conflict
+// free; the loop is software-pipelined so that LDS reads and global loads of
+// later sub-steps are issued between the MFMAs of the current one, with one
+// workgroup barrier per K step.  The epilogue is fused and runs straight from
+// the accumulator registers: int32 store, or dequantise (+bias) and cast.
+#include <type_traits>
+
 #include "aq_common.h"
 
 namespace aq {
 
 constexpr int BM = 256, BN = 128, BK = 128;
-constexpr int PITCH = BK + 16;
-constexpr int WAVE_M = 128, WAVE_N = 64;  // 2 x 2 wavefronts
+constexpr int NSTAGE = 3;  // LDS stages: 3 x 48 KiB of the 160 KiB
+#ifndef AQ_WAVES_M
+#define AQ_WAVES_M 4
+#endif
+constexpr int WAVES_M = AQ_WAVES_M, WAVES_N = 2;  // wavefronts per workgroup: two per SIMD by default
+constexpr int NWAVES = WAVES_M * WAVES_N, NTHREADS = NWAVES * 64;
+constexpr int WAVE_M = BM / WAVES_M, WAVE_N = BN / WAVES_N;
 constexpr int TM = WAVE_M / 32, TN = WAVE_N / 32;
-constexpr int A_LOADS = BM * BK / 16 / 256;  // 16-byte vectors per thread per K step
-constexpr int B_LOADS = BN * BK / 16 / 256;
+constexpr int A_LOADS = BM * BK / 16 / NTHREADS;  // 16-byte vectors per thread per K step
+constexpr int B_LOADS = BN * BK / 16 / NTHREADS;
 constexpr int NUM_XCD = 8;
 constexpr int GROUP_M = 4;
 
@@ -67,53 +77,163 @@ struct Acc<true> {
   using type = v16f;
 };
 
+// s_waitcnt with only the vector-memory counter constrained (gfx9 encoding:
+// vmcnt in bits 3:0 and 15:14, expcnt 6:4 and lgkmcnt 11:8 left at their maxima).
+#define AQ_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(0x0f70 | ((n) & 15) | (((n) >> 4) << 14))
+// Workgroup barrier without the memory fence of __syncthreads(): the fence
+// would drain every outstanding global->LDS load, including the ones issued
+// two K steps ahead on purpose.  The empty asm statements stop the compiler
+// from moving LDS accesses across it.
+#define AQ_BARRIER()                   \
+  do {                                 \
+    asm volatile("" ::: "memory");     \
+    __builtin_amdgcn_s_barrier();      \
+    asm volatile("" ::: "memory");     \
+  } while (0)
+
+typedef __attribute__((address_space(3))) void lds_void;
+
+
+template <bool FP8>
+struct Frag {
+  using type = v4i;  // 16 bytes of K per lane: v_mfma_i32_32x32x32_i8
+};
+template <>
+struct Frag<true> {
+  using type = v8i;  // 32 bytes of K per lane: v_mfma_scale_f32_32x32x64_f8f6f4
+};
+
+template <bool FP8>
+__device__ __forceinline__ typename Acc<FP8>::type mma(const typename Frag<FP8>::type& a,
+                                                       const typename Frag<FP8>::type& b,
+                                                       const typename Acc<FP8>::type& c) {
+  if constexpr (!FP8) {
+    return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
+  } else {
+    // E8M0 scale 127 = 2^0 for both operands: plain e4m3 x e4m3.
+    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
+  }
+}
+
+// Issue order of one pipeline slot, as scheduling groups: GROUPS times
+// [1 MFMA, NDS LDS reads, this group's share of the NLD global loads].
+// (0x008 = MFMA, 0x100 = LDS read, 0x020 = vector-memory read.)
+template <int G, int GROUPS, int NDS, int NLD>
+__device__ __forceinline__ void sched_pattern() {
+  if constexpr (G < GROUPS) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    __builtin_amdgcn_sched_group_barrier(0x100, NDS, 0);
+    constexpr int nl = ((G + 1) * NLD) / GROUPS - (G * NLD) / GROUPS;
+    if constexpr (nl > 0) __builtin_amdgcn_sched_group_barrier(0x020, nl, 0);
+    sched_pattern<G + 1, GROUPS, NDS, NLD>();
+  }
+}
+
 template <bool FP8, int OUT>
-__global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
-  __shared__ __attribute__((aligned(16))) uint8_t smem[2 * (BM + BN) * PITCH];
-  uint8_t* const sA0 = smem;
-  uint8_t* const sB0 = smem + BM * PITCH;
-  constexpr int STAGE = (BM + BN) * PITCH;
+__global__ __launch_bounds__(NTHREADS) void gemm_kernel(GemmArgs p) {
+  // NSTAGE stages of [A tile 256 x 128 B][B tile 128 x 128 B], rows unpadded.
+  // Global->LDS loads land 64 lanes x 16 B contiguously (8 rows of 128 B), so
+  // the bank-conflict-free layout is obtained by permuting which 16-byte piece
+  // of its row each lane fetches: piece c of row r is stored at slot
+  // c ^ ((r / 2) % 8).  LDS has 64 banks here (two 128-byte rows per bank
+  // line) and a 16-byte-per-lane read is served 16 lanes at a time, so 16
+  // consecutive rows reading the same piece must land on 16 distinct slots.
+  constexpr int STAGE = (BM + BN) * BK;
+  __shared__ __attribute__((aligned(1024))) uint8_t smem[NSTAGE * STAGE];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int wave_m = wave >> 1, wave_n = wave & 1;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
 
   int tile_m, tile_n;
   tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
   const int m0 = tile_m * BM, n0 = tile_n * BN;
   const int M = p.M, N = p.N, K = p.K;
 
-  // ---- global -> LDS staging assignment: vector c = i*256 + tid, row = c/8
-  const int ld_row = tid >> 3;       // + 32*i
-  const int ld_kc = (tid & 7) * 16;  // byte offset inside the K step
   // Tile-local buffer descriptors: rows past the M / N edge fall outside and read as zero.
   const int rows_a = (M - m0) < BM ? (M - m0) : BM;
   const int rows_b = (N - n0) < BN ? (N - n0) : BN;
   const __amdgpu_buffer_rsrc_t Ar = make_rsrc(p.A + (int64_t)m0 * K, (uint32_t)rows_a * (uint32_t)K);
   const __amdgpu_buffer_rsrc_t Br = make_rsrc(p.B + (int64_t)n0 * K, (uint32_t)rows_b * (uint32_t)K);
-  const uint32_t ld_off = (uint32_t)ld_row * (uint32_t)K + ld_kc;  // + 32*i rows, + k0
-  const uint32_t row32 = 32u * (uint32_t)K;
 
-  uint4 ra[A_LOADS], rb[B_LOADS];
-  auto gload = [&](int k0) {
-    // K is a multiple of 16: a vector is all in or all out.  Vectors past K
-    // would alias the next row, so they are pushed out of the descriptor.
-    const bool ok = (k0 + ld_kc) < K;
-    const uint32_t base = ok ? ld_off + (uint32_t)k0 : OOB_OFFSET;
+  // Epilogue operands are fetched first of all, so their latency is hidden
+  // behind the whole K loop: per-row activation scales as 16 float4 per lane
+  // (accumulator register r of lane l belongs to row (r/4)*8 + (l/32)*4 + r%4),
+  // per-column weight scale and bias as one scalar per 32x32 tile column.
+  const int col = lane & 31;
+  const int rq = (lane >> 5) * 4;  // row offset of this lane's half inside each group of 8 rows
+  const int mw = __builtin_amdgcn_readfirstlane(m0 + wave_m * WAVE_M);  // wavefront-uniform: keep it scalar
+  float sx1 = 1.0f, sw1 = 1.0f;
+  float sxr[TM][4][4];  // [i][g][q]: row i*32 + g*8 + rq + q
+  float swn[TN], bn[TN];
+  bool has_bias = false;
+  if constexpr (FP8) {
+    sx1 = *p.sx;
+    sw1 = *p.sw;
+  } else if constexpr (OUT != OUT_I32) {
+    // rows past M fall outside the descriptor and read as zero (their outputs are never stored)
+    const int rows_left = __builtin_amdgcn_readfirstlane((M - mw) > 0 ? (M - mw) : 0);
+    const __amdgpu_buffer_rsrc_t Sr =
+        make_rsrc(p.sx + (rows_left ? mw : 0), (uint32_t)(rows_left < WAVE_M ? rows_left : WAVE_M) * 4u);
+    if ((M & 3) == 0) {  // uniform: the 4 rows of a float4 are all in or all out, and 16-byte aligned
 #pragma unroll
-    for (int i = 0; i < A_LOADS; ++i) ra[i] = buffer_load_16(Ar, ok ? base + i * row32 : OOB_OFFSET);
+      for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int i = 0; i < B_LOADS; ++i) rb[i] = buffer_load_16(Br, ok ? base + i * row32 : OOB_OFFSET);
-  };
-  const int lds_st = ld_row * PITCH + ld_kc;
-  auto lstore = [&](int buf) {
-    uint8_t* a = sA0 + buf * STAGE + lds_st;
-    uint8_t* b = sB0 + buf * STAGE + lds_st;
+        for (int g = 0; g < 4; ++g) {
+          const uint4 t = buffer_load_16(Sr, (uint32_t)(i * 32 + g * 8 + rq) * 4u);
+          sxr[i][g][0] = __uint_as_float(t.x);
+          sxr[i][g][1] = __uint_as_float(t.y);
+          sxr[i][g][2] = __uint_as_float(t.z);
+          sxr[i][g][3] = __uint_as_float(t.w);
+        }
+    } else {
 #pragma unroll
-    for (int i = 0; i < A_LOADS; ++i) *reinterpret_cast<uint4*>(a + i * 32 * PITCH) = ra[i];
+      for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int i = 0; i < B_LOADS; ++i) *reinterpret_cast<uint4*>(b + i * 32 * PITCH) = rb[i];
+        for (int g = 0; g < 4; ++g)
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+            sxr[i][g][q] = __uint_as_float(
+                (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(Sr, (i * 32 + g * 8 + rq + q) * 4, 0, 0));
+    }
+    has_bias = p.bias != nullptr;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int n = n0 + wave_n * WAVE_N + j * 32 + col;
+      const int nc = n < N ? n : (N - 1);
+      swn[j] = p.sw[nc];
+      bn[j] = 0.0f;
+      if (has_bias)
+        bn[j] = p.bias_dtype == AQ_BF16 ? bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(p.bias)[nc])
+                                        : reinterpret_cast<const float*>(p.bias)[nc];
+    }
+  }
+
+  // One load instruction of a wavefront fills 1 KiB = 8 tile rows.  Wavefront w
+  // owns the 8-row groups w, w+NWAVES, w+2*NWAVES, ... of A and of B.
+  // Row of lane l in group j: 8j + l/8, so (row/2) % 8 = 4*(w & 1) + l/16
+  // (NWAVES is even, so j and w have the same parity).
+  static_assert(NWAVES % 2 == 0, "the piece permutation assumes group and wavefront share parity");
+  const int ld_row = wave * 8 + (lane >> 3);  // + 8*NWAVES*i
+  const int ld_piece = ((lane & 7) ^ (4 * (wave & 1) + (lane >> 4))) * 16;  // piece this lane fetches
+  const uint32_t ld_off = (uint32_t)ld_row * (uint32_t)K + ld_piece;
+  const uint32_t row32 = (uint32_t)(8 * NWAVES) * (uint32_t)K;  // byte distance between a wavefront's row groups
+  constexpr int NLOADS = A_LOADS + B_LOADS;
+  // load number `idx` (0..NLOADS-1) of K step kt into stage buffer `buf`
+  auto issue_load = [&](int kt, int buf, int idx) {
+    const int k0 = kt * BK;
+    // K is a multiple of 16: a piece is all in or all out.  Pieces past K would
+    // alias the next row, so they are pushed outside the descriptor (-> zeros).
+    const uint32_t off = (k0 + ld_piece) < K ? ld_off + (uint32_t)k0 : OOB_OFFSET;
+    uint8_t* st = smem + buf * STAGE + wave * 1024;
+    if (idx < A_LOADS)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(Ar, (lds_void*)(st + idx * (1024 * NWAVES)), 16,
+                                               off == OOB_OFFSET ? OOB_OFFSET : off + idx * row32, 0, 0, 0);
+    else
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(Br, (lds_void*)(st + BM * BK + (idx - A_LOADS) * (1024 * NWAVES)), 16,
+                                               off == OOB_OFFSET ? OOB_OFFSET : off + (idx - A_LOADS) * row32,
+                                               0, 0, 0);
   };
 
   using acc_t = typename Acc<FP8>::type;
@@ -125,119 +245,237 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
-  // fragment read offsets: lane -> row lane%32, k bytes (lane/32)*FRAG within a sub-step
-  constexpr int FRAG = FP8 ? 32 : 16;  // bytes of K per lane per MFMA
-  constexpr int KSUB = 2 * FRAG;       // K per MFMA: 32 (int8) or 64 (fp8)
-  const int fr_a = (wave_m * WAVE_M + (lane & 31)) * PITCH + (lane >> 5) * FRAG;
-  const int fr_b = (wave_n * WAVE_N + (lane & 31)) * PITCH + (lane >> 5) * FRAG;
+  // Fragment reads: lane -> tile row lane%32; its K pieces within a 128-byte row
+  // are (ks*2 + lane/32) for int8 (16 B per MFMA) and (ks*4 + (lane/32)*2 + {0,1})
+  // for FP8 (32 B per MFMA); slot = piece ^ ((row/2) % 8) and (row/2) % 8 == (lane/2) % 8.
+  const int fr_a = (wave_m * WAVE_M + (lane & 31)) * BK;
+  const int fr_b = BM * BK + (wave_n * WAVE_N + (lane & 31)) * BK;
+  const int fsw = (lane >> 1) & 7;
+  const int swz = FP8 ? ((((lane >> 5) * 2) ^ fsw) << 4) : (((lane >> 5) ^ fsw) << 4);
+  constexpr int KSUB = FP8 ? 64 : 32;  // K per MFMA
+  constexpr int NKS = BK / KSUB;       // MFMA sub-steps per stage: 4 (int8) or 2 (FP8)
+  static_assert(NKS % 2 == 0, "fragment double-buffering alternates per sub-step");
+  using frag_t = typename Frag<FP8>::type;
+  auto load_frags = [&](const uint8_t* st, int ks, frag_t (&a)[TM], frag_t (&b)[TN]) {
+    if constexpr (!FP8) {
+      const int o = ((ks * 2) << 4) ^ swz;
+#pragma unroll
+      for (int i = 0; i < TM; ++i) a[i] = *reinterpret_cast<const v4i*>(st + fr_a + i * 32 * BK + o);
+#pragma unroll
+      for (int j = 0; j < TN; ++j) b[j] = *reinterpret_cast<const v4i*>(st + fr_b + j * 32 * BK + o);
+    } else {
+      const int o0 = ((ks * 4) << 4) ^ swz, o1 = o0 ^ 16;
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        const v4i lo = *reinterpret_cast<const v4i*>(st + fr_a + i * 32 * BK + o0);
+        const v4i hi = *reinterpret_cast<const v4i*>(st + fr_a + i * 32 * BK + o1);
+        a[i] = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+      }
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const v4i lo = *reinterpret_cast<const v4i*>(st + fr_b + j * 32 * BK + o0);
+        const v4i hi = *reinterpret_cast<const v4i*>(st + fr_b + j * 32 * BK + o1);
+        b[j] = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+      }
+    }
+  };
+
+  // One pipeline slot = the TM*TN MFMAs of one sub-step, with the LDS reads of
+  // the next sub-step's fragments and (LOADS) a share of the global->LDS loads
+  // of a later stage interleaved between them, so that a wavefront (the only
+  // one on its SIMD) never queues a burst of memory instructions in front of
+  // the matrix core.
+  frag_t af[2][TM], bf[2][TN];
+  // slot number Q (0 = slot A .. NKS-1) issues loads [Q*NLOADS/NKS, (Q+1)*NLOADS/NKS) of its stage
+  auto slot = [&](auto cur_c, const uint8_t* st_next, int ks_next, auto loads_c, int kt_ld, int buf_ld,
+                  auto q_c) {
+    constexpr int CUR = decltype(cur_c)::value;
+    constexpr bool LOADS = decltype(loads_c)::value;
+    constexpr int Q = decltype(q_c)::value;
+    constexpr int LD0 = (Q * NLOADS) / NKS, LPS = ((Q + 1) * NLOADS) / NKS - LD0;
+    load_frags(st_next, ks_next, af[CUR ^ 1], bf[CUR ^ 1]);
+    if constexpr (LOADS) {
+#pragma unroll
+      for (int q = 0; q < LPS; ++q) issue_load(kt_ld, buf_ld, LD0 + q);
+    }
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) acc[i][j] = mma<FP8>(af[CUR][i], bf[CUR][j], acc[i][j]);
+    // issue order: one MFMA, then the LDS reads (and at most one global load) it covers
+    constexpr int NMMA = TM * TN;
+    constexpr int NDS = (TM + TN) * (FP8 ? 2 : 1);
+    constexpr int GROUPS = NMMA > 4 ? NMMA - 2 : NMMA;
+    sched_pattern<0, GROUPS, (NDS + GROUPS - 1) / GROUPS, LOADS ? LPS : 0>();
+    if constexpr (GROUPS < NMMA) __builtin_amdgcn_sched_group_barrier(0x008, NMMA - GROUPS, 0);
+  };
+  using std::integral_constant;
+  using k0 = integral_constant<int, 0>;
+  using k1 = integral_constant<int, 1>;
+  using q0 = integral_constant<int, 0>;
+  using q1 = integral_constant<int, 1>;
+  using q2 = integral_constant<int, 2>;
+  using q3 = integral_constant<int, 3>;
+  using yes = integral_constant<bool, true>;
+  using no = integral_constant<bool, false>;
 
   const int nk = (K + BK - 1) / BK;
-  gload(0);
-  lstore(0);
-  __syncthreads();
-  for (int kt = 0; kt < nk; ++kt) {
-    const int cur = kt & 1;
-    if (kt + 1 < nk) gload((kt + 1) * BK);
-    const uint8_t* a = sA0 + cur * STAGE + fr_a;
-    const uint8_t* b = sB0 + cur * STAGE + fr_b;
+  // Rotated software pipeline over K steps ("stages" s = 0 .. nk-1):
+  //   iteration s:  slots    MFMAs of (s, 0 .. NKS-2)       | read fragments (s, 1 .. NKS-1)
+  //                 wait for this wavefront's loads of stage s+1, barrier
+  //                 slot A   MFMAs of (s, last sub-step)    | read fragments (s+1, 0)
+  // with the loads of stage s+3 spread from slot A of s over the slots of s+1.
+  // At the barrier every wavefront holds the last fragments of stage s in
+  // registers, so stage s's LDS buffer is free for the loads of stage s+3 right
+  // after it, and stage s+1 is complete and visible for slot A's fragment reads.
+  // Loads past the last K step are still issued (outside the descriptors they
+  // write zeros into a stage nobody reads) so that the count of outstanding
+  // loads per wavefront is the same at every wait.
 #pragma unroll
-    for (int ks = 0; ks < BK / KSUB; ++ks) {
-      if constexpr (!FP8) {
-        v4i af[TM], bf[TN];
+  for (int st = 0; st < NSTAGE; ++st)
 #pragma unroll
-        for (int i = 0; i < TM; ++i) af[i] = *reinterpret_cast<const v4i*>(a + i * 32 * PITCH + ks * KSUB);
-#pragma unroll
-        for (int j = 0; j < TN; ++j) bf[j] = *reinterpret_cast<const v4i*>(b + j * 32 * PITCH + ks * KSUB);
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-          for (int j = 0; j < TN; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bf[j], acc[i][j], 0, 0, 0);
-      } else {
-        v8i af[TM], bf[TN];
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-          const v4i lo = *reinterpret_cast<const v4i*>(a + i * 32 * PITCH + ks * KSUB);
-          const v4i hi = *reinterpret_cast<const v4i*>(a + i * 32 * PITCH + ks * KSUB + 16);
-          af[i] = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-        }
-#pragma unroll
-        for (int j = 0; j < TN; ++j) {
-          const v4i lo = *reinterpret_cast<const v4i*>(b + j * 32 * PITCH + ks * KSUB);
-          const v4i hi = *reinterpret_cast<const v4i*>(b + j * 32 * PITCH + ks * KSUB + 16);
-          bf[j] = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-        }
-        // E8M0 scale 127 = 2^0 for both operands: plain e4m3 x e4m3.
-        const int one = 0x7f7f7f7f;
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-          for (int j = 0; j < TN; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af[i], bf[j], acc[i][j], 0, 0, 0,
-                                                                        one, 0, one);
-      }
-    }
-    if (kt + 1 < nk) lstore(cur ^ 1);
-    __syncthreads();
+    for (int q = 0; q < NLOADS; ++q) issue_load(st, st, q);
+  AQ_WAIT_VMCNT(2 * NLOADS);  // stage 0 has landed
+  AQ_BARRIER();
+  load_frags(smem, 0, af[0], bf[0]);
+  // sub-steps 0 .. NKS-2 of stage 0 (no loads to issue yet: stages 0..2 are in flight)
+  if constexpr (NKS == 4) {
+    slot(k0{}, smem, 1, no{}, 0, 0, q1{});
+    slot(k1{}, smem, 2, no{}, 0, 0, q2{});
+    slot(k0{}, smem, 3, no{}, 0, 0, q3{});
+  } else {
+    slot(k0{}, smem, 1, no{}, 0, 0, q1{});
   }
+  __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the last fragments of stage 0 are in registers
+  AQ_WAIT_VMCNT(NLOADS);               // stage 1 has landed
+  AQ_BARRIER();
+  // slot A of stage 0: its buffer (0) is free now and takes stage 3
+  slot(k1{}, smem + STAGE, 0, yes{}, NSTAGE, 0, q0{});
+  int b_prev = 0;  // buffer of stage s-1
+  for (int s = 1; s < nk; ++s) {
+    const int b_cur = b_prev == NSTAGE - 1 ? 0 : b_prev + 1;
+    const int b_next = b_cur == NSTAGE - 1 ? 0 : b_cur + 1;
+    const uint8_t* stc = smem + b_cur * STAGE;
+    // sub-steps 0 .. NKS-2 of stage s; the rest of stage s+2's loads go into stage s-1's buffer
+    if constexpr (NKS == 4) {
+      slot(k0{}, stc, 1, yes{}, s - 1 + NSTAGE, b_prev, q1{});
+      slot(k1{}, stc, 2, yes{}, s - 1 + NSTAGE, b_prev, q2{});
+      slot(k0{}, stc, 3, yes{}, s - 1 + NSTAGE, b_prev, q3{});
+    } else {
+      slot(k0{}, stc, 1, yes{}, s - 1 + NSTAGE, b_prev, q1{});
+    }
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the last fragments of stage s are in registers
+    AQ_WAIT_VMCNT(NLOADS);               // stage s+1 has landed (stage s+2 may still be in flight)
+    AQ_BARRIER();
+    // slot A: last sub-step of stage s | first fragments of stage s+1 | first loads of stage s+3
+    slot(k1{}, smem + b_next * STAGE, 0, yes{}, s + NSTAGE, b_cur, q0{});
+    b_prev = b_cur;
+  }
+  AQ_WAIT_VMCNT(0);  // drain the padding loads before the workgroup's LDS can be released
 
-  // ---- epilogue.  32x32 accumulator: register r of lane l holds
-  //      row (r/4)*8 + (l/32)*4 + r%4, column l%32.
-  float sx1 = 1.0f, sw1 = 1.0f;
-  if constexpr (FP8) {
-    sx1 = *p.sx;
-    sw1 = *p.sw;
-  }
+  // ---- epilogue, straight from the accumulator registers (no LDS, no barrier).
+  // A lane owns one output column per 32x32 tile and 64 of the wavefront's 128
+  // rows.  Stores go through a buffer descriptor based at the wavefront's first
+  // output: the lane part of the address (its column, its half of the 8-row
+  // group) is one VGPR computed once, the row part is a scalar offset, so no
+  // vector ALU work is spent on addresses.  Lanes whose column is past N carry
+  // an out-of-range offset and their stores are dropped by the hardware.
+  // bf16 outputs are paired across neighbouring lanes: each lane converts its
+  // two rows (2h, 2h+1) into one packed dword, swaps it with its neighbour
+  // (DPP quad_perm [1,0,3,2]) and byte-permutes the two into "my row, both
+  // columns": even lanes write row 2h, odd lanes row 2h+1, 4 bytes per lane,
+  // 64 contiguous bytes per row segment.
+  constexpr int ESZ = (OUT == OUT_BF16) ? 2 : 4;
+  const int nw = __builtin_amdgcn_readfirstlane(n0 + wave_n * WAVE_N);  // first column of this wavefront
+  const __amdgpu_buffer_rsrc_t Cr =
+      make_rsrc(reinterpret_cast<uint8_t*>(p.C) + ((int64_t)mw * N + nw) * ESZ, 0x40000000u);
+  const bool pair_ok = (N & 1) == 0;  // uniform: bf16 rows start dword-aligned, pairs never straddle N
+  const bool odd = lane & 1;
+  const uint32_t perm_sel = odd ? 0x03020706u : 0x05040100u;
+  const uint32_t rowb = (uint32_t)N * ESZ;
+  const bool rows_inside = mw + WAVE_M <= M;  // uniform
+  // CHECK_M: some rows of this wavefront are past M.  PAIR: the bf16 dword path.
+  auto store_all = [&](auto check_c, auto pair_c) {
+    constexpr bool CHECK_M = decltype(check_c)::value;
+    constexpr bool PAIR = (OUT == OUT_BF16) && decltype(pair_c)::value;
 #pragma unroll
-  for (int j = 0; j < TN; ++j) {
-    const int n = n0 + wave_n * WAVE_N + j * 32 + (lane & 31);
-    const bool n_ok = n < N;
-    float swn = 1.0f, bn = 0.0f;
-    bool has_bias = false;
-    if constexpr (!FP8 && OUT != OUT_I32) {
-      if (n_ok) {
-        swn = p.sw[n];
-        if (p.bias) {
-          has_bias = true;
-          bn = p.bias_dtype == AQ_BF16 ? bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(p.bias)[n])
-                                       : reinterpret_cast<const float*>(p.bias)[n];
-        }
-      }
-    }
+    for (int j = 0; j < TN; ++j) {
+      const int cj = j * 32 + col;  // column inside the wavefront's 64
+      const bool n_ok = nw + cj < N;
+      // lane part of the byte offset; the pairing path stores at the even column of the pair
+      const uint32_t vbase =
+          n_ok ? (uint32_t)rq * rowb + (uint32_t)(PAIR ? (cj & ~1) : cj) * ESZ + (PAIR && odd ? rowb : 0u)
+               : OOB_OFFSET;
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
-      const int mb = m0 + wave_m * WAVE_M + i * 32 + (lane >> 5) * 4;
+      for (int i = 0; i < TM; ++i) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int m = mb + (r >> 2) * 8 + (r & 3);
-        if (m < M && n_ok) {
-          const int64_t o = (int64_t)m * N + n;
+        for (int g = 0; g < 4; ++g) {
+          const int r0 = i * 32 + g * 8;  // + rq + q : row inside the wavefront's 128
           if constexpr (OUT == OUT_I32) {
-            reinterpret_cast<int32_t*>(p.C)[o] = acc[i][j][r];
-          } else {
-            float y;
-            if constexpr (FP8) {
-              y = __fmul_rn(__fmul_rn(acc[i][j][r], sx1), sw1);
-            } else {
-              // three separately rounded fp32 operations, never contracted
-              y = __fmul_rn(__fmul_rn((float)acc[i][j][r], p.sx[m]), swn);
-              if (has_bias) y = __fadd_rn(y, bn);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              uint32_t vo = vbase;
+              if (CHECK_M && mw + r0 + rq + q >= M) vo = OOB_OFFSET;
+              __builtin_amdgcn_raw_buffer_store_b32((uint32_t)acc[i][j][g * 4 + q], Cr, vo, (r0 + q) * rowb, 0);
             }
-            if constexpr (OUT == OUT_F32)
-              reinterpret_cast<float*>(p.C)[o] = y;
-            else
-              reinterpret_cast<uint16_t*>(p.C)[o] = (uint16_t)f32_to_bf16_bits(y);
+          } else {
+            float y[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              if constexpr (FP8) {
+                y[q] = __fmul_rn(__fmul_rn(acc[i][j][g * 4 + q], sx1), sw1);
+              } else {
+                // three separately rounded fp32 operations, never contracted.  Without a bias
+                // bn is +0: the product of an integer and two positive scales is never -0,
+                // so adding it changes no bit.
+                y[q] = __fadd_rn(__fmul_rn(__fmul_rn((float)acc[i][j][g * 4 + q], sxr[i][g][q]), swn[j]), bn[j]);
+              }
+            }
+            if constexpr (OUT == OUT_F32) {
+#pragma unroll
+              for (int q = 0; q < 4; ++q) {
+                uint32_t vo = vbase;
+                if (CHECK_M && mw + r0 + rq + q >= M) vo = OOB_OFFSET;
+                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(y[q]), Cr, vo, (r0 + q) * rowb, 0);
+              }
+            } else if constexpr (PAIR) {
+#pragma unroll
+              for (int h = 0; h < 2; ++h) {
+                const uint32_t mine = pack_bf16x2(y[2 * h], y[2 * h + 1]);  // lo: row 2h, hi: row 2h+1
+                const uint32_t other =
+                    (uint32_t)__builtin_amdgcn_mov_dpp((int)mine, 0xB1 /* quad_perm [1,0,3,2] */, 0xf, 0xf, true);
+                // even lane: {mine.lo, other.lo} = row 2h, columns (c, c+1)
+                // odd lane:  {other.hi, mine.hi} = row 2h+1, columns (c-1, c)
+                const uint32_t pk = __builtin_amdgcn_perm(other, mine, perm_sel);
+                uint32_t vo = vbase;
+                if (CHECK_M && mw + r0 + rq + 2 * h + (odd ? 1 : 0) >= M) vo = OOB_OFFSET;
+                __builtin_amdgcn_raw_buffer_store_b32(pk, Cr, vo, (r0 + 2 * h) * rowb, 0);
+              }
+            } else {
+#pragma unroll
+              for (int q = 0; q < 4; ++q) {
+                uint32_t vo = vbase;
+                if (CHECK_M && mw + r0 + rq + q >= M) vo = OOB_OFFSET;
+                __builtin_amdgcn_raw_buffer_store_b16((uint16_t)f32_to_bf16_bits(y[q]), Cr, vo, (r0 + q) * rowb, 0);
+              }
+            }
           }
         }
       }
     }
-  }
+  };
+  if (rows_inside && pair_ok)
+    store_all(no{}, yes{});   // interior tiles: straight-line, no per-row checks
+  else if (pair_ok)
+    store_all(yes{}, yes{});
+  else
+    store_all(yes{}, no{});
 }
 
 template <bool FP8, int OUT>
 static int launch(const GemmArgs& a, hipStream_t st) {
   const unsigned grid = (unsigned)(a.tiles_m * a.tiles_n);
-  hipLaunchKernelGGL((gemm_kernel<FP8, OUT>), dim3(grid), dim3(256), 0, st, a);
+  hipLaunchKernelGGL((gemm_kernel<FP8, OUT>), dim3(grid), dim3(NTHREADS), 0, st, a);
   return (int)hipGetLastError();
 }
 

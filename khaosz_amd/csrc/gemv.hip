@@ -1,37 +1,65 @@
 // Decode path (M <= 16 tokens): a weight-streaming int8 GEMV.  The weight
 // matrix is read exactly once with 16-byte loads, one wavefront reading 1 KiB
 // contiguous of a row per instruction; the few activation rows are quantised
-// by the row-wise kernel into the caller's workspace, copied to LDS and reused
-// by every row of W.  Products are v_dot4_i32_i8 (no MFMA tiles, no LDS
-// staging of W); a wavefront reduces its 4 x MT partial sums with a transposed
-// butterfly so that each lane ends up owning one output, then applies the same
-// dequantising epilogue as the MFMA GEMM.  The int32 sums are exact, so the
-// result is bit-identical to quantise + GEMM.
+// by the row-wise kernel into the caller's workspace, pulled into LDS once per
+// workgroup by direct global->LDS loads and reused by every row of W.
+// Products are v_dot4_i32_i8 (no MFMA tiles, no LDS staging of W); a wavefront
+// reduces its 4 x MT partial sums with a transposed butterfly so that each
+// lane ends up owning one output, then applies the same dequantising epilogue
+// as the MFMA GEMM.  The int32 sums are exact, so the result is bit-identical
+// to quantise + GEMM.
+//
+// Every byte the kernel will need is requested before anything is waited for:
+// a wavefront first issues its share of the activation copy, then the weight
+// loads of its first two K chunks, and only then waits for the activations.
+#include <type_traits>
+
 #include "aq_common.h"
 
 namespace aq {
 
-constexpr int GV_ROWS = 4;        // weight rows per wavefront pass
-constexpr int GV_WAVES = 4;       // wavefronts per workgroup
-constexpr int GV_CHUNK = 64 * 16; // K bytes one wavefront covers per load
+#ifndef AQ_GV_ROWS
+#define AQ_GV_ROWS 4
+#endif
+#ifndef AQ_GV_WAVES
+#define AQ_GV_WAVES 8
+#endif
+constexpr int GV_ROWS = AQ_GV_ROWS;    // weight rows per wavefront pass
+constexpr int GV_WAVES = AQ_GV_WAVES;  // wavefronts per workgroup
+constexpr int GV_THREADS = GV_WAVES * 64;
+constexpr int GV_CHUNK = 64 * 16;  // K bytes one wavefront covers per load
+constexpr int GV_DEPTH = 2;        // weight chunks in flight per wavefront
 
-// Reduce V values per lane across the 64 lanes.  While more than one value is
-// live, partners exchange halves (reduce-scatter); afterwards plain butterfly
-// adds.  On return v[0] of lane l is the full sum of value index
-// l >> (6 - log2 V).
+typedef __attribute__((address_space(3))) void gv_lds_void;
+typedef unsigned gv_u2 __attribute__((ext_vector_type(2)));
+
+// Reduce V values per lane across the 64 lanes so that afterwards v[0] of lane
+// l holds the full sum of value index l >> (6 - log2 V) (for V <= 64).
+// Lane-bit 5 and 4 stages use the gfx950 half/row swaps: one swap exchanges the
+// two halves a pair of values needs, one add finishes it.  The remaining
+// stages (at most 15 live values for V = 64) use cross-lane shuffles.
 template <int CUR, int OFF>
 struct Butterfly {
   template <int V>
   __device__ static __forceinline__ void run(int (&v)[V], int lane) {
     if constexpr (CUR > 1) {
       constexpr int H = CUR / 2;
-      const bool up = (lane & OFF) != 0;
+      if constexpr (OFF == 32 || OFF == 16) {
 #pragma unroll
-      for (int i = 0; i < H; ++i) {
-        const int lo = v[i], hi = v[i + H];
-        const int send = up ? lo : hi;
-        const int keep = up ? hi : lo;
-        v[i] = keep + __shfl_xor(send, OFF, AQ_WAVE);
+        for (int i = 0; i < H; ++i) {
+          const gv_u2 r = OFF == 32 ? __builtin_amdgcn_permlane32_swap((unsigned)v[i], (unsigned)v[i + H], false, false)
+                                    : __builtin_amdgcn_permlane16_swap((unsigned)v[i], (unsigned)v[i + H], false, false);
+          v[i] = (int)(r.x + r.y);
+        }
+      } else {
+        const bool up = (lane & OFF) != 0;
+#pragma unroll
+        for (int i = 0; i < H; ++i) {
+          const int lo = v[i], hi = v[i + H];
+          const int send = up ? lo : hi;
+          const int keep = up ? hi : lo;
+          v[i] = keep + __shfl_xor(send, OFF, AQ_WAVE);
+        }
       }
       if constexpr (OFF > 1) Butterfly<H, OFF / 2>::run(v, lane);
     } else {
@@ -54,22 +82,55 @@ struct GemvArgs {
   int bias_dtype, y_dtype;
 };
 
+#define GV_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(0x0f70 | ((n) & 15) | (((n) >> 4) << 14))
+
 template <int MT>
-__global__ __launch_bounds__(GV_WAVES * 64) void gemv_w8a8_kernel(GemvArgs p) {
-  extern __shared__ __attribute__((aligned(16))) uint8_t xs[];  // [MT][K]
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+__global__ __launch_bounds__(GV_THREADS) void gemv_w8a8_kernel(GemvArgs p) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t xs[];  // [MT][K] activation codes
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int K = p.K, N = p.N, M = p.M;
-  // wavefront-uniform first row, made scalar so the buffer descriptor lives in SGPRs
+  // wavefront-uniform first row, kept scalar so the buffer descriptor lives in SGPRs
   const int n0 = __builtin_amdgcn_readfirstlane((blockIdx.x * GV_WAVES + wave) * GV_ROWS);
 
-  // Issue the first weight loads before anything else: they are the long pole.
-  // The descriptor spans this wavefront's rows only; rows past N and bytes
-  // past K fall outside it and read as zero.
+  // 0. After the reduction lane l owns output (row n0 + idx / MT, token idx % MT)
+  // with idx = l >> (6 - log2(rows * MT)).  Its scales and bias are requested
+  // now, ahead of everything else, so the epilogue never waits on memory.
+  constexpr int V = GV_ROWS * MT;
+  constexpr int SH = 6 - ilog2(V);
+  static_assert(V <= 64, "one output per lane at most");
+  const int oidx = lane >> SH;
+  const int om = oidx % MT, on = n0 + oidx / MT;
+  const bool out_lane = (lane & ((1 << SH) - 1)) == 0 && om < M && on < N;
+  float sxv = 0.0f, swv = 0.0f, bv = 0.0f;
+  if (out_lane) {
+    sxv = p.sx[om];
+    swv = p.sw[on];
+    if (p.bias)
+      bv = p.bias_dtype == AQ_BF16 ? bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(p.bias)[on])
+                                   : reinterpret_cast<const float*>(p.bias)[on];
+  }
+
+  // 1. activation codes -> LDS, 16 bytes per lane, straight from global memory.
+  // Rows m >= M lie outside the descriptor and arrive as zeros.
+  const __amdgpu_buffer_rsrc_t Xr = make_rsrc(p.xq, (uint32_t)M * (uint32_t)K);
+  const int xbytes = MT * K;
+  const int xrounds = (xbytes + GV_THREADS * 16 - 1) / (GV_THREADS * 16);
+  for (int r = 0; r < xrounds; ++r) {
+    const int base = (r * GV_WAVES + wave) * 1024;  // this wavefront's 1 KiB of the copy
+    if (base < xbytes)  // uniform; xbytes is a multiple of 16 but not always of 1024:
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(Xr, (gv_lds_void*)(xs + base), 16,
+                                               (base + lane * 16) < xbytes ? (uint32_t)(base + lane * 16) : OOB_OFFSET,
+                                               0, 0, 0);
+  }
+
+  // 2. the first GV_DEPTH weight chunks of this wavefront's rows.  The
+  // descriptor spans these rows only; rows past N and bytes past K fall
+  // outside it and read as zero.
   const int nchunk = (K + GV_CHUNK - 1) / GV_CHUNK;
   const int rows = n0 < N ? ((N - n0) < GV_ROWS ? (N - n0) : GV_ROWS) : 0;
   const __amdgpu_buffer_rsrc_t Wr =
       make_rsrc(p.wq + (int64_t)(n0 < N ? n0 : 0) * K, (uint32_t)rows * (uint32_t)K);
-  const uint4 zero = make_uint4(0, 0, 0, 0);
   auto wload = [&](int c, uint4 (&dst)[GV_ROWS]) {
     const int kb = c * GV_CHUNK + lane * 16;
     const bool ok = kb < K;  // past K the offset would alias the next row
@@ -77,65 +138,68 @@ __global__ __launch_bounds__(GV_WAVES * 64) void gemv_w8a8_kernel(GemvArgs p) {
     for (int r = 0; r < GV_ROWS; ++r)
       dst[r] = buffer_load_16(Wr, ok ? (uint32_t)r * (uint32_t)K + (uint32_t)kb : OOB_OFFSET);
   };
-  uint4 w[GV_ROWS];
-  wload(0, w);
+  uint4 w[GV_DEPTH][GV_ROWS];
+#pragma unroll
+  for (int d = 0; d < GV_DEPTH; ++d) wload(d, w[d]);  // chunks past the end read zeros
 
-  // activation codes -> LDS, rows >= M zero
-  const int nvec_row = K / 16;
-  for (int v = tid; v < MT * nvec_row; v += GV_WAVES * 64) {
-    const int m = v / nvec_row;
-    uint4 val = zero;
-    if (m < M) val = reinterpret_cast<const uint4*>(p.xq)[v];
-    reinterpret_cast<uint4*>(xs)[v] = val;
-  }
-  __syncthreads();
+  // 3. the activation copy is older than the weight loads: wait until at most
+  // those are outstanding, then make every wavefront's part visible.
+  GV_WAIT_VMCNT(GV_DEPTH * GV_ROWS);
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
 
   int acc[GV_ROWS * MT];
 #pragma unroll
   for (int i = 0; i < GV_ROWS * MT; ++i) acc[i] = 0;
 
-  for (int c = 0; c < nchunk; ++c) {
+  auto consume = [&](int c, const uint4 (&wc)[GV_ROWS]) {
     const int kb = c * GV_CHUNK + lane * 16;
-    uint4 wn[GV_ROWS];
-    if (c + 1 < nchunk) {
-      wload(c + 1, wn);
-    } else {
-#pragma unroll
-      for (int r = 0; r < GV_ROWS; ++r) wn[r] = zero;
-    }
     const int kx = kb < K ? kb : 0;  // lanes past the end multiply zeros; keep the LDS read in range
+    // activation rows in blocks of 4: four LDS reads in flight cover the 64 dot
+    // products of the previous block without holding all MT rows in registers
+    constexpr int MB = MT < 4 ? MT : 4;
 #pragma unroll
-    for (int m = 0; m < MT; ++m) {
-      const uint4 x = *reinterpret_cast<const uint4*>(xs + m * K + kx);
+    for (int m0 = 0; m0 < MT; m0 += MB) {
+      uint4 x[MB];
 #pragma unroll
-      for (int r = 0; r < GV_ROWS; ++r) {
-        int a = acc[r * MT + m];
-        a = __builtin_amdgcn_sdot4((int)w[r].x, (int)x.x, a, false);
-        a = __builtin_amdgcn_sdot4((int)w[r].y, (int)x.y, a, false);
-        a = __builtin_amdgcn_sdot4((int)w[r].z, (int)x.z, a, false);
-        a = __builtin_amdgcn_sdot4((int)w[r].w, (int)x.w, a, false);
-        acc[r * MT + m] = a;
+      for (int i = 0; i < MB; ++i) x[i] = *reinterpret_cast<const uint4*>(xs + (m0 + i) * K + kx);
+#pragma unroll
+      for (int i = 0; i < MB; ++i) {
+#pragma unroll
+        for (int r = 0; r < GV_ROWS; ++r) {
+          int a = acc[r * MT + m0 + i];
+          a = __builtin_amdgcn_sdot4((int)wc[r].x, (int)x[i].x, a, false);
+          a = __builtin_amdgcn_sdot4((int)wc[r].y, (int)x[i].y, a, false);
+          a = __builtin_amdgcn_sdot4((int)wc[r].z, (int)x[i].z, a, false);
+          a = __builtin_amdgcn_sdot4((int)wc[r].w, (int)x[i].w, a, false);
+          acc[r * MT + m0 + i] = a;
+        }
       }
+      if constexpr (MT > 8) __builtin_amdgcn_sched_barrier(0);
     }
-#pragma unroll
-    for (int r = 0; r < GV_ROWS; ++r) w[r] = wn[r];
+  };
+  // K loop.  Rows of up to 2 KiB (the common decode shapes) are two chunks that
+  // are already in flight: no loop.  Longer rows rotate two register buffers.
+  static_assert(GV_DEPTH == 2, "the K loop below rotates exactly two buffers");
+  consume(0, w[0]);
+  if (nchunk > 2) wload(2, w[0]);
+  __builtin_amdgcn_sched_barrier(0);
+  if (nchunk > 1) consume(1, w[1]);
+  for (int c = 2; c < nchunk; c += 2) {
+    if (c + 1 < nchunk) wload(c + 1, w[1]);
+    __builtin_amdgcn_sched_barrier(0);
+    consume(c, w[0]);
+    if (c + 2 < nchunk) wload(c + 2, w[0]);
+    __builtin_amdgcn_sched_barrier(0);
+    if (c + 1 < nchunk) consume(c + 1, w[1]);
   }
 
-  constexpr int V = GV_ROWS * MT;
   Butterfly<V, 32>::run(acc, lane);
-  constexpr int SH = 6 - ilog2(V);
-  if ((lane & ((1 << SH) - 1)) != 0) return;
-  const int idx = lane >> SH;
-  const int r = idx / MT, m = idx % MT;
-  const int n = n0 + r;
-  if (m >= M || n >= N) return;
-  float y = __fmul_rn(__fmul_rn((float)acc[0], p.sx[m]), p.sw[n]);
-  if (p.bias) {
-    const float b = p.bias_dtype == AQ_BF16 ? bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(p.bias)[n])
-                                            : reinterpret_cast<const float*>(p.bias)[n];
-    y = __fadd_rn(y, b);
-  }
-  const int64_t o = (int64_t)m * N + n;
+  if (!out_lane) return;
+  float y = __fmul_rn(__fmul_rn((float)acc[0], sxv), swv);
+  if (p.bias) y = __fadd_rn(y, bv);
+  const int64_t o = (int64_t)om * N + on;
   if (p.y_dtype == AQ_BF16)
     reinterpret_cast<uint16_t*>(p.y)[o] = (uint16_t)f32_to_bf16_bits(y);
   else
@@ -151,11 +215,197 @@ static int launch_gemv(const GemvArgs& a, hipStream_t st) {
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return (int)e;
   }
-  hipLaunchKernelGGL((gemv_w8a8_kernel<MT>), dim3(grid), dim3(GV_WAVES * 64), lds, st, a);
+  hipLaunchKernelGGL((gemv_w8a8_kernel<MT>), dim3(grid), dim3(GV_THREADS), lds, st, a);
   return (int)hipGetLastError();
 }
 
 constexpr int64_t GV_MAX_LDS = 160 * 1024;  // LDS of one gfx950 CU
+#ifndef AQ_GV_MFMA_MIN_M
+#define AQ_GV_MFMA_MIN_M 8
+#endif
+constexpr int GV_MFMA_MIN_M = AQ_GV_MFMA_MIN_M;  // more tokens than this take the matrix-core variant
+
+// ---------------------------------------------------------------------------
+// Streaming variant for 5..16 tokens.  With that many tokens the 16 dot
+// products every weight dword needs make the vector ALU, not HBM, the limit
+// of the kernel above.  This one keeps its structure -- every weight byte goes
+// HBM -> registers exactly once, no LDS staging or macro-tiling of W -- but
+// hands the products to the matrix core: a wavefront owns 16 weight rows, loads
+// them 16 bytes per lane directly in the v_mfma_i32_16x16x64_i8 operand order
+// (lane l: row l%16, K bytes 64j + 16*(l/16) .. +16 of step j, so the four
+// lanes of a row cover 64 contiguous bytes and two consecutive steps consume
+// whole 128-byte lines), and multiplies against the token codes held in LDS.
+// The 16 x 16 result has rows = weight rows and columns = tokens, so a lane
+// ends up with 4 consecutive outputs of one token: no cross-lane reduction.
+// Two wavefronts share a row group, each taking half of K; the halves are
+// summed through LDS (exact int32).
+constexpr int GM_ROWS = 16;    // weight rows per wavefront
+constexpr int GM_KSPLIT = 2;   // wavefronts sharing a row group
+constexpr int GM_GROUPS = 2;   // row groups per workgroup
+constexpr int GM_WAVES = GM_KSPLIT * GM_GROUPS;
+constexpr int GM_BATCH = 8;    // MFMA steps (64 K bytes each) per register batch
+
+__global__ __launch_bounds__(GM_WAVES * 64) void gemv_mfma_kernel(GemvArgs p) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t xs[];  // [16][K + 16] token codes, then the partial sums
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int grp = wave / GM_KSPLIT, kh = wave % GM_KSPLIT;
+  const int K = p.K, N = p.N, M = p.M;
+  const int n0 = __builtin_amdgcn_readfirstlane((blockIdx.x * GM_GROUPS + grp) * GM_ROWS);
+  const int pitch = K + 16;  // 16 token rows then start 4 banks apart: conflict-free 16-byte reads
+  const int khalf = K / GM_KSPLIT;  // a multiple of 64 (checked by the launcher)
+  const int nstep = khalf / 64;
+
+  // epilogue operands first: lane l -> token l%16, rows (l/16)*4 .. +3 of the group
+  const int tok = lane & 15;
+  const int rbase = n0 + (lane >> 4) * 4;
+  float sxv = 0.0f, swv[4], bv[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    swv[r] = 0.0f;
+    bv[r] = 0.0f;
+  }
+  if (kh == 0) {  // uniform: only the first half's wavefront writes outputs
+    if (tok < M) sxv = p.sx[tok];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int n = rbase + r < N ? rbase + r : N - 1;
+      swv[r] = p.sw[n];
+      if (p.bias)
+        bv[r] = p.bias_dtype == AQ_BF16 ? bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(p.bias)[n])
+                                        : reinterpret_cast<const float*>(p.bias)[n];
+    }
+  }
+
+  // weight stream: descriptor over this wavefront's 16 rows; rows past N read as zero
+  const int rows = n0 < N ? ((N - n0) < GM_ROWS ? (N - n0) : GM_ROWS) : 0;
+  const __amdgpu_buffer_rsrc_t Wr =
+      make_rsrc(p.wq + (int64_t)(n0 < N ? n0 : 0) * K, (uint32_t)rows * (uint32_t)K);
+  const uint32_t woff = (uint32_t)(lane & 15) * (uint32_t)K + (uint32_t)(kh * khalf + (lane >> 4) * 16);
+  uint4 wa[GM_BATCH], wb[GM_BATCH];
+  auto wload = [&](int step0, uint4 (&dst)[GM_BATCH]) {
+#pragma unroll
+    for (int j = 0; j < GM_BATCH; ++j)
+      dst[j] = buffer_load_16(Wr, (step0 + j) < nstep ? woff + (uint32_t)(step0 + j) * 64u : OOB_OFFSET);
+  };
+
+  // token codes -> LDS (padded rows; tokens >= M lie outside the descriptor and arrive as zeros).
+  // Their loads are issued before the weight loads, so they return first and the
+  // LDS fill overlaps the weight stream's flight time.
+  const __amdgpu_buffer_rsrc_t Xr = make_rsrc(p.xq, (uint32_t)M * (uint32_t)K);
+  const int nvec_row = K / 16;
+  const int nvec = 16 * nvec_row;
+  constexpr int XV = 8;  // vectors per thread per round: 16 x 2048 codes in one round of 256 threads
+  uint4 xv[XV];
+  auto xload = [&](int v0) {
+#pragma unroll
+    for (int i = 0; i < XV; ++i) {
+      const int v = v0 + i * (GM_WAVES * 64) + tid;
+      xv[i] = buffer_load_16(Xr, v < nvec ? (uint32_t)v * 16u : OOB_OFFSET);
+    }
+  };
+  auto xstore = [&](int v0) {
+#pragma unroll
+    for (int i = 0; i < XV; ++i) {
+      const int v = v0 + i * (GM_WAVES * 64) + tid;
+      if (v < nvec) {
+        const int m = v / nvec_row, c = v - m * nvec_row;
+        *reinterpret_cast<uint4*>(xs + m * pitch + c * 16) = xv[i];
+      }
+    }
+  };
+  xload(0);
+  wload(0, wa);
+  wload(GM_BATCH, wb);
+  xstore(0);
+  for (int v0 = XV * GM_WAVES * 64; v0 < nvec; v0 += XV * GM_WAVES * 64) {  // rows longer than 2048
+    xload(v0);
+    xstore(v0);
+  }
+  // LDS writes done, then a barrier without a memory fence: the weight loads stay in flight
+  __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+
+  v4i acc = {0, 0, 0, 0};
+  const uint8_t* xl = xs + tok * pitch + kh * khalf + (lane >> 4) * 16;
+  auto consume = [&](int step0, const uint4 (&wc)[GM_BATCH]) {
+#pragma unroll
+    for (int j = 0; j < GM_BATCH; ++j) {
+      const int st = (step0 + j) < nstep ? (step0 + j) : 0;  // steps past the end multiply zero weights
+      const v4i x = *reinterpret_cast<const v4i*>(xl + st * 64);
+      const v4i wv = {(int)wc[j].x, (int)wc[j].y, (int)wc[j].z, (int)wc[j].w};
+      acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(wv, x, acc, 0, 0, 0);
+    }
+  };
+  for (int s0 = 0; s0 < nstep; s0 += 2 * GM_BATCH) {
+    consume(s0, wa);
+    if (s0 + 2 * GM_BATCH < nstep) wload(s0 + 2 * GM_BATCH, wa);
+    if (s0 + GM_BATCH < nstep) consume(s0 + GM_BATCH, wb);
+    if (s0 + 3 * GM_BATCH < nstep) wload(s0 + 3 * GM_BATCH, wb);
+  }
+
+  // sum the K halves: the second wavefront of each group parks its 4 sums in LDS
+  __syncthreads();  // everyone is done reading the token codes: the buffer is reused
+  int* part = reinterpret_cast<int*>(xs) + grp * 256;
+  if (kh != 0) {
+    *reinterpret_cast<v4i*>(part + lane * 4) = acc;
+  }
+  __syncthreads();
+  if (kh != 0) return;
+  const v4i other = *reinterpret_cast<const v4i*>(part + lane * 4);
+  acc += other;
+
+  if (tok >= M) return;
+  float y[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    y[r] = __fmul_rn(__fmul_rn((float)acc[r], sxv), swv[r]);
+    if (p.bias) y[r] = __fadd_rn(y[r], bv[r]);
+  }
+  const int64_t o = (int64_t)tok * N + rbase;
+  if (p.y_dtype == AQ_BF16) {
+    uint16_t* dst = reinterpret_cast<uint16_t*>(p.y) + o;
+    if ((N & 3) == 0 && rbase + 3 < N) {  // 8-byte aligned and fully inside
+      uint2 pk;
+      pk.x = pack_bf16x2(y[0], y[1]);
+      pk.y = pack_bf16x2(y[2], y[3]);
+      *reinterpret_cast<uint2*>(dst) = pk;
+    } else {
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (rbase + r < N) dst[r] = (uint16_t)f32_to_bf16_bits(y[r]);
+    }
+  } else {
+    float* dst = reinterpret_cast<float*>(p.y) + o;
+    if ((N & 3) == 0 && rbase + 3 < N) {
+      *reinterpret_cast<float4*>(dst) = make_float4(y[0], y[1], y[2], y[3]);
+    } else {
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (rbase + r < N) dst[r] = y[r];
+    }
+  }
+}
+
+static int launch_gemv_mfma(const GemvArgs& a, hipStream_t st) {
+  const unsigned grid = (unsigned)((a.N + GM_ROWS * GM_GROUPS - 1) / (GM_ROWS * GM_GROUPS));
+  const size_t lds = (size_t)16 * (a.K + 16);
+  if (lds > 64 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_mfma_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return (int)e;
+  }
+  hipLaunchKernelGGL(gemv_mfma_kernel, dim3(grid), dim3(GM_WAVES * 64), lds, st, a);
+  return (int)hipGetLastError();
+}
+
+// the streaming MFMA variant needs each K half to be whole 64-byte steps and its padded codes to fit LDS
+static bool gemv_mfma_ok(int64_t M, int64_t K) {
+  return M > GV_MFMA_MIN_M && (K % (64 * GM_KSPLIT)) == 0 && 16 * (K + 16) <= GV_MAX_LDS;
+}
+
 
 static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
@@ -182,6 +432,7 @@ static int gemv_check(const int8_t* wq, const float* sw, const void* bias, int b
 }
 
 static int gemv_dispatch(const aq::GemvArgs& a, int mt, hipStream_t st) {
+  if (aq::gemv_mfma_ok(a.M, a.K)) return aq::launch_gemv_mfma(a, st);
   switch (mt) {
     case 1: return aq::launch_gemv<1>(a, st);
     case 2: return aq::launch_gemv<2>(a, st);

@@ -40,23 +40,72 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
   return *reinterpret_cast<const uint32_t*>(&b);
 }
 
+// Maximum of a non-negative value over the 64 lanes, returned in every lane
+// (as a wavefront-uniform scalar).  Four DPP steps (quad swaps, then the
+// half-row and row mirrors) leave each row of 16 lanes holding its maximum;
+// the four row results are read out and combined on the scalar unit, where
+// non-negative floats order like their bit patterns.
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int off = 32; off >= 1; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, AQ_WAVE));
-  return v;
+  int x = __float_as_int(v);
+#define AQ_DPP_MAX(ctrl)                                                                      \
+  x = __float_as_int(fmaxf(__int_as_float(x),                                                 \
+                           __int_as_float(__builtin_amdgcn_update_dpp(x, x, ctrl, 0xf, 0xf, false))))
+  AQ_DPP_MAX(0xB1);   // quad_perm [1,0,3,2]
+  AQ_DPP_MAX(0x4E);   // quad_perm [2,3,0,1]
+  AQ_DPP_MAX(0x141);  // row_half_mirror
+  AQ_DPP_MAX(0x140);  // row_mirror
+#undef AQ_DPP_MAX
+  const uint32_t a = (uint32_t)__builtin_amdgcn_readlane(x, 0), b = (uint32_t)__builtin_amdgcn_readlane(x, 16);
+  const uint32_t c = (uint32_t)__builtin_amdgcn_readlane(x, 32), d = (uint32_t)__builtin_amdgcn_readlane(x, 48);
+  const uint32_t ab = a > b ? a : b, cd = c > d ? c : d;
+  return __uint_as_float(ab > cd ? ab : cd);
 }
 
-// q = clamp(rint(a / s), -127, 127) with a correctly rounded divide.
-// Fast path: a * (1/s) is within 127 * 3 ulp of the true quotient, so whenever
-// it is further than 2^-6 from a rounding boundary the rounded integer is
-// already decided; only the rare near-tie lanes pay for the IEEE divide.
-__device__ __forceinline__ int quant_code(float a, float s, float rs) {
-  float t = a * rs;
-  float n = rintf(t);
-  float d = fabsf(t - n);
-  if (__builtin_expect(!(d <= 0.484375f), 0)) n = rintf(__fdiv_rn(a, s));  // also taken for inf/NaN
+// Exact definition: q = clamp(rint(a / s), -127, 127), correctly rounded divide,
+// round-half-to-even.  Returned as a 32-bit pattern whose low byte is the code.
+__device__ __forceinline__ uint32_t quant_code_exact(float a, float s) {
+  float n = rintf(__fdiv_rn(a, s));
   n = fminf(fmaxf(n, -127.0f), 127.0f);
-  return (int)n;
+  return (uint32_t)(int)n;
+}
+
+// The same codes for N values of one row at a fraction of the instructions.
+// With rs = rcp(s) (1 ulp) the exact product a * rs is within
+// 127.5 * 2^-23 = 1.5e-5 of the true quotient Q = a / s, whose own correctly
+// rounded value fl(Q) is within another 7.6e-6.  One fused multiply-add with
+// the constant 1.5 * 2^23 rounds a * rs to the nearest-even integer n and leaves
+// it in the low mantissa bits (so the low byte of the float IS the
+// two's-complement code); a second one gives the residual r = a * rs - n.
+// |a| never exceeds the row's amax = 127 s, so no clamp is needed.  Unless |r|
+// is within 2^-14 = 6.1e-5 of one half, rint(fl(Q)) = n.  A group in which some
+// value is that close is redone with the exact definition; with bf16 inputs
+// exact ties such as a = amax / 2 are common (one value in 400), so about half
+// of all 512-value groups take that path, and it is taken per group rather
+// than per value because a branch per value costs more than the divides it
+// saves.  `fast_ok` must be false for rows whose scale is not a normal float
+// (rcp is then useless).
+template <int N>
+__device__ __forceinline__ void quant_codes(const float* a, float s, float rs, bool fast_ok, uint32_t* out) {
+  const float magic = 12582912.0f;          // 1.5 * 2^23
+  const float decided = 0.49993896484375f;  // 0.5 - 2^-14
+  float dmax = 0.0f;
+#pragma unroll
+  for (int i = 0; i < N; ++i) {
+    const float um = __builtin_fmaf(a[i], rs, magic);
+    out[i] = __float_as_uint(um);
+    dmax = fmaxf(dmax, fabsf(__builtin_fmaf(a[i], rs, -(um - magic))));
+  }
+  if (__builtin_expect(!fast_ok || !(dmax <= decided), 0)) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) out[i] = quant_code_exact(a[i], s);
+  }
+}
+
+// low bytes of four 32-bit patterns -> one dword (a in bits 7:0 .. d in bits 31:24)
+__device__ __forceinline__ uint32_t pack_low_bytes(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
+  const uint32_t ab = __builtin_amdgcn_perm(b, a, 0x0c0c0400u);  // {a.b0, b.b0, 0, 0}
+  const uint32_t cd = __builtin_amdgcn_perm(d, c, 0x0c0c0400u);
+  return __builtin_amdgcn_perm(cd, ab, 0x05040100u);             // {ab.b0, ab.b1, cd.b0, cd.b1}
 }
 
 // Raw buffer descriptor over [base, base + bytes): loads whose byte offset

@@ -43,73 +43,155 @@ __device__ __forceinline__ float vec_amax(const float* f) {
   return m;
 }
 
-__device__ __forceinline__ uint32_t pack4(int a, int b, int c, int d) {
-  return (uint32_t)(a & 0xff) | ((uint32_t)(b & 0xff) << 8) | ((uint32_t)(c & 0xff) << 16) |
-         ((uint32_t)(d & 0xff) << 24);
-}
-
 template <bool BF16>
-__device__ __forceinline__ void quant_store(const uint4& v, float s, float rs, int8_t* dst) {
-  float f[RowIn<BF16>::EPV];
+__device__ __forceinline__ void quant_store(const uint4& v, float s, float rs, bool fast_ok, int8_t* dst) {
+  constexpr int EPV = RowIn<BF16>::EPV;
+  float f[EPV];
+  uint32_t c[EPV];
   RowIn<BF16>::unpack(v, f);
+  quant_codes<EPV>(f, s, rs, fast_ok, c);
   if constexpr (BF16) {
     uint2 o;
-    o.x = pack4(quant_code(f[0], s, rs), quant_code(f[1], s, rs), quant_code(f[2], s, rs),
-                quant_code(f[3], s, rs));
-    o.y = pack4(quant_code(f[4], s, rs), quant_code(f[5], s, rs), quant_code(f[6], s, rs),
-                quant_code(f[7], s, rs));
+    o.x = pack_low_bytes(c[0], c[1], c[2], c[3]);
+    o.y = pack_low_bytes(c[4], c[5], c[6], c[7]);
     *reinterpret_cast<uint2*>(dst) = o;
   } else {
-    *reinterpret_cast<uint32_t*>(dst) = pack4(quant_code(f[0], s, rs), quant_code(f[1], s, rs),
-                                              quant_code(f[2], s, rs), quant_code(f[3], s, rs));
+    *reinterpret_cast<uint32_t*>(dst) = pack_low_bytes(c[0], c[1], c[2], c[3]);
   }
 }
 
-// One wavefront per row.  The first NC vectors of the lane stay in registers
-// between the absmax pass and the rounding pass; longer rows are re-read
-// (from L2) for the part that does not fit.
-template <bool BF16, int NC>
+// One wavefront per row at a time.  The first NC vectors of the lane stay in
+// registers between the absmax pass and the rounding pass; longer rows are
+// re-read (from L2) for the part that does not fit.  A wavefront walks rows
+// row0, row0 + stride, ... and, when PREFETCH, requests the next row's vectors
+// before it reduces, rounds and stores the current one, so that the reads of
+// one row overlap the arithmetic and the writes of another (all wavefronts of a
+// one-row-per-wavefront launch start together and would otherwise read, then
+// compute, then write in lockstep).
+template <bool BF16, int NC, bool PREFETCH, bool FULL>
 __global__ __launch_bounds__(256) void quant_rowwise_i8_kernel(const void* __restrict__ x, int64_t M,
                                                                  int K, int64_t ldx,
                                                                  int8_t* __restrict__ q,
                                                                  float* __restrict__ scale) {
   constexpr int EPV = RowIn<BF16>::EPV;
   const int lane = threadIdx.x & 63;
-  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int64_t stride = (int64_t)gridDim.x * 4;
+  int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= M) return;
   const int nvec = K / EPV;  // 16-byte vectors per row
+  auto row_src = [&](int64_t r) {
+    return reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(x) + r * ldx * (BF16 ? 2 : 4));
+  };
+  auto load_cache = [&](int64_t r, uint4 (&c)[NC]) {
+    const uint4* src = row_src(r);
+#pragma unroll
+    for (int i = 0; i < NC; ++i) {
+      const int v = i * 64 + lane;
+      if (FULL || v < nvec) c[i] = src[v];
+    }
+  };
+  auto process = [&](int64_t r, const uint4 (&c)[NC]) {
+    const uint4* src = row_src(r);
+    int8_t* dst = q + r * (int64_t)K;
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NC; ++i) {
+      if (FULL || i * 64 + lane < nvec) {
+        float f[EPV];
+        RowIn<BF16>::unpack(c[i], f);
+        amax = fmaxf(amax, vec_amax<EPV>(f));
+      }
+    }
+    if constexpr (!FULL) {
+      for (int v = NC * 64 + lane; v < nvec; v += 64) {
+        float f[EPV];
+        RowIn<BF16>::unpack(src[v], f);
+        amax = fmaxf(amax, vec_amax<EPV>(f));
+      }
+    }
+    amax = wave_max(amax);
+    float s = __fdiv_rn(amax, 127.0f);
+    if (amax == 0.0f) s = 1.0f;
+    const float rs = __builtin_amdgcn_rcpf(s);
+    const bool fast_ok = s >= 1.17549435e-38f;  // normal scale: rcp is finite and accurate to 1 ulp
+    if (lane == 0) scale[r] = s;
+#pragma unroll
+    for (int i = 0; i < NC; ++i) {
+      const int v = i * 64 + lane;
+      if (FULL || v < nvec) quant_store<BF16>(c[i], s, rs, fast_ok, dst + (int64_t)v * EPV);
+    }
+    if constexpr (!FULL) {
+      for (int v = NC * 64 + lane; v < nvec; v += 64)
+        quant_store<BF16>(src[v], s, rs, fast_ok, dst + (int64_t)v * EPV);
+    }
+  };
+
+  if constexpr (PREFETCH) {
+    uint4 cur[NC], nxt[NC];
+    load_cache(row, cur);
+    while (true) {
+      const int64_t r1 = row + stride;
+      if (r1 < M) load_cache(r1, nxt);  // uniform per wavefront
+      process(row, cur);
+      if (r1 >= M) break;
+#pragma unroll
+      for (int i = 0; i < NC; ++i) cur[i] = nxt[i];
+      row = r1;
+    }
+  } else {
+    for (; row < M; row += stride) {
+      uint4 c[NC];
+      load_cache(row, c);
+      process(row, c);
+    }
+  }
+}
+
+// One workgroup (4 wavefronts) per row, for rows long enough to feed 256 lanes.
+// A lane holds NV 16-byte vectors; the row maximum is combined across the four
+// wavefronts through LDS.  Compared with one wavefront per row this quarters
+// the work that remains after a row's last byte has arrived, which is what
+// bounds a launch whose rows are all requested at once.
+template <bool BF16, int NV>
+__global__ __launch_bounds__(256) void quant_row_wg_kernel(const void* __restrict__ x, int K, int64_t ldx,
+                                                            int8_t* __restrict__ q, float* __restrict__ scale) {
+  constexpr int EPV = RowIn<BF16>::EPV;
+  __shared__ float wmax[4];
+  const int tid = threadIdx.x;
+  const int64_t row = blockIdx.x;
+  const int nvec = K / EPV;
   const uint4* src =
       reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(x) + row * ldx * (BF16 ? 2 : 4));
   int8_t* dst = q + row * (int64_t)K;
-
-  uint4 cache[NC];
+  uint4 c[NV];
   float amax = 0.0f;
 #pragma unroll
-  for (int i = 0; i < NC; ++i) {
-    const int v = i * 64 + lane;
-    if (v < nvec) {
-      cache[i] = src[v];
+  for (int i = 0; i < NV; ++i) {
+    const int v = i * 256 + tid;
+    if (v < nvec) c[i] = src[v];
+  }
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    if (i * 256 + tid < nvec) {
       float f[EPV];
-      RowIn<BF16>::unpack(cache[i], f);
+      RowIn<BF16>::unpack(c[i], f);
       amax = fmaxf(amax, vec_amax<EPV>(f));
     }
   }
-  for (int v = NC * 64 + lane; v < nvec; v += 64) {
-    float f[EPV];
-    RowIn<BF16>::unpack(src[v], f);
-    amax = fmaxf(amax, vec_amax<EPV>(f));
-  }
   amax = wave_max(amax);
+  if ((tid & 63) == 0) wmax[tid >> 6] = amax;
+  __syncthreads();
+  amax = fmaxf(fmaxf(wmax[0], wmax[1]), fmaxf(wmax[2], wmax[3]));
   float s = __fdiv_rn(amax, 127.0f);
   if (amax == 0.0f) s = 1.0f;
   const float rs = __builtin_amdgcn_rcpf(s);
-  if (lane == 0) scale[row] = s;
+  const bool fast_ok = s >= 1.17549435e-38f;  // normal scale: rcp is finite and accurate to 1 ulp
+  if (tid == 0) scale[row] = s;
 #pragma unroll
-  for (int i = 0; i < NC; ++i) {
-    const int v = i * 64 + lane;
-    if (v < nvec) quant_store<BF16>(cache[i], s, rs, dst + (int64_t)v * EPV);
+  for (int i = 0; i < NV; ++i) {
+    const int v = i * 256 + tid;
+    if (v < nvec) quant_store<BF16>(c[i], s, rs, fast_ok, dst + (int64_t)v * EPV);
   }
-  for (int v = NC * 64 + lane; v < nvec; v += 64) quant_store<BF16>(src[v], s, rs, dst + (int64_t)v * EPV);
 }
 
 // ---------------------------------------------------------------- FP8 tensor
@@ -131,8 +213,15 @@ __global__ __launch_bounds__(256) void amax_kernel(const void* __restrict__ x, i
     amax = fmaxf(amax, vec_amax<EPV>(f));
   }
   amax = wave_max(amax);
-  // |x| >= 0, so the IEEE bit patterns order like unsigned integers.
-  if ((threadIdx.x & 63) == 0 && amax > 0.0f) atomicMax(amax_bits, __float_as_uint(amax));
+  // one atomic per workgroup: same-address atomics serialise at the L2
+  __shared__ float wmax[4];
+  if ((threadIdx.x & 63) == 0) wmax[threadIdx.x >> 6] = amax;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const float m = fmaxf(fmaxf(wmax[0], wmax[1]), fmaxf(wmax[2], wmax[3]));
+    // |x| >= 0, so the IEEE bit patterns order like unsigned integers.
+    if (m > 0.0f) atomicMax(amax_bits, __float_as_uint(m));
+  }
 }
 
 __device__ __forceinline__ float fp8_prescale(float a, float s) {
@@ -191,13 +280,58 @@ extern "C" int aq_quant_rowwise_i8(const void* x, int x_dtype, int64_t M, int64_
   const int esz = x_dtype == AQ_BF16 ? 2 : 4;
   if (aq::check_ptr16(x) || aq::check_ptr16(q) || ((ldx * esz) & 15)) return AQ_E_ALIGN;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  const unsigned grid = (unsigned)((M + 3) / 4);
-  if (x_dtype == AQ_BF16)
-    hipLaunchKernelGGL((aq::quant_rowwise_i8_kernel<true, 16>), dim3(grid), dim3(256), 0, st, x, M,
-                       (int)K, ldx, q, scale);
-  else
-    hipLaunchKernelGGL((aq::quant_rowwise_i8_kernel<false, 16>), dim3(grid), dim3(256), 0, st, x, M,
-                       (int)K, ldx, q, scale);
+  // Rows that fit 4 cached vectors per lane (2048 bf16 / 1024 fp32) take the
+  // double-buffered kernel; with enough rows each wavefront gets two of them so
+  // that reads, arithmetic and writes of different rows overlap.
+  const int epv = x_dtype == AQ_BF16 ? 8 : 4;
+  const int64_t nvec = K / epv;
+  const int64_t wg_min_vec = x_dtype == AQ_BF16 ? 257 : 128;  // bf16 rows of <= 2048 do as well one wavefront per row
+  if (M >= 64 && nvec >= wg_min_vec && nvec <= 1024) {
+    // enough rows to fill the device and rows of 128..1024 vectors: one workgroup per row
+    const unsigned g = (unsigned)M;
+    if (x_dtype == AQ_BF16) {
+      if (nvec <= 256)
+        hipLaunchKernelGGL((aq::quant_row_wg_kernel<true, 1>), dim3(g), dim3(256), 0, st, x, (int)K, ldx, q, scale);
+      else if (nvec <= 512)
+        hipLaunchKernelGGL((aq::quant_row_wg_kernel<true, 2>), dim3(g), dim3(256), 0, st, x, (int)K, ldx, q, scale);
+      else
+        hipLaunchKernelGGL((aq::quant_row_wg_kernel<true, 4>), dim3(g), dim3(256), 0, st, x, (int)K, ldx, q, scale);
+    } else {
+      if (nvec <= 256)
+        hipLaunchKernelGGL((aq::quant_row_wg_kernel<false, 1>), dim3(g), dim3(256), 0, st, x, (int)K, ldx, q, scale);
+      else if (nvec <= 512)
+        hipLaunchKernelGGL((aq::quant_row_wg_kernel<false, 2>), dim3(g), dim3(256), 0, st, x, (int)K, ldx, q, scale);
+      else
+        hipLaunchKernelGGL((aq::quant_row_wg_kernel<false, 4>), dim3(g), dim3(256), 0, st, x, (int)K, ldx, q, scale);
+    }
+    return (int)hipGetLastError();
+  }
+  const bool small_row = K <= 4 * 64 * epv;
+  const bool full_row = K == 4 * 64 * epv;  // every lane holds exactly 4 vectors: no bounds checks
+  int64_t wgs = (M + 3) / 4;
+  if (small_row && M >= 2048) wgs = (wgs + 1) / 2;
+  const unsigned grid = (unsigned)wgs;
+  if (x_dtype == AQ_BF16) {
+    if (full_row)
+      hipLaunchKernelGGL((aq::quant_rowwise_i8_kernel<true, 4, true, true>), dim3(grid), dim3(256), 0, st, x, M,
+                         (int)K, ldx, q, scale);
+    else if (small_row)
+      hipLaunchKernelGGL((aq::quant_rowwise_i8_kernel<true, 4, true, false>), dim3(grid), dim3(256), 0, st, x, M,
+                         (int)K, ldx, q, scale);
+    else
+      hipLaunchKernelGGL((aq::quant_rowwise_i8_kernel<true, 16, false, false>), dim3(grid), dim3(256), 0, st, x,
+                         M, (int)K, ldx, q, scale);
+  } else {
+    if (full_row)
+      hipLaunchKernelGGL((aq::quant_rowwise_i8_kernel<false, 4, true, true>), dim3(grid), dim3(256), 0, st, x, M,
+                         (int)K, ldx, q, scale);
+    else if (small_row)
+      hipLaunchKernelGGL((aq::quant_rowwise_i8_kernel<false, 4, true, false>), dim3(grid), dim3(256), 0, st, x, M,
+                         (int)K, ldx, q, scale);
+    else
+      hipLaunchKernelGGL((aq::quant_rowwise_i8_kernel<false, 16, false, false>), dim3(grid), dim3(256), 0, st, x,
+                         M, (int)K, ldx, q, scale);
+  }
   return (int)hipGetLastError();
 }
 
@@ -212,7 +346,7 @@ extern "C" int aq_quant_tensor_fp8(const void* x, int x_dtype, int64_t numel, ui
   const int epv = x_dtype == AQ_BF16 ? 8 : 4;
   const int64_t nvec = numel / epv;
   int64_t blocks = (nvec + 255) / 256;
-  if (blocks > 2048) blocks = 2048;  // 8 workgroups per CU, grid-stride beyond
+  if (blocks > 1024) blocks = 1024;  // 4 workgroups per CU, grid-stride beyond
   if (blocks < 1) blocks = 1;
   hipLaunchKernelGGL(aq::fill_u32_kernel, dim3(1), dim3(64), 0, st, amax_ws, 0u);
   if (x_dtype == AQ_BF16) {

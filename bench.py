@@ -35,9 +35,14 @@ PEAK_HBM_GBS = 8000.0        # MI355X HBM3E, published
 PEAK_INT8_TOPS = 5000.0      # dense int8 MFMA, published (no sparsity)
 PEAK_FP8_TFLOPS = 5000.0     # dense FP8 MFMA, published
 
-# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs,
-# scaled by a copy kernel of known size; None until such a run has been made for the workload.
-MEASURED_TRAFFIC = {"decode": None, "prefill": None, "fp8": None}
+# Bytes per launch that the dominant kernel moves past the L2 (FETCH_SIZE + WRITE_SIZE from two
+# rocprofv3 --pmc runs of this script, each scaled by what the same counter reads for kernels of
+# known size in the same run: 2048 B per FETCH_SIZE unit, 1024 B per WRITE_SIZE unit).
+MEASURED_TRAFFIC = {
+    "decode": {1: 16.87e6 + 0.02e6, 4: 16.96e6 + 0.07e6, 16: 17.19e6 + 0.26e6},
+    "prefill": 33.76e6 + 16.80e6,  # the fetch side is L2 fills by 8 XCDs (12.58 MB of distinct input)
+    "fp8": 100.76e6 + 8.39e6,
+}
 
 
 def parse():
@@ -135,7 +140,7 @@ def bench_decode(torch, ops, args, dev):
         "value": gbs, "unit": "GB/s", "ms_per_step": ms, "eager_ms_per_step": ms_eager,
         "bytes_per_step": bytes_alg, "dtype": "int8",
         "roofline": {"bound": "hbm", "kernel": "gemv_w8a8_kernel", "achieved": gbs_k, "peak": PEAK_HBM_GBS,
-                     "unit": "GB/s", "frac": gbs_k / PEAK_HBM_GBS, "traffic": MEASURED_TRAFFIC["decode"],
+                     "unit": "GB/s", "frac": gbs_k / PEAK_HBM_GBS, "traffic": MEASURED_TRAFFIC["decode"].get(M),
                      "kernel_us": ms_k * 1e3, "algorithmic_bytes": bytes_alg,
                      "llc_resident_gbs": bytes_alg / (ms_res * 1e-3) / 1e9, "weight_buffers": nbuf},
         "shape": (M, N, K),
@@ -227,6 +232,64 @@ def bench_fp8(torch, ops, args, dev):
     }
 
 
+def measure_ceilings(torch, ops, dev):
+    """What this part delivers on trivial kernels: an MFMA-only loop (constant operands, so the
+    clock is not power-limited: an upper bound), a 1 GiB streaming read, and a one-shot 16 MiB
+    read (the size of the decode weight), which no kernel of that size can beat."""
+    lib = ops._abi.load()
+    st = torch.cuda.current_stream().cuda_stream
+    sink = torch.zeros(4, dtype=torch.int32, device=dev)
+
+    def timed(fn, n):
+        fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(n):
+            fn(i)
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e-3 / n
+
+    out = {}
+    iters = 4000
+    for kind, name, ops_per in ((0, "mfma_i8_32x32x32_tops", 65536), (2, "mfma_fp8_32x32x64_tflops", 131072)):
+        t = timed(lambda i=0: lib.aq_probe_mfma(kind, 1024, iters, sink.data_ptr(), st), 3)
+        out[name] = 1024 * 4 * iters * 8 * ops_per / t / 1e12
+    big = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+    t = timed(lambda i=0: lib.aq_probe_read(big.data_ptr(), big.numel(), 2048, sink.data_ptr(), st), 3)
+    out["hbm_stream_read_gbs"] = big.numel() / t / 1e9
+    del big
+    small = [torch.empty(16 << 20, dtype=torch.uint8, device=dev) for _ in range(40)]
+
+    def one_shot(i=0):
+        lib.aq_probe_read(small[i % 40].data_ptr(), 16 << 20, 2048, sink.data_ptr(), st)
+
+    for i in range(40):
+        one_shot(i)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        st2 = side.cuda_stream
+        with torch.cuda.graph(g, stream=side):
+            for i in range(40):
+                lib.aq_probe_read(small[i].data_ptr(), 16 << 20, 2048, sink.data_ptr(), st2)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    g.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    g.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    out["one_shot_16mib_read_us"] = e0.elapsed_time(e1) * 1e3 / 40
+    out["one_shot_16mib_read_gbs"] = (16 << 20) / (out["one_shot_16mib_read_us"] * 1e-6) / 1e9
+    return out
+
+
 def cpu_baseline(workload, shape, unit, per_step):
     """The C oracle on the same shape, on this host's cores.  Test infrastructure used as the
     reported baseline only: it never feeds the GPU path."""
@@ -297,6 +360,7 @@ def main():
                     a2.m = m
                     r = bench_decode(torch, ops, a2, dev)
                     extra[f"decode_m{m}"] = r
+        ceilings = measure_ceilings(torch, ops, dev)
     per_step = main_res.get("bytes_per_step") or main_res.get("ops_per_step") or main_res.get("flops_per_step")
     cpu = None
     if not args.no_cpu:
@@ -313,7 +377,7 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": main_res["dtype"],
         "data": "synthetic", "config": {"workload": main_res["workload"], "timing": "HIP graph replay of the timed steps",
                                         "eager_ms_per_step": main_res.get("eager_ms_per_step")},
-        "roofline": main_res["roofline"], "cpu_baseline": cpu,
+        "roofline": main_res["roofline"], "cpu_baseline": cpu, "measured_ceilings": ceilings,
         "also": {k: {kk: vv for kk, vv in v.items()} for k, v in extra.items()},
     }
     print(json.dumps(line))

@@ -139,7 +139,7 @@ def bench_decode(torch, ops, args, dev):
         "workload": f"decode_gemv_w8a8 M={M} K={K} N={N} bf16->int8 per-token, W int8 per-channel, bf16 out",
         "value": gbs, "unit": "GB/s", "ms_per_step": ms, "eager_ms_per_step": ms_eager,
         "bytes_per_step": bytes_alg, "dtype": "int8",
-        "roofline": {"bound": "hbm", "kernel": "gemv_w8a8_kernel", "achieved": gbs_k, "peak": PEAK_HBM_GBS,
+        "roofline": {"bound": "hbm", "kernel": "gemv_mfma_kernel" if M > 8 else "gemv_w8a8_kernel", "achieved": gbs_k, "peak": PEAK_HBM_GBS,
                      "unit": "GB/s", "frac": gbs_k / PEAK_HBM_GBS, "traffic": MEASURED_TRAFFIC["decode"].get(M),
                      "kernel_us": ms_k * 1e3, "algorithmic_bytes": bytes_alg,
                      "llc_resident_gbs": bytes_alg / (ms_res * 1e-3) / 1e9, "weight_buffers": nbuf},
@@ -229,6 +229,46 @@ def bench_fp8(torch, ops, args, dev):
                      "unit": "TFLOP/s", "frac": tk / PEAK_FP8_TFLOPS, "traffic": MEASURED_TRAFFIC["fp8"],
                      "kernel_us": ms_k * 1e3, "algorithmic_flops": flops},
         "shape": (M, N, K),
+    }
+
+
+def bench_block(torch, ops, args, dev):
+    """BASELINE configs[4]: one int8-quantized 1B-class decoder block, 8 x 512 prefill then 64 decode steps."""
+    from khaosz_amd.block import ContiguousKV, DecoderBlock, decode_mask, rotary_table
+    from khaosz_amd.linear import quantize_model
+
+    dt = torch.bfloat16
+    B, S, steps, dim = 8, 512, 64, 2048
+    torch.manual_seed(7)
+    blk = DecoderBlock(dim, 16, 5632, 4)
+    blk.reset_parameters()
+    blk = blk.to(dev).to(dt)
+    quantize_model(blk)
+    tab = rotary_table(128, S + steps, device=dev)
+    x = torch.randn(B, S, dim, device=dev).to(dt)
+    xs = torch.randn(steps, B, 1, dim, device=dev).to(dt)
+    cache = ContiguousKV(B, S + steps, 4, 128, dev, dt)
+    fr = lambda a, n: tab[a:a + n].unsqueeze(0).expand(B, -1, -1)
+    masks = [decode_mask(B, S + t + 1, dev, dt) for t in range(steps)]
+
+    def prefill(i=0):
+        return blk(x, fr(0, S), None, cache.bind(S))
+
+    def decode_all(i=0):
+        for t in range(steps):
+            blk(xs[t], fr(S + t, 1), masks[t], cache.bind(S + t + 1))
+
+    ms_pre = graph_time_ms(torch, prefill, 10, 3)
+    prefill()
+    ms_dec = graph_time_ms(torch, decode_all, 3, 2) / steps
+    lin_ops = 2.0 * B * S * 45088768
+    lin_bytes = 45088768
+    return {
+        "workload": "decoder_block hidden=2048 16q/4kv x128 ffn=5632, 7 Linears W8A8, bf16; 8x512 prefill + 64 decode steps (M=8)",
+        "value": ms_pre + steps * ms_dec, "unit": "ms", "prefill_ms": ms_pre, "decode_ms_per_step": ms_dec,
+        "linear_only_prefill_tops_if_all_time_were_linear": lin_ops / (ms_pre * 1e-3) / 1e12,
+        "linear_only_decode_gbs_if_all_time_were_linear": lin_bytes / (ms_dec * 1e-3) / 1e9,
+        "dtype": "int8", "ms_per_step": ms_pre + steps * ms_dec, "roofline": {}, "shape": (B * S, 0, 0),
     }
 
 
@@ -354,6 +394,7 @@ def main():
             for name in ("decode", "prefill", "fp8"):
                 if name != args.workload:
                     extra[name] = fns[name](torch, ops, args, dev)
+            extra["block"] = bench_block(torch, ops, args, dev)
             if args.workload == "decode":
                 for m in (1, 4):
                     a2 = argparse.Namespace(**vars(args))

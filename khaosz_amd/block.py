@@ -1,0 +1,146 @@
+"""The callers of Linear inside one decoder block, restated so that the
+quantized path can be exercised at the shapes a real model presents.
+
+Structure follows the reference (pre-norm residual block with GQA and a SwiGLU
+MLP), each piece citing the file it restates; only the seven projections are
+this package's own arithmetic, everything else is the same stock torch call the
+reference makes.  The KV cache here is a contiguous per-sequence buffer with the
+two methods attention needs (``write`` / ``gather``), standing in for the paged
+``KvcacheView`` (astrai/inference/core/cache.py:277-290), whose page management
+belongs to the serving layer.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+from torch import Tensor
+
+from .linear import Linear
+
+
+class RMSNorm(nn.Module):
+    """``F.rms_norm`` with a learned gain (astrai/model/components/norm.py:7-15)."""
+
+    def __init__(self, dim: int, norm_eps: float):
+        super().__init__()
+        self.weight = nn.Parameter(torch.ones(dim))
+        self.norm_eps = norm_eps
+
+    def forward(self, x: Tensor) -> Tensor:
+        return F.rms_norm(x, (x.shape[-1],), self.weight, self.norm_eps)
+
+
+def rotary_table(head_dim: int, max_len: int, base: float = 10000.0, device=None) -> Tensor:
+    """complex64 ``[max_len, head_dim/2]`` with angle ``t * base**(-2i/d)``
+    (astrai/model/components/rope.py:8-19: float64 angles, float32 cos/sin)."""
+    inv = base ** (-torch.arange(0, head_dim, 2, dtype=torch.float64, device=device) / head_dim)
+    ang = torch.outer(torch.arange(max_len, dtype=torch.float64, device=device), inv).float()
+    return torch.polar(torch.ones_like(ang), ang)
+
+
+def apply_rotary(x: Tensor, freqs: Tensor) -> Tensor:
+    """Rotate interleaved pairs ``(x[2i], x[2i+1])`` of ``x [B, S, H, D]`` by ``freqs [B, S, D/2]``
+    in float32 and cast back (rope.py:26-33)."""
+    xc = torch.view_as_complex(x.float().reshape(*x.shape[:-1], -1, 2))
+    out = torch.view_as_real(xc * freqs.unsqueeze(2)).flatten(-2)
+    return out.to(x.dtype)
+
+
+class ContiguousKV:
+    """KV cache for one block: ``[B, max_len, Hkv, D]``; ``total_len`` is the length after the
+    tokens being written, as in ``KvcacheView`` (cache.py:282-290)."""
+
+    def __init__(self, batch: int, max_len: int, n_kv_heads: int, head_dim: int, device, dtype):
+        self.k = torch.zeros((batch, max_len, n_kv_heads, head_dim), device=device, dtype=dtype)
+        self.v = torch.zeros_like(self.k)
+        self.total_len = 0
+
+    def bind(self, total_len: int) -> "ContiguousKV":
+        self.total_len = total_len
+        return self
+
+    def write(self, layer_id: int, k: Tensor, v: Tensor) -> None:
+        start = self.total_len - k.size(1)
+        self.k[:, start:self.total_len] = k
+        self.v[:, start:self.total_len] = v
+
+    def gather(self, layer_id: int) -> Tuple[Tensor, Tensor]:
+        return self.k[:, :self.total_len], self.v[:, :self.total_len]
+
+
+class GQA(nn.Module):
+    """Grouped-query attention (astrai/model/components/attention.py:32-109), without the
+    optional qk-norm and output gate that BASELINE config 5 leaves off."""
+
+    def __init__(self, dim: int, n_heads: int, n_kv_heads: int, layer_id: int = 0):
+        super().__init__()
+        if dim % n_heads or n_heads % n_kv_heads:
+            raise ValueError("dim must divide into heads and heads into kv heads")
+        self.head_dim = dim // n_heads
+        self.n_heads, self.n_kv_heads, self.layer_id = n_heads, n_kv_heads, layer_id
+        self.q_proj = Linear(dim, n_heads * self.head_dim)
+        self.k_proj = Linear(dim, n_kv_heads * self.head_dim)
+        self.v_proj = Linear(dim, n_kv_heads * self.head_dim)
+        self.o_proj = Linear(dim, dim)
+
+    def forward(self, x: Tensor, rotary_emb: Tensor, attn_mask: Optional[Tensor] = None,
+                cache: Optional[ContiguousKV] = None) -> Tensor:
+        B, S, _ = x.shape
+        q = self.q_proj(x).reshape(B, S, self.n_heads, self.head_dim)
+        k = self.k_proj(x).reshape(B, S, self.n_kv_heads, self.head_dim)
+        v = self.v_proj(x).reshape(B, S, self.n_kv_heads, self.head_dim)
+        q, k = apply_rotary(q, rotary_emb), apply_rotary(k, rotary_emb)
+        if cache is not None:
+            cache.write(self.layer_id, k, v)
+            k, v = cache.gather(self.layer_id)
+        rep = self.n_heads // self.n_kv_heads
+        if rep > 1:  # attention.py:15-23
+            k = k.repeat_interleave(rep, dim=2)
+            v = v.repeat_interleave(rep, dim=2)
+        out = F.scaled_dot_product_attention(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), attn_mask,
+                                             is_causal=attn_mask is None)
+        return self.o_proj(out.transpose(1, 2).reshape(B, S, -1))
+
+
+class MLP(nn.Module):
+    """``down(up(x) * silu(gate(x)))`` (astrai/model/components/mlp.py:16-27)."""
+
+    def __init__(self, dim: int, dim_ffn: int):
+        super().__init__()
+        self.up = Linear(dim, dim_ffn)
+        self.gate = Linear(dim, dim_ffn)
+        self.down = Linear(dim_ffn, dim)
+
+    def forward(self, x: Tensor) -> Tensor:
+        return self.down(self.up(x) * F.silu(self.gate(x)))
+
+
+class DecoderBlock(nn.Module):
+    """``x += attn(norm(x)); x += mlp(norm(x))`` (astrai/model/components/decoder_block.py:12-59)."""
+
+    def __init__(self, dim: int, n_heads: int, dim_ffn: int, n_kv_heads: int, norm_eps: float = 1e-5,
+                 layer_id: int = 0):
+        super().__init__()
+        self.attention = GQA(dim, n_heads, n_kv_heads, layer_id)
+        self.input_norm = RMSNorm(dim, norm_eps)
+        self.post_attention_norm = RMSNorm(dim, norm_eps)
+        self.mlp = MLP(dim, dim_ffn)
+
+    def reset_parameters(self) -> None:
+        for m in self.modules():
+            if isinstance(m, Linear):
+                m.reset_parameters()
+
+    def forward(self, x: Tensor, rotary_emb: Tensor, attention_mask: Optional[Tensor] = None,
+                cache: Optional[ContiguousKV] = None) -> Tensor:
+        x = self.attention(self.input_norm(x), rotary_emb, attention_mask, cache) + x
+        return self.mlp(self.post_attention_norm(x)) + x
+
+
+def decode_mask(batch: int, total_len: int, device, dtype) -> Tensor:
+    """Additive mask ``[B, 1, 1, T]`` of a single new token attending to everything cached
+    (what astrai/model/transformer.py:17-46 builds for a decode step without padding)."""
+    return torch.zeros((batch, 1, 1, total_len), device=device, dtype=dtype)

@@ -1,0 +1,147 @@
+"""The decoder block that hosts the quantized Linears (BASELINE config 5).
+CPU tests pin the float restatement against closed forms and a hand-written
+attention; GPU tests put QuantLinear into it through quantize_model."""
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from khaosz_amd.block import (ContiguousKV, DecoderBlock, GQA, RMSNorm, apply_rotary, decode_mask, rotary_table)
+from khaosz_amd.linear import QuantLinear, quantize_model
+
+
+def _freqs(table, B, start, S):
+    return table[start:start + S].unsqueeze(0).expand(B, -1, -1)
+
+
+def test_rotary_is_a_position_dependent_rotation():
+    tab = rotary_table(16, 32)
+    assert tab.shape == (32, 8) and tab.dtype == torch.complex64
+    assert torch.allclose(tab[0], torch.ones(8, dtype=torch.complex64))
+    theta = 10000.0 ** (-torch.arange(0, 16, 2, dtype=torch.float64) / 16)
+    assert torch.allclose(torch.angle(tab[5]).double(), (5 * theta + math.pi) % (2 * math.pi) - math.pi, atol=1e-6)
+    x = torch.randn(2, 4, 3, 16)
+    y = apply_rotary(x, _freqs(tab, 2, 7, 4))
+    assert torch.allclose(y.norm(dim=-1), x.norm(dim=-1), atol=1e-5)           # rotations keep the norm
+    assert torch.allclose(apply_rotary(x, _freqs(tab, 2, 0, 1).expand(2, 4, 8)), x)  # position 0 is the identity
+    # pair (2i, 2i+1) is rotated by angle p * theta_i
+    p, i = 9, 3
+    a = torch.zeros(1, 1, 1, 16)
+    a[..., 2 * i] = 1.0
+    r = apply_rotary(a, _freqs(tab, 1, p, 1))[0, 0, 0]
+    assert abs(r[2 * i].item() - math.cos(p * theta[i])) < 1e-6 and abs(r[2 * i + 1].item() - math.sin(p * theta[i])) < 1e-6
+    # scores depend on the position difference only
+    q, k = torch.randn(1, 1, 1, 16), torch.randn(1, 1, 1, 16)
+    s1 = (apply_rotary(q, _freqs(tab, 1, 12, 1)) * apply_rotary(k, _freqs(tab, 1, 5, 1))).sum()
+    s2 = (apply_rotary(q, _freqs(tab, 1, 20, 1)) * apply_rotary(k, _freqs(tab, 1, 13, 1))).sum()
+    assert abs(s1 - s2) < 1e-4
+
+
+def test_rmsnorm_closed_form():
+    n = RMSNorm(24, 1e-5)
+    with torch.no_grad():
+        n.weight.copy_(torch.randn(24))
+    x = torch.randn(3, 5, 24)
+    want = x / torch.sqrt((x * x).mean(-1, keepdim=True) + 1e-5) * n.weight
+    assert torch.allclose(n(x), want, atol=1e-5)
+
+
+def test_gqa_matches_a_hand_written_causal_attention():
+    torch.manual_seed(0)
+    dim, H, Hkv, B, S = 32, 4, 2, 2, 6
+    att = GQA(dim, H, Hkv)
+    for l in (att.q_proj, att.k_proj, att.v_proj, att.o_proj):
+        l.reset_parameters()
+    x = torch.randn(B, S, dim)
+    tab = rotary_table(dim // H, 16)
+    fr = _freqs(tab, B, 0, S)
+    y = att(x, fr)
+    D = dim // H
+    q = apply_rotary((x @ att.q_proj.weight.T).view(B, S, H, D), fr)
+    k = apply_rotary((x @ att.k_proj.weight.T).view(B, S, Hkv, D), fr)
+    v = (x @ att.v_proj.weight.T).view(B, S, Hkv, D)
+    out = torch.zeros(B, S, H, D)
+    for b in range(B):
+        for h in range(H):
+            g = h // (H // Hkv)
+            for i in range(S):
+                sc = torch.stack([(q[b, i, h] * k[b, j, g]).sum() / math.sqrt(D) for j in range(i + 1)])
+                w = torch.softmax(sc, 0)
+                out[b, i, h] = sum(w[j] * v[b, j, g] for j in range(i + 1))
+    want = out.reshape(B, S, dim) @ att.o_proj.weight.T
+    assert torch.allclose(y, want, atol=1e-4)
+
+
+def _block(dim=64, heads=4, kv=2, ffn=176, seed=0):
+    torch.manual_seed(seed)
+    b = DecoderBlock(dim, heads, ffn, kv)
+    b.reset_parameters()
+    return b
+
+
+def test_block_residual_structure_and_decode_equals_prefill_on_cpu():
+    blk = _block()
+    B, S, dim = 2, 9, 64
+    tab = rotary_table(16, 32)
+    x = torch.randn(B, S + 1, dim)
+    full = blk(x, _freqs(tab, B, 0, S + 1))
+    # by hand: x1 = x + attn(norm(x)); y = x1 + mlp(norm(x1))
+    x1 = x + blk.attention(blk.input_norm(x), _freqs(tab, B, 0, S + 1))
+    assert torch.allclose(full, x1 + blk.mlp(blk.post_attention_norm(x1)), atol=1e-6)
+    cache = ContiguousKV(B, 32, 2, 16, "cpu", torch.float32)
+    pre = blk(x[:, :S], _freqs(tab, B, 0, S), None, cache.bind(S))
+    assert torch.allclose(pre, full[:, :S], atol=1e-5)
+    step = blk(x[:, S:], _freqs(tab, B, S, 1), decode_mask(B, S + 1, "cpu", torch.float32), cache.bind(S + 1))
+    assert torch.allclose(step[:, 0], full[:, S], atol=1e-5)
+
+
+@pytest.mark.gpu
+def test_quantized_block_tracks_the_float_block():
+    dev = "cuda:0"
+    blk = _block(dim=256, heads=4, kv=2, ffn=704).to(dev)
+    B, S = 2, 40
+    tab = rotary_table(64, 128, device=dev)
+    x = torch.randn(B, S, 256, device=dev)
+    with torch.inference_mode():
+        ref = blk(x, _freqs(tab, B, 0, S))
+        assert quantize_model(blk) == 7
+        assert all(isinstance(m, QuantLinear) for m in (blk.attention.q_proj, blk.attention.o_proj, blk.mlp.down))
+        y = blk(x, _freqs(tab, B, 0, S))
+    rel = ((y - ref).norm() / ref.norm()).item()
+    assert rel < 3e-2, rel
+
+
+@pytest.mark.gpu
+def test_config5_block_prefill_then_decode_bf16():
+    """hidden 2048, 16 query / 4 KV heads of 128, FFN 5632, all 7 Linears W8A8, bf16 activations;
+    a shortened run of the config (2 x 96 prefill, 3 decode steps) checked against the float block, and
+    each decode step against the same token's row of a longer prefill."""
+    dev, dt = "cuda:0", torch.bfloat16
+    torch.manual_seed(5)
+    blk = DecoderBlock(2048, 16, 5632, 4)
+    blk.reset_parameters()
+    blk = blk.to(dev)
+    B, S, steps = 2, 96, 3
+    tab = rotary_table(128, 256, device=dev)
+    x = torch.randn(B, S + steps, 2048, device=dev)
+    with torch.inference_mode():
+        ref = blk(x, _freqs(tab, B, 0, S + steps))                  # float32 block, whole sequence
+        fblk = blk.to(dt)
+        assert quantize_model(fblk) == 7
+        xb = x.to(dt)
+        full = fblk(xb, _freqs(tab, B, 0, S + steps))               # quantized, whole sequence (MFMA path)
+        cache = ContiguousKV(B, 256, 4, 128, dev, dt)
+        pre = fblk(xb[:, :S], _freqs(tab, B, 0, S), None, cache.bind(S))
+        outs = [pre]
+        for t in range(steps):                                      # decode path (M = B = 2)
+            pos = S + t
+            outs.append(fblk(xb[:, pos:pos + 1], _freqs(tab, B, pos, 1), decode_mask(B, pos + 1, dev, dt),
+                             cache.bind(pos + 1)))
+        seq = torch.cat(outs, dim=1)
+    assert seq.shape == (B, S + steps, 2048) and seq.dtype == dt
+    rel = ((full.float() - ref).norm() / ref.norm()).item()
+    assert rel < 3e-2, rel
+    # decode rows equal the prefill rows of the same tokens up to bf16 attention numerics
+    rel_d = ((seq.float() - full.float()).norm() / full.float().norm()).item()
+    assert rel_d < 1e-2, rel_d

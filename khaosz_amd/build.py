@@ -34,7 +34,7 @@ def _stale(out, deps):
 
 def build(force: bool = True, verbose: bool = False) -> str:
     os.makedirs(OBJ_DIR, exist_ok=True)
-    headers = [os.path.join(CSRC, "aq_common.h"), os.path.join(HERE, "..", "include", "astrai_q.h")]
+    headers = [os.path.join(CSRC, "aq_common.h"), os.path.join(CSRC, "aq_rows.h"), os.path.join(HERE, "..", "include", "astrai_q.h")]
 
     def compile_one(src):
         s = os.path.join(CSRC, src)

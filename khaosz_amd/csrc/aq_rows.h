@@ -1,0 +1,124 @@
+// Row-wise int8 quantisation pieces shared by the stand-alone quantise kernels
+// and the decode kernels that quantise their few activation rows themselves.
+#pragma once
+#include "aq_common.h"
+
+namespace aq {
+
+template <bool BF16>
+struct RowIn;
+template <>
+struct RowIn<true> {  // 8 bf16 per 16-byte vector
+  static constexpr int EPV = 8;
+  __device__ static __forceinline__ void unpack(const uint4& v, float* f) {
+    f[0] = __uint_as_float(v.x << 16);
+    f[1] = __uint_as_float(v.x & 0xffff0000u);
+    f[2] = __uint_as_float(v.y << 16);
+    f[3] = __uint_as_float(v.y & 0xffff0000u);
+    f[4] = __uint_as_float(v.z << 16);
+    f[5] = __uint_as_float(v.z & 0xffff0000u);
+    f[6] = __uint_as_float(v.w << 16);
+    f[7] = __uint_as_float(v.w & 0xffff0000u);
+  }
+};
+template <>
+struct RowIn<false> {  // 4 fp32 per 16-byte vector
+  static constexpr int EPV = 4;
+  __device__ static __forceinline__ void unpack(const uint4& v, float* f) {
+    f[0] = __uint_as_float(v.x);
+    f[1] = __uint_as_float(v.y);
+    f[2] = __uint_as_float(v.z);
+    f[3] = __uint_as_float(v.w);
+  }
+};
+
+template <int EPV>
+__device__ __forceinline__ float vec_amax(const float* f) {
+  float m = 0.0f;
+#pragma unroll
+  for (int i = 0; i < EPV; ++i) m = fmaxf(m, fabsf(f[i]));
+  return m;
+}
+
+// Symmetric absmax scale of one row from its wavefront-wide maximum:
+// s = amax / 127 (1 for an all-zero row), rs = rcp(s), and whether rs may be used.
+struct RowScale {
+  float s, rs;
+  bool fast_ok;
+};
+__device__ __forceinline__ RowScale row_scale(float amax) {
+  RowScale r;
+  r.s = __fdiv_rn(amax, 127.0f);
+  if (amax == 0.0f) r.s = 1.0f;
+  r.rs = __builtin_amdgcn_rcpf(r.s);
+  r.fast_ok = r.s >= 1.17549435e-38f;  // normal scale: rcp is finite and accurate to 1 ulp
+  return r;
+}
+
+// One wavefront quantises RPW rows of the activation straight into LDS.
+// Wavefront `wave` of `nwaves` owns rows wave, wave + nwaves, ...; a lane holds
+// VPL 16-byte vectors per row (vector lane + 64*i), all requested by issue()
+// before anything is waited for, so the caller can queue other loads behind
+// them.  finish() reduces, rounds and writes the codes of row m to
+// xs + m*pitch and its scale to sx[m]; rows >= M (up to MT) are zero-filled.
+template <bool BF16, int RPW, int VPL>
+struct RowsToLds {
+  static constexpr int EPV = RowIn<BF16>::EPV;
+  uint4 c[RPW][VPL];
+
+  __device__ __forceinline__ void issue(const void* x, int M, int K, int64_t ldx, int wave, int nwaves, int lane) {
+    const int nvec = K / EPV;
+#pragma unroll
+    for (int j = 0; j < RPW; ++j) {
+      const int m = wave + j * nwaves;
+      const uint4* src =
+          reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(x) + (int64_t)m * ldx * (BF16 ? 2 : 4));
+#pragma unroll
+      for (int i = 0; i < VPL; ++i) {
+        const int v = i * 64 + lane;
+        c[j][i] = make_uint4(0, 0, 0, 0);
+        if (m < M && v < nvec) c[j][i] = src[v];
+      }
+    }
+  }
+
+  __device__ __forceinline__ void finish(int M, int MT, int K, uint8_t* xs, int pitch, float* sx, int wave,
+                                         int nwaves, int lane) {
+    const int nvec = K / EPV;
+#pragma unroll
+    for (int j = 0; j < RPW; ++j) {
+      const int m = wave + j * nwaves;
+      if (m >= MT) continue;  // uniform
+      float amax = 0.0f;
+#pragma unroll
+      for (int i = 0; i < VPL; ++i) {
+        float f[EPV];
+        RowIn<BF16>::unpack(c[j][i], f);  // vectors past the row or of rows >= M are zero
+        amax = fmaxf(amax, vec_amax<EPV>(f));
+      }
+      const RowScale rsc = row_scale(wave_max(amax));
+      if (lane == 0 && m < M) sx[m] = rsc.s;
+#pragma unroll
+      for (int i = 0; i < VPL; ++i) {
+        const int v = i * 64 + lane;
+        if (v < nvec) {
+          float f[EPV];
+          uint32_t code[EPV];
+          RowIn<BF16>::unpack(c[j][i], f);
+          quant_codes<EPV>(f, rsc.s, rsc.rs, rsc.fast_ok, code);  // zero rows give zero codes
+          uint8_t* dst = xs + m * pitch + v * EPV;
+          if constexpr (BF16) {
+            uint2 o;
+            o.x = pack_low_bytes(code[0], code[1], code[2], code[3]);
+            o.y = pack_low_bytes(code[4], code[5], code[6], code[7]);
+            *reinterpret_cast<uint2*>(dst) = o;
+          } else {
+            *reinterpret_cast<uint32_t*>(dst) = pack_low_bytes(code[0], code[1], code[2], code[3]);
+          }
+        }
+      }
+    }
+  }
+};
+
+}  // namespace aq

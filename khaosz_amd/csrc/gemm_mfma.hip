@@ -157,58 +157,9 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(GemmArgs p) {
   const __amdgpu_buffer_rsrc_t Ar = make_rsrc(p.A + (int64_t)m0 * K, (uint32_t)rows_a * (uint32_t)K);
   const __amdgpu_buffer_rsrc_t Br = make_rsrc(p.B + (int64_t)n0 * K, (uint32_t)rows_b * (uint32_t)K);
 
-  // Epilogue operands are fetched first of all, so their latency is hidden
-  // behind the whole K loop: per-row activation scales as 16 float4 per lane
-  // (accumulator register r of lane l belongs to row (r/4)*8 + (l/32)*4 + r%4),
-  // per-column weight scale and bias as one scalar per 32x32 tile column.
   const int col = lane & 31;
   const int rq = (lane >> 5) * 4;  // row offset of this lane's half inside each group of 8 rows
   const int mw = __builtin_amdgcn_readfirstlane(m0 + wave_m * WAVE_M);  // wavefront-uniform: keep it scalar
-  float sx1 = 1.0f, sw1 = 1.0f;
-  float sxr[TM][4][4];  // [i][g][q]: row i*32 + g*8 + rq + q
-  float swn[TN], bn[TN];
-  bool has_bias = false;
-  if constexpr (FP8) {
-    sx1 = *p.sx;
-    sw1 = *p.sw;
-  } else if constexpr (OUT != OUT_I32) {
-    // rows past M fall outside the descriptor and read as zero (their outputs are never stored)
-    const int rows_left = __builtin_amdgcn_readfirstlane((M - mw) > 0 ? (M - mw) : 0);
-    const __amdgpu_buffer_rsrc_t Sr =
-        make_rsrc(p.sx + (rows_left ? mw : 0), (uint32_t)(rows_left < WAVE_M ? rows_left : WAVE_M) * 4u);
-    if ((M & 3) == 0) {  // uniform: the 4 rows of a float4 are all in or all out, and 16-byte aligned
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const uint4 t = buffer_load_16(Sr, (uint32_t)(i * 32 + g * 8 + rq) * 4u);
-          sxr[i][g][0] = __uint_as_float(t.x);
-          sxr[i][g][1] = __uint_as_float(t.y);
-          sxr[i][g][2] = __uint_as_float(t.z);
-          sxr[i][g][3] = __uint_as_float(t.w);
-        }
-    } else {
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int g = 0; g < 4; ++g)
-#pragma unroll
-          for (int q = 0; q < 4; ++q)
-            sxr[i][g][q] = __uint_as_float(
-                (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(Sr, (i * 32 + g * 8 + rq + q) * 4, 0, 0));
-    }
-    has_bias = p.bias != nullptr;
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const int n = n0 + wave_n * WAVE_N + j * 32 + col;
-      const int nc = n < N ? n : (N - 1);
-      swn[j] = p.sw[nc];
-      bn[j] = 0.0f;
-      if (has_bias)
-        bn[j] = p.bias_dtype == AQ_BF16 ? bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(p.bias)[nc])
-                                        : reinterpret_cast<const float*>(p.bias)[nc];
-    }
-  }
 
   // One load instruction of a wavefront fills 1 KiB = 8 tile rows.  Wavefront w
   // owns the 8-row groups w, w+NWAVES, w+2*NWAVES, ... of A and of B.
@@ -331,11 +282,70 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(GemmArgs p) {
   // Loads past the last K step are still issued (outside the descriptors they
   // write zeros into a stage nobody reads) so that the count of outstanding
   // loads per wavefront is the same at every wait.
+  // Epilogue operands, requested right behind stage 0 so that their latency is
+  // hidden behind the whole K loop and they never delay the first tile: per-row
+  // activation scales as float4 per lane (accumulator register r of lane l
+  // belongs to row (r/4)*8 + (l/32)*4 + r%4), per-column weight scale and bias
+  // as one scalar per 32x32 tile column.  Nothing is done with the values until
+  // the epilogue (bias stays a raw bit pattern), so no wait is placed here.
+  float sx1 = 1.0f, sw1 = 1.0f;
+  float sxr[TM][4][4];  // [i][g][q]: row i*32 + g*8 + rq + q
+  float swn[TN];
+  uint32_t bias_raw[TN];
+  const bool has_bias = !FP8 && OUT != OUT_I32 && p.bias != nullptr;
+  const bool bias_bf16 = p.bias_dtype == AQ_BF16;
+  auto load_epilogue_operands = [&]() {
+    if constexpr (FP8) {
+      sx1 = *p.sx;
+      sw1 = *p.sw;
+    } else if constexpr (OUT != OUT_I32) {
+      // rows past M fall outside the descriptor and read as zero (their outputs are never stored)
+      const int rows_left = __builtin_amdgcn_readfirstlane((M - mw) > 0 ? (M - mw) : 0);
+      const __amdgpu_buffer_rsrc_t Sr =
+          make_rsrc(p.sx + (rows_left ? mw : 0), (uint32_t)(rows_left < WAVE_M ? rows_left : WAVE_M) * 4u);
+      if ((M & 3) == 0) {  // uniform: the 4 rows of a float4 are all in or all out, and 16-byte aligned
 #pragma unroll
-  for (int st = 0; st < NSTAGE; ++st)
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const uint4 t = buffer_load_16(Sr, (uint32_t)(i * 32 + g * 8 + rq) * 4u);
+            sxr[i][g][0] = __uint_as_float(t.x);
+            sxr[i][g][1] = __uint_as_float(t.y);
+            sxr[i][g][2] = __uint_as_float(t.z);
+            sxr[i][g][3] = __uint_as_float(t.w);
+          }
+      } else {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int g = 0; g < 4; ++g)
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+              sxr[i][g][q] = __uint_as_float(
+                  (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(Sr, (i * 32 + g * 8 + rq + q) * 4, 0, 0));
+      }
+      const __amdgpu_buffer_rsrc_t Wsr = make_rsrc(p.sw, (uint32_t)N * 4u);
+      const __amdgpu_buffer_rsrc_t Bsr =
+          make_rsrc(has_bias ? p.bias : p.sw, has_bias ? (uint32_t)N * (bias_bf16 ? 2u : 4u) : 0u);
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const uint32_t n = (uint32_t)(n0 + wave_n * WAVE_N + j * 32 + col);  // past N: outside -> 0
+        swn[j] = __uint_as_float((uint32_t)__builtin_amdgcn_raw_buffer_load_b32(Wsr, n * 4u, 0, 0));
+        bias_raw[j] = bias_bf16 ? (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(Bsr, n * 2u, 0, 0)
+                                : (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(Bsr, n * 4u, 0, 0);
+      }
+    }
+  };
+#pragma unroll
+  for (int q = 0; q < NLOADS; ++q) issue_load(0, 0, q);
+  asm volatile("" ::: "memory");  // keep the request order: stage 0, epilogue operands, stages 1 and 2
+  load_epilogue_operands();
+  asm volatile("" ::: "memory");
+#pragma unroll
+  for (int st = 1; st < NSTAGE; ++st)
 #pragma unroll
     for (int q = 0; q < NLOADS; ++q) issue_load(st, st, q);
-  AQ_WAIT_VMCNT(2 * NLOADS);  // stage 0 has landed
+  AQ_WAIT_VMCNT(2 * NLOADS);  // all but the two youngest stages: stage 0 (and the operands) have landed
   AQ_BARRIER();
   load_frags(smem, 0, af[0], bf[0]);
   // sub-steps 0 .. NKS-2 of stage 0 (no loads to issue yet: stages 0..2 are in flight)
@@ -402,6 +412,9 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(GemmArgs p) {
     for (int j = 0; j < TN; ++j) {
       const int cj = j * 32 + col;  // column inside the wavefront's 64
       const bool n_ok = nw + cj < N;
+      float bn = 0.0f;
+      if constexpr (!FP8 && OUT != OUT_I32)
+        bn = !has_bias ? 0.0f : bias_bf16 ? bf16_bits_to_f32(bias_raw[j]) : __uint_as_float(bias_raw[j]);
       // lane part of the byte offset; the pairing path stores at the even column of the pair
       const uint32_t vbase =
           n_ok ? (uint32_t)rq * rowb + (uint32_t)(PAIR ? (cj & ~1) : cj) * ESZ + (PAIR && odd ? rowb : 0u)
@@ -428,7 +441,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(GemmArgs p) {
                 // three separately rounded fp32 operations, never contracted.  Without a bias
                 // bn is +0: the product of an integer and two positive scales is never -0,
                 // so adding it changes no bit.
-                y[q] = __fadd_rn(__fmul_rn(__fmul_rn((float)acc[i][j][g * 4 + q], sxr[i][g][q]), swn[j]), bn[j]);
+                y[q] = __fadd_rn(__fmul_rn(__fmul_rn((float)acc[i][j][g * 4 + q], sxr[i][g][q]), swn[j]), bn);
               }
             }
             if constexpr (OUT == OUT_F32) {

@@ -15,6 +15,7 @@
 #include <type_traits>
 
 #include "aq_common.h"
+#include "aq_rows.h"
 
 namespace aq {
 
@@ -72,7 +73,8 @@ struct Butterfly {
 constexpr int ilog2(int v) { return v <= 1 ? 0 : 1 + ilog2(v / 2); }
 
 struct GemvArgs {
-  const int8_t* xq;   // [M, K] codes (workspace)
+  const void* x;      // [M, K] bf16 activations (fused-quantise kernels), row stride K
+  const int8_t* xq;   // [M, K] codes (kernels that take codes)
   const float* sx;    // [M]
   const int8_t* wq;   // [N, K]
   const float* sw;    // [N]
@@ -84,9 +86,11 @@ struct GemvArgs {
 
 #define GV_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(0x0f70 | ((n) & 15) | (((n) >> 4) << 14))
 
-template <int MT>
+// FUSED: the kernel quantises the bf16 activation rows itself (VPL 16-byte vectors
+// per lane per row) instead of copying codes a separate launch produced.
+template <int MT, bool FUSED, int VPL>
 __global__ __launch_bounds__(GV_THREADS) void gemv_w8a8_kernel(GemvArgs p) {
-  extern __shared__ __attribute__((aligned(16))) uint8_t xs[];  // [MT][K] activation codes
+  extern __shared__ __attribute__((aligned(16))) uint8_t xs[];  // [MT][K] activation codes, then [MT] scales
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int K = p.K, N = p.N, M = p.M;
@@ -103,25 +107,34 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_w8a8_kernel(GemvArgs p) {
   const int om = oidx % MT, on = n0 + oidx / MT;
   const bool out_lane = (lane & ((1 << SH) - 1)) == 0 && om < M && on < N;
   float sxv = 0.0f, swv = 0.0f, bv = 0.0f;
+  float* sx_lds = reinterpret_cast<float*>(xs + MT * K);
   if (out_lane) {
-    sxv = p.sx[om];
+    if constexpr (!FUSED) sxv = p.sx[om];
     swv = p.sw[on];
     if (p.bias)
       bv = p.bias_dtype == AQ_BF16 ? bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(p.bias)[on])
                                    : reinterpret_cast<const float*>(p.bias)[on];
   }
 
-  // 1. activation codes -> LDS, 16 bytes per lane, straight from global memory.
-  // Rows m >= M lie outside the descriptor and arrive as zeros.
-  const __amdgpu_buffer_rsrc_t Xr = make_rsrc(p.xq, (uint32_t)M * (uint32_t)K);
-  const int xbytes = MT * K;
-  const int xrounds = (xbytes + GV_THREADS * 16 - 1) / (GV_THREADS * 16);
-  for (int r = 0; r < xrounds; ++r) {
-    const int base = (r * GV_WAVES + wave) * 1024;  // this wavefront's 1 KiB of the copy
-    if (base < xbytes)  // uniform; xbytes is a multiple of 16 but not always of 1024:
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(Xr, (gv_lds_void*)(xs + base), 16,
-                                               (base + lane * 16) < xbytes ? (uint32_t)(base + lane * 16) : OOB_OFFSET,
-                                               0, 0, 0);
+  // 1. activation codes -> LDS.  Either copied, 16 bytes per lane, straight from
+  // global memory (rows m >= M lie outside the descriptor and arrive as zeros),
+  // or produced here: each wavefront requests its rows of the bf16 activation now
+  // and quantises them while the weight loads queued behind are in flight.
+  constexpr int RPW = (MT + GV_WAVES - 1) / GV_WAVES;
+  RowsToLds<true, RPW, VPL> xrows;
+  if constexpr (FUSED) {
+    xrows.issue(p.x, M, K, K, wave, GV_WAVES, lane);
+  } else {
+    const __amdgpu_buffer_rsrc_t Xr = make_rsrc(p.xq, (uint32_t)M * (uint32_t)K);
+    const int xbytes = MT * K;
+    const int xrounds = (xbytes + GV_THREADS * 16 - 1) / (GV_THREADS * 16);
+    for (int r = 0; r < xrounds; ++r) {
+      const int base = (r * GV_WAVES + wave) * 1024;  // this wavefront's 1 KiB of the copy
+      if (base < xbytes)  // uniform; xbytes is a multiple of 16 but not always of 1024:
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(
+            Xr, (gv_lds_void*)(xs + base), 16,
+            (base + lane * 16) < xbytes ? (uint32_t)(base + lane * 16) : OOB_OFFSET, 0, 0, 0);
+    }
   }
 
   // 2. the first GV_DEPTH weight chunks of this wavefront's rows.  The
@@ -142,12 +155,22 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_w8a8_kernel(GemvArgs p) {
 #pragma unroll
   for (int d = 0; d < GV_DEPTH; ++d) wload(d, w[d]);  // chunks past the end read zeros
 
-  // 3. the activation copy is older than the weight loads: wait until at most
-  // those are outstanding, then make every wavefront's part visible.
-  GV_WAIT_VMCNT(GV_DEPTH * GV_ROWS);
+  // 3. the activation requests are older than the weight loads: wait until at
+  // most those are outstanding (the fused path's own use of the rows makes the
+  // compiler place that wait), then make every wavefront's part visible through
+  // a barrier that does not drain the weight loads.
+  if constexpr (FUSED) {
+    xrows.finish(M, MT, K, xs, K, sx_lds, wave, GV_WAVES, lane);
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wavefront's LDS writes are done
+  } else {
+    GV_WAIT_VMCNT(GV_DEPTH * GV_ROWS);
+  }
   asm volatile("" ::: "memory");
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
+  if constexpr (FUSED) {
+    if (out_lane) sxv = sx_lds[om];
+  }
 
   int acc[GV_ROWS * MT];
 #pragma unroll
@@ -206,16 +229,16 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_w8a8_kernel(GemvArgs p) {
     reinterpret_cast<float*>(p.y)[o] = y;
 }
 
-template <int MT>
+template <int MT, bool FUSED, int VPL>
 static int launch_gemv(const GemvArgs& a, hipStream_t st) {
   const unsigned grid = (unsigned)((a.N + GV_ROWS * GV_WAVES - 1) / (GV_ROWS * GV_WAVES));
-  const size_t lds = (size_t)MT * a.K;
+  const size_t lds = (size_t)MT * a.K + MT * sizeof(float);
   if (lds > 64 * 1024) {  // beyond the default dynamic-LDS limit: opt this kernel in (idempotent)
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_w8a8_kernel<MT>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_w8a8_kernel<MT, FUSED, VPL>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return (int)e;
   }
-  hipLaunchKernelGGL((gemv_w8a8_kernel<MT>), dim3(grid), dim3(GV_THREADS), lds, st, a);
+  hipLaunchKernelGGL((gemv_w8a8_kernel<MT, FUSED, VPL>), dim3(grid), dim3(GV_THREADS), lds, st, a);
   return (int)hipGetLastError();
 }
 
@@ -241,12 +264,16 @@ constexpr int GV_MFMA_MIN_M = AQ_GV_MFMA_MIN_M;  // more tokens than this take t
 // summed through LDS (exact int32).
 constexpr int GM_ROWS = 16;    // weight rows per wavefront
 constexpr int GM_KSPLIT = 2;   // wavefronts sharing a row group
-constexpr int GM_GROUPS = 2;   // row groups per workgroup
+#ifndef AQ_GM_GROUPS
+#define AQ_GM_GROUPS 2
+#endif
+constexpr int GM_GROUPS = AQ_GM_GROUPS;   // row groups per workgroup
 constexpr int GM_WAVES = GM_KSPLIT * GM_GROUPS;
 constexpr int GM_BATCH = 8;    // MFMA steps (64 K bytes each) per register batch
 
+template <bool FUSED>
 __global__ __launch_bounds__(GM_WAVES * 64) void gemv_mfma_kernel(GemvArgs p) {
-  extern __shared__ __attribute__((aligned(16))) uint8_t xs[];  // [16][K + 16] token codes, then the partial sums
+  extern __shared__ __attribute__((aligned(16))) uint8_t xs[];  // [16][K + 16] token codes, [16] scales; later the partial sums
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int grp = wave / GM_KSPLIT, kh = wave % GM_KSPLIT;
@@ -265,8 +292,11 @@ __global__ __launch_bounds__(GM_WAVES * 64) void gemv_mfma_kernel(GemvArgs p) {
     swv[r] = 0.0f;
     bv[r] = 0.0f;
   }
+  float* sx_lds = reinterpret_cast<float*>(xs + 16 * pitch);
   if (kh == 0) {  // uniform: only the first half's wavefront writes outputs
-    if (tok < M) sxv = p.sx[tok];
+    if constexpr (!FUSED) {
+      if (tok < M) sxv = p.sx[tok];
+    }
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const int n = rbase + r < N ? rbase + r : N - 1;
@@ -289,44 +319,56 @@ __global__ __launch_bounds__(GM_WAVES * 64) void gemv_mfma_kernel(GemvArgs p) {
       dst[j] = buffer_load_16(Wr, (step0 + j) < nstep ? woff + (uint32_t)(step0 + j) * 64u : OOB_OFFSET);
   };
 
-  // token codes -> LDS (padded rows; tokens >= M lie outside the descriptor and arrive as zeros).
-  // Their loads are issued before the weight loads, so they return first and the
-  // LDS fill overlaps the weight stream's flight time.
-  const __amdgpu_buffer_rsrc_t Xr = make_rsrc(p.xq, (uint32_t)M * (uint32_t)K);
-  const int nvec_row = K / 16;
-  const int nvec = 16 * nvec_row;
-  constexpr int XV = 8;  // vectors per thread per round: 16 x 2048 codes in one round of 256 threads
-  uint4 xv[XV];
-  auto xload = [&](int v0) {
+  // token codes -> LDS (padded rows; tokens >= M are zero).  Their loads are
+  // issued before the weight loads, so they return first and the LDS fill --
+  // or, when FUSED, the quantisation of the bf16 rows (4 rows per wavefront,
+  // 4 vectors per lane per row: K <= 2048) -- overlaps the weight stream's flight time.
+  if constexpr (FUSED) {
+    RowsToLds<true, (16 + GM_WAVES - 1) / GM_WAVES, 4> rows;
+    rows.issue(p.x, M, K, K, wave, GM_WAVES, lane);
+    wload(0, wa);
+    wload(GM_BATCH, wb);
+    rows.finish(M, 16, K, xs, pitch, sx_lds, wave, GM_WAVES, lane);
+  } else {
+    const __amdgpu_buffer_rsrc_t Xr = make_rsrc(p.xq, (uint32_t)M * (uint32_t)K);
+    const int nvec_row = K / 16;
+    const int nvec = 16 * nvec_row;
+    constexpr int XV = 2048 / (GM_WAVES * 64);  // vectors per thread per round: 16 x 2048 codes in one round
+    uint4 xv[XV];
+    auto xload = [&](int v0) {
 #pragma unroll
-    for (int i = 0; i < XV; ++i) {
-      const int v = v0 + i * (GM_WAVES * 64) + tid;
-      xv[i] = buffer_load_16(Xr, v < nvec ? (uint32_t)v * 16u : OOB_OFFSET);
-    }
-  };
-  auto xstore = [&](int v0) {
-#pragma unroll
-    for (int i = 0; i < XV; ++i) {
-      const int v = v0 + i * (GM_WAVES * 64) + tid;
-      if (v < nvec) {
-        const int m = v / nvec_row, c = v - m * nvec_row;
-        *reinterpret_cast<uint4*>(xs + m * pitch + c * 16) = xv[i];
+      for (int i = 0; i < XV; ++i) {
+        const int v = v0 + i * (GM_WAVES * 64) + tid;
+        xv[i] = buffer_load_16(Xr, v < nvec ? (uint32_t)v * 16u : OOB_OFFSET);
       }
+    };
+    auto xstore = [&](int v0) {
+#pragma unroll
+      for (int i = 0; i < XV; ++i) {
+        const int v = v0 + i * (GM_WAVES * 64) + tid;
+        if (v < nvec) {
+          const int m = v / nvec_row, c = v - m * nvec_row;
+          *reinterpret_cast<uint4*>(xs + m * pitch + c * 16) = xv[i];
+        }
+      }
+    };
+    xload(0);
+    wload(0, wa);
+    wload(GM_BATCH, wb);
+    xstore(0);
+    for (int v0 = XV * GM_WAVES * 64; v0 < nvec; v0 += XV * GM_WAVES * 64) {  // rows longer than 2048
+      xload(v0);
+      xstore(v0);
     }
-  };
-  xload(0);
-  wload(0, wa);
-  wload(GM_BATCH, wb);
-  xstore(0);
-  for (int v0 = XV * GM_WAVES * 64; v0 < nvec; v0 += XV * GM_WAVES * 64) {  // rows longer than 2048
-    xload(v0);
-    xstore(v0);
   }
   // LDS writes done, then a barrier without a memory fence: the weight loads stay in flight
   __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
   asm volatile("" ::: "memory");
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
+  if constexpr (FUSED) {
+    if (kh == 0 && tok < M) sxv = sx_lds[tok];
+  }
 
   v4i acc = {0, 0, 0, 0};
   const uint8_t* xl = xs + tok * pitch + kh * khalf + (lane >> 4) * 16;
@@ -389,21 +431,22 @@ __global__ __launch_bounds__(GM_WAVES * 64) void gemv_mfma_kernel(GemvArgs p) {
   }
 }
 
+template <bool FUSED>
 static int launch_gemv_mfma(const GemvArgs& a, hipStream_t st) {
   const unsigned grid = (unsigned)((a.N + GM_ROWS * GM_GROUPS - 1) / (GM_ROWS * GM_GROUPS));
-  const size_t lds = (size_t)16 * (a.K + 16);
+  const size_t lds = (size_t)16 * (a.K + 16) + 16 * sizeof(float);
   if (lds > 64 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_mfma_kernel),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_mfma_kernel<FUSED>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return (int)e;
   }
-  hipLaunchKernelGGL(gemv_mfma_kernel, dim3(grid), dim3(GM_WAVES * 64), lds, st, a);
+  hipLaunchKernelGGL((gemv_mfma_kernel<FUSED>), dim3(grid), dim3(GM_WAVES * 64), lds, st, a);
   return (int)hipGetLastError();
 }
 
 // the streaming MFMA variant needs each K half to be whole 64-byte steps and its padded codes to fit LDS
 static bool gemv_mfma_ok(int64_t M, int64_t K) {
-  return M > GV_MFMA_MIN_M && (K % (64 * GM_KSPLIT)) == 0 && 16 * (K + 16) <= GV_MAX_LDS;
+  return M > GV_MFMA_MIN_M && (K % (64 * GM_KSPLIT)) == 0 && 16 * (K + 16) + 64 <= GV_MAX_LDS;
 }
 
 
@@ -426,19 +469,35 @@ static int gemv_check(const int8_t* wq, const float* sw, const void* bias, int b
   if (aq::check_ptr16(wq)) return AQ_E_ALIGN;
   if (N > (1 << 30)) return AQ_E_RANGE;
   const int mt = M <= 1 ? 1 : M <= 2 ? 2 : M <= 4 ? 4 : M <= 8 ? 8 : 16;
-  if ((int64_t)mt * K > aq::GV_MAX_LDS) return AQ_E_RANGE;
+  if ((int64_t)mt * K + 64 > aq::GV_MAX_LDS) return AQ_E_RANGE;
   *mt_out = mt;
   return AQ_OK;
 }
 
 static int gemv_dispatch(const aq::GemvArgs& a, int mt, hipStream_t st) {
-  if (aq::gemv_mfma_ok(a.M, a.K)) return aq::launch_gemv_mfma(a, st);
+  if (aq::gemv_mfma_ok(a.M, a.K)) return aq::launch_gemv_mfma<false>(a, st);
   switch (mt) {
-    case 1: return aq::launch_gemv<1>(a, st);
-    case 2: return aq::launch_gemv<2>(a, st);
-    case 4: return aq::launch_gemv<4>(a, st);
-    case 8: return aq::launch_gemv<8>(a, st);
-    default: return aq::launch_gemv<16>(a, st);
+    case 1: return aq::launch_gemv<1, false, 4>(a, st);
+    case 2: return aq::launch_gemv<2, false, 4>(a, st);
+    case 4: return aq::launch_gemv<4, false, 4>(a, st);
+    case 8: return aq::launch_gemv<8, false, 4>(a, st);
+    default: return aq::launch_gemv<16, false, 4>(a, st);
+  }
+}
+
+// One launch for up to 8 bf16 rows that fit the in-kernel quantiser's register
+// budget; returns -1 when the shape has to take the two-launch path.  With more
+// than 8 rows every workgroup would repeat 2+ row quantisations per wavefront
+// on its critical path, which measures no faster than the separate launch.
+static int gemv_dispatch_fused(const aq::GemvArgs& a, int mt, hipStream_t st) {
+  const int64_t vpl = (a.K / 8 + 63) / 64;  // 16-byte vectors per lane per bf16 row
+  if (mt > 8 || vpl > 16) return -1;
+  const bool small = vpl <= 4;
+  switch (mt) {
+    case 1: return small ? aq::launch_gemv<1, true, 4>(a, st) : aq::launch_gemv<1, true, 16>(a, st);
+    case 2: return small ? aq::launch_gemv<2, true, 4>(a, st) : aq::launch_gemv<2, true, 16>(a, st);
+    case 4: return small ? aq::launch_gemv<4, true, 4>(a, st) : aq::launch_gemv<4, true, 16>(a, st);
+    default: return small ? aq::launch_gemv<8, true, 4>(a, st) : aq::launch_gemv<8, true, 16>(a, st);
   }
 }
 
@@ -475,6 +534,21 @@ extern "C" int aq_gemv_w8a8_decode(const void* x, int x_dtype, const int8_t* wq,
   if (!x || !ws) return AQ_E_NULL;
   if (aq::check_ptr16(x) || aq::check_ptr16(ws)) return AQ_E_ALIGN;
   if (ws_bytes < aq_gemv_w8a8_workspace_bytes(M, K)) return AQ_E_WORKSPACE;
+  if (x_dtype == AQ_BF16) {  // one launch: the GEMV kernel quantises the rows itself
+    aq::GemvArgs a{};
+    a.x = x;
+    a.wq = wq;
+    a.sw = sw;
+    a.bias = bias;
+    a.y = y;
+    a.M = (int)M;
+    a.N = (int)N;
+    a.K = (int)K;
+    a.bias_dtype = bias_dtype;
+    a.y_dtype = y_dtype;
+    const int frc = gemv_dispatch_fused(a, mt, static_cast<hipStream_t>(stream));
+    if (frc >= 0) return frc;
+  }
   int8_t* xq = static_cast<int8_t*>(ws);
   float* sx = reinterpret_cast<float*>(static_cast<char*>(ws) + aq::align256((size_t)(M * K)));
   rc = aq_quant_rowwise_i8(x, x_dtype, M, K, K, xq, sx, stream);

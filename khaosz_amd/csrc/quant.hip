@@ -3,45 +3,11 @@
 // kernels: 16-byte loads per lane, one wavefront per row, wavefront-wide
 // absmax through cross-lane shuffles, no LDS.
 #include "aq_common.h"
+#include "aq_rows.h"
 
 namespace aq {
 
 // ---------------------------------------------------------------- int8 rows
-
-template <bool BF16>
-struct RowIn;
-template <>
-struct RowIn<true> {  // 8 bf16 per 16-byte vector
-  static constexpr int EPV = 8;
-  __device__ static __forceinline__ void unpack(const uint4& v, float* f) {
-    f[0] = __uint_as_float(v.x << 16);
-    f[1] = __uint_as_float(v.x & 0xffff0000u);
-    f[2] = __uint_as_float(v.y << 16);
-    f[3] = __uint_as_float(v.y & 0xffff0000u);
-    f[4] = __uint_as_float(v.z << 16);
-    f[5] = __uint_as_float(v.z & 0xffff0000u);
-    f[6] = __uint_as_float(v.w << 16);
-    f[7] = __uint_as_float(v.w & 0xffff0000u);
-  }
-};
-template <>
-struct RowIn<false> {  // 4 fp32 per 16-byte vector
-  static constexpr int EPV = 4;
-  __device__ static __forceinline__ void unpack(const uint4& v, float* f) {
-    f[0] = __uint_as_float(v.x);
-    f[1] = __uint_as_float(v.y);
-    f[2] = __uint_as_float(v.z);
-    f[3] = __uint_as_float(v.w);
-  }
-};
-
-template <int EPV>
-__device__ __forceinline__ float vec_amax(const float* f) {
-  float m = 0.0f;
-#pragma unroll
-  for (int i = 0; i < EPV; ++i) m = fmaxf(m, fabsf(f[i]));
-  return m;
-}
 
 template <bool BF16>
 __device__ __forceinline__ void quant_store(const uint4& v, float s, float rs, bool fast_ok, int8_t* dst) {

@@ -263,7 +263,10 @@ constexpr int GV_MFMA_MIN_M = AQ_GV_MFMA_MIN_M;  // more tokens than this take t
 // Two wavefronts share a row group, each taking half of K; the halves are
 // summed through LDS (exact int32).
 constexpr int GM_ROWS = 16;    // weight rows per wavefront
-constexpr int GM_KSPLIT = 2;   // wavefronts sharing a row group
+#ifndef AQ_GM_KSPLIT
+#define AQ_GM_KSPLIT 2
+#endif
+constexpr int GM_KSPLIT = AQ_GM_KSPLIT;   // wavefronts sharing a row group
 #ifndef AQ_GM_GROUPS
 #define AQ_GM_GROUPS 2
 #endif
@@ -388,16 +391,16 @@ __global__ __launch_bounds__(GM_WAVES * 64) void gemv_mfma_kernel(GemvArgs p) {
     if (s0 + 3 * GM_BATCH < nstep) wload(s0 + 3 * GM_BATCH, wb);
   }
 
-  // sum the K halves: the second wavefront of each group parks its 4 sums in LDS
+  // sum the K parts: all but the first wavefront of each group park their 4 sums in LDS
   __syncthreads();  // everyone is done reading the token codes: the buffer is reused
-  int* part = reinterpret_cast<int*>(xs) + grp * 256;
+  int* part = reinterpret_cast<int*>(xs) + grp * (GM_KSPLIT - 1) * 256;
   if (kh != 0) {
-    *reinterpret_cast<v4i*>(part + lane * 4) = acc;
+    *reinterpret_cast<v4i*>(part + (kh - 1) * 256 + lane * 4) = acc;
   }
   __syncthreads();
   if (kh != 0) return;
-  const v4i other = *reinterpret_cast<const v4i*>(part + lane * 4);
-  acc += other;
+#pragma unroll
+  for (int k = 0; k < GM_KSPLIT - 1; ++k) acc += *reinterpret_cast<const v4i*>(part + k * 256 + lane * 4);
 
   if (tok >= M) return;
   float y[4];

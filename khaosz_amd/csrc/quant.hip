@@ -251,8 +251,10 @@ extern "C" int aq_quant_rowwise_i8(const void* x, int x_dtype, int64_t M, int64_
   // that reads, arithmetic and writes of different rows overlap.
   const int epv = x_dtype == AQ_BF16 ? 8 : 4;
   const int64_t nvec = K / epv;
-  const int64_t wg_min_vec = x_dtype == AQ_BF16 ? 257 : 128;  // bf16 rows of <= 2048 do as well one wavefront per row
-  if (M >= 64 && nvec >= wg_min_vec && nvec <= 1024) {
+  // bf16 rows of <= 2048 do as well one wavefront per row once there are enough rows to fill the
+  // device; a handful of rows (decode) always gains from the shorter per-lane chain of a workgroup per row
+  const int64_t wg_min_vec = (x_dtype == AQ_BF16 && M >= 64) ? 257 : 128;
+  if (nvec >= wg_min_vec && nvec <= 1024) {
     // enough rows to fill the device and rows of 128..1024 vectors: one workgroup per row
     const unsigned g = (unsigned)M;
     if (x_dtype == AQ_BF16) {

@@ -103,6 +103,16 @@ int aq_gemv_w8a8_codes(const int8_t *xq, const float *sx, const int8_t *wq, cons
 int aq_linear_fp8(const uint8_t *xq, const float *sx, const uint8_t *wq, const float *sw,
                   void *y, int y_dtype, int64_t M, int64_t N, int64_t K, void *stream);
 
+/* Tuning and test hook, no counterpart in the reference: the GEMM entry points
+ * pick their workgroup tile (256 x 128, or 128 x 128 with a split K step when
+ * the larger one would leave compute units idle) from M and N.  rows = 128 or
+ * 256 forces one of them for every later call of this process, 0 restores the
+ * choice by shape; anything else is AQ_E_SHAPE.  Results never depend on it
+ * for the int8 path (exact int32 sums); FP8 outputs may differ in the last
+ * bits of the fp32 accumulation.  Process-wide and unsynchronised: set it
+ * while no GEMM call is in progress on another thread. */
+int aq_set_gemm_tile(int rows);
+
 /* ---- measurement probes: no counterpart in the reference, not on the Linear
  * path.  They measure what this part's matrix cores and HBM deliver so that the
  * benchmark can quote kernels against measured as well as published ceilings.

@@ -27,6 +27,7 @@ SYMBOLS = {
     "aq_probe_mfma": (_int, [_int, _int, _int, _vp, _vp]),
     "aq_probe_copy": (_int, [_vp, _vp, _i64, _int, _vp]),
     "aq_probe_read": (_int, [_vp, _i64, _int, _vp, _vp]),
+    "aq_set_gemm_tile": (_int, [_int]),
 }
 
 _lib = None

@@ -8,7 +8,10 @@
 // (each lane feeds 16 or 32 consecutive k of one row), so no transpose is ever
 // materialised.  A workgroup of 8 wavefronts (two per SIMD) owns a 256 x 128
 // tile of C; each wavefront a 64 x 64 sub-tile held as 2 x 2 MFMA 32x32
-// accumulators.  K is walked in 128-byte steps through three LDS stages that
+// accumulators.  (When that gives too few tiles to occupy the device, the
+// tile is 128 x 128 instead and the two wavefronts that share a sub-tile each
+// take half of every K step; their accumulators are summed through LDS at the
+// end.)  K is walked in 128-byte steps through three (four) LDS stages that
 // are filled by direct global->LDS loads (no register staging), with an XOR
 // permutation of 16-byte pieces that makes the fragment reads bank-conflict
 // free; the loop is software-pipelined so that LDS reads and global loads of
@@ -21,17 +24,16 @@
 
 namespace aq {
 
-constexpr int BM = 256, BN = 128, BK = 128;
-constexpr int NSTAGE = 3;  // LDS stages: 3 x 48 KiB of the 160 KiB
-#ifndef AQ_WAVES_M
-#define AQ_WAVES_M 4
-#endif
-constexpr int WAVES_M = AQ_WAVES_M, WAVES_N = 2;  // wavefronts per workgroup: two per SIMD by default
-constexpr int NWAVES = WAVES_M * WAVES_N, NTHREADS = NWAVES * 64;
-constexpr int WAVE_M = BM / WAVES_M, WAVE_N = BN / WAVES_N;
+// Two shapes of workgroup, both 8 wavefronts (two per SIMD) of 64 x 64 sub-tiles:
+//   WM = 4, WK = 1: 256 x 128 tile, 4 x 2 wavefronts, 3 LDS stages of 48 KiB;
+//   WM = 2, WK = 2: 128 x 128 tile, 2 x 2 x 2 wavefronts (the last factor splits
+//                   each K step), 4 LDS stages of 32 KiB.
+constexpr int BN = 128, BK = 128;
+constexpr int WAVES_N = 2, NWAVES = 8, NTHREADS = NWAVES * 64;
+constexpr int WAVE_M = 64, WAVE_N = BN / WAVES_N;
 constexpr int TM = WAVE_M / 32, TN = WAVE_N / 32;
-constexpr int A_LOADS = BM * BK / 16 / NTHREADS;  // 16-byte vectors per thread per K step
-constexpr int B_LOADS = BN * BK / 16 / NTHREADS;
+constexpr int B_LOADS = BN * BK / 16 / NTHREADS;  // 16-byte vectors per thread per K step
+constexpr int BM_MAX = 256;
 constexpr int NUM_XCD = 8;
 constexpr int GROUP_M = 4;
 
@@ -129,9 +131,13 @@ __device__ __forceinline__ void sched_pattern() {
   }
 }
 
-template <bool FP8, int OUT>
+template <bool FP8, int OUT, int WM, int WK>
 __global__ __launch_bounds__(NTHREADS) void gemm_kernel(GemmArgs p) {
-  // NSTAGE stages of [A tile 256 x 128 B][B tile 128 x 128 B], rows unpadded.
+  static_assert(WM * WAVES_N * WK == NWAVES, "8 wavefronts per workgroup");
+  constexpr int BM = WM * WAVE_M;
+  constexpr int NSTAGE = WK == 1 ? 3 : 4;
+  constexpr int A_LOADS = BM * BK / 16 / NTHREADS;
+  // NSTAGE stages of [A tile BM x 128 B][B tile 128 x 128 B], rows unpadded.
   // Global->LDS loads land 64 lanes x 16 B contiguously (8 rows of 128 B), so
   // the bank-conflict-free layout is obtained by permuting which 16-byte piece
   // of its row each lane fetches: piece c of row r is stored at slot
@@ -144,7 +150,8 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(GemmArgs p) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
+  const int wave_k = WK == 1 ? 0 : wave / (WM * WAVES_N), wave_mn = WK == 1 ? wave : wave % (WM * WAVES_N);
+  const int wave_m = wave_mn / WAVES_N, wave_n = wave_mn % WAVES_N;
 
   int tile_m, tile_n;
   tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
@@ -202,10 +209,11 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(GemmArgs p) {
   const int fr_a = (wave_m * WAVE_M + (lane & 31)) * BK;
   const int fr_b = BM * BK + (wave_n * WAVE_N + (lane & 31)) * BK;
   const int fsw = (lane >> 1) & 7;
-  const int swz = FP8 ? ((((lane >> 5) * 2) ^ fsw) << 4) : (((lane >> 5) ^ fsw) << 4);
   constexpr int KSUB = FP8 ? 64 : 32;  // K per MFMA
-  constexpr int NKS = BK / KSUB;       // MFMA sub-steps per stage: 4 (int8) or 2 (FP8)
-  static_assert(NKS % 2 == 0, "fragment double-buffering alternates per sub-step");
+  constexpr int NKS = BK / KSUB / WK;  // MFMA sub-steps per stage and wavefront: 4 or 2 (int8), 2 or 1 (FP8)
+  // this wavefront's sub-steps of a stage start at piece wave_k * NKS * KSUB / 16; NKS is a power
+  // of two, so adding the sub-step number to that base is an XOR and folds into the permutation
+  const int swz = (FP8 ? ((((lane >> 5) * 2) ^ fsw) << 4) : (((lane >> 5) ^ fsw) << 4)) ^ (wave_k * NKS * KSUB);
   using frag_t = typename Frag<FP8>::type;
   auto load_frags = [&](const uint8_t* st, int ks, frag_t (&a)[TM], frag_t (&b)[TN]) {
     if constexpr (!FP8) {
@@ -275,9 +283,9 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(GemmArgs p) {
   //   iteration s:  slots    MFMAs of (s, 0 .. NKS-2)       | read fragments (s, 1 .. NKS-1)
   //                 wait for this wavefront's loads of stage s+1, barrier
   //                 slot A   MFMAs of (s, last sub-step)    | read fragments (s+1, 0)
-  // with the loads of stage s+3 spread from slot A of s over the slots of s+1.
+  // with the loads of stage s+NSTAGE spread from slot A of s over the slots of s+1.
   // At the barrier every wavefront holds the last fragments of stage s in
-  // registers, so stage s's LDS buffer is free for the loads of stage s+3 right
+  // registers, so stage s's LDS buffer is free for the loads of stage s+NSTAGE right
   // after it, and stage s+1 is complete and visible for slot A's fragment reads.
   // Loads past the last K step are still issued (outside the descriptors they
   // write zeros into a stage nobody reads) so that the count of outstanding
@@ -338,50 +346,95 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(GemmArgs p) {
   };
 #pragma unroll
   for (int q = 0; q < NLOADS; ++q) issue_load(0, 0, q);
-  asm volatile("" ::: "memory");  // keep the request order: stage 0, epilogue operands, stages 1 and 2
-  load_epilogue_operands();
+  asm volatile("" ::: "memory");  // keep the request order: stage 0, epilogue operands, the other stages
+  if (wave_k == 0) load_epilogue_operands();  // uniform: only these wavefronts run the epilogue
   asm volatile("" ::: "memory");
 #pragma unroll
   for (int st = 1; st < NSTAGE; ++st)
 #pragma unroll
     for (int q = 0; q < NLOADS; ++q) issue_load(st, st, q);
-  AQ_WAIT_VMCNT(2 * NLOADS);  // all but the two youngest stages: stage 0 (and the operands) have landed
+
+  // sub-steps 0 .. NKS-2 of a stage whose first fragments sit in af[C0]
+  auto middle_slots = [&](auto c0_c, const uint8_t* stc, auto loads_c, int kt_ld, int buf_ld) {
+    constexpr int C0 = decltype(c0_c)::value;
+    using c0 = integral_constant<int, C0>;
+    using c1 = integral_constant<int, C0 ^ 1>;
+    if constexpr (NKS == 4) {
+      slot(c0{}, stc, 1, loads_c, kt_ld, buf_ld, q1{});
+      slot(c1{}, stc, 2, loads_c, kt_ld, buf_ld, q2{});
+      slot(c0{}, stc, 3, loads_c, kt_ld, buf_ld, q3{});
+    } else if constexpr (NKS == 2) {
+      slot(c0{}, stc, 1, loads_c, kt_ld, buf_ld, q1{});
+    }
+  };
+  // the fragment buffer the last sub-step of such a stage computes from
+  auto last_of = [](auto c0_c) { return integral_constant<int, (NKS % 2 == 0) ? (decltype(c0_c)::value ^ 1) : decltype(c0_c)::value>{}; };
+
+  AQ_WAIT_VMCNT((NSTAGE - 1) * NLOADS);  // all but the younger stages: stage 0 (and the operands) have landed
   AQ_BARRIER();
   load_frags(smem, 0, af[0], bf[0]);
-  // sub-steps 0 .. NKS-2 of stage 0 (no loads to issue yet: stages 0..2 are in flight)
-  if constexpr (NKS == 4) {
-    slot(k0{}, smem, 1, no{}, 0, 0, q1{});
-    slot(k1{}, smem, 2, no{}, 0, 0, q2{});
-    slot(k0{}, smem, 3, no{}, 0, 0, q3{});
-  } else {
-    slot(k0{}, smem, 1, no{}, 0, 0, q1{});
-  }
-  __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the last fragments of stage 0 are in registers
-  AQ_WAIT_VMCNT(NLOADS);               // stage 1 has landed
+  middle_slots(k0{}, smem, no{}, 0, 0);  // no loads to issue yet: every stage buffer is in flight
+  __builtin_amdgcn_s_waitcnt(0xc07f);        // lgkmcnt(0): the last fragments of stage 0 are in registers
+  AQ_WAIT_VMCNT((NSTAGE - 2) * NLOADS);  // stage 1 has landed
   AQ_BARRIER();
-  // slot A of stage 0: its buffer (0) is free now and takes stage 3
-  slot(k1{}, smem + STAGE, 0, yes{}, NSTAGE, 0, q0{});
+  // slot A of stage 0: its buffer (0) is free now and takes stage NSTAGE
+  slot(last_of(k0{}), smem + STAGE, 0, yes{}, NSTAGE, 0, q0{});
   int b_prev = 0;  // buffer of stage s-1
-  for (int s = 1; s < nk; ++s) {
+  auto stage = [&](int s, auto c0_c) {
     const int b_cur = b_prev == NSTAGE - 1 ? 0 : b_prev + 1;
     const int b_next = b_cur == NSTAGE - 1 ? 0 : b_cur + 1;
-    const uint8_t* stc = smem + b_cur * STAGE;
-    // sub-steps 0 .. NKS-2 of stage s; the rest of stage s+2's loads go into stage s-1's buffer
-    if constexpr (NKS == 4) {
-      slot(k0{}, stc, 1, yes{}, s - 1 + NSTAGE, b_prev, q1{});
-      slot(k1{}, stc, 2, yes{}, s - 1 + NSTAGE, b_prev, q2{});
-      slot(k0{}, stc, 3, yes{}, s - 1 + NSTAGE, b_prev, q3{});
-    } else {
-      slot(k0{}, stc, 1, yes{}, s - 1 + NSTAGE, b_prev, q1{});
-    }
-    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the last fragments of stage s are in registers
-    AQ_WAIT_VMCNT(NLOADS);               // stage s+1 has landed (stage s+2 may still be in flight)
+    // sub-steps 0 .. NKS-2 of stage s; the rest of stage s-1+NSTAGE's loads go into stage s-1's buffer
+    middle_slots(c0_c, smem + b_cur * STAGE, yes{}, s - 1 + NSTAGE, b_prev);
+    __builtin_amdgcn_s_waitcnt(0xc07f);        // lgkmcnt(0): the last fragments of stage s are in registers
+    AQ_WAIT_VMCNT((NSTAGE - 2) * NLOADS);  // stage s+1 has landed (later ones may still be in flight)
     AQ_BARRIER();
-    // slot A: last sub-step of stage s | first fragments of stage s+1 | first loads of stage s+3
-    slot(k1{}, smem + b_next * STAGE, 0, yes{}, s + NSTAGE, b_cur, q0{});
+    // slot A: last sub-step of stage s | first fragments of stage s+1 | first loads of stage s+NSTAGE
+    slot(last_of(c0_c), smem + b_next * STAGE, 0, yes{}, s + NSTAGE, b_cur, q0{});
     b_prev = b_cur;
+  };
+  if constexpr (NKS % 2 == 0) {
+    for (int s = 1; s < nk; ++s) stage(s, k0{});
+  } else {  // one sub-step per stage: the fragment buffers alternate per stage
+    int s = 1;
+    for (; s + 1 < nk; s += 2) {
+      stage(s, k1{});
+      stage(s + 1, k0{});
+    }
+    if (s < nk) stage(s, k1{});
   }
-  AQ_WAIT_VMCNT(0);  // drain the padding loads before the workgroup's LDS can be released
+  AQ_WAIT_VMCNT(0);  // drain the padding loads before the workgroup's LDS can be released or reused
+
+  if constexpr (WK == 2) {
+    // The two wavefronts of a sub-tile hold the sums over their halves of every K step.  The
+    // second one parks its accumulators in LDS (16 KiB per sub-tile, over the stage buffers,
+    // which nobody reads any more once every wavefront is past this barrier); the first adds
+    // them and runs the epilogue alone.  int32 sums are exact in any order; FP8 partial sums
+    // are fp32, inside the stated tolerance.
+    __syncthreads();
+    using part_t = std::conditional_t<FP8, v4f, v4i>;
+    part_t* red = reinterpret_cast<part_t*>(smem) + wave_mn * 1024 + lane;
+    if (wave_k == 1) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+          for (int g = 0; g < 4; ++g)
+            red[((i * TN + j) * 4 + g) * 64] = part_t{acc[i][j][g * 4], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
+    }
+    __syncthreads();
+    if (wave_k == 1) return;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const part_t t = red[((i * TN + j) * 4 + g) * 64];
+#pragma unroll
+          for (int q = 0; q < 4; ++q) acc[i][j][g * 4 + q] += t[q];
+        }
+  }
 
   // ---- epilogue, straight from the accumulator registers (no LDS, no barrier).
   // A lane owns one output column per 32x32 tile and 64 of the wavefront's 128
@@ -485,10 +538,31 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(GemmArgs p) {
     store_all(yes{}, no{});
 }
 
+// 256-row tiles unless they leave much of the device idle: a workgroup per compute unit at a
+// time, so the cost of a launch is its number of rounds over the 256 compute units, and a
+// 128-row tile costs a little over half of a 256-row one.
+static int g_forced_tile = 0;  // 0: by shape; 128 / 256: forced (tuning and tests)
+
+static bool use_small_tile(int64_t M, int64_t N) {
+  if (g_forced_tile) return g_forced_tile == 128;
+  constexpr int64_t CUS = 256;
+  const int64_t tn = (N + BN - 1) / BN;
+  const int64_t rounds_big = ((M + 255) / 256 * tn + CUS - 1) / CUS;
+  const int64_t rounds_small = ((M + 127) / 128 * tn + CUS - 1) / CUS;
+  return rounds_small * 0.6 < (double)rounds_big;
+}
+
 template <bool FP8, int OUT>
-static int launch(const GemmArgs& a, hipStream_t st) {
+static int launch(GemmArgs& a, hipStream_t st) {
+  const bool small = use_small_tile(a.M, a.N);
+  const int bm = small ? 128 : 256;
+  a.tiles_m = (a.M + bm - 1) / bm;
+  a.tiles_n = (a.N + BN - 1) / BN;
   const unsigned grid = (unsigned)(a.tiles_m * a.tiles_n);
-  hipLaunchKernelGGL((gemm_kernel<FP8, OUT>), dim3(grid), dim3(NTHREADS), 0, st, a);
+  if (small)
+    hipLaunchKernelGGL((gemm_kernel<FP8, OUT, 2, 2>), dim3(grid), dim3(NTHREADS), 0, st, a);
+  else
+    hipLaunchKernelGGL((gemm_kernel<FP8, OUT, 4, 1>), dim3(grid), dim3(NTHREADS), 0, st, a);
   return (int)hipGetLastError();
 }
 
@@ -499,7 +573,7 @@ static int check_gemm(const void* A, const void* B, const void* C, int64_t M, in
   if (check_ptr16(A) || check_ptr16(B) || check_ptr16(C)) return AQ_E_ALIGN;
   // 32-bit tile-relative offsets: 256 rows * K bytes must fit an int
   if (K > (1 << 22) || M > (1 << 30) || N > (1 << 30)) return AQ_E_RANGE;
-  if (((M + BM - 1) / BM) * ((N + BN - 1) / BN) > (int64_t)0x7fffffff) return AQ_E_RANGE;
+  if (((M + 127) / 128) * ((N + BN - 1) / BN) > (int64_t)0x7fffffff) return AQ_E_RANGE;
   return AQ_OK;
 }
 
@@ -511,12 +585,16 @@ static GemmArgs make_args(const void* A, const void* B, void* C, int64_t M, int6
   a.M = (int)M;
   a.N = (int)N;
   a.K = (int)K;
-  a.tiles_m = (int)((M + BM - 1) / BM);
-  a.tiles_n = (int)((N + BN - 1) / BN);
   return a;
 }
 
 }  // namespace aq
+
+extern "C" int aq_set_gemm_tile(int rows) {
+  if (rows != 0 && rows != 128 && rows != 256) return AQ_E_SHAPE;
+  aq::g_forced_tile = rows;
+  return AQ_OK;
+}
 
 extern "C" int aq_gemm_i8_i32(const int8_t* xq, const int8_t* wq, int32_t* acc, int64_t M, int64_t N,
                               int64_t K, void* stream) {

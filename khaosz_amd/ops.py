@@ -206,6 +206,11 @@ def gemv_w8a8_codes(xq, sx, wq, sw, bias=None, out_dtype=torch.bfloat16) -> torc
     return y
 
 
+def set_gemm_tile(rows: int) -> None:
+    """Force the GEMM workgroup tile to 128 or 256 rows for this process (0: choose by shape)."""
+    _abi.check(_abi.load().aq_set_gemm_tile(int(rows)), "aq_set_gemm_tile")
+
+
 def linear_fp8(xq, sx, wq, sw, out_dtype=torch.bfloat16) -> torch.Tensor:
     """FP8 e4m3fn GEMM with fp32 accumulation: y = (acc * sx[0]) * sw[0]."""
     _need_gpu(xq, sx, wq, sw)

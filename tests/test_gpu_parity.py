@@ -95,21 +95,29 @@ GEMM_SHAPES = [(1, 1, 16), (37, 91, 48), (17, 5, 2048), (256, 128, 128), (257, 1
                (512, 384, 5632), (1000, 520, 1024)]
 
 
+@pytest.fixture(params=[128, 256])
+def tile(request):
+    """Run a GEMM test once per workgroup tile shape (the library would pick one by shape)."""
+    ops.set_gemm_tile(request.param)
+    yield request.param
+    ops.set_gemm_tile(0)
+
+
 def rand_codes(M, K, seed):
     g = torch.Generator().manual_seed(seed)
     return torch.randint(-127, 128, (M, K), generator=g, dtype=torch.int8)
 
 
 @pytest.mark.parametrize("M,N,K", GEMM_SHAPES)
-def test_gemm_i8_i32_bit_exact(oracle, M, N, K):
-    _say("gemm_i8_i32", M, N, K)
+def test_gemm_i8_i32_bit_exact(oracle, tile, M, N, K):
+    _say("gemm_i8_i32", M, N, K, tile)
     xq, wq = rand_codes(M, K, 1), rand_codes(N, K, 2)
     acc = ops.gemm_i8_i32(xq.to(DEV), wq.to(DEV))
     want = oracle.c_gemm_i8_i32(xq.numpy(), wq.numpy())
     assert np.array_equal(to_np(acc), want)
 
 
-def test_gemm_i8_extremes(oracle):
+def test_gemm_i8_extremes(oracle, tile):
     K = 8192
     xq = torch.full((40, K), 127, dtype=torch.int8)
     wq = torch.full((33, K), -127, dtype=torch.int8)
@@ -118,7 +126,7 @@ def test_gemm_i8_extremes(oracle):
     assert np.all(acc[:, ::2] == K * 127 * 127) and np.all(acc[:, 1::2] == -K * 127 * 127)
 
 
-def test_gemm_i8_one_hot_pins_operand_order():
+def test_gemm_i8_one_hot_pins_operand_order(tile):
     # xq has a single 1 at (m, k=m*3 % K); wq[n, k] = n*K + k small codes -> acc[m, n] = wq[n, k_m]
     M, N, K = 70, 45, 64
     xq = torch.zeros((M, K), dtype=torch.int8)
@@ -132,9 +140,9 @@ def test_gemm_i8_one_hot_pins_operand_order():
 
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("bias_kind", ["none", "f32", "bf16"])
-def test_linear_w8a8_epilogue_bit_exact(oracle, out_dtype, bias_kind):
-    M, N, K = 150, 200, 512
-    _say("linear_w8a8", out_dtype, bias_kind)
+@pytest.mark.parametrize("M,N,K", [(150, 200, 512), (77, 91, 144)])  # the second: odd N, rows not a multiple of 4
+def test_linear_w8a8_epilogue_bit_exact(oracle, tile, M, N, K, out_dtype, bias_kind):
+    _say("linear_w8a8", M, N, K, out_dtype, bias_kind, tile)
     x = make_x(M, K, 5, outlier_cols=3)
     w = make_x(N, K, 6) * 0.02
     xq, sx = oracle.c_quant_rowwise_i8(x.numpy())
@@ -217,7 +225,7 @@ def test_quant_tensor_fp8_codes_bit_exact(oracle):
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 1, 16), (33, 70, 144), (256, 128, 1024), (300, 260, 2048), (64, 96, 8192)])
-def test_linear_fp8_within_tolerance(oracle, M, N, K):
+def test_linear_fp8_within_tolerance(oracle, tile, M, N, K):
     _say("linear_fp8", M, N, K)
     x = make_x(M, K, 41)
     w = make_x(N, K, 42) * 0.02
@@ -238,7 +246,7 @@ def test_linear_fp8_within_tolerance(oracle, M, N, K):
     np.testing.assert_allclose(y32, yc, rtol=1e-2, atol=1e-3 * rms)
 
 
-def test_linear_fp8_one_hot_pins_operand_order(oracle):
+def test_linear_fp8_one_hot_pins_operand_order(oracle, tile):
     M, N, K = 40, 35, 128
     tab = oracle.np_e4m3fn_table()
     xq = np.zeros((M, K), np.uint8)

@@ -367,7 +367,33 @@ def cpu_baseline(workload, shape, unit, per_step):
     dt = t_total / reps
     scale = 1e9 if unit == "GB/s" else 1e12
     return {"value": per_step / dt / scale, "unit": unit, "cores": threads, "kind": "port",
-            "sample": f"{reps} full passes of the same shape (quantise + int8 GEMM + epilogue), {dt * 1e3:.2f} ms each"}
+            "sample": f"{reps} full passes of the same shape (quantise + int8 GEMM + epilogue), {dt * 1e3:.2f} ms each",
+            "reference_float_path": float_linear_cpu(M, N, K, bias is not None)}
+
+
+def float_linear_cpu(M, N, K, with_bias):
+    """The reference's own arithmetic for this call, F.linear (astrai/model/components/linear.py:21),
+    on the host in fp32 and bf16: a float GEMM by the vendor BLAS, not the quantized path."""
+    import torch
+    import torch.nn.functional as F
+
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(M, K, generator=g)
+    w = torch.randn(N, K, generator=g) * 0.02
+    b = torch.randn(N, generator=g) * 0.01 if with_bias else None
+    out = {"threads": torch.get_num_threads()}
+    for name, dt in (("fp32", torch.float32), ("bf16", torch.bfloat16)):
+        xx, ww, bb = x.to(dt), w.to(dt), (b.to(dt) if b is not None else None)
+        with torch.inference_mode():
+            F.linear(xx, ww, bb)
+            reps, t_total = 0, 0.0
+            while t_total < 2.0 and reps < 200:
+                t0 = time.perf_counter()
+                F.linear(xx, ww, bb)
+                t_total += time.perf_counter() - t0
+                reps += 1
+        out[name + "_ms"] = t_total / reps * 1e3
+    return out
 
 
 def main():

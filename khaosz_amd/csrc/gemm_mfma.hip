@@ -482,7 +482,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(GemmArgs p) {
             for (int q = 0; q < 4; ++q) {
               uint32_t vo = vbase;
               if (CHECK_M && mw + r0 + rq + q >= M) vo = OOB_OFFSET;
-              __builtin_amdgcn_raw_buffer_store_b32((uint32_t)acc[i][j][g * 4 + q], Cr, vo, (r0 + q) * rowb, 0);
+              __builtin_amdgcn_raw_buffer_store_b32((uint32_t)acc[i][j][g * 4 + q], Cr, vo, (r0 + q) * rowb, STORE_WT);
             }
           } else {
             float y[4];
@@ -502,7 +502,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(GemmArgs p) {
               for (int q = 0; q < 4; ++q) {
                 uint32_t vo = vbase;
                 if (CHECK_M && mw + r0 + rq + q >= M) vo = OOB_OFFSET;
-                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(y[q]), Cr, vo, (r0 + q) * rowb, 0);
+                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(y[q]), Cr, vo, (r0 + q) * rowb, STORE_WT);
               }
             } else if constexpr (PAIR) {
 #pragma unroll
@@ -515,14 +515,14 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(GemmArgs p) {
                 const uint32_t pk = __builtin_amdgcn_perm(other, mine, perm_sel);
                 uint32_t vo = vbase;
                 if (CHECK_M && mw + r0 + rq + 2 * h + (odd ? 1 : 0) >= M) vo = OOB_OFFSET;
-                __builtin_amdgcn_raw_buffer_store_b32(pk, Cr, vo, (r0 + 2 * h) * rowb, 0);
+                __builtin_amdgcn_raw_buffer_store_b32(pk, Cr, vo, (r0 + 2 * h) * rowb, STORE_WT);
               }
             } else {
 #pragma unroll
               for (int q = 0; q < 4; ++q) {
                 uint32_t vo = vbase;
                 if (CHECK_M && mw + r0 + rq + q >= M) vo = OOB_OFFSET;
-                __builtin_amdgcn_raw_buffer_store_b16((uint16_t)f32_to_bf16_bits(y[q]), Cr, vo, (r0 + q) * rowb, 0);
+                __builtin_amdgcn_raw_buffer_store_b16((uint16_t)f32_to_bf16_bits(y[q]), Cr, vo, (r0 + q) * rowb, STORE_WT);
               }
             }
           }

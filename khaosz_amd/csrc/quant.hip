@@ -20,9 +20,9 @@ __device__ __forceinline__ void quant_store(const uint4& v, float s, float rs, b
     uint2 o;
     o.x = pack_low_bytes(c[0], c[1], c[2], c[3]);
     o.y = pack_low_bytes(c[4], c[5], c[6], c[7]);
-    *reinterpret_cast<uint2*>(dst) = o;
+    store_wt(reinterpret_cast<uint2*>(dst), o);
   } else {
-    *reinterpret_cast<uint32_t*>(dst) = pack_low_bytes(c[0], c[1], c[2], c[3]);
+    store_wt(reinterpret_cast<uint32_t*>(dst), pack_low_bytes(c[0], c[1], c[2], c[3]));
   }
 }
 
@@ -221,9 +221,9 @@ __global__ __launch_bounds__(256) void cast_fp8_kernel(const void* __restrict__ 
       uint2 o;
       o.x = (uint32_t)w0;
       o.y = (uint32_t)w1;
-      *reinterpret_cast<uint2*>(q + v * EPV) = o;
+      store_wt(reinterpret_cast<uint2*>(q + v * EPV), o);
     } else {
-      *reinterpret_cast<uint32_t*>(q + v * EPV) = (uint32_t)w0;
+      store_wt(reinterpret_cast<uint32_t*>(q + v * EPV), (uint32_t)w0);
     }
   }
 }

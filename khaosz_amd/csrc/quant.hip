@@ -162,31 +162,52 @@ __global__ __launch_bounds__(256) void quant_row_wg_kernel(const void* __restric
 
 // ---------------------------------------------------------------- FP8 tensor
 
+constexpr int FP8_BATCH = 4;  // 16-byte loads a thread keeps in flight in the per-tensor passes
+constexpr int AMAX_THREADS = 1024;  // few, large workgroups: the pass ends with one atomic per workgroup
+
 __global__ void fill_u32_kernel(uint32_t* p, uint32_t v) {
   if (threadIdx.x == 0 && blockIdx.x == 0) *p = v;
 }
 
 template <bool BF16>
-__global__ __launch_bounds__(256) void amax_kernel(const void* __restrict__ x, int64_t nvec,
+__global__ __launch_bounds__(AMAX_THREADS) void amax_kernel(const void* __restrict__ x, int64_t nvec,
                                                     uint32_t* __restrict__ amax_bits) {
   constexpr int EPV = RowIn<BF16>::EPV;
   const uint4* src = reinterpret_cast<const uint4*>(x);
   float amax = 0.0f;
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-  for (int64_t v = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; v < nvec; v += stride) {
-    float f[EPV];
-    RowIn<BF16>::unpack(src[v], f);
-    amax = fmaxf(amax, vec_amax<EPV>(f));
+  // FP8_BATCH independent 16-byte loads in flight per thread; indices past the end re-read the
+  // last vector, which cannot change a maximum
+  for (int64_t v = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; v < nvec; v += FP8_BATCH * stride) {
+    uint4 t[FP8_BATCH];
+#pragma unroll
+    for (int u = 0; u < FP8_BATCH; ++u) {
+      const int64_t i = v + u * stride;
+      t[u] = src[i < nvec ? i : nvec - 1];
+    }
+#pragma unroll
+    for (int u = 0; u < FP8_BATCH; ++u) {
+      float f[EPV];
+      RowIn<BF16>::unpack(t[u], f);
+      amax = fmaxf(amax, vec_amax<EPV>(f));
+    }
   }
   amax = wave_max(amax);
   // one atomic per workgroup: same-address atomics serialise at the L2
-  __shared__ float wmax[4];
+  __shared__ float wmax[AMAX_THREADS / 64];
   if ((threadIdx.x & 63) == 0) wmax[threadIdx.x >> 6] = amax;
   __syncthreads();
   if (threadIdx.x == 0) {
-    const float m = fmaxf(fmaxf(wmax[0], wmax[1]), fmaxf(wmax[2], wmax[3]));
-    // |x| >= 0, so the IEEE bit patterns order like unsigned integers.
-    if (m > 0.0f) atomicMax(amax_bits, __float_as_uint(m));
+    float m = 0.0f;
+#pragma unroll
+    for (int w = 0; w < AMAX_THREADS / 64; ++w) m = fmaxf(m, wmax[w]);
+    // |x| >= 0, so the IEEE bit patterns order like unsigned integers.  Same-address atomics
+    // from 8 XCDs serialise at about 15 ns each (2048 of them cost 30 us), so look first (a device-scope load; a stale
+    // value only costs an atomic that was not needed): after the first few workgroups hardly
+    // any partial maximum still exceeds the running one.
+    const uint32_t mb = __float_as_uint(m);
+    if (m > 0.0f && mb > __hip_atomic_load(amax_bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
+      atomicMax(amax_bits, mb);
   }
 }
 
@@ -207,23 +228,34 @@ __global__ __launch_bounds__(256) void cast_fp8_kernel(const void* __restrict__ 
   if (blockIdx.x == 0 && threadIdx.x == 0) *scale = s;
   const uint4* src = reinterpret_cast<const uint4*>(x);
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-  for (int64_t v = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; v < nvec; v += stride) {
-    float f[EPV];
-    RowIn<BF16>::unpack(src[v], f);
+  for (int64_t v0 = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; v0 < nvec; v0 += FP8_BATCH * stride) {
+    uint4 t[FP8_BATCH];
 #pragma unroll
-    for (int i = 0; i < EPV; ++i) f[i] = fp8_prescale(f[i], s);
-    // v_cvt_pk_fp8_f32: two fp32 -> two OCP e4m3fn codes, round to nearest even.
-    int w0 = __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], 0, false);
-    w0 = __builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], w0, true);
-    if constexpr (BF16) {
-      int w1 = __builtin_amdgcn_cvt_pk_fp8_f32(f[4], f[5], 0, false);
-      w1 = __builtin_amdgcn_cvt_pk_fp8_f32(f[6], f[7], w1, true);
-      uint2 o;
-      o.x = (uint32_t)w0;
-      o.y = (uint32_t)w1;
-      store_wt(reinterpret_cast<uint2*>(q + v * EPV), o);
-    } else {
-      store_wt(reinterpret_cast<uint32_t*>(q + v * EPV), (uint32_t)w0);
+    for (int u = 0; u < FP8_BATCH; ++u) {
+      const int64_t i = v0 + u * stride;
+      t[u] = src[i < nvec ? i : nvec - 1];
+    }
+#pragma unroll
+    for (int u = 0; u < FP8_BATCH; ++u) {
+      const int64_t v = v0 + u * stride;
+      if (v >= nvec) break;
+      float f[EPV];
+      RowIn<BF16>::unpack(t[u], f);
+#pragma unroll
+      for (int i = 0; i < EPV; ++i) f[i] = fp8_prescale(f[i], s);
+      // v_cvt_pk_fp8_f32: two fp32 -> two OCP e4m3fn codes, round to nearest even.
+      int w0 = __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], 0, false);
+      w0 = __builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], w0, true);
+      if constexpr (BF16) {
+        int w1 = __builtin_amdgcn_cvt_pk_fp8_f32(f[4], f[5], 0, false);
+        w1 = __builtin_amdgcn_cvt_pk_fp8_f32(f[6], f[7], w1, true);
+        uint2 o;
+        o.x = (uint32_t)w0;
+        o.y = (uint32_t)w1;
+        store_wt(reinterpret_cast<uint2*>(q + v * EPV), o);
+      } else {
+        store_wt(reinterpret_cast<uint32_t*>(q + v * EPV), (uint32_t)w0);
+      }
     }
   }
 }
@@ -314,15 +346,18 @@ extern "C" int aq_quant_tensor_fp8(const void* x, int x_dtype, int64_t numel, ui
   const int epv = x_dtype == AQ_BF16 ? 8 : 4;
   const int64_t nvec = numel / epv;
   int64_t blocks = (nvec + 255) / 256;
-  if (blocks > 1024) blocks = 1024;  // 4 workgroups per CU, grid-stride beyond
+  if (blocks > 2048) blocks = 2048;  // 8 workgroups per CU, grid-stride beyond
   if (blocks < 1) blocks = 1;
+  int64_t ablocks = (nvec + aq::AMAX_THREADS * aq::FP8_BATCH - 1) / (aq::AMAX_THREADS * aq::FP8_BATCH);
+  if (ablocks > 256) ablocks = 256;  // one per CU
+  if (ablocks < 1) ablocks = 1;
   hipLaunchKernelGGL(aq::fill_u32_kernel, dim3(1), dim3(64), 0, st, amax_ws, 0u);
   if (x_dtype == AQ_BF16) {
-    hipLaunchKernelGGL((aq::amax_kernel<true>), dim3((unsigned)blocks), dim3(256), 0, st, x, nvec, amax_ws);
+    hipLaunchKernelGGL((aq::amax_kernel<true>), dim3((unsigned)ablocks), dim3(aq::AMAX_THREADS), 0, st, x, nvec, amax_ws);
     hipLaunchKernelGGL((aq::cast_fp8_kernel<true>), dim3((unsigned)blocks), dim3(256), 0, st, x, nvec,
                        amax_ws, q, scale);
   } else {
-    hipLaunchKernelGGL((aq::amax_kernel<false>), dim3((unsigned)blocks), dim3(256), 0, st, x, nvec, amax_ws);
+    hipLaunchKernelGGL((aq::amax_kernel<false>), dim3((unsigned)ablocks), dim3(aq::AMAX_THREADS), 0, st, x, nvec, amax_ws);
     hipLaunchKernelGGL((aq::cast_fp8_kernel<false>), dim3((unsigned)blocks), dim3(256), 0, st, x, nvec,
                        amax_ws, q, scale);
   }

@@ -69,33 +69,32 @@ __device__ __forceinline__ uint32_t quant_code_exact(float a, float s) {
   return (uint32_t)(int)n;
 }
 
-// The same codes for N values of one row at a fraction of the instructions.
-// With rs = rcp(s) (1 ulp) the exact product a * rs is within
-// 127.5 * 2^-23 = 1.5e-5 of the true quotient Q = a / s, whose own correctly
-// rounded value fl(Q) is within another 7.6e-6.  One fused multiply-add with
-// the constant 1.5 * 2^23 rounds a * rs to the nearest-even integer n and leaves
-// it in the low mantissa bits (so the low byte of the float IS the
-// two's-complement code); a second one gives the residual r = a * rs - n.
-// |a| never exceeds the row's amax = 127 s, so no clamp is needed.  Unless |r|
-// is within 2^-14 = 6.1e-5 of one half, rint(fl(Q)) = n.  A group in which some
-// value is that close is redone with the exact definition; with bf16 inputs
-// exact ties such as a = amax / 2 are common (one value in 400), so about half
-// of all 512-value groups take that path, and it is taken per group rather
-// than per value because a branch per value costs more than the divides it
-// saves.  `fast_ok` must be false for rows whose scale is not a normal float
-// (rcp is then useless).
+// The same codes for N values of one row without the range handling of a
+// general divide.  rs must be the once-refined reciprocal of s,
+//   y0 = rcp(s), rs = fma(fma(-s, y0, 1), y0, y0),
+// and then   q0 = a * rs,  q1 = fma(fma(-s, q0, a), rs, q0),  q2 = fma(fma(-s, q1, a), rs, q1)
+// is, operation for operation, the sequence the compiler emits for a correctly
+// rounded fp32 divide once its operands are in range (its scaling and fix-up
+// steps are the identity there): q2 = fl(a / s).  Adding 1.5 * 2^23 rounds q2 to
+// the nearest-even integer n and leaves it in the low mantissa bits, so the low
+// byte of the sum IS the two's-complement code; |a| never exceeds the row's
+// amax = 127 s, so no clamp is needed.  No branch, no per-value fallback: bf16
+// inputs hit exact ties (a = amax / 2 ...) once in 400 values, which makes any
+// "fast path unless near a tie" scheme take its slow path in most wavefronts.
+// `lean_ok` must be false for rows whose scale is outside [2^-64, 2^64], where
+// the residuals could leave the normal range; those rows take the full divide.
 template <int N>
-__device__ __forceinline__ void quant_codes(const float* a, float s, float rs, bool fast_ok, uint32_t* out) {
-  const float magic = 12582912.0f;          // 1.5 * 2^23
-  const float decided = 0.49993896484375f;  // 0.5 - 2^-14
-  float dmax = 0.0f;
+__device__ __forceinline__ void quant_codes(const float* a, float s, float rs, bool lean_ok, uint32_t* out) {
+  const float magic = 12582912.0f;  // 1.5 * 2^23
+  if (__builtin_expect(lean_ok, 1)) {
 #pragma unroll
-  for (int i = 0; i < N; ++i) {
-    const float um = __builtin_fmaf(a[i], rs, magic);
-    out[i] = __float_as_uint(um);
-    dmax = fmaxf(dmax, fabsf(__builtin_fmaf(a[i], rs, -(um - magic))));
-  }
-  if (__builtin_expect(!fast_ok || !(dmax <= decided), 0)) {
+    for (int i = 0; i < N; ++i) {
+      float q = a[i] * rs;
+      q = __builtin_fmaf(__builtin_fmaf(-s, q, a[i]), rs, q);
+      q = __builtin_fmaf(__builtin_fmaf(-s, q, a[i]), rs, q);
+      out[i] = __float_as_uint(q + magic);
+    }
+  } else {
 #pragma unroll
     for (int i = 0; i < N; ++i) out[i] = quant_code_exact(a[i], s);
   }

@@ -41,7 +41,8 @@ __device__ __forceinline__ float vec_amax(const float* f) {
 }
 
 // Symmetric absmax scale of one row from its wavefront-wide maximum:
-// s = amax / 127 (1 for an all-zero row), rs = rcp(s), and whether rs may be used.
+// s = amax / 127 (1 for an all-zero row), rs = the once-refined reciprocal of s
+// that quant_codes expects, and whether s is in the range where it may be used.
 struct RowScale {
   float s, rs;
   bool fast_ok;
@@ -50,8 +51,9 @@ __device__ __forceinline__ RowScale row_scale(float amax) {
   RowScale r;
   r.s = __fdiv_rn(amax, 127.0f);
   if (amax == 0.0f) r.s = 1.0f;
-  r.rs = __builtin_amdgcn_rcpf(r.s);
-  r.fast_ok = r.s >= 1.17549435e-38f;  // normal scale: rcp is finite and accurate to 1 ulp
+  const float y0 = __builtin_amdgcn_rcpf(r.s);
+  r.rs = __builtin_fmaf(__builtin_fmaf(-r.s, y0, 1.0f), y0, y0);
+  r.fast_ok = r.s >= 5.421010862427522e-20f && r.s <= 1.8446744073709552e19f;  // [2^-64, 2^64]
   return r;
 }
 

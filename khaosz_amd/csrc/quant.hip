@@ -76,10 +76,9 @@ __global__ __launch_bounds__(256) void quant_rowwise_i8_kernel(const void* __res
       }
     }
     amax = wave_max(amax);
-    float s = __fdiv_rn(amax, 127.0f);
-    if (amax == 0.0f) s = 1.0f;
-    const float rs = __builtin_amdgcn_rcpf(s);
-    const bool fast_ok = s >= 1.17549435e-38f;  // normal scale: rcp is finite and accurate to 1 ulp
+    const RowScale rsc = row_scale(amax);
+    const float s = rsc.s, rs = rsc.rs;
+    const bool fast_ok = rsc.fast_ok;
     if (lane == 0) scale[r] = s;
 #pragma unroll
     for (int i = 0; i < NC; ++i) {
@@ -148,10 +147,9 @@ __global__ __launch_bounds__(256) void quant_row_wg_kernel(const void* __restric
   if ((tid & 63) == 0) wmax[tid >> 6] = amax;
   __syncthreads();
   amax = fmaxf(fmaxf(wmax[0], wmax[1]), fmaxf(wmax[2], wmax[3]));
-  float s = __fdiv_rn(amax, 127.0f);
-  if (amax == 0.0f) s = 1.0f;
-  const float rs = __builtin_amdgcn_rcpf(s);
-  const bool fast_ok = s >= 1.17549435e-38f;  // normal scale: rcp is finite and accurate to 1 ulp
+  const RowScale rsc = row_scale(amax);
+  const float s = rsc.s, rs = rsc.rs;
+  const bool fast_ok = rsc.fast_ok;
   if (tid == 0) scale[row] = s;
 #pragma unroll
   for (int i = 0; i < NV; ++i) {

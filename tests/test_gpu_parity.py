@@ -84,6 +84,45 @@ def test_quant_rowwise_ties_and_strided_rows(oracle):
     assert np.array_equal(to_np(q2), qo) and np.array_equal(to_np(s2), so)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_quant_rowwise_scale_range_and_dense_ties(oracle, dtype):
+    """Rows whose scale sweeps the whole fp32 exponent range (the kernels switch to a full
+    divide outside [2^-64, 2^64]: both sides and both borders are hit), each row dense in exact
+    and near ties: multiples of amax/254 are half-integers after division by amax/127."""
+    K = 2048
+    exps = list(range(-140, 121, 4)) + [-64, -63, -65, 64, 63, 65, -71, -57, 57, 71]
+    g = torch.Generator().manual_seed(11)
+    rows = []
+    for e in exps:
+        amax = 127.0 * 2.0 ** e * (1.0 + 0.37 * torch.rand(1, generator=g).item())
+        k = torch.randint(-254, 255, (K,), generator=g).double()
+        r = (k * (amax / 254.0)).float()          # ties and integers in equal parts
+        r[::3] = (torch.randn(K, generator=g).double()[::3] * (amax / 3.0)).clamp(-amax, amax).float()
+        r[5] = amax
+        rows.append(r)
+    x = torch.stack(rows)
+    x = x[torch.isfinite(x).all(dim=1)]
+    xd = x.to(DEV, dtype)
+    q, s_ = ops.quant_rowwise_i8(xd)
+    if dtype == torch.bfloat16:
+        qo, so = oracle.c_quant_rowwise_i8(bf16_bits(xd), bf16_bits=True)
+    else:
+        qo, so = oracle.c_quant_rowwise_i8(to_np(xd))
+    assert np.array_equal(to_np(s_).view(np.uint32), so.view(np.uint32))
+    bad = np.argwhere(to_np(q) != qo)
+    assert bad.size == 0, f"first mismatches (row, col): {bad[:5].tolist()}"
+    # the same rows through the decode kernel that quantises in-kernel (bf16, up to 8 rows a call)
+    if dtype == torch.bfloat16:
+        wq = torch.zeros((64, K), dtype=torch.int8)
+        wq[torch.arange(64), torch.arange(64) * 31 % K] = 1      # y[m, n] = code of column 31n % K times sx
+        sw = torch.ones(64)
+        for r0 in range(0, xd.shape[0], 8):
+            xs = xd[r0:r0 + 8].contiguous()
+            y = ops.gemv_w8a8_decode(xs, wq.to(DEV), sw.to(DEV), None, out_dtype=torch.float32)
+            want = qo[r0:r0 + 8][:, (np.arange(64) * 31) % K].astype(np.float32) * so[r0:r0 + 8, None]
+            assert np.array_equal(to_np(y), want), f"rows {r0}.."
+
+
 def test_quant_rowwise_empty():
     q, s = ops.quant_rowwise_i8(torch.empty((0, 32), device=DEV))
     assert q.shape == (0, 32) and s.shape == (0,)

@@ -234,7 +234,7 @@ def bench_fp8(torch, ops, args, dev):
 
 def bench_block(torch, ops, args, dev):
     """BASELINE configs[4]: one int8-quantized 1B-class decoder block, 8 x 512 prefill then 64 decode steps."""
-    from khaosz_amd.block import ContiguousKV, DecoderBlock, decode_mask, rotary_table
+    from khaosz_amd.block import DecoderBlock, PagedKV, decode_mask, rotary_table
     from khaosz_amd.linear import quantize_model
 
     dt = torch.bfloat16
@@ -247,16 +247,20 @@ def bench_block(torch, ops, args, dev):
     tab = rotary_table(128, S + steps, device=dev)
     x = torch.randn(B, S, dim, device=dev).to(dt)
     xs = torch.randn(steps, B, 1, dim, device=dev).to(dt)
-    cache = ContiguousKV(B, S + steps, 4, 128, dev, dt)
+    page = 64  # the serving scheduler's default page size (astrai/inference/core/scheduler.py:26)
+    pages_per_seq = (S + steps + page - 1) // page
+    cache = PagedKV(B * pages_per_seq, page, 4, 128, dev, dt)
+    # physical pages dealt out in a fixed shuffled order, as after some allocation history
+    table = torch.randperm(B * pages_per_seq, generator=torch.Generator().manual_seed(8)).view(B, pages_per_seq).to(dev)
     fr = lambda a, n: tab[a:a + n].unsqueeze(0).expand(B, -1, -1)
     masks = [decode_mask(B, S + t + 1, dev, dt) for t in range(steps)]
 
     def prefill(i=0):
-        return blk(x, fr(0, S), None, cache.bind(S))
+        return blk(x, fr(0, S), None, cache.bind(table, S))
 
     def decode_all(i=0):
         for t in range(steps):
-            blk(xs[t], fr(S + t, 1), masks[t], cache.bind(S + t + 1))
+            blk(xs[t], fr(S + t, 1), masks[t], cache.bind(table, S + t + 1))
 
     ms_pre = graph_time_ms(torch, prefill, 10, 3)
     prefill()
@@ -282,7 +286,7 @@ def bench_block(torch, ops, args, dev):
     lin_ops = 2.0 * B * S * 45088768
     lin_bytes = 45088768
     return {
-        "workload": "decoder_block hidden=2048 16q/4kv x128 ffn=5632, 7 Linears W8A8, bf16; 8x512 prefill + 64 decode steps (M=8)",
+        "workload": "decoder_block hidden=2048 16q/4kv x128 ffn=5632, 7 Linears W8A8, bf16; 8x512 prefill through a paged KV cache (64-token pages) + 64 decode steps (M=8)",
         "value": ms_pre + steps * ms_dec, "unit": "ms", "prefill_ms": ms_pre, "decode_ms_per_step": ms_dec,
         "linears_prefill_ms": ms_lin_pre, "linears_prefill_tops": lin_ops / (ms_lin_pre * 1e-3) / 1e12,
         "linears_decode_ms_per_step": ms_lin_dec, "linears_decode_gbs": lin_bytes / (ms_lin_dec * 1e-3) / 1e9,

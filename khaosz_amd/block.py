@@ -4,10 +4,12 @@ quantized path can be exercised at the shapes a real model presents.
 Structure follows the reference (pre-norm residual block with GQA and a SwiGLU
 MLP), each piece citing the file it restates; only the seven projections are
 this package's own arithmetic, everything else is the same stock torch call the
-reference makes.  The KV cache here is a contiguous per-sequence buffer with the
-two methods attention needs (``write`` / ``gather``), standing in for the paged
-``KvcacheView`` (astrai/inference/core/cache.py:277-290), whose page management
-belongs to the serving layer.
+reference makes.  Two KV caches offer the two methods attention needs (``write`` / ``gather``,
+the ``KvcacheView`` interface, astrai/inference/core/cache.py:277-290): a
+contiguous per-sequence buffer, and a paged one with the storage layout and the
+write / gather semantics of the reference's ``Storage`` (cache.py:187-274).
+Page allocation, prefix sharing and eviction belong to the serving layer and are
+not restated: the page table is handed in.
 """
 from __future__ import annotations
 
@@ -71,6 +73,74 @@ class ContiguousKV:
         return self.k[:, :self.total_len], self.v[:, :self.total_len]
 
 
+class PagedKV:
+    """Paged KV cache for one block: pages ``[n_pages, page_size, Hkv, D]`` and a page table
+    ``[B, pages_per_sequence]`` of physical page ids, -1 for a logical page that is not
+    mapped (cache.py:187-274).  ``write`` places the new tokens at logical positions
+    ``total_len - S .. total_len`` page by page; rows whose page is unmapped are skipped.
+    ``gather`` materialises ``[B, total_len, Hkv, D]`` through the table, zeros where unmapped.
+    Which table entries are mapped is decided on a host copy of the table made at bind time,
+    so neither method synchronises with the device (the reference tests the device tensor,
+    ``cache.py:233,262``) and both can be captured in a HIP graph."""
+
+    def __init__(self, n_pages: int, page_size: int, n_kv_heads: int, head_dim: int, device, dtype):
+        self.page_size = page_size
+        self.k = torch.zeros((n_pages, page_size, n_kv_heads, head_dim), device=device, dtype=dtype)
+        self.v = torch.zeros_like(self.k)
+        self.page_table: Optional[Tensor] = None
+        self._mapped = None      # host bool [B, P]
+        self._safe = None        # device table with -1 replaced by 0
+        self._invalid = None     # device bool [B, P * page_size] or None when everything is mapped
+        self.total_len = 0
+
+    def bind(self, page_table: Optional[Tensor] = None, total_len: int = 0) -> "PagedKV":
+        if page_table is not None and page_table is not self.page_table:
+            host = page_table.detach().cpu()
+            self.page_table = page_table
+            self._mapped = host >= 0
+            self._safe = page_table.clamp(min=0)
+            self._invalid = None
+            if not bool(self._mapped.all()):
+                inv = (~self._mapped).unsqueeze(-1).expand(-1, -1, self.page_size).flatten(1, 2)
+                self._invalid = inv.to(page_table.device)
+        if self.page_table is None:
+            raise ValueError("bind() needs a page table")
+        self.total_len = total_len
+        return self
+
+    def write(self, layer_id: int, k: Tensor, v: Tensor) -> None:
+        S = k.size(1)
+        if S == 0:
+            return
+        start, ps = self.total_len - S, self.page_size
+        if start < 0 or (self.total_len + ps - 1) // ps > self.page_table.size(1):
+            raise ValueError("tokens fall outside the page table")
+        done = 0
+        for pi in range(start // ps, (self.total_len - 1) // ps + 1):
+            lo = max(pi * ps, start)
+            hi = min((pi + 1) * ps, self.total_len)
+            off, n = lo - pi * ps, hi - lo
+            rows = self._mapped[:, pi]
+            if bool(rows.all()):
+                phys = self._safe[:, pi]
+                self.k[phys, off:off + n] = k[:, done:done + n]
+                self.v[phys, off:off + n] = v[:, done:done + n]
+            elif bool(rows.any()):
+                sel = rows.nonzero().flatten().to(k.device)
+                phys = self._safe[sel, pi]
+                self.k[phys, off:off + n] = k[sel, done:done + n]
+                self.v[phys, off:off + n] = v[sel, done:done + n]
+            done += n
+
+    def gather(self, layer_id: int) -> Tuple[Tensor, Tensor]:
+        k = self.k[self._safe].flatten(1, 2)
+        v = self.v[self._safe].flatten(1, 2)
+        if self._invalid is not None:
+            m = self._invalid[:, :, None, None]
+            k, v = k.masked_fill(m, 0.0), v.masked_fill(m, 0.0)
+        return k[:, :self.total_len], v[:, :self.total_len]
+
+
 class GQA(nn.Module):
     """Grouped-query attention (astrai/model/components/attention.py:32-109), without the
     optional qk-norm and output gate that BASELINE config 5 leaves off."""
@@ -87,7 +157,7 @@ class GQA(nn.Module):
         self.o_proj = Linear(dim, dim)
 
     def forward(self, x: Tensor, rotary_emb: Tensor, attn_mask: Optional[Tensor] = None,
-                cache: Optional[ContiguousKV] = None) -> Tensor:
+                cache=None) -> Tensor:
         B, S, _ = x.shape
         q = self.q_proj(x).reshape(B, S, self.n_heads, self.head_dim)
         k = self.k_proj(x).reshape(B, S, self.n_kv_heads, self.head_dim)
@@ -135,7 +205,7 @@ class DecoderBlock(nn.Module):
                 m.reset_parameters()
 
     def forward(self, x: Tensor, rotary_emb: Tensor, attention_mask: Optional[Tensor] = None,
-                cache: Optional[ContiguousKV] = None) -> Tensor:
+                cache=None) -> Tensor:
         x = self.attention(self.input_norm(x), rotary_emb, attention_mask, cache) + x
         return self.mlp(self.post_attention_norm(x)) + x
 

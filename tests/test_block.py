@@ -7,7 +7,8 @@ import pytest
 import torch
 import torch.nn.functional as F
 
-from khaosz_amd.block import (ContiguousKV, DecoderBlock, GQA, RMSNorm, apply_rotary, decode_mask, rotary_table)
+from khaosz_amd.block import (ContiguousKV, DecoderBlock, GQA, PagedKV, RMSNorm, apply_rotary, decode_mask,
+                              rotary_table)
 from khaosz_amd.linear import QuantLinear, quantize_model
 
 
@@ -96,6 +97,53 @@ def test_block_residual_structure_and_decode_equals_prefill_on_cpu():
     assert torch.allclose(step[:, 0], full[:, S], atol=1e-5)
 
 
+def test_paged_kv_write_gather_round_trip_and_unmapped_pages():
+    """What the reference's cache tests check for Storage (tests/inference/test_cache.py:210-279):
+    tokens written through a page table come back in order through gather, across page borders,
+    in scattered physical pages, chunk by chunk; unmapped logical pages are skipped on write
+    and read back as zeros."""
+    B, H, D, ps = 3, 2, 4, 8
+    cache = PagedKV(n_pages=16, page_size=ps, n_kv_heads=H, head_dim=D, device="cpu", dtype=torch.float32)
+    table = torch.tensor([[5, 2, 9], [0, 7, 11], [3, 14, 1]])
+    g = torch.Generator().manual_seed(0)
+    k = torch.randn(B, 21, H, D, generator=g)
+    v = torch.randn(B, 21, H, D, generator=g)
+    cache.bind(table, 13).write(0, k[:, :13], v[:, :13])           # spans pages 0 and 1
+    cache.bind(table, 14).write(0, k[:, 13:14], v[:, 13:14])       # one decode token
+    cache.bind(table, 21).write(0, k[:, 14:], v[:, 14:])           # crosses into page 2
+    kk, vv = cache.bind(table, 21).gather(0)
+    assert torch.equal(kk, k) and torch.equal(vv, v)
+    kk, _ = cache.bind(table, 10).gather(0)
+    assert torch.equal(kk, k[:, :10])
+    assert torch.equal(cache.k[9, :5], k[0, 16:21])                 # sequence 0, logical page 2 -> physical 9
+    # sequence 1 has no third page: its tokens there are dropped, the others are kept
+    cache2 = PagedKV(16, ps, H, D, "cpu", torch.float32)
+    holes = torch.tensor([[5, 2, 9], [0, 7, -1], [3, 14, 1]])
+    cache2.bind(holes, 21).write(0, k, v)
+    kk, vv = cache2.gather(0)
+    assert torch.equal(kk[0], k[0]) and torch.equal(kk[2], k[2])
+    assert torch.equal(kk[1, :16], k[1, :16]) and not kk[1, 16:].any() and not vv[1, 16:].any()
+    with pytest.raises(ValueError):
+        cache.bind(table, 25).write(0, k[:, :1], v[:, :1])          # beyond the table
+
+
+def test_paged_cache_gives_the_block_the_same_outputs_as_the_contiguous_one():
+    blk = _block()
+    B, S, dim = 2, 9, 64
+    tab = rotary_table(16, 32)
+    x = torch.randn(B, S + 2, dim)
+    outs = []
+    for cache, bind in ((ContiguousKV(B, 32, 2, 16, "cpu", torch.float32), lambda c, n: c.bind(n)),
+                        (PagedKV(8, 4, 2, 16, "cpu", torch.float32),
+                         lambda c, n, t=torch.tensor([[6, 1, 3], [0, 5, 2]]): c.bind(t, n))):
+        o = [blk(x[:, :S], _freqs(tab, B, 0, S), None, bind(cache, S))]
+        for t in range(2):
+            o.append(blk(x[:, S + t:S + t + 1], _freqs(tab, B, S + t, 1),
+                         decode_mask(B, S + t + 1, "cpu", torch.float32), bind(cache, S + t + 1)))
+        outs.append(torch.cat(o, dim=1))
+    assert torch.equal(outs[0], outs[1])
+
+
 @pytest.mark.gpu
 def test_quantized_block_tracks_the_float_block():
     dev = "cuda:0"
@@ -131,13 +179,14 @@ def test_config5_block_prefill_then_decode_bf16():
         assert quantize_model(fblk) == 7
         xb = x.to(dt)
         full = fblk(xb, _freqs(tab, B, 0, S + steps))               # quantized, whole sequence (MFMA path)
-        cache = ContiguousKV(B, 256, 4, 128, dev, dt)
-        pre = fblk(xb[:, :S], _freqs(tab, B, 0, S), None, cache.bind(S))
+        cache = PagedKV(8, 64, 4, 128, dev, dt)                     # paged, 64-token pages, scattered
+        table = torch.tensor([[5, 0], [2, 7]], device=dev)
+        pre = fblk(xb[:, :S], _freqs(tab, B, 0, S), None, cache.bind(table, S))
         outs = [pre]
         for t in range(steps):                                      # decode path (M = B = 2)
             pos = S + t
             outs.append(fblk(xb[:, pos:pos + 1], _freqs(tab, B, pos, 1), decode_mask(B, pos + 1, dev, dt),
-                             cache.bind(pos + 1)))
+                             cache.bind(table, pos + 1)))
         seq = torch.cat(outs, dim=1)
     assert seq.shape == (B, S + steps, 2048) and seq.dtype == dt
     rel = ((full.float() - ref).norm() / ref.norm()).item()

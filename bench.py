@@ -381,8 +381,8 @@ def cpu_baseline(workload, shape, unit, per_step):
     bias = None if workload == "decode" else (rng.standard_normal(N) * 0.01).astype(np.float32)
     oracle.c_linear_w8a8(x[: min(M, 64)], wq, sw, bias, x_bf16_bits=True, bf16_out=True)  # warm the threads
     reps, t_total = 0, 0.0
-    budget = 6.0
-    while t_total < budget and reps < 400:
+    budget = 10.0  # seconds of CPU work per leg
+    while t_total < budget and reps < 20000:
         t0 = time.perf_counter()
         oracle.c_linear_w8a8(x, wq, sw, bias, x_bf16_bits=True, bf16_out=True)
         t_total += time.perf_counter() - t0

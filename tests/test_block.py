@@ -194,3 +194,39 @@ def test_config5_block_prefill_then_decode_bf16():
     # decode rows equal the prefill rows of the same tokens up to bf16 attention numerics
     rel_d = ((seq.float() - full.float()).norm() / full.float().norm()).item()
     assert rel_d < 1e-2, rel_d
+
+
+@pytest.mark.gpu
+def test_quantized_block_checkpoint_round_trip_through_safetensors(tmp_path):
+    """The reference saves and loads weights as safetensors state dicts (astrai/serialization.py:19-25,
+    astrai/model/automodel.py:54-91).  A quantized block's state dict (qweight / w_scale per
+    projection) survives that path bit for bit, and a float checkpoint with the reference's
+    ``*.weight`` keys loads into an already quantized block (quantised on load)."""
+    from safetensors.torch import load_file, save_file
+
+    dev = "cuda:0"
+    flt = _block(dim=256, heads=4, kv=2, ffn=704).to(dev)
+    save_file({k: v.contiguous() for k, v in flt.state_dict().items()}, str(tmp_path / "float.safetensors"))
+    qblk = _block(dim=256, heads=4, kv=2, ffn=704).to(dev)
+    qblk.load_state_dict(flt.state_dict())
+    assert quantize_model(qblk) == 7
+    sd = qblk.state_dict()
+    assert "attention.q_proj.qweight" in sd and "attention.q_proj.w_scale" in sd and "mlp.down.qweight" in sd
+    assert not any(k.endswith("_proj.weight") for k in sd)
+    save_file({k: v.contiguous() for k, v in sd.items()}, str(tmp_path / "quant.safetensors"))
+
+    x = torch.randn(2, 24, 256, device=dev)
+    tab = rotary_table(64, 64, device=dev)
+    with torch.inference_mode():
+        want = qblk(x, _freqs(tab, 2, 0, 24))
+        # quantized checkpoint -> fresh quantized block
+        a = _block(dim=256, heads=4, kv=2, ffn=704).to(dev)
+        quantize_model(a)
+        a.load_state_dict(load_file(str(tmp_path / "quant.safetensors"), device=dev))
+        assert torch.equal(a(x, _freqs(tab, 2, 0, 24)), want)
+        # float checkpoint with the reference's key names -> fresh quantized block
+        b = _block(dim=256, heads=4, kv=2, ffn=704).to(dev)
+        quantize_model(b)
+        b.load_state_dict(load_file(str(tmp_path / "float.safetensors"), device=dev))
+        assert torch.equal(b.attention.q_proj.qweight, qblk.attention.q_proj.qweight)
+        assert torch.equal(b(x, _freqs(tab, 2, 0, 24)), want)

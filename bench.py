@@ -6,7 +6,7 @@
 A "step" is one pass of the hot path over one batch of synthetic input that is
 already resident in HBM:
 
-  decode  (default; BASELINE configs[1], M=16)  x bf16 [16, 2048] -> per-token int8 quantise ->
+  decode  (default; benchmark configuration 1 of 5 (0-based), M=16)  x bf16 [16, 2048] -> per-token int8 quantise ->
           int8 GEMV against W int8 [8192, 2048] -> dequant -> y bf16.  HBM-bound; value = GB/s of
           algorithmic bytes N*K + 4N + 2MK + 2MN.  The weight rotates over 40 distinct buffers
           (671 MB) so that no step finds its weight in the 256 MB last-level cache.
@@ -233,7 +233,7 @@ def bench_fp8(torch, ops, args, dev):
 
 
 def bench_block(torch, ops, args, dev):
-    """BASELINE configs[4]: one int8-quantized 1B-class decoder block, 8 x 512 prefill then 64 decode steps."""
+    """benchmark configuration 4 of 5 (0-based): one int8-quantized 1B-class decoder block, 8 x 512 prefill then 64 decode steps."""
     from khaosz_amd.block import DecoderBlock, PagedKV, decode_mask, rotary_table
     from khaosz_amd.linear import quantize_model
 

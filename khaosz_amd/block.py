@@ -143,7 +143,7 @@ class PagedKV:
 
 class GQA(nn.Module):
     """Grouped-query attention (astrai/model/components/attention.py:32-109), without the
-    optional qk-norm and output gate that BASELINE config 5 leaves off."""
+    optional qk-norm and output gate that benchmark configuration 5 leaves off."""
 
     def __init__(self, dim: int, n_heads: int, n_kv_heads: int, layer_id: int = 0):
         super().__init__()

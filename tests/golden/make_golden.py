@@ -10,7 +10,7 @@ seeded torch/numpy draws, so the fixtures can be regenerated bit for bit:
 
 small.npz      full tensors of a tiny case (M=8, K=64, N=16) for every stage
 config1.json   SHA-256 of the codes / scales / accumulators / outputs of
-               BASELINE config 1 (X 64x2048 with 4 outlier columns x20,
+               benchmark configuration 1 (X 64x2048 with 4 outlier columns x20,
                W 2048x2048 N(0, 0.02), seed 0)
 """
 import hashlib

@@ -1,4 +1,4 @@
-"""The decoder block that hosts the quantized Linears (BASELINE config 5).
+"""The decoder block that hosts the quantized Linears (benchmark configuration 5).
 CPU tests pin the float restatement against closed forms and a hand-written
 attention; GPU tests put QuantLinear into it through quantize_model."""
 import math

@@ -300,7 +300,7 @@ def test_linear_fp8_one_hot_pins_operand_order(oracle, tile):
 # -------------------------------------------------------------- module level
 
 def test_config1_quant_linear_matches_oracle_and_float_reference(oracle):
-    """BASELINE config 1: X 64x2048 fp32 with 4 outlier columns x20, W 2048x2048 N(0, 0.02)."""
+    """benchmark configuration 1: X 64x2048 fp32 with 4 outlier columns x20, W 2048x2048 N(0, 0.02)."""
     g = torch.Generator().manual_seed(0)
     x = torch.randn(64, 2048, generator=g)
     cols = torch.randperm(2048, generator=g)[:4]
@@ -383,7 +383,7 @@ def test_quantize_model_on_gpu_preserves_outputs_within_quantisation_error():
 # ------------------------------------------- full-size, size-independent checks
 
 def test_full_size_prefill_checksum_of_checksums(oracle):
-    """BASELINE config 3 at full size (M=4096, K=N=2048, 1 % outlier channels x10)."""
+    """benchmark configuration 3 at full size (M=4096, K=N=2048, 1 % outlier channels x10)."""
     M, N, K = 4096, 2048, 2048
     x = make_x(M, K, 51, outlier_cols=20, outlier_gain=10.0).to(torch.bfloat16).to(DEV)
     w = (make_x(N, K, 52) * 0.02).to(DEV)
@@ -414,7 +414,7 @@ def test_full_size_prefill_checksum_of_checksums(oracle):
 
 
 def test_full_size_fp8_linearity_in_scales(oracle):
-    """BASELINE config 4 at full size (M=2048, K=8192, N=2048)."""
+    """benchmark configuration 4 at full size (M=2048, K=8192, N=2048)."""
     M, N, K = 2048, 2048, 8192
     x = make_x(M, K, 61).to(torch.bfloat16).to(DEV)
     w = (make_x(N, K, 62) * 0.02).to(DEV)

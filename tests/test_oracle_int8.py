@@ -148,7 +148,7 @@ def test_epilogue_c_equals_numpy_f32_and_bf16(oracle):
 
 
 def _config1(seed=0):
-    """BASELINE config 1: X 64x2048 N(0,1) with 4 seeded outlier columns x20,
+    """benchmark configuration 1: X 64x2048 N(0,1) with 4 seeded outlier columns x20,
     W 2048x2048 N(0, 0.02)."""
     g = torch.Generator().manual_seed(seed)
     x = torch.randn(64, 2048, generator=g)

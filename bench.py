@@ -235,7 +235,7 @@ def bench_fp8(torch, ops, args, dev):
 def bench_block(torch, ops, args, dev):
     """benchmark configuration 4 of 5 (0-based): one int8-quantized 1B-class decoder block, 8 x 512 prefill then 64 decode steps."""
     from khaosz_amd.block import DecoderBlock, PagedKV, decode_mask, rotary_table
-    from khaosz_amd.linear import quantize_model
+    from khaosz_amd.linear import fuse_shared_inputs, quantize_model
 
     dt = torch.bfloat16
     B, S, steps, dim = 8, 512, 64, 2048
@@ -262,16 +262,21 @@ def bench_block(torch, ops, args, dev):
         for t in range(steps):
             blk(xs[t], fr(S + t, 1), masks[t], cache.bind(table, S + t + 1))
 
+    # first with the seven projections launched one by one, as the reference's forward calls them,
+    # then with q/k/v and up/gate fused into one projection each (bit-identical outputs)
+    ms_pre_sep = graph_time_ms(torch, prefill, 10, 3)
+    prefill()
+    ms_dec_sep = graph_time_ms(torch, decode_all, 3, 2) / steps
+    fuse_shared_inputs(blk)
     ms_pre = graph_time_ms(torch, prefill, 10, 3)
     prefill()
     ms_dec = graph_time_ms(torch, decode_all, 3, 2) / steps
 
-    # The seven Linears alone, at the shapes and in the order the block calls them (same modules,
+    # The Linears alone (q/k/v and up/gate fused), at the shapes and in the order the block calls them (same modules,
     # inputs of the right shape): what of the block's time is this library's, what is the stock
     # torch attention / RoPE / norm / KV work around it.
     att, mlp = blk.attention, blk.mlp
-    lin_calls = [(att.q_proj, dim), (att.k_proj, dim), (att.v_proj, dim), (att.o_proj, dim),
-                 (mlp.up, dim), (mlp.gate, dim), (mlp.down, 5632)]
+    lin_calls = [(att._qkv, dim), (att.o_proj, dim), (mlp._upgate, dim), (mlp.down, 5632)]
 
     def linears_only(rows):
         ins = {k: torch.randn(rows, k, device=dev).to(dt) for k in (dim, 5632)}
@@ -288,6 +293,7 @@ def bench_block(torch, ops, args, dev):
     return {
         "workload": "decoder_block hidden=2048 16q/4kv x128 ffn=5632, 7 Linears W8A8, bf16; 8x512 prefill through a paged KV cache (64-token pages) + 64 decode steps (M=8)",
         "value": ms_pre + steps * ms_dec, "unit": "ms", "prefill_ms": ms_pre, "decode_ms_per_step": ms_dec,
+        "separate_projections": {"prefill_ms": ms_pre_sep, "decode_ms_per_step": ms_dec_sep},
         "linears_prefill_ms": ms_lin_pre, "linears_prefill_tops": lin_ops / (ms_lin_pre * 1e-3) / 1e12,
         "linears_decode_ms_per_step": ms_lin_dec, "linears_decode_gbs": lin_bytes / (ms_lin_dec * 1e-3) / 1e9,
         "non_linear_prefill_ms": ms_pre - ms_lin_pre, "non_linear_decode_ms_per_step": ms_dec - ms_lin_dec,

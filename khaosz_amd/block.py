@@ -20,7 +20,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 from torch import Tensor
 
-from .linear import Linear
+from .linear import Linear, QuantLinear
 
 
 class RMSNorm(nn.Module):
@@ -155,13 +155,27 @@ class GQA(nn.Module):
         self.k_proj = Linear(dim, n_kv_heads * self.head_dim)
         self.v_proj = Linear(dim, n_kv_heads * self.head_dim)
         self.o_proj = Linear(dim, dim)
+        self._qkv: Optional[QuantLinear] = None  # not a registered child: the state dict keeps q/k/v keys
+
+    def fuse_projections(self) -> bool:
+        """q, k and v read the same input (attention.py:83-85): once they are quantized, run them
+        as one ``[Hq*D + 2*Hkv*D, dim]`` projection -- one activation quantisation, one launch."""
+        if self._qkv is None and all(isinstance(m, QuantLinear) for m in (self.q_proj, self.k_proj, self.v_proj)):
+            object.__setattr__(self, "_qkv", QuantLinear.concat([self.q_proj, self.k_proj, self.v_proj]))
+            return True
+        return False
 
     def forward(self, x: Tensor, rotary_emb: Tensor, attn_mask: Optional[Tensor] = None,
                 cache=None) -> Tensor:
         B, S, _ = x.shape
-        q = self.q_proj(x).reshape(B, S, self.n_heads, self.head_dim)
-        k = self.k_proj(x).reshape(B, S, self.n_kv_heads, self.head_dim)
-        v = self.v_proj(x).reshape(B, S, self.n_kv_heads, self.head_dim)
+        if self._qkv is not None:
+            nq, nkv = self.n_heads * self.head_dim, self.n_kv_heads * self.head_dim
+            q, k, v = self._qkv(x).split((nq, nkv, nkv), dim=-1)
+        else:
+            q, k, v = self.q_proj(x), self.k_proj(x), self.v_proj(x)
+        q = q.reshape(B, S, self.n_heads, self.head_dim)
+        k = k.reshape(B, S, self.n_kv_heads, self.head_dim)
+        v = v.reshape(B, S, self.n_kv_heads, self.head_dim)
         q, k = apply_rotary(q, rotary_emb), apply_rotary(k, rotary_emb)
         if cache is not None:
             cache.write(self.layer_id, k, v)
@@ -183,8 +197,19 @@ class MLP(nn.Module):
         self.up = Linear(dim, dim_ffn)
         self.gate = Linear(dim, dim_ffn)
         self.down = Linear(dim_ffn, dim)
+        self._upgate: Optional[QuantLinear] = None
+
+    def fuse_projections(self) -> bool:
+        """up and gate read the same input (mlp.py:25): one ``[2*dim_ffn, dim]`` projection."""
+        if self._upgate is None and isinstance(self.up, QuantLinear) and isinstance(self.gate, QuantLinear):
+            object.__setattr__(self, "_upgate", QuantLinear.concat([self.up, self.gate]))
+            return True
+        return False
 
     def forward(self, x: Tensor) -> Tensor:
+        if self._upgate is not None:
+            up, gate = self._upgate(x).chunk(2, dim=-1)
+            return self.down(up * F.silu(gate))
         return self.down(self.up(x) * F.silu(self.gate(x)))
 
 

@@ -14,7 +14,7 @@ from __future__ import annotations
 
 import logging
 import math
-from typing import Iterable, Optional, Set
+from typing import Iterable, Optional, Sequence, Set
 
 import torch
 import torch.nn as nn
@@ -91,6 +91,35 @@ class QuantLinear(Linear):
         if base.bias is not None:
             q.bias = nn.Parameter(base.bias.detach().clone(), requires_grad=False)
         return q
+
+    @classmethod
+    def concat(cls, parts: Sequence["QuantLinear"]) -> "QuantLinear":
+        """One module computing ``cat([p(x) for p in parts], -1)`` for projections that read the
+        same input (q/k/v: attention.py:83-85; up/gate: mlp.py:25): the activation is quantised
+        once and the weights are streamed by one launch.  Per-channel weight scales and per-token
+        activation scales make every output element the same arithmetic as in its own module, so
+        the result is bit-identical.  Afterwards the parts' ``qweight`` / ``w_scale`` (and bias)
+        are row slices of the fused buffers: no second copy of the weights is kept."""
+        parts = list(parts)
+        if not parts or any(not isinstance(p, QuantLinear) for p in parts):
+            raise ValueError("concat needs QuantLinear modules")
+        if len({p.in_dim for p in parts}) != 1 or len({p.bias is None for p in parts}) != 1:
+            raise ValueError("parts must share in_dim and all have, or all lack, a bias")
+        dev = parts[0].qweight.device
+        fused = cls(parts[0].in_dim, sum(p.out_dim for p in parts), bias=parts[0].bias is not None, device=dev)
+        fused.qweight = torch.cat([p.qweight for p in parts], dim=0)
+        fused.w_scale = torch.cat([p.w_scale for p in parts], dim=0)
+        if fused.bias is not None:
+            fused.bias = nn.Parameter(torch.cat([p.bias.detach() for p in parts], dim=0), requires_grad=False)
+        row = 0
+        for p in parts:
+            n = p.out_dim
+            p.qweight = fused.qweight[row:row + n]
+            p.w_scale = fused.w_scale[row:row + n]
+            if p.bias is not None:
+                p.bias = nn.Parameter(fused.bias.detach()[row:row + n], requires_grad=False)
+            row += n
+        return fused
 
     def load_float_weight(self, w: Tensor) -> None:
         if tuple(w.shape) != tuple(self.qweight.shape):
@@ -210,6 +239,19 @@ class Fp8Linear(Linear):
 
 TARGET_MODULES_ATTN = {"q_proj", "k_proj", "v_proj", "o_proj"}
 TARGET_MODULES_FFN = {"up", "gate", "down"}
+
+
+def fuse_shared_inputs(model: nn.Module) -> int:
+    """Call ``fuse_projections()`` on every module that offers it (attention and MLP blocks whose
+    projections read one input); returns how many fused modules were built.  Run it after
+    ``quantize_model`` and after loading weights: the fused module owns the weight storage from
+    then on."""
+    n = 0
+    for m in model.modules():
+        f = getattr(m, "fuse_projections", None)
+        if callable(f):
+            n += int(f())
+    return n
 
 
 def _is_float_linear(m: nn.Module, extra: Iterable[type]) -> bool:

@@ -230,3 +230,33 @@ def test_quantized_block_checkpoint_round_trip_through_safetensors(tmp_path):
         b.load_state_dict(load_file(str(tmp_path / "float.safetensors"), device=dev))
         assert torch.equal(b.attention.q_proj.qweight, qblk.attention.q_proj.qweight)
         assert torch.equal(b(x, _freqs(tab, 2, 0, 24)), want)
+
+
+@pytest.mark.gpu
+def test_fused_shared_input_projections_are_bit_identical():
+    """q/k/v and up/gate run as one concatenated projection each: same bits as the seven separate
+    modules on both the prefill (MFMA GEMM) and the decode (GEMV) path, same state-dict keys, and a
+    later load_state_dict reaches the fused storage because the parts are views of it."""
+    from khaosz_amd import fuse_shared_inputs
+
+    dev, dt = "cuda:0", torch.bfloat16
+    a = _block(dim=256, heads=4, kv=2, ffn=704).to(dev).to(dt)
+    b = _block(dim=256, heads=4, kv=2, ffn=704).to(dev).to(dt)
+    b.load_state_dict(a.state_dict())
+    assert quantize_model(a) == 7 and quantize_model(b) == 7
+    keys = set(b.state_dict().keys())
+    assert fuse_shared_inputs(b) == 2 and fuse_shared_inputs(b) == 0
+    assert set(b.state_dict().keys()) == keys
+    assert b.attention._qkv.out_dim == 256 + 2 * 128 and b.mlp._upgate.out_dim == 2 * 704
+    assert b.attention.k_proj.qweight.data_ptr() == b.attention._qkv.qweight[256:].data_ptr()
+    tab = rotary_table(64, 64, device=dev)
+    x = torch.randn(2, 40, 256, device=dev).to(dt)
+    with torch.inference_mode():
+        assert torch.equal(b(x, _freqs(tab, 2, 0, 40)), a(x, _freqs(tab, 2, 0, 40)))          # M = 80
+        xd = x[:, :3].contiguous()
+        assert torch.equal(b(xd, _freqs(tab, 2, 0, 3)), a(xd, _freqs(tab, 2, 0, 3)))          # M = 6
+        # new weights loaded after fusing land in the fused buffers
+        c = _block(dim=256, heads=4, kv=2, ffn=704).to(dev).to(dt)
+        quantize_model(c)
+        b.load_state_dict(c.state_dict())
+        assert torch.equal(b(x, _freqs(tab, 2, 0, 40)), c(x, _freqs(tab, 2, 0, 40)))

@@ -24,14 +24,19 @@
 
 namespace aq {
 
-// Two shapes of workgroup, both 8 wavefronts (two per SIMD) of 64 x 64 sub-tiles:
-//   WM = 4, WK = 1: 256 x 128 tile, 4 x 2 wavefronts, 3 LDS stages of 48 KiB;
-//   WM = 2, WK = 2: 128 x 128 tile, 2 x 2 x 2 wavefronts (the last factor splits
-//                   each K step), 4 LDS stages of 32 KiB.
+// Shapes of workgroup, all 8 wavefronts (two per SIMD), WM x 2 x WK of them, each
+// accumulating a (32 TM) x 64 sub-tile:
+//   WM = 4, TM = 2, WK = 1: 256 x 128 tile, 3 LDS stages of 48 KiB;
+//   WM = 2, TM = 2, WK = 2: 128 x 128 tile, 4 LDS stages of 32 KiB, the two wavefronts of a
+//                           sub-tile split every K step.
+// With WK = 2 the pair exchanges half of its accumulators through LDS at the end, so that
+// each wavefront finishes (and stores) 16 TM x 64 of the sums.
+// (WM = 2, TM = 4, WK = 2 -- a 256 x 128 tile of 128 x 64 sub-tiles, 6 fragment reads per
+// 8 MFMAs instead of 8 -- also builds, and measures 10 % slower than the first shape.)
 constexpr int BN = 128, BK = 128;
 constexpr int WAVES_N = 2, NWAVES = 8, NTHREADS = NWAVES * 64;
-constexpr int WAVE_M = 64, WAVE_N = BN / WAVES_N;
-constexpr int TM = WAVE_M / 32, TN = WAVE_N / 32;
+constexpr int WAVE_N = BN / WAVES_N;
+constexpr int TN = WAVE_N / 32;
 constexpr int B_LOADS = BN * BK / 16 / NTHREADS;  // 16-byte vectors per thread per K step
 constexpr int BM_MAX = 256;
 constexpr int NUM_XCD = 8;
@@ -131,11 +136,14 @@ __device__ __forceinline__ void sched_pattern() {
   }
 }
 
-template <bool FP8, int OUT, int WM, int WK>
+template <bool FP8, int OUT, int WM, int TM, int WK>
 __global__ __launch_bounds__(NTHREADS) void gemm_kernel(GemmArgs p) {
   static_assert(WM * WAVES_N * WK == NWAVES, "8 wavefronts per workgroup");
+  static_assert(TM % WK == 0, "the K-split pair divides the sub-tile's row blocks");
+  constexpr int WAVE_M = 32 * TM;
   constexpr int BM = WM * WAVE_M;
-  constexpr int NSTAGE = WK == 1 ? 3 : 4;
+  constexpr int TME = TM / WK;  // row blocks a wavefront finishes and stores
+  constexpr int NSTAGE = BM == 256 ? 3 : 4;
   constexpr int A_LOADS = BM * BK / 16 / NTHREADS;
   // NSTAGE stages of [A tile BM x 128 B][B tile 128 x 128 B], rows unpadded.
   // Global->LDS loads land 64 lanes x 16 B contiguously (8 rows of 128 B), so
@@ -166,7 +174,8 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(GemmArgs p) {
 
   const int col = lane & 31;
   const int rq = (lane >> 5) * 4;  // row offset of this lane's half inside each group of 8 rows
-  const int mw = __builtin_amdgcn_readfirstlane(m0 + wave_m * WAVE_M);  // wavefront-uniform: keep it scalar
+  // first row of the part of the sub-tile this wavefront finishes (wavefront-uniform: kept scalar)
+  const int mw = __builtin_amdgcn_readfirstlane(m0 + wave_m * WAVE_M + wave_k * (32 * TME));
 
   // One load instruction of a wavefront fills 1 KiB = 8 tile rows.  Wavefront w
   // owns the 8-row groups w, w+NWAVES, w+2*NWAVES, ... of A and of B.
@@ -297,7 +306,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(GemmArgs p) {
   // as one scalar per 32x32 tile column.  Nothing is done with the values until
   // the epilogue (bias stays a raw bit pattern), so no wait is placed here.
   float sx1 = 1.0f, sw1 = 1.0f;
-  float sxr[TM][4][4];  // [i][g][q]: row i*32 + g*8 + rq + q
+  float sxr[TME][4][4];  // [i][g][q]: row mw + i*32 + g*8 + rq + q
   float swn[TN];
   uint32_t bias_raw[TN];
   const bool has_bias = !FP8 && OUT != OUT_I32 && p.bias != nullptr;
@@ -310,10 +319,10 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(GemmArgs p) {
       // rows past M fall outside the descriptor and read as zero (their outputs are never stored)
       const int rows_left = __builtin_amdgcn_readfirstlane((M - mw) > 0 ? (M - mw) : 0);
       const __amdgpu_buffer_rsrc_t Sr =
-          make_rsrc(p.sx + (rows_left ? mw : 0), (uint32_t)(rows_left < WAVE_M ? rows_left : WAVE_M) * 4u);
+          make_rsrc(p.sx + (rows_left ? mw : 0), (uint32_t)(rows_left < 32 * TME ? rows_left : 32 * TME) * 4u);
       if ((M & 3) == 0) {  // uniform: the 4 rows of a float4 are all in or all out, and 16-byte aligned
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
+        for (int i = 0; i < TME; ++i)
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
             const uint4 t = buffer_load_16(Sr, (uint32_t)(i * 32 + g * 8 + rq) * 4u);
@@ -324,7 +333,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(GemmArgs p) {
           }
       } else {
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
+        for (int i = 0; i < TME; ++i)
 #pragma unroll
           for (int g = 0; g < 4; ++g)
 #pragma unroll
@@ -347,7 +356,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(GemmArgs p) {
 #pragma unroll
   for (int q = 0; q < NLOADS; ++q) issue_load(0, 0, q);
   asm volatile("" ::: "memory");  // keep the request order: stage 0, epilogue operands, the other stages
-  if (wave_k == 0) load_epilogue_operands();  // uniform: only these wavefronts run the epilogue
+  load_epilogue_operands();
   asm volatile("" ::: "memory");
 #pragma unroll
   for (int st = 1; st < NSTAGE; ++st)
@@ -405,32 +414,47 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(GemmArgs p) {
   AQ_WAIT_VMCNT(0);  // drain the padding loads before the workgroup's LDS can be released or reused
 
   if constexpr (WK == 2) {
-    // The two wavefronts of a sub-tile hold the sums over their halves of every K step.  The
-    // second one parks its accumulators in LDS (16 KiB per sub-tile, over the stage buffers,
-    // which nobody reads any more once every wavefront is past this barrier); the first adds
-    // them and runs the epilogue alone.  int32 sums are exact in any order; FP8 partial sums
-    // are fp32, inside the stated tolerance.
+    // The two wavefronts of a sub-tile hold the sums over their halves of every K step.  Each
+    // keeps half of the row blocks (the first wavefront the upper ones) and parks the other half
+    // in LDS for its partner (over the stage buffers, which nobody reads any more once every
+    // wavefront is past the barrier); then both add what the partner left for them and run the
+    // epilogue on their half.  int32 sums are exact in any order; FP8 partial sums are fp32,
+    // inside the stated tolerance.
     __syncthreads();
     using part_t = std::conditional_t<FP8, v4f, v4i>;
-    part_t* red = reinterpret_cast<part_t*>(smem) + wave_mn * 1024 + lane;
-    if (wave_k == 1) {
+    constexpr int SLOT = TME * TN * 4 * 64;  // part_t elements one wavefront parks
+    part_t* mine = reinterpret_cast<part_t*>(smem) + (wave_mn * 2 + wave_k) * SLOT + lane;
+    part_t* theirs = reinterpret_cast<part_t*>(smem) + (wave_mn * 2 + (wave_k ^ 1)) * SLOT + lane;
+    static_assert(NWAVES * SLOT * 16 <= NSTAGE * STAGE, "the parked accumulators fit the stage buffers");
+    if (wave_k == 0) {  // uniform
 #pragma unroll
-      for (int i = 0; i < TM; ++i)
+      for (int i = 0; i < TME; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
 #pragma unroll
           for (int g = 0; g < 4; ++g)
-            red[((i * TN + j) * 4 + g) * 64] = part_t{acc[i][j][g * 4], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
+            mine[((i * TN + j) * 4 + g) * 64] = part_t{acc[TME + i][j][g * 4], acc[TME + i][j][g * 4 + 1],
+                                                       acc[TME + i][j][g * 4 + 2], acc[TME + i][j][g * 4 + 3]};
+    } else {
+#pragma unroll
+      for (int i = 0; i < TME; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+#pragma unroll
+          for (int g = 0; g < 4; ++g)
+            mine[((i * TN + j) * 4 + g) * 64] =
+                part_t{acc[i][j][g * 4], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
+          acc[i][j] = acc[TME + i][j];  // the lower row blocks move to the front: the epilogue indexes from 0
+        }
     }
     __syncthreads();
-    if (wave_k == 1) return;
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+    for (int i = 0; i < TME; ++i)
 #pragma unroll
       for (int j = 0; j < TN; ++j)
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-          const part_t t = red[((i * TN + j) * 4 + g) * 64];
+          const part_t t = theirs[((i * TN + j) * 4 + g) * 64];
 #pragma unroll
           for (int q = 0; q < 4; ++q) acc[i][j][g * 4 + q] += t[q];
         }
@@ -456,7 +480,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(GemmArgs p) {
   const bool odd = lane & 1;
   const uint32_t perm_sel = odd ? 0x03020706u : 0x05040100u;
   const uint32_t rowb = (uint32_t)N * ESZ;
-  const bool rows_inside = mw + WAVE_M <= M;  // uniform
+  const bool rows_inside = mw + 32 * TME <= M;  // uniform
   // CHECK_M: some rows of this wavefront are past M.  PAIR: the bf16 dword path.
   auto store_all = [&](auto check_c, auto pair_c) {
     constexpr bool CHECK_M = decltype(check_c)::value;
@@ -473,7 +497,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(GemmArgs p) {
           n_ok ? (uint32_t)rq * rowb + (uint32_t)(PAIR ? (cj & ~1) : cj) * ESZ + (PAIR && odd ? rowb : 0u)
                : OOB_OFFSET;
 #pragma unroll
-      for (int i = 0; i < TM; ++i) {
+      for (int i = 0; i < TME; ++i) {
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
           const int r0 = i * 32 + g * 8;  // + rq + q : row inside the wavefront's 128
@@ -560,9 +584,9 @@ static int launch(GemmArgs& a, hipStream_t st) {
   a.tiles_n = (a.N + BN - 1) / BN;
   const unsigned grid = (unsigned)(a.tiles_m * a.tiles_n);
   if (small)
-    hipLaunchKernelGGL((gemm_kernel<FP8, OUT, 2, 2>), dim3(grid), dim3(NTHREADS), 0, st, a);
+    hipLaunchKernelGGL((gemm_kernel<FP8, OUT, 2, 2, 2>), dim3(grid), dim3(NTHREADS), 0, st, a);
   else
-    hipLaunchKernelGGL((gemm_kernel<FP8, OUT, 4, 1>), dim3(grid), dim3(NTHREADS), 0, st, a);
+    hipLaunchKernelGGL((gemm_kernel<FP8, OUT, 4, 2, 1>), dim3(grid), dim3(NTHREADS), 0, st, a);
   return (int)hipGetLastError();
 }
 

@@ -176,11 +176,17 @@ def bench_prefill(torch, ops, args, dev):
     def quant_only(i):
         ys[0] = ops.quant_rowwise_i8(xs[i % nbuf])
 
+    gamma = (1 + 0.1 * torch.randn(K, generator=g, device=dev)).to(torch.bfloat16)
+
+    def norm_quant_only(i):  # RMSNorm fused with the same quantisation (what feeds q/k/v and up/gate)
+        ys[0] = ops.rmsnorm_quant_rowwise_i8(xs[i % nbuf], gamma, 1e-5)
+
     ops_alg = 2.0 * M * N * K
     steps = max(10, min(args.steps, 100))
     ms = graph_time_ms(torch, step, steps, args.warmup)
     ms_k = graph_time_ms(torch, kernel_only, steps, args.warmup)
     ms_q = graph_time_ms(torch, quant_only, steps, args.warmup)
+    ms_nq = graph_time_ms(torch, norm_quant_only, steps, args.warmup)
     tops = ops_alg / (ms * 1e-3) / 1e12
     tops_k = ops_alg / (ms_k * 1e-3) / 1e12
     qbytes = 2 * M * K + M * K + 4 * M
@@ -192,6 +198,8 @@ def bench_prefill(torch, ops, args, dev):
                      "kernel_us": ms_k * 1e3, "algorithmic_ops": ops_alg},
         "quantise_kernel": {"us": ms_q * 1e3, "gbs": qbytes / (ms_q * 1e-3) / 1e9, "frac_hbm": qbytes / (ms_q * 1e-3) / 1e9 / PEAK_HBM_GBS,
                             "algorithmic_bytes": qbytes},
+        "rmsnorm_quantise_kernel": {"us": ms_nq * 1e3, "gbs": (qbytes + 2 * K) / (ms_nq * 1e-3) / 1e9,
+                                    "algorithmic_bytes": qbytes + 2 * K},
         "shape": (M, N, K),
     }
 
@@ -268,6 +276,11 @@ def bench_block(torch, ops, args, dev):
     prefill()
     ms_dec_sep = graph_time_ms(torch, decode_all, 3, 2) / steps
     fuse_shared_inputs(blk)
+    ms_pre_proj = graph_time_ms(torch, prefill, 10, 3)
+    prefill()
+    ms_dec_proj = graph_time_ms(torch, decode_all, 3, 2) / steps
+    # and with RMSNorm + activation quantisation as one launch in front of each fused projection
+    fuse_shared_inputs(blk, norms=True)
     ms_pre = graph_time_ms(torch, prefill, 10, 3)
     prefill()
     ms_dec = graph_time_ms(torch, decode_all, 3, 2) / steps
@@ -294,6 +307,7 @@ def bench_block(torch, ops, args, dev):
         "workload": "decoder_block hidden=2048 16q/4kv x128 ffn=5632, 7 Linears W8A8, bf16; 8x512 prefill through a paged KV cache (64-token pages) + 64 decode steps (M=8)",
         "value": ms_pre + steps * ms_dec, "unit": "ms", "prefill_ms": ms_pre, "decode_ms_per_step": ms_dec,
         "separate_projections": {"prefill_ms": ms_pre_sep, "decode_ms_per_step": ms_dec_sep},
+        "fused_projections_separate_norms": {"prefill_ms": ms_pre_proj, "decode_ms_per_step": ms_dec_proj},
         "linears_prefill_ms": ms_lin_pre, "linears_prefill_tops": lin_ops / (ms_lin_pre * 1e-3) / 1e12,
         "linears_decode_ms_per_step": ms_lin_dec, "linears_decode_gbs": lin_bytes / (ms_lin_dec * 1e-3) / 1e9,
         "non_linear_prefill_ms": ms_pre - ms_lin_pre, "non_linear_decode_ms_per_step": ms_dec - ms_lin_dec,

@@ -103,6 +103,21 @@ int aq_gemv_w8a8_codes(const int8_t *xq, const float *sx, const int8_t *wq, cons
 int aq_linear_fp8(const uint8_t *xq, const float *sx, const uint8_t *wq, const float *sw,
                   void *y, int y_dtype, int64_t M, int64_t N, int64_t K, void *stream);
 
+/* RMSNorm followed by per-token quantisation, one launch: the codes and scales
+ * aq_quant_rowwise_i8 would give for y = x * rsqrt(mean(x^2) + eps) * gamma held
+ * in fp32.  Fuses the reference's F.rms_norm (astrai/model/components/norm.py:14-15)
+ * with the activation quantisation of the Linears that consume it
+ * (q/k/v: attention.py:83-85 via decoder_block.py:50-51; up/gate: mlp.py:25 via
+ * decoder_block.py:57); the normalised activations are never written.
+ * x: [M, K] (row stride ldx elements), gamma: [K] in the same dtype as x.
+ * Fixed arithmetic: the sum of squares is accumulated per 64-lane stripe of
+ * 16-byte vectors and combined by a butterfly (see the oracle), mean = ss / K,
+ * r = 1 / sqrt(mean + eps) correctly rounded, y = (x * r) * gamma.  K a
+ * multiple of 16 and at most 16384 (bf16) / 8192 (fp32) elements. */
+int aq_rmsnorm_quant_rowwise_i8(const void *x, int x_dtype, const void *gamma, int gamma_dtype,
+                                float eps, int64_t M, int64_t K, int64_t ldx, int8_t *q,
+                                float *scale, void *stream);
+
 /* Tuning and test hook, no counterpart in the reference: the GEMM entry points
  * pick their workgroup tile (256 x 128, or 128 x 128 with a split K step when
  * the larger one would leave compute units idle) from M and N.  rows = 128 or

@@ -20,6 +20,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 from torch import Tensor
 
+from . import ops
 from .linear import Linear, QuantLinear
 
 
@@ -166,11 +167,14 @@ class GQA(nn.Module):
         return False
 
     def forward(self, x: Tensor, rotary_emb: Tensor, attn_mask: Optional[Tensor] = None,
-                cache=None) -> Tensor:
+                cache=None, codes: Optional[Tuple[Tensor, Tensor]] = None) -> Tensor:
+        """``codes``: the already normalised and quantised input ``(xq [B*S, dim], sx [B*S])`` from a
+        fused norm; ``x`` then only gives the shape and dtype."""
         B, S, _ = x.shape
         if self._qkv is not None:
             nq, nkv = self.n_heads * self.head_dim, self.n_kv_heads * self.head_dim
-            q, k, v = self._qkv(x).split((nq, nkv, nkv), dim=-1)
+            qkv = self._qkv(x) if codes is None else self._qkv.forward_codes(codes[0], codes[1], x.dtype).view(B, S, -1)
+            q, k, v = qkv.split((nq, nkv, nkv), dim=-1)
         else:
             q, k, v = self.q_proj(x), self.k_proj(x), self.v_proj(x)
         q = q.reshape(B, S, self.n_heads, self.head_dim)
@@ -206,9 +210,11 @@ class MLP(nn.Module):
             return True
         return False
 
-    def forward(self, x: Tensor) -> Tensor:
+    def forward(self, x: Tensor, codes: Optional[Tuple[Tensor, Tensor]] = None) -> Tensor:
         if self._upgate is not None:
-            up, gate = self._upgate(x).chunk(2, dim=-1)
+            ug = self._upgate(x) if codes is None else self._upgate.forward_codes(codes[0], codes[1], x.dtype).view(
+                *x.shape[:-1], -1)
+            up, gate = ug.chunk(2, dim=-1)
             return self.down(up * F.silu(gate))
         return self.down(self.up(x) * F.silu(self.gate(x)))
 
@@ -223,14 +229,29 @@ class DecoderBlock(nn.Module):
         self.input_norm = RMSNorm(dim, norm_eps)
         self.post_attention_norm = RMSNorm(dim, norm_eps)
         self.mlp = MLP(dim, dim_ffn)
+        self._norm_quant = False
 
     def reset_parameters(self) -> None:
         for m in self.modules():
             if isinstance(m, Linear):
                 m.reset_parameters()
 
+    def fuse_norm_quant(self) -> bool:
+        """Both norms feed fused quantized projections only (q/k/v, up/gate): compute norm and
+        per-token quantisation in one launch and never write the normalised activations.  The
+        bf16 rounding of the norm output disappears, so outputs move by less than the
+        quantisation noise (not bit-identical to the unfused block)."""
+        if self.attention._qkv is not None and self.mlp._upgate is not None:
+            self._norm_quant = True
+        return self._norm_quant
+
     def forward(self, x: Tensor, rotary_emb: Tensor, attention_mask: Optional[Tensor] = None,
                 cache=None) -> Tensor:
+        if self._norm_quant and x.is_cuda and x.dtype == self.input_norm.weight.dtype:
+            n1, n2 = self.input_norm, self.post_attention_norm
+            x = self.attention(x, rotary_emb, attention_mask, cache,
+                               codes=ops.rmsnorm_quant_rowwise_i8(x, n1.weight, n1.norm_eps)) + x
+            return self.mlp(x, codes=ops.rmsnorm_quant_rowwise_i8(x, n2.weight, n2.norm_eps)) + x
         x = self.attention(self.input_norm(x), rotary_emb, attention_mask, cache) + x
         return self.mlp(self.post_attention_norm(x)) + x
 

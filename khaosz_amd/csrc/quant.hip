@@ -158,6 +158,109 @@ __global__ __launch_bounds__(256) void quant_row_wg_kernel(const void* __restric
   }
 }
 
+// -------------------------------------------------- RMSNorm -> row quantise
+//
+// y = x * (1 / sqrt(mean(x^2) + eps)) * gamma, quantised per row exactly like
+// quant_rowwise_i8 would quantise y held in fp32 (no bf16 rounding in between).
+// The sum of squares has a fixed order so that the result does not depend on
+// the launch: lane l of the row's wavefront adds x*x (a rounded product, then a
+// rounded add) over its 16-byte vectors l, l + 64, ... in ascending order,
+// elements in memory order, and the 64 partial sums are combined by the
+// butterfly p[l] += p[l ^ 1], ^2, ^4, ^8, ^16, ^32.  mean = ss / K,
+// r = 1 / sqrt(mean + eps) with correctly rounded divide and square root,
+// y = (x * r) * gamma as two rounded products.
+__device__ __forceinline__ float wave_sum_butterfly(float v) {
+  // After the xor-1 and xor-2 steps a quad holds one value, after the half-row
+  // mirror a half row does, after the row mirror a row does: the mirrors pair
+  // the same partial sums as xor 4 and xor 8 would.
+  v = __fadd_rn(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xf, 0xf, false)));
+  v = __fadd_rn(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xf, 0xf, false)));
+  v = __fadd_rn(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xf, 0xf, false)));
+  v = __fadd_rn(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xf, 0xf, false)));
+  v = __fadd_rn(v, __shfl_xor(v, 16, 64));
+  v = __fadd_rn(v, __shfl_xor(v, 32, 64));
+  return v;
+}
+
+// One wavefront per row; a lane keeps its NC vectors of the row in registers
+// across the three passes (sum of squares, absmax of y, rounding).  GREG: the
+// lane's gamma vectors are loaded once and kept too (short rows); otherwise
+// they are re-read, from L2, in both passes over y.
+template <bool BF16, int NC, bool GREG>
+__global__ __launch_bounds__(256) void rmsnorm_quant_kernel(const void* __restrict__ x, const void* __restrict__ gamma,
+                                                            float eps, int64_t M, int K, int64_t ldx,
+                                                            int8_t* __restrict__ q, float* __restrict__ scale) {
+  constexpr int EPV = RowIn<BF16>::EPV;
+  const int lane = threadIdx.x & 63;
+  const int64_t stride = (int64_t)gridDim.x * 4;
+  const int nvec = K / EPV;
+  const uint4* gsrc = reinterpret_cast<const uint4*>(gamma);
+  uint4 gv[GREG ? NC : 1];
+  if constexpr (GREG) {
+#pragma unroll
+    for (int i = 0; i < NC; ++i) {
+      const int v = i * 64 + lane;
+      gv[i] = v < nvec ? gsrc[v] : make_uint4(0, 0, 0, 0);
+    }
+  }
+  const float kf = (float)K;
+  for (int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6); row < M; row += stride) {
+    const uint4* src = reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(x) + row * ldx * (BF16 ? 2 : 4));
+    uint4 c[NC];
+#pragma unroll
+    for (int i = 0; i < NC; ++i) {
+      const int v = i * 64 + lane;
+      c[i] = v < nvec ? src[v] : make_uint4(0, 0, 0, 0);  // zeros add nothing to any of the passes
+    }
+    float ss = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NC; ++i) {
+      float f[EPV];
+      RowIn<BF16>::unpack(c[i], f);
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) ss = __fadd_rn(ss, __fmul_rn(f[e], f[e]));
+    }
+    ss = wave_sum_butterfly(ss);
+    const float r = __fdiv_rn(1.0f, sqrtf(__fadd_rn(__fdiv_rn(ss, kf), eps)));  // sqrtf: correctly rounded (the __fsqrt_rn intrinsic is the 1-ulp native root)
+    auto normed = [&](int i, float* y) {
+      float f[EPV], g[EPV];
+      RowIn<BF16>::unpack(c[i], f);
+      const int v = i * 64 + lane;
+      RowIn<BF16>::unpack(GREG ? gv[GREG ? i : 0] : (v < nvec ? gsrc[v] : make_uint4(0, 0, 0, 0)), g);
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) y[e] = __fmul_rn(__fmul_rn(f[e], r), g[e]);
+    };
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NC; ++i) {
+      float y[EPV];
+      normed(i, y);
+      amax = fmaxf(amax, vec_amax<EPV>(y));
+    }
+    const RowScale rsc = row_scale(wave_max(amax));
+    if (lane == 0) scale[row] = rsc.s;
+    int8_t* dst = q + row * (int64_t)K;
+#pragma unroll
+    for (int i = 0; i < NC; ++i) {
+      const int v = i * 64 + lane;
+      if (v < nvec) {
+        float y[EPV];
+        uint32_t code[EPV];
+        normed(i, y);
+        quant_codes<EPV>(y, rsc.s, rsc.rs, rsc.fast_ok, code);
+        if constexpr (BF16) {
+          uint2 o;
+          o.x = pack_low_bytes(code[0], code[1], code[2], code[3]);
+          o.y = pack_low_bytes(code[4], code[5], code[6], code[7]);
+          store_wt(reinterpret_cast<uint2*>(dst + (int64_t)v * EPV), o);
+        } else {
+          store_wt(reinterpret_cast<uint32_t*>(dst + (int64_t)v * EPV), pack_low_bytes(code[0], code[1], code[2], code[3]));
+        }
+      }
+    }
+  }
+}
+
 // ---------------------------------------------------------------- FP8 tensor
 
 constexpr int FP8_BATCH = 4;  // 16-byte loads a thread keeps in flight in the per-tensor passes
@@ -331,6 +434,40 @@ extern "C" int aq_quant_rowwise_i8(const void* x, int x_dtype, int64_t M, int64_
                          M, (int)K, ldx, q, scale);
   }
   return (int)hipGetLastError();
+}
+
+template <bool BF16>
+static int launch_rmsnorm_quant(const void* x, const void* gamma, float eps, int64_t M, int64_t K, int64_t ldx,
+                                int8_t* q, float* scale, hipStream_t st) {
+  const int64_t vpl = (K / (BF16 ? 8 : 4) + 63) / 64;  // vectors per lane
+  int64_t wgs = (M + 3) / 4;
+  if (wgs > 1024) wgs = 1024;  // four workgroups per CU; wavefronts walk the remaining rows
+  const dim3 g((unsigned)wgs), b(256);
+  if (vpl <= 4)
+    hipLaunchKernelGGL((aq::rmsnorm_quant_kernel<BF16, 4, true>), g, b, 0, st, x, gamma, eps, M, (int)K, ldx, q, scale);
+  else if (vpl <= 12)
+    hipLaunchKernelGGL((aq::rmsnorm_quant_kernel<BF16, 12, false>), g, b, 0, st, x, gamma, eps, M, (int)K, ldx, q, scale);
+  else if (vpl <= 32)
+    hipLaunchKernelGGL((aq::rmsnorm_quant_kernel<BF16, 32, false>), g, b, 0, st, x, gamma, eps, M, (int)K, ldx, q, scale);
+  else
+    return AQ_E_RANGE;
+  return (int)hipGetLastError();
+}
+
+extern "C" int aq_rmsnorm_quant_rowwise_i8(const void* x, int x_dtype, const void* gamma, int gamma_dtype, float eps,
+                                           int64_t M, int64_t K, int64_t ldx, int8_t* q, float* scale,
+                                           void* stream) {
+  if (x_dtype != AQ_F32 && x_dtype != AQ_BF16) return AQ_E_DTYPE;
+  if (gamma_dtype != x_dtype) return AQ_E_DTYPE;  // the norm's gain lives in the activations' dtype
+  if (M < 0 || K <= 0 || (K % 16) != 0 || ldx < K || !(eps >= 0.0f)) return AQ_E_SHAPE;
+  if (M == 0) return AQ_OK;
+  if (!x || !gamma || !q || !scale) return AQ_E_NULL;
+  const int esz = x_dtype == AQ_BF16 ? 2 : 4;
+  if (aq::check_ptr16(x) || aq::check_ptr16(gamma) || aq::check_ptr16(q) || ((ldx * esz) & 15)) return AQ_E_ALIGN;
+  if (M > (int64_t)1 << 31) return AQ_E_RANGE;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  return x_dtype == AQ_BF16 ? launch_rmsnorm_quant<true>(x, gamma, eps, M, K, ldx, q, scale, st)
+                            : launch_rmsnorm_quant<false>(x, gamma, eps, M, K, ldx, q, scale, st);
 }
 
 extern "C" int aq_quant_tensor_fp8(const void* x, int x_dtype, int64_t numel, uint8_t* q,

@@ -181,6 +181,16 @@ class QuantLinear(Linear):
             y = ops.linear_w8a8(xq, sx, self.qweight, self.w_scale, self.bias, out_dtype=x.dtype)
         return y.reshape(*lead, self.qweight.shape[0])
 
+    def forward_codes(self, xq: Tensor, sx: Tensor, out_dtype: torch.dtype) -> Tensor:
+        """The same projection for an input that is already quantised (``xq int8 [M, K]``,
+        ``sx float32 [M]``): what a producer that fuses the quantisation hands over, or what
+        several projections of one input share.  Returns ``[M, out_dim]``."""
+        if xq.dim() != 2 or xq.shape[1] != self.qweight.shape[1]:
+            raise ValueError(f"expected codes [M, {self.qweight.shape[1]}], got {tuple(xq.shape)}")
+        if xq.shape[0] <= self.DECODE_MAX_ROWS:
+            return ops.gemv_w8a8_codes(xq, sx, self.qweight, self.w_scale, self.bias, out_dtype=out_dtype)
+        return ops.linear_w8a8(xq, sx, self.qweight, self.w_scale, self.bias, out_dtype=out_dtype)
+
     def extra_repr(self) -> str:
         return f"in_dim={self.in_dim}, out_dim={self.out_dim}, bias={self.bias is not None}, w8a8"
 
@@ -241,16 +251,24 @@ TARGET_MODULES_ATTN = {"q_proj", "k_proj", "v_proj", "o_proj"}
 TARGET_MODULES_FFN = {"up", "gate", "down"}
 
 
-def fuse_shared_inputs(model: nn.Module) -> int:
+def fuse_shared_inputs(model: nn.Module, norms: bool = False) -> int:
     """Call ``fuse_projections()`` on every module that offers it (attention and MLP blocks whose
     projections read one input); returns how many fused modules were built.  Run it after
     ``quantize_model`` and after loading weights: the fused module owns the weight storage from
-    then on."""
+    then on.  Outputs stay bit-identical.  ``norms=True`` additionally lets blocks compute
+    RMSNorm and the quantisation of its output in one launch (``fuse_norm_quant()``), which
+    drops the bf16 rounding of the normalised activations: not bit-identical, inside the
+    quantisation noise."""
     n = 0
     for m in model.modules():
         f = getattr(m, "fuse_projections", None)
         if callable(f):
             n += int(f())
+    if norms:
+        for m in model.modules():
+            f = getattr(m, "fuse_norm_quant", None)
+            if callable(f):
+                f()
     return n
 
 

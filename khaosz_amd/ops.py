@@ -72,6 +72,27 @@ def quant_rowwise_i8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     return q, s
 
 
+def rmsnorm_quant_rowwise_i8(x: torch.Tensor, gamma: torch.Tensor, eps: float) -> Tuple[torch.Tensor, torch.Tensor]:
+    """RMSNorm (gain ``gamma``, same dtype as ``x``) fused with the per-token quantisation of its
+    output: ``[..., K]`` -> (codes int8 ``[M, K]``, scales float32 ``[M]``)."""
+    _need_gpu(x, gamma)
+    x2 = _rows(x, "x")
+    M, K = x2.shape
+    _check_k(K)
+    if gamma.dtype != x2.dtype or gamma.numel() != K:
+        raise ValueError("gamma must have the activations' dtype and K elements")
+    gamma = gamma.contiguous()
+    q = torch.empty((M, K), dtype=torch.int8, device=x2.device)
+    s = torch.empty((M,), dtype=torch.float32, device=x2.device)
+    if M:
+        with torch.cuda.device(x2.device):
+            rc = _abi.load().aq_rmsnorm_quant_rowwise_i8(x2.data_ptr(), _dt(x2, "x"), gamma.data_ptr(), _dt(gamma, "gamma"),
+                                                         float(eps), M, K, x2.stride(0), q.data_ptr(), s.data_ptr(),
+                                                         _stream(x2))
+        _abi.check(rc, "aq_rmsnorm_quant_rowwise_i8")
+    return q, s
+
+
 def quant_tensor_fp8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     """Per-tensor OCP e4m3fn -> (codes uint8 with x's shape, scale f32 [1])."""
     _need_gpu(x)

@@ -40,6 +40,12 @@
  *   oq_linear_fp8         restatement; accumulation order makes the GEMM a
  *                         tolerance (1e-2) comparison, never bit-exact.
  *
+ *   oq_rmsnorm_quant_i8   the norm itself restates F.rms_norm (norm.py:14-15) with a
+ *                         fixed summation order; pinned against float64 and torch's
+ *                         F.rms_norm within rounding, against the numpy restatement
+ *                         bit for bit, and on closed forms (constant rows, unit gain).
+ *                         Its quantisation half is oq_quant_rowwise_i8 above.
+ *
  * Build: gcc -O3 -march=native -fopenmp -ffp-contract=off -fno-fast-math
  *        -shared -fPIC (oracle/build_oracle.py).  OpenMP only parallelises over
  *        rows; every row's arithmetic is the scalar definition above.
@@ -170,6 +176,71 @@ void oq_quant_rowwise_i8_bf16(const uint16_t *x, int64_t M, int64_t K, int64_t l
     quant_row_f32(tmp, K, q + m * K, scale + m);
     free(tmp);
   }
+}
+
+/* --------------------------------------------- RMSNorm -> row-wise quantise */
+
+/* y = x * (1 / sqrt(mean(x^2) + eps)) * gamma  (F.rms_norm with a gain:
+ * astrai/model/components/norm.py:14-15), then quantised per row like any other
+ * fp32 row.  The sum of squares has a fixed order: the row is cut into vectors
+ * of `epv` consecutive elements (16 bytes of the input: 4 fp32 or 8 bf16);
+ * stripe l = v % 64 adds the rounded products x*x of its vectors in ascending
+ * order, elements in memory order; the 64 stripe sums are combined by the
+ * butterfly p[l] = p[l] + p[l ^ off], off = 1, 2, 4, 8, 16, 32. */
+static void rmsnorm_row(const float *a, const float *g, float eps, int64_t K, int epv, float *y) {
+  float p[64], t[64];
+  for (int l = 0; l < 64; ++l) p[l] = 0.0f;
+  const int64_t nvec = K / epv;
+  for (int64_t v = 0; v < nvec; ++v) {
+    const int l = (int)(v % 64);
+    for (int e = 0; e < epv; ++e) {
+      const float x = a[v * epv + e];
+      const float sq = x * x;
+      p[l] = p[l] + sq;
+    }
+  }
+  for (int off = 1; off < 64; off <<= 1) {
+    for (int l = 0; l < 64; ++l) t[l] = p[l] + p[l ^ off];
+    for (int l = 0; l < 64; ++l) p[l] = t[l];
+  }
+  const float mean = p[0] / (float)K;
+  const float r = 1.0f / sqrtf(mean + eps);
+  for (int64_t k = 0; k < K; ++k) {
+    const float xr = a[k] * r;
+    y[k] = xr * g[k];
+  }
+}
+
+/* x: [M, K] fp32 (row stride ldx), gamma: [K] fp32; y_out (optional) receives the
+ * normalised rows in fp32. */
+void oq_rmsnorm_quant_i8_f32(const float *x, const float *gamma, float eps, int64_t M, int64_t K,
+                             int64_t ldx, int8_t *q, float *scale, float *y_out) {
+#pragma omp parallel for schedule(static)
+  for (int64_t m = 0; m < M; ++m) {
+    float *y = (float *)malloc((size_t)K * sizeof(float));
+    rmsnorm_row(x + m * ldx, gamma, eps, K, 4, y);
+    quant_row_f32(y, K, q + m * K, scale + m);
+    if (y_out) memcpy(y_out + m * K, y, (size_t)K * sizeof(float));
+    free(y);
+  }
+}
+
+/* bf16 input and gain, widened to fp32 first (exact); vectors are 8 elements. */
+void oq_rmsnorm_quant_i8_bf16(const uint16_t *x, const uint16_t *gamma, float eps, int64_t M,
+                              int64_t K, int64_t ldx, int8_t *q, float *scale, float *y_out) {
+  float *g = (float *)malloc((size_t)K * sizeof(float));
+  for (int64_t k = 0; k < K; ++k) g[k] = oq_bf16_to_f32(gamma[k]);
+#pragma omp parallel for schedule(static)
+  for (int64_t m = 0; m < M; ++m) {
+    float *a = (float *)malloc((size_t)K * 2 * sizeof(float));
+    float *y = a + K;
+    for (int64_t k = 0; k < K; ++k) a[k] = oq_bf16_to_f32(x[m * ldx + k]);
+    rmsnorm_row(a, g, eps, K, 8, y);
+    quant_row_f32(y, K, q + m * K, scale + m);
+    if (y_out) memcpy(y_out + m * K, y, (size_t)K * sizeof(float));
+    free(a);
+  }
+  free(g);
 }
 
 /* ------------------------------------------------------------- int8 GEMM */

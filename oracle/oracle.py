@@ -98,6 +98,36 @@ def np_quant_rowwise_i8(x: np.ndarray):
     return q, s
 
 
+def np_rmsnorm(x: np.ndarray, gamma: np.ndarray, eps: float, epv: int) -> np.ndarray:
+    """y = x * (1 / sqrt(mean(x^2) + eps)) * gamma in fp32 with the fixed summation order of
+    the C oracle: 64 stripes of ``epv``-element vectors, then an xor butterfly."""
+    x = np.ascontiguousarray(x, dtype=F32)
+    gamma = np.ascontiguousarray(gamma, dtype=F32)
+    M, K = x.shape
+    nvec = K // epv
+    pad = (-nvec) % 64
+    sq = (x * x).astype(F32).reshape(M, nvec, epv)
+    if pad:
+        sq = np.concatenate([sq, np.zeros((M, pad, epv), F32)], axis=1)
+    sq = sq.reshape(M, -1, 64, epv)            # [M, round, stripe, element]
+    p = np.zeros((M, 64), F32)
+    for rnd in range(sq.shape[1]):
+        for e in range(epv):
+            p = (p + sq[:, rnd, :, e]).astype(F32)
+    idx = np.arange(64)
+    off = 1
+    while off < 64:
+        p = (p + p[:, idx ^ off]).astype(F32)
+        off <<= 1
+    mean = (p[:, 0] / F32(K)).astype(F32)
+    r = (F32(1.0) / np.sqrt((mean + F32(eps)).astype(F32)).astype(F32)).astype(F32)
+    return ((x * r[:, None]).astype(F32) * gamma[None, :]).astype(F32)
+
+
+def np_rmsnorm_quant_i8(x: np.ndarray, gamma: np.ndarray, eps: float, epv: int):
+    return np_quant_rowwise_i8(np_rmsnorm(x, gamma, eps, epv))
+
+
 def np_gemm_i8_i32(xq: np.ndarray, wq: np.ndarray) -> np.ndarray:
     acc = xq.astype(np.int64) @ wq.astype(np.int64).T
     assert np.all(np.abs(acc) < 2 ** 31)
@@ -166,6 +196,8 @@ def _load():
     lib.oq_f32_to_e4m3fn.argtypes = [ctypes.c_float]
     lib.oq_quant_rowwise_i8_f32.argtypes = [vp, i64, i64, i64, vp, vp]
     lib.oq_quant_rowwise_i8_bf16.argtypes = [vp, i64, i64, i64, vp, vp]
+    lib.oq_rmsnorm_quant_i8_f32.argtypes = [vp, vp, ctypes.c_float, i64, i64, i64, vp, vp, vp]
+    lib.oq_rmsnorm_quant_i8_bf16.argtypes = [vp, vp, ctypes.c_float, i64, i64, i64, vp, vp, vp]
     lib.oq_gemm_i8_i32.argtypes = [vp, vp, vp, i64, i64, i64]
     lib.oq_dequant_epilogue.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64]
     lib.oq_linear_w8a8_f32.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i64]
@@ -177,7 +209,7 @@ def _load():
     for name in (
         "oq_set_num_threads oq_quant_rowwise_i8_f32 oq_quant_rowwise_i8_bf16 oq_gemm_i8_i32 "
         "oq_dequant_epilogue oq_linear_w8a8_f32 oq_linear_w8a8_bf16 oq_quant_tensor_fp8_f32 "
-        "oq_quant_tensor_fp8_bf16 oq_linear_fp8 oq_linear_f32"
+        "oq_quant_tensor_fp8_bf16 oq_linear_fp8 oq_linear_f32 oq_rmsnorm_quant_i8_f32 oq_rmsnorm_quant_i8_bf16"
     ).split():
         getattr(lib, name).restype = None
     _lib = lib
@@ -227,6 +259,21 @@ def c_quant_rowwise_i8(x: np.ndarray, bf16_bits: bool = False):
     fn = lib.oq_quant_rowwise_i8_bf16 if bf16_bits else lib.oq_quant_rowwise_i8_f32
     fn(_p(x), M, K, K, _p(q), _p(s))
     return q, s
+
+
+def c_rmsnorm_quant_i8(x: np.ndarray, gamma: np.ndarray, eps: float, bf16_bits: bool = False, want_y: bool = False):
+    """x: [M,K] and gamma: [K], fp32 or (``bf16_bits``) uint16 bf16 patterns -> (codes, scale[, y fp32])."""
+    lib = _load()
+    dt = np.uint16 if bf16_bits else F32
+    x, gamma = _c(x, dt), _c(gamma, dt)
+    M, K = x.shape
+    assert gamma.shape == (K,)
+    q = np.empty((M, K), np.int8)
+    s = np.empty((M,), F32)
+    y = np.empty((M, K), F32) if want_y else None
+    fn = lib.oq_rmsnorm_quant_i8_bf16 if bf16_bits else lib.oq_rmsnorm_quant_i8_f32
+    fn(_p(x), _p(gamma), ctypes.c_float(eps), M, K, K, _p(q), _p(s), _p(y) if want_y else None)
+    return (q, s, y) if want_y else (q, s)
 
 
 def c_gemm_i8_i32(xq: np.ndarray, wq: np.ndarray) -> np.ndarray:

@@ -260,3 +260,34 @@ def test_fused_shared_input_projections_are_bit_identical():
         quantize_model(c)
         b.load_state_dict(c.state_dict())
         assert torch.equal(b(x, _freqs(tab, 2, 0, 40)), c(x, _freqs(tab, 2, 0, 40)))
+
+
+@pytest.mark.gpu
+def test_fused_norm_quantise_stays_inside_the_quantisation_noise():
+    """RMSNorm + per-token quantisation in one launch for both norms of the block: outputs move by
+    far less than the quantisation error itself (the bf16 rounding of the norm output is gone),
+    on the prefill and the decode path."""
+    from khaosz_amd import fuse_shared_inputs
+
+    dev, dt = "cuda:0", torch.bfloat16
+    flt = _block(dim=256, heads=4, kv=2, ffn=704).to(dev)
+    a = _block(dim=256, heads=4, kv=2, ffn=704).to(dev).to(dt)
+    a.load_state_dict({k: v.to(dt) for k, v in flt.state_dict().items()})
+    b = _block(dim=256, heads=4, kv=2, ffn=704).to(dev).to(dt)
+    b.load_state_dict(a.state_dict())
+    quantize_model(a), quantize_model(b)
+    fuse_shared_inputs(a)
+    fuse_shared_inputs(b, norms=True)
+    assert b._norm_quant and not a._norm_quant
+    tab = rotary_table(64, 64, device=dev)
+    x = torch.randn(2, 40, 256, device=dev)
+    with torch.inference_mode():
+        ref = flt(x, _freqs(tab, 2, 0, 40))
+        for xs in (x.to(dt), x[:, :3].contiguous().to(dt)):            # M = 80 and M = 6
+            S = xs.shape[1]
+            ya, yb = a(xs, _freqs(tab, 2, 0, S)), b(xs, _freqs(tab, 2, 0, S))
+            r = ref[:, :S]
+            err_a = ((ya.float() - r).norm() / r.norm()).item()
+            err_b = ((yb.float() - r).norm() / r.norm()).item()
+            assert err_b < 3e-2 and err_b < 1.2 * err_a + 1e-3, (err_a, err_b)
+            assert ((ya.float() - yb.float()).norm() / r.norm()).item() < 1.5e-2

@@ -123,6 +123,46 @@ def test_quant_rowwise_scale_range_and_dense_ties(oracle, dtype):
             assert np.array_equal(to_np(y), want), f"rows {r0}.."
 
 
+@pytest.mark.parametrize("M,K", [(1, 16), (7, 48), (5, 1040), (64, 2048), (8, 5632), (130, 4096), (3, 16384)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_rmsnorm_quant_bit_exact(oracle, M, K, dtype):
+    if dtype == torch.float32 and K > 8192:
+        pytest.skip("fp32 rows longer than 8192 are outside the kernel's register budget")
+    _say("rmsnorm_quant", M, K, dtype)
+    g = torch.Generator().manual_seed(M * 13 + K)
+    x = torch.randn(M, K, generator=g) * (0.05 + 5 * torch.rand(M, 1, generator=g))
+    if M > 4:
+        x[1] = 0                                   # zero row: eps keeps the root finite, codes 0
+        x[2] *= 1e-18
+        x[3] *= 1e12
+    gamma = 1 + 0.2 * torch.randn(K, generator=g)
+    xd, gd = x.to(DEV, dtype), gamma.to(DEV, dtype)
+    q, s = ops.rmsnorm_quant_rowwise_i8(xd, gd, 1e-5)
+    if dtype == torch.bfloat16:
+        qo, so = oracle.c_rmsnorm_quant_i8(bf16_bits(xd), bf16_bits(gd), 1e-5, bf16_bits=True)
+    else:
+        qo, so = oracle.c_rmsnorm_quant_i8(to_np(xd), to_np(gd), 1e-5)
+    assert np.array_equal(to_np(s).view(np.uint32), so.view(np.uint32))
+    bad = np.argwhere(to_np(q) != qo)
+    assert bad.size == 0, f"first mismatches (row, col): {bad[:5].tolist()}"
+
+
+def test_rmsnorm_quant_tracks_torch_rms_norm_then_quantise():
+    """Against the unfused flow (F.rms_norm, norm.py:14-15, then the row quantiser): the fused kernel
+    skips the bf16 rounding of the normalised activations, so codes may differ by one step."""
+    x = make_x(64, 2048, seed=9).to(DEV, torch.bfloat16)
+    gamma = (1 + 0.1 * make_x(1, 2048, seed=10)[0]).to(DEV, torch.bfloat16)
+    q, s = ops.rmsnorm_quant_rowwise_i8(x, gamma, 1e-5)
+    q2, s2 = ops.quant_rowwise_i8(torch.nn.functional.rms_norm(x, (2048,), gamma, 1e-5))
+    assert torch.allclose(s, s2, rtol=1e-2)
+    d = (q.int() - q2.int()).abs()
+    assert d.max().item() <= 1 and (d != 0).float().mean().item() < 0.2
+    with pytest.raises(ValueError):
+        ops.rmsnorm_quant_rowwise_i8(x, gamma.float(), 1e-5)       # gain in another dtype
+    with pytest.raises(ValueError):
+        ops.rmsnorm_quant_rowwise_i8(torch.zeros(2, 32768, device=DEV), torch.ones(32768, device=DEV), 1e-5)
+
+
 def test_quant_rowwise_empty():
     q, s = ops.quant_rowwise_i8(torch.empty((0, 32), device=DEV))
     assert q.shape == (0, 32) and s.shape == (0,)

@@ -113,10 +113,22 @@ int aq_linear_fp8(const uint8_t *xq, const float *sx, const uint8_t *wq, const f
  * Fixed arithmetic: the sum of squares is accumulated per 64-lane stripe of
  * 16-byte vectors and combined by a butterfly (see the oracle), mean = ss / K,
  * r = 1 / sqrt(mean + eps) correctly rounded, y = (x * r) * gamma.  K a
- * multiple of 16 and at most 16384 (bf16) / 8192 (fp32) elements. */
+ * multiple of 16 and at most 12288 (bf16) / 6144 (fp32) elements (AQ_E_RANGE beyond). */
 int aq_rmsnorm_quant_rowwise_i8(const void *x, int x_dtype, const void *gamma, int gamma_dtype,
                                 float eps, int64_t M, int64_t K, int64_t ldx, int8_t *q,
                                 float *scale, void *stream);
+
+/* SwiGLU followed by per-token quantisation, one launch: ug is the output
+ * [M, 2F] (row stride ld elements) of the fused up/gate projection, columns
+ * [0, F) = up(x), [F, 2F) = gate(x); h = up * silu(gate) (mlp.py:25-26) is
+ * formed in fp32 and quantised per row, giving the codes [M, F] and scales [M]
+ * that the down projection (mlp.py:26) consumes.  h is never written.
+ * Fixed arithmetic: silu(g) = g / (1 + e), e = exp(-g) from a fixed sequence of
+ * fused multiply-adds (degree-5 polynomial after range reduction; the oracle
+ * repeats it bit for bit), correctly rounded divide, one rounded product.
+ * F a multiple of 16 and at most 6144 (bf16) / 3072 (fp32) elements. */
+int aq_swiglu_quant_rowwise_i8(const void *ug, int dtype, int64_t M, int64_t F, int64_t ld,
+                               int8_t *q, float *scale, void *stream);
 
 /* Tuning and test hook, no counterpart in the reference: the GEMM entry points
  * pick their workgroup tile (256 x 128, or 128 x 128 with a split K step when

@@ -202,6 +202,7 @@ class MLP(nn.Module):
         self.gate = Linear(dim, dim_ffn)
         self.down = Linear(dim_ffn, dim)
         self._upgate: Optional[QuantLinear] = None
+        self._swiglu_quant = False  # set by DecoderBlock.fuse_norm_quant(): not bit-identical, opt-in
 
     def fuse_projections(self) -> bool:
         """up and gate read the same input (mlp.py:25): one ``[2*dim_ffn, dim]`` projection."""
@@ -214,6 +215,10 @@ class MLP(nn.Module):
         if self._upgate is not None:
             ug = self._upgate(x) if codes is None else self._upgate.forward_codes(codes[0], codes[1], x.dtype).view(
                 *x.shape[:-1], -1)
+            if self._swiglu_quant and isinstance(self.down, QuantLinear) and ug.is_cuda:
+                # activation, product and the down projection's quantisation in one launch
+                hq, hs = ops.swiglu_quant_rowwise_i8(ug)
+                return self.down.forward_codes(hq, hs, x.dtype).view(*x.shape[:-1], -1)
             up, gate = ug.chunk(2, dim=-1)
             return self.down(up * F.silu(gate))
         return self.down(self.up(x) * F.silu(self.gate(x)))
@@ -243,6 +248,7 @@ class DecoderBlock(nn.Module):
         quantisation noise (not bit-identical to the unfused block)."""
         if self.attention._qkv is not None and self.mlp._upgate is not None:
             self._norm_quant = True
+            self.mlp._swiglu_quant = True  # likewise: silu * up and the quantisation for `down` in one launch
         return self._norm_quant
 
     def forward(self, x: Tensor, rotary_emb: Tensor, attention_mask: Optional[Tensor] = None,

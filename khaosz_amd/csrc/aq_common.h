@@ -100,6 +100,32 @@ __device__ __forceinline__ void quant_codes(const float* a, float s, float rs, b
   }
 }
 
+// exp(x) for |x| <= 87 from operations that round identically on every IEEE
+// machine (products, fused multiply-adds, rint, an exponent-field add), so that
+// the CPU oracle reproduces it bit for bit; library exponentials differ in their
+// last bits between implementations.  n = rint(x log2 e), r = x - n ln 2 in two
+// pieces, e^r = 1 + r + r^2 P(r) with the classic degree-5 minimax P (error below
+// 2 ulp), scaled by 2^n through the exponent field.
+__device__ __forceinline__ float exp_repro(float x) {
+  x = fminf(fmaxf(x, -87.0f), 87.0f);
+  const float n = rintf(__fmul_rn(x, 1.44269504088896341f));
+  float r = __builtin_fmaf(n, -0.693359375f, x);
+  r = __builtin_fmaf(n, 2.12194440e-4f, r);
+  float p = 1.9875691500e-4f;
+  p = __builtin_fmaf(p, r, 1.3981999507e-3f);
+  p = __builtin_fmaf(p, r, 8.3334519073e-3f);
+  p = __builtin_fmaf(p, r, 4.1665795894e-2f);
+  p = __builtin_fmaf(p, r, 1.6666665459e-1f);
+  p = __builtin_fmaf(p, r, 5.0000001201e-1f);
+  const float y = __fadd_rn(__builtin_fmaf(p, __fmul_rn(r, r), r), 1.0f);
+  return __int_as_float(__float_as_int(y) + ((int)n << 23));
+}
+
+// SwiGLU on fp32 values: u * (g / (1 + exp(-g))), a correctly rounded divide and one product.
+__device__ __forceinline__ float swiglu_repro(float u, float g) {
+  return __fmul_rn(u, __fdiv_rn(g, __fadd_rn(1.0f, exp_repro(-g))));
+}
+
 // low bytes of four 32-bit patterns -> one dword (a in bits 7:0 .. d in bits 31:24)
 __device__ __forceinline__ uint32_t pack_low_bytes(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
   const uint32_t ab = __builtin_amdgcn_perm(b, a, 0x0c0c0400u);  // {a.b0, b.b0, 0, 0}

@@ -261,6 +261,64 @@ __global__ __launch_bounds__(256) void rmsnorm_quant_kernel(const void* __restri
   }
 }
 
+// ------------------------------------------------ SwiGLU -> row quantise
+//
+// h = up * silu(gate) for one row of the fused up/gate projection's output
+// ([up | gate], 2 F columns), quantised per row like any fp32 row: the codes and
+// scales the down projection consumes.  Replaces the activation, the product and
+// the quantiser launches (three passes over [M, F]) by one.  A lane first turns
+// its NC vector pairs into h (fp32, kept in registers; the inputs die as it goes),
+// then reduces the absmax and rounds.
+template <bool BF16, int NC>
+__global__ __launch_bounds__(256) void swiglu_quant_kernel(const void* __restrict__ ug, int64_t M, int F, int64_t ld,
+                                                           int8_t* __restrict__ q, float* __restrict__ scale) {
+  constexpr int EPV = RowIn<BF16>::EPV;
+  const int lane = threadIdx.x & 63;
+  const int64_t stride = (int64_t)gridDim.x * 4;
+  const int nvec = F / EPV;
+  for (int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6); row < M; row += stride) {
+    const uint4* up = reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(ug) + row * ld * (BF16 ? 2 : 4));
+    const uint4* gate = up + nvec;
+    uint4 cu[NC], cg[NC];
+#pragma unroll
+    for (int i = 0; i < NC; ++i) {
+      const int v = i * 64 + lane;
+      cu[i] = v < nvec ? up[v] : make_uint4(0, 0, 0, 0);
+      cg[i] = v < nvec ? gate[v] : make_uint4(0, 0, 0, 0);
+    }
+    float h[NC][EPV];
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NC; ++i) {
+      float u[EPV], g[EPV];
+      RowIn<BF16>::unpack(cu[i], u);
+      RowIn<BF16>::unpack(cg[i], g);
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) h[i][e] = swiglu_repro(u[e], g[e]);  // 0 * silu(0) = 0 past the row
+      amax = fmaxf(amax, vec_amax<EPV>(h[i]));
+    }
+    const RowScale rsc = row_scale(wave_max(amax));
+    if (lane == 0) scale[row] = rsc.s;
+    int8_t* dst = q + row * (int64_t)F;
+#pragma unroll
+    for (int i = 0; i < NC; ++i) {
+      const int v = i * 64 + lane;
+      if (v < nvec) {
+        uint32_t code[EPV];
+        quant_codes<EPV>(h[i], rsc.s, rsc.rs, rsc.fast_ok, code);
+        if constexpr (BF16) {
+          uint2 o;
+          o.x = pack_low_bytes(code[0], code[1], code[2], code[3]);
+          o.y = pack_low_bytes(code[4], code[5], code[6], code[7]);
+          store_wt(reinterpret_cast<uint2*>(dst + (int64_t)v * EPV), o);
+        } else {
+          store_wt(reinterpret_cast<uint32_t*>(dst + (int64_t)v * EPV), pack_low_bytes(code[0], code[1], code[2], code[3]));
+        }
+      }
+    }
+  }
+}
+
 // ---------------------------------------------------------------- FP8 tensor
 
 constexpr int FP8_BATCH = 4;  // 16-byte loads a thread keeps in flight in the per-tensor passes
@@ -447,8 +505,8 @@ static int launch_rmsnorm_quant(const void* x, const void* gamma, float eps, int
     hipLaunchKernelGGL((aq::rmsnorm_quant_kernel<BF16, 4, true>), g, b, 0, st, x, gamma, eps, M, (int)K, ldx, q, scale);
   else if (vpl <= 12)
     hipLaunchKernelGGL((aq::rmsnorm_quant_kernel<BF16, 12, false>), g, b, 0, st, x, gamma, eps, M, (int)K, ldx, q, scale);
-  else if (vpl <= 32)
-    hipLaunchKernelGGL((aq::rmsnorm_quant_kernel<BF16, 32, false>), g, b, 0, st, x, gamma, eps, M, (int)K, ldx, q, scale);
+  else if (vpl <= 24)  // 24 vectors per lane is what fits the register file without spilling for bf16 rows
+    hipLaunchKernelGGL((aq::rmsnorm_quant_kernel<BF16, 24, false>), g, b, 0, st, x, gamma, eps, M, (int)K, ldx, q, scale);
   else
     return AQ_E_RANGE;
   return (int)hipGetLastError();
@@ -468,6 +526,36 @@ extern "C" int aq_rmsnorm_quant_rowwise_i8(const void* x, int x_dtype, const voi
   hipStream_t st = static_cast<hipStream_t>(stream);
   return x_dtype == AQ_BF16 ? launch_rmsnorm_quant<true>(x, gamma, eps, M, K, ldx, q, scale, st)
                             : launch_rmsnorm_quant<false>(x, gamma, eps, M, K, ldx, q, scale, st);
+}
+
+template <bool BF16>
+static int launch_swiglu_quant(const void* ug, int64_t M, int64_t F, int64_t ld, int8_t* q, float* scale,
+                               hipStream_t st) {
+  const int64_t vpl = (F / (BF16 ? 8 : 4) + 63) / 64;  // vector pairs per lane
+  int64_t wgs = (M + 3) / 4;
+  if (wgs > 1024) wgs = 1024;
+  const dim3 g((unsigned)wgs), b(256);
+  if (vpl <= 4)
+    hipLaunchKernelGGL((aq::swiglu_quant_kernel<BF16, 4>), g, b, 0, st, ug, M, (int)F, ld, q, scale);
+  else if (vpl <= 12)
+    hipLaunchKernelGGL((aq::swiglu_quant_kernel<BF16, 12>), g, b, 0, st, ug, M, (int)F, ld, q, scale);
+  else
+    return AQ_E_RANGE;
+  return (int)hipGetLastError();
+}
+
+extern "C" int aq_swiglu_quant_rowwise_i8(const void* ug, int dtype, int64_t M, int64_t F, int64_t ld, int8_t* q,
+                                          float* scale, void* stream) {
+  if (dtype != AQ_F32 && dtype != AQ_BF16) return AQ_E_DTYPE;
+  if (M < 0 || F <= 0 || (F % 16) != 0 || ld < 2 * F) return AQ_E_SHAPE;
+  if (M == 0) return AQ_OK;
+  if (!ug || !q || !scale) return AQ_E_NULL;
+  const int esz = dtype == AQ_BF16 ? 2 : 4;
+  if (aq::check_ptr16(ug) || aq::check_ptr16(q) || ((ld * esz) & 15)) return AQ_E_ALIGN;
+  if (M > (int64_t)1 << 31) return AQ_E_RANGE;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  return dtype == AQ_BF16 ? launch_swiglu_quant<true>(ug, M, F, ld, q, scale, st)
+                          : launch_swiglu_quant<false>(ug, M, F, ld, q, scale, st);
 }
 
 extern "C" int aq_quant_tensor_fp8(const void* x, int x_dtype, int64_t numel, uint8_t* q,

@@ -93,6 +93,26 @@ def rmsnorm_quant_rowwise_i8(x: torch.Tensor, gamma: torch.Tensor, eps: float) -
     return q, s
 
 
+def swiglu_quant_rowwise_i8(ug: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``ug [..., 2F] = [up | gate]`` -> codes and scales of ``up * silu(gate)`` per row
+    (int8 ``[M, F]``, float32 ``[M]``), without writing the product."""
+    _need_gpu(ug)
+    u2 = _rows(ug, "ug")
+    M, F2 = u2.shape
+    if F2 % 2:
+        raise ValueError("the last dimension holds up and gate side by side: it must be even")
+    F = F2 // 2
+    _check_k(F)
+    q = torch.empty((M, F), dtype=torch.int8, device=u2.device)
+    s = torch.empty((M,), dtype=torch.float32, device=u2.device)
+    if M:
+        with torch.cuda.device(u2.device):
+            rc = _abi.load().aq_swiglu_quant_rowwise_i8(u2.data_ptr(), _dt(u2, "ug"), M, F, u2.stride(0), q.data_ptr(),
+                                                        s.data_ptr(), _stream(u2))
+        _abi.check(rc, "aq_swiglu_quant_rowwise_i8")
+    return q, s
+
+
 def quant_tensor_fp8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     """Per-tensor OCP e4m3fn -> (codes uint8 with x's shape, scale f32 [1])."""
     _need_gpu(x)

@@ -45,6 +45,12 @@
  *                         F.rms_norm within rounding, against the numpy restatement
  *                         bit for bit, and on closed forms (constant rows, unit gain).
  *                         Its quantisation half is oq_quant_rowwise_i8 above.
+ *   oq_swiglu_quant_i8    up * silu(gate) (mlp.py:25-26) with an exponential built from
+ *                         fused multiply-adds only; pinned against float64 / libm and
+ *                         torch's F.silu within rounding, against the numpy
+ *                         restatement bit for bit (numpy has no fma: the comparison
+ *                         runs the polynomial in float64 products rounded once, which
+ *                         is what an fma is), and on closed forms (g = 0, large |g|).
  *
  * Build: gcc -O3 -march=native -fopenmp -ffp-contract=off -fno-fast-math
  *        -shared -fPIC (oracle/build_oracle.py).  OpenMP only parallelises over
@@ -241,6 +247,62 @@ void oq_rmsnorm_quant_i8_bf16(const uint16_t *x, const uint16_t *gamma, float ep
     free(a);
   }
   free(g);
+}
+
+/* ------------------------------------------------ SwiGLU -> row-wise quantise */
+
+/* exp(x) for |x| <= 87 from operations that round identically everywhere:
+ * n = rint(x log2 e), r = x - n ln 2 in two pieces, e^r = 1 + r + r^2 P(r), then
+ * the exponent field is advanced by n. */
+float oq_exp_repro(float x) {
+  if (x < -87.0f) x = -87.0f;
+  if (x > 87.0f) x = 87.0f;
+  const float t = x * 1.44269504088896341f;
+  const float n = rintf(t);
+  float r = fmaf(n, -0.693359375f, x);
+  r = fmaf(n, 2.12194440e-4f, r);
+  float p = 1.9875691500e-4f;
+  p = fmaf(p, r, 1.3981999507e-3f);
+  p = fmaf(p, r, 8.3334519073e-3f);
+  p = fmaf(p, r, 4.1665795894e-2f);
+  p = fmaf(p, r, 1.6666665459e-1f);
+  p = fmaf(p, r, 5.0000001201e-1f);
+  const float rr = r * r;
+  const float y = fmaf(p, rr, r) + 1.0f;
+  return bits_to_f32((uint32_t)((int32_t)f32_to_bits(y) + ((int32_t)n << 23)));
+}
+
+float oq_swiglu(float u, float g) {
+  const float e = oq_exp_repro(-g);
+  const float d = 1.0f + e;
+  const float sg = g / d;
+  return u * sg;
+}
+
+/* ug: [M, 2F] (row stride ld), columns [0,F) = up, [F,2F) = gate; codes [M, F]. */
+void oq_swiglu_quant_i8_f32(const float *ug, int64_t M, int64_t F, int64_t ld, int8_t *q,
+                            float *scale, float *h_out) {
+#pragma omp parallel for schedule(static)
+  for (int64_t m = 0; m < M; ++m) {
+    float *h = (float *)malloc((size_t)F * sizeof(float));
+    for (int64_t k = 0; k < F; ++k) h[k] = oq_swiglu(ug[m * ld + k], ug[m * ld + F + k]);
+    quant_row_f32(h, F, q + m * F, scale + m);
+    if (h_out) memcpy(h_out + m * F, h, (size_t)F * sizeof(float));
+    free(h);
+  }
+}
+
+void oq_swiglu_quant_i8_bf16(const uint16_t *ug, int64_t M, int64_t F, int64_t ld, int8_t *q,
+                             float *scale, float *h_out) {
+#pragma omp parallel for schedule(static)
+  for (int64_t m = 0; m < M; ++m) {
+    float *h = (float *)malloc((size_t)F * sizeof(float));
+    for (int64_t k = 0; k < F; ++k)
+      h[k] = oq_swiglu(oq_bf16_to_f32(ug[m * ld + k]), oq_bf16_to_f32(ug[m * ld + F + k]));
+    quant_row_f32(h, F, q + m * F, scale + m);
+    if (h_out) memcpy(h_out + m * F, h, (size_t)F * sizeof(float));
+    free(h);
+  }
 }
 
 /* ------------------------------------------------------------- int8 GEMM */

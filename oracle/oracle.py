@@ -128,6 +128,31 @@ def np_rmsnorm_quant_i8(x: np.ndarray, gamma: np.ndarray, eps: float, epv: int):
     return np_quant_rowwise_i8(np_rmsnorm(x, gamma, eps, epv))
 
 
+def _fma32(a, b, c):
+    """fp32 fused multiply-add on arrays: the product of two fp32 values is exact in float64, and
+    the float64 sum is rounded once more to fp32; the double rounding can only matter when the
+    float64 sum lands exactly on an fp32 midpoint, which the callers' tests would show."""
+    return (a.astype(np.float64) * b.astype(np.float64) + c.astype(np.float64)).astype(F32)
+
+
+def np_exp_repro(x: np.ndarray) -> np.ndarray:
+    x = np.clip(np.asarray(x, F32), F32(-87.0), F32(87.0)).astype(F32)
+    n = np.rint((x * F32(1.44269504088896341)).astype(F32)).astype(F32)
+    r = _fma32(n, np.full_like(n, F32(-0.693359375)), x)
+    r = _fma32(n, np.full_like(n, F32(2.12194440e-4)), r)
+    p = np.full_like(r, F32(1.9875691500e-4))
+    for c in (1.3981999507e-3, 8.3334519073e-3, 4.1665795894e-2, 1.6666665459e-1, 5.0000001201e-1):
+        p = _fma32(p, r, np.full_like(r, F32(c)))
+    y = (_fma32(p, (r * r).astype(F32), r) + F32(1.0)).astype(F32)
+    return (y.view(np.int32) + (n.astype(np.int32) << 23)).view(F32)
+
+
+def np_swiglu(u: np.ndarray, g: np.ndarray) -> np.ndarray:
+    u, g = np.asarray(u, F32), np.asarray(g, F32)
+    d = (F32(1.0) + np_exp_repro(-g)).astype(F32)
+    return (u * (g / d).astype(F32)).astype(F32)
+
+
 def np_gemm_i8_i32(xq: np.ndarray, wq: np.ndarray) -> np.ndarray:
     acc = xq.astype(np.int64) @ wq.astype(np.int64).T
     assert np.all(np.abs(acc) < 2 ** 31)
@@ -198,6 +223,10 @@ def _load():
     lib.oq_quant_rowwise_i8_bf16.argtypes = [vp, i64, i64, i64, vp, vp]
     lib.oq_rmsnorm_quant_i8_f32.argtypes = [vp, vp, ctypes.c_float, i64, i64, i64, vp, vp, vp]
     lib.oq_rmsnorm_quant_i8_bf16.argtypes = [vp, vp, ctypes.c_float, i64, i64, i64, vp, vp, vp]
+    lib.oq_swiglu_quant_i8_f32.argtypes = [vp, i64, i64, i64, vp, vp, vp]
+    lib.oq_swiglu_quant_i8_bf16.argtypes = [vp, i64, i64, i64, vp, vp, vp]
+    lib.oq_exp_repro.argtypes = [ctypes.c_float]
+    lib.oq_exp_repro.restype = ctypes.c_float
     lib.oq_gemm_i8_i32.argtypes = [vp, vp, vp, i64, i64, i64]
     lib.oq_dequant_epilogue.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64]
     lib.oq_linear_w8a8_f32.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i64]
@@ -209,7 +238,8 @@ def _load():
     for name in (
         "oq_set_num_threads oq_quant_rowwise_i8_f32 oq_quant_rowwise_i8_bf16 oq_gemm_i8_i32 "
         "oq_dequant_epilogue oq_linear_w8a8_f32 oq_linear_w8a8_bf16 oq_quant_tensor_fp8_f32 "
-        "oq_quant_tensor_fp8_bf16 oq_linear_fp8 oq_linear_f32 oq_rmsnorm_quant_i8_f32 oq_rmsnorm_quant_i8_bf16"
+        "oq_quant_tensor_fp8_bf16 oq_linear_fp8 oq_linear_f32 oq_rmsnorm_quant_i8_f32 oq_rmsnorm_quant_i8_bf16 "
+        "oq_swiglu_quant_i8_f32 oq_swiglu_quant_i8_bf16"
     ).split():
         getattr(lib, name).restype = None
     _lib = lib
@@ -274,6 +304,20 @@ def c_rmsnorm_quant_i8(x: np.ndarray, gamma: np.ndarray, eps: float, bf16_bits: 
     fn = lib.oq_rmsnorm_quant_i8_bf16 if bf16_bits else lib.oq_rmsnorm_quant_i8_f32
     fn(_p(x), _p(gamma), ctypes.c_float(eps), M, K, K, _p(q), _p(s), _p(y) if want_y else None)
     return (q, s, y) if want_y else (q, s)
+
+
+def c_swiglu_quant_i8(ug: np.ndarray, bf16_bits: bool = False, want_h: bool = False):
+    """ug: [M, 2F] = [up | gate], fp32 or (``bf16_bits``) uint16 bf16 patterns -> (codes [M,F], scale[, h fp32])."""
+    lib = _load()
+    ug = _c(ug, np.uint16 if bf16_bits else F32)
+    M, F2 = ug.shape
+    Fh = F2 // 2
+    q = np.empty((M, Fh), np.int8)
+    s = np.empty((M,), F32)
+    h = np.empty((M, Fh), F32) if want_h else None
+    fn = lib.oq_swiglu_quant_i8_bf16 if bf16_bits else lib.oq_swiglu_quant_i8_f32
+    fn(_p(ug), M, Fh, F2, _p(q), _p(s), _p(h) if want_h else None)
+    return (q, s, h) if want_h else (q, s)
 
 
 def c_gemm_i8_i32(xq: np.ndarray, wq: np.ndarray) -> np.ndarray:

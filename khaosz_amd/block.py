@@ -215,7 +215,8 @@ class MLP(nn.Module):
         if self._upgate is not None:
             ug = self._upgate(x) if codes is None else self._upgate.forward_codes(codes[0], codes[1], x.dtype).view(
                 *x.shape[:-1], -1)
-            if self._swiglu_quant and isinstance(self.down, QuantLinear) and ug.is_cuda:
+            if (self._swiglu_quant and isinstance(self.down, QuantLinear) and ug.is_cuda
+                    and ug.shape[-1] // 2 <= ops.SWIGLU_QUANT_MAX_F.get(ug.dtype, 0)):
                 # activation, product and the down projection's quantisation in one launch
                 hq, hs = ops.swiglu_quant_rowwise_i8(ug)
                 return self.down.forward_codes(hq, hs, x.dtype).view(*x.shape[:-1], -1)
@@ -253,7 +254,8 @@ class DecoderBlock(nn.Module):
 
     def forward(self, x: Tensor, rotary_emb: Tensor, attention_mask: Optional[Tensor] = None,
                 cache=None) -> Tensor:
-        if self._norm_quant and x.is_cuda and x.dtype == self.input_norm.weight.dtype:
+        if (self._norm_quant and x.is_cuda and x.dtype == self.input_norm.weight.dtype
+                and x.shape[-1] <= ops.RMSNORM_QUANT_MAX_K.get(x.dtype, 0)):
             n1, n2 = self.input_norm, self.post_attention_norm
             x = self.attention(x, rotary_emb, attention_mask, cache,
                                codes=ops.rmsnorm_quant_rowwise_i8(x, n1.weight, n1.norm_eps)) + x

@@ -72,6 +72,11 @@ def quant_rowwise_i8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     return q, s
 
 
+# longest rows the fused row kernels keep in registers (elements): bf16, fp32
+RMSNORM_QUANT_MAX_K = {torch.bfloat16: 12288, torch.float32: 6144}
+SWIGLU_QUANT_MAX_F = {torch.bfloat16: 6144, torch.float32: 3072}
+
+
 def rmsnorm_quant_rowwise_i8(x: torch.Tensor, gamma: torch.Tensor, eps: float) -> Tuple[torch.Tensor, torch.Tensor]:
     """RMSNorm (gain ``gamma``, same dtype as ``x``) fused with the per-token quantisation of its
     output: ``[..., K]`` -> (codes int8 ``[M, K]``, scales float32 ``[M]``)."""

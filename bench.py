@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized-Linear hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload decode|prefill|fp8]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload decode|prefill|fp8|block]
 
 A "step" is one pass of the hot path over one batch of synthetic input that is
 already resident in HBM:
@@ -50,7 +50,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="decode", choices=["decode", "prefill", "fp8"])
+    ap.add_argument("--workload", default="decode", choices=["decode", "prefill", "fp8", "block"])
     ap.add_argument("--m", type=int, default=16, help="decode rows (1..16)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary workloads")
@@ -283,6 +283,10 @@ def bench_block(torch, ops, args, dev):
     fuse_shared_inputs(blk, norms=True)
     ms_pre = graph_time_ms(torch, prefill, 10, 3)
     prefill()
+    ms_dec_norms = graph_time_ms(torch, decode_all, 3, 2) / steps
+    # and the single-token steps through the in-place paged attention kernels
+    fuse_shared_inputs(blk, norms=True, decode_attention=True)
+    prefill()
     ms_dec = graph_time_ms(torch, decode_all, 3, 2) / steps
 
     # The Linears alone (q/k/v and up/gate fused), at the shapes and in the order the block calls them (same modules,
@@ -308,6 +312,7 @@ def bench_block(torch, ops, args, dev):
         "value": ms_pre + steps * ms_dec, "unit": "ms", "prefill_ms": ms_pre, "decode_ms_per_step": ms_dec,
         "separate_projections": {"prefill_ms": ms_pre_sep, "decode_ms_per_step": ms_dec_sep},
         "fused_projections_separate_norms": {"prefill_ms": ms_pre_proj, "decode_ms_per_step": ms_dec_proj},
+        "fused_norms_torch_attention": {"prefill_ms": ms_pre, "decode_ms_per_step": ms_dec_norms},
         "linears_prefill_ms": ms_lin_pre, "linears_prefill_tops": lin_ops / (ms_lin_pre * 1e-3) / 1e12,
         "linears_decode_ms_per_step": ms_lin_dec, "linears_decode_gbs": lin_bytes / (ms_lin_dec * 1e-3) / 1e9,
         "non_linear_prefill_ms": ms_pre - ms_lin_pre, "non_linear_decode_ms_per_step": ms_dec - ms_lin_dec,
@@ -455,15 +460,14 @@ def main():
         sys.exit(2)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    fns = {"decode": bench_decode, "prefill": bench_prefill, "fp8": bench_fp8}
+    fns = {"decode": bench_decode, "prefill": bench_prefill, "fp8": bench_fp8, "block": bench_block}
     with torch.inference_mode():
         main_res = fns[args.workload](torch, ops, args, dev)
         extra = {}
         if not args.no_extra:
-            for name in ("decode", "prefill", "fp8"):
+            for name in ("decode", "prefill", "fp8", "block"):
                 if name != args.workload:
                     extra[name] = fns[name](torch, ops, args, dev)
-            extra["block"] = bench_block(torch, ops, args, dev)
             if args.workload == "decode":
                 for m in (1, 4):
                     a2 = argparse.Namespace(**vars(args))
@@ -473,7 +477,7 @@ def main():
         ceilings = measure_ceilings(torch, ops, dev)
     per_step = main_res.get("bytes_per_step") or main_res.get("ops_per_step") or main_res.get("flops_per_step")
     cpu = None
-    if not args.no_cpu:
+    if not args.no_cpu and args.workload != "block":
         cpu = cpu_baseline(args.workload, main_res["shape"], main_res["unit"], per_step)
         if not args.no_extra and "prefill" in extra:
             # one pass of the prefill shape as well, so both halves of the metric have a CPU figure
@@ -484,7 +488,7 @@ def main():
     line = {
         "metric": METRIC, "value": main_res["value"], "unit": main_res["unit"], "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": main_res["ms_per_step"],
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": main_res["dtype"],
+        "higher_is_better": main_res["unit"] != "ms", "scaling": "weak", "vs_baseline": None, "dtype": main_res["dtype"],
         "data": "synthetic", "config": {"workload": main_res["workload"], "timing": "HIP graph replay of the timed steps",
                                         "eager_ms_per_step": main_res.get("eager_ms_per_step")},
         "roofline": main_res["roofline"], "cpu_baseline": cpu, "measured_ceilings": ceilings,

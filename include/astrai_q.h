@@ -130,6 +130,35 @@ int aq_rmsnorm_quant_rowwise_i8(const void *x, int x_dtype, const void *gamma, i
 int aq_swiglu_quant_rowwise_i8(const void *ug, int dtype, int64_t M, int64_t F, int64_t ld,
                                int8_t *q, float *scale, void *stream);
 
+/* ---- decode-step attention over the paged KV cache (what sits between the qkv
+ * and the output projection at decode; bf16, head dimension 128).
+ *
+ * aq_rope_kv_write: for the one new token of each of B sequences, rotate the q
+ * and k heads of qkv [B, (Hq + 2 Hkv) * D] (q heads, then k heads, then v heads:
+ * the fused projection's column order) by freqs [B, D/2, 2] = (cos, sin) pairs --
+ * interleaved pairs (x[2i], x[2i+1]), fp32, as apply_rotary_emb does
+ * (astrai/model/components/rope.py:26-33) -- store q to q_out [B, Hq, D], and write
+ * the rotated k and the v into slot pos % page_size of page
+ * page_table[b, pos / page_size] of k_cache / v_cache
+ * [n_pages, page_size, Hkv, D] (Storage.write, astrai/inference/core/cache.py:216-252;
+ * a sequence whose page is unmapped, entry < 0, is skipped there too).
+ *
+ * aq_paged_attn_decode: out [B, Hq, D] = softmax(scale * q K^T) V over positions
+ * 0 .. total_len-1 of each sequence, read through page_table [B, P] in place --
+ * replaces Storage.gather (cache.py:254-274), repeat_kv (attention.py:15-23) and
+ * scaled_dot_product_attention (attention.py:98-100) for a step without padding
+ * mask.  Query heads h*G .. h*G+G-1 use KV head h, G = Hq / Hkv in {1, 2, 4, 8}.
+ * Positions whose page is unmapped count as zero keys and values (what gather's
+ * zero fill gives).  fp32 scores and sums; results within bf16 rounding of the
+ * reference flow, not bit-identical to it (summation order, exp2). */
+int aq_rope_kv_write(const void *qkv, const float *freqs, const int64_t *page_table, int64_t P,
+                     int64_t pos, int64_t page_size, void *k_cache, void *v_cache, int64_t n_pages,
+                     void *q_out, int64_t B, int64_t Hq, int64_t Hkv, int64_t D, void *stream);
+int aq_paged_attn_decode(const void *q, const void *k_cache, const void *v_cache,
+                         const int64_t *page_table, int64_t P, int64_t total_len, int64_t page_size,
+                         int64_t n_pages, float scale, void *out, int64_t B, int64_t Hq, int64_t Hkv,
+                         int64_t D, void *stream);
+
 /* Tuning and test hook, no counterpart in the reference: the GEMM entry points
  * pick their workgroup tile (256 x 128, or 128 x 128 with a split K step when
  * the larger one would leave compute units idle) from M and N.  rows = 128 or

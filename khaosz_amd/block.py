@@ -157,6 +157,7 @@ class GQA(nn.Module):
         self.v_proj = Linear(dim, n_kv_heads * self.head_dim)
         self.o_proj = Linear(dim, dim)
         self._qkv: Optional[QuantLinear] = None  # not a registered child: the state dict keeps q/k/v keys
+        self._decode_attention = False
 
     def fuse_projections(self) -> bool:
         """q, k and v read the same input (attention.py:83-85): once they are quantized, run them
@@ -166,11 +167,29 @@ class GQA(nn.Module):
             return True
         return False
 
+    def fuse_decode_attention(self) -> bool:
+        """A step with one new token per sequence on a paged cache: rotate q/k and write k/v into
+        their page slot in one launch, then attend over the pages in place in another
+        (``ops.rope_kv_write``, ``ops.paged_attn_decode``), instead of the gather / repeat_kv /
+        generic attention sequence.  Needs the fused q/k/v projection, bf16 and head dimension
+        128, and assumes what the serving loop's decode step has: no padding inside the cached
+        length (the additive mask is all zeros).  Outputs agree within bf16 rounding."""
+        if self._qkv is not None and self.head_dim == 128 and self.n_heads // self.n_kv_heads in (1, 2, 4, 8):
+            self._decode_attention = True
+        return self._decode_attention
+
     def forward(self, x: Tensor, rotary_emb: Tensor, attn_mask: Optional[Tensor] = None,
                 cache=None, codes: Optional[Tuple[Tensor, Tensor]] = None) -> Tensor:
         """``codes``: the already normalised and quantised input ``(xq [B*S, dim], sx [B*S])`` from a
         fused norm; ``x`` then only gives the shape and dtype."""
         B, S, _ = x.shape
+        if (self._decode_attention and S == 1 and isinstance(cache, PagedKV) and x.is_cuda
+                and x.dtype == torch.bfloat16):
+            qkv = self._qkv(x) if codes is None else self._qkv.forward_codes(codes[0], codes[1], x.dtype)
+            q = ops.rope_kv_write(qkv.view(B, -1), rotary_emb.reshape(B, -1), cache.page_table, cache.total_len - 1,
+                                  cache.k, cache.v, self.n_heads, self.n_kv_heads)
+            out = ops.paged_attn_decode(q, cache.k, cache.v, cache.page_table, cache.total_len)
+            return self.o_proj(out.view(B, 1, -1))
         if self._qkv is not None:
             nq, nkv = self.n_heads * self.head_dim, self.n_kv_heads * self.head_dim
             qkv = self._qkv(x) if codes is None else self._qkv.forward_codes(codes[0], codes[1], x.dtype).view(B, S, -1)

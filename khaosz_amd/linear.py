@@ -251,14 +251,16 @@ TARGET_MODULES_ATTN = {"q_proj", "k_proj", "v_proj", "o_proj"}
 TARGET_MODULES_FFN = {"up", "gate", "down"}
 
 
-def fuse_shared_inputs(model: nn.Module, norms: bool = False) -> int:
+def fuse_shared_inputs(model: nn.Module, norms: bool = False, decode_attention: bool = False) -> int:
     """Call ``fuse_projections()`` on every module that offers it (attention and MLP blocks whose
     projections read one input); returns how many fused modules were built.  Run it after
     ``quantize_model`` and after loading weights: the fused module owns the weight storage from
     then on.  Outputs stay bit-identical.  ``norms=True`` additionally lets blocks compute
     RMSNorm and the quantisation of its output in one launch (``fuse_norm_quant()``), which
     drops the bf16 rounding of the normalised activations: not bit-identical, inside the
-    quantisation noise."""
+    quantisation noise.  ``decode_attention=True`` lets attention modules with a fused q/k/v
+    projection run single-token steps on a paged cache through the in-place attention kernels
+    (``fuse_decode_attention()``)."""
     n = 0
     for m in model.modules():
         f = getattr(m, "fuse_projections", None)
@@ -267,6 +269,11 @@ def fuse_shared_inputs(model: nn.Module, norms: bool = False) -> int:
     if norms:
         for m in model.modules():
             f = getattr(m, "fuse_norm_quant", None)
+            if callable(f):
+                f()
+    if decode_attention:
+        for m in model.modules():
+            f = getattr(m, "fuse_decode_attention", None)
             if callable(f):
                 f()
     return n

@@ -252,6 +252,66 @@ def gemv_w8a8_codes(xq, sx, wq, sw, bias=None, out_dtype=torch.bfloat16) -> torc
     return y
 
 
+def rope_kv_write(qkv: torch.Tensor, freqs: torch.Tensor, page_table: torch.Tensor, pos: int, k_cache: torch.Tensor,
+                  v_cache: torch.Tensor, n_heads: int, n_kv_heads: int) -> torch.Tensor:
+    """One new token per sequence: rotate q and k of ``qkv [B, (Hq + 2 Hkv) * 128]`` by ``freqs``
+    (complex64 ``[B, 64]`` or float32 ``[B, 64, 2]``), write k and v into the paged caches
+    ``[n_pages, page, Hkv, 128]`` at logical position ``pos``; returns the rotated ``q [B, Hq, 128]``."""
+    _need_gpu(qkv, freqs, page_table, k_cache, v_cache)
+    B = qkv.shape[0]
+    D = k_cache.shape[-1]
+    if qkv.dtype != torch.bfloat16 or k_cache.dtype != torch.bfloat16 or v_cache.dtype != torch.bfloat16:
+        raise ValueError("rope_kv_write takes bfloat16 activations and caches")
+    if qkv.dim() != 2 or qkv.shape[1] != (n_heads + 2 * n_kv_heads) * D:
+        raise ValueError(f"qkv must be [B, {(n_heads + 2 * n_kv_heads) * D}], got {tuple(qkv.shape)}")
+    if k_cache.dim() != 4 or k_cache.shape != v_cache.shape or k_cache.shape[2] != n_kv_heads:
+        raise ValueError("caches must be [n_pages, page, Hkv, D] and alike")
+    if not (k_cache.is_contiguous() and v_cache.is_contiguous()):
+        raise ValueError("caches must be contiguous")
+    fr = torch.view_as_real(freqs) if freqs.is_complex() else freqs
+    fr = fr.reshape(B, D // 2, 2).to(torch.float32).contiguous()
+    if page_table.dtype != torch.int64 or page_table.dim() != 2 or page_table.shape[0] != B:
+        raise ValueError("page_table must be int64 [B, P]")
+    page_table = page_table.contiguous()
+    qkv = qkv.contiguous()
+    q = torch.empty((B, n_heads, D), dtype=torch.bfloat16, device=qkv.device)
+    if B:
+        with torch.cuda.device(qkv.device):
+            rc = _abi.load().aq_rope_kv_write(qkv.data_ptr(), fr.data_ptr(), page_table.data_ptr(), page_table.shape[1],
+                                              int(pos), k_cache.shape[1], k_cache.data_ptr(), v_cache.data_ptr(),
+                                              k_cache.shape[0], q.data_ptr(), B, n_heads, n_kv_heads, D, _stream(qkv))
+        _abi.check(rc, "aq_rope_kv_write")
+    return q
+
+
+def paged_attn_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, page_table: torch.Tensor,
+                      total_len: int, scale: Optional[float] = None) -> torch.Tensor:
+    """``softmax(scale * q K^T) V`` for one query token per sequence over the first ``total_len``
+    positions of each sequence's pages: ``q [B, Hq, 128]`` -> ``[B, Hq, 128]`` (bfloat16)."""
+    _need_gpu(q, k_cache, v_cache, page_table)
+    if q.dtype != torch.bfloat16 or k_cache.dtype != torch.bfloat16 or v_cache.dtype != torch.bfloat16:
+        raise ValueError("paged_attn_decode takes bfloat16 tensors")
+    if q.dim() != 3 or k_cache.dim() != 4 or k_cache.shape != v_cache.shape or q.shape[2] != k_cache.shape[3]:
+        raise ValueError("q must be [B, Hq, D] and the caches [n_pages, page, Hkv, D]")
+    if not (k_cache.is_contiguous() and v_cache.is_contiguous()):
+        raise ValueError("caches must be contiguous")
+    B, Hq, D = q.shape
+    Hkv = k_cache.shape[2]
+    if page_table.dtype != torch.int64 or page_table.dim() != 2 or page_table.shape[0] != B:
+        raise ValueError("page_table must be int64 [B, P]")
+    page_table, q = page_table.contiguous(), q.contiguous()
+    out = torch.empty_like(q)
+    if B:
+        with torch.cuda.device(q.device):
+            rc = _abi.load().aq_paged_attn_decode(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+                                                  page_table.data_ptr(), page_table.shape[1], int(total_len),
+                                                  k_cache.shape[1], k_cache.shape[0],
+                                                  float(scale if scale is not None else D ** -0.5), out.data_ptr(),
+                                                  B, Hq, Hkv, D, _stream(q))
+        _abi.check(rc, "aq_paged_attn_decode")
+    return out
+
+
 def set_gemm_tile(rows: int) -> None:
     """Force the GEMM workgroup tile to 128 or 256 rows for this process (0: choose by shape)."""
     _abi.check(_abi.load().aq_set_gemm_tile(int(rows)), "aq_set_gemm_tile")

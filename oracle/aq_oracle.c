@@ -51,6 +51,11 @@
  *                         restatement bit for bit (numpy has no fma: the comparison
  *                         runs the polynomial in float64 products rounded once, which
  *                         is what an fma is), and on closed forms (g = 0, large |g|).
+ *   oq_rope_kv_write,     restate apply_rotary_emb (rope.py:26-33), Storage.write / gather
+ *   oq_paged_attn_decode  (cache.py:216-274), repeat_kv and softmax attention
+ *                         (attention.py:15-23,93-103) for one new token per sequence;
+ *                         pinned against torch (complex multiply, index writes,
+ *                         scaled_dot_product_attention in fp32) within rounding.
  *
  * Build: gcc -O3 -march=native -fopenmp -ffp-contract=off -fno-fast-math
  *        -shared -fPIC (oracle/build_oracle.py).  OpenMP only parallelises over
@@ -303,6 +308,91 @@ void oq_swiglu_quant_i8_bf16(const uint16_t *ug, int64_t M, int64_t F, int64_t l
     if (h_out) memcpy(h_out + m * F, h, (size_t)F * sizeof(float));
     free(h);
   }
+}
+
+/* ------------------------------------------- decode attention over paged KV */
+
+/* One new token per sequence at logical position pos.  qkv: [B, (Hq+2Hkv)*D] bf16,
+ * q heads then k heads then v heads; freqs: [B, D/2, 2] (cos, sin).  Interleaved
+ * pairs are rotated in fp32 -- (x0 + i x1)(c + i s), products and sums rounded
+ * one by one -- and cast to bf16 (rope.py:26-33).  q goes to q_out [B, Hq, D]; k
+ * and v go to slot pos % page of page table[b, pos / page] of the caches
+ * [n_pages, page, Hkv, D]; sequences whose page is unmapped are skipped
+ * (cache.py:216-252). */
+void oq_rope_kv_write(const uint16_t *qkv, const float *freqs, const int64_t *table, int64_t P,
+                      int64_t pos, int64_t page, uint16_t *kc, uint16_t *vc, int64_t n_pages,
+                      uint16_t *q_out, int64_t B, int64_t Hq, int64_t Hkv, int64_t D) {
+  const int64_t heads = Hq + 2 * Hkv;
+  for (int64_t b = 0; b < B; ++b) {
+    const int64_t lp = pos / page;
+    const int64_t phys = lp < P ? table[b * P + lp] : -1;
+    for (int64_t h = 0; h < heads; ++h) {
+      const uint16_t *src = qkv + (b * heads + h) * D;
+      uint16_t tmp[1024];
+      for (int64_t i = 0; i < D / 2; ++i) {
+        if (h < Hq + Hkv) {
+          const float x0 = oq_bf16_to_f32(src[2 * i]), x1 = oq_bf16_to_f32(src[2 * i + 1]);
+          const float c = freqs[(b * (D / 2) + i) * 2], sn = freqs[(b * (D / 2) + i) * 2 + 1];
+          const float a = x0 * c, bb = x1 * sn, cc = x0 * sn, dd = x1 * c;
+          tmp[2 * i] = oq_f32_to_bf16(a - bb);
+          tmp[2 * i + 1] = oq_f32_to_bf16(cc + dd);
+        } else {
+          tmp[2 * i] = src[2 * i];
+          tmp[2 * i + 1] = src[2 * i + 1];
+        }
+      }
+      if (h < Hq) {
+        memcpy(q_out + (b * Hq + h) * D, tmp, (size_t)D * 2);
+      } else if (phys >= 0 && phys < n_pages) {
+        const int is_k = h < Hq + Hkv;
+        const int64_t kvh = is_k ? h - Hq : h - Hq - Hkv;
+        uint16_t *dst = (is_k ? kc : vc) + ((phys * page + pos % page) * Hkv + kvh) * D;
+        memcpy(dst, tmp, (size_t)D * 2);
+      }
+    }
+  }
+}
+
+/* out[b, h, :] = softmax_t(scale * q[b,h] . K[b,t,h/G]) V[b,t,h/G], t < T, read through
+ * the page table; unmapped pages are zero keys and values (cache.py:254-274 zero
+ * fill).  fp32, t and d ascending, libm expf. */
+void oq_paged_attn_decode(const uint16_t *q, const uint16_t *kc, const uint16_t *vc,
+                          const int64_t *table, int64_t P, int64_t T, int64_t page, int64_t n_pages,
+                          float scale, uint16_t *out, int64_t B, int64_t Hq, int64_t Hkv, int64_t D) {
+  const int64_t G = Hq / Hkv;
+#pragma omp parallel for schedule(static) collapse(2)
+  for (int64_t b = 0; b < B; ++b)
+    for (int64_t h = 0; h < Hq; ++h) {
+      const int64_t kvh = h / G;
+      float *s = (float *)malloc((size_t)T * sizeof(float));
+      float *acc = (float *)calloc((size_t)D, sizeof(float));
+      float m = -INFINITY;
+      for (int64_t t = 0; t < T; ++t) {
+        const int64_t lp = t / page;
+        const int64_t phys = lp < P ? table[b * P + lp] : -1;
+        float d = 0.0f;
+        if (phys >= 0 && phys < n_pages) {
+          const uint16_t *k = kc + ((phys * page + t % page) * Hkv + kvh) * D;
+          for (int64_t i = 0; i < D; ++i) d += oq_bf16_to_f32(q[(b * Hq + h) * D + i]) * oq_bf16_to_f32(k[i]);
+        }
+        s[t] = d * scale;
+        if (s[t] > m) m = s[t];
+      }
+      float l = 0.0f;
+      for (int64_t t = 0; t < T; ++t) {
+        const float pt = expf(s[t] - m);
+        l += pt;
+        const int64_t lp = t / page;
+        const int64_t phys = lp < P ? table[b * P + lp] : -1;
+        if (phys >= 0 && phys < n_pages) {
+          const uint16_t *v = vc + ((phys * page + t % page) * Hkv + kvh) * D;
+          for (int64_t i = 0; i < D; ++i) acc[i] += pt * oq_bf16_to_f32(v[i]);
+        }
+      }
+      for (int64_t i = 0; i < D; ++i) out[(b * Hq + h) * D + i] = oq_f32_to_bf16(acc[i] / l);
+      free(s);
+      free(acc);
+    }
 }
 
 /* ------------------------------------------------------------- int8 GEMM */

@@ -227,6 +227,8 @@ def _load():
     lib.oq_swiglu_quant_i8_bf16.argtypes = [vp, i64, i64, i64, vp, vp, vp]
     lib.oq_exp_repro.argtypes = [ctypes.c_float]
     lib.oq_exp_repro.restype = ctypes.c_float
+    lib.oq_rope_kv_write.argtypes = [vp, vp, vp, i64, i64, i64, vp, vp, i64, vp, i64, i64, i64, i64]
+    lib.oq_paged_attn_decode.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, ctypes.c_float, vp, i64, i64, i64, i64]
     lib.oq_gemm_i8_i32.argtypes = [vp, vp, vp, i64, i64, i64]
     lib.oq_dequant_epilogue.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64]
     lib.oq_linear_w8a8_f32.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i64]
@@ -239,7 +241,7 @@ def _load():
         "oq_set_num_threads oq_quant_rowwise_i8_f32 oq_quant_rowwise_i8_bf16 oq_gemm_i8_i32 "
         "oq_dequant_epilogue oq_linear_w8a8_f32 oq_linear_w8a8_bf16 oq_quant_tensor_fp8_f32 "
         "oq_quant_tensor_fp8_bf16 oq_linear_fp8 oq_linear_f32 oq_rmsnorm_quant_i8_f32 oq_rmsnorm_quant_i8_bf16 "
-        "oq_swiglu_quant_i8_f32 oq_swiglu_quant_i8_bf16"
+        "oq_swiglu_quant_i8_f32 oq_swiglu_quant_i8_bf16 oq_rope_kv_write oq_paged_attn_decode"
     ).split():
         getattr(lib, name).restype = None
     _lib = lib
@@ -318,6 +320,31 @@ def c_swiglu_quant_i8(ug: np.ndarray, bf16_bits: bool = False, want_h: bool = Fa
     fn = lib.oq_swiglu_quant_i8_bf16 if bf16_bits else lib.oq_swiglu_quant_i8_f32
     fn(_p(ug), M, Fh, F2, _p(q), _p(s), _p(h) if want_h else None)
     return (q, s, h) if want_h else (q, s)
+
+
+def c_rope_kv_write(qkv, freqs, table, pos, kc, vc, Hq, Hkv):
+    """bf16 bit patterns (uint16) throughout; kc / vc [n_pages, page, Hkv, D] are updated in place.
+    Returns the rotated q [B, Hq, D]."""
+    lib = _load()
+    qkv, freqs, table = _c(qkv, np.uint16), _c(freqs, F32), _c(table, np.int64)
+    assert kc.dtype == np.uint16 and vc.dtype == np.uint16 and kc.flags.c_contiguous and vc.flags.c_contiguous
+    B = qkv.shape[0]
+    n_pages, page, _, D = kc.shape
+    q = np.empty((B, Hq, D), np.uint16)
+    lib.oq_rope_kv_write(_p(qkv), _p(freqs), _p(table), table.shape[1], pos, page, _p(kc), _p(vc), n_pages, _p(q),
+                         B, Hq, Hkv, D)
+    return q
+
+
+def c_paged_attn_decode(q, kc, vc, table, total_len, scale):
+    lib = _load()
+    q, kc, vc, table = _c(q, np.uint16), _c(kc, np.uint16), _c(vc, np.uint16), _c(table, np.int64)
+    B, Hq, D = q.shape
+    n_pages, page, Hkv, _ = kc.shape
+    out = np.empty((B, Hq, D), np.uint16)
+    lib.oq_paged_attn_decode(_p(q), _p(kc), _p(vc), _p(table), table.shape[1], total_len, page, n_pages,
+                             ctypes.c_float(scale), _p(out), B, Hq, Hkv, D)
+    return out
 
 
 def c_gemm_i8_i32(xq: np.ndarray, wq: np.ndarray) -> np.ndarray:

@@ -291,3 +291,40 @@ def test_fused_norm_quantise_stays_inside_the_quantisation_noise():
             err_b = ((yb.float() - r).norm() / r.norm()).item()
             assert err_b < 3e-2 and err_b < 1.2 * err_a + 1e-3, (err_a, err_b)
             assert ((ya.float() - yb.float()).norm() / r.norm()).item() < 1.5e-2
+
+
+@pytest.mark.gpu
+def test_decode_attention_kernels_track_the_torch_attention_path():
+    """Single-token steps on a paged cache through rope_kv_write + paged_attn_decode against the
+    same quantized block running gather / repeat_kv / scaled_dot_product_attention: same cache
+    contents up to one bf16 step of the rotation, outputs within bf16 rounding, for several steps."""
+    from khaosz_amd import fuse_shared_inputs
+
+    dev, dt = "cuda:0", torch.bfloat16
+    torch.manual_seed(3)
+    a = DecoderBlock(512, 4, 1408, 2)             # head dimension 128, two query heads per KV head
+    a.reset_parameters()
+    a = a.to(dev).to(dt)
+    b = DecoderBlock(512, 4, 1408, 2).to(dev).to(dt)
+    b.load_state_dict(a.state_dict())
+    quantize_model(a), quantize_model(b)
+    fuse_shared_inputs(a)
+    fuse_shared_inputs(b, decode_attention=True)
+    assert b.attention._decode_attention and not a.attention._decode_attention
+    B, S, steps, page = 3, 70, 4, 16
+    tab = rotary_table(128, 128, device=dev)
+    table = torch.tensor([[7, 0, 9, 3, 12], [1, 8, 4, 10, 5], [2, 11, 6, 13, 14]], device=dev)
+    ca, cb = PagedKV(16, page, 2, 128, dev, dt), PagedKV(16, page, 2, 128, dev, dt)
+    x = torch.randn(B, S + steps, 512, device=dev).to(dt)
+    with torch.inference_mode():
+        pa = a(x[:, :S], _freqs(tab, B, 0, S), None, ca.bind(table, S))
+        pb = b(x[:, :S], _freqs(tab, B, 0, S), None, cb.bind(table, S))
+        assert torch.equal(pa, pb)                                   # prefill takes the same path in both
+        for t in range(steps):
+            pos = S + t
+            mask = decode_mask(B, pos + 1, dev, dt)
+            ya = a(x[:, pos:pos + 1], _freqs(tab, B, pos, 1), mask, ca.bind(table, pos + 1))
+            yb = b(x[:, pos:pos + 1], _freqs(tab, B, pos, 1), mask, cb.bind(table, pos + 1))
+            rel = ((ya.float() - yb.float()).norm() / ya.float().norm()).item()
+            assert rel < 1e-2, (t, rel)
+        assert torch.allclose(ca.k.float(), cb.k.float(), rtol=1e-2, atol=1e-2) and torch.equal(ca.v, cb.v)

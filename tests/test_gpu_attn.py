@@ -1,0 +1,77 @@
+"""Decode-step attention kernels against the oracle, through the C ABI (GPU)."""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+from khaosz_amd import ops  # noqa: E402
+
+DEV = "cuda:0"
+
+
+def _say(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def _bits(t):
+    return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16).copy()
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,page,pos", [(1, 1, 1, 4, 0), (3, 4, 2, 8, 13), (8, 16, 4, 64, 575), (5, 8, 1, 16, 31)])
+def test_rope_kv_write_bit_exact(oracle, B, Hq, Hkv, page, pos):
+    _say("rope_kv_write", B, Hq, Hkv, page, pos)
+    D = 128
+    P = pos // page + 2
+    n_pages = B * P + 3
+    g = torch.Generator().manual_seed(B * 100 + pos)
+    qkv = torch.randn(B, (Hq + 2 * Hkv) * D, generator=g).to(torch.bfloat16)
+    ang = torch.rand(B, D // 2, generator=g) * 6.28
+    freqs = torch.polar(torch.ones_like(ang), ang)
+    table = torch.randperm(n_pages, generator=g)[:B * P].view(B, P)
+    if B > 2:
+        table[1, pos // page] = -1                      # this sequence's token has no page: skipped
+    kc = torch.randn(n_pages, page, Hkv, D, generator=g).to(torch.bfloat16)
+    vc = torch.randn(n_pages, page, Hkv, D, generator=g).to(torch.bfloat16)
+    kb, vb = _bits(kc), _bits(vc)
+    qo = oracle.c_rope_kv_write(_bits(qkv), torch.view_as_real(freqs).numpy(), table.numpy(), pos, kb, vb, Hq, Hkv)
+    kd, vd = kc.to(DEV), vc.to(DEV)
+    q = ops.rope_kv_write(qkv.to(DEV), freqs.to(DEV), table.to(DEV), pos, kd, vd, Hq, Hkv)
+    assert np.array_equal(_bits(q), qo)
+    assert np.array_equal(_bits(kd), kb) and np.array_equal(_bits(vd), vb)
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,page,T", [(1, 1, 1, 4, 1), (2, 8, 2, 16, 70), (8, 16, 4, 64, 576), (3, 8, 1, 16, 1000),
+                                              (2, 4, 2, 64, 513)])
+def test_paged_attn_decode_within_bf16_rounding(oracle, B, Hq, Hkv, page, T):
+    _say("paged_attn_decode", B, Hq, Hkv, page, T)
+    D = 128
+    P = (T + page - 1) // page
+    n_pages = B * P + 2
+    g = torch.Generator().manual_seed(T)
+    q = (torch.randn(B, Hq, D, generator=g) * 1.5).to(torch.bfloat16)
+    kc = torch.randn(n_pages, page, Hkv, D, generator=g).to(torch.bfloat16)
+    vc = torch.randn(n_pages, page, Hkv, D, generator=g).to(torch.bfloat16)
+    table = torch.randperm(n_pages, generator=g)[:B * P].view(B, P)
+    if P > 2:
+        table[B - 1, 1] = -1                             # an unmapped page in the middle: zero keys and values
+    want = torch.from_numpy(oracle.c_paged_attn_decode(_bits(q), _bits(kc), _bits(vc), table.numpy(), T,
+                                                       D ** -0.5).view(np.int16)).view(torch.bfloat16).float()
+    out = ops.paged_attn_decode(q.to(DEV), kc.to(DEV), vc.to(DEV), table.to(DEV), T).cpu().float()
+    # stated tolerance: 1e-2 relative for bf16 outputs (different summation order, exp2 instead of exp)
+    assert torch.allclose(out, want, rtol=1e-2, atol=1e-2)
+    assert ((out - want).norm() / want.norm()).item() < 4e-3
+
+
+def test_attn_argument_checks():
+    q = torch.zeros(2, 4, 64, dtype=torch.bfloat16, device=DEV)
+    kc = torch.zeros(4, 8, 2, 64, dtype=torch.bfloat16, device=DEV)
+    tab = torch.zeros(2, 2, dtype=torch.int64, device=DEV)
+    with pytest.raises(ValueError):
+        ops.paged_attn_decode(q, kc, kc.clone(), tab, 5)          # head dimension 64 is not supported
+    q = torch.zeros(2, 6, 128, dtype=torch.bfloat16, device=DEV)
+    kc = torch.zeros(4, 8, 2, 128, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(ValueError):
+        ops.paged_attn_decode(q, kc, kc.clone(), tab, 5)          # 3 query heads per KV head

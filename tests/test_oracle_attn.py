@@ -1,0 +1,63 @@
+"""Pins the oracle's decode attention over a paged KV cache (CPU) against torch: the complex
+multiply of apply_rotary_emb (astrai/model/components/rope.py:26-33), index writes and gathers
+through a page table (astrai/inference/core/cache.py:216-274) and scaled_dot_product_attention
+with repeated KV heads (astrai/model/components/attention.py:15-23,93-103)."""
+import numpy as np
+import torch
+import torch.nn.functional as F
+
+
+def _bits(t):
+    return t.contiguous().view(torch.int16).numpy().view(np.uint16).copy()
+
+
+def _bf16(a):
+    return torch.from_numpy(a.view(np.int16).copy()).view(torch.bfloat16)
+
+
+def test_rope_and_page_write_match_torch(oracle):
+    B, Hq, Hkv, D, page, n_pages, pos = 3, 4, 2, 128, 8, 12, 13
+    g = torch.Generator().manual_seed(0)
+    qkv = torch.randn(B, (Hq + 2 * Hkv) * D, generator=g).to(torch.bfloat16)
+    ang = torch.rand(B, D // 2, generator=g) * 6.28
+    freqs = torch.polar(torch.ones_like(ang), ang)                       # complex64 [B, D/2]
+    table = torch.tensor([[5, 2, 9], [0, -1, 11], [3, 7, 1]])            # sequence 1: page of pos 13 unmapped
+    kc = torch.zeros(n_pages, page, Hkv, D, dtype=torch.bfloat16)
+    vc = torch.zeros_like(kc)
+    kb, vb = _bits(kc), _bits(vc)
+    q = oracle.c_rope_kv_write(_bits(qkv), torch.view_as_real(freqs).numpy(), table.numpy(), pos, kb, vb, Hq, Hkv)
+    # torch: the reference's expression
+    x = qkv.view(B, 1, Hq + 2 * Hkv, D)
+    xr = torch.view_as_real(torch.view_as_complex(x.float().reshape(B, 1, -1, D // 2, 2)) *
+                            freqs.view(B, 1, 1, D // 2)).flatten(-2).to(torch.bfloat16)
+    assert torch.equal(_bf16(q), xr[:, 0, :Hq])
+    for b in range(B):
+        phys = table[b, pos // page].item()
+        if phys < 0:
+            continue
+        assert torch.equal(_bf16(kb)[phys, pos % page], xr[b, 0, Hq:Hq + Hkv])
+        assert torch.equal(_bf16(vb)[phys, pos % page], x[b, 0, Hq + Hkv:])
+    untouched = torch.ones(n_pages, page, dtype=torch.bool)
+    untouched[5 // 1 * 0 + table[0, 1], pos % page] = False
+    untouched[table[2, 1], pos % page] = False
+    assert not _bf16(kb)[untouched].any() and not _bf16(vb)[untouched].any()
+
+
+def test_paged_attention_matches_torch_sdpa(oracle):
+    B, Hq, Hkv, D, page, n_pages, T = 2, 8, 2, 128, 16, 10, 70
+    g = torch.Generator().manual_seed(1)
+    q = torch.randn(B, Hq, D, generator=g).to(torch.bfloat16)
+    kc = torch.randn(n_pages, page, Hkv, D, generator=g).to(torch.bfloat16)
+    vc = torch.randn(n_pages, page, Hkv, D, generator=g).to(torch.bfloat16)
+    table = torch.tensor([[4, 0, 7, 2, 9], [1, 8, -1, 3, 5]])           # an unmapped page inside sequence 1
+    out = _bf16(oracle.c_paged_attn_decode(_bits(q), _bits(kc), _bits(vc), table.numpy(), T, D ** -0.5)).float()
+    # torch: gather with zero fill, repeat heads, attention in fp32
+    safe = table.clamp(min=0)
+    k = kc[safe].flatten(1, 2).float()
+    v = vc[safe].flatten(1, 2).float()
+    hole = (table < 0).unsqueeze(-1).expand(-1, -1, page).flatten(1, 2)[:, :, None, None]
+    k, v = k.masked_fill(hole, 0.0)[:, :T], v.masked_fill(hole, 0.0)[:, :T]
+    k, v = k.repeat_interleave(Hq // Hkv, dim=2), v.repeat_interleave(Hq // Hkv, dim=2)
+    ref = F.scaled_dot_product_attention(q.float().unsqueeze(2), k.transpose(1, 2), v.transpose(1, 2))[:, :, 0]
+    assert torch.allclose(out, ref, rtol=1e-2, atol=1e-2)
+    assert (out - ref).norm() / ref.norm() < 3e-3

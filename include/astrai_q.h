@@ -135,7 +135,9 @@ int aq_swiglu_quant_rowwise_i8(const void *ug, int dtype, int64_t M, int64_t F, 
  *
  * aq_rope_kv_write: for the one new token of each of B sequences, rotate the q
  * and k heads of qkv [B, (Hq + 2 Hkv) * D] (q heads, then k heads, then v heads:
- * the fused projection's column order) by freqs [B, D/2, 2] = (cos, sin) pairs --
+ * the fused projection's column order) by freqs [B, D/2, 2] = (cos, sin) pairs
+ * (freqs_stride floats from one sequence's table to the next; 0 when all sequences
+ * are at the same position and share one) --
  * interleaved pairs (x[2i], x[2i+1]), fp32, as apply_rotary_emb does
  * (astrai/model/components/rope.py:26-33) -- store q to q_out [B, Hq, D], and write
  * the rotated k and the v into slot pos % page_size of page
@@ -151,7 +153,8 @@ int aq_swiglu_quant_rowwise_i8(const void *ug, int dtype, int64_t M, int64_t F, 
  * Positions whose page is unmapped count as zero keys and values (what gather's
  * zero fill gives).  fp32 scores and sums; results within bf16 rounding of the
  * reference flow, not bit-identical to it (summation order, exp2). */
-int aq_rope_kv_write(const void *qkv, const float *freqs, const int64_t *page_table, int64_t P,
+int aq_rope_kv_write(const void *qkv, const float *freqs, int64_t freqs_stride,
+                     const int64_t *page_table, int64_t P,
                      int64_t pos, int64_t page_size, void *k_cache, void *v_cache, int64_t n_pages,
                      void *q_out, int64_t B, int64_t Hq, int64_t Hkv, int64_t D, void *stream);
 int aq_paged_attn_decode(const void *q, const void *k_cache, const void *v_cache,

@@ -21,12 +21,11 @@
 namespace aq {
 
 constexpr int AD = 128;          // head dimension
-constexpr int ATT_WAVES = 8;     // wavefronts per (sequence, KV head)
-constexpr int ATT_THREADS = ATT_WAVES * 64;
 
 struct RopeArgs {
   const uint16_t* qkv;   // [B, (Hq + 2 Hkv) * D]
-  const float* freqs;    // [B, D/2, 2] (cos, sin) of the new token's position
+  const float* freqs;    // [B, D/2, 2] (cos, sin) of the new token's position; sequence stride freqs_stride floats
+  int64_t freqs_stride;
   const int64_t* table;  // [B, P]
   uint16_t* kc;          // [n_pages, page, Hkv, D]
   uint16_t* vc;
@@ -44,7 +43,7 @@ __global__ __launch_bounds__(64) void rope_kv_write_kernel(RopeArgs p) {
   uint32_t out = pair;
   if (h < p.Hq + p.Hkv) {  // q and k heads rotate, v heads do not
     const float x0 = bf16_bits_to_f32((uint16_t)(pair & 0xffffu)), x1 = bf16_bits_to_f32((uint16_t)(pair >> 16));
-    const float2 cs = reinterpret_cast<const float2*>(p.freqs + (int64_t)b * AD)[lane];
+    const float2 cs = reinterpret_cast<const float2*>(p.freqs + (int64_t)b * p.freqs_stride)[lane];
     // (x0 + i x1)(c + i s): four rounded products, one rounded difference, one rounded sum
     const float r0 = __fsub_rn(__fmul_rn(x0, cs.x), __fmul_rn(x1, cs.y));
     const float r1 = __fadd_rn(__fmul_rn(x0, cs.y), __fmul_rn(x1, cs.x));
@@ -76,16 +75,19 @@ struct AttnArgs {
 
 // Workgroup = one (sequence, KV head): its G query heads share every K and V
 // byte.  The T cached positions are cut into batches of 64; wavefront w takes
-// batches w, w + 8, ...  In a batch lane l owns key position t0 + l for the
-// scores (its 256-byte K row against the G queries held in LDS) and the
-// dimension pair (2l, 2l+1) for the weighted sum of V rows.  Each wavefront keeps
-// a running maximum, denominator and numerator per head (online softmax); the
-// eight partial results are merged through LDS at the end.
-template <int G>
-__global__ __launch_bounds__(ATT_THREADS) void paged_attn_decode_kernel(AttnArgs p) {
+// batches w, w + ATT_WAVES, ...  In a batch lane l owns key position t0 + l for
+// the scores (its 256-byte K row against the G queries held in LDS) and the
+// dimension pair (2l, 2l+1) for the weighted sum of V rows.  All of a batch's
+// loads -- 16 per lane for K, 64 for V -- are requested before anything is
+// computed: with a few dozen workgroups on the device the kernel lives on memory
+// latency, not bandwidth.  Each wavefront keeps a running maximum, denominator
+// and numerator per head (online softmax); the partial results are merged
+// through LDS at the end.
+template <int G, int ATT_WAVES>
+__global__ __launch_bounds__(ATT_WAVES * 64) void paged_attn_decode_kernel(AttnArgs p) {
+  constexpr int ATT_THREADS = ATT_WAVES * 64;
   __shared__ float q_s[G][AD];                       // queries, pre-scaled
   __shared__ float p_s[ATT_WAVES][64][G];            // a batch's probabilities, per wavefront
-  __shared__ int64_t row_s[ATT_WAVES][64];           // a batch's row offsets into the caches (-1: zero row)
   __shared__ float m_s[ATT_WAVES][G], l_s[ATT_WAVES][G];
   __shared__ float acc_s[ATT_WAVES][G][AD];
   const int tid = threadIdx.x, lane = tid & 63;
@@ -124,6 +126,15 @@ __global__ __launch_bounds__(ATT_THREADS) void paged_attn_decode_kernel(AttnArgs
     } else {
 #pragma unroll
       for (int c = 0; c < AD / 8; ++c) kv[c] = make_uint4(0, 0, 0, 0);
+    }
+    // the V rows of the whole batch: the row offset of key j sits in lane j
+    const int nkeys = (T - t0) < 64 ? (int)(T - t0) : 64;
+    uint32_t vv[64];
+#pragma unroll
+    for (int j = 0; j < 64; ++j) {
+      const int lo = __builtin_amdgcn_readlane((int)(uint32_t)row, j), hi = __builtin_amdgcn_readlane((int)(row >> 32), j);
+      const int64_t r = ((int64_t)hi << 32) | (uint32_t)lo;  // wavefront-uniform
+      vv[j] = (j < nkeys && r >= 0) ? reinterpret_cast<const uint32_t*>(p.vc + r)[lane] : 0u;
     }
     float s[G];
 #pragma unroll
@@ -172,29 +183,18 @@ __global__ __launch_bounds__(ATT_THREADS) void paged_attn_decode_kernel(AttnArgs
       m[g] = mn;
       p_s[wave][lane][g] = pv;
     }
-    row_s[wave][lane] = row;
     __builtin_amdgcn_s_waitcnt(0xc07f);  // this wavefront's LDS writes are done (wavefront-private region)
     asm volatile("" ::: "memory");
-    // ---- numerator: lane owns dimensions 2l, 2l+1 of every V row of the batch
-    const int nkeys = (T - t0) < 64 ? (int)(T - t0) : 64;
-    for (int j0 = 0; j0 < nkeys; j0 += 8) {
-      uint32_t vv[8];
+    // ---- numerator: lane owns dimensions 2l, 2l+1 of every V row of the batch (zero rows and
+    // positions past T carry probability-weighted zeros)
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const int64_t r = (j0 + j) < nkeys ? row_s[wave][j0 + j] : -1;  // uniform
-        vv[j] = r >= 0 ? reinterpret_cast<const uint32_t*>(p.vc + r)[lane] : 0u;
-      }
+    for (int j = 0; j < 64; ++j) {
+      const float v0 = __uint_as_float(vv[j] << 16), v1 = __uint_as_float(vv[j] & 0xffff0000u);
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        if (j0 + j < nkeys) {
-          const float v0 = __uint_as_float(vv[j] << 16), v1 = __uint_as_float(vv[j] & 0xffff0000u);
-#pragma unroll
-          for (int g = 0; g < G; ++g) {
-            const float pj = p_s[wave][j0 + j][g];
-            acc0[g] = __builtin_fmaf(pj, v0, acc0[g]);
-            acc1[g] = __builtin_fmaf(pj, v1, acc1[g]);
-          }
-        }
+      for (int g = 0; g < G; ++g) {
+        const float pj = p_s[wave][j][g];
+        acc0[g] = __builtin_fmaf(pj, v0, acc0[g]);
+        acc1[g] = __builtin_fmaf(pj, v1, acc1[g]);
       }
     }
     asm volatile("" ::: "memory");
@@ -228,20 +228,22 @@ __global__ __launch_bounds__(ATT_THREADS) void paged_attn_decode_kernel(AttnArgs
 
 }  // namespace aq
 
-extern "C" int aq_rope_kv_write(const void* qkv, const float* freqs, const int64_t* page_table, int64_t P,
+extern "C" int aq_rope_kv_write(const void* qkv, const float* freqs, int64_t freqs_stride, const int64_t* page_table, int64_t P,
                                 int64_t pos, int64_t page_size, void* k_cache, void* v_cache, int64_t n_pages,
                                 void* q_out, int64_t B, int64_t Hq, int64_t Hkv, int64_t D, void* stream) {
   if (D != aq::AD) return AQ_E_SHAPE;
   if (B < 0 || Hq <= 0 || Hkv <= 0 || P <= 0 || pos < 0 || page_size <= 0 || n_pages <= 0) return AQ_E_SHAPE;
+  if (freqs_stride != 0 && freqs_stride < D) return AQ_E_SHAPE;
   if (B == 0) return AQ_OK;
   if (!qkv || !freqs || !page_table || !k_cache || !v_cache || !q_out) return AQ_E_NULL;
   if (aq::check_ptr16(qkv) || aq::check_ptr16(k_cache) || aq::check_ptr16(v_cache) || aq::check_ptr16(q_out) ||
-      (reinterpret_cast<uintptr_t>(freqs) & 7u))
+      (reinterpret_cast<uintptr_t>(freqs) & 7u) || (freqs_stride & 1))
     return AQ_E_ALIGN;
   if (B * (Hq + 2 * Hkv) > (int64_t)0x7fffffff) return AQ_E_RANGE;
   aq::RopeArgs a{};
   a.qkv = static_cast<const uint16_t*>(qkv);
   a.freqs = freqs;
+  a.freqs_stride = freqs_stride;
   a.table = page_table;
   a.kc = static_cast<uint16_t*>(k_cache);
   a.vc = static_cast<uint16_t*>(v_cache);
@@ -285,13 +287,15 @@ extern "C" int aq_paged_attn_decode(const void* q, const void* k_cache, const vo
   a.B = (int)B;
   a.Hq = (int)Hq;
   a.Hkv = (int)Hkv;
-  const dim3 grid((unsigned)(B * Hkv)), block(aq::ATT_THREADS);
+  // 8 wavefronts per (sequence, KV head): 256 registers each, enough to hold a batch's K and V
+  // loads in flight together
+  const dim3 grid((unsigned)(B * Hkv)), block(512);
   hipStream_t st = static_cast<hipStream_t>(stream);
   switch (Hq / Hkv) {
-    case 1: hipLaunchKernelGGL((aq::paged_attn_decode_kernel<1>), grid, block, 0, st, a); break;
-    case 2: hipLaunchKernelGGL((aq::paged_attn_decode_kernel<2>), grid, block, 0, st, a); break;
-    case 4: hipLaunchKernelGGL((aq::paged_attn_decode_kernel<4>), grid, block, 0, st, a); break;
-    case 8: hipLaunchKernelGGL((aq::paged_attn_decode_kernel<8>), grid, block, 0, st, a); break;
+    case 1: hipLaunchKernelGGL((aq::paged_attn_decode_kernel<1, 8>), grid, block, 0, st, a); break;
+    case 2: hipLaunchKernelGGL((aq::paged_attn_decode_kernel<2, 8>), grid, block, 0, st, a); break;
+    case 4: hipLaunchKernelGGL((aq::paged_attn_decode_kernel<4, 8>), grid, block, 0, st, a); break;
+    case 8: hipLaunchKernelGGL((aq::paged_attn_decode_kernel<8, 8>), grid, block, 0, st, a); break;
     default: return AQ_E_SHAPE;  // query heads per KV head: 1, 2, 4 or 8
   }
   return (int)hipGetLastError();

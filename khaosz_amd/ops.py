@@ -269,7 +269,13 @@ def rope_kv_write(qkv: torch.Tensor, freqs: torch.Tensor, page_table: torch.Tens
     if not (k_cache.is_contiguous() and v_cache.is_contiguous()):
         raise ValueError("caches must be contiguous")
     fr = torch.view_as_real(freqs) if freqs.is_complex() else freqs
-    fr = fr.reshape(B, D // 2, 2).to(torch.float32).contiguous()
+    if fr.dtype != torch.float32 or fr.shape[0] != B or fr.numel() // max(B, 1) != D or fr.stride(-1) != 1:
+        raise ValueError(f"freqs must be complex64 [B, {D // 2}] or float32 [B, {D // 2}, 2]")
+    if B > 1 and fr.stride(0) == 0:      # one table broadcast to every sequence: no copy
+        fr_stride, fr = 0, fr[0].contiguous()
+    else:
+        fr = fr.reshape(B, D).contiguous()
+        fr_stride = D
     if page_table.dtype != torch.int64 or page_table.dim() != 2 or page_table.shape[0] != B:
         raise ValueError("page_table must be int64 [B, P]")
     page_table = page_table.contiguous()
@@ -277,7 +283,8 @@ def rope_kv_write(qkv: torch.Tensor, freqs: torch.Tensor, page_table: torch.Tens
     q = torch.empty((B, n_heads, D), dtype=torch.bfloat16, device=qkv.device)
     if B:
         with torch.cuda.device(qkv.device):
-            rc = _abi.load().aq_rope_kv_write(qkv.data_ptr(), fr.data_ptr(), page_table.data_ptr(), page_table.shape[1],
+            rc = _abi.load().aq_rope_kv_write(qkv.data_ptr(), fr.data_ptr(), fr_stride, page_table.data_ptr(),
+                                              page_table.shape[1],
                                               int(pos), k_cache.shape[1], k_cache.data_ptr(), v_cache.data_ptr(),
                                               k_cache.shape[0], q.data_ptr(), B, n_heads, n_kv_heads, D, _stream(qkv))
         _abi.check(rc, "aq_rope_kv_write")

@@ -287,6 +287,11 @@ def bench_block(torch, ops, args, dev):
     # and the single-token steps through the in-place paged attention kernels
     fuse_shared_inputs(blk, norms=True, decode_attention=True)
     prefill()
+    ms_dec_att = graph_time_ms(torch, decode_all, 3, 2) / steps
+    # and the two residual adds inside the epilogues of o_proj and down (bit-identical)
+    fuse_shared_inputs(blk, norms=True, decode_attention=True, residuals=True)
+    ms_pre_norms, ms_pre = ms_pre, graph_time_ms(torch, prefill, 10, 3)
+    prefill()
     ms_dec = graph_time_ms(torch, decode_all, 3, 2) / steps
 
     # The Linears alone (q/k/v and up/gate fused), at the shapes and in the order the block calls them (same modules,
@@ -312,7 +317,8 @@ def bench_block(torch, ops, args, dev):
         "value": ms_pre + steps * ms_dec, "unit": "ms", "prefill_ms": ms_pre, "decode_ms_per_step": ms_dec,
         "separate_projections": {"prefill_ms": ms_pre_sep, "decode_ms_per_step": ms_dec_sep},
         "fused_projections_separate_norms": {"prefill_ms": ms_pre_proj, "decode_ms_per_step": ms_dec_proj},
-        "fused_norms_torch_attention": {"prefill_ms": ms_pre, "decode_ms_per_step": ms_dec_norms},
+        "fused_norms_torch_attention": {"prefill_ms": ms_pre_norms, "decode_ms_per_step": ms_dec_norms},
+        "paged_decode_attention_separate_adds": {"prefill_ms": ms_pre_norms, "decode_ms_per_step": ms_dec_att},
         "linears_prefill_ms": ms_lin_pre, "linears_prefill_tops": lin_ops / (ms_lin_pre * 1e-3) / 1e12,
         "linears_decode_ms_per_step": ms_lin_dec, "linears_decode_gbs": lin_bytes / (ms_lin_dec * 1e-3) / 1e9,
         "non_linear_prefill_ms": ms_pre - ms_lin_pre, "non_linear_decode_ms_per_step": ms_dec - ms_lin_dec,
@@ -485,12 +491,15 @@ def main():
                                                             extra["prefill"]["ops_per_step"])
     for r in [main_res, *extra.values()]:
         r.pop("shape", None)
+    top = ("workload", "value", "unit", "ms_per_step", "dtype", "roofline", "eager_ms_per_step")
+    detail = {k: v for k, v in main_res.items() if k not in top} if args.workload == "block" else None
     line = {
         "metric": METRIC, "value": main_res["value"], "unit": main_res["unit"], "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": main_res["ms_per_step"],
         "higher_is_better": main_res["unit"] != "ms", "scaling": "weak", "vs_baseline": None, "dtype": main_res["dtype"],
         "data": "synthetic", "config": {"workload": main_res["workload"], "timing": "HIP graph replay of the timed steps",
-                                        "eager_ms_per_step": main_res.get("eager_ms_per_step")},
+                                        "eager_ms_per_step": main_res.get("eager_ms_per_step"),
+                                        **({"detail": detail} if detail else {})},
         "roofline": main_res["roofline"], "cpu_baseline": cpu, "measured_ceilings": ceilings,
         "also": {k: {kk: vv for kk, vv in v.items()} for k, v in extra.items()},
     }

@@ -96,6 +96,25 @@ int aq_gemv_w8a8_codes(const int8_t *xq, const float *sx, const int8_t *wq, cons
                        const void *bias, int bias_dtype, void *y, int y_dtype, int64_t M,
                        int64_t N, int64_t K, void *stream);
 
+/* The three entry points above with the residual connection around the Linear
+ * fused into the epilogue: y = round(linear) + residual, rounded to y_dtype
+ * again -- the bits of the reference's separate elementwise add
+ * (`attn_output + x`, `self.mlp(...) + x`, astrai/model/components/
+ * decoder_block.py:56-57), without the extra pass over [M, N].
+ * residual: [M, N] contiguous in y_dtype, or NULL (then identical to the entry
+ * points above).  It may be y itself: every element is read by the lane that
+ * writes it. */
+int aq_linear_w8a8_residual(const int8_t *xq, const float *sx, const int8_t *wq, const float *sw,
+                            const void *bias, int bias_dtype, const void *residual, void *y,
+                            int y_dtype, int64_t M, int64_t N, int64_t K, void *stream);
+int aq_gemv_w8a8_decode_residual(const void *x, int x_dtype, const int8_t *wq, const float *sw,
+                                 const void *bias, int bias_dtype, const void *residual, void *y,
+                                 int y_dtype, int64_t M, int64_t N, int64_t K, void *ws,
+                                 size_t ws_bytes, void *stream);
+int aq_gemv_w8a8_codes_residual(const int8_t *xq, const float *sx, const int8_t *wq, const float *sw,
+                                const void *bias, int bias_dtype, const void *residual, void *y,
+                                int y_dtype, int64_t M, int64_t N, int64_t K, void *stream);
+
 /* FP8 Linear: y[m, n] = (sum_k f(xq[m,k]) * f(wq[n,k])) * sx[0] * sw[0] with
  * fp32 accumulation, cast to y_dtype.  xq: [M, K], wq: [N, K] e4m3fn codes;
  * sx, sw: device scalars written by aq_quant_tensor_fp8.  Replaces F.linear
@@ -152,7 +171,15 @@ int aq_swiglu_quant_rowwise_i8(const void *ug, int dtype, int64_t M, int64_t F, 
  * mask.  Query heads h*G .. h*G+G-1 use KV head h, G = Hq / Hkv in {1, 2, 4, 8}.
  * Positions whose page is unmapped count as zero keys and values (what gather's
  * zero fill gives).  fp32 scores and sums; results within bf16 rounding of the
- * reference flow, not bit-identical to it (summation order, exp2). */
+ * reference flow, not bit-identical to it (summation order, exp2).
+ * The positions of a sequence are cut into slices that run as separate
+ * workgroups; with more than one slice their partial results pass through
+ * `workspace` (16-byte aligned device memory of at least
+ * aq_paged_attn_decode_workspace_bytes(B, Hq, Hkv, total_len) bytes, which is 0
+ * when one slice suffices -- then workspace may be NULL) and a second, small
+ * kernel combines them.  A workspace that is too small is AQ_E_WORKSPACE.  The size
+ * grows with total_len: a caller that sizes it once uses the longest sequence
+ * it will serve. */
 int aq_rope_kv_write(const void *qkv, const float *freqs, int64_t freqs_stride,
                      const int64_t *page_table, int64_t P,
                      int64_t pos, int64_t page_size, void *k_cache, void *v_cache, int64_t n_pages,
@@ -160,7 +187,8 @@ int aq_rope_kv_write(const void *qkv, const float *freqs, int64_t freqs_stride,
 int aq_paged_attn_decode(const void *q, const void *k_cache, const void *v_cache,
                          const int64_t *page_table, int64_t P, int64_t total_len, int64_t page_size,
                          int64_t n_pages, float scale, void *out, int64_t B, int64_t Hq, int64_t Hkv,
-                         int64_t D, void *stream);
+                         int64_t D, void *workspace, int64_t workspace_bytes, void *stream);
+int64_t aq_paged_attn_decode_workspace_bytes(int64_t B, int64_t Hq, int64_t Hkv, int64_t total_len);
 
 /* Tuning and test hook, no counterpart in the reference: the GEMM entry points
  * pick their workgroup tile (256 x 128, or 128 x 128 with a split K step when

@@ -22,12 +22,18 @@ SYMBOLS = {
     "aq_quant_tensor_fp8": (_int, [_vp, _int, _i64, _vp, _vp, _vp, _vp]),
     "aq_gemm_i8_i32": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "aq_linear_w8a8": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _vp, _int, _i64, _i64, _i64, _vp]),
+    "aq_linear_w8a8_residual": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _vp, _vp, _int, _i64, _i64, _i64, _vp]),
     "aq_gemv_w8a8_workspace_bytes": (_sz, [_i64, _i64]),
     "aq_gemv_w8a8_decode": (_int, [_vp, _int, _vp, _vp, _vp, _int, _vp, _int, _i64, _i64, _i64, _vp, _sz, _vp]),
     "aq_gemv_w8a8_codes": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _vp, _int, _i64, _i64, _i64, _vp]),
+    "aq_gemv_w8a8_decode_residual": (_int, [_vp, _int, _vp, _vp, _vp, _int, _vp, _vp, _int, _i64, _i64, _i64, _vp, _sz,
+                                            _vp]),
+    "aq_gemv_w8a8_codes_residual": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _vp, _vp, _int, _i64, _i64, _i64, _vp]),
     "aq_linear_fp8": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _vp]),
     "aq_rope_kv_write": (_int, [_vp, _vp, _i64, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _vp, _i64, _i64, _i64, _i64, _vp]),
-    "aq_paged_attn_decode": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, ctypes.c_float, _vp, _i64, _i64, _i64, _i64, _vp]),
+    "aq_paged_attn_decode": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, ctypes.c_float, _vp, _i64, _i64, _i64, _i64,
+                                    _vp, _i64, _vp]),
+    "aq_paged_attn_decode_workspace_bytes": (_i64, [_i64, _i64, _i64, _i64]),
     "aq_probe_mfma": (_int, [_int, _int, _int, _vp, _vp]),
     "aq_probe_copy": (_int, [_vp, _vp, _i64, _int, _vp]),
     "aq_probe_read": (_int, [_vp, _i64, _int, _vp, _vp]),

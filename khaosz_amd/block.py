@@ -178,10 +178,20 @@ class GQA(nn.Module):
             self._decode_attention = True
         return self._decode_attention
 
+    def _out(self, out: Tensor, residual: Optional[Tensor]) -> Tensor:
+        """o_proj, plus the residual stream when the caller hands it over."""
+        if residual is None:
+            return self.o_proj(out)
+        if isinstance(self.o_proj, QuantLinear):
+            return self.o_proj(out, residual=residual)
+        return self.o_proj(out) + residual
+
     def forward(self, x: Tensor, rotary_emb: Tensor, attn_mask: Optional[Tensor] = None,
-                cache=None, codes: Optional[Tuple[Tensor, Tensor]] = None) -> Tensor:
+                cache=None, codes: Optional[Tuple[Tensor, Tensor]] = None,
+                residual: Optional[Tensor] = None) -> Tensor:
         """``codes``: the already normalised and quantised input ``(xq [B*S, dim], sx [B*S])`` from a
-        fused norm; ``x`` then only gives the shape and dtype."""
+        fused norm; ``x`` then only gives the shape and dtype.  ``residual``: added to the output
+        (in o_proj's epilogue when it is quantized)."""
         B, S, _ = x.shape
         if (self._decode_attention and S == 1 and isinstance(cache, PagedKV) and x.is_cuda
                 and x.dtype == torch.bfloat16):
@@ -189,7 +199,7 @@ class GQA(nn.Module):
             q = ops.rope_kv_write(qkv.view(B, -1), rotary_emb.reshape(B, -1), cache.page_table, cache.total_len - 1,
                                   cache.k, cache.v, self.n_heads, self.n_kv_heads)
             out = ops.paged_attn_decode(q, cache.k, cache.v, cache.page_table, cache.total_len)
-            return self.o_proj(out.view(B, 1, -1))
+            return self._out(out.view(B, 1, -1), residual)
         if self._qkv is not None:
             nq, nkv = self.n_heads * self.head_dim, self.n_kv_heads * self.head_dim
             qkv = self._qkv(x) if codes is None else self._qkv.forward_codes(codes[0], codes[1], x.dtype).view(B, S, -1)
@@ -209,7 +219,7 @@ class GQA(nn.Module):
             v = v.repeat_interleave(rep, dim=2)
         out = F.scaled_dot_product_attention(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), attn_mask,
                                              is_causal=attn_mask is None)
-        return self.o_proj(out.transpose(1, 2).reshape(B, S, -1))
+        return self._out(out.transpose(1, 2).reshape(B, S, -1), residual)
 
 
 class MLP(nn.Module):
@@ -230,7 +240,11 @@ class MLP(nn.Module):
             return True
         return False
 
-    def forward(self, x: Tensor, codes: Optional[Tuple[Tensor, Tensor]] = None) -> Tensor:
+    def forward(self, x: Tensor, codes: Optional[Tuple[Tensor, Tensor]] = None,
+                residual: Optional[Tensor] = None) -> Tensor:
+        if residual is not None and not isinstance(self.down, QuantLinear):
+            return self.forward(x, codes) + residual
+        kw = {} if residual is None else {"residual": residual}
         if self._upgate is not None:
             ug = self._upgate(x) if codes is None else self._upgate.forward_codes(codes[0], codes[1], x.dtype).view(
                 *x.shape[:-1], -1)
@@ -238,10 +252,10 @@ class MLP(nn.Module):
                     and ug.shape[-1] // 2 <= ops.SWIGLU_QUANT_MAX_F.get(ug.dtype, 0)):
                 # activation, product and the down projection's quantisation in one launch
                 hq, hs = ops.swiglu_quant_rowwise_i8(ug)
-                return self.down.forward_codes(hq, hs, x.dtype).view(*x.shape[:-1], -1)
+                return self.down.forward_codes(hq, hs, x.dtype, **kw).view(*x.shape[:-1], -1)
             up, gate = ug.chunk(2, dim=-1)
-            return self.down(up * F.silu(gate))
-        return self.down(self.up(x) * F.silu(self.gate(x)))
+            return self.down(up * F.silu(gate), **kw)
+        return self.down(self.up(x) * F.silu(self.gate(x)), **kw)
 
 
 class DecoderBlock(nn.Module):
@@ -255,6 +269,7 @@ class DecoderBlock(nn.Module):
         self.post_attention_norm = RMSNorm(dim, norm_eps)
         self.mlp = MLP(dim, dim_ffn)
         self._norm_quant = False
+        self._residual_adds = False
 
     def reset_parameters(self) -> None:
         for m in self.modules():
@@ -271,16 +286,28 @@ class DecoderBlock(nn.Module):
             self.mlp._swiglu_quant = True  # likewise: silu * up and the quantisation for `down` in one launch
         return self._norm_quant
 
+    def fuse_residual_adds(self) -> bool:
+        """Hand the residual stream to o_proj and down, which add it in their epilogue when they
+        are quantized (bit-identical to the separate add, one pass over the activations less)."""
+        self._residual_adds = True
+        return True
+
     def forward(self, x: Tensor, rotary_emb: Tensor, attention_mask: Optional[Tensor] = None,
                 cache=None) -> Tensor:
+        if self._residual_adds:  # each branch's last projection adds the stream it is given
+            kw = lambda r: {"residual": r}
+            add = lambda y, r: y
+        else:
+            kw = lambda r: {}
+            add = lambda y, r: y + r
         if (self._norm_quant and x.is_cuda and x.dtype == self.input_norm.weight.dtype
                 and x.shape[-1] <= ops.RMSNORM_QUANT_MAX_K.get(x.dtype, 0)):
             n1, n2 = self.input_norm, self.post_attention_norm
-            x = self.attention(x, rotary_emb, attention_mask, cache,
-                               codes=ops.rmsnorm_quant_rowwise_i8(x, n1.weight, n1.norm_eps)) + x
-            return self.mlp(x, codes=ops.rmsnorm_quant_rowwise_i8(x, n2.weight, n2.norm_eps)) + x
-        x = self.attention(self.input_norm(x), rotary_emb, attention_mask, cache) + x
-        return self.mlp(self.post_attention_norm(x)) + x
+            x = add(self.attention(x, rotary_emb, attention_mask, cache,
+                                   codes=ops.rmsnorm_quant_rowwise_i8(x, n1.weight, n1.norm_eps), **kw(x)), x)
+            return add(self.mlp(x, codes=ops.rmsnorm_quant_rowwise_i8(x, n2.weight, n2.norm_eps), **kw(x)), x)
+        x = add(self.attention(self.input_norm(x), rotary_emb, attention_mask, cache, **kw(x)), x)
+        return add(self.mlp(self.post_attention_norm(x), **kw(x)), x)
 
 
 def decode_mask(batch: int, total_len: int, device, dtype) -> Tensor:

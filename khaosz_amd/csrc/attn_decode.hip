@@ -68,136 +68,162 @@ struct AttnArgs {
   const uint16_t* vc;
   const int64_t* table;  // [B, P]
   uint16_t* out;         // [B, Hq, D]
+  float* ws;             // partial results [B, Hq, NS, ATT_PART] when NS > 1
   int64_t P, T, page, n_pages;
   float scale_log2e;     // softmax scale times log2(e): scores live in the exp2 domain
-  int B, Hq, Hkv;
+  int B, Hq, Hkv, NS;
 };
 
-// Workgroup = one (sequence, KV head): its G query heads share every K and V
-// byte.  The T cached positions are cut into batches of 64; wavefront w takes
-// batches w, w + ATT_WAVES, ...  In a batch lane l owns key position t0 + l for
-// the scores (its 256-byte K row against the G queries held in LDS) and the
-// dimension pair (2l, 2l+1) for the weighted sum of V rows.  All of a batch's
-// loads -- 16 per lane for K, 64 for V -- are requested before anything is
-// computed: with a few dozen workgroups on the device the kernel lives on memory
-// latency, not bandwidth.  Each wavefront keeps a running maximum, denominator
-// and numerator per head (online softmax); the partial results are merged
-// through LDS at the end.
-template <int G, int ATT_WAVES>
+constexpr int ATT_WAVES = 4;
+constexpr int ATT_NL = 16;                   // row loads per wavefront, 4 rows each
+constexpr int ATT_KPW = 4 * ATT_NL;          // positions per wavefront
+constexpr int ATT_KPG = ATT_WAVES * ATT_KPW; // positions per workgroup
+constexpr int ATT_PART = AD + 4;  // numerator[AD], maximum, denominator, 2 floats of padding
+
+__device__ __forceinline__ float row16_sum(float v) {  // sum over each row of 16 lanes, result in all of them
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xf, 0xf, false));   // quad_perm [1,0,3,2]
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xf, 0xf, false));   // quad_perm [2,3,0,1]
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xf, 0xf, false));  // row_half_mirror
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xf, 0xf, false));  // row_mirror
+  return v;
+}
+
+__device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float c) {
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a), __builtin_bit_cast(bf16x2, b), c, false);
+}
+
+// Workgroup = one (sequence, KV head, slice of the cached positions): the G
+// query heads of the KV head share every K and V byte.  A wavefront owns 4*NL
+// consecutive positions, a workgroup 16*NL; the NS slices of a sequence run as
+// separate workgroups so that a decode batch of a few sequences still spreads
+// over the device.  Rows are read 16 bytes per lane: a load instruction covers
+// 4 whole 256-byte rows (lane = 16*key + chunk), NL of them for K and NL for V
+// are requested before anything is computed.
+//   scores   every lane dots its 8 dimensions with the G queries (packed bf16
+//            dot product, fp32 accumulation), a DPP butterfly sums the 16 lanes
+//            of a row, and lane (chunk = i, key = j) keeps the score of key
+//            4i + j of the batch -- one key per lane for the softmax;
+//   softmax  maximum and denominator across the wavefront, probabilities to LDS;
+//   values   lane accumulates p * V over the keys it loaded (8 dimensions x G
+//            heads), the four key groups are summed with two xor shuffles.
+// The wavefronts' (maximum, denominator, numerator) are merged through LDS and
+// either normalised into the output (NS == 1) or left in the workspace for
+// attn_merge_kernel.
+template <int G>
 __global__ __launch_bounds__(ATT_WAVES * 64) void paged_attn_decode_kernel(AttnArgs p) {
+  constexpr int NL = ATT_NL, KPW = ATT_KPW, KPG = ATT_KPG;
   constexpr int ATT_THREADS = ATT_WAVES * 64;
-  __shared__ float q_s[G][AD];                       // queries, pre-scaled
-  __shared__ float p_s[ATT_WAVES][64][G];            // a batch's probabilities, per wavefront
+  __shared__ __align__(16) float p_s[ATT_WAVES][KPW][G];
   __shared__ float m_s[ATT_WAVES][G], l_s[ATT_WAVES][G];
-  __shared__ float acc_s[ATT_WAVES][G][AD];
+  __shared__ __align__(16) float acc_s[ATT_WAVES][G][AD];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int b = blockIdx.x / p.Hkv, kvh = blockIdx.x % p.Hkv;
+  const int sub = lane >> 4, ch = lane & 15;  // key within a load, 16-byte chunk of the row
+  // the KV heads of one slice are neighbours in the launch order: together they read whole
+  // [position][Hkv][D] stretches of the pages at about the same time
+  const int kvh = blockIdx.x % p.Hkv, bs = blockIdx.x / p.Hkv;
+  const int split = bs % p.NS, b = bs / p.NS;
+  const int64_t T = p.T;
+  const int64_t t0 = (int64_t)split * KPG + wave * KPW;  // first position of this wavefront
 
-  for (int i = tid; i < G * AD; i += ATT_THREADS) {
-    const int g = i / AD, d = i % AD;
-    q_s[g][d] = __fmul_rn(bf16_bits_to_f32(p.q[((int64_t)b * p.Hq + kvh * G + g) * AD + d]), p.scale_log2e);
-  }
-  __syncthreads();
-
-  float m[G], l[G], acc0[G], acc1[G];
+  float m[G], l[G], acc[G][8];
 #pragma unroll
   for (int g = 0; g < G; ++g) {
     m[g] = -INFINITY;
     l[g] = 0.0f;
-    acc0[g] = 0.0f;
-    acc1[g] = 0.0f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[g][e] = 0.0f;
   }
-  const int64_t T = p.T;
-  for (int64_t t0 = (int64_t)wave * 64; t0 < T; t0 += ATT_WAVES * 64) {
-    // ---- scores of key t0 + lane
-    const int64_t t = t0 + lane;
-    int64_t row = -1;  // element offset of this key's row, or -1
-    if (t < T) {
-      const int64_t lp = t / p.page;
-      const int64_t phys = lp < p.P ? p.table[(int64_t)b * p.P + lp] : -1;
-      if (phys >= 0 && phys < p.n_pages) row = ((phys * p.page + t % p.page) * p.Hkv + kvh) * AD;
-    }
-    uint4 kv[AD / 8];
-    if (row >= 0) {
-      const uint4* src = reinterpret_cast<const uint4*>(p.kc + row);
-#pragma unroll
-      for (int c = 0; c < AD / 8; ++c) kv[c] = src[c];
-    } else {
-#pragma unroll
-      for (int c = 0; c < AD / 8; ++c) kv[c] = make_uint4(0, 0, 0, 0);
-    }
-    // the V rows of the whole batch: the row offset of key j sits in lane j
-    const int nkeys = (T - t0) < 64 ? (int)(T - t0) : 64;
-    uint32_t vv[64];
-#pragma unroll
-    for (int j = 0; j < 64; ++j) {
-      const int lo = __builtin_amdgcn_readlane((int)(uint32_t)row, j), hi = __builtin_amdgcn_readlane((int)(row >> 32), j);
-      const int64_t r = ((int64_t)hi << 32) | (uint32_t)lo;  // wavefront-uniform
-      vv[j] = (j < nkeys && r >= 0) ? reinterpret_cast<const uint32_t*>(p.vc + r)[lane] : 0u;
-    }
-    float s[G];
-#pragma unroll
-    for (int g = 0; g < G; ++g) s[g] = 0.0f;
-#pragma unroll
-    for (int c = 0; c < AD / 8; ++c) {
-      float k8[8];
-      k8[0] = __uint_as_float(kv[c].x << 16);
-      k8[1] = __uint_as_float(kv[c].x & 0xffff0000u);
-      k8[2] = __uint_as_float(kv[c].y << 16);
-      k8[3] = __uint_as_float(kv[c].y & 0xffff0000u);
-      k8[4] = __uint_as_float(kv[c].z << 16);
-      k8[5] = __uint_as_float(kv[c].z & 0xffff0000u);
-      k8[6] = __uint_as_float(kv[c].w << 16);
-      k8[7] = __uint_as_float(kv[c].w & 0xffff0000u);
-#pragma unroll
-      for (int g = 0; g < G; ++g) {
-        const float4 qa = *reinterpret_cast<const float4*>(&q_s[g][c * 8]);
-        const float4 qb = *reinterpret_cast<const float4*>(&q_s[g][c * 8 + 4]);
-        s[g] = __builtin_fmaf(k8[0], qa.x, s[g]);
-        s[g] = __builtin_fmaf(k8[1], qa.y, s[g]);
-        s[g] = __builtin_fmaf(k8[2], qa.z, s[g]);
-        s[g] = __builtin_fmaf(k8[3], qa.w, s[g]);
-        s[g] = __builtin_fmaf(k8[4], qb.x, s[g]);
-        s[g] = __builtin_fmaf(k8[5], qb.y, s[g]);
-        s[g] = __builtin_fmaf(k8[6], qb.z, s[g]);
-        s[g] = __builtin_fmaf(k8[7], qb.w, s[g]);
+  if (t0 < T) {  // wavefront-uniform
+    // lane L < KPW looks up the row of position t0 + L (element offset, -1: unmapped or past T)
+    int64_t row = -1;
+    {
+      const int64_t t = t0 + lane;
+      if (lane < KPW && t < T) {
+        const int64_t lp = t / p.page;
+        const int64_t phys = lp < p.P ? p.table[(int64_t)b * p.P + lp] : -1;
+        if (phys >= 0 && phys < p.n_pages) row = ((phys * p.page + t % p.page) * p.Hkv + kvh) * AD;
       }
     }
-    // ---- online softmax update, per head
+    uint4 qv[G];  // this lane's 8 dimensions of each query
+#pragma unroll
+    for (int g = 0; g < G; ++g)
+      qv[g] = *reinterpret_cast<const uint4*>(p.q + ((int64_t)b * p.Hq + kvh * G + g) * AD + ch * 8);
+    uint4 kv[NL], vv[NL];
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+      const int src = i * 4 + sub;
+      const int lo = __shfl((int)(uint32_t)row, src, 64), hi = __shfl((int)(row >> 32), src, 64);
+      const int64_t r = ((int64_t)hi << 32) | (uint32_t)lo;
+      kv[i] = make_uint4(0, 0, 0, 0);
+      vv[i] = make_uint4(0, 0, 0, 0);
+      if (r >= 0) {
+        kv[i] = *reinterpret_cast<const uint4*>(p.kc + r + ch * 8);
+        vv[i] = *reinterpret_cast<const uint4*>(p.vc + r + ch * 8);
+      }
+    }
+    // ---- scores
+    float sc[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) sc[g] = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        float d = dot2_bf16(kv[i].x, qv[g].x, 0.0f);
+        d = dot2_bf16(kv[i].y, qv[g].y, d);
+        d = dot2_bf16(kv[i].z, qv[g].z, d);
+        d = dot2_bf16(kv[i].w, qv[g].w, d);
+        d = row16_sum(d);
+        if (ch == i) sc[g] = d;
+      }
+    }
+    // ---- softmax over the wavefront's positions: this lane owns position t0 + 4*ch + sub
+    const int own = ch * 4 + sub;
+    const bool valid = ch < NL && t0 + own < T;
 #pragma unroll
     for (int g = 0; g < G; ++g) {
-      const float sv = t < T ? s[g] : -INFINITY;
+      const float sv = valid ? sc[g] * p.scale_log2e : -INFINITY;
       float bm = sv;
 #pragma unroll
       for (int off = 32; off > 0; off >>= 1) bm = fmaxf(bm, __shfl_xor(bm, off, 64));
-      const float mn = fmaxf(m[g], bm);  // finite: lane 0 of every batch is a valid position
-      const float alpha = exp2f(m[g] - mn);
-      const float pv = t < T ? exp2f(sv - mn) : 0.0f;
+      const float pv = valid ? exp2f(sv - bm) : 0.0f;  // bm is finite: position t0 is valid
       float ps = pv;
 #pragma unroll
       for (int off = 32; off > 0; off >>= 1) ps += __shfl_xor(ps, off, 64);
-      l[g] = l[g] * alpha + ps;
-      acc0[g] *= alpha;
-      acc1[g] *= alpha;
-      m[g] = mn;
-      p_s[wave][lane][g] = pv;
+      m[g] = bm;
+      l[g] = ps;
+      if (ch < NL) p_s[wave][own][g] = pv;
     }
     __builtin_amdgcn_s_waitcnt(0xc07f);  // this wavefront's LDS writes are done (wavefront-private region)
     asm volatile("" ::: "memory");
-    // ---- numerator: lane owns dimensions 2l, 2l+1 of every V row of the batch (zero rows and
-    // positions past T carry probability-weighted zeros)
+    // ---- numerator (unmapped rows and positions past T contribute zeros)
 #pragma unroll
-    for (int j = 0; j < 64; ++j) {
-      const float v0 = __uint_as_float(vv[j] << 16), v1 = __uint_as_float(vv[j] & 0xffff0000u);
+    for (int i = 0; i < NL; ++i) {
+      float v8[8];
+      v8[0] = __uint_as_float(vv[i].x << 16);
+      v8[1] = __uint_as_float(vv[i].x & 0xffff0000u);
+      v8[2] = __uint_as_float(vv[i].y << 16);
+      v8[3] = __uint_as_float(vv[i].y & 0xffff0000u);
+      v8[4] = __uint_as_float(vv[i].z << 16);
+      v8[5] = __uint_as_float(vv[i].z & 0xffff0000u);
+      v8[6] = __uint_as_float(vv[i].w << 16);
+      v8[7] = __uint_as_float(vv[i].w & 0xffff0000u);
 #pragma unroll
       for (int g = 0; g < G; ++g) {
-        const float pj = p_s[wave][j][g];
-        acc0[g] = __builtin_fmaf(pj, v0, acc0[g]);
-        acc1[g] = __builtin_fmaf(pj, v1, acc1[g]);
+        const float pj = p_s[wave][i * 4 + sub][g];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[g][e] = __builtin_fmaf(pj, v8[e], acc[g][e]);
       }
     }
-    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int g = 0; g < G; ++g)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        acc[g][e] += __shfl_xor(acc[g][e], 16, 64);
+        acc[g][e] += __shfl_xor(acc[g][e], 32, 64);
+      }
   }
   // ---- merge the wavefronts' partial results
 #pragma unroll
@@ -206,25 +232,54 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void paged_attn_decode_kernel(AttnA
       m_s[wave][g] = m[g];
       l_s[wave][g] = l[g];
     }
-    acc_s[wave][g][2 * lane] = acc0[g];
-    acc_s[wave][g][2 * lane + 1] = acc1[g];
+    if (sub == 0) {
+      *reinterpret_cast<float4*>(&acc_s[wave][g][ch * 8]) = make_float4(acc[g][0], acc[g][1], acc[g][2], acc[g][3]);
+      *reinterpret_cast<float4*>(&acc_s[wave][g][ch * 8 + 4]) = make_float4(acc[g][4], acc[g][5], acc[g][6], acc[g][7]);
+    }
   }
   __syncthreads();
-  for (int i = tid; i < G * AD; i += ATT_THREADS) {
-    const int g = i / AD, d = i % AD;
+  for (int i = tid; i < G * AD / 2; i += ATT_THREADS) {
+    const int g = i / (AD / 2), d = (i % (AD / 2)) * 2;  // dimensions d, d + 1
     float mm = -INFINITY;
 #pragma unroll
     for (int w = 0; w < ATT_WAVES; ++w) mm = fmaxf(mm, m_s[w][g]);
-    float num = 0.0f, den = 0.0f;
+    float n0 = 0.0f, n1 = 0.0f, den = 0.0f;
 #pragma unroll
     for (int w = 0; w < ATT_WAVES; ++w) {
-      const float a = m_s[w][g] == -INFINITY ? 0.0f : exp2f(m_s[w][g] - mm);  // wavefronts without a batch
-      num = __builtin_fmaf(acc_s[w][g][d], a, num);
+      const float a = m_s[w][g] == -INFINITY ? 0.0f : exp2f(m_s[w][g] - mm);  // wavefronts past T
+      n0 = __builtin_fmaf(acc_s[w][g][d], a, n0);
+      n1 = __builtin_fmaf(acc_s[w][g][d + 1], a, n1);
       den = __builtin_fmaf(l_s[w][g], a, den);
     }
-    p.out[((int64_t)b * p.Hq + kvh * G + g) * AD + d] = (uint16_t)f32_to_bf16_bits(num / den);
+    const int64_t head = (int64_t)b * p.Hq + kvh * G + g;
+    if (p.NS == 1) {
+      store_wt(reinterpret_cast<uint32_t*>(p.out + head * AD + d), pack_bf16x2(n0 / den, n1 / den));
+    } else {
+      float* part = p.ws + (head * p.NS + split) * ATT_PART;
+      store_wt(reinterpret_cast<uint2*>(part + d), make_uint2(__float_as_uint(n0), __float_as_uint(n1)));
+      if (d == 0) store_wt(reinterpret_cast<uint2*>(part + AD), make_uint2(__float_as_uint(mm), __float_as_uint(den)));
+    }
   }
 }
+
+// Combines the NS slices of one (sequence, query head): thread = dimension pair.
+__global__ __launch_bounds__(AD / 2) void attn_merge_kernel(const float* ws, uint16_t* out, int NS) {
+  const int d = threadIdx.x * 2;
+  const float* part = ws + (int64_t)blockIdx.x * NS * ATT_PART;
+  float mm = -INFINITY;
+  for (int s = 0; s < NS; ++s) mm = fmaxf(mm, part[s * ATT_PART + AD]);  // slice 0 always holds a position
+  float n0 = 0.0f, n1 = 0.0f, den = 0.0f;
+  for (int s = 0; s < NS; ++s) {
+    const float a = exp2f(part[s * ATT_PART + AD] - mm);
+    const float2 v = *reinterpret_cast<const float2*>(part + s * ATT_PART + d);
+    n0 = __builtin_fmaf(v.x, a, n0);
+    n1 = __builtin_fmaf(v.y, a, n1);
+    den = __builtin_fmaf(part[s * ATT_PART + AD + 1], a, den);
+  }
+  store_wt(reinterpret_cast<uint32_t*>(out + (int64_t)blockIdx.x * AD + d), pack_bf16x2(n0 / den, n1 / den));
+}
+
+inline int64_t attn_slices(int64_t T) { return (T + ATT_KPG - 1) / ATT_KPG; }
 
 }  // namespace aq
 
@@ -260,10 +315,16 @@ extern "C" int aq_rope_kv_write(const void* qkv, const float* freqs, int64_t fre
   return (int)hipGetLastError();
 }
 
+extern "C" int64_t aq_paged_attn_decode_workspace_bytes(int64_t B, int64_t Hq, int64_t Hkv, int64_t total_len) {
+  if (B <= 0 || Hq <= 0 || Hkv <= 0 || total_len <= 0) return 0;
+  const int64_t ns = aq::attn_slices(total_len);
+  return ns == 1 ? 0 : B * Hq * ns * aq::ATT_PART * (int64_t)sizeof(float);
+}
+
 extern "C" int aq_paged_attn_decode(const void* q, const void* k_cache, const void* v_cache,
                                     const int64_t* page_table, int64_t P, int64_t total_len, int64_t page_size,
                                     int64_t n_pages, float scale, void* out, int64_t B, int64_t Hq, int64_t Hkv,
-                                    int64_t D, void* stream) {
+                                    int64_t D, void* workspace, int64_t workspace_bytes, void* stream) {
   if (D != aq::AD) return AQ_E_SHAPE;
   if (B < 0 || Hq <= 0 || Hkv <= 0 || (Hq % Hkv) != 0 || P <= 0 || total_len <= 0 || page_size <= 0 ||
       n_pages <= 0 || !(scale > 0.0f))
@@ -272,13 +333,20 @@ extern "C" int aq_paged_attn_decode(const void* q, const void* k_cache, const vo
   if (!q || !k_cache || !v_cache || !page_table || !out) return AQ_E_NULL;
   if (aq::check_ptr16(q) || aq::check_ptr16(k_cache) || aq::check_ptr16(v_cache) || aq::check_ptr16(out))
     return AQ_E_ALIGN;
-  if (B * Hkv > (int64_t)0x7fffffff) return AQ_E_RANGE;
+  const int64_t ns = aq::attn_slices(total_len);
+  if (B * Hkv * ns > (int64_t)0x7fffffff || B * Hq > (int64_t)0x7fffffff) return AQ_E_RANGE;
+  if (ns > 1) {
+    if (!workspace) return AQ_E_NULL;
+    if (aq::check_ptr16(workspace)) return AQ_E_ALIGN;
+    if (workspace_bytes < B * Hq * ns * aq::ATT_PART * (int64_t)sizeof(float)) return AQ_E_WORKSPACE;
+  }
   aq::AttnArgs a{};
   a.q = static_cast<const uint16_t*>(q);
   a.kc = static_cast<const uint16_t*>(k_cache);
   a.vc = static_cast<const uint16_t*>(v_cache);
   a.table = page_table;
   a.out = static_cast<uint16_t*>(out);
+  a.ws = static_cast<float*>(workspace);
   a.P = P;
   a.T = total_len;
   a.page = page_size;
@@ -287,16 +355,18 @@ extern "C" int aq_paged_attn_decode(const void* q, const void* k_cache, const vo
   a.B = (int)B;
   a.Hq = (int)Hq;
   a.Hkv = (int)Hkv;
-  // 8 wavefronts per (sequence, KV head): 256 registers each, enough to hold a batch's K and V
-  // loads in flight together
-  const dim3 grid((unsigned)(B * Hkv)), block(512);
+  a.NS = (int)ns;
+  const dim3 grid((unsigned)(B * Hkv * ns)), block(aq::ATT_WAVES * 64);
   hipStream_t st = static_cast<hipStream_t>(stream);
   switch (Hq / Hkv) {
-    case 1: hipLaunchKernelGGL((aq::paged_attn_decode_kernel<1, 8>), grid, block, 0, st, a); break;
-    case 2: hipLaunchKernelGGL((aq::paged_attn_decode_kernel<2, 8>), grid, block, 0, st, a); break;
-    case 4: hipLaunchKernelGGL((aq::paged_attn_decode_kernel<4, 8>), grid, block, 0, st, a); break;
-    case 8: hipLaunchKernelGGL((aq::paged_attn_decode_kernel<8, 8>), grid, block, 0, st, a); break;
+    case 1: hipLaunchKernelGGL(aq::paged_attn_decode_kernel<1>, grid, block, 0, st, a); break;
+    case 2: hipLaunchKernelGGL(aq::paged_attn_decode_kernel<2>, grid, block, 0, st, a); break;
+    case 4: hipLaunchKernelGGL(aq::paged_attn_decode_kernel<4>, grid, block, 0, st, a); break;
+    case 8: hipLaunchKernelGGL(aq::paged_attn_decode_kernel<8>, grid, block, 0, st, a); break;
     default: return AQ_E_SHAPE;  // query heads per KV head: 1, 2, 4 or 8
   }
+  int rc = (int)hipGetLastError();
+  if (rc != 0 || ns == 1) return rc;
+  hipLaunchKernelGGL(aq::attn_merge_kernel, dim3((unsigned)(B * Hq)), dim3(aq::AD / 2), 0, st, a.ws, a.out, a.NS);
   return (int)hipGetLastError();
 }

@@ -54,6 +54,7 @@ struct GemmArgs {
   const float* sw;   // int8: [N]; fp8: [1]
   const void* bias;  // [N] or null
   int bias_dtype;
+  const void* res;   // [M, N] residual in the output's type, or null; may be C itself
 };
 
 // Workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2.
@@ -476,6 +477,11 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(GemmArgs p) {
   const int nw = __builtin_amdgcn_readfirstlane(n0 + wave_n * WAVE_N);  // first column of this wavefront
   const __amdgpu_buffer_rsrc_t Cr =
       make_rsrc(reinterpret_cast<uint8_t*>(p.C) + ((int64_t)mw * N + nw) * ESZ, 0x40000000u);
+  // Residual: the same window over the tensor that is added to the rounded output; each lane
+  // reads exactly the elements it then writes, so the residual may be the output itself.
+  const bool has_res = OUT != OUT_I32 && p.res != nullptr;  // uniform
+  const __amdgpu_buffer_rsrc_t Rr = make_rsrc(
+      reinterpret_cast<const uint8_t*>(has_res ? p.res : p.C) + ((int64_t)mw * N + nw) * ESZ, has_res ? 0x40000000u : 0u);
   const bool pair_ok = (N & 1) == 0;  // uniform: bf16 rows start dword-aligned, pairs never straddle N
   const bool odd = lane & 1;
   const uint32_t perm_sel = odd ? 0x03020706u : 0x05040100u;
@@ -496,6 +502,28 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(GemmArgs p) {
       const uint32_t vbase =
           n_ok ? (uint32_t)rq * rowb + (uint32_t)(PAIR ? (cj & ~1) : cj) * ESZ + (PAIR && odd ? rowb : 0u)
                : OOB_OFFSET;
+      // the residual elements of this column, requested together ahead of the arithmetic
+      constexpr int RPG = PAIR ? 2 : 4;  // loads per 4-row group: packed row pairs, or single elements
+      uint32_t rr[TME][4][RPG];
+      if constexpr (OUT != OUT_I32) {
+        if (has_res) {
+#pragma unroll
+          for (int i = 0; i < TME; ++i)
+#pragma unroll
+            for (int g = 0; g < 4; ++g)
+#pragma unroll
+              for (int q = 0; q < RPG; ++q) {
+                const int r0 = i * 32 + g * 8;
+                const int rowq = PAIR ? 2 * q : q;
+                uint32_t vo = vbase;
+                if (CHECK_M && mw + r0 + rq + rowq + (PAIR && odd ? 1 : 0) >= M) vo = OOB_OFFSET;
+                if constexpr (OUT == OUT_F32 || PAIR)
+                  rr[i][g][q] = __builtin_amdgcn_raw_buffer_load_b32(Rr, vo, (r0 + rowq) * rowb, 0);
+                else
+                  rr[i][g][q] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(Rr, vo, (r0 + rowq) * rowb, 0);
+              }
+        }
+      }
 #pragma unroll
       for (int i = 0; i < TME; ++i) {
 #pragma unroll
@@ -526,6 +554,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(GemmArgs p) {
               for (int q = 0; q < 4; ++q) {
                 uint32_t vo = vbase;
                 if (CHECK_M && mw + r0 + rq + q >= M) vo = OOB_OFFSET;
+                if (has_res) y[q] = __fadd_rn(y[q], __uint_as_float(rr[i][g][q]));
                 __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(y[q]), Cr, vo, (r0 + q) * rowb, STORE_WT);
               }
             } else if constexpr (PAIR) {
@@ -536,7 +565,12 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(GemmArgs p) {
                     (uint32_t)__builtin_amdgcn_mov_dpp((int)mine, 0xB1 /* quad_perm [1,0,3,2] */, 0xf, 0xf, true);
                 // even lane: {mine.lo, other.lo} = row 2h, columns (c, c+1)
                 // odd lane:  {other.hi, mine.hi} = row 2h+1, columns (c-1, c)
-                const uint32_t pk = __builtin_amdgcn_perm(other, mine, perm_sel);
+                uint32_t pk = __builtin_amdgcn_perm(other, mine, perm_sel);
+                if (has_res) {  // rounded output + residual, rounded again: what a separate add gives
+                  const uint32_t r = rr[i][g][h];
+                  pk = pack_bf16x2(__fadd_rn(__uint_as_float(pk << 16), __uint_as_float(r << 16)),
+                                   __fadd_rn(__uint_as_float(pk & 0xffff0000u), __uint_as_float(r & 0xffff0000u)));
+                }
                 uint32_t vo = vbase;
                 if (CHECK_M && mw + r0 + rq + 2 * h + (odd ? 1 : 0) >= M) vo = OOB_OFFSET;
                 __builtin_amdgcn_raw_buffer_store_b32(pk, Cr, vo, (r0 + 2 * h) * rowb, STORE_WT);
@@ -546,7 +580,9 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(GemmArgs p) {
               for (int q = 0; q < 4; ++q) {
                 uint32_t vo = vbase;
                 if (CHECK_M && mw + r0 + rq + q >= M) vo = OOB_OFFSET;
-                __builtin_amdgcn_raw_buffer_store_b16((uint16_t)f32_to_bf16_bits(y[q]), Cr, vo, (r0 + q) * rowb, STORE_WT);
+                uint32_t ob = f32_to_bf16_bits(y[q]);
+                if (has_res) ob = f32_to_bf16_bits(__fadd_rn(__uint_as_float(ob << 16), __uint_as_float(rr[i][g][q] << 16)));
+                __builtin_amdgcn_raw_buffer_store_b16((uint16_t)ob, Cr, vo, (r0 + q) * rowb, STORE_WT);
               }
             }
           }
@@ -631,6 +667,12 @@ extern "C" int aq_gemm_i8_i32(const int8_t* xq, const int8_t* wq, int32_t* acc, 
 extern "C" int aq_linear_w8a8(const int8_t* xq, const float* sx, const int8_t* wq, const float* sw,
                               const void* bias, int bias_dtype, void* y, int y_dtype, int64_t M,
                               int64_t N, int64_t K, void* stream) {
+  return aq_linear_w8a8_residual(xq, sx, wq, sw, bias, bias_dtype, nullptr, y, y_dtype, M, N, K, stream);
+}
+
+extern "C" int aq_linear_w8a8_residual(const int8_t* xq, const float* sx, const int8_t* wq, const float* sw,
+                                       const void* bias, int bias_dtype, const void* residual, void* y, int y_dtype,
+                                       int64_t M, int64_t N, int64_t K, void* stream) {
   if (y_dtype != AQ_F32 && y_dtype != AQ_BF16) return AQ_E_DTYPE;
   if (bias && bias_dtype != AQ_F32 && bias_dtype != AQ_BF16) return AQ_E_DTYPE;
   int rc = aq::check_gemm(xq, wq, y, M, N, K);
@@ -641,6 +683,7 @@ extern "C" int aq_linear_w8a8(const int8_t* xq, const float* sx, const int8_t* w
   a.sw = sw;
   a.bias = bias;
   a.bias_dtype = bias_dtype;
+  a.res = residual;
   hipStream_t st = static_cast<hipStream_t>(stream);
   return y_dtype == AQ_BF16 ? aq::launch<false, aq::OUT_BF16>(a, st) : aq::launch<false, aq::OUT_F32>(a, st);
 }

@@ -79,10 +79,18 @@ struct GemvArgs {
   const int8_t* wq;   // [N, K]
   const float* sw;    // [N]
   const void* bias;   // [N] or null
+  const void* res;    // [M, N] residual in y's dtype (row stride ldr), or null; may be y itself
   void* y;            // [M, N]
+  int64_t ldr;
   int M, N, K;
   int bias_dtype, y_dtype;
 };
+
+// y (+ residual): the projection is rounded to the output type first and the
+// sum rounded again, the bits a separate elementwise add of the two tensors gives.
+__device__ __forceinline__ float add_residual_bf16(float y, uint32_t res_bits) {
+  return __fadd_rn(bf16_bits_to_f32((uint16_t)f32_to_bf16_bits(y)), bf16_bits_to_f32((uint16_t)res_bits));
+}
 
 #define GV_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(0x0f70 | ((n) & 15) | (((n) >> 4) << 14))
 
@@ -107,6 +115,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_w8a8_kernel(GemvArgs p) {
   const int om = oidx % MT, on = n0 + oidx / MT;
   const bool out_lane = (lane & ((1 << SH) - 1)) == 0 && om < M && on < N;
   float sxv = 0.0f, swv = 0.0f, bv = 0.0f;
+  uint32_t rv = 0;  // residual element, raw bits
   float* sx_lds = reinterpret_cast<float*>(xs + MT * K);
   if (out_lane) {
     if constexpr (!FUSED) sxv = p.sx[om];
@@ -114,6 +123,9 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_w8a8_kernel(GemvArgs p) {
     if (p.bias)
       bv = p.bias_dtype == AQ_BF16 ? bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(p.bias)[on])
                                    : reinterpret_cast<const float*>(p.bias)[on];
+    if (p.res)
+      rv = p.y_dtype == AQ_BF16 ? reinterpret_cast<const uint16_t*>(p.res)[om * p.ldr + on]
+                                : reinterpret_cast<const uint32_t*>(p.res)[om * p.ldr + on];
   }
 
   // 1. activation codes -> LDS.  Either copied, 16 bytes per lane, straight from
@@ -222,6 +234,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_w8a8_kernel(GemvArgs p) {
   if (!out_lane) return;
   float y = __fmul_rn(__fmul_rn((float)acc[0], sxv), swv);
   if (p.bias) y = __fadd_rn(y, bv);
+  if (p.res) y = p.y_dtype == AQ_BF16 ? add_residual_bf16(y, rv) : __fadd_rn(y, __uint_as_float(rv));
   const int64_t o = (int64_t)om * N + on;
   if (p.y_dtype == AQ_BF16)
     reinterpret_cast<uint16_t*>(p.y)[o] = (uint16_t)f32_to_bf16_bits(y);
@@ -290,10 +303,12 @@ __global__ __launch_bounds__(GM_WAVES * 64) void gemv_mfma_kernel(GemvArgs p) {
   const int tok = lane & 15;
   const int rbase = n0 + (lane >> 4) * 4;
   float sxv = 0.0f, swv[4], bv[4];
+  uint32_t rv[4];  // residual elements, raw bits
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
     swv[r] = 0.0f;
     bv[r] = 0.0f;
+    rv[r] = 0;
   }
   float* sx_lds = reinterpret_cast<float*>(xs + 16 * pitch);
   if (kh == 0) {  // uniform: only the first half's wavefront writes outputs
@@ -307,6 +322,9 @@ __global__ __launch_bounds__(GM_WAVES * 64) void gemv_mfma_kernel(GemvArgs p) {
       if (p.bias)
         bv[r] = p.bias_dtype == AQ_BF16 ? bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(p.bias)[n])
                                         : reinterpret_cast<const float*>(p.bias)[n];
+      if (p.res && tok < M)
+        rv[r] = p.y_dtype == AQ_BF16 ? reinterpret_cast<const uint16_t*>(p.res)[tok * p.ldr + n]
+                                     : reinterpret_cast<const uint32_t*>(p.res)[tok * p.ldr + n];
     }
   }
 
@@ -408,6 +426,7 @@ __global__ __launch_bounds__(GM_WAVES * 64) void gemv_mfma_kernel(GemvArgs p) {
   for (int r = 0; r < 4; ++r) {
     y[r] = __fmul_rn(__fmul_rn((float)acc[r], sxv), swv[r]);
     if (p.bias) y[r] = __fadd_rn(y[r], bv[r]);
+    if (p.res) y[r] = p.y_dtype == AQ_BF16 ? add_residual_bf16(y[r], rv[r]) : __fadd_rn(y[r], __uint_as_float(rv[r]));
   }
   const int64_t o = (int64_t)tok * N + rbase;
   if (p.y_dtype == AQ_BF16) {
@@ -504,9 +523,9 @@ static int gemv_dispatch_fused(const aq::GemvArgs& a, int mt, hipStream_t st) {
   }
 }
 
-extern "C" int aq_gemv_w8a8_codes(const int8_t* xq, const float* sx, const int8_t* wq, const float* sw,
-                                  const void* bias, int bias_dtype, void* y, int y_dtype, int64_t M,
-                                  int64_t N, int64_t K, void* stream) {
+extern "C" int aq_gemv_w8a8_codes_residual(const int8_t* xq, const float* sx, const int8_t* wq, const float* sw,
+                                           const void* bias, int bias_dtype, const void* residual,
+                                           void* y, int y_dtype, int64_t M, int64_t N, int64_t K, void* stream) {
   int mt = 0;
   int rc = gemv_check(wq, sw, bias, bias_dtype, y, y_dtype, M, N, K, &mt);
   if (rc || M == 0 || N == 0) return rc;
@@ -518,6 +537,8 @@ extern "C" int aq_gemv_w8a8_codes(const int8_t* xq, const float* sx, const int8_
   a.wq = wq;
   a.sw = sw;
   a.bias = bias;
+  a.res = residual;
+  a.ldr = N;
   a.y = y;
   a.M = (int)M;
   a.N = (int)N;
@@ -527,9 +548,16 @@ extern "C" int aq_gemv_w8a8_codes(const int8_t* xq, const float* sx, const int8_
   return gemv_dispatch(a, mt, static_cast<hipStream_t>(stream));
 }
 
-extern "C" int aq_gemv_w8a8_decode(const void* x, int x_dtype, const int8_t* wq, const float* sw,
-                                   const void* bias, int bias_dtype, void* y, int y_dtype, int64_t M,
-                                   int64_t N, int64_t K, void* ws, size_t ws_bytes, void* stream) {
+extern "C" int aq_gemv_w8a8_codes(const int8_t* xq, const float* sx, const int8_t* wq, const float* sw,
+                                  const void* bias, int bias_dtype, void* y, int y_dtype, int64_t M,
+                                  int64_t N, int64_t K, void* stream) {
+  return aq_gemv_w8a8_codes_residual(xq, sx, wq, sw, bias, bias_dtype, nullptr, y, y_dtype, M, N, K, stream);
+}
+
+extern "C" int aq_gemv_w8a8_decode_residual(const void* x, int x_dtype, const int8_t* wq, const float* sw,
+                                            const void* bias, int bias_dtype, const void* residual,
+                                            void* y, int y_dtype, int64_t M, int64_t N, int64_t K, void* ws,
+                                            size_t ws_bytes, void* stream) {
   if (x_dtype != AQ_F32 && x_dtype != AQ_BF16) return AQ_E_DTYPE;
   int mt = 0;
   int rc = gemv_check(wq, sw, bias, bias_dtype, y, y_dtype, M, N, K, &mt);
@@ -543,6 +571,8 @@ extern "C" int aq_gemv_w8a8_decode(const void* x, int x_dtype, const int8_t* wq,
     a.wq = wq;
     a.sw = sw;
     a.bias = bias;
+    a.res = residual;
+    a.ldr = N;
     a.y = y;
     a.M = (int)M;
     a.N = (int)N;
@@ -556,5 +586,12 @@ extern "C" int aq_gemv_w8a8_decode(const void* x, int x_dtype, const int8_t* wq,
   float* sx = reinterpret_cast<float*>(static_cast<char*>(ws) + aq::align256((size_t)(M * K)));
   rc = aq_quant_rowwise_i8(x, x_dtype, M, K, K, xq, sx, stream);
   if (rc) return rc;
-  return aq_gemv_w8a8_codes(xq, sx, wq, sw, bias, bias_dtype, y, y_dtype, M, N, K, stream);
+  return aq_gemv_w8a8_codes_residual(xq, sx, wq, sw, bias, bias_dtype, residual, y, y_dtype, M, N, K, stream);
+}
+
+extern "C" int aq_gemv_w8a8_decode(const void* x, int x_dtype, const int8_t* wq, const float* sw,
+                                   const void* bias, int bias_dtype, void* y, int y_dtype, int64_t M,
+                                   int64_t N, int64_t K, void* ws, size_t ws_bytes, void* stream) {
+  return aq_gemv_w8a8_decode_residual(x, x_dtype, wq, sw, bias, bias_dtype, nullptr, y, y_dtype, M, N, K, ws, ws_bytes,
+                                      stream);
 }

@@ -319,6 +319,50 @@ __global__ __launch_bounds__(256) void swiglu_quant_kernel(const void* __restric
   }
 }
 
+// The same with a workgroup per row, one vector pair per thread: with few rows a
+// wavefront per row leaves the device empty while each lane works through a
+// dozen vector pairs of exponentials.  The row maximum crosses the wavefronts
+// through LDS; a maximum does not depend on the order, so codes and scales are
+// the same bits as the kernel above gives.
+template <bool BF16>
+__global__ __launch_bounds__(1024) void swiglu_quant_wg_kernel(const void* __restrict__ ug, int F, int64_t ld,
+                                                               int8_t* __restrict__ q, float* __restrict__ scale) {
+  constexpr int EPV = RowIn<BF16>::EPV;
+  __shared__ float wmax[16];
+  const int v = threadIdx.x, lane = v & 63, wave = v >> 6, nwaves = blockDim.x >> 6;
+  const int nvec = F / EPV;
+  const int64_t row = blockIdx.x;
+  const uint4* up = reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(ug) + row * ld * (BF16 ? 2 : 4));
+  const uint4* gate = up + nvec;
+  const uint4 cu = v < nvec ? up[v] : make_uint4(0, 0, 0, 0);
+  const uint4 cg = v < nvec ? gate[v] : make_uint4(0, 0, 0, 0);
+  float u[EPV], g[EPV], h[EPV];
+  RowIn<BF16>::unpack(cu, u);
+  RowIn<BF16>::unpack(cg, g);
+#pragma unroll
+  for (int e = 0; e < EPV; ++e) h[e] = swiglu_repro(u[e], g[e]);
+  const float wm = wave_max(vec_amax<EPV>(h));
+  if (lane == 0) wmax[wave] = wm;
+  __syncthreads();
+  float amax = 0.0f;
+  for (int w = 0; w < nwaves; ++w) amax = fmaxf(amax, wmax[w]);
+  const RowScale rsc = row_scale(amax);
+  if (v == 0) scale[row] = rsc.s;
+  if (v < nvec) {
+    int8_t* dst = q + row * (int64_t)F;
+    uint32_t code[EPV];
+    quant_codes<EPV>(h, rsc.s, rsc.rs, rsc.fast_ok, code);
+    if constexpr (BF16) {
+      uint2 o;
+      o.x = pack_low_bytes(code[0], code[1], code[2], code[3]);
+      o.y = pack_low_bytes(code[4], code[5], code[6], code[7]);
+      store_wt(reinterpret_cast<uint2*>(dst + (int64_t)v * EPV), o);
+    } else {
+      store_wt(reinterpret_cast<uint32_t*>(dst + (int64_t)v * EPV), pack_low_bytes(code[0], code[1], code[2], code[3]));
+    }
+  }
+}
+
 // ---------------------------------------------------------------- FP8 tensor
 
 constexpr int FP8_BATCH = 4;  // 16-byte loads a thread keeps in flight in the per-tensor passes
@@ -528,10 +572,19 @@ extern "C" int aq_rmsnorm_quant_rowwise_i8(const void* x, int x_dtype, const voi
                             : launch_rmsnorm_quant<false>(x, gamma, eps, M, K, ldx, q, scale, st);
 }
 
+#ifndef AQ_SWIGLU_WG_MAX_M
+#define AQ_SWIGLU_WG_MAX_M 1024
+#endif
 template <bool BF16>
 static int launch_swiglu_quant(const void* ug, int64_t M, int64_t F, int64_t ld, int8_t* q, float* scale,
                                hipStream_t st) {
   const int64_t vpl = (F / (BF16 ? 8 : 4) + 63) / 64;  // vector pairs per lane
+  if (vpl > 12) return AQ_E_RANGE;
+  if (vpl > 1 && M <= AQ_SWIGLU_WG_MAX_M) {  // few rows: a workgroup of vpl wavefronts per row
+    hipLaunchKernelGGL((aq::swiglu_quant_wg_kernel<BF16>), dim3((unsigned)M), dim3((unsigned)vpl * 64), 0, st, ug, (int)F,
+                       ld, q, scale);
+    return (int)hipGetLastError();
+  }
   int64_t wgs = (M + 3) / 4;
   if (wgs > 1024) wgs = 1024;
   const dim3 g((unsigned)wgs), b(256);

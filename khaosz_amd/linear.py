@@ -161,7 +161,9 @@ class QuantLinear(Linear):
                                       error_msgs)
 
     # -- forward ----------------------------------------------------------------
-    def forward(self, x: Tensor) -> Tensor:
+    def forward(self, x: Tensor, residual: Optional[Tensor] = None) -> Tensor:
+        """``residual`` (shape and dtype of the output): returns ``linear(x) + residual`` with the add
+        done in the kernel's epilogue, bit-identical to adding the two tensors afterwards."""
         _no_grad_guard(x)
         lead = x.shape[:-1]
         x2 = x.reshape(-1, x.shape[-1])
@@ -175,21 +177,24 @@ class QuantLinear(Linear):
             ws = self._workspace
             if ws is None or ws.device != x.device or ws.numel() < need:
                 ws = self._workspace = torch.empty((need,), dtype=torch.uint8, device=x.device)
-            y = ops.gemv_w8a8_decode(x2, self.qweight, self.w_scale, self.bias, out_dtype=x.dtype, workspace=ws)
+            y = ops.gemv_w8a8_decode(x2, self.qweight, self.w_scale, self.bias, out_dtype=x.dtype, workspace=ws,
+                                     residual=residual)
         else:
             xq, sx = ops.quant_rowwise_i8(x2)
-            y = ops.linear_w8a8(xq, sx, self.qweight, self.w_scale, self.bias, out_dtype=x.dtype)
+            y = ops.linear_w8a8(xq, sx, self.qweight, self.w_scale, self.bias, out_dtype=x.dtype, residual=residual)
         return y.reshape(*lead, self.qweight.shape[0])
 
-    def forward_codes(self, xq: Tensor, sx: Tensor, out_dtype: torch.dtype) -> Tensor:
+    def forward_codes(self, xq: Tensor, sx: Tensor, out_dtype: torch.dtype,
+                      residual: Optional[Tensor] = None) -> Tensor:
         """The same projection for an input that is already quantised (``xq int8 [M, K]``,
         ``sx float32 [M]``): what a producer that fuses the quantisation hands over, or what
         several projections of one input share.  Returns ``[M, out_dim]``."""
         if xq.dim() != 2 or xq.shape[1] != self.qweight.shape[1]:
             raise ValueError(f"expected codes [M, {self.qweight.shape[1]}], got {tuple(xq.shape)}")
         if xq.shape[0] <= self.DECODE_MAX_ROWS:
-            return ops.gemv_w8a8_codes(xq, sx, self.qweight, self.w_scale, self.bias, out_dtype=out_dtype)
-        return ops.linear_w8a8(xq, sx, self.qweight, self.w_scale, self.bias, out_dtype=out_dtype)
+            return ops.gemv_w8a8_codes(xq, sx, self.qweight, self.w_scale, self.bias, out_dtype=out_dtype,
+                                       residual=residual)
+        return ops.linear_w8a8(xq, sx, self.qweight, self.w_scale, self.bias, out_dtype=out_dtype, residual=residual)
 
     def extra_repr(self) -> str:
         return f"in_dim={self.in_dim}, out_dim={self.out_dim}, bias={self.bias is not None}, w8a8"
@@ -251,7 +256,8 @@ TARGET_MODULES_ATTN = {"q_proj", "k_proj", "v_proj", "o_proj"}
 TARGET_MODULES_FFN = {"up", "gate", "down"}
 
 
-def fuse_shared_inputs(model: nn.Module, norms: bool = False, decode_attention: bool = False) -> int:
+def fuse_shared_inputs(model: nn.Module, norms: bool = False, decode_attention: bool = False,
+                       residuals: bool = False) -> int:
     """Call ``fuse_projections()`` on every module that offers it (attention and MLP blocks whose
     projections read one input); returns how many fused modules were built.  Run it after
     ``quantize_model`` and after loading weights: the fused module owns the weight storage from
@@ -260,7 +266,9 @@ def fuse_shared_inputs(model: nn.Module, norms: bool = False, decode_attention: 
     drops the bf16 rounding of the normalised activations: not bit-identical, inside the
     quantisation noise.  ``decode_attention=True`` lets attention modules with a fused q/k/v
     projection run single-token steps on a paged cache through the in-place attention kernels
-    (``fuse_decode_attention()``)."""
+    (``fuse_decode_attention()``).  ``residuals=True`` lets blocks hand the residual stream to the
+    quantized projection that ends each branch (``fuse_residual_adds()``): the add happens in that
+    kernel's epilogue, bit-identical to the separate add."""
     n = 0
     for m in model.modules():
         f = getattr(m, "fuse_projections", None)
@@ -274,6 +282,11 @@ def fuse_shared_inputs(model: nn.Module, norms: bool = False, decode_attention: 
     if decode_attention:
         for m in model.modules():
             f = getattr(m, "fuse_decode_attention", None)
+            if callable(f):
+                f()
+    if residuals:
+        for m in model.modules():
+            f = getattr(m, "fuse_residual_adds", None)
             if callable(f):
                 f()
     return n

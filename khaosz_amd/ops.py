@@ -163,9 +163,22 @@ def _bias_args(bias: Optional[torch.Tensor], N: int):
     return b, _dt(b, "bias")
 
 
-def linear_w8a8(xq, sx, wq, sw, bias=None, out_dtype=torch.bfloat16) -> torch.Tensor:
-    """MFMA GEMM with the fused epilogue y = (acc * sx[m]) * sw[n] (+ bias[n])."""
-    _need_gpu(xq, sx, wq, sw, bias)
+def _residual_arg(residual, M, N, out_dtype, dev):
+    """A residual is added to the rounded output (``y = round(linear) + residual``, rounded again:
+    the bits of a separate elementwise add); it holds M*N elements of the output's dtype."""
+    if residual is None:
+        return None
+    if residual.dtype != out_dtype or residual.numel() != M * N or residual.device != dev:
+        raise ValueError(f"residual must hold {M}x{N} {out_dtype} elements on {dev}, got {residual.dtype} "
+                         f"{tuple(residual.shape)} on {residual.device}")
+    if residual.dim() < 1 or residual.shape[-1] != N:
+        raise ValueError(f"residual's last dimension must be {N}, got {tuple(residual.shape)}")
+    return residual.contiguous()
+
+
+def linear_w8a8(xq, sx, wq, sw, bias=None, out_dtype=torch.bfloat16, residual=None) -> torch.Tensor:
+    """MFMA GEMM with the fused epilogue y = (acc * sx[m]) * sw[n] (+ bias[n]) (+ residual[m, n])."""
+    _need_gpu(xq, sx, wq, sw, bias, residual)
     if xq.dtype != torch.int8 or wq.dtype != torch.int8:
         raise ValueError("linear_w8a8 takes int8 codes")
     if xq.dim() != 2 or wq.dim() != 2 or xq.shape[1] != wq.shape[1]:
@@ -179,19 +192,24 @@ def linear_w8a8(xq, sx, wq, sw, bias=None, out_dtype=torch.bfloat16) -> torch.Te
         raise ValueError(f"out_dtype {out_dtype} is not supported")
     xq, wq, sx, sw = xq.contiguous(), wq.contiguous(), sx.contiguous(), sw.contiguous()
     b, bdt = _bias_args(bias, N)
+    r = _residual_arg(residual, M, N, out_dtype, xq.device)
     y = torch.empty((M, N), dtype=out_dtype, device=xq.device)
     if M and N:
         with torch.cuda.device(xq.device):
-            rc = _abi.load().aq_linear_w8a8(xq.data_ptr(), sx.data_ptr(), wq.data_ptr(), sw.data_ptr(),
-                                            b.data_ptr() if b is not None else None, bdt, y.data_ptr(),
-                                            _DT[out_dtype], M, N, K, _stream(xq))
+            rc = _abi.load().aq_linear_w8a8_residual(xq.data_ptr(), sx.data_ptr(), wq.data_ptr(), sw.data_ptr(),
+                                                     b.data_ptr() if b is not None else None, bdt,
+                                                     r.data_ptr() if r is not None else None, y.data_ptr(),
+                                                     _DT[out_dtype], M, N, K, _stream(xq))
         _abi.check(rc, "aq_linear_w8a8")
+    elif r is not None:
+        y.copy_(r.view(M, N))
     return y
 
 
-def gemv_w8a8_decode(x, wq, sw, bias=None, out_dtype=None, workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+def gemv_w8a8_decode(x, wq, sw, bias=None, out_dtype=None, workspace: Optional[torch.Tensor] = None,
+                     residual=None) -> torch.Tensor:
     """Decode path for at most 16 rows of ``x [M, K]``: fused per-token quantise + int8 GEMV + epilogue."""
-    _need_gpu(x, wq, sw, bias, workspace)
+    _need_gpu(x, wq, sw, bias, workspace, residual)
     x2 = _rows(x, "gemv_w8a8_decode")
     M, K = x2.shape
     N = wq.shape[0]
@@ -213,20 +231,24 @@ def gemv_w8a8_decode(x, wq, sw, bias=None, out_dtype=None, workspace: Optional[t
         workspace = torch.empty((max(need, 16),), dtype=torch.uint8, device=x.device)
     elif workspace.numel() * workspace.element_size() < need:
         raise ValueError(f"workspace holds {workspace.numel() * workspace.element_size()} bytes, {need} needed")
+    r = _residual_arg(residual, M, N, out_dtype, x.device)
     y = torch.empty((M, N), dtype=out_dtype, device=x.device)
     if M and N:
         with torch.cuda.device(x.device):
-            rc = lib.aq_gemv_w8a8_decode(x2.data_ptr(), _dt(x2, "x"), wq.data_ptr(), sw.data_ptr(),
-                                         b.data_ptr() if b is not None else None, bdt, y.data_ptr(), _DT[out_dtype],
-                                         M, N, K, workspace.data_ptr(), workspace.numel() * workspace.element_size(),
-                                         _stream(x))
+            rc = lib.aq_gemv_w8a8_decode_residual(x2.data_ptr(), _dt(x2, "x"), wq.data_ptr(), sw.data_ptr(),
+                                                  b.data_ptr() if b is not None else None, bdt,
+                                                  r.data_ptr() if r is not None else None, y.data_ptr(),
+                                                  _DT[out_dtype], M, N, K, workspace.data_ptr(),
+                                                  workspace.numel() * workspace.element_size(), _stream(x))
         _abi.check(rc, "aq_gemv_w8a8_decode")
+    elif r is not None:
+        y.copy_(r.view(M, N))
     return y
 
 
-def gemv_w8a8_codes(xq, sx, wq, sw, bias=None, out_dtype=torch.bfloat16) -> torch.Tensor:
+def gemv_w8a8_codes(xq, sx, wq, sw, bias=None, out_dtype=torch.bfloat16, residual=None) -> torch.Tensor:
     """The decode GEMV on activation codes the caller already holds (at most 16 rows)."""
-    _need_gpu(xq, sx, wq, sw, bias)
+    _need_gpu(xq, sx, wq, sw, bias, residual)
     if xq.dtype != torch.int8 or wq.dtype != torch.int8:
         raise ValueError("gemv_w8a8_codes takes int8 codes")
     if xq.dim() != 2 or wq.dim() != 2 or xq.shape[1] != wq.shape[1]:
@@ -242,13 +264,17 @@ def gemv_w8a8_codes(xq, sx, wq, sw, bias=None, out_dtype=torch.bfloat16) -> torc
         raise ValueError(f"out_dtype {out_dtype} is not supported")
     xq, wq, sx, sw = xq.contiguous(), wq.contiguous(), sx.contiguous(), sw.contiguous()
     b, bdt = _bias_args(bias, N)
+    r = _residual_arg(residual, M, N, out_dtype, xq.device)
     y = torch.empty((M, N), dtype=out_dtype, device=xq.device)
     if M and N:
         with torch.cuda.device(xq.device):
-            rc = _abi.load().aq_gemv_w8a8_codes(xq.data_ptr(), sx.data_ptr(), wq.data_ptr(), sw.data_ptr(),
-                                                b.data_ptr() if b is not None else None, bdt, y.data_ptr(),
-                                                _DT[out_dtype], M, N, K, _stream(xq))
+            rc = _abi.load().aq_gemv_w8a8_codes_residual(xq.data_ptr(), sx.data_ptr(), wq.data_ptr(), sw.data_ptr(),
+                                                         b.data_ptr() if b is not None else None, bdt,
+                                                         r.data_ptr() if r is not None else None, y.data_ptr(),
+                                                         _DT[out_dtype], M, N, K, _stream(xq))
         _abi.check(rc, "aq_gemv_w8a8_codes")
+    elif r is not None:
+        y.copy_(r.view(M, N))
     return y
 
 
@@ -291,10 +317,18 @@ def rope_kv_write(qkv: torch.Tensor, freqs: torch.Tensor, page_table: torch.Tens
     return q
 
 
+def paged_attn_workspace_bytes(B: int, n_heads: int, n_kv_heads: int, total_len: int) -> int:
+    """Bytes of device workspace ``paged_attn_decode`` needs for this shape (0: none)."""
+    return int(_abi.load().aq_paged_attn_decode_workspace_bytes(B, n_heads, n_kv_heads, int(total_len)))
+
+
 def paged_attn_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, page_table: torch.Tensor,
-                      total_len: int, scale: Optional[float] = None) -> torch.Tensor:
+                      total_len: int, scale: Optional[float] = None,
+                      workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``softmax(scale * q K^T) V`` for one query token per sequence over the first ``total_len``
-    positions of each sequence's pages: ``q [B, Hq, 128]`` -> ``[B, Hq, 128]`` (bfloat16)."""
+    positions of each sequence's pages: ``q [B, Hq, 128]`` -> ``[B, Hq, 128]`` (bfloat16).
+    ``workspace``: a contiguous device tensor of at least ``paged_attn_workspace_bytes`` bytes
+    to reuse across calls; allocated per call when omitted or too small."""
     _need_gpu(q, k_cache, v_cache, page_table)
     if q.dtype != torch.bfloat16 or k_cache.dtype != torch.bfloat16 or v_cache.dtype != torch.bfloat16:
         raise ValueError("paged_attn_decode takes bfloat16 tensors")
@@ -309,12 +343,18 @@ def paged_attn_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     page_table, q = page_table.contiguous(), q.contiguous()
     out = torch.empty_like(q)
     if B:
+        need = paged_attn_workspace_bytes(B, Hq, Hkv, total_len)
+        if need and (workspace is None or not workspace.is_contiguous() or workspace.device != q.device
+                     or workspace.numel() * workspace.element_size() < need):
+            workspace = torch.empty(need // 4, dtype=torch.float32, device=q.device)
+        ws_ptr = workspace.data_ptr() if need else None
+        ws_bytes = workspace.numel() * workspace.element_size() if need else 0
         with torch.cuda.device(q.device):
             rc = _abi.load().aq_paged_attn_decode(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                                                   page_table.data_ptr(), page_table.shape[1], int(total_len),
                                                   k_cache.shape[1], k_cache.shape[0],
                                                   float(scale if scale is not None else D ** -0.5), out.data_ptr(),
-                                                  B, Hq, Hkv, D, _stream(q))
+                                                  B, Hq, Hkv, D, ws_ptr, ws_bytes, _stream(q))
         _abi.check(rc, "aq_paged_attn_decode")
     return out
 

@@ -263,6 +263,34 @@ def test_fused_shared_input_projections_are_bit_identical():
 
 
 @pytest.mark.gpu
+def test_residual_adds_in_the_projection_epilogue_are_bit_identical():
+    """o_proj and down add the residual stream in their epilogue (GEMM for prefill, GEMV for
+    decode rows, with and without the fused norms): the same bits as the separate adds."""
+    from khaosz_amd import fuse_shared_inputs
+
+    dev, dt = "cuda:0", torch.bfloat16
+    for norms in (False, True):
+        a = _block(dim=256, heads=4, kv=2, ffn=704).to(dev).to(dt)
+        b = _block(dim=256, heads=4, kv=2, ffn=704).to(dev).to(dt)
+        b.load_state_dict(a.state_dict())
+        quantize_model(a), quantize_model(b)
+        fuse_shared_inputs(a, norms=norms)
+        fuse_shared_inputs(b, norms=norms, residuals=True)
+        tab = rotary_table(64, 64, device=dev)
+        x = (torch.randn(2, 40, 256, device=dev) * 3).to(dt)
+        with torch.inference_mode():
+            assert torch.equal(b(x, _freqs(tab, 2, 0, 40)), a(x, _freqs(tab, 2, 0, 40)))      # M = 80
+            for rows in (1, 3, 6):                                                            # M = 2, 6, 12
+                xd = x[:, :rows].contiguous()
+                assert torch.equal(b(xd, _freqs(tab, 2, 0, rows)), a(xd, _freqs(tab, 2, 0, rows)))
+    # a float block takes the same flag and simply adds
+    f = _block(dim=256, heads=4, kv=2, ffn=704).to(dev).to(dt)
+    want = f(x, _freqs(tab, 2, 0, 40))
+    fuse_shared_inputs(f, residuals=True)
+    assert torch.equal(f(x, _freqs(tab, 2, 0, 40)), want)
+
+
+@pytest.mark.gpu
 def test_fused_norm_quantise_stays_inside_the_quantisation_noise():
     """RMSNorm + per-token quantisation in one launch for both norms of the block: outputs move by
     far less than the quantisation error itself (the bf16 rounding of the norm output is gone),

@@ -44,7 +44,8 @@ def test_rope_kv_write_bit_exact(oracle, B, Hq, Hkv, page, pos):
 
 
 @pytest.mark.parametrize("B,Hq,Hkv,page,T", [(1, 1, 1, 4, 1), (2, 8, 2, 16, 70), (8, 16, 4, 64, 576), (3, 8, 1, 16, 1000),
-                                              (2, 4, 2, 64, 513)])
+                                              (2, 4, 2, 64, 513), (1, 2, 2, 8, 64), (2, 2, 1, 4, 65), (1, 4, 4, 32, 256),
+                                              (2, 16, 2, 16, 257), (40, 8, 8, 16, 300), (1, 8, 1, 64, 5000)])
 def test_paged_attn_decode_within_bf16_rounding(oracle, B, Hq, Hkv, page, T):
     _say("paged_attn_decode", B, Hq, Hkv, page, T)
     D = 128
@@ -63,6 +64,34 @@ def test_paged_attn_decode_within_bf16_rounding(oracle, B, Hq, Hkv, page, T):
     # stated tolerance: 1e-2 relative for bf16 outputs (different summation order, exp2 instead of exp)
     assert torch.allclose(out, want, rtol=1e-2, atol=1e-2)
     assert ((out - want).norm() / want.norm()).item() < 4e-3
+
+
+def test_paged_attn_workspace_reuse_and_checks(oracle):
+    """A caller-owned workspace gives the same bits as a per-call one; a short one is refused."""
+    _say("paged_attn_workspace")
+    from khaosz_amd import _abi
+    B, Hq, Hkv, page, T, D = 4, 8, 2, 16, 700, 128
+    P = (T + page - 1) // page
+    g = torch.Generator().manual_seed(5)
+    q = torch.randn(B, Hq, D, generator=g).to(torch.bfloat16).to(DEV)
+    kc = torch.randn(B * P, page, Hkv, D, generator=g).to(torch.bfloat16).to(DEV)
+    vc = torch.randn(B * P, page, Hkv, D, generator=g).to(torch.bfloat16).to(DEV)
+    table = torch.randperm(B * P, generator=g).view(B, P).to(DEV)
+    need = ops.paged_attn_workspace_bytes(B, Hq, Hkv, T)
+    assert need > 0 and need % 16 == 0
+    assert ops.paged_attn_workspace_bytes(1, 1, 1, 10) == 0
+    ws = torch.full((need // 4 + 64,), float("nan"), device=DEV)      # stale contents must not matter
+    a = ops.paged_attn_decode(q, kc, vc, table, T)
+    b = ops.paged_attn_decode(q, kc, vc, table, T, workspace=ws)
+    c = ops.paged_attn_decode(q, kc, vc, table, T, workspace=ws)
+    assert torch.equal(a, b) and torch.equal(a, c)
+    out = torch.empty_like(q)
+    lib = _abi.load()
+    args = (q.data_ptr(), kc.data_ptr(), vc.data_ptr(), table.data_ptr(), P, T, page, B * P, D ** -0.5, out.data_ptr(),
+            B, Hq, Hkv, D)
+    assert lib.aq_paged_attn_decode(*args, ws.data_ptr(), need - 16, None) == -5    # AQ_E_WORKSPACE
+    assert lib.aq_paged_attn_decode(*args, None, 0, None) == -1                  # AQ_E_NULL
+    torch.cuda.synchronize()
 
 
 def test_attn_argument_checks():

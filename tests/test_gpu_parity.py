@@ -163,7 +163,7 @@ def test_rmsnorm_quant_tracks_torch_rms_norm_then_quantise():
         ops.rmsnorm_quant_rowwise_i8(torch.zeros(2, 32768, device=DEV), torch.ones(32768, device=DEV), 1e-5)
 
 
-@pytest.mark.parametrize("M,F", [(1, 16), (7, 48), (5, 1040), (64, 2048), (8, 5632), (130, 704)])
+@pytest.mark.parametrize("M,F", [(1, 16), (7, 48), (5, 1040), (64, 2048), (8, 5632), (130, 704), (1100, 1040)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_swiglu_quant_bit_exact(oracle, M, F, dtype):
     if dtype == torch.float32 and F > 3072:
@@ -277,6 +277,34 @@ def test_linear_w8a8_epilogue_bit_exact(oracle, tile, M, N, K, out_dtype, bias_k
     else:
         want = oracle.c_dequant_epilogue(acc, sx, sw, bias_np, bf16_out=True)
         assert np.array_equal(bf16_bits(y), want)
+    # with a residual: the bits of the reference's separate add of the two tensors (decoder_block.py:56-57)
+    r = (torch.randn(M, N, generator=torch.Generator().manual_seed(8)) * 2).to(DEV, out_dtype)
+    y2 = ops.linear_w8a8(torch.from_numpy(xq).to(DEV), torch.from_numpy(sx).to(DEV), torch.from_numpy(wq).to(DEV),
+                         torch.from_numpy(sw).to(DEV), bias, out_dtype=out_dtype, residual=r)
+    assert torch.equal(y2, y + r)
+
+
+def test_linear_residual_may_alias_the_output(tile):
+    """x += linear(h): the residual pointer is the output pointer (GEMM and GEMV entry points)."""
+    from khaosz_amd import _abi
+    lib = _abi.load()
+    for M in (200, 7):
+        N, K = 384, 256
+        g = torch.Generator().manual_seed(M)
+        xq = torch.randint(-127, 128, (M, K), generator=g, dtype=torch.int8).to(DEV)
+        wq = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8).to(DEV)
+        sx = (torch.rand(M, generator=g) * 1e-2 + 1e-3).to(DEV)
+        sw = (torch.rand(N, generator=g) * 1e-2 + 1e-3).to(DEV)
+        r = torch.randn(M, N, generator=g).to(DEV, torch.bfloat16)
+        fn = ops.linear_w8a8 if M > 16 else ops.gemv_w8a8_codes
+        want = fn(xq, sx, wq, sw, residual=r)
+        assert torch.equal(want, fn(xq, sx, wq, sw) + r)
+        y = r.clone()
+        entry = lib.aq_linear_w8a8_residual if M > 16 else lib.aq_gemv_w8a8_codes_residual
+        rc = entry(xq.data_ptr(), sx.data_ptr(), wq.data_ptr(), sw.data_ptr(), None, 0, y.data_ptr(), y.data_ptr(), 1,
+                   M, N, K, None)
+        torch.cuda.synchronize()
+        assert rc == 0 and torch.equal(y, want)
 
 
 # ------------------------------------------------------------------- decode
@@ -295,6 +323,10 @@ def test_gemv_decode_bit_exact(oracle, M, N, K):
         want = oracle.c_linear_w8a8(bf16_bits(x), wq, sw, None if bias is None else bias.numpy(),
                                     x_bf16_bits=True, bf16_out=True)
         assert np.array_equal(bf16_bits(y), want)
+        r = (torch.randn(M, N, generator=torch.Generator().manual_seed(14)) * 2).to(DEV, torch.bfloat16)
+        y2 = ops.gemv_w8a8_decode(x.to(DEV), torch.from_numpy(wq).to(DEV), torch.from_numpy(sw).to(DEV),
+                                  None if bias is None else bias.to(DEV), out_dtype=torch.bfloat16, residual=r)
+        assert torch.equal(y2, y + r)
 
 
 def test_gemv_f32_in_out_and_agrees_with_gemm_path(oracle):
@@ -309,6 +341,9 @@ def test_gemv_f32_in_out_and_agrees_with_gemm_path(oracle):
     xq, sx = ops.quant_rowwise_i8(x.to(DEV))
     y2 = ops.linear_w8a8(xq, sx, wqd, swd, out_dtype=torch.float32)
     assert torch.equal(y, y2)
+    r = torch.randn(M, N, generator=torch.Generator().manual_seed(23)).to(DEV)
+    assert torch.equal(ops.gemv_w8a8_decode(x.to(DEV), wqd, swd, out_dtype=torch.float32, residual=r), y + r)
+    assert torch.equal(ops.gemv_w8a8_codes(xq, sx, wqd, swd, out_dtype=torch.float32, residual=r), y + r)
 
 
 # ---------------------------------------------------------------------- FP8

@@ -84,6 +84,7 @@ struct GemvArgs {
   int64_t ldr;
   int M, N, K;
   int bias_dtype, y_dtype;
+  int ksplit, groups;  // matrix-core variant: wavefronts sharing a row group, row groups per workgroup
 };
 
 // y (+ residual): the projection is rounded to the output type first and the
@@ -96,6 +97,11 @@ __device__ __forceinline__ float add_residual_bf16(float y, uint32_t res_bits) {
 
 // FUSED: the kernel quantises the bf16 activation rows itself (VPL 16-byte vectors
 // per lane per row) instead of copying codes a separate launch produced.
+// Wavefronts per workgroup: GV_WAVES for the fused kernels (they split the row
+// quantisation among them: with fewer, each would round several rows one after
+// the other before any product can start), taken from the launch otherwise.  A
+// workgroup covers GV_ROWS * wavefronts weight rows; the launcher shrinks it
+// when N is too small for 8-wavefront workgroups to reach every compute unit.
 template <int MT, bool FUSED, int VPL>
 __global__ __launch_bounds__(GV_THREADS) void gemv_w8a8_kernel(GemvArgs p) {
   extern __shared__ __attribute__((aligned(16))) uint8_t xs[];  // [MT][K] activation codes, then [MT] scales
@@ -103,7 +109,9 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_w8a8_kernel(GemvArgs p) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int K = p.K, N = p.N, M = p.M;
   // wavefront-uniform first row, kept scalar so the buffer descriptor lives in SGPRs
-  const int n0 = __builtin_amdgcn_readfirstlane((blockIdx.x * GV_WAVES + wave) * GV_ROWS);
+  constexpr int WAVES = GV_WAVES;
+  const int nwaves = FUSED ? WAVES : (int)(blockDim.x >> 6);
+  const int n0 = __builtin_amdgcn_readfirstlane((blockIdx.x * nwaves + wave) * GV_ROWS);
 
   // 0. After the reduction lane l owns output (row n0 + idx / MT, token idx % MT)
   // with idx = l >> (6 - log2(rows * MT)).  Its scales and bias are requested
@@ -132,16 +140,16 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_w8a8_kernel(GemvArgs p) {
   // global memory (rows m >= M lie outside the descriptor and arrive as zeros),
   // or produced here: each wavefront requests its rows of the bf16 activation now
   // and quantises them while the weight loads queued behind are in flight.
-  constexpr int RPW = (MT + GV_WAVES - 1) / GV_WAVES;
+  constexpr int RPW = FUSED ? (MT + WAVES - 1) / WAVES : 1;
   RowsToLds<true, RPW, VPL> xrows;
   if constexpr (FUSED) {
-    xrows.issue(p.x, M, K, K, wave, GV_WAVES, lane);
+    xrows.issue(p.x, M, K, K, wave, WAVES, lane);
   } else {
     const __amdgpu_buffer_rsrc_t Xr = make_rsrc(p.xq, (uint32_t)M * (uint32_t)K);
     const int xbytes = MT * K;
-    const int xrounds = (xbytes + GV_THREADS * 16 - 1) / (GV_THREADS * 16);
+    const int xrounds = (xbytes + nwaves * 1024 - 1) / (nwaves * 1024);
     for (int r = 0; r < xrounds; ++r) {
-      const int base = (r * GV_WAVES + wave) * 1024;  // this wavefront's 1 KiB of the copy
+      const int base = (r * nwaves + wave) * 1024;  // this wavefront's 1 KiB of the copy
       if (base < xbytes)  // uniform; xbytes is a multiple of 16 but not always of 1024:
         __builtin_amdgcn_raw_ptr_buffer_load_lds(
             Xr, (gv_lds_void*)(xs + base), 16,
@@ -172,7 +180,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_w8a8_kernel(GemvArgs p) {
   // compiler place that wait), then make every wavefront's part visible through
   // a barrier that does not drain the weight loads.
   if constexpr (FUSED) {
-    xrows.finish(M, MT, K, xs, K, sx_lds, wave, GV_WAVES, lane);
+    xrows.finish(M, MT, K, xs, K, sx_lds, wave, WAVES, lane);
     __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wavefront's LDS writes are done
   } else {
     GV_WAIT_VMCNT(GV_DEPTH * GV_ROWS);
@@ -242,16 +250,25 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_w8a8_kernel(GemvArgs p) {
     reinterpret_cast<float*>(p.y)[o] = y;
 }
 
+// Wavefronts per workgroup for N weight rows: 8, halved (down to 2) while the launch would have
+// fewer workgroups than the device has compute units.
+static int gemv_waves(int N) {
+  int waves = GV_WAVES;
+  while (waves > 2 && (N + GV_ROWS * waves - 1) / (GV_ROWS * waves) < 256) waves >>= 1;
+  return waves;
+}
+
 template <int MT, bool FUSED, int VPL>
 static int launch_gemv(const GemvArgs& a, hipStream_t st) {
-  const unsigned grid = (unsigned)((a.N + GV_ROWS * GV_WAVES - 1) / (GV_ROWS * GV_WAVES));
+  const int waves = FUSED ? GV_WAVES : gemv_waves(a.N);
+  const unsigned grid = (unsigned)((a.N + GV_ROWS * waves - 1) / (GV_ROWS * waves));
   const size_t lds = (size_t)MT * a.K + MT * sizeof(float);
   if (lds > 64 * 1024) {  // beyond the default dynamic-LDS limit: opt this kernel in (idempotent)
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_w8a8_kernel<MT, FUSED, VPL>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return (int)e;
   }
-  hipLaunchKernelGGL((gemv_w8a8_kernel<MT, FUSED, VPL>), dim3(grid), dim3(GV_THREADS), lds, st, a);
+  hipLaunchKernelGGL((gemv_w8a8_kernel<MT, FUSED, VPL>), dim3(grid), dim3(waves * 64), lds, st, a);
   return (int)hipGetLastError();
 }
 
@@ -273,30 +290,24 @@ constexpr int GV_MFMA_MIN_M = AQ_GV_MFMA_MIN_M;  // more tokens than this take t
 // whole 128-byte lines), and multiplies against the token codes held in LDS.
 // The 16 x 16 result has rows = weight rows and columns = tokens, so a lane
 // ends up with 4 consecutive outputs of one token: no cross-lane reduction.
-// Two wavefronts share a row group, each taking half of K; the halves are
-// summed through LDS (exact int32).
+// ksplit wavefronts share a row group, each taking a part of K; the parts are
+// summed through LDS (exact int32).  A workgroup holds `groups` row groups:
+// 2 x 2 wavefronts when N fills the device that way, fewer rows per workgroup
+// and more K parts when it does not.
 constexpr int GM_ROWS = 16;    // weight rows per wavefront
-#ifndef AQ_GM_KSPLIT
-#define AQ_GM_KSPLIT 2
-#endif
-constexpr int GM_KSPLIT = AQ_GM_KSPLIT;   // wavefronts sharing a row group
-#ifndef AQ_GM_GROUPS
-#define AQ_GM_GROUPS 2
-#endif
-constexpr int GM_GROUPS = AQ_GM_GROUPS;   // row groups per workgroup
-constexpr int GM_WAVES = GM_KSPLIT * GM_GROUPS;
+constexpr int GM_MAX_WAVES = 8;
 constexpr int GM_BATCH = 8;    // MFMA steps (64 K bytes each) per register batch
 
-template <bool FUSED>
-__global__ __launch_bounds__(GM_WAVES * 64) void gemv_mfma_kernel(GemvArgs p) {
+__global__ __launch_bounds__(GM_MAX_WAVES * 64) void gemv_mfma_kernel(GemvArgs p) {
   extern __shared__ __attribute__((aligned(16))) uint8_t xs[];  // [16][K + 16] token codes, [16] scales; later the partial sums
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int grp = wave / GM_KSPLIT, kh = wave % GM_KSPLIT;
+  const int nthreads = p.ksplit * p.groups * 64;
+  const int grp = wave / p.ksplit, kh = wave % p.ksplit;
   const int K = p.K, N = p.N, M = p.M;
-  const int n0 = __builtin_amdgcn_readfirstlane((blockIdx.x * GM_GROUPS + grp) * GM_ROWS);
+  const int n0 = __builtin_amdgcn_readfirstlane((blockIdx.x * p.groups + grp) * GM_ROWS);
   const int pitch = K + 16;  // 16 token rows then start 4 banks apart: conflict-free 16-byte reads
-  const int khalf = K / GM_KSPLIT;  // a multiple of 64 (checked by the launcher)
+  const int khalf = K / p.ksplit;  // a multiple of 64 (checked by the launcher)
   const int nstep = khalf / 64;
 
   // epilogue operands first: lane l -> token l%16, rows (l/16)*4 .. +3 of the group
@@ -311,10 +322,8 @@ __global__ __launch_bounds__(GM_WAVES * 64) void gemv_mfma_kernel(GemvArgs p) {
     rv[r] = 0;
   }
   float* sx_lds = reinterpret_cast<float*>(xs + 16 * pitch);
-  if (kh == 0) {  // uniform: only the first half's wavefront writes outputs
-    if constexpr (!FUSED) {
-      if (tok < M) sxv = p.sx[tok];
-    }
+  if (kh == 0) {  // uniform: only the first part's wavefront writes outputs
+    if (tok < M) sxv = p.sx[tok];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const int n = rbase + r < N ? rbase + r : N - 1;
@@ -341,32 +350,25 @@ __global__ __launch_bounds__(GM_WAVES * 64) void gemv_mfma_kernel(GemvArgs p) {
   };
 
   // token codes -> LDS (padded rows; tokens >= M are zero).  Their loads are
-  // issued before the weight loads, so they return first and the LDS fill --
-  // or, when FUSED, the quantisation of the bf16 rows (4 rows per wavefront,
-  // 4 vectors per lane per row: K <= 2048) -- overlaps the weight stream's flight time.
-  if constexpr (FUSED) {
-    RowsToLds<true, (16 + GM_WAVES - 1) / GM_WAVES, 4> rows;
-    rows.issue(p.x, M, K, K, wave, GM_WAVES, lane);
-    wload(0, wa);
-    wload(GM_BATCH, wb);
-    rows.finish(M, 16, K, xs, pitch, sx_lds, wave, GM_WAVES, lane);
-  } else {
+  // issued before the weight loads, so they return first and the LDS fill
+  // overlaps the weight stream's flight time.
+  {
     const __amdgpu_buffer_rsrc_t Xr = make_rsrc(p.xq, (uint32_t)M * (uint32_t)K);
     const int nvec_row = K / 16;
     const int nvec = 16 * nvec_row;
-    constexpr int XV = 2048 / (GM_WAVES * 64);  // vectors per thread per round: 16 x 2048 codes in one round
+    constexpr int XV = 8;  // vectors per thread per round: 16 x 2048 codes in one round of 256 threads
     uint4 xv[XV];
     auto xload = [&](int v0) {
 #pragma unroll
       for (int i = 0; i < XV; ++i) {
-        const int v = v0 + i * (GM_WAVES * 64) + tid;
+        const int v = v0 + i * nthreads + tid;
         xv[i] = buffer_load_16(Xr, v < nvec ? (uint32_t)v * 16u : OOB_OFFSET);
       }
     };
     auto xstore = [&](int v0) {
 #pragma unroll
       for (int i = 0; i < XV; ++i) {
-        const int v = v0 + i * (GM_WAVES * 64) + tid;
+        const int v = v0 + i * nthreads + tid;
         if (v < nvec) {
           const int m = v / nvec_row, c = v - m * nvec_row;
           *reinterpret_cast<uint4*>(xs + m * pitch + c * 16) = xv[i];
@@ -377,7 +379,7 @@ __global__ __launch_bounds__(GM_WAVES * 64) void gemv_mfma_kernel(GemvArgs p) {
     wload(0, wa);
     wload(GM_BATCH, wb);
     xstore(0);
-    for (int v0 = XV * GM_WAVES * 64; v0 < nvec; v0 += XV * GM_WAVES * 64) {  // rows longer than 2048
+    for (int v0 = XV * nthreads; v0 < nvec; v0 += XV * nthreads) {  // longer rows
       xload(v0);
       xstore(v0);
     }
@@ -387,9 +389,6 @@ __global__ __launch_bounds__(GM_WAVES * 64) void gemv_mfma_kernel(GemvArgs p) {
   asm volatile("" ::: "memory");
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
-  if constexpr (FUSED) {
-    if (kh == 0 && tok < M) sxv = sx_lds[tok];
-  }
 
   v4i acc = {0, 0, 0, 0};
   const uint8_t* xl = xs + tok * pitch + kh * khalf + (lane >> 4) * 16;
@@ -411,14 +410,13 @@ __global__ __launch_bounds__(GM_WAVES * 64) void gemv_mfma_kernel(GemvArgs p) {
 
   // sum the K parts: all but the first wavefront of each group park their 4 sums in LDS
   __syncthreads();  // everyone is done reading the token codes: the buffer is reused
-  int* part = reinterpret_cast<int*>(xs) + grp * (GM_KSPLIT - 1) * 256;
+  int* part = reinterpret_cast<int*>(xs) + grp * (p.ksplit - 1) * 256;
   if (kh != 0) {
     *reinterpret_cast<v4i*>(part + (kh - 1) * 256 + lane * 4) = acc;
   }
   __syncthreads();
   if (kh != 0) return;
-#pragma unroll
-  for (int k = 0; k < GM_KSPLIT - 1; ++k) acc += *reinterpret_cast<const v4i*>(part + k * 256 + lane * 4);
+  for (int k = 0; k < p.ksplit - 1; ++k) acc += *reinterpret_cast<const v4i*>(part + k * 256 + lane * 4);
 
   if (tok >= M) return;
   float y[4];
@@ -453,24 +451,33 @@ __global__ __launch_bounds__(GM_WAVES * 64) void gemv_mfma_kernel(GemvArgs p) {
   }
 }
 
-template <bool FUSED>
-static int launch_gemv_mfma(const GemvArgs& a, hipStream_t st) {
-  const unsigned grid = (unsigned)((a.N + GM_ROWS * GM_GROUPS - 1) / (GM_ROWS * GM_GROUPS));
+// the streaming MFMA variant needs K in whole 128-byte steps (two K parts of 64-byte MFMA steps)
+// and its padded codes to fit LDS
+static bool gemv_mfma_ok(int64_t M, int64_t K) {
+  return M > GV_MFMA_MIN_M && (K % 128) == 0 && 16 * (K + 16) + 64 <= GV_MAX_LDS;
+}
+
+static int launch_gemv_mfma(GemvArgs a, hipStream_t st) {
+  // 2 row groups x 2 K parts per workgroup by default; with too few rows for that to give every
+  // compute unit a workgroup, one row group per workgroup and up to 8 K parts
+  a.ksplit = 2;
+  a.groups = 2;
+  if ((a.N + 31) / 32 < 256) {
+    a.groups = 1;
+    while (a.ksplit < GM_MAX_WAVES && (a.N + 15) / 16 * (a.ksplit / 2) < 256 && a.K % (128 * a.ksplit) == 0 &&
+           a.K / (2 * a.ksplit) >= 512)
+      a.ksplit *= 2;
+  }
+  const unsigned grid = (unsigned)((a.N + GM_ROWS * a.groups - 1) / (GM_ROWS * a.groups));
   const size_t lds = (size_t)16 * (a.K + 16) + 16 * sizeof(float);
   if (lds > 64 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_mfma_kernel<FUSED>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_mfma_kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return (int)e;
   }
-  hipLaunchKernelGGL((gemv_mfma_kernel<FUSED>), dim3(grid), dim3(GM_WAVES * 64), lds, st, a);
+  hipLaunchKernelGGL(gemv_mfma_kernel, dim3(grid), dim3(a.ksplit * a.groups * 64), lds, st, a);
   return (int)hipGetLastError();
 }
-
-// the streaming MFMA variant needs each K half to be whole 64-byte steps and its padded codes to fit LDS
-static bool gemv_mfma_ok(int64_t M, int64_t K) {
-  return M > GV_MFMA_MIN_M && (K % (64 * GM_KSPLIT)) == 0 && 16 * (K + 16) + 64 <= GV_MAX_LDS;
-}
-
 
 static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
@@ -497,7 +504,7 @@ static int gemv_check(const int8_t* wq, const float* sw, const void* bias, int b
 }
 
 static int gemv_dispatch(const aq::GemvArgs& a, int mt, hipStream_t st) {
-  if (aq::gemv_mfma_ok(a.M, a.K)) return aq::launch_gemv_mfma<false>(a, st);
+  if (aq::gemv_mfma_ok(a.M, a.K)) return aq::launch_gemv_mfma(a, st);
   switch (mt) {
     case 1: return aq::launch_gemv<1, false, 4>(a, st);
     case 2: return aq::launch_gemv<2, false, 4>(a, st);

@@ -190,6 +190,19 @@ int aq_paged_attn_decode(const void *q, const void *k_cache, const void *v_cache
                          int64_t D, void *workspace, int64_t workspace_bytes, void *stream);
 int64_t aq_paged_attn_decode_workspace_bytes(int64_t B, int64_t Hq, int64_t Hkv, int64_t total_len);
 
+/* aq_rope_kv_write and aq_paged_attn_decode as one call for the usual decode
+ * step: the new token sits at position total_len - 1.  Queries are rotated by
+ * the workgroups that use them; the new key and value are rotated, stored into
+ * their page slot and attended to from registers.  Caches and outputs are the
+ * bits the two separate calls give.  freqs must be 16-byte aligned and
+ * freqs_stride a multiple of 4 floats (or 0); workspace as for
+ * aq_paged_attn_decode. */
+int aq_rope_paged_attn_decode(const void *qkv, const float *freqs, int64_t freqs_stride,
+                              const int64_t *page_table, int64_t P, int64_t total_len,
+                              int64_t page_size, void *k_cache, void *v_cache, int64_t n_pages,
+                              float scale, void *out, int64_t B, int64_t Hq, int64_t Hkv, int64_t D,
+                              void *workspace, int64_t workspace_bytes, void *stream);
+
 /* Tuning and test hook, no counterpart in the reference: the GEMM entry points
  * pick their workgroup tile (256 x 128, or 128 x 128 with a split K step when
  * the larger one would leave compute units idle) from M and N.  rows = 128 or

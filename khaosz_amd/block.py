@@ -169,9 +169,9 @@ class GQA(nn.Module):
 
     def fuse_decode_attention(self) -> bool:
         """A step with one new token per sequence on a paged cache: rotate q/k and write k/v into
-        their page slot in one launch, then attend over the pages in place in another
-        (``ops.rope_kv_write``, ``ops.paged_attn_decode``), instead of the gather / repeat_kv /
-        generic attention sequence.  Needs the fused q/k/v projection, bf16 and head dimension
+        their page slot and attend over the pages in place, all in one launch
+        (``ops.rope_paged_attn_decode``), instead of the gather / repeat_kv / generic attention
+        sequence.  Needs the fused q/k/v projection, bf16 and head dimension
         128, and assumes what the serving loop's decode step has: no padding inside the cached
         length (the additive mask is all zeros).  Outputs agree within bf16 rounding."""
         if self._qkv is not None and self.head_dim == 128 and self.n_heads // self.n_kv_heads in (1, 2, 4, 8):
@@ -196,9 +196,8 @@ class GQA(nn.Module):
         if (self._decode_attention and S == 1 and isinstance(cache, PagedKV) and x.is_cuda
                 and x.dtype == torch.bfloat16):
             qkv = self._qkv(x) if codes is None else self._qkv.forward_codes(codes[0], codes[1], x.dtype)
-            q = ops.rope_kv_write(qkv.view(B, -1), rotary_emb.reshape(B, -1), cache.page_table, cache.total_len - 1,
-                                  cache.k, cache.v, self.n_heads, self.n_kv_heads)
-            out = ops.paged_attn_decode(q, cache.k, cache.v, cache.page_table, cache.total_len)
+            out = ops.rope_paged_attn_decode(qkv.view(B, -1), rotary_emb.reshape(B, -1), cache.page_table,
+                                             cache.total_len, cache.k, cache.v, self.n_heads, self.n_kv_heads)
             return self._out(out.view(B, 1, -1), residual)
         if self._qkv is not None:
             nq, nkv = self.n_heads * self.head_dim, self.n_kv_heads * self.head_dim

@@ -69,6 +69,11 @@ struct AttnArgs {
   const int64_t* table;  // [B, P]
   uint16_t* out;         // [B, Hq, D]
   float* ws;             // partial results [B, Hq, NS, ATT_PART] when NS > 1
+  const uint16_t* qkv;   // ROPE kernels: [B, (Hq + 2 Hkv) * D] projections of the new token (position T - 1)
+  const float* freqs;    // ROPE kernels: its rotary table, as in RopeArgs
+  uint16_t* kc_w;        // ROPE kernels: the caches again, writable
+  uint16_t* vc_w;
+  int64_t freqs_stride;
   int64_t P, T, page, n_pages;
   float scale_log2e;     // softmax scale times log2(e): scores live in the exp2 domain
   int B, Hq, Hkv, NS;
@@ -110,7 +115,29 @@ __device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float c) {
 // The wavefronts' (maximum, denominator, numerator) are merged through LDS and
 // either normalised into the output (NS == 1) or left in the workspace for
 // attn_merge_kernel.
-template <int G>
+// Rotates 8 consecutive elements (4 interleaved pairs) exactly as rope_kv_write_kernel does.
+__device__ __forceinline__ uint4 rope8(uint4 x, const float* cs /* 4 (cos, sin) pairs */) {
+  const float4 a = *reinterpret_cast<const float4*>(cs), b = *reinterpret_cast<const float4*>(cs + 4);
+  const float c[4] = {a.x, a.z, b.x, b.z}, sn[4] = {a.y, a.w, b.y, b.w};
+  const uint32_t in[4] = {x.x, x.y, x.z, x.w};
+  uint32_t o[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float x0 = __uint_as_float(in[i] << 16), x1 = __uint_as_float(in[i] & 0xffff0000u);
+    const float r0 = __fsub_rn(__fmul_rn(x0, c[i]), __fmul_rn(x1, sn[i]));
+    const float r1 = __fadd_rn(__fmul_rn(x0, sn[i]), __fmul_rn(x1, c[i]));
+    o[i] = pack_bf16x2(r0, r1);
+  }
+  return make_uint4(o[0], o[1], o[2], o[3]);
+}
+
+// ROPE: the kernel also does rope_kv_write_kernel's work for the new token at
+// position T - 1 -- every workgroup rotates its own queries from the raw
+// projection, and the one wavefront whose positions include T - 1 rotates the
+// new key, stores it and the new value into their page slot and uses them from
+// registers instead of what it read from the cache.  Same roundings, so caches
+// and outputs are the bits the two separate launches give.
+template <int G, bool ROPE>
 __global__ __launch_bounds__(ATT_WAVES * 64) void paged_attn_decode_kernel(AttnArgs p) {
   constexpr int NL = ATT_NL, KPW = ATT_KPW, KPG = ATT_KPG;
   constexpr int ATT_THREADS = ATT_WAVES * 64;
@@ -147,9 +174,24 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void paged_attn_decode_kernel(AttnA
       }
     }
     uint4 qv[G];  // this lane's 8 dimensions of each query
+    uint4 knew = make_uint4(0, 0, 0, 0), vnew = make_uint4(0, 0, 0, 0);
+    const bool has_new = ROPE && T - 1 >= t0 && T - 1 < t0 + KPW;  // wavefront-uniform
+    if constexpr (ROPE) {
+      const int64_t heads = p.Hq + 2 * p.Hkv;
+      const uint16_t* tok = p.qkv + (int64_t)b * heads * AD;
+      const float* cs = p.freqs + (int64_t)b * p.freqs_stride + ch * 8;
 #pragma unroll
-    for (int g = 0; g < G; ++g)
-      qv[g] = *reinterpret_cast<const uint4*>(p.q + ((int64_t)b * p.Hq + kvh * G + g) * AD + ch * 8);
+      for (int g = 0; g < G; ++g)
+        qv[g] = rope8(*reinterpret_cast<const uint4*>(tok + (int64_t)(kvh * G + g) * AD + ch * 8), cs);
+      if (has_new) {
+        knew = rope8(*reinterpret_cast<const uint4*>(tok + (int64_t)(p.Hq + kvh) * AD + ch * 8), cs);
+        vnew = *reinterpret_cast<const uint4*>(tok + (int64_t)(p.Hq + p.Hkv + kvh) * AD + ch * 8);
+      }
+    } else {
+#pragma unroll
+      for (int g = 0; g < G; ++g)
+        qv[g] = *reinterpret_cast<const uint4*>(p.q + ((int64_t)b * p.Hq + kvh * G + g) * AD + ch * 8);
+    }
     uint4 kv[NL], vv[NL];
 #pragma unroll
     for (int i = 0; i < NL; ++i) {
@@ -159,8 +201,15 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void paged_attn_decode_kernel(AttnA
       kv[i] = make_uint4(0, 0, 0, 0);
       vv[i] = make_uint4(0, 0, 0, 0);
       if (r >= 0) {
-        kv[i] = *reinterpret_cast<const uint4*>(p.kc + r + ch * 8);
-        vv[i] = *reinterpret_cast<const uint4*>(p.vc + r + ch * 8);
+        if (ROPE && has_new && t0 + src == T - 1) {  // the new token: from registers, and into its slot
+          kv[i] = knew;
+          vv[i] = vnew;
+          *reinterpret_cast<uint4*>(p.kc_w + r + ch * 8) = knew;
+          *reinterpret_cast<uint4*>(p.vc_w + r + ch * 8) = vnew;
+        } else {
+          kv[i] = *reinterpret_cast<const uint4*>(p.kc + r + ch * 8);
+          vv[i] = *reinterpret_cast<const uint4*>(p.vc + r + ch * 8);
+        }
       }
     }
     // ---- scores
@@ -321,18 +370,22 @@ extern "C" int64_t aq_paged_attn_decode_workspace_bytes(int64_t B, int64_t Hq, i
   return ns == 1 ? 0 : B * Hq * ns * aq::ATT_PART * (int64_t)sizeof(float);
 }
 
-extern "C" int aq_paged_attn_decode(const void* q, const void* k_cache, const void* v_cache,
-                                    const int64_t* page_table, int64_t P, int64_t total_len, int64_t page_size,
-                                    int64_t n_pages, float scale, void* out, int64_t B, int64_t Hq, int64_t Hkv,
-                                    int64_t D, void* workspace, int64_t workspace_bytes, void* stream) {
+// q == nullptr: the fused form, queries and the new token come from qkv / freqs.
+static int attn_decode(const void* q, const void* qkv, const float* freqs, int64_t freqs_stride, void* k_cache,
+                       void* v_cache, const int64_t* page_table, int64_t P, int64_t total_len, int64_t page_size,
+                       int64_t n_pages, float scale, void* out, int64_t B, int64_t Hq, int64_t Hkv, int64_t D,
+                       void* workspace, int64_t workspace_bytes, void* stream) {
+  const bool rope = q == nullptr;
   if (D != aq::AD) return AQ_E_SHAPE;
   if (B < 0 || Hq <= 0 || Hkv <= 0 || (Hq % Hkv) != 0 || P <= 0 || total_len <= 0 || page_size <= 0 ||
       n_pages <= 0 || !(scale > 0.0f))
     return AQ_E_SHAPE;
+  if (rope && freqs_stride != 0 && freqs_stride < D) return AQ_E_SHAPE;
   if (B == 0) return AQ_OK;
-  if (!q || !k_cache || !v_cache || !page_table || !out) return AQ_E_NULL;
-  if (aq::check_ptr16(q) || aq::check_ptr16(k_cache) || aq::check_ptr16(v_cache) || aq::check_ptr16(out))
+  if (!(rope ? (qkv != nullptr && freqs != nullptr) : (q != nullptr)) || !k_cache || !v_cache || !page_table || !out) return AQ_E_NULL;
+  if (aq::check_ptr16(rope ? qkv : q) || aq::check_ptr16(k_cache) || aq::check_ptr16(v_cache) || aq::check_ptr16(out))
     return AQ_E_ALIGN;
+  if (rope && (aq::check_ptr16(freqs) || (freqs_stride & 3))) return AQ_E_ALIGN;
   const int64_t ns = aq::attn_slices(total_len);
   if (B * Hkv * ns > (int64_t)0x7fffffff || B * Hq > (int64_t)0x7fffffff) return AQ_E_RANGE;
   if (ns > 1) {
@@ -342,8 +395,13 @@ extern "C" int aq_paged_attn_decode(const void* q, const void* k_cache, const vo
   }
   aq::AttnArgs a{};
   a.q = static_cast<const uint16_t*>(q);
+  a.qkv = static_cast<const uint16_t*>(qkv);
+  a.freqs = freqs;
+  a.freqs_stride = freqs_stride;
   a.kc = static_cast<const uint16_t*>(k_cache);
   a.vc = static_cast<const uint16_t*>(v_cache);
+  a.kc_w = static_cast<uint16_t*>(k_cache);
+  a.vc_w = static_cast<uint16_t*>(v_cache);
   a.table = page_table;
   a.out = static_cast<uint16_t*>(out);
   a.ws = static_cast<float*>(workspace);
@@ -358,15 +416,40 @@ extern "C" int aq_paged_attn_decode(const void* q, const void* k_cache, const vo
   a.NS = (int)ns;
   const dim3 grid((unsigned)(B * Hkv * ns)), block(aq::ATT_WAVES * 64);
   hipStream_t st = static_cast<hipStream_t>(stream);
+#define AQ_ATTN_CASE(G_)                                                                           \
+  case G_:                                                                                         \
+    if (rope) hipLaunchKernelGGL((aq::paged_attn_decode_kernel<G_, true>), grid, block, 0, st, a); \
+    else hipLaunchKernelGGL((aq::paged_attn_decode_kernel<G_, false>), grid, block, 0, st, a);     \
+    break;
   switch (Hq / Hkv) {
-    case 1: hipLaunchKernelGGL(aq::paged_attn_decode_kernel<1>, grid, block, 0, st, a); break;
-    case 2: hipLaunchKernelGGL(aq::paged_attn_decode_kernel<2>, grid, block, 0, st, a); break;
-    case 4: hipLaunchKernelGGL(aq::paged_attn_decode_kernel<4>, grid, block, 0, st, a); break;
-    case 8: hipLaunchKernelGGL(aq::paged_attn_decode_kernel<8>, grid, block, 0, st, a); break;
+    AQ_ATTN_CASE(1)
+    AQ_ATTN_CASE(2)
+    AQ_ATTN_CASE(4)
+    AQ_ATTN_CASE(8)
     default: return AQ_E_SHAPE;  // query heads per KV head: 1, 2, 4 or 8
   }
+#undef AQ_ATTN_CASE
   int rc = (int)hipGetLastError();
   if (rc != 0 || ns == 1) return rc;
   hipLaunchKernelGGL(aq::attn_merge_kernel, dim3((unsigned)(B * Hq)), dim3(aq::AD / 2), 0, st, a.ws, a.out, a.NS);
   return (int)hipGetLastError();
+}
+
+extern "C" int aq_paged_attn_decode(const void* q, const void* k_cache, const void* v_cache,
+                                    const int64_t* page_table, int64_t P, int64_t total_len, int64_t page_size,
+                                    int64_t n_pages, float scale, void* out, int64_t B, int64_t Hq, int64_t Hkv,
+                                    int64_t D, void* workspace, int64_t workspace_bytes, void* stream) {
+  if (!q && B > 0) return AQ_E_NULL;
+  return attn_decode(q, nullptr, nullptr, 0, const_cast<void*>(k_cache), const_cast<void*>(v_cache), page_table, P,
+                     total_len, page_size, n_pages, scale, out, B, Hq, Hkv, D, workspace, workspace_bytes, stream);
+}
+
+extern "C" int aq_rope_paged_attn_decode(const void* qkv, const float* freqs, int64_t freqs_stride,
+                                         const int64_t* page_table, int64_t P, int64_t total_len, int64_t page_size,
+                                         void* k_cache, void* v_cache, int64_t n_pages, float scale, void* out,
+                                         int64_t B, int64_t Hq, int64_t Hkv, int64_t D, void* workspace,
+                                         int64_t workspace_bytes, void* stream) {
+  if ((!qkv || !freqs) && B > 0) return AQ_E_NULL;
+  return attn_decode(nullptr, qkv, freqs, freqs_stride, k_cache, v_cache, page_table, P, total_len, page_size, n_pages,
+                     scale, out, B, Hq, Hkv, D, workspace, workspace_bytes, stream);
 }

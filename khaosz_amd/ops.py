@@ -278,16 +278,14 @@ def gemv_w8a8_codes(xq, sx, wq, sw, bias=None, out_dtype=torch.bfloat16, residua
     return y
 
 
-def rope_kv_write(qkv: torch.Tensor, freqs: torch.Tensor, page_table: torch.Tensor, pos: int, k_cache: torch.Tensor,
-                  v_cache: torch.Tensor, n_heads: int, n_kv_heads: int) -> torch.Tensor:
-    """One new token per sequence: rotate q and k of ``qkv [B, (Hq + 2 Hkv) * 128]`` by ``freqs``
-    (complex64 ``[B, 64]`` or float32 ``[B, 64, 2]``), write k and v into the paged caches
-    ``[n_pages, page, Hkv, 128]`` at logical position ``pos``; returns the rotated ``q [B, Hq, 128]``."""
+def _rope_args(qkv, freqs, page_table, k_cache, v_cache, n_heads, n_kv_heads, what):
+    """Checks shared by the decode-step entry points; returns (qkv, freqs as float32, its batch
+    stride in floats, page_table), contiguous."""
     _need_gpu(qkv, freqs, page_table, k_cache, v_cache)
     B = qkv.shape[0]
     D = k_cache.shape[-1]
     if qkv.dtype != torch.bfloat16 or k_cache.dtype != torch.bfloat16 or v_cache.dtype != torch.bfloat16:
-        raise ValueError("rope_kv_write takes bfloat16 activations and caches")
+        raise ValueError(f"{what} takes bfloat16 activations and caches")
     if qkv.dim() != 2 or qkv.shape[1] != (n_heads + 2 * n_kv_heads) * D:
         raise ValueError(f"qkv must be [B, {(n_heads + 2 * n_kv_heads) * D}], got {tuple(qkv.shape)}")
     if k_cache.dim() != 4 or k_cache.shape != v_cache.shape or k_cache.shape[2] != n_kv_heads:
@@ -304,8 +302,17 @@ def rope_kv_write(qkv: torch.Tensor, freqs: torch.Tensor, page_table: torch.Tens
         fr_stride = D
     if page_table.dtype != torch.int64 or page_table.dim() != 2 or page_table.shape[0] != B:
         raise ValueError("page_table must be int64 [B, P]")
-    page_table = page_table.contiguous()
-    qkv = qkv.contiguous()
+    return qkv.contiguous(), fr, fr_stride, page_table.contiguous()
+
+
+def rope_kv_write(qkv: torch.Tensor, freqs: torch.Tensor, page_table: torch.Tensor, pos: int, k_cache: torch.Tensor,
+                  v_cache: torch.Tensor, n_heads: int, n_kv_heads: int) -> torch.Tensor:
+    """One new token per sequence: rotate q and k of ``qkv [B, (Hq + 2 Hkv) * 128]`` by ``freqs``
+    (complex64 ``[B, 64]`` or float32 ``[B, 64, 2]``), write k and v into the paged caches
+    ``[n_pages, page, Hkv, 128]`` at logical position ``pos``; returns the rotated ``q [B, Hq, 128]``."""
+    qkv, fr, fr_stride, page_table = _rope_args(qkv, freqs, page_table, k_cache, v_cache, n_heads, n_kv_heads,
+                                                "rope_kv_write")
+    B, D = qkv.shape[0], k_cache.shape[-1]
     q = torch.empty((B, n_heads, D), dtype=torch.bfloat16, device=qkv.device)
     if B:
         with torch.cuda.device(qkv.device):
@@ -315,6 +322,41 @@ def rope_kv_write(qkv: torch.Tensor, freqs: torch.Tensor, page_table: torch.Tens
                                               k_cache.shape[0], q.data_ptr(), B, n_heads, n_kv_heads, D, _stream(qkv))
         _abi.check(rc, "aq_rope_kv_write")
     return q
+
+
+def _attn_workspace(workspace, need, dev):
+    if need and (workspace is None or not workspace.is_contiguous() or workspace.device != dev
+                 or workspace.numel() * workspace.element_size() < need or workspace.data_ptr() % 16):
+        workspace = torch.empty(need // 4, dtype=torch.float32, device=dev)
+    if not need:
+        return None, 0
+    return workspace.data_ptr(), workspace.numel() * workspace.element_size()
+
+
+def rope_paged_attn_decode(qkv: torch.Tensor, freqs: torch.Tensor, page_table: torch.Tensor, total_len: int,
+                           k_cache: torch.Tensor, v_cache: torch.Tensor, n_heads: int, n_kv_heads: int,
+                           scale: Optional[float] = None, workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``rope_kv_write`` at position ``total_len - 1`` and ``paged_attn_decode`` over ``total_len``
+    positions as one launch (plus the small merge launch for long sequences): same caches and
+    outputs, bit for bit.  Returns the attention output ``[B, Hq, 128]``."""
+    qkv, fr, fr_stride, page_table = _rope_args(qkv, freqs, page_table, k_cache, v_cache, n_heads, n_kv_heads,
+                                                "rope_paged_attn_decode")
+    B, D = qkv.shape[0], k_cache.shape[-1]
+    if total_len < 1:
+        raise ValueError("total_len counts the new token: at least 1")
+    out = torch.empty((B, n_heads, D), dtype=torch.bfloat16, device=qkv.device)
+    if B:
+        ws_ptr, ws_bytes = _attn_workspace(workspace, paged_attn_workspace_bytes(B, n_heads, n_kv_heads, total_len),
+                                           qkv.device)
+        with torch.cuda.device(qkv.device):
+            rc = _abi.load().aq_rope_paged_attn_decode(qkv.data_ptr(), fr.data_ptr(), fr_stride, page_table.data_ptr(),
+                                                       page_table.shape[1], int(total_len), k_cache.shape[1],
+                                                       k_cache.data_ptr(), v_cache.data_ptr(), k_cache.shape[0],
+                                                       float(scale if scale is not None else D ** -0.5),
+                                                       out.data_ptr(), B, n_heads, n_kv_heads, D, ws_ptr, ws_bytes,
+                                                       _stream(qkv))
+        _abi.check(rc, "aq_rope_paged_attn_decode")
+    return out
 
 
 def paged_attn_workspace_bytes(B: int, n_heads: int, n_kv_heads: int, total_len: int) -> int:
@@ -343,12 +385,7 @@ def paged_attn_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     page_table, q = page_table.contiguous(), q.contiguous()
     out = torch.empty_like(q)
     if B:
-        need = paged_attn_workspace_bytes(B, Hq, Hkv, total_len)
-        if need and (workspace is None or not workspace.is_contiguous() or workspace.device != q.device
-                     or workspace.numel() * workspace.element_size() < need):
-            workspace = torch.empty(need // 4, dtype=torch.float32, device=q.device)
-        ws_ptr = workspace.data_ptr() if need else None
-        ws_bytes = workspace.numel() * workspace.element_size() if need else 0
+        ws_ptr, ws_bytes = _attn_workspace(workspace, paged_attn_workspace_bytes(B, Hq, Hkv, total_len), q.device)
         with torch.cuda.device(q.device):
             rc = _abi.load().aq_paged_attn_decode(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                                                   page_table.data_ptr(), page_table.shape[1], int(total_len),

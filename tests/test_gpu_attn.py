@@ -94,6 +94,41 @@ def test_paged_attn_workspace_reuse_and_checks(oracle):
     torch.cuda.synchronize()
 
 
+@pytest.mark.parametrize("B,Hq,Hkv,page,T", [(1, 1, 1, 4, 1), (2, 8, 2, 16, 70), (8, 16, 4, 64, 576), (3, 8, 1, 16, 1000),
+                                              (2, 4, 2, 64, 513), (2, 2, 1, 4, 65), (1, 4, 4, 32, 256), (5, 16, 2, 16, 257)])
+def test_rope_paged_attn_decode_equals_the_two_launches(B, Hq, Hkv, page, T):
+    """The fused decode step (rotate, write the new token, attend) against rope_kv_write followed by
+    paged_attn_decode: caches and outputs bit for bit, including a sequence whose new page is unmapped."""
+    _say("rope_paged_attn_decode", B, Hq, Hkv, page, T)
+    D = 128
+    P = (T + page - 1) // page
+    n_pages = B * P + 2
+    g = torch.Generator().manual_seed(T + 1)
+    qkv = torch.randn(B, (Hq + 2 * Hkv) * D, generator=g).to(torch.bfloat16).to(DEV)
+    ang = torch.rand(B, D // 2, generator=g) * 6.28
+    freqs = torch.polar(torch.ones_like(ang), ang).to(DEV)
+    kc = torch.randn(n_pages, page, Hkv, D, generator=g).to(torch.bfloat16).to(DEV)
+    vc = torch.randn(n_pages, page, Hkv, D, generator=g).to(torch.bfloat16).to(DEV)
+    table = torch.randperm(n_pages, generator=g)[:B * P].view(B, P)
+    if B > 2:
+        table[1, (T - 1) // page] = -1
+    table = table.to(DEV)
+    k1, v1, k2, v2 = kc.clone(), vc.clone(), kc.clone(), vc.clone()
+    q = ops.rope_kv_write(qkv, freqs, table, T - 1, k1, v1, Hq, Hkv)
+    want = ops.paged_attn_decode(q, k1, v1, table, T)
+    out = ops.rope_paged_attn_decode(qkv, freqs, table, T, k2, v2, Hq, Hkv)
+    assert torch.equal(k1, k2) and torch.equal(v1, v2)
+    assert not torch.equal(k1, kc)
+    assert torch.equal(out, want)
+    # one rotary table shared by the batch (stride 0)
+    if B > 1:
+        shared = freqs[:1].expand(B, -1)
+        q = ops.rope_kv_write(qkv, shared, table, T - 1, k1, v1, Hq, Hkv)
+        want = ops.paged_attn_decode(q, k1, v1, table, T)
+        assert torch.equal(ops.rope_paged_attn_decode(qkv, shared, table, T, k2, v2, Hq, Hkv), want)
+        assert torch.equal(k1, k2) and torch.equal(v1, v2)
+
+
 def test_attn_argument_checks():
     q = torch.zeros(2, 4, 64, dtype=torch.bfloat16, device=DEV)
     kc = torch.zeros(4, 8, 2, 64, dtype=torch.bfloat16, device=DEV)

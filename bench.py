@@ -284,8 +284,10 @@ def bench_block(torch, ops, args, dev):
     ms_pre = graph_time_ms(torch, prefill, 10, 3)
     prefill()
     ms_dec_norms = graph_time_ms(torch, decode_all, 3, 2) / steps
-    # and the single-token steps through the in-place paged attention kernels
+    # and the paged-cache kernels: rotary + page writes in one launch at prefill, rotary + page
+    # write + in-place attention in one launch for the single-token steps
     fuse_shared_inputs(blk, norms=True, decode_attention=True)
+    ms_pre_att = graph_time_ms(torch, prefill, 10, 3)
     prefill()
     ms_dec_att = graph_time_ms(torch, decode_all, 3, 2) / steps
     # and the two residual adds inside the epilogues of o_proj and down (bit-identical)
@@ -342,7 +344,7 @@ def bench_block(torch, ops, args, dev):
         "separate_projections": {"prefill_ms": ms_pre_sep, "decode_ms_per_step": ms_dec_sep},
         "fused_projections_separate_norms": {"prefill_ms": ms_pre_proj, "decode_ms_per_step": ms_dec_proj},
         "fused_norms_torch_attention": {"prefill_ms": ms_pre_norms, "decode_ms_per_step": ms_dec_norms},
-        "paged_decode_attention_separate_adds": {"prefill_ms": ms_pre_norms, "decode_ms_per_step": ms_dec_att},
+        "paged_attention_kernels_separate_adds": {"prefill_ms": ms_pre_att, "decode_ms_per_step": ms_dec_att},
         "linears_prefill_ms": ms_lin_pre, "linears_prefill_tops": lin_ops / (ms_lin_pre * 1e-3) / 1e12,
         "linears_decode_ms_per_step": ms_lin_dec, "linears_decode_gbs": lin_bytes / (ms_lin_dec * 1e-3) / 1e9,
         "non_linear_prefill_ms": ms_pre - ms_lin_pre, "non_linear_decode_ms_per_step": ms_dec - ms_lin_dec,

@@ -149,20 +149,23 @@ int aq_rmsnorm_quant_rowwise_i8(const void *x, int x_dtype, const void *gamma, i
 int aq_swiglu_quant_rowwise_i8(const void *ug, int dtype, int64_t M, int64_t F, int64_t ld,
                                int8_t *q, float *scale, void *stream);
 
-/* ---- decode-step attention over the paged KV cache (what sits between the qkv
- * and the output projection at decode; bf16, head dimension 128).
+/* ---- attention around the paged KV cache (what sits between the qkv and the
+ * output projection; bf16, head dimension 128).
  *
- * aq_rope_kv_write: for the one new token of each of B sequences, rotate the q
- * and k heads of qkv [B, (Hq + 2 Hkv) * D] (q heads, then k heads, then v heads:
- * the fused projection's column order) by freqs [B, D/2, 2] = (cos, sin) pairs
- * (freqs_stride floats from one sequence's table to the next; 0 when all sequences
- * are at the same position and share one) --
+ * aq_rope_kv_write: for the S new tokens of each of B sequences (S = 1 at
+ * decode, the prompt length at prefill), rotate the q and k heads of
+ * qkv [B, S, (Hq + 2 Hkv) * D] (q heads, then k heads, then v heads: the fused
+ * projection's column order) by freqs [S, D/2, 2] = (cos, sin) pairs per sequence
+ * (freqs_stride floats from one sequence's table to the next; 0 when all
+ * sequences are at the same positions and share one; 16-byte aligned) --
  * interleaved pairs (x[2i], x[2i+1]), fp32, as apply_rotary_emb does
- * (astrai/model/components/rope.py:26-33) -- store q to q_out [B, Hq, D], and write
- * the rotated k and the v into slot pos % page_size of page
- * page_table[b, pos / page_size] of k_cache / v_cache
- * [n_pages, page_size, Hkv, D] (Storage.write, astrai/inference/core/cache.py:216-252;
- * a sequence whose page is unmapped, entry < 0, is skipped there too).
+ * (astrai/model/components/rope.py:26-33) -- store q to q_out [B, S, Hq, D], the
+ * rotated k to k_out [B, S, Hkv, D] when that is not NULL (for an attention over
+ * the new tokens themselves), and write the rotated k and the v of token s into
+ * slot (pos + s) % page_size of page page_table[b, (pos + s) / page_size] of
+ * k_cache / v_cache [n_pages, page_size, Hkv, D] (Storage.write,
+ * astrai/inference/core/cache.py:216-252; tokens whose page is unmapped, entry
+ * < 0, are skipped there too).
  *
  * aq_paged_attn_decode: out [B, Hq, D] = softmax(scale * q K^T) V over positions
  * 0 .. total_len-1 of each sequence, read through page_table [B, P] in place --
@@ -181,9 +184,10 @@ int aq_swiglu_quant_rowwise_i8(const void *ug, int dtype, int64_t M, int64_t F, 
  * grows with total_len: a caller that sizes it once uses the longest sequence
  * it will serve. */
 int aq_rope_kv_write(const void *qkv, const float *freqs, int64_t freqs_stride,
-                     const int64_t *page_table, int64_t P,
-                     int64_t pos, int64_t page_size, void *k_cache, void *v_cache, int64_t n_pages,
-                     void *q_out, int64_t B, int64_t Hq, int64_t Hkv, int64_t D, void *stream);
+                     const int64_t *page_table, int64_t P, int64_t pos, int64_t S,
+                     int64_t page_size, void *k_cache, void *v_cache, int64_t n_pages,
+                     void *q_out, void *k_out, int64_t B, int64_t Hq, int64_t Hkv, int64_t D,
+                     void *stream);
 int aq_paged_attn_decode(const void *q, const void *k_cache, const void *v_cache,
                          const int64_t *page_table, int64_t P, int64_t total_len, int64_t page_size,
                          int64_t n_pages, float scale, void *out, int64_t B, int64_t Hq, int64_t Hkv,

@@ -109,6 +109,11 @@ class PagedKV:
         self.total_len = total_len
         return self
 
+    @property
+    def all_mapped(self) -> bool:
+        """Every entry of the bound page table names a page."""
+        return self._invalid is None
+
     def write(self, layer_id: int, k: Tensor, v: Tensor) -> None:
         S = k.size(1)
         if S == 0:
@@ -168,12 +173,15 @@ class GQA(nn.Module):
         return False
 
     def fuse_decode_attention(self) -> bool:
-        """A step with one new token per sequence on a paged cache: rotate q/k and write k/v into
-        their page slot and attend over the pages in place, all in one launch
+        """Use the paged-cache kernels.  A step with one new token per sequence rotates q/k,
+        writes k/v into their page slot and attends over the pages in place, all in one launch
         (``ops.rope_paged_attn_decode``), instead of the gather / repeat_kv / generic attention
-        sequence.  Needs the fused q/k/v projection, bf16 and head dimension
-        128, and assumes what the serving loop's decode step has: no padding inside the cached
-        length (the additive mask is all zeros).  Outputs agree within bf16 rounding."""
+        sequence; it assumes what the serving loop's decode step has: no padding inside the
+        cached length (the additive mask is all zeros).  Several new tokens (prefill) get the
+        rotation and the page writes as one launch (``ops.rope_kv_write``) in front of the stock
+        attention, which then reads the new keys directly and shares KV heads without
+        repeating them.  Needs the fused q/k/v projection, bf16 and head dimension 128.
+        Outputs agree within bf16 rounding."""
         if self._qkv is not None and self.head_dim == 128 and self.n_heads // self.n_kv_heads in (1, 2, 4, 8):
             self._decode_attention = True
         return self._decode_attention
@@ -199,6 +207,23 @@ class GQA(nn.Module):
             out = ops.rope_paged_attn_decode(qkv.view(B, -1), rotary_emb.reshape(B, -1), cache.page_table,
                                              cache.total_len, cache.k, cache.v, self.n_heads, self.n_kv_heads)
             return self._out(out.view(B, 1, -1), residual)
+        if (self._decode_attention and isinstance(cache, PagedKV) and x.is_cuda and x.dtype == torch.bfloat16
+                and S <= cache.total_len):
+            # several new tokens (prefill): rotation and the page writes as one launch; the attention
+            # itself stays the stock one, over the new keys directly when nothing older is cached
+            nq, nkv = self.n_heads * self.head_dim, self.n_kv_heads * self.head_dim
+            qkv = self._qkv(x) if codes is None else self._qkv.forward_codes(codes[0], codes[1], x.dtype).view(B, S, -1)
+            start = cache.total_len - S
+            q, k = ops.rope_kv_write(qkv, rotary_emb, cache.page_table, start, cache.k, cache.v, self.n_heads,
+                                     self.n_kv_heads, return_k=True)
+            if start == 0 and cache.all_mapped:
+                v = qkv[..., nq + nkv:].view(B, S, self.n_kv_heads, self.head_dim)
+            else:
+                k, v = cache.gather(self.layer_id)
+            out = F.scaled_dot_product_attention(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), attn_mask,
+                                                 is_causal=attn_mask is None,
+                                                 enable_gqa=self.n_heads != self.n_kv_heads)
+            return self._out(out.transpose(1, 2).reshape(B, S, -1), residual)
         if self._qkv is not None:
             nq, nkv = self.n_heads * self.head_dim, self.n_kv_heads * self.head_dim
             qkv = self._qkv(x) if codes is None else self._qkv.forward_codes(codes[0], codes[1], x.dtype).view(B, S, -1)

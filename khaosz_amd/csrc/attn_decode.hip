@@ -5,9 +5,10 @@
 // astrai/inference/core/cache.py:254-274).  Two kernels replace that for a step
 // with one new token per sequence:
 //
-//   rope_kv_write   rotates q and k of the new token (interleaved pairs, fp32,
+//   rope_kv_write   rotates q and k of the new tokens (interleaved pairs, fp32,
 //                   rope.py:26-33), stores q, and writes k and v into their page
-//                   slot (cache.py:216-252);
+//                   slots (cache.py:216-252) -- one token per sequence at decode,
+//                   the whole prompt at prefill;
 //   paged_attn      softmax(q K^T / sqrt(D)) V over the pages of each sequence,
 //                   all query heads of a KV head in one workgroup (grouped-query
 //                   attention without materialising the repeated heads,
@@ -22,44 +23,59 @@ namespace aq {
 
 constexpr int AD = 128;          // head dimension
 
+// Rotates 8 consecutive elements (4 interleaved pairs): (x0 + i x1)(c + i s) with four rounded
+// products, one rounded difference and one rounded sum per pair.
+__device__ __forceinline__ uint4 rope8(uint4 x, const float* cs /* 4 (cos, sin) pairs */) {
+  const float4 a = *reinterpret_cast<const float4*>(cs), b = *reinterpret_cast<const float4*>(cs + 4);
+  const float c[4] = {a.x, a.z, b.x, b.z}, sn[4] = {a.y, a.w, b.y, b.w};
+  const uint32_t in[4] = {x.x, x.y, x.z, x.w};
+  uint32_t o[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float x0 = __uint_as_float(in[i] << 16), x1 = __uint_as_float(in[i] & 0xffff0000u);
+    const float r0 = __fsub_rn(__fmul_rn(x0, c[i]), __fmul_rn(x1, sn[i]));
+    const float r1 = __fadd_rn(__fmul_rn(x0, sn[i]), __fmul_rn(x1, c[i]));
+    o[i] = pack_bf16x2(r0, r1);
+  }
+  return make_uint4(o[0], o[1], o[2], o[3]);
+}
+
 struct RopeArgs {
-  const uint16_t* qkv;   // [B, (Hq + 2 Hkv) * D]
-  const float* freqs;    // [B, D/2, 2] (cos, sin) of the new token's position; sequence stride freqs_stride floats
+  const uint16_t* qkv;   // [B, S, (Hq + 2 Hkv) * D]
+  const float* freqs;    // [S, D/2, 2] (cos, sin) per sequence; sequences freqs_stride floats apart (0: shared)
   int64_t freqs_stride;
   const int64_t* table;  // [B, P]
   uint16_t* kc;          // [n_pages, page, Hkv, D]
   uint16_t* vc;
-  uint16_t* q_out;       // [B, Hq, D]
-  int64_t P, pos, page, n_pages;
+  uint16_t* q_out;       // [B, S, Hq, D]
+  uint16_t* k_out;       // [B, S, Hkv, D] rotated keys, or null
+  int64_t P, pos, page, n_pages, S;
   int B, Hq, Hkv;
 };
 
-// one wavefront per head vector: lane l owns the pair (2l, 2l+1)
-__global__ __launch_bounds__(64) void rope_kv_write_kernel(RopeArgs p) {
-  const int lane = threadIdx.x;
-  const int heads = p.Hq + 2 * p.Hkv;
-  const int b = blockIdx.x / heads, h = blockIdx.x % heads;
-  const uint32_t pair = reinterpret_cast<const uint32_t*>(p.qkv + ((int64_t)b * heads + h) * AD)[lane];
-  uint32_t out = pair;
-  if (h < p.Hq + p.Hkv) {  // q and k heads rotate, v heads do not
-    const float x0 = bf16_bits_to_f32((uint16_t)(pair & 0xffffu)), x1 = bf16_bits_to_f32((uint16_t)(pair >> 16));
-    const float2 cs = reinterpret_cast<const float2*>(p.freqs + (int64_t)b * p.freqs_stride)[lane];
-    // (x0 + i x1)(c + i s): four rounded products, one rounded difference, one rounded sum
-    const float r0 = __fsub_rn(__fmul_rn(x0, cs.x), __fmul_rn(x1, cs.y));
-    const float r1 = __fadd_rn(__fmul_rn(x0, cs.y), __fmul_rn(x1, cs.x));
-    out = pack_bf16x2(r0, r1);
-  }
+// one thread per 16-byte chunk (8 elements) of a head vector of a token
+__global__ __launch_bounds__(256) void rope_kv_write_kernel(RopeArgs p) {
+  const int64_t heads = p.Hq + 2 * p.Hkv;
+  const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (c >= (int64_t)p.B * p.S * heads * (AD / 8)) return;
+  const int ch = (int)(c & 15);
+  const int64_t hv = c >> 4, tokn = hv / heads;
+  const int h = (int)(hv % heads);
+  const int64_t b = tokn / p.S, s = tokn % p.S;
+  uint4 x = *reinterpret_cast<const uint4*>(p.qkv + hv * AD + ch * 8);
+  if (h < p.Hq + p.Hkv) x = rope8(x, p.freqs + b * p.freqs_stride + s * AD + ch * 8);  // v heads do not rotate
   if (h < p.Hq) {
-    reinterpret_cast<uint32_t*>(p.q_out + ((int64_t)b * p.Hq + h) * AD)[lane] = out;
+    *reinterpret_cast<uint4*>(p.q_out + (tokn * p.Hq + h) * AD + ch * 8) = x;
     return;
   }
-  const int64_t lp = p.pos / p.page;
-  const int64_t phys = lp < p.P ? p.table[(int64_t)b * p.P + lp] : -1;
-  if (phys < 0 || phys >= p.n_pages) return;  // unmapped: the token is dropped, as in the reference
   const bool is_k = h < p.Hq + p.Hkv;
   const int kvh = is_k ? h - p.Hq : h - p.Hq - p.Hkv;
-  uint16_t* dst = (is_k ? p.kc : p.vc) + ((phys * p.page + p.pos % p.page) * p.Hkv + kvh) * AD;
-  reinterpret_cast<uint32_t*>(dst)[lane] = out;
+  if (is_k && p.k_out) *reinterpret_cast<uint4*>(p.k_out + (tokn * p.Hkv + kvh) * AD + ch * 8) = x;
+  const int64_t pos = p.pos + s, lp = pos / p.page;
+  const int64_t phys = lp < p.P ? p.table[b * p.P + lp] : -1;
+  if (phys < 0 || phys >= p.n_pages) return;  // unmapped: the token is dropped, as in the reference
+  uint16_t* dst = (is_k ? p.kc : p.vc) + ((phys * p.page + pos % p.page) * p.Hkv + kvh) * AD + ch * 8;
+  *reinterpret_cast<uint4*>(dst) = x;
 }
 
 struct AttnArgs {
@@ -115,22 +131,6 @@ __device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float c) {
 // The wavefronts' (maximum, denominator, numerator) are merged through LDS and
 // either normalised into the output (NS == 1) or left in the workspace for
 // attn_merge_kernel.
-// Rotates 8 consecutive elements (4 interleaved pairs) exactly as rope_kv_write_kernel does.
-__device__ __forceinline__ uint4 rope8(uint4 x, const float* cs /* 4 (cos, sin) pairs */) {
-  const float4 a = *reinterpret_cast<const float4*>(cs), b = *reinterpret_cast<const float4*>(cs + 4);
-  const float c[4] = {a.x, a.z, b.x, b.z}, sn[4] = {a.y, a.w, b.y, b.w};
-  const uint32_t in[4] = {x.x, x.y, x.z, x.w};
-  uint32_t o[4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const float x0 = __uint_as_float(in[i] << 16), x1 = __uint_as_float(in[i] & 0xffff0000u);
-    const float r0 = __fsub_rn(__fmul_rn(x0, c[i]), __fmul_rn(x1, sn[i]));
-    const float r1 = __fadd_rn(__fmul_rn(x0, sn[i]), __fmul_rn(x1, c[i]));
-    o[i] = pack_bf16x2(r0, r1);
-  }
-  return make_uint4(o[0], o[1], o[2], o[3]);
-}
-
 // ROPE: the kernel also does rope_kv_write_kernel's work for the new token at
 // position T - 1 -- every workgroup rotates its own queries from the raw
 // projection, and the one wavefront whose positions include T - 1 rotates the
@@ -332,18 +332,20 @@ inline int64_t attn_slices(int64_t T) { return (T + ATT_KPG - 1) / ATT_KPG; }
 
 }  // namespace aq
 
-extern "C" int aq_rope_kv_write(const void* qkv, const float* freqs, int64_t freqs_stride, const int64_t* page_table, int64_t P,
-                                int64_t pos, int64_t page_size, void* k_cache, void* v_cache, int64_t n_pages,
-                                void* q_out, int64_t B, int64_t Hq, int64_t Hkv, int64_t D, void* stream) {
+extern "C" int aq_rope_kv_write(const void* qkv, const float* freqs, int64_t freqs_stride, const int64_t* page_table,
+                                int64_t P, int64_t pos, int64_t S, int64_t page_size, void* k_cache, void* v_cache,
+                                int64_t n_pages, void* q_out, void* k_out, int64_t B, int64_t Hq, int64_t Hkv, int64_t D,
+                                void* stream) {
   if (D != aq::AD) return AQ_E_SHAPE;
-  if (B < 0 || Hq <= 0 || Hkv <= 0 || P <= 0 || pos < 0 || page_size <= 0 || n_pages <= 0) return AQ_E_SHAPE;
-  if (freqs_stride != 0 && freqs_stride < D) return AQ_E_SHAPE;
-  if (B == 0) return AQ_OK;
+  if (B < 0 || S < 0 || Hq <= 0 || Hkv <= 0 || P <= 0 || pos < 0 || page_size <= 0 || n_pages <= 0) return AQ_E_SHAPE;
+  if (freqs_stride != 0 && freqs_stride < S * D) return AQ_E_SHAPE;
+  if (B == 0 || S == 0) return AQ_OK;
   if (!qkv || !freqs || !page_table || !k_cache || !v_cache || !q_out) return AQ_E_NULL;
   if (aq::check_ptr16(qkv) || aq::check_ptr16(k_cache) || aq::check_ptr16(v_cache) || aq::check_ptr16(q_out) ||
-      (reinterpret_cast<uintptr_t>(freqs) & 7u) || (freqs_stride & 1))
+      aq::check_ptr16(freqs) || (freqs_stride & 3) || (k_out && aq::check_ptr16(k_out)))
     return AQ_E_ALIGN;
-  if (B * (Hq + 2 * Hkv) > (int64_t)0x7fffffff) return AQ_E_RANGE;
+  const int64_t chunks = B * S * (Hq + 2 * Hkv) * (aq::AD / 8);
+  if (chunks > (int64_t)0x7fffffff * 256) return AQ_E_RANGE;
   aq::RopeArgs a{};
   a.qkv = static_cast<const uint16_t*>(qkv);
   a.freqs = freqs;
@@ -352,14 +354,16 @@ extern "C" int aq_rope_kv_write(const void* qkv, const float* freqs, int64_t fre
   a.kc = static_cast<uint16_t*>(k_cache);
   a.vc = static_cast<uint16_t*>(v_cache);
   a.q_out = static_cast<uint16_t*>(q_out);
+  a.k_out = static_cast<uint16_t*>(k_out);
   a.P = P;
   a.pos = pos;
   a.page = page_size;
   a.n_pages = n_pages;
+  a.S = S;
   a.B = (int)B;
   a.Hq = (int)Hq;
   a.Hkv = (int)Hkv;
-  hipLaunchKernelGGL(aq::rope_kv_write_kernel, dim3((unsigned)(B * (Hq + 2 * Hkv))), dim3(64), 0,
+  hipLaunchKernelGGL(aq::rope_kv_write_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0,
                      static_cast<hipStream_t>(stream), a);
   return (int)hipGetLastError();
 }

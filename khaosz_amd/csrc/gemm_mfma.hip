@@ -491,38 +491,50 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(GemmArgs p) {
   auto store_all = [&](auto check_c, auto pair_c) {
     constexpr bool CHECK_M = decltype(check_c)::value;
     constexpr bool PAIR = (OUT == OUT_BF16) && decltype(pair_c)::value;
+    // lane part of the byte offset of column j; the pairing path stores at the even column of the pair
+    auto lane_offset = [&](int j) -> uint32_t {
+      const int cj = j * 32 + col;  // column inside the wavefront's 64
+      return nw + cj < N ? (uint32_t)rq * rowb + (uint32_t)(PAIR ? (cj & ~1) : cj) * ESZ + (PAIR && odd ? rowb : 0u)
+                         : OOB_OFFSET;
+    };
+    // The residual elements a lane will add, requested ahead of the arithmetic: all columns at once on
+    // the paired bf16 path (32 registers; the stores of one column would otherwise sit between the
+    // loads of the next and their use), column by column on the others.
+    constexpr int RPG = PAIR ? 2 : 4;  // loads per 4-row group: packed row pairs, or single elements
+    constexpr bool HOIST = PAIR;
+    uint32_t rr[TN][TME][4][RPG];
+    auto load_residual = [&](int j) {
+      const uint32_t vbase = lane_offset(j);
+#pragma unroll
+      for (int i = 0; i < TME; ++i)
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+#pragma unroll
+          for (int q = 0; q < RPG; ++q) {
+            const int r0 = i * 32 + g * 8;
+            const int rowq = PAIR ? 2 * q : q;
+            uint32_t vo = vbase;
+            if (CHECK_M && mw + r0 + rq + rowq + (PAIR && odd ? 1 : 0) >= M) vo = OOB_OFFSET;
+            if constexpr (OUT == OUT_F32 || PAIR)
+              rr[j][i][g][q] = __builtin_amdgcn_raw_buffer_load_b32(Rr, vo, (r0 + rowq) * rowb, 0);
+            else
+              rr[j][i][g][q] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(Rr, vo, (r0 + rowq) * rowb, 0);
+          }
+    };
+    if constexpr (OUT != OUT_I32 && HOIST) {
+      if (has_res) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) load_residual(j);
+      }
+    }
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
-      const int cj = j * 32 + col;  // column inside the wavefront's 64
-      const bool n_ok = nw + cj < N;
       float bn = 0.0f;
       if constexpr (!FP8 && OUT != OUT_I32)
         bn = !has_bias ? 0.0f : bias_bf16 ? bf16_bits_to_f32(bias_raw[j]) : __uint_as_float(bias_raw[j]);
-      // lane part of the byte offset; the pairing path stores at the even column of the pair
-      const uint32_t vbase =
-          n_ok ? (uint32_t)rq * rowb + (uint32_t)(PAIR ? (cj & ~1) : cj) * ESZ + (PAIR && odd ? rowb : 0u)
-               : OOB_OFFSET;
-      // the residual elements of this column, requested together ahead of the arithmetic
-      constexpr int RPG = PAIR ? 2 : 4;  // loads per 4-row group: packed row pairs, or single elements
-      uint32_t rr[TME][4][RPG];
-      if constexpr (OUT != OUT_I32) {
-        if (has_res) {
-#pragma unroll
-          for (int i = 0; i < TME; ++i)
-#pragma unroll
-            for (int g = 0; g < 4; ++g)
-#pragma unroll
-              for (int q = 0; q < RPG; ++q) {
-                const int r0 = i * 32 + g * 8;
-                const int rowq = PAIR ? 2 * q : q;
-                uint32_t vo = vbase;
-                if (CHECK_M && mw + r0 + rq + rowq + (PAIR && odd ? 1 : 0) >= M) vo = OOB_OFFSET;
-                if constexpr (OUT == OUT_F32 || PAIR)
-                  rr[i][g][q] = __builtin_amdgcn_raw_buffer_load_b32(Rr, vo, (r0 + rowq) * rowb, 0);
-                else
-                  rr[i][g][q] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(Rr, vo, (r0 + rowq) * rowb, 0);
-              }
-        }
+      const uint32_t vbase = lane_offset(j);
+      if constexpr (OUT != OUT_I32 && !HOIST) {
+        if (has_res) load_residual(j);
       }
 #pragma unroll
       for (int i = 0; i < TME; ++i) {
@@ -554,7 +566,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(GemmArgs p) {
               for (int q = 0; q < 4; ++q) {
                 uint32_t vo = vbase;
                 if (CHECK_M && mw + r0 + rq + q >= M) vo = OOB_OFFSET;
-                if (has_res) y[q] = __fadd_rn(y[q], __uint_as_float(rr[i][g][q]));
+                if (has_res) y[q] = __fadd_rn(y[q], __uint_as_float(rr[j][i][g][q]));
                 __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(y[q]), Cr, vo, (r0 + q) * rowb, STORE_WT);
               }
             } else if constexpr (PAIR) {
@@ -567,7 +579,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(GemmArgs p) {
                 // odd lane:  {other.hi, mine.hi} = row 2h+1, columns (c-1, c)
                 uint32_t pk = __builtin_amdgcn_perm(other, mine, perm_sel);
                 if (has_res) {  // rounded output + residual, rounded again: what a separate add gives
-                  const uint32_t r = rr[i][g][h];
+                  const uint32_t r = rr[j][i][g][h];
                   pk = pack_bf16x2(__fadd_rn(__uint_as_float(pk << 16), __uint_as_float(r << 16)),
                                    __fadd_rn(__uint_as_float(pk & 0xffff0000u), __uint_as_float(r & 0xffff0000u)));
                 }
@@ -581,7 +593,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(GemmArgs p) {
                 uint32_t vo = vbase;
                 if (CHECK_M && mw + r0 + rq + q >= M) vo = OOB_OFFSET;
                 uint32_t ob = f32_to_bf16_bits(y[q]);
-                if (has_res) ob = f32_to_bf16_bits(__fadd_rn(__uint_as_float(ob << 16), __uint_as_float(rr[i][g][q] << 16)));
+                if (has_res) ob = f32_to_bf16_bits(__fadd_rn(__uint_as_float(ob << 16), __uint_as_float(rr[j][i][g][q] << 16)));
                 __builtin_amdgcn_raw_buffer_store_b16((uint16_t)ob, Cr, vo, (r0 + q) * rowb, STORE_WT);
               }
             }

@@ -279,49 +279,61 @@ def gemv_w8a8_codes(xq, sx, wq, sw, bias=None, out_dtype=torch.bfloat16, residua
 
 
 def _rope_args(qkv, freqs, page_table, k_cache, v_cache, n_heads, n_kv_heads, what):
-    """Checks shared by the decode-step entry points; returns (qkv, freqs as float32, its batch
-    stride in floats, page_table), contiguous."""
+    """Checks shared by the rotary / KV-write entry points; returns (qkv [B, S, W], freqs as
+    float32, its batch stride in floats, page_table), contiguous."""
     _need_gpu(qkv, freqs, page_table, k_cache, v_cache)
-    B = qkv.shape[0]
     D = k_cache.shape[-1]
+    W = (n_heads + 2 * n_kv_heads) * D
     if qkv.dtype != torch.bfloat16 or k_cache.dtype != torch.bfloat16 or v_cache.dtype != torch.bfloat16:
         raise ValueError(f"{what} takes bfloat16 activations and caches")
-    if qkv.dim() != 2 or qkv.shape[1] != (n_heads + 2 * n_kv_heads) * D:
-        raise ValueError(f"qkv must be [B, {(n_heads + 2 * n_kv_heads) * D}], got {tuple(qkv.shape)}")
+    if qkv.dim() not in (2, 3) or qkv.shape[-1] != W:
+        raise ValueError(f"qkv must be [B, {W}] or [B, S, {W}], got {tuple(qkv.shape)}")
+    if qkv.dim() == 2:
+        qkv = qkv.unsqueeze(1)
+    B, S = qkv.shape[0], qkv.shape[1]
     if k_cache.dim() != 4 or k_cache.shape != v_cache.shape or k_cache.shape[2] != n_kv_heads:
         raise ValueError("caches must be [n_pages, page, Hkv, D] and alike")
     if not (k_cache.is_contiguous() and v_cache.is_contiguous()):
         raise ValueError("caches must be contiguous")
     fr = torch.view_as_real(freqs) if freqs.is_complex() else freqs
-    if fr.dtype != torch.float32 or fr.shape[0] != B or fr.numel() // max(B, 1) != D or fr.stride(-1) != 1:
-        raise ValueError(f"freqs must be complex64 [B, {D // 2}] or float32 [B, {D // 2}, 2]")
+    if fr.dtype != torch.float32 or fr.shape[0] != B or fr.numel() // max(B, 1) != S * D or fr.stride(-1) != 1:
+        raise ValueError(f"freqs must be complex64 [B, (S,) {D // 2}] or float32 [B, (S,) {D // 2}, 2]")
     if B > 1 and fr.stride(0) == 0:      # one table broadcast to every sequence: no copy
         fr_stride, fr = 0, fr[0].contiguous()
     else:
-        fr = fr.reshape(B, D).contiguous()
-        fr_stride = D
+        fr = fr.reshape(B, S * D).contiguous()
+        fr_stride = S * D
+    if fr.data_ptr() % 16:
+        fr = fr.clone()
     if page_table.dtype != torch.int64 or page_table.dim() != 2 or page_table.shape[0] != B:
         raise ValueError("page_table must be int64 [B, P]")
     return qkv.contiguous(), fr, fr_stride, page_table.contiguous()
 
 
 def rope_kv_write(qkv: torch.Tensor, freqs: torch.Tensor, page_table: torch.Tensor, pos: int, k_cache: torch.Tensor,
-                  v_cache: torch.Tensor, n_heads: int, n_kv_heads: int) -> torch.Tensor:
-    """One new token per sequence: rotate q and k of ``qkv [B, (Hq + 2 Hkv) * 128]`` by ``freqs``
-    (complex64 ``[B, 64]`` or float32 ``[B, 64, 2]``), write k and v into the paged caches
-    ``[n_pages, page, Hkv, 128]`` at logical position ``pos``; returns the rotated ``q [B, Hq, 128]``."""
+                  v_cache: torch.Tensor, n_heads: int, n_kv_heads: int, return_k: bool = False):
+    """New tokens of every sequence -- ``qkv [B, (Hq + 2 Hkv) * 128]`` (one each) or ``[B, S, ...]``:
+    rotate q and k by ``freqs`` (complex64 ``[B, (S,) 64]`` or float32 ``[B, (S,) 64, 2]``), write k and
+    v into the paged caches ``[n_pages, page, Hkv, 128]`` at logical positions ``pos .. pos + S - 1``;
+    returns the rotated ``q [B, (S,) Hq, 128]``, and with ``return_k`` also the rotated
+    ``k [B, (S,) Hkv, 128]``."""
+    one = qkv.dim() == 2
     qkv, fr, fr_stride, page_table = _rope_args(qkv, freqs, page_table, k_cache, v_cache, n_heads, n_kv_heads,
                                                 "rope_kv_write")
-    B, D = qkv.shape[0], k_cache.shape[-1]
-    q = torch.empty((B, n_heads, D), dtype=torch.bfloat16, device=qkv.device)
-    if B:
+    B, S, D = qkv.shape[0], qkv.shape[1], k_cache.shape[-1]
+    q = torch.empty((B, S, n_heads, D), dtype=torch.bfloat16, device=qkv.device)
+    k = torch.empty((B, S, n_kv_heads, D), dtype=torch.bfloat16, device=qkv.device) if return_k else None
+    if B and S:
         with torch.cuda.device(qkv.device):
             rc = _abi.load().aq_rope_kv_write(qkv.data_ptr(), fr.data_ptr(), fr_stride, page_table.data_ptr(),
-                                              page_table.shape[1],
-                                              int(pos), k_cache.shape[1], k_cache.data_ptr(), v_cache.data_ptr(),
-                                              k_cache.shape[0], q.data_ptr(), B, n_heads, n_kv_heads, D, _stream(qkv))
+                                              page_table.shape[1], int(pos), S, k_cache.shape[1], k_cache.data_ptr(),
+                                              v_cache.data_ptr(), k_cache.shape[0], q.data_ptr(),
+                                              k.data_ptr() if return_k else None, B, n_heads, n_kv_heads, D,
+                                              _stream(qkv))
         _abi.check(rc, "aq_rope_kv_write")
-    return q
+    if one:
+        q, k = q.squeeze(1), (k.squeeze(1) if return_k else None)
+    return (q, k) if return_k else q
 
 
 def _attn_workspace(workspace, need, dev):
@@ -339,6 +351,8 @@ def rope_paged_attn_decode(qkv: torch.Tensor, freqs: torch.Tensor, page_table: t
     """``rope_kv_write`` at position ``total_len - 1`` and ``paged_attn_decode`` over ``total_len``
     positions as one launch (plus the small merge launch for long sequences): same caches and
     outputs, bit for bit.  Returns the attention output ``[B, Hq, 128]``."""
+    if qkv.dim() != 2:
+        raise ValueError(f"one new token per sequence: qkv must be [B, W], got {tuple(qkv.shape)}")
     qkv, fr, fr_stride, page_table = _rope_args(qkv, freqs, page_table, k_cache, v_cache, n_heads, n_kv_heads,
                                                 "rope_paged_attn_decode")
     B, D = qkv.shape[0], k_cache.shape[-1]

@@ -43,6 +43,43 @@ def test_rope_kv_write_bit_exact(oracle, B, Hq, Hkv, page, pos):
     assert np.array_equal(_bits(kd), kb) and np.array_equal(_bits(vd), vb)
 
 
+@pytest.mark.parametrize("B,S,Hq,Hkv,page,pos", [(1, 5, 1, 1, 4, 0), (3, 21, 4, 2, 8, 13), (2, 130, 16, 4, 64, 0)])
+def test_rope_kv_write_several_tokens_bit_exact(oracle, B, S, Hq, Hkv, page, pos):
+    """A prompt (or a chunk of one) in one launch: the oracle applied token by token."""
+    _say("rope_kv_write seq", B, S, Hq, Hkv, page, pos)
+    D = 128
+    P = (pos + S + page - 1) // page + 1
+    n_pages = B * P + 3
+    g = torch.Generator().manual_seed(B * 100 + S)
+    qkv = torch.randn(B, S, (Hq + 2 * Hkv) * D, generator=g).to(torch.bfloat16)
+    ang = torch.rand(B, S, D // 2, generator=g) * 6.28
+    freqs = torch.polar(torch.ones_like(ang), ang)
+    table = torch.randperm(n_pages, generator=g)[:B * P].view(B, P)
+    if B > 2:
+        table[1, (pos + 3) // page] = -1                # tokens of that page are dropped
+    kc = torch.randn(n_pages, page, Hkv, D, generator=g).to(torch.bfloat16)
+    vc = torch.randn(n_pages, page, Hkv, D, generator=g).to(torch.bfloat16)
+    kb, vb = _bits(kc), _bits(vc)
+    fr = torch.view_as_real(freqs).numpy()
+    qo = np.stack([oracle.c_rope_kv_write(_bits(qkv[:, s]), np.ascontiguousarray(fr[:, s]), table.numpy(), pos + s,
+                                          kb, vb, Hq, Hkv) for s in range(S)], axis=1)
+    kd, vd = kc.to(DEV), vc.to(DEV)
+    q, k = ops.rope_kv_write(qkv.to(DEV), freqs.to(DEV), table.to(DEV), pos, kd, vd, Hq, Hkv, return_k=True)
+    assert q.shape == (B, S, Hq, D) and k.shape == (B, S, Hkv, D)
+    assert np.array_equal(_bits(q), qo.reshape(B, S, Hq, D))
+    assert np.array_equal(_bits(kd), kb) and np.array_equal(_bits(vd), vb)
+    # the returned keys are what went into the mapped slots
+    mapped = table[torch.arange(B)[:, None], (pos + torch.arange(S))[None, :] // page] >= 0
+    slot = (table[torch.arange(B)[:, None], (pos + torch.arange(S))[None, :] // page].clamp(min=0),
+            ((pos + torch.arange(S)) % page)[None, :].expand(B, -1))
+    assert torch.equal(k.cpu()[mapped], kd.cpu()[slot[0], slot[1]][mapped])
+    # one table shared by all sequences (batch stride 0)
+    shared = freqs[:1].expand(B, -1, -1)
+    qs = ops.rope_kv_write(qkv.to(DEV), shared.to(DEV), table.to(DEV), pos, kd, vd, Hq, Hkv)
+    qw = ops.rope_kv_write(qkv.to(DEV), shared.contiguous().to(DEV), table.to(DEV), pos, kd, vd, Hq, Hkv)
+    assert torch.equal(qs, qw)
+
+
 @pytest.mark.parametrize("B,Hq,Hkv,page,T", [(1, 1, 1, 4, 1), (2, 8, 2, 16, 70), (8, 16, 4, 64, 576), (3, 8, 1, 16, 1000),
                                               (2, 4, 2, 64, 513), (1, 2, 2, 8, 64), (2, 2, 1, 4, 65), (1, 4, 4, 32, 256),
                                               (2, 16, 2, 16, 257), (40, 8, 8, 16, 300), (1, 8, 1, 64, 5000)])

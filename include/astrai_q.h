@@ -145,12 +145,12 @@ int aq_rmsnorm_quant_rowwise_i8(const void *x, int x_dtype, const void *gamma, i
  * Fixed arithmetic: silu(g) = g / (1 + e), e = exp(-g) from a fixed sequence of
  * fused multiply-adds (degree-5 polynomial after range reduction; the oracle
  * repeats it bit for bit), correctly rounded divide, one rounded product.
- * F a multiple of 16 and at most 6144 (bf16) / 3072 (fp32) elements. */
+ * F a multiple of 16 and at most 8192 (bf16) / 4096 (fp32) elements. */
 int aq_swiglu_quant_rowwise_i8(const void *ug, int dtype, int64_t M, int64_t F, int64_t ld,
                                int8_t *q, float *scale, void *stream);
 
 /* ---- attention around the paged KV cache (what sits between the qkv and the
- * output projection; bf16, head dimension 128).
+ * output projection; bf16, head dimension D = 64 or 128).
  *
  * aq_rope_kv_write: for the S new tokens of each of B sequences (S = 1 at
  * decode, the prompt length at prefill), rotate the q and k heads of
@@ -171,7 +171,7 @@ int aq_swiglu_quant_rowwise_i8(const void *ug, int dtype, int64_t M, int64_t F, 
  * 0 .. total_len-1 of each sequence, read through page_table [B, P] in place --
  * replaces Storage.gather (cache.py:254-274), repeat_kv (attention.py:15-23) and
  * scaled_dot_product_attention (attention.py:98-100) for a step without padding
- * mask.  Query heads h*G .. h*G+G-1 use KV head h, G = Hq / Hkv in {1, 2, 4, 8}.
+ * mask.  Query heads h*G .. h*G+G-1 use KV head h, G = Hq / Hkv in {1, 2, 3, 4, 6, 8}.
  * Positions whose page is unmapped count as zero keys and values (what gather's
  * zero fill gives).  fp32 scores and sums; results within bf16 rounding of the
  * reference flow, not bit-identical to it (summation order, exp2).

@@ -180,9 +180,11 @@ class GQA(nn.Module):
         cached length (the additive mask is all zeros).  Several new tokens (prefill) get the
         rotation and the page writes as one launch (``ops.rope_kv_write``) in front of the stock
         attention, which then reads the new keys directly and shares KV heads without
-        repeating them.  Needs the fused q/k/v projection, bf16 and head dimension 128.
+        repeating them.  Needs the fused q/k/v projection, bf16, head dimension 64 or 128 and
+        1, 2, 3, 4, 6 or 8 query heads per KV head.
         Outputs agree within bf16 rounding."""
-        if self._qkv is not None and self.head_dim == 128 and self.n_heads // self.n_kv_heads in (1, 2, 4, 8):
+        if (self._qkv is not None and self.head_dim in (64, 128)
+                and self.n_heads // self.n_kv_heads in (1, 2, 3, 4, 6, 8)):
             self._decode_attention = True
         return self._decode_attention
 

@@ -1,27 +1,26 @@
-// Decode-step attention around the quantized projections, reading the paged KV
-// cache in place: the reference gathers every page into a contiguous
-// [B, T, Hkv, D] copy, repeats the KV heads and calls a generic attention per
-// layer and per step (astrai/model/components/attention.py:83-103,
-// astrai/inference/core/cache.py:254-274).  Two kernels replace that for a step
-// with one new token per sequence:
+// Attention around the quantized projections, on the paged KV cache in place:
+// the reference rotates q and k with complex multiplies, writes k/v page by
+// page, gathers every page into a contiguous [B, T, Hkv, D] copy, repeats the
+// KV heads and calls a generic attention, per layer and per step
+// (astrai/model/components/attention.py:83-103,
+// astrai/inference/core/cache.py:216-274).  Kernels here:
 //
 //   rope_kv_write   rotates q and k of the new tokens (interleaved pairs, fp32,
 //                   rope.py:26-33), stores q, and writes k and v into their page
 //                   slots (cache.py:216-252) -- one token per sequence at decode,
 //                   the whole prompt at prefill;
-//   paged_attn      softmax(q K^T / sqrt(D)) V over the pages of each sequence,
-//                   all query heads of a KV head in one workgroup (grouped-query
-//                   attention without materialising the repeated heads,
-//                   attention.py:15-23).
+//   paged_attn      softmax(q K^T / sqrt(D)) V for one query token per sequence
+//                   over the pages of that sequence, all query heads of a KV
+//                   head in one workgroup (grouped-query attention without
+//                   materialising the repeated heads, attention.py:15-23);
+//                   optionally doing rope_kv_write's work for that token itself.
 //
-// bf16 tensors, head dimension 128, fp32 arithmetic.  Unmapped pages (table
-// entry < 0 or out of range) are skipped on write and read as zero keys and
-// values, as the reference's gather does.
+// bf16 tensors, head dimension 64 or 128, fp32 arithmetic.  Unmapped pages
+// (table entry < 0 or out of range) are skipped on write and read as zero keys
+// and values, as the reference's gather does.
 #include "aq_common.h"
 
 namespace aq {
-
-constexpr int AD = 128;          // head dimension
 
 // Rotates 8 consecutive elements (4 interleaved pairs): (x0 + i x1)(c + i s) with four rounded
 // products, one rounded difference and one rounded sum per pair.
@@ -50,31 +49,32 @@ struct RopeArgs {
   uint16_t* q_out;       // [B, S, Hq, D]
   uint16_t* k_out;       // [B, S, Hkv, D] rotated keys, or null
   int64_t P, pos, page, n_pages, S;
-  int B, Hq, Hkv;
+  int B, Hq, Hkv, D;
 };
 
 // one thread per 16-byte chunk (8 elements) of a head vector of a token
 __global__ __launch_bounds__(256) void rope_kv_write_kernel(RopeArgs p) {
   const int64_t heads = p.Hq + 2 * p.Hkv;
+  const int cph = p.D / 8;  // chunks per head vector
   const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (c >= (int64_t)p.B * p.S * heads * (AD / 8)) return;
-  const int ch = (int)(c & 15);
-  const int64_t hv = c >> 4, tokn = hv / heads;
+  if (c >= (int64_t)p.B * p.S * heads * cph) return;
+  const int ch = (int)(c % cph);
+  const int64_t hv = c / cph, tokn = hv / heads;
   const int h = (int)(hv % heads);
   const int64_t b = tokn / p.S, s = tokn % p.S;
-  uint4 x = *reinterpret_cast<const uint4*>(p.qkv + hv * AD + ch * 8);
-  if (h < p.Hq + p.Hkv) x = rope8(x, p.freqs + b * p.freqs_stride + s * AD + ch * 8);  // v heads do not rotate
+  uint4 x = *reinterpret_cast<const uint4*>(p.qkv + hv * p.D + ch * 8);
+  if (h < p.Hq + p.Hkv) x = rope8(x, p.freqs + b * p.freqs_stride + s * p.D + ch * 8);  // v heads do not rotate
   if (h < p.Hq) {
-    *reinterpret_cast<uint4*>(p.q_out + (tokn * p.Hq + h) * AD + ch * 8) = x;
+    *reinterpret_cast<uint4*>(p.q_out + (tokn * p.Hq + h) * p.D + ch * 8) = x;
     return;
   }
   const bool is_k = h < p.Hq + p.Hkv;
   const int kvh = is_k ? h - p.Hq : h - p.Hq - p.Hkv;
-  if (is_k && p.k_out) *reinterpret_cast<uint4*>(p.k_out + (tokn * p.Hkv + kvh) * AD + ch * 8) = x;
+  if (is_k && p.k_out) *reinterpret_cast<uint4*>(p.k_out + (tokn * p.Hkv + kvh) * p.D + ch * 8) = x;
   const int64_t pos = p.pos + s, lp = pos / p.page;
   const int64_t phys = lp < p.P ? p.table[b * p.P + lp] : -1;
   if (phys < 0 || phys >= p.n_pages) return;  // unmapped: the token is dropped, as in the reference
-  uint16_t* dst = (is_k ? p.kc : p.vc) + ((phys * p.page + pos % p.page) * p.Hkv + kvh) * AD + ch * 8;
+  uint16_t* dst = (is_k ? p.kc : p.vc) + ((phys * p.page + pos % p.page) * p.Hkv + kvh) * p.D + ch * 8;
   *reinterpret_cast<uint4*>(dst) = x;
 }
 
@@ -84,7 +84,7 @@ struct AttnArgs {
   const uint16_t* vc;
   const int64_t* table;  // [B, P]
   uint16_t* out;         // [B, Hq, D]
-  float* ws;             // partial results [B, Hq, NS, ATT_PART] when NS > 1
+  float* ws;             // partial results [B, Hq, NS, D + 4] when NS > 1
   const uint16_t* qkv;   // ROPE kernels: [B, (Hq + 2 Hkv) * D] projections of the new token (position T - 1)
   const float* freqs;    // ROPE kernels: its rotary table, as in RopeArgs
   uint16_t* kc_w;        // ROPE kernels: the caches again, writable
@@ -96,16 +96,18 @@ struct AttnArgs {
 };
 
 constexpr int ATT_WAVES = 4;
-constexpr int ATT_NL = 16;                   // row loads per wavefront, 4 rows each
-constexpr int ATT_KPW = 4 * ATT_NL;          // positions per wavefront
+constexpr int ATT_KPW = 64;                  // positions per wavefront
 constexpr int ATT_KPG = ATT_WAVES * ATT_KPW; // positions per workgroup
-constexpr int ATT_PART = AD + 4;  // numerator[AD], maximum, denominator, 2 floats of padding
+constexpr int ATT_MAX_D = 128;
 
-__device__ __forceinline__ float row16_sum(float v) {  // sum over each row of 16 lanes, result in all of them
+// sum over each group of LANES (8 or 16) consecutive lanes, result in all of them
+template <int LANES>
+__device__ __forceinline__ float lanes_sum(float v) {
   v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xf, 0xf, false));   // quad_perm [1,0,3,2]
   v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xf, 0xf, false));   // quad_perm [2,3,0,1]
   v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xf, 0xf, false));  // row_half_mirror
-  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xf, 0xf, false));  // row_mirror
+  if constexpr (LANES == 16)
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xf, 0xf, false));  // row_mirror
   return v;
 }
 
@@ -115,19 +117,20 @@ __device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float c) {
 }
 
 // Workgroup = one (sequence, KV head, slice of the cached positions): the G
-// query heads of the KV head share every K and V byte.  A wavefront owns 4*NL
-// consecutive positions, a workgroup 16*NL; the NS slices of a sequence run as
+// query heads of the KV head share every K and V byte.  A wavefront owns 64
+// consecutive positions, a workgroup 256; the NS slices of a sequence run as
 // separate workgroups so that a decode batch of a few sequences still spreads
 // over the device.  Rows are read 16 bytes per lane: a load instruction covers
-// 4 whole 256-byte rows (lane = 16*key + chunk), NL of them for K and NL for V
-// are requested before anything is computed.
+// RPL = 1024 / (2 D) whole rows (lane = CPR * key + chunk, CPR = D / 8 chunks
+// per row), 64 / RPL of them for K and as many for V are requested before
+// anything is computed.
 //   scores   every lane dots its 8 dimensions with the G queries (packed bf16
-//            dot product, fp32 accumulation), a DPP butterfly sums the 16 lanes
+//            dot product, fp32 accumulation), a DPP butterfly sums the CPR lanes
 //            of a row, and lane (chunk = i, key = j) keeps the score of key
-//            4i + j of the batch -- one key per lane for the softmax;
+//            RPL * i + j of the batch -- one key per lane for the softmax;
 //   softmax  maximum and denominator across the wavefront, probabilities to LDS;
 //   values   lane accumulates p * V over the keys it loaded (8 dimensions x G
-//            heads), the four key groups are summed with two xor shuffles.
+//            heads), the RPL key groups are summed with xor shuffles.
 // The wavefronts' (maximum, denominator, numerator) are merged through LDS and
 // either normalised into the output (NS == 1) or left in the workspace for
 // attn_merge_kernel.
@@ -137,16 +140,21 @@ __device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float c) {
 // new key, stores it and the new value into their page slot and uses them from
 // registers instead of what it read from the cache.  Same roundings, so caches
 // and outputs are the bits the two separate launches give.
-template <int G, bool ROPE>
+template <int G, int D, bool ROPE>
 __global__ __launch_bounds__(ATT_WAVES * 64) void paged_attn_decode_kernel(AttnArgs p) {
-  constexpr int NL = ATT_NL, KPW = ATT_KPW, KPG = ATT_KPG;
+  constexpr int CPR = D / 8;     // 16-byte chunks per row: 16 or 8
+  constexpr int RPL = 64 / CPR;  // rows per load instruction: 4 or 8
+  constexpr int NL = 64 / RPL;   // loads per wavefront (= CPR)
+  constexpr int KPW = ATT_KPW, KPG = ATT_KPG;
   constexpr int ATT_THREADS = ATT_WAVES * 64;
+  constexpr int PART = D + 4;    // numerator[D], maximum, denominator, 2 floats of padding
+  static_assert(D == 64 || D == 128, "head dimension");
   __shared__ __align__(16) float p_s[ATT_WAVES][KPW][G];
   __shared__ float m_s[ATT_WAVES][G], l_s[ATT_WAVES][G];
-  __shared__ __align__(16) float acc_s[ATT_WAVES][G][AD];
+  __shared__ __align__(16) float acc_s[ATT_WAVES][G][D];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int sub = lane >> 4, ch = lane & 15;  // key within a load, 16-byte chunk of the row
+  const int sub = lane / CPR, ch = lane % CPR;  // key within a load, 16-byte chunk of the row
   // the KV heads of one slice are neighbours in the launch order: together they read whole
   // [position][Hkv][D] stretches of the pages at about the same time
   const int kvh = blockIdx.x % p.Hkv, bs = blockIdx.x / p.Hkv;
@@ -163,14 +171,14 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void paged_attn_decode_kernel(AttnA
     for (int e = 0; e < 8; ++e) acc[g][e] = 0.0f;
   }
   if (t0 < T) {  // wavefront-uniform
-    // lane L < KPW looks up the row of position t0 + L (element offset, -1: unmapped or past T)
+    // lane L looks up the row of position t0 + L (element offset, -1: unmapped or past T)
     int64_t row = -1;
     {
       const int64_t t = t0 + lane;
-      if (lane < KPW && t < T) {
+      if (t < T) {
         const int64_t lp = t / p.page;
         const int64_t phys = lp < p.P ? p.table[(int64_t)b * p.P + lp] : -1;
-        if (phys >= 0 && phys < p.n_pages) row = ((phys * p.page + t % p.page) * p.Hkv + kvh) * AD;
+        if (phys >= 0 && phys < p.n_pages) row = ((phys * p.page + t % p.page) * p.Hkv + kvh) * D;
       }
     }
     uint4 qv[G];  // this lane's 8 dimensions of each query
@@ -178,24 +186,24 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void paged_attn_decode_kernel(AttnA
     const bool has_new = ROPE && T - 1 >= t0 && T - 1 < t0 + KPW;  // wavefront-uniform
     if constexpr (ROPE) {
       const int64_t heads = p.Hq + 2 * p.Hkv;
-      const uint16_t* tok = p.qkv + (int64_t)b * heads * AD;
+      const uint16_t* tok = p.qkv + (int64_t)b * heads * D;
       const float* cs = p.freqs + (int64_t)b * p.freqs_stride + ch * 8;
 #pragma unroll
       for (int g = 0; g < G; ++g)
-        qv[g] = rope8(*reinterpret_cast<const uint4*>(tok + (int64_t)(kvh * G + g) * AD + ch * 8), cs);
+        qv[g] = rope8(*reinterpret_cast<const uint4*>(tok + (int64_t)(kvh * G + g) * D + ch * 8), cs);
       if (has_new) {
-        knew = rope8(*reinterpret_cast<const uint4*>(tok + (int64_t)(p.Hq + kvh) * AD + ch * 8), cs);
-        vnew = *reinterpret_cast<const uint4*>(tok + (int64_t)(p.Hq + p.Hkv + kvh) * AD + ch * 8);
+        knew = rope8(*reinterpret_cast<const uint4*>(tok + (int64_t)(p.Hq + kvh) * D + ch * 8), cs);
+        vnew = *reinterpret_cast<const uint4*>(tok + (int64_t)(p.Hq + p.Hkv + kvh) * D + ch * 8);
       }
     } else {
 #pragma unroll
       for (int g = 0; g < G; ++g)
-        qv[g] = *reinterpret_cast<const uint4*>(p.q + ((int64_t)b * p.Hq + kvh * G + g) * AD + ch * 8);
+        qv[g] = *reinterpret_cast<const uint4*>(p.q + ((int64_t)b * p.Hq + kvh * G + g) * D + ch * 8);
     }
     uint4 kv[NL], vv[NL];
 #pragma unroll
     for (int i = 0; i < NL; ++i) {
-      const int src = i * 4 + sub;
+      const int src = i * RPL + sub;
       const int lo = __shfl((int)(uint32_t)row, src, 64), hi = __shfl((int)(row >> 32), src, 64);
       const int64_t r = ((int64_t)hi << 32) | (uint32_t)lo;
       kv[i] = make_uint4(0, 0, 0, 0);
@@ -224,13 +232,13 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void paged_attn_decode_kernel(AttnA
         d = dot2_bf16(kv[i].y, qv[g].y, d);
         d = dot2_bf16(kv[i].z, qv[g].z, d);
         d = dot2_bf16(kv[i].w, qv[g].w, d);
-        d = row16_sum(d);
+        d = lanes_sum<CPR>(d);
         if (ch == i) sc[g] = d;
       }
     }
-    // ---- softmax over the wavefront's positions: this lane owns position t0 + 4*ch + sub
-    const int own = ch * 4 + sub;
-    const bool valid = ch < NL && t0 + own < T;
+    // ---- softmax over the wavefront's positions: this lane owns position t0 + RPL * ch + sub
+    const int own = ch * RPL + sub;
+    const bool valid = t0 + own < T;
 #pragma unroll
     for (int g = 0; g < G; ++g) {
       const float sv = valid ? sc[g] * p.scale_log2e : -INFINITY;
@@ -243,7 +251,7 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void paged_attn_decode_kernel(AttnA
       for (int off = 32; off > 0; off >>= 1) ps += __shfl_xor(ps, off, 64);
       m[g] = bm;
       l[g] = ps;
-      if (ch < NL) p_s[wave][own][g] = pv;
+      p_s[wave][own][g] = pv;
     }
     __builtin_amdgcn_s_waitcnt(0xc07f);  // this wavefront's LDS writes are done (wavefront-private region)
     asm volatile("" ::: "memory");
@@ -261,7 +269,7 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void paged_attn_decode_kernel(AttnA
       v8[7] = __uint_as_float(vv[i].w & 0xffff0000u);
 #pragma unroll
       for (int g = 0; g < G; ++g) {
-        const float pj = p_s[wave][i * 4 + sub][g];
+        const float pj = p_s[wave][i * RPL + sub][g];
 #pragma unroll
         for (int e = 0; e < 8; ++e) acc[g][e] = __builtin_fmaf(pj, v8[e], acc[g][e]);
       }
@@ -270,8 +278,8 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void paged_attn_decode_kernel(AttnA
     for (int g = 0; g < G; ++g)
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        acc[g][e] += __shfl_xor(acc[g][e], 16, 64);
-        acc[g][e] += __shfl_xor(acc[g][e], 32, 64);
+#pragma unroll
+        for (int off = CPR; off < 64; off <<= 1) acc[g][e] += __shfl_xor(acc[g][e], off, 64);
       }
   }
   // ---- merge the wavefronts' partial results
@@ -287,8 +295,8 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void paged_attn_decode_kernel(AttnA
     }
   }
   __syncthreads();
-  for (int i = tid; i < G * AD / 2; i += ATT_THREADS) {
-    const int g = i / (AD / 2), d = (i % (AD / 2)) * 2;  // dimensions d, d + 1
+  for (int i = tid; i < G * D / 2; i += ATT_THREADS) {
+    const int g = i / (D / 2), d = (i % (D / 2)) * 2;  // dimensions d, d + 1
     float mm = -INFINITY;
 #pragma unroll
     for (int w = 0; w < ATT_WAVES; ++w) mm = fmaxf(mm, m_s[w][g]);
@@ -302,33 +310,37 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void paged_attn_decode_kernel(AttnA
     }
     const int64_t head = (int64_t)b * p.Hq + kvh * G + g;
     if (p.NS == 1) {
-      store_wt(reinterpret_cast<uint32_t*>(p.out + head * AD + d), pack_bf16x2(n0 / den, n1 / den));
+      store_wt(reinterpret_cast<uint32_t*>(p.out + head * D + d), pack_bf16x2(n0 / den, n1 / den));
     } else {
-      float* part = p.ws + (head * p.NS + split) * ATT_PART;
+      float* part = p.ws + (head * p.NS + split) * PART;
       store_wt(reinterpret_cast<uint2*>(part + d), make_uint2(__float_as_uint(n0), __float_as_uint(n1)));
-      if (d == 0) store_wt(reinterpret_cast<uint2*>(part + AD), make_uint2(__float_as_uint(mm), __float_as_uint(den)));
+      if (d == 0) store_wt(reinterpret_cast<uint2*>(part + D), make_uint2(__float_as_uint(mm), __float_as_uint(den)));
     }
   }
 }
 
-// Combines the NS slices of one (sequence, query head): thread = dimension pair.
-__global__ __launch_bounds__(AD / 2) void attn_merge_kernel(const float* ws, uint16_t* out, int NS) {
-  const int d = threadIdx.x * 2;
-  const float* part = ws + (int64_t)blockIdx.x * NS * ATT_PART;
+// Combines the NS slices of one (sequence, query head): thread = dimension pair (D / 2 threads).
+__global__ __launch_bounds__(ATT_MAX_D / 2) void attn_merge_kernel(const float* ws, uint16_t* out, int NS, int D) {
+  const int d = threadIdx.x * 2, part_sz = D + 4;
+  const float* part = ws + (int64_t)blockIdx.x * NS * part_sz;
   float mm = -INFINITY;
-  for (int s = 0; s < NS; ++s) mm = fmaxf(mm, part[s * ATT_PART + AD]);  // slice 0 always holds a position
+  for (int s = 0; s < NS; ++s) mm = fmaxf(mm, part[s * part_sz + D]);  // slice 0 always holds a position
   float n0 = 0.0f, n1 = 0.0f, den = 0.0f;
   for (int s = 0; s < NS; ++s) {
-    const float a = exp2f(part[s * ATT_PART + AD] - mm);
-    const float2 v = *reinterpret_cast<const float2*>(part + s * ATT_PART + d);
+    const float a = exp2f(part[s * part_sz + D] - mm);
+    const float2 v = *reinterpret_cast<const float2*>(part + s * part_sz + d);
     n0 = __builtin_fmaf(v.x, a, n0);
     n1 = __builtin_fmaf(v.y, a, n1);
-    den = __builtin_fmaf(part[s * ATT_PART + AD + 1], a, den);
+    den = __builtin_fmaf(part[s * part_sz + D + 1], a, den);
   }
-  store_wt(reinterpret_cast<uint32_t*>(out + (int64_t)blockIdx.x * AD + d), pack_bf16x2(n0 / den, n1 / den));
+  store_wt(reinterpret_cast<uint32_t*>(out + (int64_t)blockIdx.x * D + d), pack_bf16x2(n0 / den, n1 / den));
 }
 
 inline int64_t attn_slices(int64_t T) { return (T + ATT_KPG - 1) / ATT_KPG; }
+// sized for the larger head dimension, so that the size does not depend on D
+inline int64_t attn_workspace_bytes(int64_t B, int64_t Hq, int64_t ns) {
+  return B * Hq * ns * (ATT_MAX_D + 4) * (int64_t)sizeof(float);
+}
 
 }  // namespace aq
 
@@ -336,7 +348,7 @@ extern "C" int aq_rope_kv_write(const void* qkv, const float* freqs, int64_t fre
                                 int64_t P, int64_t pos, int64_t S, int64_t page_size, void* k_cache, void* v_cache,
                                 int64_t n_pages, void* q_out, void* k_out, int64_t B, int64_t Hq, int64_t Hkv, int64_t D,
                                 void* stream) {
-  if (D != aq::AD) return AQ_E_SHAPE;
+  if (D != 64 && D != 128) return AQ_E_SHAPE;
   if (B < 0 || S < 0 || Hq <= 0 || Hkv <= 0 || P <= 0 || pos < 0 || page_size <= 0 || n_pages <= 0) return AQ_E_SHAPE;
   if (freqs_stride != 0 && freqs_stride < S * D) return AQ_E_SHAPE;
   if (B == 0 || S == 0) return AQ_OK;
@@ -344,7 +356,7 @@ extern "C" int aq_rope_kv_write(const void* qkv, const float* freqs, int64_t fre
   if (aq::check_ptr16(qkv) || aq::check_ptr16(k_cache) || aq::check_ptr16(v_cache) || aq::check_ptr16(q_out) ||
       aq::check_ptr16(freqs) || (freqs_stride & 3) || (k_out && aq::check_ptr16(k_out)))
     return AQ_E_ALIGN;
-  const int64_t chunks = B * S * (Hq + 2 * Hkv) * (aq::AD / 8);
+  const int64_t chunks = B * S * (Hq + 2 * Hkv) * (D / 8);
   if (chunks > (int64_t)0x7fffffff * 256) return AQ_E_RANGE;
   aq::RopeArgs a{};
   a.qkv = static_cast<const uint16_t*>(qkv);
@@ -363,6 +375,7 @@ extern "C" int aq_rope_kv_write(const void* qkv, const float* freqs, int64_t fre
   a.B = (int)B;
   a.Hq = (int)Hq;
   a.Hkv = (int)Hkv;
+  a.D = (int)D;
   hipLaunchKernelGGL(aq::rope_kv_write_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0,
                      static_cast<hipStream_t>(stream), a);
   return (int)hipGetLastError();
@@ -371,7 +384,15 @@ extern "C" int aq_rope_kv_write(const void* qkv, const float* freqs, int64_t fre
 extern "C" int64_t aq_paged_attn_decode_workspace_bytes(int64_t B, int64_t Hq, int64_t Hkv, int64_t total_len) {
   if (B <= 0 || Hq <= 0 || Hkv <= 0 || total_len <= 0) return 0;
   const int64_t ns = aq::attn_slices(total_len);
-  return ns == 1 ? 0 : B * Hq * ns * aq::ATT_PART * (int64_t)sizeof(float);
+  return ns == 1 ? 0 : aq::attn_workspace_bytes(B, Hq, ns);
+}
+
+template <int G, int D>
+static void attn_launch(bool rope, dim3 grid, dim3 block, hipStream_t st, const aq::AttnArgs& a) {
+  if (rope)
+    hipLaunchKernelGGL((aq::paged_attn_decode_kernel<G, D, true>), grid, block, 0, st, a);
+  else
+    hipLaunchKernelGGL((aq::paged_attn_decode_kernel<G, D, false>), grid, block, 0, st, a);
 }
 
 // q == nullptr: the fused form, queries and the new token come from qkv / freqs.
@@ -380,13 +401,16 @@ static int attn_decode(const void* q, const void* qkv, const float* freqs, int64
                        int64_t n_pages, float scale, void* out, int64_t B, int64_t Hq, int64_t Hkv, int64_t D,
                        void* workspace, int64_t workspace_bytes, void* stream) {
   const bool rope = q == nullptr;
-  if (D != aq::AD) return AQ_E_SHAPE;
+  if (D != 64 && D != 128) return AQ_E_SHAPE;
   if (B < 0 || Hq <= 0 || Hkv <= 0 || (Hq % Hkv) != 0 || P <= 0 || total_len <= 0 || page_size <= 0 ||
       n_pages <= 0 || !(scale > 0.0f))
     return AQ_E_SHAPE;
+  const int64_t G = Hq / Hkv;
+  if (G != 1 && G != 2 && G != 3 && G != 4 && G != 6 && G != 8) return AQ_E_SHAPE;  // query heads per KV head
   if (rope && freqs_stride != 0 && freqs_stride < D) return AQ_E_SHAPE;
   if (B == 0) return AQ_OK;
-  if (!(rope ? (qkv != nullptr && freqs != nullptr) : (q != nullptr)) || !k_cache || !v_cache || !page_table || !out) return AQ_E_NULL;
+  if (!(rope ? (qkv != nullptr && freqs != nullptr) : (q != nullptr)) || !k_cache || !v_cache || !page_table || !out)
+    return AQ_E_NULL;
   if (aq::check_ptr16(rope ? qkv : q) || aq::check_ptr16(k_cache) || aq::check_ptr16(v_cache) || aq::check_ptr16(out))
     return AQ_E_ALIGN;
   if (rope && (aq::check_ptr16(freqs) || (freqs_stride & 3))) return AQ_E_ALIGN;
@@ -395,7 +419,7 @@ static int attn_decode(const void* q, const void* qkv, const float* freqs, int64
   if (ns > 1) {
     if (!workspace) return AQ_E_NULL;
     if (aq::check_ptr16(workspace)) return AQ_E_ALIGN;
-    if (workspace_bytes < B * Hq * ns * aq::ATT_PART * (int64_t)sizeof(float)) return AQ_E_WORKSPACE;
+    if (workspace_bytes < aq::attn_workspace_bytes(B, Hq, ns)) return AQ_E_WORKSPACE;
   }
   aq::AttnArgs a{};
   a.q = static_cast<const uint16_t*>(q);
@@ -420,22 +444,24 @@ static int attn_decode(const void* q, const void* qkv, const float* freqs, int64
   a.NS = (int)ns;
   const dim3 grid((unsigned)(B * Hkv * ns)), block(aq::ATT_WAVES * 64);
   hipStream_t st = static_cast<hipStream_t>(stream);
-#define AQ_ATTN_CASE(G_)                                                                           \
-  case G_:                                                                                         \
-    if (rope) hipLaunchKernelGGL((aq::paged_attn_decode_kernel<G_, true>), grid, block, 0, st, a); \
-    else hipLaunchKernelGGL((aq::paged_attn_decode_kernel<G_, false>), grid, block, 0, st, a);     \
+#define AQ_ATTN_CASE(G_)                                            \
+  case G_:                                                          \
+    if (D == 128) attn_launch<G_, 128>(rope, grid, block, st, a);   \
+    else attn_launch<G_, 64>(rope, grid, block, st, a);             \
     break;
-  switch (Hq / Hkv) {
+  switch (G) {
     AQ_ATTN_CASE(1)
     AQ_ATTN_CASE(2)
+    AQ_ATTN_CASE(3)
     AQ_ATTN_CASE(4)
+    AQ_ATTN_CASE(6)
     AQ_ATTN_CASE(8)
-    default: return AQ_E_SHAPE;  // query heads per KV head: 1, 2, 4 or 8
   }
 #undef AQ_ATTN_CASE
   int rc = (int)hipGetLastError();
   if (rc != 0 || ns == 1) return rc;
-  hipLaunchKernelGGL(aq::attn_merge_kernel, dim3((unsigned)(B * Hq)), dim3(aq::AD / 2), 0, st, a.ws, a.out, a.NS);
+  hipLaunchKernelGGL(aq::attn_merge_kernel, dim3((unsigned)(B * Hq)), dim3((unsigned)(D / 2)), 0, st, a.ws, a.out, a.NS,
+                     (int)D);
   return (int)hipGetLastError();
 }
 

@@ -579,8 +579,9 @@ template <bool BF16>
 static int launch_swiglu_quant(const void* ug, int64_t M, int64_t F, int64_t ld, int8_t* q, float* scale,
                                hipStream_t st) {
   const int64_t vpl = (F / (BF16 ? 8 : 4) + 63) / 64;  // vector pairs per lane
-  if (vpl > 12) return AQ_E_RANGE;
-  if (vpl > 1 && M <= AQ_SWIGLU_WG_MAX_M) {  // few rows: a workgroup of vpl wavefronts per row
+  if (vpl > 16) return AQ_E_RANGE;
+  // few rows, or rows too long for one wavefront's registers: a workgroup of vpl wavefronts per row
+  if (vpl > 1 && (M <= AQ_SWIGLU_WG_MAX_M || vpl > 12)) {
     hipLaunchKernelGGL((aq::swiglu_quant_wg_kernel<BF16>), dim3((unsigned)M), dim3((unsigned)vpl * 64), 0, st, ug, (int)F,
                        ld, q, scale);
     return (int)hipGetLastError();

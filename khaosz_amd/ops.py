@@ -74,7 +74,7 @@ def quant_rowwise_i8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
 
 # longest rows the fused row kernels keep in registers (elements): bf16, fp32
 RMSNORM_QUANT_MAX_K = {torch.bfloat16: 12288, torch.float32: 6144}
-SWIGLU_QUANT_MAX_F = {torch.bfloat16: 6144, torch.float32: 3072}
+SWIGLU_QUANT_MAX_F = {torch.bfloat16: 8192, torch.float32: 4096}
 
 
 def rmsnorm_quant_rowwise_i8(x: torch.Tensor, gamma: torch.Tensor, eps: float) -> Tuple[torch.Tensor, torch.Tensor]:
@@ -312,11 +312,11 @@ def _rope_args(qkv, freqs, page_table, k_cache, v_cache, n_heads, n_kv_heads, wh
 
 def rope_kv_write(qkv: torch.Tensor, freqs: torch.Tensor, page_table: torch.Tensor, pos: int, k_cache: torch.Tensor,
                   v_cache: torch.Tensor, n_heads: int, n_kv_heads: int, return_k: bool = False):
-    """New tokens of every sequence -- ``qkv [B, (Hq + 2 Hkv) * 128]`` (one each) or ``[B, S, ...]``:
+    """New tokens of every sequence -- ``qkv [B, (Hq + 2 Hkv) * D]`` (one each, D = 64 or 128) or ``[B, S, ...]``:
     rotate q and k by ``freqs`` (complex64 ``[B, (S,) 64]`` or float32 ``[B, (S,) 64, 2]``), write k and
-    v into the paged caches ``[n_pages, page, Hkv, 128]`` at logical positions ``pos .. pos + S - 1``;
-    returns the rotated ``q [B, (S,) Hq, 128]``, and with ``return_k`` also the rotated
-    ``k [B, (S,) Hkv, 128]``."""
+    v into the paged caches ``[n_pages, page, Hkv, D]`` at logical positions ``pos .. pos + S - 1``;
+    returns the rotated ``q [B, (S,) Hq, D]``, and with ``return_k`` also the rotated
+    ``k [B, (S,) Hkv, D]``."""
     one = qkv.dim() == 2
     qkv, fr, fr_stride, page_table = _rope_args(qkv, freqs, page_table, k_cache, v_cache, n_heads, n_kv_heads,
                                                 "rope_kv_write")
@@ -350,7 +350,7 @@ def rope_paged_attn_decode(qkv: torch.Tensor, freqs: torch.Tensor, page_table: t
                            scale: Optional[float] = None, workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``rope_kv_write`` at position ``total_len - 1`` and ``paged_attn_decode`` over ``total_len``
     positions as one launch (plus the small merge launch for long sequences): same caches and
-    outputs, bit for bit.  Returns the attention output ``[B, Hq, 128]``."""
+    outputs, bit for bit.  Returns the attention output ``[B, Hq, D]``."""
     if qkv.dim() != 2:
         raise ValueError(f"one new token per sequence: qkv must be [B, W], got {tuple(qkv.shape)}")
     qkv, fr, fr_stride, page_table = _rope_args(qkv, freqs, page_table, k_cache, v_cache, n_heads, n_kv_heads,
@@ -382,7 +382,7 @@ def paged_attn_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
                       total_len: int, scale: Optional[float] = None,
                       workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``softmax(scale * q K^T) V`` for one query token per sequence over the first ``total_len``
-    positions of each sequence's pages: ``q [B, Hq, 128]`` -> ``[B, Hq, 128]`` (bfloat16).
+    positions of each sequence's pages: ``q [B, Hq, D]`` -> ``[B, Hq, D]`` (bfloat16, D = 64 or 128).
     ``workspace``: a contiguous device tensor of at least ``paged_attn_workspace_bytes`` bytes
     to reuse across calls; allocated per call when omitted or too small."""
     _need_gpu(q, k_cache, v_cache, page_table)

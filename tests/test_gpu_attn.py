@@ -20,10 +20,10 @@ def _bits(t):
     return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16).copy()
 
 
+@pytest.mark.parametrize("D", [128, 64])
 @pytest.mark.parametrize("B,Hq,Hkv,page,pos", [(1, 1, 1, 4, 0), (3, 4, 2, 8, 13), (8, 16, 4, 64, 575), (5, 8, 1, 16, 31)])
-def test_rope_kv_write_bit_exact(oracle, B, Hq, Hkv, page, pos):
-    _say("rope_kv_write", B, Hq, Hkv, page, pos)
-    D = 128
+def test_rope_kv_write_bit_exact(oracle, B, Hq, Hkv, page, pos, D):
+    _say("rope_kv_write", B, Hq, Hkv, page, pos, D)
     P = pos // page + 2
     n_pages = B * P + 3
     g = torch.Generator().manual_seed(B * 100 + pos)
@@ -43,11 +43,11 @@ def test_rope_kv_write_bit_exact(oracle, B, Hq, Hkv, page, pos):
     assert np.array_equal(_bits(kd), kb) and np.array_equal(_bits(vd), vb)
 
 
+@pytest.mark.parametrize("D", [128, 64])
 @pytest.mark.parametrize("B,S,Hq,Hkv,page,pos", [(1, 5, 1, 1, 4, 0), (3, 21, 4, 2, 8, 13), (2, 130, 16, 4, 64, 0)])
-def test_rope_kv_write_several_tokens_bit_exact(oracle, B, S, Hq, Hkv, page, pos):
+def test_rope_kv_write_several_tokens_bit_exact(oracle, B, S, Hq, Hkv, page, pos, D):
     """A prompt (or a chunk of one) in one launch: the oracle applied token by token."""
-    _say("rope_kv_write seq", B, S, Hq, Hkv, page, pos)
-    D = 128
+    _say("rope_kv_write seq", B, S, Hq, Hkv, page, pos, D)
     P = (pos + S + page - 1) // page + 1
     n_pages = B * P + 3
     g = torch.Generator().manual_seed(B * 100 + S)
@@ -82,10 +82,11 @@ def test_rope_kv_write_several_tokens_bit_exact(oracle, B, S, Hq, Hkv, page, pos
 
 @pytest.mark.parametrize("B,Hq,Hkv,page,T", [(1, 1, 1, 4, 1), (2, 8, 2, 16, 70), (8, 16, 4, 64, 576), (3, 8, 1, 16, 1000),
                                               (2, 4, 2, 64, 513), (1, 2, 2, 8, 64), (2, 2, 1, 4, 65), (1, 4, 4, 32, 256),
-                                              (2, 16, 2, 16, 257), (40, 8, 8, 16, 300), (1, 8, 1, 64, 5000)])
-def test_paged_attn_decode_within_bf16_rounding(oracle, B, Hq, Hkv, page, T):
-    _say("paged_attn_decode", B, Hq, Hkv, page, T)
-    D = 128
+                                              (2, 16, 2, 16, 257), (40, 8, 8, 16, 300), (1, 8, 1, 64, 5000),
+                                              (4, 24, 4, 128, 640), (2, 6, 2, 16, 100)])
+@pytest.mark.parametrize("D", [128, 64])
+def test_paged_attn_decode_within_bf16_rounding(oracle, B, Hq, Hkv, page, T, D):
+    _say("paged_attn_decode", B, Hq, Hkv, page, T, D)
     P = (T + page - 1) // page
     n_pages = B * P + 2
     g = torch.Generator().manual_seed(T)
@@ -132,12 +133,13 @@ def test_paged_attn_workspace_reuse_and_checks(oracle):
 
 
 @pytest.mark.parametrize("B,Hq,Hkv,page,T", [(1, 1, 1, 4, 1), (2, 8, 2, 16, 70), (8, 16, 4, 64, 576), (3, 8, 1, 16, 1000),
-                                              (2, 4, 2, 64, 513), (2, 2, 1, 4, 65), (1, 4, 4, 32, 256), (5, 16, 2, 16, 257)])
-def test_rope_paged_attn_decode_equals_the_two_launches(B, Hq, Hkv, page, T):
+                                              (2, 4, 2, 64, 513), (2, 2, 1, 4, 65), (1, 4, 4, 32, 256), (5, 16, 2, 16, 257),
+                                              (4, 24, 4, 128, 640), (2, 6, 2, 16, 100)])
+@pytest.mark.parametrize("D", [128, 64])
+def test_rope_paged_attn_decode_equals_the_two_launches(B, Hq, Hkv, page, T, D):
     """The fused decode step (rotate, write the new token, attend) against rope_kv_write followed by
     paged_attn_decode: caches and outputs bit for bit, including a sequence whose new page is unmapped."""
-    _say("rope_paged_attn_decode", B, Hq, Hkv, page, T)
-    D = 128
+    _say("rope_paged_attn_decode", B, Hq, Hkv, page, T, D)
     P = (T + page - 1) // page
     n_pages = B * P + 2
     g = torch.Generator().manual_seed(T + 1)
@@ -167,12 +169,12 @@ def test_rope_paged_attn_decode_equals_the_two_launches(B, Hq, Hkv, page, T):
 
 
 def test_attn_argument_checks():
-    q = torch.zeros(2, 4, 64, dtype=torch.bfloat16, device=DEV)
-    kc = torch.zeros(4, 8, 2, 64, dtype=torch.bfloat16, device=DEV)
+    q = torch.zeros(2, 4, 32, dtype=torch.bfloat16, device=DEV)
+    kc = torch.zeros(4, 8, 2, 32, dtype=torch.bfloat16, device=DEV)
     tab = torch.zeros(2, 2, dtype=torch.int64, device=DEV)
     with pytest.raises(ValueError):
-        ops.paged_attn_decode(q, kc, kc.clone(), tab, 5)          # head dimension 64 is not supported
-    q = torch.zeros(2, 6, 128, dtype=torch.bfloat16, device=DEV)
+        ops.paged_attn_decode(q, kc, kc.clone(), tab, 5)          # head dimension 32 is not supported
+    q = torch.zeros(2, 10, 128, dtype=torch.bfloat16, device=DEV)
     kc = torch.zeros(4, 8, 2, 128, dtype=torch.bfloat16, device=DEV)
     with pytest.raises(ValueError):
-        ops.paged_attn_decode(q, kc, kc.clone(), tab, 5)          # 3 query heads per KV head
+        ops.paged_attn_decode(q, kc, kc.clone(), tab, 5)          # 5 query heads per KV head

@@ -50,7 +50,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="decode", choices=["decode", "prefill", "fp8", "block"])
+    ap.add_argument("--workload", default="decode", choices=["decode", "prefill", "fp8", "block", "model"])
     ap.add_argument("--m", type=int, default=16, help="decode rows (1..16)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary workloads")
@@ -352,6 +352,67 @@ def bench_block(torch, ops, args, dev):
     }
 
 
+def bench_model(torch, ops, args, dev):
+    """The reference's own generation benchmark (scripts/tools/benchmark.py:219-248): 24 layers of width 1536,
+    24 query / 4 KV heads of 64, FFN 6912, vocabulary 10000, bf16, 128-token pages; prefill 4 x 512 tokens, then
+    128 decode steps of 4 sequences.  The float model runs the reference's flow in stock torch; the quantized one
+    has the 168 block projections and the vocabulary projection in W8A8 with every fusion this package offers."""
+    from khaosz_amd import AutoRegressiveLM, LMConfig, fuse_shared_inputs, quantize_model
+
+    dt = torch.bfloat16
+    cfg = LMConfig(vocab_size=10000, dim=1536, n_layers=24, n_heads=24, n_kv_heads=4, dim_ffn=6912, max_len=2048)
+    B, S, gen, page = 4, 512, 128, 128
+    torch.manual_seed(11)
+    model = AutoRegressiveLM(cfg).to(dev).to(dt).eval()
+    P = (S + gen + page - 1) // page
+    cache = model.new_cache(B * P, page)
+    table = torch.arange(B * P, device=dev).view(B, P)  # pages handed out in order, as the benchmark's fresh pool does
+    g = torch.Generator(device="cpu").manual_seed(12)
+    prompt = torch.randint(0, cfg.vocab_size, (B, S), generator=g).to(dev)
+    gen_ids = torch.randint(0, cfg.vocab_size, (B, gen), generator=g).to(dev)
+
+    def prefill(i=0):
+        return model(prompt, paged_cache=cache.bind(table, S), start_pos=0)["logits"]
+
+    def decode_all(i=0):
+        for t in range(gen):
+            model(gen_ids[:, t:t + 1], paged_cache=cache.bind(table, S + t + 1), start_pos=S + t)
+
+    def measure():
+        pre_eager = eager_time_ms(torch, prefill, 5, 2)
+        pre_graph = graph_time_ms(torch, prefill, 3, 1)
+        prefill()
+        dec_eager = eager_time_ms(torch, decode_all, 2, 1) / gen
+        dec_graph = graph_time_ms(torch, decode_all, 1, 1) / gen
+        return {"prefill_ms": pre_graph, "prefill_tok_s": B * S / (pre_graph * 1e-3),
+                "prefill_eager_ms": pre_eager, "prefill_eager_tok_s": B * S / (pre_eager * 1e-3),
+                "decode_ms_per_step": dec_graph, "decode_tok_s": B / (dec_graph * 1e-3),
+                "decode_eager_ms_per_step": dec_eager, "decode_eager_tok_s": B / (dec_eager * 1e-3)}
+
+    flt = measure()
+    ref_logits = prefill().float()
+    n = quantize_model(model, target_modules={"q_proj", "k_proj", "v_proj", "o_proj", "up", "gate", "down", "lm_head"})
+    qsep = measure()  # quantized, every projection on its own and torch around them, as a drop-in gives
+    fuse_shared_inputs(model, norms=True, decode_attention=True, residuals=True)
+    q = measure()
+    ql = prefill().float()
+    err = ((ql - ref_logits).norm() / ref_logits.norm()).item()
+    weight_bytes = sum(m.qweight.numel() for m in model.modules() if hasattr(m, "qweight"))
+    return {
+        "workload": "generation benchmark of the reference (24 x 1536, 24q/4kv x 64, ffn 6912, vocab 10000, bf16, "
+                    "128-token pages): prefill 4 x 512, then 128 decode steps of 4 sequences; W8A8, all fusions, "
+                    "HIP graph replay",
+        "value": q["decode_tok_s"], "unit": "tok/s", "ms_per_step": q["decode_ms_per_step"], "dtype": "int8",
+        "quantized_linears": n, "int8_weight_bytes": weight_bytes,
+        "decode_weight_stream_gbs": weight_bytes / (q["decode_ms_per_step"] * 1e-3) / 1e9,
+        "quantized_fused": q, "quantized_drop_in": qsep, "float_bf16_torch": flt,
+        "prefill_logits_rel_err_vs_float": err,
+        "speedup_decode_vs_float_graph": flt["decode_ms_per_step"] / q["decode_ms_per_step"],
+        "speedup_prefill_vs_float_graph": flt["prefill_ms"] / q["prefill_ms"],
+        "roofline": {}, "shape": (B, 0, 0),
+    }
+
+
 def measure_ceilings(torch, ops, dev):
     """What this part delivers on trivial kernels: an MFMA-only loop (constant operands, so the
     clock is not power-limited: an upper bound), a 1 GiB streaming read, and a one-shot 16 MiB
@@ -492,12 +553,13 @@ def main():
         sys.exit(2)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    fns = {"decode": bench_decode, "prefill": bench_prefill, "fp8": bench_fp8, "block": bench_block}
+    fns = {"decode": bench_decode, "prefill": bench_prefill, "fp8": bench_fp8, "block": bench_block,
+           "model": bench_model}
     with torch.inference_mode():
         main_res = fns[args.workload](torch, ops, args, dev)
         extra = {}
         if not args.no_extra:
-            for name in ("decode", "prefill", "fp8", "block"):
+            for name in ("decode", "prefill", "fp8", "block"):  # "model" only on request: it takes a minute
                 if name != args.workload:
                     extra[name] = fns[name](torch, ops, args, dev)
             if args.workload == "decode":
@@ -509,7 +571,7 @@ def main():
         ceilings = measure_ceilings(torch, ops, dev)
     per_step = main_res.get("bytes_per_step") or main_res.get("ops_per_step") or main_res.get("flops_per_step")
     cpu = None
-    if not args.no_cpu and args.workload != "block":
+    if not args.no_cpu and args.workload not in ("block", "model"):
         cpu = cpu_baseline(args.workload, main_res["shape"], main_res["unit"], per_step)
         if not args.no_extra and "prefill" in extra:
             # one pass of the prefill shape as well, so both halves of the metric have a CPU figure
@@ -518,7 +580,7 @@ def main():
     for r in [main_res, *extra.values()]:
         r.pop("shape", None)
     top = ("workload", "value", "unit", "ms_per_step", "dtype", "roofline", "eager_ms_per_step")
-    detail = {k: v for k, v in main_res.items() if k not in top} if args.workload == "block" else None
+    detail = {k: v for k, v in main_res.items() if k not in top} if args.workload in ("block", "model") else None
     line = {
         "metric": METRIC, "value": main_res["value"], "unit": main_res["unit"], "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": main_res["ms_per_step"],

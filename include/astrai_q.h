@@ -115,6 +115,20 @@ int aq_gemv_w8a8_codes_residual(const int8_t *xq, const float *sx, const int8_t 
                                 const void *bias, int bias_dtype, const void *residual, void *y,
                                 int y_dtype, int64_t M, int64_t N, int64_t K, void *stream);
 
+/* aq_gemv_w8a8_decode_residual with the RMSNorm in front of the Linear folded in:
+ * y = linear(quantise(rmsnorm(x) * gamma)) (+ bias) (+ residual), the codes and
+ * scales being those aq_rmsnorm_quant_rowwise_i8 gives (same fixed arithmetic),
+ * so the result equals that call followed by aq_gemv_w8a8_codes_residual bit
+ * for bit.  One launch for up to 8 bf16 rows of at most 2048 elements, those two
+ * calls through ws otherwise.  gamma: [K] in x's dtype; residual may be NULL.
+ * Replaces the norm + Linear pairs of a decode step (decoder_block.py:50-51,57
+ * feeding attention.py:83-85 and mlp.py:25). */
+int aq_gemv_w8a8_decode_rmsnorm(const void *x, int x_dtype, const void *gamma, float eps,
+                                const int8_t *wq, const float *sw, const void *bias,
+                                int bias_dtype, const void *residual, void *y, int y_dtype,
+                                int64_t M, int64_t N, int64_t K, void *ws, size_t ws_bytes,
+                                void *stream);
+
 /* FP8 Linear: y[m, n] = (sum_k f(xq[m,k]) * f(wq[n,k])) * sx[0] * sw[0] with
  * fp32 accumulation, cast to y_dtype.  xq: [M, K], wq: [N, K] e4m3fn codes;
  * sx, sw: device scalars written by aq_quant_tensor_fp8.  Replaces F.linear

@@ -75,7 +75,8 @@ class ContiguousKV:
 
 
 class PagedKV:
-    """Paged KV cache for one block: pages ``[n_pages, page_size, Hkv, D]`` and a page table
+    """Paged KV cache for ``n_layers`` blocks (one by default): pages
+    ``[n_layers, n_pages, page_size, Hkv, D]`` (cache.py:187-214) and a page table
     ``[B, pages_per_sequence]`` of physical page ids, -1 for a logical page that is not
     mapped (cache.py:187-274).  ``write`` places the new tokens at logical positions
     ``total_len - S .. total_len`` page by page; rows whose page is unmapped are skipped.
@@ -84,11 +85,13 @@ class PagedKV:
     so neither method synchronises with the device (the reference tests the device tensor,
     ``cache.py:233,262``) and both can be captured in a HIP graph."""
 
-    def __init__(self, n_pages: int, page_size: int, n_kv_heads: int, head_dim: int, device, dtype):
+    def __init__(self, n_pages: int, page_size: int, n_kv_heads: int, head_dim: int, device, dtype,
+                 n_layers: int = 1):
         self.page_size = page_size
-        self.k = torch.zeros((n_pages, page_size, n_kv_heads, head_dim), device=device, dtype=dtype)
-        self.v = torch.zeros_like(self.k)
+        self.k_layers = torch.zeros((n_layers, n_pages, page_size, n_kv_heads, head_dim), device=device, dtype=dtype)
+        self.v_layers = torch.zeros_like(self.k_layers)
         self.page_table: Optional[Tensor] = None
+        self._attn_ws: Optional[Tensor] = None
         self._mapped = None      # host bool [B, P]
         self._safe = None        # device table with -1 replaced by 0
         self._invalid = None     # device bool [B, P * page_size] or None when everything is mapped
@@ -109,6 +112,26 @@ class PagedKV:
         self.total_len = total_len
         return self
 
+    def attn_workspace(self, n_heads: int) -> Optional[Tensor]:
+        """Scratch for the decode attention kernel's partial results, sized once for the longest
+        sequence the bound page table can hold and shared by all layers (they run one after the other)."""
+        B, P = self.page_table.shape
+        need = ops.paged_attn_workspace_bytes(B, n_heads, self.k_layers.shape[3], P * self.page_size)
+        if need == 0:
+            return None
+        if self._attn_ws is None or self._attn_ws.numel() * 4 < need:
+            self._attn_ws = torch.empty(need // 4, dtype=torch.float32, device=self.k_layers.device)
+        return self._attn_ws
+
+    @property
+    def k(self) -> Tensor:
+        """Layer 0's key pages (the whole cache of a single block)."""
+        return self.k_layers[0]
+
+    @property
+    def v(self) -> Tensor:
+        return self.v_layers[0]
+
     @property
     def all_mapped(self) -> bool:
         """Every entry of the bound page table names a page."""
@@ -121,6 +144,7 @@ class PagedKV:
         start, ps = self.total_len - S, self.page_size
         if start < 0 or (self.total_len + ps - 1) // ps > self.page_table.size(1):
             raise ValueError("tokens fall outside the page table")
+        kc, vc = self.k_layers[layer_id], self.v_layers[layer_id]
         done = 0
         for pi in range(start // ps, (self.total_len - 1) // ps + 1):
             lo = max(pi * ps, start)
@@ -129,18 +153,18 @@ class PagedKV:
             rows = self._mapped[:, pi]
             if bool(rows.all()):
                 phys = self._safe[:, pi]
-                self.k[phys, off:off + n] = k[:, done:done + n]
-                self.v[phys, off:off + n] = v[:, done:done + n]
+                kc[phys, off:off + n] = k[:, done:done + n]
+                vc[phys, off:off + n] = v[:, done:done + n]
             elif bool(rows.any()):
                 sel = rows.nonzero().flatten().to(k.device)
                 phys = self._safe[sel, pi]
-                self.k[phys, off:off + n] = k[sel, done:done + n]
-                self.v[phys, off:off + n] = v[sel, done:done + n]
+                kc[phys, off:off + n] = k[sel, done:done + n]
+                vc[phys, off:off + n] = v[sel, done:done + n]
             done += n
 
     def gather(self, layer_id: int) -> Tuple[Tensor, Tensor]:
-        k = self.k[self._safe].flatten(1, 2)
-        v = self.v[self._safe].flatten(1, 2)
+        k = self.k_layers[layer_id][self._safe].flatten(1, 2)
+        v = self.v_layers[layer_id][self._safe].flatten(1, 2)
         if self._invalid is not None:
             m = self._invalid[:, :, None, None]
             k, v = k.masked_fill(m, 0.0), v.masked_fill(m, 0.0)
@@ -196,28 +220,38 @@ class GQA(nn.Module):
             return self.o_proj(out, residual=residual)
         return self.o_proj(out) + residual
 
+    def _project_qkv(self, x: Tensor, codes, norm) -> Tensor:
+        if codes is not None:
+            return self._qkv.forward_codes(codes[0], codes[1], x.dtype).view(*x.shape[:-1], -1)
+        return self._qkv(x) if norm is None else self._qkv(x, norm=norm)
+
     def forward(self, x: Tensor, rotary_emb: Tensor, attn_mask: Optional[Tensor] = None,
                 cache=None, codes: Optional[Tuple[Tensor, Tensor]] = None,
-                residual: Optional[Tensor] = None) -> Tensor:
+                residual: Optional[Tensor] = None, norm=None) -> Tensor:
         """``codes``: the already normalised and quantised input ``(xq [B*S, dim], sx [B*S])`` from a
-        fused norm; ``x`` then only gives the shape and dtype.  ``residual``: added to the output
-        (in o_proj's epilogue when it is quantized)."""
+        fused norm; ``x`` then only gives the shape and dtype.  ``norm = (gain, eps)``: ``x`` is the
+        un-normalised stream and the norm runs inside the fused q/k/v projection.  ``residual``:
+        added to the output (in o_proj's epilogue when it is quantized)."""
         B, S, _ = x.shape
+        if norm is not None and self._qkv is None:
+            x, norm = F.rms_norm(x, (x.shape[-1],), norm[0], norm[1]), None
         if (self._decode_attention and S == 1 and isinstance(cache, PagedKV) and x.is_cuda
                 and x.dtype == torch.bfloat16):
-            qkv = self._qkv(x) if codes is None else self._qkv.forward_codes(codes[0], codes[1], x.dtype)
+            qkv = self._project_qkv(x, codes, norm)
             out = ops.rope_paged_attn_decode(qkv.view(B, -1), rotary_emb.reshape(B, -1), cache.page_table,
-                                             cache.total_len, cache.k, cache.v, self.n_heads, self.n_kv_heads)
+                                             cache.total_len, cache.k_layers[self.layer_id],
+                                             cache.v_layers[self.layer_id], self.n_heads, self.n_kv_heads,
+                                             workspace=cache.attn_workspace(self.n_heads))
             return self._out(out.view(B, 1, -1), residual)
         if (self._decode_attention and isinstance(cache, PagedKV) and x.is_cuda and x.dtype == torch.bfloat16
                 and S <= cache.total_len):
             # several new tokens (prefill): rotation and the page writes as one launch; the attention
             # itself stays the stock one, over the new keys directly when nothing older is cached
             nq, nkv = self.n_heads * self.head_dim, self.n_kv_heads * self.head_dim
-            qkv = self._qkv(x) if codes is None else self._qkv.forward_codes(codes[0], codes[1], x.dtype).view(B, S, -1)
+            qkv = self._project_qkv(x, codes, norm)
             start = cache.total_len - S
-            q, k = ops.rope_kv_write(qkv, rotary_emb, cache.page_table, start, cache.k, cache.v, self.n_heads,
-                                     self.n_kv_heads, return_k=True)
+            q, k = ops.rope_kv_write(qkv, rotary_emb, cache.page_table, start, cache.k_layers[self.layer_id],
+                                     cache.v_layers[self.layer_id], self.n_heads, self.n_kv_heads, return_k=True)
             if start == 0 and cache.all_mapped:
                 v = qkv[..., nq + nkv:].view(B, S, self.n_kv_heads, self.head_dim)
             else:
@@ -228,7 +262,7 @@ class GQA(nn.Module):
             return self._out(out.transpose(1, 2).reshape(B, S, -1), residual)
         if self._qkv is not None:
             nq, nkv = self.n_heads * self.head_dim, self.n_kv_heads * self.head_dim
-            qkv = self._qkv(x) if codes is None else self._qkv.forward_codes(codes[0], codes[1], x.dtype).view(B, S, -1)
+            qkv = self._project_qkv(x, codes, norm)
             q, k, v = qkv.split((nq, nkv, nkv), dim=-1)
         else:
             q, k, v = self.q_proj(x), self.k_proj(x), self.v_proj(x)
@@ -267,13 +301,18 @@ class MLP(nn.Module):
         return False
 
     def forward(self, x: Tensor, codes: Optional[Tuple[Tensor, Tensor]] = None,
-                residual: Optional[Tensor] = None) -> Tensor:
+                residual: Optional[Tensor] = None, norm=None) -> Tensor:
+        """``codes`` / ``norm``: as for the attention block (the input of up and gate)."""
+        if norm is not None and self._upgate is None:
+            x, norm = F.rms_norm(x, (x.shape[-1],), norm[0], norm[1]), None
         if residual is not None and not isinstance(self.down, QuantLinear):
-            return self.forward(x, codes) + residual
+            return self.forward(x, codes, norm=norm) + residual
         kw = {} if residual is None else {"residual": residual}
         if self._upgate is not None:
-            ug = self._upgate(x) if codes is None else self._upgate.forward_codes(codes[0], codes[1], x.dtype).view(
-                *x.shape[:-1], -1)
+            if codes is not None:
+                ug = self._upgate.forward_codes(codes[0], codes[1], x.dtype).view(*x.shape[:-1], -1)
+            else:
+                ug = self._upgate(x) if norm is None else self._upgate(x, norm=norm)
             if (self._swiglu_quant and isinstance(self.down, QuantLinear) and ug.is_cuda
                     and ug.shape[-1] // 2 <= ops.SWIGLU_QUANT_MAX_F.get(ug.dtype, 0)):
                 # activation, product and the down projection's quantisation in one launch
@@ -329,9 +368,8 @@ class DecoderBlock(nn.Module):
         if (self._norm_quant and x.is_cuda and x.dtype == self.input_norm.weight.dtype
                 and x.shape[-1] <= ops.RMSNORM_QUANT_MAX_K.get(x.dtype, 0)):
             n1, n2 = self.input_norm, self.post_attention_norm
-            x = add(self.attention(x, rotary_emb, attention_mask, cache,
-                                   codes=ops.rmsnorm_quant_rowwise_i8(x, n1.weight, n1.norm_eps), **kw(x)), x)
-            return add(self.mlp(x, codes=ops.rmsnorm_quant_rowwise_i8(x, n2.weight, n2.norm_eps), **kw(x)), x)
+            x = add(self.attention(x, rotary_emb, attention_mask, cache, norm=(n1.weight, n1.norm_eps), **kw(x)), x)
+            return add(self.mlp(x, norm=(n2.weight, n2.norm_eps), **kw(x)), x)
         x = add(self.attention(self.input_norm(x), rotary_emb, attention_mask, cache, **kw(x)), x)
         return add(self.mlp(self.post_attention_norm(x), **kw(x)), x)
 

@@ -57,16 +57,52 @@ __device__ __forceinline__ RowScale row_scale(float amax) {
   return r;
 }
 
+// Sum across the wavefront in a fixed order: p[l] += p[l ^ 1], ^2, ^4, ^8, ^16, ^32, every add
+// rounded.  After the xor-1 and xor-2 steps a quad holds one value, after the half-row mirror a
+// half row does, after the row mirror a row does: the mirrors pair the same partial sums as
+// xor 4 and xor 8 would.
+__device__ __forceinline__ float wave_sum_butterfly(float v) {
+  v = __fadd_rn(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xf, 0xf, false)));
+  v = __fadd_rn(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xf, 0xf, false)));
+  v = __fadd_rn(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xf, 0xf, false)));
+  v = __fadd_rn(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xf, 0xf, false)));
+  v = __fadd_rn(v, __shfl_xor(v, 16, 64));
+  v = __fadd_rn(v, __shfl_xor(v, 32, 64));
+  return v;
+}
+
+// 1 / sqrt(mean(x^2) + eps) of a row from its sum of squares: correctly rounded divide, add,
+// square root (sqrtf; the __fsqrt_rn intrinsic is the 1-ulp native root) and divide.
+__device__ __forceinline__ float rms_scale(float ss, float k, float eps) {
+  return __fdiv_rn(1.0f, sqrtf(__fadd_rn(__fdiv_rn(ss, k), eps)));
+}
+
 // One wavefront quantises RPW rows of the activation straight into LDS.
 // Wavefront `wave` of `nwaves` owns rows wave, wave + nwaves, ...; a lane holds
 // VPL 16-byte vectors per row (vector lane + 64*i), all requested by issue()
 // before anything is waited for, so the caller can queue other loads behind
 // them.  finish() reduces, rounds and writes the codes of row m to
 // xs + m*pitch and its scale to sx[m]; rows >= M (up to MT) are zero-filled.
+// With NORM the rows are RMS-normalised first, y = (x * r) * gamma with
+// r = rms_scale(sum of squares in the fixed order: a lane adds the rounded
+// squares of its vectors lane, lane + 64, ... in ascending order, elements in
+// memory order, then the butterfly): the arithmetic of the stand-alone
+// norm-and-quantise kernel, bit for bit.  gamma is requested by issue_gamma().
 template <bool BF16, int RPW, int VPL>
 struct RowsToLds {
   static constexpr int EPV = RowIn<BF16>::EPV;
   uint4 c[RPW][VPL];
+  uint4 gv[VPL];
+
+  __device__ __forceinline__ void issue_gamma(const void* gamma, int K, int lane) {
+    const int nvec = K / EPV;
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) {
+      const int v = i * 64 + lane;
+      gv[i] = make_uint4(0, 0, 0, 0);
+      if (v < nvec) gv[i] = reinterpret_cast<const uint4*>(gamma)[v];
+    }
+  }
 
   __device__ __forceinline__ void issue(const void* x, int M, int K, int64_t ldx, int wave, int nwaves, int lane) {
     const int nvec = K / EPV;
@@ -84,18 +120,43 @@ struct RowsToLds {
     }
   }
 
+  // vector i of row j as the values to quantise
+  template <bool NORM>
+  __device__ __forceinline__ void values(int j, int i, float r, float* f) const {
+    RowIn<BF16>::unpack(c[j][i], f);  // vectors past the row or of rows >= M are zero
+    if constexpr (NORM) {
+      float g[EPV];
+      RowIn<BF16>::unpack(gv[i], g);
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) f[e] = __fmul_rn(__fmul_rn(f[e], r), g[e]);
+    }
+  }
+
+  template <bool NORM = false>
   __device__ __forceinline__ void finish(int M, int MT, int K, uint8_t* xs, int pitch, float* sx, int wave,
-                                         int nwaves, int lane) {
+                                         int nwaves, int lane, float eps = 0.0f) {
     const int nvec = K / EPV;
 #pragma unroll
     for (int j = 0; j < RPW; ++j) {
       const int m = wave + j * nwaves;
       if (m >= MT) continue;  // uniform
+      float r = 1.0f;
+      if constexpr (NORM) {
+        float ss = 0.0f;
+#pragma unroll
+        for (int i = 0; i < VPL; ++i) {
+          float f[EPV];
+          RowIn<BF16>::unpack(c[j][i], f);
+#pragma unroll
+          for (int e = 0; e < EPV; ++e) ss = __fadd_rn(ss, __fmul_rn(f[e], f[e]));
+        }
+        r = rms_scale(wave_sum_butterfly(ss), (float)K, eps);
+      }
       float amax = 0.0f;
 #pragma unroll
       for (int i = 0; i < VPL; ++i) {
         float f[EPV];
-        RowIn<BF16>::unpack(c[j][i], f);  // vectors past the row or of rows >= M are zero
+        values<NORM>(j, i, r, f);
         amax = fmaxf(amax, vec_amax<EPV>(f));
       }
       const RowScale rsc = row_scale(wave_max(amax));
@@ -106,7 +167,7 @@ struct RowsToLds {
         if (v < nvec) {
           float f[EPV];
           uint32_t code[EPV];
-          RowIn<BF16>::unpack(c[j][i], f);
+          values<NORM>(j, i, r, f);
           quant_codes<EPV>(f, rsc.s, rsc.rs, rsc.fast_ok, code);  // zero rows give zero codes
           uint8_t* dst = xs + m * pitch + v * EPV;
           if constexpr (BF16) {

@@ -85,6 +85,8 @@ struct GemvArgs {
   int M, N, K;
   int bias_dtype, y_dtype;
   int ksplit, groups;  // matrix-core variant: wavefronts sharing a row group, row groups per workgroup
+  const void* gamma;   // NORM kernels: RMSNorm gain [K] in x's dtype
+  float eps;
 };
 
 // y (+ residual): the projection is rounded to the output type first and the
@@ -102,7 +104,8 @@ __device__ __forceinline__ float add_residual_bf16(float y, uint32_t res_bits) {
 // the other before any product can start), taken from the launch otherwise.  A
 // workgroup covers GV_ROWS * wavefronts weight rows; the launcher shrinks it
 // when N is too small for 8-wavefront workgroups to reach every compute unit.
-template <int MT, bool FUSED, int VPL>
+// NORM (with FUSED): the rows are RMS-normalised with the gain p.gamma before they are quantised.
+template <int MT, bool FUSED, int VPL, bool NORM = false>
 __global__ __launch_bounds__(GV_THREADS) void gemv_w8a8_kernel(GemvArgs p) {
   extern __shared__ __attribute__((aligned(16))) uint8_t xs[];  // [MT][K] activation codes, then [MT] scales
   const int tid = threadIdx.x, lane = tid & 63;
@@ -144,6 +147,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_w8a8_kernel(GemvArgs p) {
   RowsToLds<true, RPW, VPL> xrows;
   if constexpr (FUSED) {
     xrows.issue(p.x, M, K, K, wave, WAVES, lane);
+    if constexpr (NORM) xrows.issue_gamma(p.gamma, K, lane);
   } else {
     const __amdgpu_buffer_rsrc_t Xr = make_rsrc(p.xq, (uint32_t)M * (uint32_t)K);
     const int xbytes = MT * K;
@@ -180,7 +184,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_w8a8_kernel(GemvArgs p) {
   // compiler place that wait), then make every wavefront's part visible through
   // a barrier that does not drain the weight loads.
   if constexpr (FUSED) {
-    xrows.finish(M, MT, K, xs, K, sx_lds, wave, WAVES, lane);
+    xrows.template finish<NORM>(M, MT, K, xs, K, sx_lds, wave, WAVES, lane, p.eps);
     __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wavefront's LDS writes are done
   } else {
     GV_WAIT_VMCNT(GV_DEPTH * GV_ROWS);
@@ -258,17 +262,17 @@ static int gemv_waves(int N) {
   return waves;
 }
 
-template <int MT, bool FUSED, int VPL>
+template <int MT, bool FUSED, int VPL, bool NORM = false>
 static int launch_gemv(const GemvArgs& a, hipStream_t st) {
   const int waves = FUSED ? GV_WAVES : gemv_waves(a.N);
   const unsigned grid = (unsigned)((a.N + GV_ROWS * waves - 1) / (GV_ROWS * waves));
   const size_t lds = (size_t)MT * a.K + MT * sizeof(float);
   if (lds > 64 * 1024) {  // beyond the default dynamic-LDS limit: opt this kernel in (idempotent)
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_w8a8_kernel<MT, FUSED, VPL>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_w8a8_kernel<MT, FUSED, VPL, NORM>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return (int)e;
   }
-  hipLaunchKernelGGL((gemv_w8a8_kernel<MT, FUSED, VPL>), dim3(grid), dim3(waves * 64), lds, st, a);
+  hipLaunchKernelGGL((gemv_w8a8_kernel<MT, FUSED, VPL, NORM>), dim3(grid), dim3(waves * 64), lds, st, a);
   return (int)hipGetLastError();
 }
 
@@ -522,6 +526,15 @@ static int gemv_dispatch_fused(const aq::GemvArgs& a, int mt, hipStream_t st) {
   const int64_t vpl = (a.K / 8 + 63) / 64;  // 16-byte vectors per lane per bf16 row
   if (mt > 8 || vpl > 16) return -1;
   const bool small = vpl <= 4;
+  if (a.gamma) {  // with the norm in front: short rows only (the gain's vectors stay in registers too)
+    if (!small) return -1;
+    switch (mt) {
+      case 1: return aq::launch_gemv<1, true, 4, true>(a, st);
+      case 2: return aq::launch_gemv<2, true, 4, true>(a, st);
+      case 4: return aq::launch_gemv<4, true, 4, true>(a, st);
+      default: return aq::launch_gemv<8, true, 4, true>(a, st);
+    }
+  }
   switch (mt) {
     case 1: return small ? aq::launch_gemv<1, true, 4>(a, st) : aq::launch_gemv<1, true, 16>(a, st);
     case 2: return small ? aq::launch_gemv<2, true, 4>(a, st) : aq::launch_gemv<2, true, 16>(a, st);
@@ -592,6 +605,43 @@ extern "C" int aq_gemv_w8a8_decode_residual(const void* x, int x_dtype, const in
   int8_t* xq = static_cast<int8_t*>(ws);
   float* sx = reinterpret_cast<float*>(static_cast<char*>(ws) + aq::align256((size_t)(M * K)));
   rc = aq_quant_rowwise_i8(x, x_dtype, M, K, K, xq, sx, stream);
+  if (rc) return rc;
+  return aq_gemv_w8a8_codes_residual(xq, sx, wq, sw, bias, bias_dtype, residual, y, y_dtype, M, N, K, stream);
+}
+
+extern "C" int aq_gemv_w8a8_decode_rmsnorm(const void* x, int x_dtype, const void* gamma, float eps, const int8_t* wq,
+                                           const float* sw, const void* bias, int bias_dtype, const void* residual,
+                                           void* y, int y_dtype, int64_t M, int64_t N, int64_t K, void* ws,
+                                           size_t ws_bytes, void* stream) {
+  if (x_dtype != AQ_F32 && x_dtype != AQ_BF16) return AQ_E_DTYPE;
+  int mt = 0;
+  int rc = gemv_check(wq, sw, bias, bias_dtype, y, y_dtype, M, N, K, &mt);
+  if (rc || M == 0 || N == 0) return rc;
+  if (!x || !gamma || !ws) return AQ_E_NULL;
+  if (aq::check_ptr16(x) || aq::check_ptr16(gamma) || aq::check_ptr16(ws)) return AQ_E_ALIGN;
+  if (ws_bytes < aq_gemv_w8a8_workspace_bytes(M, K)) return AQ_E_WORKSPACE;
+  if (x_dtype == AQ_BF16) {  // one launch: the GEMV kernel normalises and quantises the rows itself
+    aq::GemvArgs a{};
+    a.x = x;
+    a.gamma = gamma;
+    a.eps = eps;
+    a.wq = wq;
+    a.sw = sw;
+    a.bias = bias;
+    a.res = residual;
+    a.ldr = N;
+    a.y = y;
+    a.M = (int)M;
+    a.N = (int)N;
+    a.K = (int)K;
+    a.bias_dtype = bias_dtype;
+    a.y_dtype = y_dtype;
+    const int frc = gemv_dispatch_fused(a, mt, static_cast<hipStream_t>(stream));
+    if (frc >= 0) return frc;
+  }
+  int8_t* xq = static_cast<int8_t*>(ws);
+  float* sx = reinterpret_cast<float*>(static_cast<char*>(ws) + aq::align256((size_t)(M * K)));
+  rc = aq_rmsnorm_quant_rowwise_i8(x, x_dtype, gamma, x_dtype, eps, M, K, K, xq, sx, stream);
   if (rc) return rc;
   return aq_gemv_w8a8_codes_residual(xq, sx, wq, sw, bias, bias_dtype, residual, y, y_dtype, M, N, K, stream);
 }

@@ -169,19 +169,6 @@ __global__ __launch_bounds__(256) void quant_row_wg_kernel(const void* __restric
 // butterfly p[l] += p[l ^ 1], ^2, ^4, ^8, ^16, ^32.  mean = ss / K,
 // r = 1 / sqrt(mean + eps) with correctly rounded divide and square root,
 // y = (x * r) * gamma as two rounded products.
-__device__ __forceinline__ float wave_sum_butterfly(float v) {
-  // After the xor-1 and xor-2 steps a quad holds one value, after the half-row
-  // mirror a half row does, after the row mirror a row does: the mirrors pair
-  // the same partial sums as xor 4 and xor 8 would.
-  v = __fadd_rn(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xf, 0xf, false)));
-  v = __fadd_rn(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xf, 0xf, false)));
-  v = __fadd_rn(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xf, 0xf, false)));
-  v = __fadd_rn(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xf, 0xf, false)));
-  v = __fadd_rn(v, __shfl_xor(v, 16, 64));
-  v = __fadd_rn(v, __shfl_xor(v, 32, 64));
-  return v;
-}
-
 // One wavefront per row; a lane keeps its NC vectors of the row in registers
 // across the three passes (sum of squares, absmax of y, rounding).  GREG: the
 // lane's gamma vectors are loaded once and kept too (short rows); otherwise
@@ -221,7 +208,7 @@ __global__ __launch_bounds__(256) void rmsnorm_quant_kernel(const void* __restri
       for (int e = 0; e < EPV; ++e) ss = __fadd_rn(ss, __fmul_rn(f[e], f[e]));
     }
     ss = wave_sum_butterfly(ss);
-    const float r = __fdiv_rn(1.0f, sqrtf(__fadd_rn(__fdiv_rn(ss, kf), eps)));  // sqrtf: correctly rounded (the __fsqrt_rn intrinsic is the 1-ulp native root)
+    const float r = rms_scale(ss, kf, eps);
     auto normed = [&](int i, float* y) {
       float f[EPV], g[EPV];
       RowIn<BF16>::unpack(c[i], f);

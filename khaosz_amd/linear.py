@@ -161,9 +161,12 @@ class QuantLinear(Linear):
                                       error_msgs)
 
     # -- forward ----------------------------------------------------------------
-    def forward(self, x: Tensor, residual: Optional[Tensor] = None) -> Tensor:
+    def forward(self, x: Tensor, residual: Optional[Tensor] = None, norm=None) -> Tensor:
         """``residual`` (shape and dtype of the output): returns ``linear(x) + residual`` with the add
-        done in the kernel's epilogue, bit-identical to adding the two tensors afterwards."""
+        done in the kernel's epilogue, bit-identical to adding the two tensors afterwards.
+        ``norm = (gain [in_dim], eps)``: returns ``linear(rms_norm(x) * gain)`` with the norm fused
+        into the activation quantisation (the normalised activations are never written; see
+        ``ops.rmsnorm_quant_rowwise_i8``)."""
         _no_grad_guard(x)
         lead = x.shape[:-1]
         x2 = x.reshape(-1, x.shape[-1])
@@ -178,9 +181,9 @@ class QuantLinear(Linear):
             if ws is None or ws.device != x.device or ws.numel() < need:
                 ws = self._workspace = torch.empty((need,), dtype=torch.uint8, device=x.device)
             y = ops.gemv_w8a8_decode(x2, self.qweight, self.w_scale, self.bias, out_dtype=x.dtype, workspace=ws,
-                                     residual=residual)
+                                     residual=residual, norm=norm)
         else:
-            xq, sx = ops.quant_rowwise_i8(x2)
+            xq, sx = ops.quant_rowwise_i8(x2) if norm is None else ops.rmsnorm_quant_rowwise_i8(x2, norm[0], norm[1])
             y = ops.linear_w8a8(xq, sx, self.qweight, self.w_scale, self.bias, out_dtype=x.dtype, residual=residual)
         return y.reshape(*lead, self.qweight.shape[0])
 

@@ -207,9 +207,11 @@ def linear_w8a8(xq, sx, wq, sw, bias=None, out_dtype=torch.bfloat16, residual=No
 
 
 def gemv_w8a8_decode(x, wq, sw, bias=None, out_dtype=None, workspace: Optional[torch.Tensor] = None,
-                     residual=None) -> torch.Tensor:
-    """Decode path for at most 16 rows of ``x [M, K]``: fused per-token quantise + int8 GEMV + epilogue."""
-    _need_gpu(x, wq, sw, bias, workspace, residual)
+                     residual=None, norm=None) -> torch.Tensor:
+    """Decode path for at most 16 rows of ``x [M, K]``: fused per-token quantise + int8 GEMV + epilogue.
+    ``norm = (gamma [K], eps)``: RMS-normalise the rows first (the codes ``rmsnorm_quant_rowwise_i8``
+    gives), in the same launch for up to 8 bfloat16 rows of at most 2048 elements."""
+    _need_gpu(x, wq, sw, bias, workspace, residual, norm[0] if norm is not None else None)
     x2 = _rows(x, "gemv_w8a8_decode")
     M, K = x2.shape
     N = wq.shape[0]
@@ -233,13 +235,26 @@ def gemv_w8a8_decode(x, wq, sw, bias=None, out_dtype=None, workspace: Optional[t
         raise ValueError(f"workspace holds {workspace.numel() * workspace.element_size()} bytes, {need} needed")
     r = _residual_arg(residual, M, N, out_dtype, x.device)
     y = torch.empty((M, N), dtype=out_dtype, device=x.device)
+    if norm is not None:
+        gamma, eps = norm
+        if gamma.dtype != x2.dtype or gamma.numel() != K:
+            raise ValueError(f"the norm's gain must be {x2.dtype} [{K}], got {gamma.dtype} {tuple(gamma.shape)}")
+        gamma = gamma.contiguous()
     if M and N:
         with torch.cuda.device(x.device):
-            rc = lib.aq_gemv_w8a8_decode_residual(x2.data_ptr(), _dt(x2, "x"), wq.data_ptr(), sw.data_ptr(),
-                                                  b.data_ptr() if b is not None else None, bdt,
-                                                  r.data_ptr() if r is not None else None, y.data_ptr(),
-                                                  _DT[out_dtype], M, N, K, workspace.data_ptr(),
-                                                  workspace.numel() * workspace.element_size(), _stream(x))
+            if norm is None:
+                rc = lib.aq_gemv_w8a8_decode_residual(x2.data_ptr(), _dt(x2, "x"), wq.data_ptr(), sw.data_ptr(),
+                                                      b.data_ptr() if b is not None else None, bdt,
+                                                      r.data_ptr() if r is not None else None, y.data_ptr(),
+                                                      _DT[out_dtype], M, N, K, workspace.data_ptr(),
+                                                      workspace.numel() * workspace.element_size(), _stream(x))
+            else:
+                rc = lib.aq_gemv_w8a8_decode_rmsnorm(x2.data_ptr(), _dt(x2, "x"), gamma.data_ptr(), float(eps),
+                                                     wq.data_ptr(), sw.data_ptr(),
+                                                     b.data_ptr() if b is not None else None, bdt,
+                                                     r.data_ptr() if r is not None else None, y.data_ptr(),
+                                                     _DT[out_dtype], M, N, K, workspace.data_ptr(),
+                                                     workspace.numel() * workspace.element_size(), _stream(x))
         _abi.check(rc, "aq_gemv_w8a8_decode")
     elif r is not None:
         y.copy_(r.view(M, N))

@@ -330,6 +330,29 @@ def test_gemv_decode_bit_exact(oracle, M, N, K):
         assert torch.equal(y2, y + r)
 
 
+@pytest.mark.parametrize("M", [1, 3, 4, 8, 12])
+@pytest.mark.parametrize("N,K", [(3072, 2048), (130, 1536), (2048, 4096), (50, 16)])
+def test_gemv_with_the_norm_folded_in_equals_norm_quantise_then_gemv(oracle, M, N, K):
+    """RMSNorm inside the decode GEMV (one launch for M <= 8, K <= 2048; two launches through the
+    workspace otherwise): the codes are those of the stand-alone norm-and-quantise kernel, which is
+    bit-exact against the oracle, so outputs must equal that kernel followed by the GEMV on codes."""
+    _say("gemv+rmsnorm", M, N, K)
+    g = torch.Generator().manual_seed(M * 31 + K)
+    x = (torch.randn(M, K, generator=g) * (0.1 + 4 * torch.rand(M, 1, generator=g))).to(torch.bfloat16).to(DEV)
+    gamma = (1 + 0.2 * torch.randn(K, generator=g)).to(torch.bfloat16).to(DEV)
+    w = make_x(N, K, 12) * 0.02
+    wq, sw = oracle.c_quant_rowwise_i8(w.numpy())
+    wqd, swd = torch.from_numpy(wq).to(DEV), torch.from_numpy(sw).to(DEV)
+    r = torch.randn(M, N, generator=g).to(torch.bfloat16).to(DEV)
+    xq, sx = ops.rmsnorm_quant_rowwise_i8(x, gamma, 1e-5)
+    qo, so = oracle.c_rmsnorm_quant_i8(bf16_bits(x), bf16_bits(gamma), 1e-5, bf16_bits=True)
+    assert np.array_equal(to_np(xq), qo) and np.array_equal(to_np(sx).view(np.uint32), so.view(np.uint32))
+    for res in (None, r):
+        want = ops.gemv_w8a8_codes(xq, sx, wqd, swd, out_dtype=torch.bfloat16, residual=res)
+        got = ops.gemv_w8a8_decode(x, wqd, swd, out_dtype=torch.bfloat16, residual=res, norm=(gamma, 1e-5))
+        assert torch.equal(got, want)
+
+
 def test_gemv_f32_in_out_and_agrees_with_gemm_path(oracle):
     M, N, K = 16, 1000, 2048
     x = make_x(M, K, 21, outlier_cols=4)

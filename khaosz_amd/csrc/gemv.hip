@@ -302,16 +302,21 @@ constexpr int GM_ROWS = 16;    // weight rows per wavefront
 constexpr int GM_MAX_WAVES = 8;
 constexpr int GM_BATCH = 8;    // MFMA steps (64 K bytes each) per register batch
 
+// KS, GR: K parts and row groups per workgroup fixed at compile time (the common 2 x 2 shape), or 0: taken
+// from the arguments.  RES: a residual is added (a compile-time switch: a conditional early load makes the
+// compiler drain the weight loads at the join, 0.4 us of a 6.5 us launch).
+template <int KS, int GR, bool RES>
 __global__ __launch_bounds__(GM_MAX_WAVES * 64) void gemv_mfma_kernel(GemvArgs p) {
   extern __shared__ __attribute__((aligned(16))) uint8_t xs[];  // [16][K + 16] token codes, [16] scales; later the partial sums
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int nthreads = p.ksplit * p.groups * 64;
-  const int grp = wave / p.ksplit, kh = wave % p.ksplit;
+  const int ksplit = KS ? KS : p.ksplit, groups = GR ? GR : p.groups;
+  const int nthreads = ksplit * groups * 64;
+  const int grp = wave / ksplit, kh = wave % ksplit;
   const int K = p.K, N = p.N, M = p.M;
-  const int n0 = __builtin_amdgcn_readfirstlane((blockIdx.x * p.groups + grp) * GM_ROWS);
+  const int n0 = __builtin_amdgcn_readfirstlane((blockIdx.x * groups + grp) * GM_ROWS);
   const int pitch = K + 16;  // 16 token rows then start 4 banks apart: conflict-free 16-byte reads
-  const int khalf = K / p.ksplit;  // a multiple of 64 (checked by the launcher)
+  const int khalf = K / ksplit;  // a multiple of 64 (checked by the launcher)
   const int nstep = khalf / 64;
 
   // epilogue operands first: lane l -> token l%16, rows (l/16)*4 .. +3 of the group
@@ -335,7 +340,7 @@ __global__ __launch_bounds__(GM_MAX_WAVES * 64) void gemv_mfma_kernel(GemvArgs p
       if (p.bias)
         bv[r] = p.bias_dtype == AQ_BF16 ? bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(p.bias)[n])
                                         : reinterpret_cast<const float*>(p.bias)[n];
-      if (p.res && tok < M)
+      if (RES && tok < M)
         rv[r] = p.y_dtype == AQ_BF16 ? reinterpret_cast<const uint16_t*>(p.res)[tok * p.ldr + n]
                                      : reinterpret_cast<const uint32_t*>(p.res)[tok * p.ldr + n];
     }
@@ -414,13 +419,13 @@ __global__ __launch_bounds__(GM_MAX_WAVES * 64) void gemv_mfma_kernel(GemvArgs p
 
   // sum the K parts: all but the first wavefront of each group park their 4 sums in LDS
   __syncthreads();  // everyone is done reading the token codes: the buffer is reused
-  int* part = reinterpret_cast<int*>(xs) + grp * (p.ksplit - 1) * 256;
+  int* part = reinterpret_cast<int*>(xs) + grp * (ksplit - 1) * 256;
   if (kh != 0) {
     *reinterpret_cast<v4i*>(part + (kh - 1) * 256 + lane * 4) = acc;
   }
   __syncthreads();
   if (kh != 0) return;
-  for (int k = 0; k < p.ksplit - 1; ++k) acc += *reinterpret_cast<const v4i*>(part + k * 256 + lane * 4);
+  for (int k = 0; k < ksplit - 1; ++k) acc += *reinterpret_cast<const v4i*>(part + k * 256 + lane * 4);
 
   if (tok >= M) return;
   float y[4];
@@ -428,7 +433,7 @@ __global__ __launch_bounds__(GM_MAX_WAVES * 64) void gemv_mfma_kernel(GemvArgs p
   for (int r = 0; r < 4; ++r) {
     y[r] = __fmul_rn(__fmul_rn((float)acc[r], sxv), swv[r]);
     if (p.bias) y[r] = __fadd_rn(y[r], bv[r]);
-    if (p.res) y[r] = p.y_dtype == AQ_BF16 ? add_residual_bf16(y[r], rv[r]) : __fadd_rn(y[r], __uint_as_float(rv[r]));
+    if constexpr (RES) y[r] = p.y_dtype == AQ_BF16 ? add_residual_bf16(y[r], rv[r]) : __fadd_rn(y[r], __uint_as_float(rv[r]));
   }
   const int64_t o = (int64_t)tok * N + rbase;
   if (p.y_dtype == AQ_BF16) {
@@ -474,12 +479,20 @@ static int launch_gemv_mfma(GemvArgs a, hipStream_t st) {
   }
   const unsigned grid = (unsigned)((a.N + GM_ROWS * a.groups - 1) / (GM_ROWS * a.groups));
   const size_t lds = (size_t)16 * (a.K + 16) + 16 * sizeof(float);
+  const bool fixed = a.ksplit == 2 && a.groups == 2, res = a.res != nullptr;
+  const void* fn = fixed ? (res ? reinterpret_cast<const void*>(&gemv_mfma_kernel<2, 2, true>)
+                                : reinterpret_cast<const void*>(&gemv_mfma_kernel<2, 2, false>))
+                         : (res ? reinterpret_cast<const void*>(&gemv_mfma_kernel<0, 0, true>)
+                                : reinterpret_cast<const void*>(&gemv_mfma_kernel<0, 0, false>));
   if (lds > 64 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_mfma_kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return (int)e;
   }
-  hipLaunchKernelGGL(gemv_mfma_kernel, dim3(grid), dim3(a.ksplit * a.groups * 64), lds, st, a);
+  const dim3 g(grid), b(a.ksplit * a.groups * 64);
+  if (fixed && res) hipLaunchKernelGGL((gemv_mfma_kernel<2, 2, true>), g, b, lds, st, a);
+  else if (fixed) hipLaunchKernelGGL((gemv_mfma_kernel<2, 2, false>), g, b, lds, st, a);
+  else if (res) hipLaunchKernelGGL((gemv_mfma_kernel<0, 0, true>), g, b, lds, st, a);
+  else hipLaunchKernelGGL((gemv_mfma_kernel<0, 0, false>), g, b, lds, st, a);
   return (int)hipGetLastError();
 }
 

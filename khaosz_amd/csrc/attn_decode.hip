@@ -100,37 +100,43 @@ constexpr int ATT_KPW = 64;                  // positions per wavefront
 constexpr int ATT_KPG = ATT_WAVES * ATT_KPW; // positions per workgroup
 constexpr int ATT_MAX_D = 128;
 
-// sum over each group of LANES (8 or 16) consecutive lanes, result in all of them
-template <int LANES>
-__device__ __forceinline__ float lanes_sum(float v) {
-  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xf, 0xf, false));   // quad_perm [1,0,3,2]
-  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xf, 0xf, false));   // quad_perm [2,3,0,1]
-  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xf, 0xf, false));  // row_half_mirror
-  if constexpr (LANES == 16)
-    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xf, 0xf, false));  // row_mirror
+// maximum / sum over each row of 16 consecutive lanes, result in all of them
+__device__ __forceinline__ float row16_max(float v) {
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xf, 0xf, false)));   // quad_perm [1,0,3,2]
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xf, 0xf, false)));   // quad_perm [2,3,0,1]
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xf, 0xf, false)));  // row_half_mirror
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xf, 0xf, false)));  // row_mirror
+  return v;
+}
+__device__ __forceinline__ float row16_sum(float v) {
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xf, 0xf, false));
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xf, 0xf, false));
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xf, 0xf, false));
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xf, 0xf, false));
   return v;
 }
 
-__device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float c) {
-  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a), __builtin_bit_cast(bf16x2, b), c, false);
-}
+typedef __bf16 attn_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float attn_f32x4 __attribute__((ext_vector_type(4)));
 
 // Workgroup = one (sequence, KV head, slice of the cached positions): the G
 // query heads of the KV head share every K and V byte.  A wavefront owns 64
 // consecutive positions, a workgroup 256; the NS slices of a sequence run as
 // separate workgroups so that a decode batch of a few sequences still spreads
-// over the device.  Rows are read 16 bytes per lane: a load instruction covers
-// RPL = 1024 / (2 D) whole rows (lane = CPR * key + chunk, CPR = D / 8 chunks
-// per row), 64 / RPL of them for K and as many for V are requested before
-// anything is computed.
-//   scores   every lane dots its 8 dimensions with the G queries (packed bf16
-//            dot product, fp32 accumulation), a DPP butterfly sums the CPR lanes
-//            of a row, and lane (chunk = i, key = j) keeps the score of key
-//            RPL * i + j of the batch -- one key per lane for the softmax;
-//   softmax  maximum and denominator across the wavefront, probabilities to LDS;
-//   values   lane accumulates p * V over the keys it loaded (8 dimensions x G
-//            heads), the RPL key groups are summed with xor shuffles.
+// over the device.  Every K and V load of a wavefront, 16 bytes per lane, is
+// requested before anything is computed.
+//   scores   on the matrix core: S[head, key] = Q K^T as v_mfma_f32_16x16x32_bf16
+//            tiles, the G <= 8 query heads padded to 16 rows, four tiles of 16
+//            keys, D / 32 steps each.  K rows are loaded straight in operand
+//            order (lane l: key l % 16 of the tile, dimensions 8 (l / 16) .. + 8
+//            of the step), queries likewise; a lane ends up with the scores of
+//            one key per tile for 4 heads;
+//   softmax  maximum and denominator over a row of 16 lanes by DPP and over the
+//            four tiles in registers; probabilities to LDS;
+//   values   V rows are loaded CPR = D / 8 lanes to a row (a load covers 4 or 8
+//            whole rows); a lane accumulates p * V over the keys it loaded (8
+//            dimensions x G heads, fma), the key groups are summed with xor
+//            shuffles.
 // The wavefronts' (maximum, denominator, numerator) are merged through LDS and
 // either normalised into the output (NS == 1) or left in the workspace for
 // attn_merge_kernel.
@@ -162,11 +168,11 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void paged_attn_decode_kernel(AttnA
   const int64_t T = p.T;
   const int64_t t0 = (int64_t)split * KPG + wave * KPW;  // first position of this wavefront
 
-  float m[G], l[G], acc[G][8];
+  constexpr int KS = D / 32;                  // matrix-core steps over the head dimension
+  const int col = lane & 15, kq = lane >> 4;  // operand row / column, group of 8 dimensions inside a step
+  float acc[G][8];
 #pragma unroll
   for (int g = 0; g < G; ++g) {
-    m[g] = -INFINITY;
-    l[g] = 0.0f;
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc[g][e] = 0.0f;
   }
@@ -181,77 +187,97 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void paged_attn_decode_kernel(AttnA
         if (phys >= 0 && phys < p.n_pages) row = ((phys * p.page + t % p.page) * p.Hkv + kvh) * D;
       }
     }
-    uint4 qv[G];  // this lane's 8 dimensions of each query
-    uint4 knew = make_uint4(0, 0, 0, 0), vnew = make_uint4(0, 0, 0, 0);
-    const bool has_new = ROPE && T - 1 >= t0 && T - 1 < t0 + KPW;  // wavefront-uniform
-    if constexpr (ROPE) {
-      const int64_t heads = p.Hq + 2 * p.Hkv;
-      const uint16_t* tok = p.qkv + (int64_t)b * heads * D;
-      const float* cs = p.freqs + (int64_t)b * p.freqs_stride + ch * 8;
-#pragma unroll
-      for (int g = 0; g < G; ++g)
-        qv[g] = rope8(*reinterpret_cast<const uint4*>(tok + (int64_t)(kvh * G + g) * D + ch * 8), cs);
-      if (has_new) {
-        knew = rope8(*reinterpret_cast<const uint4*>(tok + (int64_t)(p.Hq + kvh) * D + ch * 8), cs);
-        vnew = *reinterpret_cast<const uint4*>(tok + (int64_t)(p.Hq + p.Hkv + kvh) * D + ch * 8);
-      }
-    } else {
-#pragma unroll
-      for (int g = 0; g < G; ++g)
-        qv[g] = *reinterpret_cast<const uint4*>(p.q + ((int64_t)b * p.Hq + kvh * G + g) * D + ch * 8);
-    }
-    uint4 kv[NL], vv[NL];
-#pragma unroll
-    for (int i = 0; i < NL; ++i) {
-      const int src = i * RPL + sub;
+    auto row_of = [&](int src) -> int64_t {
       const int lo = __shfl((int)(uint32_t)row, src, 64), hi = __shfl((int)(row >> 32), src, 64);
-      const int64_t r = ((int64_t)hi << 32) | (uint32_t)lo;
-      kv[i] = make_uint4(0, 0, 0, 0);
-      vv[i] = make_uint4(0, 0, 0, 0);
-      if (r >= 0) {
-        if (ROPE && has_new && t0 + src == T - 1) {  // the new token: from registers, and into its slot
-          kv[i] = knew;
-          vv[i] = vnew;
-          *reinterpret_cast<uint4*>(p.kc_w + r + ch * 8) = knew;
-          *reinterpret_cast<uint4*>(p.vc_w + r + ch * 8) = vnew;
+      return ((int64_t)hi << 32) | (uint32_t)lo;
+    };
+    const bool has_new = ROPE && T - 1 >= t0 && T - 1 < t0 + KPW;  // wavefront-uniform
+    // ---- operands of the scores.  Queries: lane = (head col, dimensions ks * 32 + kq * 8 .. + 8); heads past G
+    // are zero rows (their loads read head 0).
+    uint4 qa[KS];
+    {
+      const int hq = col < G ? col : 0;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const int d0 = ks * 32 + kq * 8;
+        if constexpr (ROPE) {
+          const uint16_t* tok = p.qkv + (int64_t)b * (p.Hq + 2 * p.Hkv) * D;
+          qa[ks] = rope8(*reinterpret_cast<const uint4*>(tok + (int64_t)(kvh * G + hq) * D + d0),
+                         p.freqs + (int64_t)b * p.freqs_stride + d0);
         } else {
-          kv[i] = *reinterpret_cast<const uint4*>(p.kc + r + ch * 8);
-          vv[i] = *reinterpret_cast<const uint4*>(p.vc + r + ch * 8);
+          qa[ks] = *reinterpret_cast<const uint4*>(p.q + ((int64_t)b * p.Hq + kvh * G + hq) * D + d0);
+        }
+        if (col >= G) qa[ks] = make_uint4(0, 0, 0, 0);
+      }
+    }
+    // keys: tile t holds positions t0 + 16 t .. + 16; lane = (key col, the same dimensions).  Rows that are
+    // unmapped or past T read row 0 of the cache and are zeroed.
+    uint4 kb[4][KS];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const int64_t r = row_of(t * 16 + col);
+      const uint16_t* src = p.kc + (r >= 0 ? r : 0);
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        kb[t][ks] = *reinterpret_cast<const uint4*>(src + ks * 32 + kq * 8);
+        if (r < 0) kb[t][ks] = make_uint4(0, 0, 0, 0);
+      }
+      if (ROPE && has_new && r >= 0 && t0 + t * 16 + col == T - 1) {  // the new key: rotated here, used and stored
+        const uint16_t* tok = p.qkv + ((int64_t)b * (p.Hq + 2 * p.Hkv) + p.Hq + kvh) * D;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          const int d0 = ks * 32 + kq * 8;
+          kb[t][ks] = rope8(*reinterpret_cast<const uint4*>(tok + d0), p.freqs + (int64_t)b * p.freqs_stride + d0);
+          *reinterpret_cast<uint4*>(p.kc_w + r + d0) = kb[t][ks];
         }
       }
     }
-    // ---- scores
-    float sc[G];
-#pragma unroll
-    for (int g = 0; g < G; ++g) sc[g] = 0.0f;
+    // values: lane = (key sub of a load, 16-byte chunk ch of the row)
+    uint4 vv[NL];
 #pragma unroll
     for (int i = 0; i < NL; ++i) {
-#pragma unroll
-      for (int g = 0; g < G; ++g) {
-        float d = dot2_bf16(kv[i].x, qv[g].x, 0.0f);
-        d = dot2_bf16(kv[i].y, qv[g].y, d);
-        d = dot2_bf16(kv[i].z, qv[g].z, d);
-        d = dot2_bf16(kv[i].w, qv[g].w, d);
-        d = lanes_sum<CPR>(d);
-        if (ch == i) sc[g] = d;
+      const int64_t r = row_of(i * RPL + sub);
+      vv[i] = *reinterpret_cast<const uint4*>(p.vc + (r >= 0 ? r : 0) + ch * 8);
+      if (r < 0) vv[i] = make_uint4(0, 0, 0, 0);
+      if (ROPE && has_new && r >= 0 && t0 + i * RPL + sub == T - 1) {  // the new value
+        vv[i] = *reinterpret_cast<const uint4*>(p.qkv + ((int64_t)b * (p.Hq + 2 * p.Hkv) + p.Hq + p.Hkv + kvh) * D + ch * 8);
+        *reinterpret_cast<uint4*>(p.vc_w + r + ch * 8) = vv[i];
       }
     }
-    // ---- softmax over the wavefront's positions: this lane owns position t0 + RPL * ch + sub
-    const int own = ch * RPL + sub;
-    const bool valid = t0 + own < T;
+    // ---- scores: S[head][key] per tile; this lane gets key col of the tile, heads 4 kq .. + 4
+    attn_f32x4 sc[4];
 #pragma unroll
-    for (int g = 0; g < G; ++g) {
-      const float sv = valid ? sc[g] * p.scale_log2e : -INFINITY;
-      float bm = sv;
+    for (int t = 0; t < 4; ++t) {
+      attn_f32x4 c = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-      for (int off = 32; off > 0; off >>= 1) bm = fmaxf(bm, __shfl_xor(bm, off, 64));
-      const float pv = valid ? exp2f(sv - bm) : 0.0f;  // bm is finite: position t0 is valid
-      float ps = pv;
+      for (int ks = 0; ks < KS; ++ks)
+        c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(attn_bf16x8, qa[ks]),
+                                                   __builtin_bit_cast(attn_bf16x8, kb[t][ks]), c, 0, 0, 0);
+      sc[t] = c;
+    }
+    // ---- softmax over the wavefront's 64 positions, per head
 #pragma unroll
-      for (int off = 32; off > 0; off >>= 1) ps += __shfl_xor(ps, off, 64);
-      m[g] = bm;
-      l[g] = ps;
-      p_s[wave][own][g] = pv;
+    for (int r = 0; r < 4; ++r) {
+      const int head = 4 * kq + r;
+      float sv[4], mx = -INFINITY;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        sv[t] = t0 + t * 16 + col < T ? sc[t][r] * p.scale_log2e : -INFINITY;
+        mx = fmaxf(mx, sv[t]);
+      }
+      mx = row16_max(mx);  // finite: position t0 is valid
+      float sum = 0.0f;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const float pv = exp2f(sv[t] - mx);  // 0 for positions past T
+        sum += pv;
+        if (head < G) p_s[wave][t * 16 + col][head] = pv;
+      }
+      sum = row16_sum(sum);
+      if (col == 0 && head < G) {
+        m_s[wave][head] = mx;
+        l_s[wave][head] = sum;
+      }
     }
     __builtin_amdgcn_s_waitcnt(0xc07f);  // this wavefront's LDS writes are done (wavefront-private region)
     asm volatile("" ::: "memory");
@@ -281,14 +307,13 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void paged_attn_decode_kernel(AttnA
 #pragma unroll
         for (int off = CPR; off < 64; off <<= 1) acc[g][e] += __shfl_xor(acc[g][e], off, 64);
       }
+  } else if (lane < G) {  // a wavefront past T: nothing to add
+    m_s[wave][lane] = -INFINITY;
+    l_s[wave][lane] = 0.0f;
   }
   // ---- merge the wavefronts' partial results
 #pragma unroll
   for (int g = 0; g < G; ++g) {
-    if (lane == 0) {
-      m_s[wave][g] = m[g];
-      l_s[wave][g] = l[g];
-    }
     if (sub == 0) {
       *reinterpret_cast<float4*>(&acc_s[wave][g][ch * 8]) = make_float4(acc[g][0], acc[g][1], acc[g][2], acc[g][3]);
       *reinterpret_cast<float4*>(&acc_s[wave][g][ch * 8 + 4]) = make_float4(acc[g][4], acc[g][5], acc[g][6], acc[g][7]);

@@ -611,17 +611,21 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(GemmArgs p) {
 }
 
 // 256-row tiles unless they leave much of the device idle: a workgroup per compute unit at a
-// time, so the cost of a launch is its number of rounds over the 256 compute units, and a
-// 128-row tile costs a little over half of a 256-row one.
+// time, so the cost of a launch is its number of rounds over the 256 compute units.  Measured:
+// a round of 128-row tiles costs 0.72 of a round of 256-row ones, and a last round that fills
+// only part of the device costs about half a round plus half its fill (384 large tiles, 1.5
+// rounds, take 1.74 times as long as 256).
 static int g_forced_tile = 0;  // 0: by shape; 128 / 256: forced (tuning and tests)
 
 static bool use_small_tile(int64_t M, int64_t N) {
   if (g_forced_tile) return g_forced_tile == 128;
   constexpr int64_t CUS = 256;
   const int64_t tn = (N + BN - 1) / BN;
-  const int64_t rounds_big = ((M + 255) / 256 * tn + CUS - 1) / CUS;
-  const int64_t rounds_small = ((M + 127) / 128 * tn + CUS - 1) / CUS;
-  return rounds_small * 0.6 < (double)rounds_big;
+  auto rounds = [](int64_t tiles) {
+    const int64_t full = tiles / CUS, rest = tiles % CUS;
+    return (double)full + (rest ? 0.5 + 0.5 * (double)rest / CUS : 0.0);
+  };
+  return 0.72 * rounds((M + 127) / 128 * tn) < rounds((M + 255) / 256 * tn);
 }
 
 template <bool FP8, int OUT>

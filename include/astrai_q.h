@@ -221,6 +221,21 @@ int aq_rope_paged_attn_decode(const void *qkv, const float *freqs, int64_t freqs
                               float scale, void *out, int64_t B, int64_t Hq, int64_t Hkv, int64_t D,
                               void *workspace, int64_t workspace_bytes, void *stream);
 
+/* Causal self-attention over a prompt, for a prefill that starts from an empty
+ * cache (query and key positions coincide): out[b, s, h, :] =
+ * softmax_{t <= s}(scale * q[b,s,h] . k[b,t,h/G]) v[b,t,h/G], G = Hq / Hkv.
+ * Replaces repeat_kv (attention.py:15-23) + scaled_dot_product_attention with
+ * is_causal (attention.py:93-100) for that case, without repeating heads.
+ * Element (b, s, h, d) of q sits at q + (b*S + s)*q_stride + h*D + d, likewise
+ * k and v with their own token strides (elements, multiples of 8) -- so v can be
+ * read in place from the fused q/k/v projection's output; out is [B, S, Hq, D].
+ * bf16, D = 64 or 128, fp32 scores and sums on the matrix core; results within
+ * bf16 rounding of the reference flow (probabilities are rounded to bf16 before
+ * they multiply V, as flash-attention kernels do). */
+int aq_prefill_attn_causal(const void *q, int64_t q_stride, const void *k, int64_t k_stride,
+                           const void *v, int64_t v_stride, void *out, float scale, int64_t B,
+                           int64_t S, int64_t Hq, int64_t Hkv, int64_t D, void *stream);
+
 /* Tuning and test hook, no counterpart in the reference: the GEMM entry points
  * pick their workgroup tile (256 x 128, or 128 x 128 with a split K step when
  * the larger one would leave compute units idle) from M and N.  rows = 128 or

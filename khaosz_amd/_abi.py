@@ -36,6 +36,8 @@ SYMBOLS = {
                                 _i64, _vp]),
     "aq_paged_attn_decode": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, ctypes.c_float, _vp, _i64, _i64, _i64, _i64,
                                     _vp, _i64, _vp]),
+    "aq_prefill_attn_causal": (_int, [_vp, _i64, _vp, _i64, _vp, _i64, _vp, ctypes.c_float, _i64, _i64, _i64, _i64, _i64,
+                                      _vp]),
     "aq_paged_attn_decode_workspace_bytes": (_i64, [_i64, _i64, _i64, _i64]),
     "aq_rope_paged_attn_decode": (_int, [_vp, _vp, _i64, _vp, _i64, _i64, _i64, _vp, _vp, _i64, ctypes.c_float, _vp,
                                          _i64, _i64, _i64, _i64, _vp, _i64, _vp]),

@@ -245,8 +245,8 @@ class GQA(nn.Module):
             return self._out(out.view(B, 1, -1), residual)
         if (self._decode_attention and isinstance(cache, PagedKV) and x.is_cuda and x.dtype == torch.bfloat16
                 and S <= cache.total_len):
-            # several new tokens (prefill): rotation and the page writes as one launch; the attention
-            # itself stays the stock one, over the new keys directly when nothing older is cached
+            # several new tokens (prefill): rotation and the page writes as one launch; a prompt on an empty
+            # cache then runs the causal attention kernel, anything else the stock attention
             nq, nkv = self.n_heads * self.head_dim, self.n_kv_heads * self.head_dim
             qkv = self._project_qkv(x, codes, norm)
             start = cache.total_len - S
@@ -254,6 +254,8 @@ class GQA(nn.Module):
                                      cache.v_layers[self.layer_id], self.n_heads, self.n_kv_heads, return_k=True)
             if start == 0 and cache.all_mapped:
                 v = qkv[..., nq + nkv:].view(B, S, self.n_kv_heads, self.head_dim)
+                if attn_mask is None:  # a prompt attending to itself: the causal kernel, v read in place from qkv
+                    return self._out(ops.prefill_attn_causal(q, k, v).view(B, S, -1), residual)
             else:
                 k, v = cache.gather(self.layer_id)
             out = F.scaled_dot_product_attention(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), attn_mask,

@@ -12,7 +12,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(HERE, "lib", "obj")
 LIB = os.path.join(HERE, "lib", "libastrai_q.so")
-SOURCES = ["abi.hip", "quant.hip", "gemm_mfma.hip", "gemv.hip", "attn_decode.hip", "probe.hip"]
+SOURCES = ["abi.hip", "quant.hip", "gemm_mfma.hip", "gemv.hip", "attn_decode.hip", "attn_prefill.hip", "probe.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [

@@ -1,0 +1,286 @@
+// Causal self-attention over a prompt (prefill from an empty cache): what the
+// reference computes with repeat_kv + scaled_dot_product_attention
+// (astrai/model/components/attention.py:15-23, 93-100) when the query and key
+// positions coincide.  Grouped-query attention without repeating heads, bf16
+// tensors, fp32 softmax statistics and accumulation, head dimension 64 or 128.
+//
+// Workgroup = (128 query positions, one query head, one sequence), 4 wavefronts
+// of 32 query rows; K/V are walked in blocks of 64 positions up to the causal
+// limit.  Everything is computed transposed so that no register ever has to
+// change lanes:
+//
+//   S^T[key, q] = K Q^T    v_mfma_f32_32x32x16_bf16 with A = K (rows of the LDS
+//                          tile, 16-byte reads), B = Q^T (the wavefront's query
+//                          rows, held in registers for the whole kernel).  A
+//                          lane ends up with the scores of ONE query (column
+//                          l % 32) against 16 keys per 32-key tile.
+//   softmax                per query = per lane: running maximum and denominator
+//                          need one exchange with lane l ^ 32 per block, the
+//                          rescale of the output accumulator is lane-wise.
+//   O^T[d, q] += V^T P^T   B = P^T: the probabilities a lane already holds are,
+//                          packed to bf16 in register order, exactly its operand
+//                          (the matrix core does not care which key sits in which
+//                          k slot as long as A agrees); A = V^T read from an LDS
+//                          tile that was written transposed ([d][key]) when the
+//                          block was staged, two 8-byte reads per operand.
+//
+// The next block's K and V are fetched into registers while the current one is
+// being multiplied.
+#include "aq_common.h"
+
+namespace aq {
+
+struct PrefillAttnArgs {
+  const uint16_t* q;   // element (b, s, h, d) at q + (b*S + s)*q_stride + h*D + d
+  const uint16_t* k;   // likewise with KV heads
+  const uint16_t* v;
+  uint16_t* out;       // [B, S, Hq, D]
+  int64_t q_stride, k_stride, v_stride;  // elements between consecutive tokens
+  float scale_log2e;
+  int S, Hq, Hkv;
+};
+
+typedef __bf16 pa_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float pa_f32x16 __attribute__((ext_vector_type(16)));
+
+constexpr int PA_QB = 128;  // query rows per workgroup
+constexpr int PA_KB = 64;   // keys per block
+
+// Two workgroups per compute unit (2 wavefronts per SIMD, at most 256 registers each): the other workgroup's
+// matrix work is what overlaps this one's softmax and staging.
+template <int D>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void prefill_attn_kernel(PrefillAttnArgs p) {
+  constexpr int KP = D + 8;       // K tile row pitch (elements): 16-byte reads of 32 rows hit distinct banks
+  constexpr int VP = PA_KB + 4;   // V^T tile row pitch
+  constexpr int DSTEPS = D / 16;  // matrix-core steps over the head dimension
+  constexpr int DT = D / 32;      // 32-row tiles of the transposed output
+  constexpr int CPT = PA_KB * (D / 8) / 256;  // 16-byte chunks of a K (or V) block per thread: 2 or 4
+  constexpr int KS_ELEMS = PA_KB * KP, VT_ELEMS = D * VP;
+  extern __shared__ __align__(16) uint16_t pa_lds[];  // [K tile | V^T tile]
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int col = lane & 31, g = lane >> 5;
+  const int S = p.S;
+  const int q0 = blockIdx.x * PA_QB, h = blockIdx.y, b = blockIdx.z;
+  const int kvh = h / (p.Hq / p.Hkv);
+  const int qw0 = q0 + wave * 32;          // first query row of this wavefront
+  const int qpos = qw0 + col;              // this lane's query
+  const int64_t tok0 = (int64_t)b * S;
+
+  // Q^T operand: lane = (query col, dimensions 16 step + 8 g .. + 8); rows past S read row S - 1
+  uint4 qf[DSTEPS];
+  {
+    const int qr = qpos < S ? qpos : S - 1;
+    const uint16_t* src = p.q + (tok0 + qr) * p.q_stride + (int64_t)h * D + g * 8;
+#pragma unroll
+    for (int st = 0; st < DSTEPS; ++st) qf[st] = *reinterpret_cast<const uint4*>(src + st * 16);
+  }
+  // staging, fetched one block ahead: 16-byte chunks (key, 8 dimensions).  K chunks go to threads in memory
+  // order (coalesced loads, row-major LDS tile).  V is written transposed; there a wavefront's lanes take
+  // consecutive KEYS of one chunk column, so that the stores of an instruction fall into consecutive LDS
+  // words instead of 4 banks.
+  // (scalars, not arrays: the compiler kept a 4-element array of these in scratch memory)
+  uint4 kreg0, kreg1, kreg2, kreg3, vreg0, vreg1, vreg2, vreg3;
+  kreg2 = kreg3 = vreg2 = vreg3 = make_uint4(0, 0, 0, 0);
+  auto fetch1 = [&](int j, int c, uint4& kr_out, uint4& vr_out) __attribute__((always_inline)) {
+    const int idx = c * 256 + tid, key = idx / (D / 8), ch = idx % (D / 8);
+    int kr = j * PA_KB + key;
+    kr = kr < S ? kr : S - 1;  // past the prompt: any valid row, masked by causality
+    kr_out = *reinterpret_cast<const uint4*>(p.k + (tok0 + kr) * p.k_stride + (int64_t)kvh * D + ch * 8);
+    int vr = j * PA_KB + lane;
+    vr = vr < S ? vr : S - 1;
+    vr_out = *reinterpret_cast<const uint4*>(p.v + (tok0 + vr) * p.v_stride + (int64_t)kvh * D + (wave + 4 * c) * 8);
+  };
+  auto stage1 = [&](uint16_t* ks, uint16_t* vt, int c, const uint4& kr_in, const uint4& vr_in) __attribute__((always_inline)) {
+    const int idx = c * 256 + tid, key = idx / (D / 8), ch = idx % (D / 8);
+    *reinterpret_cast<uint4*>(&ks[key * KP + ch * 8]) = kr_in;
+    // V chunk (key = lane, dimensions 8 (wave + 4 c) .. + 8) into the transposed tile, two keys per 4-byte
+    // store: neighbouring lanes swap dwords (DPP) and byte-permute them into "one dimension, both keys" --
+    // even lanes then hold the even dimensions of the key pair, odd lanes the odd ones.
+    const bool odd = lane & 1;
+    const uint32_t sel = odd ? 0x03020706u : 0x05040100u;
+    uint32_t* vdst = reinterpret_cast<uint32_t*>(&vt[((wave + 4 * c) * 8 + (odd ? 1 : 0)) * VP + (lane & ~1)]);
+    const uint32_t w[4] = {vr_in.x, vr_in.y, vr_in.z, vr_in.w};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const uint32_t other = (uint32_t)__builtin_amdgcn_mov_dpp((int)w[e], 0xB1 /* quad_perm [1,0,3,2] */, 0xf, 0xf, true);
+      // even lane: {mine.lo, other.lo} = dimension 2e of keys (lane, lane + 1); odd: {other.hi, mine.hi} = 2e + 1
+      vdst[e * VP] = __builtin_amdgcn_perm(other, w[e], sel);  // e * VP words = 2e rows of VP halfwords
+    }
+  };
+#define PA_FETCH(J)                        \
+  fetch1((J), 0, kreg0, vreg0);            \
+  fetch1((J), 1, kreg1, vreg1);            \
+  if constexpr (CPT > 2) {                 \
+    fetch1((J), 2, kreg2, vreg2);          \
+    fetch1((J), 3, kreg3, vreg3);          \
+  }
+#define PA_STAGE(BUF)                                                        \
+  {                                                                          \
+    uint16_t* ks_w = pa_lds + (BUF) * (KS_ELEMS + VT_ELEMS);                  \
+    uint16_t* vt_w = ks_w + KS_ELEMS;                                        \
+    stage1(ks_w, vt_w, 0, kreg0, vreg0);                                     \
+    stage1(ks_w, vt_w, 1, kreg1, vreg1);                                     \
+    if constexpr (CPT > 2) {                                                 \
+      stage1(ks_w, vt_w, 2, kreg2, vreg2);                                   \
+      stage1(ks_w, vt_w, 3, kreg3, vreg3);                                   \
+    }                                                                        \
+  }
+
+  pa_f32x16 o[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[dt][r] = 0.0f;
+  float m = -INFINITY, l = 0.0f;  // running maximum of this lane's query; this lane's half of its denominator
+
+  const int last_q = (q0 + PA_QB < S ? q0 + PA_QB : S) - 1;
+  const int nblk = last_q / PA_KB + 1;  // blocks that hold a key some query of the workgroup may see
+  // One LDS buffer, two barriers per block; the next block's global loads are in flight while this one is
+  // multiplied.  (Two buffers with one barrier per block measured 15 % slower.)
+  const uint16_t* ks = pa_lds;
+  const uint16_t* vt = pa_lds + KS_ELEMS;
+  PA_FETCH(0)
+  for (int j = 0; j < nblk; ++j) {
+    __syncthreads();  // everyone is done reading the previous block's tiles
+    PA_STAGE(0)
+    __syncthreads();
+    if (j + 1 < nblk) {
+      PA_FETCH(j + 1)
+    }
+    const int kb0 = j * PA_KB;
+    if (kb0 > qw0 + 31) continue;  // wavefront-uniform: every key of the block is ahead of every query here
+    // ---- scores, transposed: two tiles of 32 keys
+    pa_f32x16 s[2];
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt) {
+      pa_f32x16 c;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) c[r] = 0.0f;
+      const uint16_t* krow = &ks[(kt * 32 + col) * KP + g * 8];
+#pragma unroll
+      for (int st = 0; st < DSTEPS; ++st) {
+        const uint4 a = *reinterpret_cast<const uint4*>(krow + st * 16);
+        c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(pa_bf16x8, a), __builtin_bit_cast(pa_bf16x8, qf[st]),
+                                                   c, 0, 0, 0);
+      }
+      s[kt] = c;
+    }
+    // ---- online softmax for this lane's query; register r of tile kt is key kb0 + 32 kt + 8 (r / 4) + 4 g + r % 4.
+    // Scores stay unscaled; the scale (> 0) is applied to the maximum and inside the exponent's fma.
+    const bool diag = kb0 + PA_KB - 1 > qw0;  // wavefront-uniform: some key of the block is ahead of some query
+    float bm = -INFINITY;
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        if (diag && kb0 + kt * 32 + 8 * (r / 4) + 4 * g + (r % 4) > qpos) s[kt][r] = -INFINITY;
+        bm = fmaxf(bm, s[kt][r]);
+      }
+    bm = fmaxf(bm, __shfl_xor(bm, 32, 64)) * p.scale_log2e;
+    // The running maximum only has to bound the exponents, not equal the true maximum: it is raised (and the
+    // accumulators rescaled) only when some query of the wavefront would otherwise see an exponent above 2^8;
+    // with probabilities up to 256 nothing overflows and bf16 keeps its relative precision.  After the first
+    // blocks this is rare, and the 64-register rescale is skipped.
+    const bool raise = __builtin_amdgcn_ballot_w64(bm > m + 8.0f) != 0;  // m = -inf in block 0: raised there
+    float alpha = 1.0f;
+    if (raise) {
+      const float mn = fmaxf(m, bm);  // finite from block 0 on: key 0 is visible to every query
+      alpha = __builtin_amdgcn_exp2f(m - mn);
+      m = mn;
+      l *= alpha;
+    }
+    float ps = 0.0f;
+    uint4 pf[2][2];  // P^T operands: tile kt, keys 16 s2 .. + 16
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt) {
+      float pv[16];
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        pv[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][r], p.scale_log2e, -m));
+        ps += pv[r];
+      }
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2)
+        pf[kt][s2] = make_uint4(pack_bf16x2(pv[8 * s2 + 0], pv[8 * s2 + 1]), pack_bf16x2(pv[8 * s2 + 2], pv[8 * s2 + 3]),
+                                pack_bf16x2(pv[8 * s2 + 4], pv[8 * s2 + 5]), pack_bf16x2(pv[8 * s2 + 6], pv[8 * s2 + 7]));
+    }
+    l += ps;
+    // ---- output, transposed: O^T[d, q] = alpha O^T + V^T P^T
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      pa_f32x16 c = o[dt];
+      if (raise) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) c[r] *= alpha;
+      }
+      const uint16_t* vrow = &vt[(dt * 32 + col) * VP + 4 * g];
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+          // k slots of this lane group: keys 32 kt + 16 s2 + {4 g .. + 4, 8 + 4 g .. + 4}
+          const uint2 lo = *reinterpret_cast<const uint2*>(vrow + kt * 32 + s2 * 16);
+          const uint2 hi = *reinterpret_cast<const uint2*>(vrow + kt * 32 + s2 * 16 + 8);
+          const uint4 a = make_uint4(lo.x, lo.y, hi.x, hi.y);
+          c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(pa_bf16x8, a),
+                                                     __builtin_bit_cast(pa_bf16x8, pf[kt][s2]), c, 0, 0, 0);
+        }
+      o[dt] = c;
+    }
+  }
+  // ---- normalise and store: register r of tile dt is dimension 32 dt + 8 (r / 4) + 4 g + r % 4 of query col
+  l += __shfl_xor(l, 32, 64);
+  if (qpos < S) {
+    const float inv = 1.0f / l;
+    uint16_t* dst = p.out + ((tok0 + qpos) * p.Hq + h) * D + 4 * g;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int a = 0; a < 4; ++a) {
+        uint2 w;
+        w.x = pack_bf16x2(o[dt][4 * a + 0] * inv, o[dt][4 * a + 1] * inv);
+        w.y = pack_bf16x2(o[dt][4 * a + 2] * inv, o[dt][4 * a + 3] * inv);
+        *reinterpret_cast<uint2*>(dst + dt * 32 + 8 * a) = w;
+      }
+  }
+}
+
+#undef PA_FETCH
+#undef PA_STAGE
+
+}  // namespace aq
+
+extern "C" int aq_prefill_attn_causal(const void* q, int64_t q_stride, const void* k, int64_t k_stride, const void* v,
+                                      int64_t v_stride, void* out, float scale, int64_t B, int64_t S, int64_t Hq,
+                                      int64_t Hkv, int64_t D, void* stream) {
+  if (D != 64 && D != 128) return AQ_E_SHAPE;
+  if (B < 0 || S < 0 || Hq <= 0 || Hkv <= 0 || (Hq % Hkv) != 0 || !(scale > 0.0f)) return AQ_E_SHAPE;
+  if (q_stride < Hq * D || k_stride < Hkv * D || v_stride < Hkv * D) return AQ_E_SHAPE;
+  if (B == 0 || S == 0) return AQ_OK;
+  if (!q || !k || !v || !out) return AQ_E_NULL;
+  if (aq::check_ptr16(q) || aq::check_ptr16(k) || aq::check_ptr16(v) || aq::check_ptr16(out) || (q_stride & 7) ||
+      (k_stride & 7) || (v_stride & 7))
+    return AQ_E_ALIGN;
+  if (S > (1 << 30) || Hq > 65535 || B > 65535) return AQ_E_RANGE;
+  aq::PrefillAttnArgs a{};
+  a.q = static_cast<const uint16_t*>(q);
+  a.k = static_cast<const uint16_t*>(k);
+  a.v = static_cast<const uint16_t*>(v);
+  a.out = static_cast<uint16_t*>(out);
+  a.q_stride = q_stride;
+  a.k_stride = k_stride;
+  a.v_stride = v_stride;
+  a.scale_log2e = scale * 1.44269504088896341f;
+  a.S = (int)S;
+  a.Hq = (int)Hq;
+  a.Hkv = (int)Hkv;
+  const dim3 grid((unsigned)((S + aq::PA_QB - 1) / aq::PA_QB), (unsigned)Hq, (unsigned)B);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const size_t lds = (size_t)(aq::PA_KB * (D + 8) + D * (aq::PA_KB + 4)) * sizeof(uint16_t);  // 34 KiB at most
+  if (D == 128)
+    hipLaunchKernelGGL(aq::prefill_attn_kernel<128>, grid, dim3(256), lds, st, a);
+  else
+    hipLaunchKernelGGL(aq::prefill_attn_kernel<64>, grid, dim3(256), lds, st, a);
+  return (int)hipGetLastError();
+}

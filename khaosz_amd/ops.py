@@ -388,6 +388,36 @@ def rope_paged_attn_decode(qkv: torch.Tensor, freqs: torch.Tensor, page_table: t
     return out
 
 
+def prefill_attn_causal(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: Optional[float] = None) -> torch.Tensor:
+    """Causal attention of a prompt over itself: ``q [B, S, Hq, D]``, ``k`` / ``v [B, S, Hkv, D]`` (bfloat16,
+    D = 64 or 128, last two dimensions contiguous, any token stride) -> ``[B, S, Hq, D]``."""
+    _need_gpu(q, k, v)
+    if q.dtype != torch.bfloat16 or k.dtype != torch.bfloat16 or v.dtype != torch.bfloat16:
+        raise ValueError("prefill_attn_causal takes bfloat16 tensors")
+    if q.dim() != 4 or k.dim() != 4 or k.shape != v.shape or q.shape[:2] != k.shape[:2] or q.shape[3] != k.shape[3]:
+        raise ValueError("q must be [B, S, Hq, D] and k, v [B, S, Hkv, D]")
+    B, S, Hq, D = q.shape
+    Hkv = k.shape[2]
+
+    def tokens(t, heads):
+        # rows of heads*D contiguous elements, batch stride = S * token stride: otherwise copy
+        if t.stride(3) == 1 and t.stride(2) == D and t.stride(0) == S * t.stride(1) and t.stride(1) % 8 == 0 \
+                and t.data_ptr() % 16 == 0:
+            return t, t.stride(1)
+        return t.contiguous(), heads * D
+    q, qs = tokens(q, Hq)
+    k, ks = tokens(k, Hkv)
+    v, vs = tokens(v, Hkv)
+    out = torch.empty((B, S, Hq, D), dtype=torch.bfloat16, device=q.device)
+    if B and S:
+        with torch.cuda.device(q.device):
+            rc = _abi.load().aq_prefill_attn_causal(q.data_ptr(), qs, k.data_ptr(), ks, v.data_ptr(), vs, out.data_ptr(),
+                                                    float(scale if scale is not None else D ** -0.5), B, S, Hq, Hkv, D,
+                                                    _stream(q))
+        _abi.check(rc, "aq_prefill_attn_causal")
+    return out
+
+
 def paged_attn_workspace_bytes(B: int, n_heads: int, n_kv_heads: int, total_len: int) -> int:
     """Bytes of device workspace ``paged_attn_decode`` needs for this shape (0: none)."""
     return int(_abi.load().aq_paged_attn_decode_workspace_bytes(B, n_heads, n_kv_heads, int(total_len)))

@@ -56,6 +56,11 @@
  *                         (attention.py:15-23,93-103) for one new token per sequence;
  *                         pinned against torch (complex multiply, index writes,
  *                         scaled_dot_product_attention in fp32) within rounding.
+ *   oq_prefill_attn_causal the same attention for a whole prompt (is_causal=True);
+ *                         pinned against torch's scaled_dot_product_attention in fp32
+ *                         (enable_gqa and explicit repeats) within rounding, and on
+ *                         closed forms (first position = its own value row; equal keys
+ *                         = running mean of the values).
  *
  * Build: gcc -O3 -march=native -fopenmp -ffp-contract=off -fno-fast-math
  *        -shared -fPIC (oracle/build_oracle.py).  OpenMP only parallelises over
@@ -393,6 +398,42 @@ void oq_paged_attn_decode(const uint16_t *q, const uint16_t *kc, const uint16_t 
       free(s);
       free(acc);
     }
+}
+
+/* Causal self-attention over a prompt: out[b, s, h, :] = softmax_{t <= s}(scale * q[b,s,h] . k[b,t,h/G])
+ * v[b,t,h/G] -- repeat_kv + scaled_dot_product_attention(is_causal=True) of attention.py:15-23,93-100 when
+ * query and key positions coincide.  q: [B, S, Hq, D], k, v: [B, S, Hkv, D] bf16 bit patterns; fp32, t and d
+ * ascending, libm expf. */
+void oq_prefill_attn_causal(const uint16_t *q, const uint16_t *k, const uint16_t *v, float scale, uint16_t *out,
+                            int64_t B, int64_t S, int64_t Hq, int64_t Hkv, int64_t D) {
+  const int64_t G = Hq / Hkv;
+#pragma omp parallel for schedule(dynamic) collapse(3)
+  for (int64_t b = 0; b < B; ++b)
+    for (int64_t h = 0; h < Hq; ++h)
+      for (int64_t s = 0; s < S; ++s) {
+        const int64_t kvh = h / G;
+        const uint16_t *qr = q + ((b * S + s) * Hq + h) * D;
+        float *sc = (float *)malloc((size_t)(s + 1) * sizeof(float));
+        float *acc = (float *)calloc((size_t)D, sizeof(float));
+        float m = -INFINITY;
+        for (int64_t t = 0; t <= s; ++t) {
+          const uint16_t *kr = k + ((b * S + t) * Hkv + kvh) * D;
+          float d = 0.0f;
+          for (int64_t i = 0; i < D; ++i) d += oq_bf16_to_f32(qr[i]) * oq_bf16_to_f32(kr[i]);
+          sc[t] = d * scale;
+          if (sc[t] > m) m = sc[t];
+        }
+        float l = 0.0f;
+        for (int64_t t = 0; t <= s; ++t) {
+          const float pt = expf(sc[t] - m);
+          l += pt;
+          const uint16_t *vr = v + ((b * S + t) * Hkv + kvh) * D;
+          for (int64_t i = 0; i < D; ++i) acc[i] += pt * oq_bf16_to_f32(vr[i]);
+        }
+        for (int64_t i = 0; i < D; ++i) out[((b * S + s) * Hq + h) * D + i] = oq_f32_to_bf16(acc[i] / l);
+        free(sc);
+        free(acc);
+      }
 }
 
 /* ------------------------------------------------------------- int8 GEMM */

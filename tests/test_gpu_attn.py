@@ -168,6 +168,25 @@ def test_rope_paged_attn_decode_equals_the_two_launches(B, Hq, Hkv, page, T, D):
         assert torch.equal(k1, k2) and torch.equal(v1, v2)
 
 
+@pytest.mark.parametrize("B,S,Hq,Hkv,D", [(1, 1, 1, 1, 64), (2, 37, 6, 2, 64), (1, 129, 4, 4, 128), (2, 300, 8, 2, 128),
+                                          (4, 512, 24, 4, 64), (1, 640, 4, 1, 128), (3, 64, 3, 1, 64)])
+def test_prefill_attn_causal_within_bf16_rounding(oracle, B, S, Hq, Hkv, D):
+    _say("prefill_attn_causal", B, S, Hq, Hkv, D)
+    g = torch.Generator().manual_seed(S + D)
+    q = (torch.randn(B, S, Hq, D, generator=g) * 1.5).to(torch.bfloat16)
+    # k contiguous, v a strided view into a wider tensor (as in the fused q/k/v projection's output)
+    k = torch.randn(B, S, Hkv, D, generator=g).to(torch.bfloat16)
+    wide = torch.randn(B, S, (Hq + 2 * Hkv) * D, generator=g).to(torch.bfloat16)
+    v = wide[..., (Hq + Hkv) * D:].view(B, S, Hkv, D)
+    want = torch.from_numpy(oracle.c_prefill_attn_causal(_bits(q), _bits(k), _bits(v.contiguous()), D ** -0.5)
+                            .view(np.int16)).view(torch.bfloat16).float()
+    wd = wide.to(DEV)
+    out = ops.prefill_attn_causal(q.to(DEV), k.to(DEV), wd[..., (Hq + Hkv) * D:].view(B, S, Hkv, D)).cpu().float()
+    # stated tolerance: 1e-2 for bf16 outputs (probabilities rounded to bf16, exp2, block-wise summation)
+    assert torch.allclose(out, want, rtol=1e-2, atol=1e-2)
+    assert ((out - want).norm() / want.norm()).item() < 5e-3
+
+
 def test_attn_argument_checks():
     q = torch.zeros(2, 4, 32, dtype=torch.bfloat16, device=DEV)
     kc = torch.zeros(4, 8, 2, 32, dtype=torch.bfloat16, device=DEV)

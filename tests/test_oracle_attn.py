@@ -61,3 +61,34 @@ def test_paged_attention_matches_torch_sdpa(oracle):
     ref = F.scaled_dot_product_attention(q.float().unsqueeze(2), k.transpose(1, 2), v.transpose(1, 2))[:, :, 0]
     assert torch.allclose(out, ref, rtol=1e-2, atol=1e-2)
     assert (out - ref).norm() / ref.norm() < 3e-3
+
+
+def test_prefill_attention_matches_torch_sdpa_and_closed_forms(oracle):
+    """Causal attention over a prompt: against torch's scaled_dot_product_attention in fp32, with
+    enable_gqa and with explicitly repeated KV heads (the reference's repeat_kv), and on inputs
+    whose answer is known in closed form."""
+    for (B, S, Hq, Hkv, D) in [(2, 37, 6, 2, 64), (1, 70, 4, 4, 128), (2, 5, 3, 1, 64)]:
+        g = torch.Generator().manual_seed(S)
+        q = torch.randn(B, S, Hq, D, generator=g).to(torch.bfloat16)
+        k = torch.randn(B, S, Hkv, D, generator=g).to(torch.bfloat16)
+        v = torch.randn(B, S, Hkv, D, generator=g).to(torch.bfloat16)
+        out = _bf16(oracle.c_prefill_attn_causal(_bits(q), _bits(k), _bits(v), D ** -0.5)).float()
+        qt, kt, vt = (t.float().transpose(1, 2) for t in (q, k, v))
+        rep = Hq // Hkv
+        want = F.scaled_dot_product_attention(qt, kt.repeat_interleave(rep, dim=1), vt.repeat_interleave(rep, dim=1),
+                                              is_causal=True).transpose(1, 2)
+        assert torch.allclose(out, want, rtol=1e-2, atol=1e-2)
+        assert ((out - want).norm() / want.norm()).item() < 4e-3
+        want2 = F.scaled_dot_product_attention(qt, kt, vt, is_causal=True, enable_gqa=True).transpose(1, 2)
+        assert torch.allclose(want, want2, rtol=1e-5, atol=1e-5)
+        # the first position attends to itself only: its output is its own value row, bit for bit
+        assert torch.equal(_bf16(oracle.c_prefill_attn_causal(_bits(q), _bits(k), _bits(v), D ** -0.5))[:, 0],
+                           v[:, 0].repeat_interleave(rep, dim=1))
+    # equal keys: uniform weights, so position s returns the mean of the first s + 1 value rows
+    B, S, Hq, Hkv, D = 1, 9, 2, 1, 64
+    q = torch.randn(B, S, Hq, D).to(torch.bfloat16)
+    k = torch.ones(B, S, Hkv, D).to(torch.bfloat16)
+    v = torch.randn(B, S, Hkv, D).to(torch.bfloat16)
+    out = _bf16(oracle.c_prefill_attn_causal(_bits(q), _bits(k), _bits(v), 0.125)).float()
+    mean = v.float().cumsum(1) / torch.arange(1, S + 1).view(1, S, 1, 1)
+    assert torch.allclose(out, mean.expand(B, S, Hq, D), rtol=1e-2, atol=1e-2)

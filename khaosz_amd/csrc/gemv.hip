@@ -114,7 +114,12 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_w8a8_kernel(GemvArgs p) {
   // wavefront-uniform first row, kept scalar so the buffer descriptor lives in SGPRs
   constexpr int WAVES = GV_WAVES;
   const int nwaves = FUSED ? WAVES : (int)(blockDim.x >> 6);
-  const int n0 = __builtin_amdgcn_readfirstlane((blockIdx.x * nwaves + wave) * GV_ROWS);
+  // K parts: ksplit wavefronts share a group of GV_ROWS rows, wavefront kpart taking chunks kpart,
+  // kpart + ksplit, ...; their sums meet in LDS (exact int32).  For short N and long K, where whole rows per
+  // wavefront would leave most of the device without loads in flight.
+  const int ksplit = FUSED ? 1 : p.ksplit;
+  const int kpart = wave % ksplit;
+  const int n0 = __builtin_amdgcn_readfirstlane((blockIdx.x * (nwaves / ksplit) + wave / ksplit) * GV_ROWS);
 
   // 0. After the reduction lane l owns output (row n0 + idx / MT, token idx % MT)
   // with idx = l >> (6 - log2(rows * MT)).  Its scales and bias are requested
@@ -164,12 +169,13 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_w8a8_kernel(GemvArgs p) {
   // 2. the first GV_DEPTH weight chunks of this wavefront's rows.  The
   // descriptor spans these rows only; rows past N and bytes past K fall
   // outside it and read as zero.
-  const int nchunk = (K + GV_CHUNK - 1) / GV_CHUNK;
+  const int nchunk_all = (K + GV_CHUNK - 1) / GV_CHUNK;
+  const int nchunk = (nchunk_all - kpart + ksplit - 1) / ksplit;  // this wavefront's chunks (0 is possible)
   const int rows = n0 < N ? ((N - n0) < GV_ROWS ? (N - n0) : GV_ROWS) : 0;
   const __amdgpu_buffer_rsrc_t Wr =
       make_rsrc(p.wq + (int64_t)(n0 < N ? n0 : 0) * K, (uint32_t)rows * (uint32_t)K);
   auto wload = [&](int c, uint4 (&dst)[GV_ROWS]) {
-    const int kb = c * GV_CHUNK + lane * 16;
+    const int kb = (kpart + c * ksplit) * GV_CHUNK + lane * 16;
     const bool ok = kb < K;  // past K the offset would alias the next row
 #pragma unroll
     for (int r = 0; r < GV_ROWS; ++r)
@@ -201,7 +207,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_w8a8_kernel(GemvArgs p) {
   for (int i = 0; i < GV_ROWS * MT; ++i) acc[i] = 0;
 
   auto consume = [&](int c, const uint4 (&wc)[GV_ROWS]) {
-    const int kb = c * GV_CHUNK + lane * 16;
+    const int kb = (kpart + c * ksplit) * GV_CHUNK + lane * 16;
     const int kx = kb < K ? kb : 0;  // lanes past the end multiply zeros; keep the LDS read in range
     // activation rows in blocks of 4: four LDS reads in flight cover the 64 dot
     // products of the previous block without holding all MT rows in registers
@@ -243,6 +249,13 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_w8a8_kernel(GemvArgs p) {
   }
 
   Butterfly<V, 32>::run(acc, lane);
+  if (ksplit > 1) {  // uniform over the workgroup
+    int* part = reinterpret_cast<int*>(sx_lds + MT);  // [wavefront][lane]
+    if (kpart != 0) part[wave * 64 + lane] = acc[0];
+    __syncthreads();
+    if (kpart != 0) return;
+    for (int k = 1; k < ksplit; ++k) acc[0] += part[(wave + k) * 64 + lane];
+  }
   if (!out_lane) return;
   float y = __fmul_rn(__fmul_rn((float)acc[0], sxv), swv);
   if (p.bias) y = __fadd_rn(y, bv);
@@ -254,25 +267,38 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_w8a8_kernel(GemvArgs p) {
     reinterpret_cast<float*>(p.y)[o] = y;
 }
 
-// Wavefronts per workgroup for N weight rows: 8, halved (down to 2) while the launch would have
-// fewer workgroups than the device has compute units.
-static int gemv_waves(int N) {
-  int waves = GV_WAVES;
-  while (waves > 2 && (N + GV_ROWS * waves - 1) / (GV_ROWS * waves) < 256) waves >>= 1;
-  return waves;
+// Shape of a launch for N weight rows of K bytes.  Whole rows per wavefront, 8 wavefronts per workgroup,
+// halved (down to 2) while the launch would have fewer workgroups than the device has compute units.  Rows
+// of four or more chunks on a launch that still has fewer than 1024 wavefronts are cut into 2 or 4 K parts
+// (more loads in flight; a wavefront keeps at least one chunk).
+struct GemvShape {
+  int waves, ksplit;
+};
+static GemvShape gemv_shape(int N, int K, bool fused) {
+  GemvShape sh{GV_WAVES, 1};
+  if (fused) return sh;
+  const int groups = (N + GV_ROWS - 1) / GV_ROWS, nchunk = (K + GV_CHUNK - 1) / GV_CHUNK;
+  while (nchunk >= 4 && sh.ksplit < 4 && groups * sh.ksplit < 1024 && nchunk >= 2 * sh.ksplit) sh.ksplit *= 2;
+  int per_wg = GV_WAVES / sh.ksplit;  // row groups per workgroup
+  while (per_wg > 1 && (groups + per_wg - 1) / per_wg < 256) per_wg >>= 1;
+  if (sh.ksplit == 1 && per_wg < 2) per_wg = 2;
+  sh.waves = per_wg * sh.ksplit;
+  return sh;
 }
 
 template <int MT, bool FUSED, int VPL, bool NORM = false>
-static int launch_gemv(const GemvArgs& a, hipStream_t st) {
-  const int waves = FUSED ? GV_WAVES : gemv_waves(a.N);
-  const unsigned grid = (unsigned)((a.N + GV_ROWS * waves - 1) / (GV_ROWS * waves));
-  const size_t lds = (size_t)MT * a.K + MT * sizeof(float);
+static int launch_gemv(GemvArgs a, hipStream_t st) {
+  const GemvShape sh = gemv_shape(a.N, a.K, FUSED);
+  a.ksplit = sh.ksplit;
+  const int rows_per_wg = GV_ROWS * (sh.waves / sh.ksplit);
+  const unsigned grid = (unsigned)((a.N + rows_per_wg - 1) / rows_per_wg);
+  const size_t lds = (size_t)MT * a.K + MT * sizeof(float) + (sh.ksplit > 1 ? (size_t)sh.waves * 64 * sizeof(int) : 0);
   if (lds > 64 * 1024) {  // beyond the default dynamic-LDS limit: opt this kernel in (idempotent)
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_w8a8_kernel<MT, FUSED, VPL, NORM>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return (int)e;
   }
-  hipLaunchKernelGGL((gemv_w8a8_kernel<MT, FUSED, VPL, NORM>), dim3(grid), dim3(waves * 64), lds, st, a);
+  hipLaunchKernelGGL((gemv_w8a8_kernel<MT, FUSED, VPL, NORM>), dim3(grid), dim3(sh.waves * 64), lds, st, a);
   return (int)hipGetLastError();
 }
 
@@ -515,7 +541,7 @@ static int gemv_check(const int8_t* wq, const float* sw, const void* bias, int b
   if (aq::check_ptr16(wq)) return AQ_E_ALIGN;
   if (N > (1 << 30)) return AQ_E_RANGE;
   const int mt = M <= 1 ? 1 : M <= 2 ? 2 : M <= 4 ? 4 : M <= 8 ? 8 : 16;
-  if ((int64_t)mt * K + 64 > aq::GV_MAX_LDS) return AQ_E_RANGE;
+  if ((int64_t)mt * K + 64 + 2048 > aq::GV_MAX_LDS) return AQ_E_RANGE;  // codes, scales, K-part sums
   *mt_out = mt;
   return AQ_OK;
 }

@@ -39,6 +39,21 @@ __device__ __forceinline__ uint4 rope8(uint4 x, const float* cs /* 4 (cos, sin) 
   return make_uint4(o[0], o[1], o[2], o[3]);
 }
 
+// the same on table values already in registers
+__device__ __forceinline__ uint4 rope8(uint4 x, float4 a, float4 b) {
+  const float c[4] = {a.x, a.z, b.x, b.z}, sn[4] = {a.y, a.w, b.y, b.w};
+  const uint32_t in[4] = {x.x, x.y, x.z, x.w};
+  uint32_t o[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float x0 = __uint_as_float(in[i] << 16), x1 = __uint_as_float(in[i] & 0xffff0000u);
+    const float r0 = __fsub_rn(__fmul_rn(x0, c[i]), __fmul_rn(x1, sn[i]));
+    const float r1 = __fadd_rn(__fmul_rn(x0, sn[i]), __fmul_rn(x1, c[i]));
+    o[i] = pack_bf16x2(r0, r1);
+  }
+  return make_uint4(o[0], o[1], o[2], o[3]);
+}
+
 struct RopeArgs {
   const uint16_t* qkv;   // [B, S, (Hq + 2 Hkv) * D]
   const float* freqs;    // [S, D/2, 2] (cos, sin) per sequence; sequences freqs_stride floats apart (0: shared)
@@ -176,6 +191,25 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void paged_attn_decode_kernel(AttnA
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc[g][e] = 0.0f;
   }
+  // The queries (and their rotary table values) do not depend on the page table: requested first, used after
+  // the K and V loads have been issued, so that the wavefront waits for one memory round trip less.
+  uint4 qraw[KS];
+  float4 fa[KS], fb[KS];
+  if (t0 < T) {
+    const int hq = col < G ? col : 0;  // heads past G: zero rows of the operand (their loads read head 0)
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int d0 = ks * 32 + kq * 8;
+      if constexpr (ROPE) {
+        qraw[ks] = *reinterpret_cast<const uint4*>(p.qkv + ((int64_t)b * (p.Hq + 2 * p.Hkv) + kvh * G + hq) * D + d0);
+        const float* cs = p.freqs + (int64_t)b * p.freqs_stride + d0;
+        fa[ks] = *reinterpret_cast<const float4*>(cs);
+        fb[ks] = *reinterpret_cast<const float4*>(cs + 4);
+      } else {
+        qraw[ks] = *reinterpret_cast<const uint4*>(p.q + ((int64_t)b * p.Hq + kvh * G + hq) * D + d0);
+      }
+    }
+  }
   if (t0 < T) {  // wavefront-uniform
     // lane L looks up the row of position t0 + L (element offset, -1: unmapped or past T)
     int64_t row = -1;
@@ -192,24 +226,7 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void paged_attn_decode_kernel(AttnA
       return ((int64_t)hi << 32) | (uint32_t)lo;
     };
     const bool has_new = ROPE && T - 1 >= t0 && T - 1 < t0 + KPW;  // wavefront-uniform
-    // ---- operands of the scores.  Queries: lane = (head col, dimensions ks * 32 + kq * 8 .. + 8); heads past G
-    // are zero rows (their loads read head 0).
-    uint4 qa[KS];
-    {
-      const int hq = col < G ? col : 0;
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const int d0 = ks * 32 + kq * 8;
-        if constexpr (ROPE) {
-          const uint16_t* tok = p.qkv + (int64_t)b * (p.Hq + 2 * p.Hkv) * D;
-          qa[ks] = rope8(*reinterpret_cast<const uint4*>(tok + (int64_t)(kvh * G + hq) * D + d0),
-                         p.freqs + (int64_t)b * p.freqs_stride + d0);
-        } else {
-          qa[ks] = *reinterpret_cast<const uint4*>(p.q + ((int64_t)b * p.Hq + kvh * G + hq) * D + d0);
-        }
-        if (col >= G) qa[ks] = make_uint4(0, 0, 0, 0);
-      }
-    }
+    // ---- operands of the scores
     // keys: tile t holds positions t0 + 16 t .. + 16; lane = (key col, the same dimensions).  Rows that are
     // unmapped or past T read row 0 of the cache and are zeroed.
     uint4 kb[4][KS];
@@ -227,7 +244,7 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void paged_attn_decode_kernel(AttnA
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
           const int d0 = ks * 32 + kq * 8;
-          kb[t][ks] = rope8(*reinterpret_cast<const uint4*>(tok + d0), p.freqs + (int64_t)b * p.freqs_stride + d0);
+          kb[t][ks] = rope8(*reinterpret_cast<const uint4*>(tok + d0), fa[ks], fb[ks]);
           *reinterpret_cast<uint4*>(p.kc_w + r + d0) = kb[t][ks];
         }
       }
@@ -243,6 +260,16 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void paged_attn_decode_kernel(AttnA
         vv[i] = *reinterpret_cast<const uint4*>(p.qkv + ((int64_t)b * (p.Hq + 2 * p.Hkv) + p.Hq + p.Hkv + kvh) * D + ch * 8);
         *reinterpret_cast<uint4*>(p.vc_w + r + ch * 8) = vv[i];
       }
+    }
+    // queries: lane = (head col, dimensions ks * 32 + kq * 8 .. + 8)
+    uint4 qa[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      if constexpr (ROPE)
+        qa[ks] = rope8(qraw[ks], fa[ks], fb[ks]);
+      else
+        qa[ks] = qraw[ks];
+      if (col >= G) qa[ks] = make_uint4(0, 0, 0, 0);
     }
     // ---- scores: S[head][key] per tile; this lane gets key col of the tile, heads 4 kq .. + 4
     attn_f32x4 sc[4];
@@ -269,7 +296,7 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void paged_attn_decode_kernel(AttnA
       float sum = 0.0f;
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
-        const float pv = exp2f(sv[t] - mx);  // 0 for positions past T
+        const float pv = __builtin_amdgcn_exp2f(sv[t] - mx);  // 0 for positions past T
         sum += pv;
         if (head < G) p_s[wave][t * 16 + col][head] = pv;
       }
@@ -300,25 +327,53 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void paged_attn_decode_kernel(AttnA
         for (int e = 0; e < 8; ++e) acc[g][e] = __builtin_fmaf(pj, v8[e], acc[g][e]);
       }
     }
+    // Sum over the RPL key groups (lanes CPR apart) with a transposed butterfly: at each stage a lane keeps
+    // one half of its values and trades the other half with its partner, so the 8 G values per lane cost
+    // 8 G (1 - 1 / RPL) exchanges instead of 8 G log2(RPL), and a lane ends up with 8 G / RPL finished sums.
+    {
+      constexpr int NV = 8 * G;
+      float a[NV];
 #pragma unroll
-    for (int g = 0; g < G; ++g)
+      for (int j = 0; j < NV; ++j) a[j] = acc[j / 8][j % 8];
+      int base = 0;  // first original index of the values this lane still holds
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
+      for (int st = 0; (CPR << st) < 64; ++st) {
+        const int off = CPR << st, h = NV >> (st + 1);
+        const bool up = (lane & off) != 0;
 #pragma unroll
-        for (int off = CPR; off < 64; off <<= 1) acc[g][e] += __shfl_xor(acc[g][e], off, 64);
+        for (int i = 0; i < h; ++i) {
+          if (off == 32 || off == 16) {
+            // half / row swaps: lanes without the bit receive the partner's a[i], lanes with it the partner's
+            // a[i + h], next to their own; one add finishes the exchange
+            typedef unsigned att_u2 __attribute__((ext_vector_type(2)));
+            const att_u2 r = off == 32 ? __builtin_amdgcn_permlane32_swap(__float_as_uint(a[i]), __float_as_uint(a[i + h]), false, false)
+                                       : __builtin_amdgcn_permlane16_swap(__float_as_uint(a[i]), __float_as_uint(a[i + h]), false, false);
+            a[i] = __uint_as_float(r.x) + __uint_as_float(r.y);
+          } else {
+            // select by mask rather than by ?: -- the compiler turned the latter into per-exchange branches
+            const uint32_t lo = __float_as_uint(a[i]), hi = __float_as_uint(a[i + h]);
+            const uint32_t t = (lo ^ hi) & (up ? 0xffffffffu : 0u);
+            a[i] = __uint_as_float(t ^ lo) + __shfl_xor(__uint_as_float(t ^ hi), off, 64);  // keep + partner's send
+          }
+        }
+        base += up ? h : 0;
       }
-  } else if (lane < G) {  // a wavefront past T: nothing to add
-    m_s[wave][lane] = -INFINITY;
-    l_s[wave][lane] = 0.0f;
+      asm volatile("" : "+v"(base));  // one address computation below, not a code path per value of base
+      float* dst = &acc_s[wave][0][ch * 8];
+#pragma unroll
+      for (int i = 0; i < NV / RPL; ++i) {
+        const int j = base + i;
+        dst[(j >> 3) * D + (j & 7)] = a[i];
+      }
+    }
+  } else {  // a wavefront past T: nothing to add
+    if (lane < G) {
+      m_s[wave][lane] = -INFINITY;
+      l_s[wave][lane] = 0.0f;
+    }
+    for (int i = lane; i < G * D; i += 64) acc_s[wave][i / D][i % D] = 0.0f;
   }
   // ---- merge the wavefronts' partial results
-#pragma unroll
-  for (int g = 0; g < G; ++g) {
-    if (sub == 0) {
-      *reinterpret_cast<float4*>(&acc_s[wave][g][ch * 8]) = make_float4(acc[g][0], acc[g][1], acc[g][2], acc[g][3]);
-      *reinterpret_cast<float4*>(&acc_s[wave][g][ch * 8 + 4]) = make_float4(acc[g][4], acc[g][5], acc[g][6], acc[g][7]);
-    }
-  }
   __syncthreads();
   for (int i = tid; i < G * D / 2; i += ATT_THREADS) {
     const int g = i / (D / 2), d = (i % (D / 2)) * 2;  // dimensions d, d + 1

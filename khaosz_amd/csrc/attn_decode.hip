@@ -227,38 +227,60 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void paged_attn_decode_kernel(AttnA
     };
     const bool has_new = ROPE && T - 1 >= t0 && T - 1 < t0 + KPW;  // wavefront-uniform
     // ---- operands of the scores
-    // keys: tile t holds positions t0 + 16 t .. + 16; lane = (key col, the same dimensions).  Rows that are
-    // unmapped or past T read row 0 of the cache and are zeroed.
-    uint4 kb[4][KS];
+    // keys: tile t holds positions t0 + 16 t .. + 16; lane = (key col, dimensions ks * 32 + kq * 8 .. + 8).
+    // values: lane = (key sub of a load, 16-byte chunk ch of the row).  Rows that are unmapped or past T read
+    // row 0 of the cache and are zeroed afterwards.  Every load is issued before any loaded value is touched
+    // (the fix-ups below are selects on data, kept out of the issue loops: with them inside, the compiler
+    // waited for each load before issuing the next).
+    uint4 kb[4][KS], vv[NL];
+    uint32_t kneg = 0, vneg = 0;  // bit t / i: that row is not there
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
       const int64_t r = row_of(t * 16 + col);
-      const uint16_t* src = p.kc + (r >= 0 ? r : 0);
+      kneg |= (r < 0 ? 1u : 0u) << t;
+      const uint16_t* src = p.kc + (r >= 0 ? r : 0) + kq * 8;
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        kb[t][ks] = *reinterpret_cast<const uint4*>(src + ks * 32 + kq * 8);
-        if (r < 0) kb[t][ks] = make_uint4(0, 0, 0, 0);
-      }
-      if (ROPE && has_new && r >= 0 && t0 + t * 16 + col == T - 1) {  // the new key: rotated here, used and stored
-        const uint16_t* tok = p.qkv + ((int64_t)b * (p.Hq + 2 * p.Hkv) + p.Hq + kvh) * D;
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          const int d0 = ks * 32 + kq * 8;
-          kb[t][ks] = rope8(*reinterpret_cast<const uint4*>(tok + d0), fa[ks], fb[ks]);
-          *reinterpret_cast<uint4*>(p.kc_w + r + d0) = kb[t][ks];
-        }
-      }
+      for (int ks = 0; ks < KS; ++ks) kb[t][ks] = *reinterpret_cast<const uint4*>(src + ks * 32);
     }
-    // values: lane = (key sub of a load, 16-byte chunk ch of the row)
-    uint4 vv[NL];
 #pragma unroll
     for (int i = 0; i < NL; ++i) {
       const int64_t r = row_of(i * RPL + sub);
+      vneg |= (r < 0 ? 1u : 0u) << i;
       vv[i] = *reinterpret_cast<const uint4*>(p.vc + (r >= 0 ? r : 0) + ch * 8);
-      if (r < 0) vv[i] = make_uint4(0, 0, 0, 0);
-      if (ROPE && has_new && r >= 0 && t0 + i * RPL + sub == T - 1) {  // the new value
-        vv[i] = *reinterpret_cast<const uint4*>(p.qkv + ((int64_t)b * (p.Hq + 2 * p.Hkv) + p.Hq + p.Hkv + kvh) * D + ch * 8);
-        *reinterpret_cast<uint4*>(p.vc_w + r + ch * 8) = vv[i];
+    }
+    __builtin_amdgcn_sched_barrier(0);  // nothing that waits for a load may move above the last load's issue
+    if (__builtin_amdgcn_ballot_w64(row < 0) != 0) {  // wavefront-uniform; rare: a hole, or the wavefront that holds T - 1
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+          if (kneg & (1u << t)) kb[t][ks] = make_uint4(0, 0, 0, 0);
+#pragma unroll
+      for (int i = 0; i < NL; ++i)
+        if (vneg & (1u << i)) vv[i] = make_uint4(0, 0, 0, 0);
+    }
+    if (ROPE && has_new) {  // wavefront-uniform: this wavefront owns position T - 1
+      // the new key and value: rotated here, stored into their page slot, and used from registers in place
+      // of what was just read from that slot
+      const uint16_t* tok = p.qkv + (int64_t)b * (p.Hq + 2 * p.Hkv) * D;
+      const int64_t rn = row_of((int)(T - 1 - t0));  // the same in every lane; -1: its page is unmapped
+      if (rn >= 0) {
+        const int tn = (int)(T - 1 - t0) >> 4, cn = (int)(T - 1 - t0) & 15;  // tile and column of the new key
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          const int d0 = ks * 32 + kq * 8;
+          const uint4 kn = rope8(*reinterpret_cast<const uint4*>(tok + (int64_t)(p.Hq + kvh) * D + d0), fa[ks], fb[ks]);
+          if (col == cn) *reinterpret_cast<uint4*>(p.kc_w + rn + d0) = kn;
+#pragma unroll
+          for (int t = 0; t < 4; ++t)
+            if (t == tn && col == cn) kb[t][ks] = kn;
+        }
+        const uint4 vn = *reinterpret_cast<const uint4*>(tok + (int64_t)(p.Hq + p.Hkv + kvh) * D + ch * 8);
+        const int in = (int)(T - 1 - t0) / RPL, sn = (int)(T - 1 - t0) % RPL;  // load and key group of the new value
+        if (sub == sn) *reinterpret_cast<uint4*>(p.vc_w + rn + ch * 8) = vn;
+#pragma unroll
+        for (int i = 0; i < NL; ++i)
+          if (i == in && sub == sn) vv[i] = vn;
       }
     }
     // queries: lane = (head col, dimensions ks * 32 + kq * 8 .. + 8)

@@ -221,6 +221,42 @@ int aq_rope_paged_attn_decode(const void *qkv, const float *freqs, int64_t freqs
                               float scale, void *out, int64_t B, int64_t Hq, int64_t Hkv, int64_t D,
                               void *workspace, int64_t workspace_bytes, void *stream);
 
+/* The decode step's attention and output projection without the merge launch
+ * in between.  aq_paged_attn_decode_partials / aq_rope_paged_attn_decode_partials
+ * are the two calls above stopped before their slices are combined: `partials`
+ * (16-byte aligned, at least aq_paged_attn_decode_partials_bytes(B, Hq,
+ * total_len) bytes; needed for one slice too) receives, for every (sequence,
+ * query head, slice), D numerators, the slice's maximum (log2 domain), its
+ * denominator and 2 floats of padding: [B, Hq, n_slices, D + 4] fp32 with
+ * n_slices = aq_paged_attn_decode_slices(total_len).
+ * aq_gemv_w8a8_decode_attn is aq_gemv_w8a8_decode_residual (attention.py:108,
+ * o_proj, plus decoder_block.py:53's add when residual is given) with the rows
+ * [M = B, K = Hq * D] combined from those partial results inside the kernel, by
+ * the arithmetic of the merge kernel the other path launches: outputs are the
+ * bits of aq_(rope_)paged_attn_decode followed by aq_gemv_w8a8_decode_residual.
+ * Limits (the kernel holds every slice of a row in registers): M <= 8, K <=
+ * AQ_GEMV_ATTN_MAX_K, n_slices <= AQ_GEMV_ATTN_MAX_SLICES (1024 positions);
+ * beyond them AQ_E_RANGE, and the caller takes the three-launch path. */
+#define AQ_GEMV_ATTN_MAX_K 2048
+#define AQ_GEMV_ATTN_MAX_SLICES 4
+int64_t aq_paged_attn_decode_slices(int64_t total_len);
+int64_t aq_paged_attn_decode_partials_bytes(int64_t B, int64_t Hq, int64_t total_len);
+int aq_paged_attn_decode_partials(const void *q, const void *k_cache, const void *v_cache,
+                                  const int64_t *page_table, int64_t P, int64_t total_len,
+                                  int64_t page_size, int64_t n_pages, float scale, int64_t B,
+                                  int64_t Hq, int64_t Hkv, int64_t D, void *partials,
+                                  int64_t partials_bytes, void *stream);
+int aq_rope_paged_attn_decode_partials(const void *qkv, const float *freqs, int64_t freqs_stride,
+                                       const int64_t *page_table, int64_t P, int64_t total_len,
+                                       int64_t page_size, void *k_cache, void *v_cache,
+                                       int64_t n_pages, float scale, int64_t B, int64_t Hq,
+                                       int64_t Hkv, int64_t D, void *partials,
+                                       int64_t partials_bytes, void *stream);
+int aq_gemv_w8a8_decode_attn(const float *partials, int64_t n_slices, int64_t head_dim,
+                             const int8_t *wq, const float *sw, const void *bias, int bias_dtype,
+                             const void *residual, void *y, int y_dtype, int64_t M, int64_t N,
+                             int64_t K, void *stream);
+
 /* Causal self-attention over a prompt, for a prefill that starts from an empty
  * cache (query and key positions coincide): out[b, s, h, :] =
  * softmax_{t <= s}(scale * q[b,s,h] . k[b,t,h/G]) v[b,t,h/G], G = Hq / Hkv.

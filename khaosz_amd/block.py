@@ -116,9 +116,7 @@ class PagedKV:
         """Scratch for the decode attention kernel's partial results, sized once for the longest
         sequence the bound page table can hold and shared by all layers (they run one after the other)."""
         B, P = self.page_table.shape
-        need = ops.paged_attn_workspace_bytes(B, n_heads, self.k_layers.shape[3], P * self.page_size)
-        if need == 0:
-            return None
+        need = ops.paged_attn_partials_bytes(B, n_heads, P * self.page_size)
         if self._attn_ws is None or self._attn_ws.numel() * 4 < need:
             self._attn_ws = torch.empty(need // 4, dtype=torch.float32, device=self.k_layers.device)
         return self._attn_ws
@@ -238,10 +236,16 @@ class GQA(nn.Module):
         if (self._decode_attention and S == 1 and isinstance(cache, PagedKV) and x.is_cuda
                 and x.dtype == torch.bfloat16):
             qkv = self._project_qkv(x, codes, norm)
+            # the output projection combines the attention's position slices itself when the step is small
+            # enough for its in-kernel quantiser: one launch less
+            split = (isinstance(self.o_proj, QuantLinear)
+                     and ops.attn_gemv_fusable(B, self.n_heads, self.head_dim, cache.total_len))
             out = ops.rope_paged_attn_decode(qkv.view(B, -1), rotary_emb.reshape(B, -1), cache.page_table,
                                              cache.total_len, cache.k_layers[self.layer_id],
                                              cache.v_layers[self.layer_id], self.n_heads, self.n_kv_heads,
-                                             workspace=cache.attn_workspace(self.n_heads))
+                                             workspace=cache.attn_workspace(self.n_heads), partials=split)
+            if split:
+                return self.o_proj.forward_attn(out, x.dtype, residual).view(B, 1, -1)
             return self._out(out.view(B, 1, -1), residual)
         if (self._decode_attention and isinstance(cache, PagedKV) and x.is_cuda and x.dtype == torch.bfloat16
                 and S <= cache.total_len):

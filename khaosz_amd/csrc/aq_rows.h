@@ -184,4 +184,98 @@ struct RowsToLds {
   }
 };
 
+// Rows of a decode step's attention output taken straight from the attention kernel's per-slice partial
+// results instead of from a merged bf16 tensor.  Layout [row][head][slice][D + 4] floats: D numerators,
+// the slice's maximum (log2 domain), its denominator, 2 floats of padding.  Element k of row m belongs to
+// head k / D.  issue() requests, for each of the lane's 16-byte output vectors, the 8 numerators and the
+// (maximum, denominator) pair of every slice; merge() combines them with the arithmetic of the separate
+// merge kernel (weights exp2(maximum - overall maximum), numerators and denominator accumulated by fma in
+// slice order from zero, product with the denominator's reciprocal, rounded to bf16) and leaves the packed bf16 vectors where
+// RowsToLds::issue() would have put the loaded ones, so the quantiser that follows sees the same bits.
+// The two operations every place that combines attention slices shares (the merge kernel, the
+// attention kernel's own single-slice output, AttnRows below), so that they give the same bits:
+// a slice's weight 2^(its maximum - the overall maximum) and the reciprocal of the combined
+// denominator, both the hardware's approximations (1 ulp), outputs = numerator * reciprocal.
+__device__ __forceinline__ float attn_slice_weight(float m, float mm) { return __builtin_amdgcn_exp2f(m - mm); }
+__device__ __forceinline__ float attn_inv_denominator(float den) { return __builtin_amdgcn_rcpf(den); }
+
+template <int RPW, int VPL, int NSMAX>
+struct AttnRows;
+template <int RPW, int VPL>
+struct AttnRows<RPW, VPL, 0> {};  // kernels that do not merge
+template <int RPW, int VPL, int NSMAX>
+struct AttnRows {
+  uint4 num[RPW][VPL][NSMAX][2];
+  float2 md[RPW][VPL][NSMAX];
+
+  __device__ __forceinline__ void issue(const float* parts, int M, int K, int D, int NS, int wave, int nwaves,
+                                        int lane) {
+    const int nvec = K / 8, part = D + 4, dshift = D == 64 ? 6 : 7;
+#pragma unroll
+    for (int j = 0; j < RPW; ++j) {
+      const int m = wave + j * nwaves;
+#pragma unroll
+      for (int i = 0; i < VPL; ++i) {
+        const int v = i * 64 + lane, k = v * 8;
+        const bool ok = m < M && v < nvec;
+        // (row, head) index = (m * K + k) / D; rows and vectors that are not there read element 0
+        const int64_t rh = ok ? ((int64_t)m * K + k) >> dshift : 0;
+        const float* src = parts + rh * NS * part;
+        const int d = ok ? k & (D - 1) : 0;
+#pragma unroll
+        for (int s = 0; s < NSMAX; ++s) {
+          if (s < NS) {  // uniform
+            num[j][i][s][0] = *reinterpret_cast<const uint4*>(src + s * part + d);
+            num[j][i][s][1] = *reinterpret_cast<const uint4*>(src + s * part + d + 4);
+            md[j][i][s] = *reinterpret_cast<const float2*>(src + s * part + D);
+          }
+        }
+      }
+    }
+  }
+
+  __device__ __forceinline__ void merge(uint4 (&c)[RPW][VPL], int M, int K, int NS, int wave, int nwaves,
+                                        int lane) const {
+    const int nvec = K / 8;
+#pragma unroll
+    for (int j = 0; j < RPW; ++j) {
+      const int m = wave + j * nwaves;
+#pragma unroll
+      for (int i = 0; i < VPL; ++i) {
+        const int v = i * 64 + lane;
+        float mm = -INFINITY;
+#pragma unroll
+        for (int s = 0; s < NSMAX; ++s)
+          if (s < NS) mm = fmaxf(mm, md[j][i][s].x);
+        float n[8], den = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) n[e] = 0.0f;
+#pragma unroll
+        for (int s = 0; s < NSMAX; ++s) {
+          if (s < NS) {
+            const float a = attn_slice_weight(md[j][i][s].x, mm);
+            const uint4 lo = num[j][i][s][0], hi = num[j][i][s][1];
+            n[0] = __builtin_fmaf(__uint_as_float(lo.x), a, n[0]);
+            n[1] = __builtin_fmaf(__uint_as_float(lo.y), a, n[1]);
+            n[2] = __builtin_fmaf(__uint_as_float(lo.z), a, n[2]);
+            n[3] = __builtin_fmaf(__uint_as_float(lo.w), a, n[3]);
+            n[4] = __builtin_fmaf(__uint_as_float(hi.x), a, n[4]);
+            n[5] = __builtin_fmaf(__uint_as_float(hi.y), a, n[5]);
+            n[6] = __builtin_fmaf(__uint_as_float(hi.z), a, n[6]);
+            n[7] = __builtin_fmaf(__uint_as_float(hi.w), a, n[7]);
+            den = __builtin_fmaf(md[j][i][s].y, a, den);
+          }
+        }
+        const float r = attn_inv_denominator(den);
+        uint4 o;
+        o.x = pack_bf16x2(__fmul_rn(n[0], r), __fmul_rn(n[1], r));
+        o.y = pack_bf16x2(__fmul_rn(n[2], r), __fmul_rn(n[3], r));
+        o.z = pack_bf16x2(__fmul_rn(n[4], r), __fmul_rn(n[5], r));
+        o.w = pack_bf16x2(__fmul_rn(n[6], r), __fmul_rn(n[7], r));
+        c[j][i] = (m < M && v < nvec) ? o : make_uint4(0, 0, 0, 0);
+      }
+    }
+  }
+};
+
 }  // namespace aq

@@ -19,6 +19,7 @@
 // (table entry < 0 or out of range) are skipped on write and read as zero keys
 // and values, as the reference's gather does.
 #include "aq_common.h"
+#include "aq_rows.h"
 
 namespace aq {
 
@@ -411,8 +412,9 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void paged_attn_decode_kernel(AttnA
       den = __builtin_fmaf(l_s[w][g], a, den);
     }
     const int64_t head = (int64_t)b * p.Hq + kvh * G + g;
-    if (p.NS == 1) {
-      store_wt(reinterpret_cast<uint32_t*>(p.out + head * D + d), pack_bf16x2(n0 / den, n1 / den));
+    if (p.NS == 1 && p.out != nullptr) {  // out == nullptr: the caller wants the partial results whatever NS is
+      const float r = attn_inv_denominator(den);
+      store_wt(reinterpret_cast<uint32_t*>(p.out + head * D + d), pack_bf16x2(__fmul_rn(n0, r), __fmul_rn(n1, r)));
     } else {
       float* part = p.ws + (head * p.NS + split) * PART;
       store_wt(reinterpret_cast<uint2*>(part + d), make_uint2(__float_as_uint(n0), __float_as_uint(n1)));
@@ -429,13 +431,14 @@ __global__ __launch_bounds__(ATT_MAX_D / 2) void attn_merge_kernel(const float* 
   for (int s = 0; s < NS; ++s) mm = fmaxf(mm, part[s * part_sz + D]);  // slice 0 always holds a position
   float n0 = 0.0f, n1 = 0.0f, den = 0.0f;
   for (int s = 0; s < NS; ++s) {
-    const float a = exp2f(part[s * part_sz + D] - mm);
+    const float a = attn_slice_weight(part[s * part_sz + D], mm);
     const float2 v = *reinterpret_cast<const float2*>(part + s * part_sz + d);
     n0 = __builtin_fmaf(v.x, a, n0);
     n1 = __builtin_fmaf(v.y, a, n1);
     den = __builtin_fmaf(part[s * part_sz + D + 1], a, den);
   }
-  store_wt(reinterpret_cast<uint32_t*>(out + (int64_t)blockIdx.x * D + d), pack_bf16x2(n0 / den, n1 / den));
+  const float r = attn_inv_denominator(den);
+  store_wt(reinterpret_cast<uint32_t*>(out + (int64_t)blockIdx.x * D + d), pack_bf16x2(__fmul_rn(n0, r), __fmul_rn(n1, r)));
 }
 
 inline int64_t attn_slices(int64_t T) { return (T + ATT_KPG - 1) / ATT_KPG; }
@@ -498,10 +501,11 @@ static void attn_launch(bool rope, dim3 grid, dim3 block, hipStream_t st, const 
 }
 
 // q == nullptr: the fused form, queries and the new token come from qkv / freqs.
+// partials: stop after the slices' partial results (no merge launch, `out` unused).
 static int attn_decode(const void* q, const void* qkv, const float* freqs, int64_t freqs_stride, void* k_cache,
                        void* v_cache, const int64_t* page_table, int64_t P, int64_t total_len, int64_t page_size,
                        int64_t n_pages, float scale, void* out, int64_t B, int64_t Hq, int64_t Hkv, int64_t D,
-                       void* workspace, int64_t workspace_bytes, void* stream) {
+                       void* workspace, int64_t workspace_bytes, void* stream, bool partials = false) {
   const bool rope = q == nullptr;
   if (D != 64 && D != 128) return AQ_E_SHAPE;
   if (B < 0 || Hq <= 0 || Hkv <= 0 || (Hq % Hkv) != 0 || P <= 0 || total_len <= 0 || page_size <= 0 ||
@@ -511,14 +515,16 @@ static int attn_decode(const void* q, const void* qkv, const float* freqs, int64
   if (G != 1 && G != 2 && G != 3 && G != 4 && G != 6 && G != 8) return AQ_E_SHAPE;  // query heads per KV head
   if (rope && freqs_stride != 0 && freqs_stride < D) return AQ_E_SHAPE;
   if (B == 0) return AQ_OK;
-  if (!(rope ? (qkv != nullptr && freqs != nullptr) : (q != nullptr)) || !k_cache || !v_cache || !page_table || !out)
+  if (!(rope ? (qkv != nullptr && freqs != nullptr) : (q != nullptr)) || !k_cache || !v_cache || !page_table ||
+      (!out && !partials))
     return AQ_E_NULL;
-  if (aq::check_ptr16(rope ? qkv : q) || aq::check_ptr16(k_cache) || aq::check_ptr16(v_cache) || aq::check_ptr16(out))
+  if (aq::check_ptr16(rope ? qkv : q) || aq::check_ptr16(k_cache) || aq::check_ptr16(v_cache) ||
+      (!partials && aq::check_ptr16(out)))
     return AQ_E_ALIGN;
   if (rope && (aq::check_ptr16(freqs) || (freqs_stride & 3))) return AQ_E_ALIGN;
   const int64_t ns = aq::attn_slices(total_len);
   if (B * Hkv * ns > (int64_t)0x7fffffff || B * Hq > (int64_t)0x7fffffff) return AQ_E_RANGE;
-  if (ns > 1) {
+  if (ns > 1 || partials) {
     if (!workspace) return AQ_E_NULL;
     if (aq::check_ptr16(workspace)) return AQ_E_ALIGN;
     if (workspace_bytes < aq::attn_workspace_bytes(B, Hq, ns)) return AQ_E_WORKSPACE;
@@ -533,7 +539,7 @@ static int attn_decode(const void* q, const void* qkv, const float* freqs, int64
   a.kc_w = static_cast<uint16_t*>(k_cache);
   a.vc_w = static_cast<uint16_t*>(v_cache);
   a.table = page_table;
-  a.out = static_cast<uint16_t*>(out);
+  a.out = partials ? nullptr : static_cast<uint16_t*>(out);
   a.ws = static_cast<float*>(workspace);
   a.P = P;
   a.T = total_len;
@@ -561,7 +567,7 @@ static int attn_decode(const void* q, const void* qkv, const float* freqs, int64
   }
 #undef AQ_ATTN_CASE
   int rc = (int)hipGetLastError();
-  if (rc != 0 || ns == 1) return rc;
+  if (rc != 0 || ns == 1 || partials) return rc;
   hipLaunchKernelGGL(aq::attn_merge_kernel, dim3((unsigned)(B * Hq)), dim3((unsigned)(D / 2)), 0, st, a.ws, a.out, a.NS,
                      (int)D);
   return (int)hipGetLastError();
@@ -584,4 +590,32 @@ extern "C" int aq_rope_paged_attn_decode(const void* qkv, const float* freqs, in
   if ((!qkv || !freqs) && B > 0) return AQ_E_NULL;
   return attn_decode(nullptr, qkv, freqs, freqs_stride, k_cache, v_cache, page_table, P, total_len, page_size, n_pages,
                      scale, out, B, Hq, Hkv, D, workspace, workspace_bytes, stream);
+}
+
+extern "C" int64_t aq_paged_attn_decode_slices(int64_t total_len) { return total_len <= 0 ? 0 : aq::attn_slices(total_len); }
+
+extern "C" int64_t aq_paged_attn_decode_partials_bytes(int64_t B, int64_t Hq, int64_t total_len) {
+  if (B <= 0 || Hq <= 0 || total_len <= 0) return 0;
+  return aq::attn_workspace_bytes(B, Hq, aq::attn_slices(total_len));
+}
+
+extern "C" int aq_paged_attn_decode_partials(const void* q, const void* k_cache, const void* v_cache,
+                                             const int64_t* page_table, int64_t P, int64_t total_len,
+                                             int64_t page_size, int64_t n_pages, float scale, int64_t B, int64_t Hq,
+                                             int64_t Hkv, int64_t D, void* partials, int64_t partials_bytes,
+                                             void* stream) {
+  if (!q && B > 0) return AQ_E_NULL;
+  return attn_decode(q, nullptr, nullptr, 0, const_cast<void*>(k_cache), const_cast<void*>(v_cache), page_table, P,
+                     total_len, page_size, n_pages, scale, nullptr, B, Hq, Hkv, D, partials, partials_bytes, stream,
+                     true);
+}
+
+extern "C" int aq_rope_paged_attn_decode_partials(const void* qkv, const float* freqs, int64_t freqs_stride,
+                                                  const int64_t* page_table, int64_t P, int64_t total_len,
+                                                  int64_t page_size, void* k_cache, void* v_cache, int64_t n_pages,
+                                                  float scale, int64_t B, int64_t Hq, int64_t Hkv, int64_t D,
+                                                  void* partials, int64_t partials_bytes, void* stream) {
+  if ((!qkv || !freqs) && B > 0) return AQ_E_NULL;
+  return attn_decode(nullptr, qkv, freqs, freqs_stride, k_cache, v_cache, page_table, P, total_len, page_size, n_pages,
+                     scale, nullptr, B, Hq, Hkv, D, partials, partials_bytes, stream, true);
 }

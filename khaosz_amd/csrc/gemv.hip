@@ -87,6 +87,8 @@ struct GemvArgs {
   int ksplit, groups;  // matrix-core variant: wavefronts sharing a row group, row groups per workgroup
   const void* gamma;   // NORM kernels: RMSNorm gain [K] in x's dtype
   float eps;
+  const float* parts;  // MERGE kernels: attention partial results in place of x
+  int parts_ns, parts_d;
 };
 
 // y (+ residual): the projection is rounded to the output type first and the
@@ -105,7 +107,9 @@ __device__ __forceinline__ float add_residual_bf16(float y, uint32_t res_bits) {
 // workgroup covers GV_ROWS * wavefronts weight rows; the launcher shrinks it
 // when N is too small for 8-wavefront workgroups to reach every compute unit.
 // NORM (with FUSED): the rows are RMS-normalised with the gain p.gamma before they are quantised.
-template <int MT, bool FUSED, int VPL, bool NORM = false>
+// MERGE > 0 (with FUSED): the rows are a decode step's attention output, combined here from the attention
+// kernel's partial results of up to MERGE slices (p.parts) -- the separate merge launch disappears.
+template <int MT, bool FUSED, int VPL, bool NORM = false, int MERGE = 0>
 __global__ __launch_bounds__(GV_THREADS) void gemv_w8a8_kernel(GemvArgs p) {
   extern __shared__ __attribute__((aligned(16))) uint8_t xs[];  // [MT][K] activation codes, then [MT] scales
   const int tid = threadIdx.x, lane = tid & 63;
@@ -150,7 +154,10 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_w8a8_kernel(GemvArgs p) {
   // and quantises them while the weight loads queued behind are in flight.
   constexpr int RPW = FUSED ? (MT + WAVES - 1) / WAVES : 1;
   RowsToLds<true, RPW, VPL> xrows;
-  if constexpr (FUSED) {
+  AttnRows<RPW, VPL, MERGE> arows;
+  if constexpr (MERGE > 0) {
+    arows.issue(p.parts, M, K, p.parts_d, p.parts_ns, wave, WAVES, lane);
+  } else if constexpr (FUSED) {
     xrows.issue(p.x, M, K, K, wave, WAVES, lane);
     if constexpr (NORM) xrows.issue_gamma(p.gamma, K, lane);
   } else {
@@ -190,6 +197,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_w8a8_kernel(GemvArgs p) {
   // compiler place that wait), then make every wavefront's part visible through
   // a barrier that does not drain the weight loads.
   if constexpr (FUSED) {
+    if constexpr (MERGE > 0) arows.merge(xrows.c, M, K, p.parts_ns, wave, WAVES, lane);
     xrows.template finish<NORM>(M, MT, K, xs, K, sx_lds, wave, WAVES, lane, p.eps);
     __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wavefront's LDS writes are done
   } else {
@@ -286,7 +294,7 @@ static GemvShape gemv_shape(int N, int K, bool fused) {
   return sh;
 }
 
-template <int MT, bool FUSED, int VPL, bool NORM = false>
+template <int MT, bool FUSED, int VPL, bool NORM = false, int MERGE = 0>
 static int launch_gemv(GemvArgs a, hipStream_t st) {
   const GemvShape sh = gemv_shape(a.N, a.K, FUSED);
   a.ksplit = sh.ksplit;
@@ -294,11 +302,11 @@ static int launch_gemv(GemvArgs a, hipStream_t st) {
   const unsigned grid = (unsigned)((a.N + rows_per_wg - 1) / rows_per_wg);
   const size_t lds = (size_t)MT * a.K + MT * sizeof(float) + (sh.ksplit > 1 ? (size_t)sh.waves * 64 * sizeof(int) : 0);
   if (lds > 64 * 1024) {  // beyond the default dynamic-LDS limit: opt this kernel in (idempotent)
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_w8a8_kernel<MT, FUSED, VPL, NORM>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_w8a8_kernel<MT, FUSED, VPL, NORM, MERGE>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return (int)e;
   }
-  hipLaunchKernelGGL((gemv_w8a8_kernel<MT, FUSED, VPL, NORM>), dim3(grid), dim3(sh.waves * 64), lds, st, a);
+  hipLaunchKernelGGL((gemv_w8a8_kernel<MT, FUSED, VPL, NORM, MERGE>), dim3(grid), dim3(sh.waves * 64), lds, st, a);
   return (int)hipGetLastError();
 }
 
@@ -646,6 +654,43 @@ extern "C" int aq_gemv_w8a8_decode_residual(const void* x, int x_dtype, const in
   rc = aq_quant_rowwise_i8(x, x_dtype, M, K, K, xq, sx, stream);
   if (rc) return rc;
   return aq_gemv_w8a8_codes_residual(xq, sx, wq, sw, bias, bias_dtype, residual, y, y_dtype, M, N, K, stream);
+}
+
+extern "C" int aq_gemv_w8a8_decode_attn(const float* partials, int64_t n_slices, int64_t head_dim, const int8_t* wq,
+                                        const float* sw, const void* bias, int bias_dtype, const void* residual,
+                                        void* y, int y_dtype, int64_t M, int64_t N, int64_t K, void* stream) {
+  int mt = 0;
+  int rc = gemv_check(wq, sw, bias, bias_dtype, y, y_dtype, M, N, K, &mt);
+  if (rc) return rc;
+  if ((head_dim != 64 && head_dim != 128) || (K % head_dim) != 0 || n_slices <= 0) return AQ_E_SHAPE;
+  // the in-kernel merge keeps every slice of a lane's vectors in registers
+  if (M > 8 || K > AQ_GEMV_ATTN_MAX_K || n_slices > AQ_GEMV_ATTN_MAX_SLICES) return AQ_E_RANGE;
+  if (M == 0 || N == 0) return AQ_OK;
+  if (!partials) return AQ_E_NULL;
+  if (aq::check_ptr16(partials)) return AQ_E_ALIGN;
+  aq::GemvArgs a{};
+  a.parts = partials;
+  a.parts_ns = (int)n_slices;
+  a.parts_d = (int)head_dim;
+  a.wq = wq;
+  a.sw = sw;
+  a.bias = bias;
+  a.res = residual;
+  a.ldr = N;
+  a.y = y;
+  a.M = (int)M;
+  a.N = (int)N;
+  a.K = (int)K;
+  a.bias_dtype = bias_dtype;
+  a.y_dtype = y_dtype;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  constexpr int NS = AQ_GEMV_ATTN_MAX_SLICES;
+  switch (mt) {
+    case 1: return aq::launch_gemv<1, true, 4, false, NS>(a, st);
+    case 2: return aq::launch_gemv<2, true, 4, false, NS>(a, st);
+    case 4: return aq::launch_gemv<4, true, 4, false, NS>(a, st);
+    default: return aq::launch_gemv<8, true, 4, false, NS>(a, st);
+  }
 }
 
 extern "C" int aq_gemv_w8a8_decode_rmsnorm(const void* x, int x_dtype, const void* gamma, float eps, const int8_t* wq,

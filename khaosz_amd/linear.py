@@ -199,6 +199,13 @@ class QuantLinear(Linear):
                                        residual=residual)
         return ops.linear_w8a8(xq, sx, self.qweight, self.w_scale, self.bias, out_dtype=out_dtype, residual=residual)
 
+    def forward_attn(self, parts: "ops.AttnPartials", out_dtype: torch.dtype = torch.bfloat16,
+                     residual: Optional[Tensor] = None) -> Tensor:
+        """The projection applied to a decode step's attention output that is still in slices
+        (``ops.rope_paged_attn_decode(..., partials=True)``): combined, quantised and multiplied in
+        one launch.  Returns ``[B, out_dim]``, the bits of ``forward`` on the merged output."""
+        return ops.gemv_w8a8_attn(parts, self.qweight, self.w_scale, self.bias, out_dtype=out_dtype, residual=residual)
+
     def extra_repr(self) -> str:
         return f"in_dim={self.in_dim}, out_dim={self.out_dim}, bias={self.bias is not None}, w8a8"
 

@@ -8,7 +8,7 @@ libastrai_q.so.  Together these replace the single call
 """
 from __future__ import annotations
 
-from typing import Optional, Tuple
+from typing import NamedTuple, Optional, Tuple
 
 import torch
 
@@ -360,12 +360,35 @@ def _attn_workspace(workspace, need, dev):
     return workspace.data_ptr(), workspace.numel() * workspace.element_size()
 
 
+class AttnPartials(NamedTuple):
+    """A decode step's attention stopped before its position slices are combined: ``buf`` holds
+    ``[B, n_heads, n_slices, D + 4]`` float32 (D numerators, maximum, denominator, padding)."""
+    buf: torch.Tensor
+    n_slices: int
+    B: int
+    n_heads: int
+    head_dim: int
+
+
+GEMV_ATTN_MAX_ROWS, GEMV_ATTN_MAX_K, GEMV_ATTN_MAX_SLICES = 8, 2048, 4
+
+
+def attn_gemv_fusable(B: int, n_heads: int, head_dim: int, total_len: int) -> bool:
+    """Whether ``gemv_w8a8_attn`` can, and should, combine this step's attention slices itself:
+    within the kernel's limits, and more than one slice (a single slice has no merge launch to
+    save, and the attention kernel's bf16 output is the smaller input)."""
+    return (0 < B <= GEMV_ATTN_MAX_ROWS and n_heads * head_dim <= GEMV_ATTN_MAX_K
+            and 256 < total_len <= GEMV_ATTN_MAX_SLICES * 256)
+
+
 def rope_paged_attn_decode(qkv: torch.Tensor, freqs: torch.Tensor, page_table: torch.Tensor, total_len: int,
                            k_cache: torch.Tensor, v_cache: torch.Tensor, n_heads: int, n_kv_heads: int,
-                           scale: Optional[float] = None, workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+                           scale: Optional[float] = None, workspace: Optional[torch.Tensor] = None,
+                           partials: bool = False):
     """``rope_kv_write`` at position ``total_len - 1`` and ``paged_attn_decode`` over ``total_len``
     positions as one launch (plus the small merge launch for long sequences): same caches and
-    outputs, bit for bit.  Returns the attention output ``[B, Hq, D]``."""
+    outputs, bit for bit.  Returns the attention output ``[B, Hq, D]`` -- or, with ``partials``,
+    the slices' partial results (no merge launch) for ``gemv_w8a8_attn`` to combine."""
     if qkv.dim() != 2:
         raise ValueError(f"one new token per sequence: qkv must be [B, W], got {tuple(qkv.shape)}")
     qkv, fr, fr_stride, page_table = _rope_args(qkv, freqs, page_table, k_cache, v_cache, n_heads, n_kv_heads,
@@ -373,19 +396,68 @@ def rope_paged_attn_decode(qkv: torch.Tensor, freqs: torch.Tensor, page_table: t
     B, D = qkv.shape[0], k_cache.shape[-1]
     if total_len < 1:
         raise ValueError("total_len counts the new token: at least 1")
+    lib = _abi.load()
+    scale = float(scale if scale is not None else D ** -0.5)
+    if partials:
+        if not B:
+            raise ValueError("partial results need at least one sequence")
+        need = int(lib.aq_paged_attn_decode_partials_bytes(B, n_heads, int(total_len)))
+        if (workspace is None or not workspace.is_contiguous() or workspace.device != qkv.device
+                or workspace.dtype != torch.float32 or workspace.numel() * 4 < need or workspace.data_ptr() % 16):
+            workspace = torch.empty(need // 4, dtype=torch.float32, device=qkv.device)
+        with torch.cuda.device(qkv.device):
+            rc = lib.aq_rope_paged_attn_decode_partials(qkv.data_ptr(), fr.data_ptr(), fr_stride, page_table.data_ptr(),
+                                                        page_table.shape[1], int(total_len), k_cache.shape[1],
+                                                        k_cache.data_ptr(), v_cache.data_ptr(), k_cache.shape[0],
+                                                        scale, B, n_heads, n_kv_heads, D, workspace.data_ptr(),
+                                                        workspace.numel() * 4, _stream(qkv))
+        _abi.check(rc, "aq_rope_paged_attn_decode_partials")
+        return AttnPartials(workspace, int(lib.aq_paged_attn_decode_slices(int(total_len))), B, n_heads, D)
     out = torch.empty((B, n_heads, D), dtype=torch.bfloat16, device=qkv.device)
     if B:
         ws_ptr, ws_bytes = _attn_workspace(workspace, paged_attn_workspace_bytes(B, n_heads, n_kv_heads, total_len),
                                            qkv.device)
         with torch.cuda.device(qkv.device):
-            rc = _abi.load().aq_rope_paged_attn_decode(qkv.data_ptr(), fr.data_ptr(), fr_stride, page_table.data_ptr(),
-                                                       page_table.shape[1], int(total_len), k_cache.shape[1],
-                                                       k_cache.data_ptr(), v_cache.data_ptr(), k_cache.shape[0],
-                                                       float(scale if scale is not None else D ** -0.5),
-                                                       out.data_ptr(), B, n_heads, n_kv_heads, D, ws_ptr, ws_bytes,
-                                                       _stream(qkv))
+            rc = lib.aq_rope_paged_attn_decode(qkv.data_ptr(), fr.data_ptr(), fr_stride, page_table.data_ptr(),
+                                               page_table.shape[1], int(total_len), k_cache.shape[1],
+                                               k_cache.data_ptr(), v_cache.data_ptr(), k_cache.shape[0], scale,
+                                               out.data_ptr(), B, n_heads, n_kv_heads, D, ws_ptr, ws_bytes,
+                                               _stream(qkv))
         _abi.check(rc, "aq_rope_paged_attn_decode")
     return out
+
+
+def gemv_w8a8_attn(parts: AttnPartials, wq, sw, bias=None, out_dtype=torch.bfloat16, residual=None) -> torch.Tensor:
+    """The output projection of a decode step on attention partial results: combines the slices
+    (the merge kernel's arithmetic), quantises the ``[B, n_heads * D]`` rows and multiplies, one
+    launch; the bits of ``rope_paged_attn_decode`` followed by ``gemv_w8a8_decode``."""
+    _need_gpu(parts.buf, wq, sw, bias, residual)
+    M, K = parts.B, parts.n_heads * parts.head_dim
+    N = wq.shape[0]
+    if wq.dtype != torch.int8 or wq.dim() != 2 or wq.shape[1] != K:
+        raise ValueError(f"wq must be int8 [N, {K}], got {wq.dtype} {tuple(wq.shape)}")
+    if sw.dtype != torch.float32 or sw.numel() != N:
+        raise ValueError("sw must be float32 [N]")
+    if out_dtype not in _DT:
+        raise ValueError(f"out_dtype {out_dtype} is not supported")
+    if M > GEMV_ATTN_MAX_ROWS or K > GEMV_ATTN_MAX_K or parts.n_slices > GEMV_ATTN_MAX_SLICES:
+        raise ValueError(f"gemv_w8a8_attn takes at most {GEMV_ATTN_MAX_ROWS} rows of {GEMV_ATTN_MAX_K} elements in "
+                         f"{GEMV_ATTN_MAX_SLICES} slices; got {M} x {K} in {parts.n_slices}")
+    if parts.buf.dtype != torch.float32 or parts.buf.numel() < M * parts.n_heads * parts.n_slices * (parts.head_dim + 4):
+        raise ValueError("the partial results do not cover [B, n_heads, n_slices, D + 4] float32")
+    wq, sw = wq.contiguous(), sw.contiguous()
+    b, bdt = _bias_args(bias, N)
+    r = _residual_arg(residual, M, N, out_dtype, wq.device)
+    y = torch.empty((M, N), dtype=out_dtype, device=wq.device)
+    if N:
+        with torch.cuda.device(wq.device):
+            rc = _abi.load().aq_gemv_w8a8_decode_attn(parts.buf.data_ptr(), parts.n_slices, parts.head_dim,
+                                                      wq.data_ptr(), sw.data_ptr(),
+                                                      b.data_ptr() if b is not None else None, bdt,
+                                                      r.data_ptr() if r is not None else None, y.data_ptr(),
+                                                      _DT[out_dtype], M, N, K, _stream(wq))
+        _abi.check(rc, "aq_gemv_w8a8_decode_attn")
+    return y
 
 
 def prefill_attn_causal(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: Optional[float] = None) -> torch.Tensor:
@@ -421,6 +493,11 @@ def prefill_attn_causal(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale
 def paged_attn_workspace_bytes(B: int, n_heads: int, n_kv_heads: int, total_len: int) -> int:
     """Bytes of device workspace ``paged_attn_decode`` needs for this shape (0: none)."""
     return int(_abi.load().aq_paged_attn_decode_workspace_bytes(B, n_heads, n_kv_heads, int(total_len)))
+
+
+def paged_attn_partials_bytes(B: int, n_heads: int, total_len: int) -> int:
+    """Bytes the slices' partial results of a decode step take (also enough as its workspace)."""
+    return int(_abi.load().aq_paged_attn_decode_partials_bytes(B, n_heads, int(total_len)))
 
 
 def paged_attn_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, page_table: torch.Tensor,

@@ -374,3 +374,44 @@ def test_decode_attention_kernels_track_the_torch_attention_path():
         pb = b(x[:, :S], _freqs(tab, B, 0, S), None, cb2.bind(holes, S))
         assert ((pa.float() - pb.float()).norm() / pa.float().norm()).item() < 1e-2
         assert torch.allclose(ca2.k.float(), cb2.k.float(), rtol=1e-2, atol=1e-2) and torch.equal(ca2.v, cb2.v)
+
+
+@pytest.mark.gpu
+def test_decode_step_with_the_merge_inside_the_output_projection_is_bit_identical(monkeypatch):
+    """Past 256 cached positions the attention runs in slices; the output projection then combines them
+    itself (one launch less).  Same bits as the path with the separate merge launch, with and without
+    the residual in the epilogue."""
+    from khaosz_amd import fuse_shared_inputs, ops
+
+    dev, dt = "cuda:0", torch.bfloat16
+    torch.manual_seed(5)
+    for residuals in (False, True):
+        blk = DecoderBlock(512, 8, 1408, 2)       # head dimension 64, four query heads per KV head
+        blk.reset_parameters()
+        blk = blk.to(dev).to(dt)
+        quantize_model(blk)
+        fuse_shared_inputs(blk, norms=True, decode_attention=True, residuals=residuals)
+        B, S, page = 3, 300, 32
+        P = (S + 8 + page - 1) // page
+        tab = rotary_table(64, 512, device=dev)
+        table = torch.randperm(B * P, device=dev).view(B, P)
+        c1, c2 = PagedKV(B * P, page, 2, 64, dev, dt), PagedKV(B * P, page, 2, 64, dev, dt)
+        x = torch.randn(B, S + 3, 512, device=dev).to(dt)
+        calls = []
+        real = ops.gemv_w8a8_attn
+        monkeypatch.setattr(ops, "gemv_w8a8_attn", lambda *a, **k: (calls.append(1), real(*a, **k))[1])
+        with torch.inference_mode():
+            blk(x[:, :S], _freqs(tab, B, 0, S), None, c1.bind(table, S))
+            blk(x[:, :S], _freqs(tab, B, 0, S), None, c2.bind(table, S))
+            for t in range(3):
+                pos = S + t
+                y1 = blk(x[:, pos:pos + 1], _freqs(tab, B, pos, 1), None, c1.bind(table, pos + 1))
+                n = len(calls)
+                assert n == t + 1                                      # the fused path ran
+                with monkeypatch.context() as m:
+                    m.setattr(ops, "attn_gemv_fusable", lambda *a: False)
+                    y2 = blk(x[:, pos:pos + 1], _freqs(tab, B, pos, 1), None, c2.bind(table, pos + 1))
+                assert len(calls) == n                                 # and here it did not
+                assert torch.equal(y1, y2)
+        assert torch.equal(c1.k, c2.k) and torch.equal(c1.v, c2.v)
+        monkeypatch.undo()

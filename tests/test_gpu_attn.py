@@ -197,3 +197,77 @@ def test_attn_argument_checks():
     kc = torch.zeros(4, 8, 2, 128, dtype=torch.bfloat16, device=DEV)
     with pytest.raises(ValueError):
         ops.paged_attn_decode(q, kc, kc.clone(), tab, 5)          # 5 query heads per KV head
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,page,T", [(1, 8, 2, 16, 1), (4, 24, 4, 128, 640), (8, 16, 4, 64, 576), (3, 8, 1, 16, 1000),
+                                              (2, 4, 2, 64, 513), (5, 16, 2, 16, 257), (7, 6, 2, 16, 100), (8, 8, 8, 32, 1024), (2, 32, 8, 16, 300)])
+@pytest.mark.parametrize("D", [128, 64])
+def test_output_projection_on_attention_partials_equals_the_three_launches(B, Hq, Hkv, page, T, D):
+    """attention stopped before its merge + the output projection that combines the slices itself,
+    against attention (with its merge launch) + the decode GEMV: outputs bit for bit, with and
+    without a residual, bf16 and fp32 outputs; the caches see the same writes."""
+    _say("gemv_w8a8_attn", B, Hq, Hkv, page, T, D)
+    P = (T + page - 1) // page
+    n_pages = B * P + 2
+    K, N = Hq * D, 200
+    g = torch.Generator().manual_seed(T + D)
+    qkv = torch.randn(B, (Hq + 2 * Hkv) * D, generator=g).to(torch.bfloat16).to(DEV)
+    ang = torch.rand(B, D // 2, generator=g) * 6.28
+    freqs = torch.polar(torch.ones_like(ang), ang).to(DEV)
+    kc = torch.randn(n_pages, page, Hkv, D, generator=g).to(torch.bfloat16).to(DEV)
+    vc = torch.randn(n_pages, page, Hkv, D, generator=g).to(torch.bfloat16).to(DEV)
+    table = torch.randperm(n_pages, generator=g)[:B * P].view(B, P)
+    if B > 2 and P > 1:
+        table[1, 0] = -1                                  # a hole: zero keys and values there
+    table = table.to(DEV)
+    wq = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8).to(DEV)
+    sw = (torch.rand(N, generator=g) * 0.01 + 1e-3).to(DEV)
+    bias = torch.randn(N, generator=g).to(DEV)
+    k1, v1, k2, v2 = kc.clone(), vc.clone(), kc.clone(), vc.clone()
+    assert ops.attn_gemv_fusable(B, Hq, D, T) == (K <= 2048 and T > 256)
+    attn = ops.rope_paged_attn_decode(qkv, freqs, table, T, k1, v1, Hq, Hkv)
+    if K > 2048:
+        parts = ops.rope_paged_attn_decode(qkv, freqs, table, T, k2, v2, Hq, Hkv, partials=True)
+        with pytest.raises(ValueError):
+            ops.gemv_w8a8_attn(parts, wq, sw)
+        return
+    parts = ops.rope_paged_attn_decode(qkv, freqs, table, T, k2, v2, Hq, Hkv, partials=True)
+    assert parts.n_slices == (T + 255) // 256 and (parts.B, parts.n_heads, parts.head_dim) == (B, Hq, D)
+    assert torch.equal(k1, k2) and torch.equal(v1, v2)
+    for dt in (torch.bfloat16, torch.float32):
+        res = torch.randn(B, N, generator=g).to(dt).to(DEV)
+        for b_, r_ in ((None, None), (bias, res)):
+            want = ops.gemv_w8a8_decode(attn.view(B, K), wq, sw, b_, out_dtype=dt, residual=r_)
+            got = ops.gemv_w8a8_attn(parts, wq, sw, b_, out_dtype=dt, residual=r_)
+            assert torch.equal(got, want)
+
+
+def test_attention_partials_entry_points_check_their_arguments():
+    from khaosz_amd import _abi
+    lib = _abi.load()
+    _say("attention partials checks")
+    assert lib.aq_paged_attn_decode_slices(0) == 0 and lib.aq_paged_attn_decode_slices(256) == 1
+    assert lib.aq_paged_attn_decode_slices(257) == 2
+    assert lib.aq_paged_attn_decode_partials_bytes(2, 4, 300) == 2 * 4 * 2 * 132 * 4
+    buf = torch.zeros(4096, dtype=torch.float32, device=DEV)
+    w = torch.zeros(64, 2048, dtype=torch.int8, device=DEV)
+    sw = torch.ones(64, device=DEV)
+    y = torch.zeros(8, 64, dtype=torch.bfloat16, device=DEV)
+    call = lambda ns, d, m, k: lib.aq_gemv_w8a8_decode_attn(buf.data_ptr(), ns, d, w.data_ptr(), sw.data_ptr(), None, 0,
+                                                            None, y.data_ptr(), 1, m, 64, k, None)
+    assert call(5, 128, 1, 2048) == -6      # more slices than the kernel holds: AQ_E_RANGE
+    assert call(1, 128, 9, 2048) == -6      # more rows
+    assert call(1, 128, 1, 4096) == -6      # longer rows
+    assert call(1, 96, 1, 1920) == -2       # head dimension: AQ_E_SHAPE
+    assert call(1, 128, 1, 2000) == -2      # K not whole heads
+    assert call(0, 128, 1, 2048) == -2
+    # partial results need their buffer even for one slice
+    q = torch.zeros(1, 2, 64, dtype=torch.bfloat16, device=DEV)
+    kc = torch.zeros(2, 16, 1, 64, dtype=torch.bfloat16, device=DEV)
+    tb = torch.zeros(1, 1, dtype=torch.int64, device=DEV)
+    rc = lib.aq_paged_attn_decode_partials(q.data_ptr(), kc.data_ptr(), kc.data_ptr(), tb.data_ptr(), 1, 10, 16, 2, 0.125,
+                                           1, 2, 1, 64, None, 0, None)
+    assert rc == -1                         # AQ_E_NULL
+    rc = lib.aq_paged_attn_decode_partials(q.data_ptr(), kc.data_ptr(), kc.data_ptr(), tb.data_ptr(), 1, 10, 16, 2, 0.125,
+                                           1, 2, 1, 64, buf.data_ptr(), 64, None)
+    assert rc == -5                         # AQ_E_WORKSPACE

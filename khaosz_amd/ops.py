@@ -17,8 +17,35 @@ from . import _abi
 _DT = {torch.float32: _abi.AQ_F32, torch.bfloat16: _abi.AQ_BF16}
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_cur_device = getattr(torch._C, "_cuda_getDevice", None)
+
+
 def _stream(t: torch.Tensor) -> int:
+    """torch's current HIP stream on the tensor's device, as the raw handle the C ABI takes."""
+    if _raw_stream is not None:
+        return _raw_stream(t.device.index if t.device.index is not None else torch.cuda.current_device())
     return torch.cuda.current_stream(t.device).cuda_stream
+
+
+class _OnDevice:
+    """``torch.cuda.device(dev)`` that costs nothing when ``dev`` already is the current device (the
+    usual case; a launch goes to the current device)."""
+    __slots__ = ("ctx",)
+
+    def __init__(self, dev: torch.device):
+        self.ctx = None
+        if _cur_device is None or dev.index is None or _cur_device() != dev.index:
+            self.ctx = torch.cuda.device(dev)
+
+    def __enter__(self):
+        if self.ctx is not None:
+            self.ctx.__enter__()
+
+    def __exit__(self, *exc):
+        if self.ctx is not None:
+            return self.ctx.__exit__(*exc)
+        return False
 
 
 def _need_gpu(*ts: Optional[torch.Tensor]) -> None:
@@ -65,7 +92,7 @@ def quant_rowwise_i8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     q = torch.empty((M, K), dtype=torch.int8, device=x.device)
     s = torch.empty((M,), dtype=torch.float32, device=x.device)
     if M:
-        with torch.cuda.device(x.device):
+        with _OnDevice(x.device):
             rc = _abi.load().aq_quant_rowwise_i8(x2.data_ptr(), _dt(x2, "x"), M, K, x2.stride(0), q.data_ptr(),
                                                  s.data_ptr(), _stream(x))
         _abi.check(rc, "aq_quant_rowwise_i8")
@@ -90,7 +117,7 @@ def rmsnorm_quant_rowwise_i8(x: torch.Tensor, gamma: torch.Tensor, eps: float) -
     q = torch.empty((M, K), dtype=torch.int8, device=x2.device)
     s = torch.empty((M,), dtype=torch.float32, device=x2.device)
     if M:
-        with torch.cuda.device(x2.device):
+        with _OnDevice(x2.device):
             rc = _abi.load().aq_rmsnorm_quant_rowwise_i8(x2.data_ptr(), _dt(x2, "x"), gamma.data_ptr(), _dt(gamma, "gamma"),
                                                          float(eps), M, K, x2.stride(0), q.data_ptr(), s.data_ptr(),
                                                          _stream(x2))
@@ -111,7 +138,7 @@ def swiglu_quant_rowwise_i8(ug: torch.Tensor) -> Tuple[torch.Tensor, torch.Tenso
     q = torch.empty((M, F), dtype=torch.int8, device=u2.device)
     s = torch.empty((M,), dtype=torch.float32, device=u2.device)
     if M:
-        with torch.cuda.device(u2.device):
+        with _OnDevice(u2.device):
             rc = _abi.load().aq_swiglu_quant_rowwise_i8(u2.data_ptr(), _dt(u2, "ug"), M, F, u2.stride(0), q.data_ptr(),
                                                         s.data_ptr(), _stream(u2))
         _abi.check(rc, "aq_swiglu_quant_rowwise_i8")
@@ -128,7 +155,7 @@ def quant_tensor_fp8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     q = torch.empty(xc.shape, dtype=torch.uint8, device=x.device)
     s = torch.empty((1,), dtype=torch.float32, device=x.device)
     ws = torch.empty((1,), dtype=torch.int32, device=x.device)
-    with torch.cuda.device(x.device):
+    with _OnDevice(x.device):
         rc = _abi.load().aq_quant_tensor_fp8(xc.data_ptr(), _dt(xc, "x"), n, q.data_ptr(), s.data_ptr(),
                                              ws.data_ptr(), _stream(x))
     _abi.check(rc, "aq_quant_tensor_fp8")
@@ -148,7 +175,7 @@ def gemm_i8_i32(xq: torch.Tensor, wq: torch.Tensor) -> torch.Tensor:
     _check_k(K)
     acc = torch.empty((M, N), dtype=torch.int32, device=xq.device)
     if M and N:
-        with torch.cuda.device(xq.device):
+        with _OnDevice(xq.device):
             rc = _abi.load().aq_gemm_i8_i32(xq.data_ptr(), wq.data_ptr(), acc.data_ptr(), M, N, K, _stream(xq))
         _abi.check(rc, "aq_gemm_i8_i32")
     return acc
@@ -195,7 +222,7 @@ def linear_w8a8(xq, sx, wq, sw, bias=None, out_dtype=torch.bfloat16, residual=No
     r = _residual_arg(residual, M, N, out_dtype, xq.device)
     y = torch.empty((M, N), dtype=out_dtype, device=xq.device)
     if M and N:
-        with torch.cuda.device(xq.device):
+        with _OnDevice(xq.device):
             rc = _abi.load().aq_linear_w8a8_residual(xq.data_ptr(), sx.data_ptr(), wq.data_ptr(), sw.data_ptr(),
                                                      b.data_ptr() if b is not None else None, bdt,
                                                      r.data_ptr() if r is not None else None, y.data_ptr(),
@@ -241,7 +268,7 @@ def gemv_w8a8_decode(x, wq, sw, bias=None, out_dtype=None, workspace: Optional[t
             raise ValueError(f"the norm's gain must be {x2.dtype} [{K}], got {gamma.dtype} {tuple(gamma.shape)}")
         gamma = gamma.contiguous()
     if M and N:
-        with torch.cuda.device(x.device):
+        with _OnDevice(x.device):
             if norm is None:
                 rc = lib.aq_gemv_w8a8_decode_residual(x2.data_ptr(), _dt(x2, "x"), wq.data_ptr(), sw.data_ptr(),
                                                       b.data_ptr() if b is not None else None, bdt,
@@ -282,7 +309,7 @@ def gemv_w8a8_codes(xq, sx, wq, sw, bias=None, out_dtype=torch.bfloat16, residua
     r = _residual_arg(residual, M, N, out_dtype, xq.device)
     y = torch.empty((M, N), dtype=out_dtype, device=xq.device)
     if M and N:
-        with torch.cuda.device(xq.device):
+        with _OnDevice(xq.device):
             rc = _abi.load().aq_gemv_w8a8_codes_residual(xq.data_ptr(), sx.data_ptr(), wq.data_ptr(), sw.data_ptr(),
                                                          b.data_ptr() if b is not None else None, bdt,
                                                          r.data_ptr() if r is not None else None, y.data_ptr(),
@@ -339,7 +366,7 @@ def rope_kv_write(qkv: torch.Tensor, freqs: torch.Tensor, page_table: torch.Tens
     q = torch.empty((B, S, n_heads, D), dtype=torch.bfloat16, device=qkv.device)
     k = torch.empty((B, S, n_kv_heads, D), dtype=torch.bfloat16, device=qkv.device) if return_k else None
     if B and S:
-        with torch.cuda.device(qkv.device):
+        with _OnDevice(qkv.device):
             rc = _abi.load().aq_rope_kv_write(qkv.data_ptr(), fr.data_ptr(), fr_stride, page_table.data_ptr(),
                                               page_table.shape[1], int(pos), S, k_cache.shape[1], k_cache.data_ptr(),
                                               v_cache.data_ptr(), k_cache.shape[0], q.data_ptr(),
@@ -405,7 +432,7 @@ def rope_paged_attn_decode(qkv: torch.Tensor, freqs: torch.Tensor, page_table: t
         if (workspace is None or not workspace.is_contiguous() or workspace.device != qkv.device
                 or workspace.dtype != torch.float32 or workspace.numel() * 4 < need or workspace.data_ptr() % 16):
             workspace = torch.empty(need // 4, dtype=torch.float32, device=qkv.device)
-        with torch.cuda.device(qkv.device):
+        with _OnDevice(qkv.device):
             rc = lib.aq_rope_paged_attn_decode_partials(qkv.data_ptr(), fr.data_ptr(), fr_stride, page_table.data_ptr(),
                                                         page_table.shape[1], int(total_len), k_cache.shape[1],
                                                         k_cache.data_ptr(), v_cache.data_ptr(), k_cache.shape[0],
@@ -417,7 +444,7 @@ def rope_paged_attn_decode(qkv: torch.Tensor, freqs: torch.Tensor, page_table: t
     if B:
         ws_ptr, ws_bytes = _attn_workspace(workspace, paged_attn_workspace_bytes(B, n_heads, n_kv_heads, total_len),
                                            qkv.device)
-        with torch.cuda.device(qkv.device):
+        with _OnDevice(qkv.device):
             rc = lib.aq_rope_paged_attn_decode(qkv.data_ptr(), fr.data_ptr(), fr_stride, page_table.data_ptr(),
                                                page_table.shape[1], int(total_len), k_cache.shape[1],
                                                k_cache.data_ptr(), v_cache.data_ptr(), k_cache.shape[0], scale,
@@ -450,7 +477,7 @@ def gemv_w8a8_attn(parts: AttnPartials, wq, sw, bias=None, out_dtype=torch.bfloa
     r = _residual_arg(residual, M, N, out_dtype, wq.device)
     y = torch.empty((M, N), dtype=out_dtype, device=wq.device)
     if N:
-        with torch.cuda.device(wq.device):
+        with _OnDevice(wq.device):
             rc = _abi.load().aq_gemv_w8a8_decode_attn(parts.buf.data_ptr(), parts.n_slices, parts.head_dim,
                                                       wq.data_ptr(), sw.data_ptr(),
                                                       b.data_ptr() if b is not None else None, bdt,
@@ -482,7 +509,7 @@ def prefill_attn_causal(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale
     v, vs = tokens(v, Hkv)
     out = torch.empty((B, S, Hq, D), dtype=torch.bfloat16, device=q.device)
     if B and S:
-        with torch.cuda.device(q.device):
+        with _OnDevice(q.device):
             rc = _abi.load().aq_prefill_attn_causal(q.data_ptr(), qs, k.data_ptr(), ks, v.data_ptr(), vs, out.data_ptr(),
                                                     float(scale if scale is not None else D ** -0.5), B, S, Hq, Hkv, D,
                                                     _stream(q))
@@ -522,7 +549,7 @@ def paged_attn_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     out = torch.empty_like(q)
     if B:
         ws_ptr, ws_bytes = _attn_workspace(workspace, paged_attn_workspace_bytes(B, Hq, Hkv, total_len), q.device)
-        with torch.cuda.device(q.device):
+        with _OnDevice(q.device):
             rc = _abi.load().aq_paged_attn_decode(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                                                   page_table.data_ptr(), page_table.shape[1], int(total_len),
                                                   k_cache.shape[1], k_cache.shape[0],
@@ -554,7 +581,7 @@ def linear_fp8(xq, sx, wq, sw, out_dtype=torch.bfloat16) -> torch.Tensor:
     xq, wq = xq.contiguous(), wq.contiguous()
     y = torch.empty((M, N), dtype=out_dtype, device=xq.device)
     if M and N:
-        with torch.cuda.device(xq.device):
+        with _OnDevice(xq.device):
             rc = _abi.load().aq_linear_fp8(xq.data_ptr(), sx.data_ptr(), wq.data_ptr(), sw.data_ptr(), y.data_ptr(),
                                            _DT[out_dtype], M, N, K, _stream(xq))
         _abi.check(rc, "aq_linear_fp8")

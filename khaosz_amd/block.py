@@ -170,19 +170,30 @@ class PagedKV:
 
 
 class GQA(nn.Module):
-    """Grouped-query attention (astrai/model/components/attention.py:32-109), without the
-    optional qk-norm and output gate that benchmark configuration 5 leaves off."""
+    """Grouped-query attention (astrai/model/components/attention.py:32-109), with its two
+    options: RMSNorm over the head dimension of q and k after the rotation (``use_qk_norm``,
+    attention.py:62-64,88-89) and a sigmoid output gate computed from the block input by a fifth
+    Linear (``use_gated_attention``, attention.py:66-67,105-106).  Benchmark configuration 5
+    leaves both off; with qk-norm the paged-cache kernels are not used (they store the rotated,
+    un-normalised key)."""
 
-    def __init__(self, dim: int, n_heads: int, n_kv_heads: int, layer_id: int = 0):
+    def __init__(self, dim: int, n_heads: int, n_kv_heads: int, layer_id: int = 0, use_qk_norm: bool = False,
+                 norm_eps: float = 1e-5, use_gated_attention: bool = False):
         super().__init__()
         if dim % n_heads or n_heads % n_kv_heads:
             raise ValueError("dim must divide into heads and heads into kv heads")
         self.head_dim = dim // n_heads
         self.n_heads, self.n_kv_heads, self.layer_id = n_heads, n_kv_heads, layer_id
+        self.use_qk_norm, self.use_gated_attention = use_qk_norm, use_gated_attention
         self.q_proj = Linear(dim, n_heads * self.head_dim)
         self.k_proj = Linear(dim, n_kv_heads * self.head_dim)
         self.v_proj = Linear(dim, n_kv_heads * self.head_dim)
         self.o_proj = Linear(dim, dim)
+        if use_qk_norm:
+            self.q_norm = RMSNorm(self.head_dim, norm_eps)
+            self.k_norm = RMSNorm(self.head_dim, norm_eps)
+        if use_gated_attention:
+            self.gate = Linear(dim, dim)
         self._qkv: Optional[QuantLinear] = None  # not a registered child: the state dict keeps q/k/v keys
         self._decode_attention = False
 
@@ -205,10 +216,27 @@ class GQA(nn.Module):
         repeating them.  Needs the fused q/k/v projection, bf16, head dimension 64 or 128 and
         1, 2, 3, 4, 6 or 8 query heads per KV head.
         Outputs agree within bf16 rounding."""
-        if (self._qkv is not None and self.head_dim in (64, 128)
+        if (self._qkv is not None and self.head_dim in (64, 128) and not self.use_qk_norm
                 and self.n_heads // self.n_kv_heads in (1, 2, 3, 4, 6, 8)):
             self._decode_attention = True
         return self._decode_attention
+
+    def _gated(self, out: Tensor, x: Tensor, norm, codes=None) -> Tensor:
+        """``out * sigmoid(gate(x))`` (attention.py:105-106); ``x`` is the attention input, still to
+        be normalised when ``norm`` is given, or replaced by its quantised form ``codes``."""
+        if not self.use_gated_attention:
+            return out
+        if codes is not None:
+            if not isinstance(self.gate, QuantLinear):
+                raise ValueError("a pre-quantised input needs a quantized gate projection")
+            g = self.gate.forward_codes(codes[0], codes[1], x.dtype)
+        elif norm is None:
+            g = self.gate(x)
+        elif isinstance(self.gate, QuantLinear):
+            g = self.gate(x, norm=norm)
+        else:
+            g = self.gate(F.rms_norm(x, (x.shape[-1],), norm[0], norm[1]))
+        return out * torch.sigmoid(g).view(out.shape)
 
     def _out(self, out: Tensor, residual: Optional[Tensor]) -> Tensor:
         """o_proj, plus the residual stream when the caller hands it over."""
@@ -238,7 +266,7 @@ class GQA(nn.Module):
             qkv = self._project_qkv(x, codes, norm)
             # the output projection combines the attention's position slices itself when the step is small
             # enough for its in-kernel quantiser: one launch less
-            split = (isinstance(self.o_proj, QuantLinear)
+            split = (isinstance(self.o_proj, QuantLinear) and not self.use_gated_attention
                      and ops.attn_gemv_fusable(B, self.n_heads, self.head_dim, cache.total_len))
             out = ops.rope_paged_attn_decode(qkv.view(B, -1), rotary_emb.reshape(B, -1), cache.page_table,
                                              cache.total_len, cache.k_layers[self.layer_id],
@@ -246,7 +274,7 @@ class GQA(nn.Module):
                                              workspace=cache.attn_workspace(self.n_heads), partials=split)
             if split:
                 return self.o_proj.forward_attn(out, x.dtype, residual).view(B, 1, -1)
-            return self._out(out.view(B, 1, -1), residual)
+            return self._out(self._gated(out.view(B, 1, -1), x, norm, codes), residual)
         if (self._decode_attention and isinstance(cache, PagedKV) and x.is_cuda and x.dtype == torch.bfloat16
                 and S <= cache.total_len):
             # several new tokens (prefill): rotation and the page writes as one launch; a prompt on an empty
@@ -259,13 +287,13 @@ class GQA(nn.Module):
             if start == 0 and cache.all_mapped:
                 v = qkv[..., nq + nkv:].view(B, S, self.n_kv_heads, self.head_dim)
                 if attn_mask is None:  # a prompt attending to itself: the causal kernel, v read in place from qkv
-                    return self._out(ops.prefill_attn_causal(q, k, v).view(B, S, -1), residual)
+                    return self._out(self._gated(ops.prefill_attn_causal(q, k, v).view(B, S, -1), x, norm, codes), residual)
             else:
                 k, v = cache.gather(self.layer_id)
             out = F.scaled_dot_product_attention(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), attn_mask,
                                                  is_causal=attn_mask is None,
                                                  enable_gqa=self.n_heads != self.n_kv_heads)
-            return self._out(out.transpose(1, 2).reshape(B, S, -1), residual)
+            return self._out(self._gated(out.transpose(1, 2).reshape(B, S, -1), x, norm, codes), residual)
         if self._qkv is not None:
             nq, nkv = self.n_heads * self.head_dim, self.n_kv_heads * self.head_dim
             qkv = self._project_qkv(x, codes, norm)
@@ -276,6 +304,8 @@ class GQA(nn.Module):
         k = k.reshape(B, S, self.n_kv_heads, self.head_dim)
         v = v.reshape(B, S, self.n_kv_heads, self.head_dim)
         q, k = apply_rotary(q, rotary_emb), apply_rotary(k, rotary_emb)
+        if self.use_qk_norm:  # after the rotation, as the reference does (attention.py:86-89)
+            q, k = self.q_norm(q), self.k_norm(k)
         if cache is not None:
             cache.write(self.layer_id, k, v)
             k, v = cache.gather(self.layer_id)
@@ -285,7 +315,7 @@ class GQA(nn.Module):
             v = v.repeat_interleave(rep, dim=2)
         out = F.scaled_dot_product_attention(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), attn_mask,
                                              is_causal=attn_mask is None)
-        return self._out(out.transpose(1, 2).reshape(B, S, -1), residual)
+        return self._out(self._gated(out.transpose(1, 2).reshape(B, S, -1), x, norm, codes), residual)
 
 
 class MLP(nn.Module):
@@ -333,9 +363,9 @@ class DecoderBlock(nn.Module):
     """``x += attn(norm(x)); x += mlp(norm(x))`` (astrai/model/components/decoder_block.py:12-59)."""
 
     def __init__(self, dim: int, n_heads: int, dim_ffn: int, n_kv_heads: int, norm_eps: float = 1e-5,
-                 layer_id: int = 0):
+                 layer_id: int = 0, use_qk_norm: bool = False, use_gated_attention: bool = False):
         super().__init__()
-        self.attention = GQA(dim, n_heads, n_kv_heads, layer_id)
+        self.attention = GQA(dim, n_heads, n_kv_heads, layer_id, use_qk_norm, norm_eps, use_gated_attention)
         self.input_norm = RMSNorm(dim, norm_eps)
         self.post_attention_norm = RMSNorm(dim, norm_eps)
         self.mlp = MLP(dim, dim_ffn)

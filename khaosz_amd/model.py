@@ -40,6 +40,8 @@ class LMConfig:
     norm_eps: float = 1e-5
     rope_theta: float = 10000.0
     tie_weight: bool = False
+    use_qk_norm: bool = False
+    use_gated_attention: bool = False
 
 
 class Embedding(nn.Module):
@@ -70,7 +72,8 @@ class AutoRegressiveLM(nn.Module):
         self._freqs = rotary_table(head_dim, config.max_len, config.rope_theta)
         self.embed_tokens = Embedding(config.vocab_size, config.dim)
         self.layers = nn.ModuleList([
-            DecoderBlock(config.dim, config.n_heads, config.dim_ffn, config.n_kv_heads, config.norm_eps, layer_id=i)
+            DecoderBlock(config.dim, config.n_heads, config.dim_ffn, config.n_kv_heads, config.norm_eps, layer_id=i,
+                         use_qk_norm=config.use_qk_norm, use_gated_attention=config.use_gated_attention)
             for i in range(config.n_layers)])
         self.norm = RMSNorm(config.dim, config.norm_eps)
         self.lm_head = Linear(config.dim, config.vocab_size)

@@ -74,6 +74,50 @@ def test_gqa_matches_a_hand_written_causal_attention():
     assert torch.allclose(y, want, atol=1e-4)
 
 
+def test_gqa_options_qk_norm_and_output_gate_by_hand():
+    """use_qk_norm: RMSNorm over the head dimension of q and k after the rotation
+    (attention.py:86-89); use_gated_attention: the attention output times sigmoid(gate(x)) before
+    o_proj (attention.py:105-108).  Parameter names as in the reference."""
+    torch.manual_seed(1)
+    dim, H, Hkv, B, S = 32, 4, 2, 2, 5
+    att = GQA(dim, H, Hkv, use_qk_norm=True, norm_eps=1e-5, use_gated_attention=True)
+    for l in (att.q_proj, att.k_proj, att.v_proj, att.o_proj, att.gate):
+        l.reset_parameters()
+    with torch.no_grad():
+        att.q_norm.weight.copy_(torch.rand(dim // H) + 0.5)
+        att.k_norm.weight.copy_(torch.rand(dim // H) + 0.5)
+    assert {"q_norm.weight", "k_norm.weight", "gate.weight"} <= set(att.state_dict())
+    x = torch.randn(B, S, dim)
+    tab = rotary_table(dim // H, 16)
+    fr = _freqs(tab, B, 0, S)
+    y = att(x, fr)
+    D = dim // H
+    rms = lambda t, w: t / torch.sqrt((t * t).mean(-1, keepdim=True) + 1e-5) * w
+    q = rms(apply_rotary((x @ att.q_proj.weight.T).view(B, S, H, D), fr), att.q_norm.weight)
+    k = rms(apply_rotary((x @ att.k_proj.weight.T).view(B, S, Hkv, D), fr), att.k_norm.weight)
+    v = (x @ att.v_proj.weight.T).view(B, S, Hkv, D)
+    out = torch.zeros(B, S, H, D)
+    for b in range(B):
+        for h in range(H):
+            g = h // (H // Hkv)
+            for i in range(S):
+                sc = torch.stack([(q[b, i, h] * k[b, j, g]).sum() / math.sqrt(D) for j in range(i + 1)])
+                w = torch.softmax(sc, 0)
+                out[b, i, h] = sum(w[j] * v[b, j, g] for j in range(i + 1))
+    gated = out.reshape(B, S, dim) * torch.sigmoid(x @ att.gate.weight.T)
+    assert torch.allclose(y, gated @ att.o_proj.weight.T, atol=1e-4)
+    # the cached key is the normalised one: a decode step on a cache equals the full pass
+    blk = DecoderBlock(dim, H, 88, Hkv, use_qk_norm=True, use_gated_attention=True)
+    blk.reset_parameters()
+    xs = torch.randn(B, S + 1, dim)
+    full = blk(xs, _freqs(tab, B, 0, S + 1))
+    cache = ContiguousKV(B, 16, Hkv, D, "cpu", torch.float32)
+    blk(xs[:, :S], _freqs(tab, B, 0, S), None, cache.bind(S))
+    step = blk(xs[:, S:], _freqs(tab, B, S, 1), decode_mask(B, S + 1, "cpu", torch.float32), cache.bind(S + 1))
+    assert torch.allclose(step[:, 0], full[:, S], atol=1e-5)
+    assert not blk.attention.fuse_decode_attention()           # never with qk-norm
+
+
 def _block(dim=64, heads=4, kv=2, ffn=176, seed=0):
     torch.manual_seed(seed)
     b = DecoderBlock(dim, heads, ffn, kv)
@@ -415,3 +459,43 @@ def test_decode_step_with_the_merge_inside_the_output_projection_is_bit_identica
                 assert torch.equal(y1, y2)
         assert torch.equal(c1.k, c2.k) and torch.equal(c1.v, c2.v)
         monkeypatch.undo()
+
+
+@pytest.mark.gpu
+def test_gated_attention_block_quantized_and_fused_paths_agree():
+    """A block with the output gate: the gate is a fifth quantized Linear on the attention input; the
+    fused paths (norm inside the projections, paged-cache kernels, residual epilogues) give the
+    outputs of the plain quantized block within bf16 rounding, prefill and decode, and the
+    quantized block tracks the float one."""
+    from khaosz_amd import fuse_shared_inputs
+
+    dev, dt = "cuda:0", torch.bfloat16
+    torch.manual_seed(9)
+    f = DecoderBlock(512, 8, 1408, 2, use_gated_attention=True)
+    f.reset_parameters()
+    f = f.to(dev).to(dt)
+    a = DecoderBlock(512, 8, 1408, 2, use_gated_attention=True).to(dev).to(dt)
+    b = DecoderBlock(512, 8, 1408, 2, use_gated_attention=True).to(dev).to(dt)
+    a.load_state_dict(f.state_dict()), b.load_state_dict(f.state_dict())
+    quantize_model(a), quantize_model(b)
+    assert isinstance(a.attention.gate, QuantLinear)
+    fuse_shared_inputs(b, norms=True, decode_attention=True, residuals=True)
+    assert b.attention._decode_attention
+    B, S, page = 3, 300, 32
+    P = (S + 4 + page - 1) // page
+    tab = rotary_table(64, 512, device=dev)
+    table = torch.randperm(B * P, device=dev).view(B, P)
+    cf, ca, cb = (PagedKV(B * P, page, 2, 64, dev, dt) for _ in range(3))
+    x = torch.randn(B, S + 2, 512, device=dev).to(dt)
+    rel = lambda u, w: ((u.float() - w.float()).norm() / w.float().norm()).item()
+    with torch.inference_mode():
+        pf = f(x[:, :S], _freqs(tab, B, 0, S), None, cf.bind(table, S))
+        pa = a(x[:, :S], _freqs(tab, B, 0, S), None, ca.bind(table, S))
+        pb = b(x[:, :S], _freqs(tab, B, 0, S), None, cb.bind(table, S))
+        assert rel(pa, pf) < 3e-2 and rel(pb, pa) < 1e-2
+        for t in range(2):
+            pos = S + t
+            mask = decode_mask(B, pos + 1, dev, dt)
+            ya = a(x[:, pos:pos + 1], _freqs(tab, B, pos, 1), mask, ca.bind(table, pos + 1))
+            yb = b(x[:, pos:pos + 1], _freqs(tab, B, pos, 1), mask, cb.bind(table, pos + 1))
+            assert rel(yb, ya) < 1e-2, (t, rel(yb, ya))

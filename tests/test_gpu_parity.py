@@ -485,6 +485,41 @@ def test_quant_linear_module_shapes_dispatch_and_state_dict(oracle):
         q(torch.randn(4, 256, device=DEV, requires_grad=True))
 
 
+def test_called_from_a_daemon_thread_on_a_side_stream():
+    """How the reference's serving loop calls Linear (a daemon thread under inference_mode,
+    scheduler.py:191-196, executor.py:48,81): the work must go to that thread's current stream and
+    give the bits of a main-thread call; two threads on two streams share one module."""
+    import threading
+
+    torch.manual_seed(2)
+    lin = Linear(512, 320, bias=True)
+    lin.reset_parameters()
+    q = QuantLinear.from_linear(lin.to(DEV))
+    xs = [torch.randn(m, 512, device=DEV, dtype=torch.bfloat16) for m in (4, 100)]   # decode and prefill paths
+    with torch.inference_mode():
+        want = [q(x) for x in xs]
+    torch.cuda.synchronize()
+    got, errs = {}, []
+
+    def worker(name):
+        try:
+            s = torch.cuda.Stream()
+            with torch.inference_mode(), torch.cuda.stream(s):
+                for _ in range(20):
+                    ys = [q(x) for x in xs]
+                s.synchronize()  # the launches went to this thread's stream: waiting for it alone is enough
+                got[name] = [y.clone() for y in ys]
+        except Exception as e:  # surfaced in the main thread
+            errs.append(e)
+
+    ts = [threading.Thread(target=worker, args=(i,), daemon=True) for i in range(2)]
+    [t.start() for t in ts]
+    [t.join(60) for t in ts]
+    assert not errs, errs
+    for i in range(2):
+        assert torch.equal(got[i][0], want[0]) and torch.equal(got[i][1], want[1])
+
+
 def test_quantize_model_on_gpu_preserves_outputs_within_quantisation_error():
     import torch.nn as nn
 

@@ -138,7 +138,7 @@ __device__ __forceinline__ void sched_pattern() {
 }
 
 template <bool FP8, int OUT, int WM, int TM, int WK>
-__global__ __launch_bounds__(NTHREADS) void gemm_kernel(GemmArgs p) {
+__device__ __forceinline__ void gemm_tile(const GemmArgs& p, uint8_t* smem, int pid) {
   static_assert(WM * WAVES_N * WK == NWAVES, "8 wavefronts per workgroup");
   static_assert(TM % WK == 0, "the K-split pair divides the sub-tile's row blocks");
   constexpr int WAVE_M = 32 * TM;
@@ -154,7 +154,6 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(GemmArgs p) {
   // line) and a 16-byte-per-lane read is served 16 lanes at a time, so 16
   // consecutive rows reading the same piece must land on 16 distinct slots.
   constexpr int STAGE = (BM + BN) * BK;
-  __shared__ __attribute__((aligned(1024))) uint8_t smem[NSTAGE * STAGE];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -163,7 +162,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(GemmArgs p) {
   const int wave_m = wave_mn / WAVES_N, wave_n = wave_mn % WAVES_N;
 
   int tile_m, tile_n;
-  tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
+  tile_of_block(pid, p.tiles_m, p.tiles_n, tile_m, tile_n);
   const int m0 = tile_m * BM, n0 = tile_n * BN;
   const int M = p.M, N = p.N, K = p.K;
 
@@ -610,6 +609,20 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(GemmArgs p) {
     store_all(yes{}, no{});
 }
 
+// A workgroup walks tiles pid, pid + gridDim.x, ...: with more tiles than compute units the launch is one
+// resident workgroup per compute unit instead of a queue of short-lived ones (the LDS stages allow one at a time).
+template <bool FP8, int OUT, int WM, int TM, int WK>
+__global__ __launch_bounds__(NTHREADS) void gemm_kernel(GemmArgs p) {
+  constexpr int BM = WM * 32 * TM;
+  constexpr int NSTAGE = BM == 256 ? 3 : 4;
+  __shared__ __attribute__((aligned(1024))) uint8_t smem[NSTAGE * (BM + BN) * BK];
+  const int nt = p.tiles_m * p.tiles_n;
+  for (int pid = blockIdx.x; pid < nt; pid += gridDim.x) {
+    gemm_tile<FP8, OUT, WM, TM, WK>(p, smem, pid);
+    if (pid + (int)gridDim.x < nt) __syncthreads();  // every wavefront is done with the stages before they are refilled
+  }
+}
+
 // 256-row tiles unless they leave much of the device idle: a workgroup per compute unit at a
 // time, so the cost of a launch is its number of rounds over the 256 compute units.  Measured:
 // a round of 128-row tiles costs 0.72 of a round of 256-row ones, and a last round that fills
@@ -634,7 +647,10 @@ static int launch(GemmArgs& a, hipStream_t st) {
   const int bm = small ? 128 : 256;
   a.tiles_m = (a.M + bm - 1) / bm;
   a.tiles_n = (a.N + BN - 1) / BN;
-  const unsigned grid = (unsigned)(a.tiles_m * a.tiles_n);
+  // one resident workgroup per compute unit walks the tiles (a workgroup's LDS stages fill a compute unit):
+  // 3-5 % faster than queueing a workgroup per tile once there are more tiles than compute units
+  const int64_t ntiles = (int64_t)a.tiles_m * a.tiles_n;
+  const unsigned grid = (unsigned)(ntiles < 256 ? ntiles : 256);
   if (small)
     hipLaunchKernelGGL((gemm_kernel<FP8, OUT, 2, 2, 2>), dim3(grid), dim3(NTHREADS), 0, st, a);
   else

@@ -272,6 +272,22 @@ int aq_prefill_attn_causal(const void *q, int64_t q_stride, const void *k, int64
                            const void *v, int64_t v_stride, void *out, float scale, int64_t B,
                            int64_t S, int64_t Hq, int64_t Hkv, int64_t D, void *stream);
 
+/* The same attention for a chunk of S new tokens on top of `start` cached ones (a
+ * prompt whose prefix was found in the cache, executor.py:32-57 with start_pos > 0):
+ * query s of sequence b sits at position start + s and attends to positions
+ * 0 .. start + s.  Keys and values of ALL start + S positions are read in place
+ * through page_table [B, P] from k_cache / v_cache [n_pages, page_size, Hkv, D] --
+ * the new tokens' rows must have been written first (aq_rope_kv_write) -- which
+ * replaces Storage.gather (cache.py:254-274) + repeat_kv + scaled_dot_product_attention
+ * with the explicit position mask of transformer.py:17-46 when no token is padding.
+ * Positions whose page is unmapped count as zero keys and values (gather's zero
+ * fill).  start = 0 gives aq_prefill_attn_causal's result on cached rows.
+ * start + S <= P * page_size. */
+int aq_prefill_attn_paged(const void *q, int64_t q_stride, const void *k_cache, const void *v_cache,
+                          const int64_t *page_table, int64_t P, int64_t start, int64_t page_size,
+                          int64_t n_pages, void *out, float scale, int64_t B, int64_t S, int64_t Hq,
+                          int64_t Hkv, int64_t D, void *stream);
+
 /* Tuning and test hook, no counterpart in the reference: the GEMM entry points
  * pick their workgroup tile (256 x 128, or 128 x 128 with a split K step when
  * the larger one would leave compute units idle) from M and N.  rows = 128 or

@@ -48,6 +48,8 @@ SYMBOLS = {
     "aq_rope_paged_attn_decode_partials": (_int, [_vp, _vp, _i64, _vp, _i64, _i64, _i64, _vp, _vp, _i64, ctypes.c_float,
                                                   _i64, _i64, _i64, _i64, _vp, _i64, _vp]),
     "aq_gemv_w8a8_decode_attn": (_int, [_vp, _i64, _i64, _vp, _vp, _vp, _int, _vp, _vp, _int, _i64, _i64, _i64, _vp]),
+    "aq_prefill_attn_paged": (_int, [_vp, _i64, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, ctypes.c_float, _i64, _i64, _i64,
+                                     _i64, _i64, _vp]),
     "aq_probe_mfma": (_int, [_int, _int, _int, _vp, _vp]),
     "aq_probe_copy": (_int, [_vp, _vp, _i64, _int, _vp]),
     "aq_probe_read": (_int, [_vp, _i64, _int, _vp, _vp]),

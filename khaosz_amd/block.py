@@ -277,21 +277,29 @@ class GQA(nn.Module):
             return self._out(self._gated(out.view(B, 1, -1), x, norm, codes), residual)
         if (self._decode_attention and isinstance(cache, PagedKV) and x.is_cuda and x.dtype == torch.bfloat16
                 and S <= cache.total_len):
-            # several new tokens (prefill): rotation and the page writes as one launch; a prompt on an empty
-            # cache then runs the causal attention kernel, anything else the stock attention
+            # several new tokens (prefill): rotation and the page writes as one launch.  Without a mask tensor the
+            # attention is causal by position: a prompt on an empty, fully mapped cache runs the kernel that
+            # reads the new keys and values directly (v in place from qkv); a chunk on top of cached tokens,
+            # or a table with unmapped pages, the one that reads everything through the page table.  A mask
+            # tensor (padding) goes to the stock attention.
             nq, nkv = self.n_heads * self.head_dim, self.n_kv_heads * self.head_dim
             qkv = self._project_qkv(x, codes, norm)
             start = cache.total_len - S
-            q, k = ops.rope_kv_write(qkv, rotary_emb, cache.page_table, start, cache.k_layers[self.layer_id],
-                                     cache.v_layers[self.layer_id], self.n_heads, self.n_kv_heads, return_k=True)
-            if start == 0 and cache.all_mapped:
+            direct = start == 0 and cache.all_mapped
+            kc, vc = cache.k_layers[self.layer_id], cache.v_layers[self.layer_id]
+            if attn_mask is None and not direct:
+                q = ops.rope_kv_write(qkv, rotary_emb, cache.page_table, start, kc, vc, self.n_heads, self.n_kv_heads)
+                out = ops.prefill_attn_paged(q, kc, vc, cache.page_table, start)
+                return self._out(self._gated(out.view(B, S, -1), x, norm, codes), residual)
+            q, k = ops.rope_kv_write(qkv, rotary_emb, cache.page_table, start, kc, vc, self.n_heads, self.n_kv_heads,
+                                     return_k=True)
+            if direct:
                 v = qkv[..., nq + nkv:].view(B, S, self.n_kv_heads, self.head_dim)
-                if attn_mask is None:  # a prompt attending to itself: the causal kernel, v read in place from qkv
+                if attn_mask is None:
                     return self._out(self._gated(ops.prefill_attn_causal(q, k, v).view(B, S, -1), x, norm, codes), residual)
             else:
                 k, v = cache.gather(self.layer_id)
             out = F.scaled_dot_product_attention(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), attn_mask,
-                                                 is_causal=attn_mask is None,
                                                  enable_gqa=self.n_heads != self.n_kv_heads)
             return self._out(self._gated(out.transpose(1, 2).reshape(B, S, -1), x, norm, codes), residual)
         if self._qkv is not None:

@@ -38,6 +38,13 @@ struct PrefillAttnArgs {
   int64_t q_stride, k_stride, v_stride;  // elements between consecutive tokens
   float scale_log2e;
   int S, Hq, Hkv, B;
+  // PAGED kernels: keys and values of positions 0 .. start + S - 1 are read through the page table from
+  // caches [n_pages, page, Hkv, D]; query s sits at position start + s
+  const uint16_t* kc;
+  const uint16_t* vc;
+  const int64_t* table;  // [B, P] physical page ids, < 0: unmapped (zero keys and values)
+  int64_t P, page, n_pages;
+  int start, page_shift;
 };
 
 typedef __bf16 pa_bf16x8 __attribute__((ext_vector_type(8)));
@@ -48,7 +55,9 @@ constexpr int PA_KB = 64;   // keys per block
 
 // Two workgroups per compute unit (2 wavefronts per SIMD, at most 256 registers each): the other workgroup's
 // matrix work is what overlaps this one's softmax and staging.
-template <int D>
+// PAGED: a chunk of S new tokens on top of `start` cached ones -- K and V of all start + S positions come from the
+// paged cache (the new tokens' rows have been written there already), causality is by position.
+template <int D, bool PAGED = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void prefill_attn_kernel(PrefillAttnArgs p) {
   constexpr int KP = D + 8;       // K tile row pitch (elements): 16-byte reads of 32 rows hit distinct banks
   constexpr int VP = PA_KB + 4;   // V^T tile row pitch
@@ -73,6 +82,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
   const int qw0 = q0 + wave * 32;          // first query row of this wavefront
   const int qpos = qw0 + col;              // this lane's query
   const int64_t tok0 = (int64_t)b * S;
+  const int off = PAGED ? p.start : 0;     // position of query 0
+  const int T = off + S;                   // key positions
+  const int qw0p = qw0 + off, qposp = qpos + off;  // positions of the wavefront's first / this lane's query
 
   // Q^T operand: lane = (query col, dimensions 16 step + 8 g .. + 8); rows past S read row S - 1
   uint4 qf[DSTEPS];
@@ -89,25 +101,67 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
   // (scalars, not arrays: the compiler kept a 4-element array of these in scratch memory)
   uint4 kreg0, kreg1, kreg2, kreg3, vreg0, vreg1, vreg2, vreg3;
   kreg2 = kreg3 = vreg2 = vreg3 = make_uint4(0, 0, 0, 0);
+  // element offset of position t's row for this KV head in the paged caches, -1 when its page is unmapped
+  uint32_t kneg = 0, vneg = 0;  // bit c: the row of staging chunk c is not there
+  const int pshift = PAGED ? p.page_shift : 0;  // log2 of the page size, or -1 when it is not a power of two
+  auto paged_row = [&](int t) -> int64_t {
+    const int lp = pshift >= 0 ? t >> pshift : t / (int)p.page;
+    const int in_page = pshift >= 0 ? t & ((1 << pshift) - 1) : t - lp * (int)p.page;
+    const int64_t phys = p.table[(int64_t)b * p.P + lp];
+    return (phys >= 0 && phys < p.n_pages) ? ((phys * p.page + in_page) * p.Hkv + kvh) * D : -1;
+  };
+  int64_t kro0 = -1, kro1 = -1, kro2 = -1, kro3 = -1, vro = -1;  // row offsets of the block fetched next
+  auto lookup = [&](int j) __attribute__((always_inline)) {
+    if constexpr (PAGED) {
+      auto krow_of = [&](int c) -> int64_t {
+        int kr = j * PA_KB + (c * 256 + tid) / (D / 8);
+        return paged_row(kr < T ? kr : T - 1);
+      };
+      kro0 = krow_of(0);
+      kro1 = krow_of(1);
+      if constexpr (CPT > 2) {
+        kro2 = krow_of(2);
+        kro3 = krow_of(3);
+      }
+      const int vr = j * PA_KB + lane;
+      vro = paged_row(vr < T ? vr : T - 1);
+    }
+  };
   auto fetch1 = [&](int j, int c, uint4& kr_out, uint4& vr_out) __attribute__((always_inline)) {
     const int idx = c * 256 + tid, key = idx / (D / 8), ch = idx % (D / 8);
     int kr = j * PA_KB + key;
-    kr = kr < S ? kr : S - 1;  // past the prompt: any valid row, masked by causality
-    kr_out = *reinterpret_cast<const uint4*>(p.k + (tok0 + kr) * p.k_stride + (int64_t)kvh * D + ch * 8);
+    kr = kr < T ? kr : T - 1;  // past the last position: any valid row, masked by causality
     int vr = j * PA_KB + lane;
-    vr = vr < S ? vr : S - 1;
-    vr_out = *reinterpret_cast<const uint4*>(p.v + (tok0 + vr) * p.v_stride + (int64_t)kvh * D + (wave + 4 * c) * 8);
+    vr = vr < T ? vr : T - 1;
+    if constexpr (PAGED) {
+      // the rows' offsets were looked up one block earlier (lookup below): the page-table round trip is off
+      // the prefetch's path.  Rows of unmapped pages read row 0 and are zeroed when they are staged: a
+      // select on the loaded value here would make every load of the prefetch wait for the one before it.
+      const int64_t krow = c == 0 ? kro0 : c == 1 ? kro1 : c == 2 ? kro2 : kro3, vrow = vro;
+      kr_out = *reinterpret_cast<const uint4*>(p.kc + (krow >= 0 ? krow : 0) + ch * 8);
+      vr_out = *reinterpret_cast<const uint4*>(p.vc + (vrow >= 0 ? vrow : 0) + (wave + 4 * c) * 8);
+      kneg = (kneg & ~(1u << c)) | ((krow < 0 ? 1u : 0u) << c);
+      vneg = (vneg & ~(1u << c)) | ((vrow < 0 ? 1u : 0u) << c);
+    } else {
+      kr_out = *reinterpret_cast<const uint4*>(p.k + (tok0 + kr) * p.k_stride + (int64_t)kvh * D + ch * 8);
+      vr_out = *reinterpret_cast<const uint4*>(p.v + (tok0 + vr) * p.v_stride + (int64_t)kvh * D + (wave + 4 * c) * 8);
+    }
   };
   auto stage1 = [&](uint16_t* ks, uint16_t* vt, int c, const uint4& kr_in, const uint4& vr_in) __attribute__((always_inline)) {
     const int idx = c * 256 + tid, key = idx / (D / 8), ch = idx % (D / 8);
-    *reinterpret_cast<uint4*>(&ks[key * KP + ch * 8]) = kr_in;
+    uint4 kr_z = kr_in, vr_z = vr_in;
+    if constexpr (PAGED) {
+      if (kneg & (1u << c)) kr_z = make_uint4(0, 0, 0, 0);
+      if (vneg & (1u << c)) vr_z = make_uint4(0, 0, 0, 0);
+    }
+    *reinterpret_cast<uint4*>(&ks[key * KP + ch * 8]) = kr_z;
     // V chunk (key = lane, dimensions 8 (wave + 4 c) .. + 8) into the transposed tile, two keys per 4-byte
     // store: neighbouring lanes swap dwords (DPP) and byte-permute them into "one dimension, both keys" --
     // even lanes then hold the even dimensions of the key pair, odd lanes the odd ones.
     const bool odd = lane & 1;
     const uint32_t sel = odd ? 0x03020706u : 0x05040100u;
     uint32_t* vdst = reinterpret_cast<uint32_t*>(&vt[((wave + 4 * c) * 8 + (odd ? 1 : 0)) * VP + (lane & ~1)]);
-    const uint32_t w[4] = {vr_in.x, vr_in.y, vr_in.z, vr_in.w};
+    const uint32_t w[4] = {vr_z.x, vr_z.y, vr_z.z, vr_z.w};
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const uint32_t other = (uint32_t)__builtin_amdgcn_mov_dpp((int)w[e], 0xB1 /* quad_perm [1,0,3,2] */, 0xf, 0xf, true);
@@ -141,22 +195,25 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
     for (int r = 0; r < 16; ++r) o[dt][r] = 0.0f;
   float m = -INFINITY, l = 0.0f;  // running maximum of this lane's query; this lane's half of its denominator
 
-  const int last_q = (q0 + PA_QB < S ? q0 + PA_QB : S) - 1;
+  const int last_q = (q0 + PA_QB < S ? q0 + PA_QB : S) - 1 + off;  // position of the workgroup's last query
   const int nblk = last_q / PA_KB + 1;  // blocks that hold a key some query of the workgroup may see
   // One LDS buffer, two barriers per block; the next block's global loads are in flight while this one is
   // multiplied.  (Two buffers with one barrier per block measured 15 % slower.)
   const uint16_t* ks = pa_lds;
   const uint16_t* vt = pa_lds + KS_ELEMS;
+  lookup(0);
   PA_FETCH(0)
+  if (nblk > 1) lookup(1);
   for (int j = 0; j < nblk; ++j) {
     __syncthreads();  // everyone is done reading the previous block's tiles
     PA_STAGE(0)
     __syncthreads();
     if (j + 1 < nblk) {
       PA_FETCH(j + 1)
+      if (j + 2 < nblk) lookup(j + 2);
     }
     const int kb0 = j * PA_KB;
-    if (kb0 > qw0 + 31) continue;  // wavefront-uniform: every key of the block is ahead of every query here
+    if (kb0 > qw0p + 31) continue;  // wavefront-uniform: every key of the block is ahead of every query here
     // ---- scores, transposed: two tiles of 32 keys
     pa_f32x16 s[2];
 #pragma unroll
@@ -175,13 +232,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
     }
     // ---- online softmax for this lane's query; register r of tile kt is key kb0 + 32 kt + 8 (r / 4) + 4 g + r % 4.
     // Scores stay unscaled; the scale (> 0) is applied to the maximum and inside the exponent's fma.
-    const bool diag = kb0 + PA_KB - 1 > qw0;  // wavefront-uniform: some key of the block is ahead of some query
+    const bool diag = kb0 + PA_KB - 1 > qw0p;  // wavefront-uniform: some key of the block is ahead of some query
     float bm = -INFINITY;
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        if (diag && kb0 + kt * 32 + 8 * (r / 4) + 4 * g + (r % 4) > qpos) s[kt][r] = -INFINITY;
+        if (diag && kb0 + kt * 32 + 8 * (r / 4) + 4 * g + (r % 4) > qposp) s[kt][r] = -INFINITY;
         bm = fmaxf(bm, s[kt][r]);
       }
     bm = fmaxf(bm, __shfl_xor(bm, 32, 64)) * p.scale_log2e;
@@ -288,8 +345,54 @@ extern "C" int aq_prefill_attn_causal(const void* q, int64_t q_stride, const voi
   hipStream_t st = static_cast<hipStream_t>(stream);
   const size_t lds = (size_t)(aq::PA_KB * (D + 8) + D * (aq::PA_KB + 4)) * sizeof(uint16_t);  // 34 KiB at most
   if (D == 128)
-    hipLaunchKernelGGL(aq::prefill_attn_kernel<128>, grid, dim3(256), lds, st, a);
+    hipLaunchKernelGGL((aq::prefill_attn_kernel<128, false>), grid, dim3(256), lds, st, a);
   else
-    hipLaunchKernelGGL(aq::prefill_attn_kernel<64>, grid, dim3(256), lds, st, a);
+    hipLaunchKernelGGL((aq::prefill_attn_kernel<64, false>), grid, dim3(256), lds, st, a);
+  return (int)hipGetLastError();
+}
+
+extern "C" int aq_prefill_attn_paged(const void* q, int64_t q_stride, const void* k_cache, const void* v_cache,
+                                     const int64_t* page_table, int64_t P, int64_t start, int64_t page_size,
+                                     int64_t n_pages, void* out, float scale, int64_t B, int64_t S, int64_t Hq,
+                                     int64_t Hkv, int64_t D, void* stream) {
+  if (D != 64 && D != 128) return AQ_E_SHAPE;
+  if (B < 0 || S < 0 || start < 0 || Hq <= 0 || Hkv <= 0 || (Hq % Hkv) != 0 || P <= 0 || page_size <= 0 ||
+      n_pages <= 0 || !(scale > 0.0f) || q_stride < Hq * D)
+    return AQ_E_SHAPE;
+  if (start + S > P * page_size) return AQ_E_SHAPE;  // positions the page table does not cover
+  if (B == 0 || S == 0) return AQ_OK;
+  if (!q || !k_cache || !v_cache || !page_table || !out) return AQ_E_NULL;
+  if (aq::check_ptr16(q) || aq::check_ptr16(k_cache) || aq::check_ptr16(v_cache) || aq::check_ptr16(out) ||
+      (q_stride & 7))
+    return AQ_E_ALIGN;
+  if (start + S > (1 << 30) || Hq > 65535 || B > 65535 ||
+      ((S + aq::PA_QB - 1) / aq::PA_QB) * Hq * B > (int64_t)0x7fffffff)
+    return AQ_E_RANGE;
+  aq::PrefillAttnArgs a{};
+  a.q = static_cast<const uint16_t*>(q);
+  a.out = static_cast<uint16_t*>(out);
+  a.q_stride = q_stride;
+  a.kc = static_cast<const uint16_t*>(k_cache);
+  a.vc = static_cast<const uint16_t*>(v_cache);
+  a.table = page_table;
+  a.P = P;
+  a.page = page_size;
+  a.n_pages = n_pages;
+  a.start = (int)start;
+  a.page_shift = -1;
+  for (int sh = 0; sh < 31; ++sh)
+    if (page_size == ((int64_t)1 << sh)) a.page_shift = sh;
+  a.scale_log2e = scale * 1.44269504088896341f;
+  a.S = (int)S;
+  a.Hq = (int)Hq;
+  a.Hkv = (int)Hkv;
+  a.B = (int)B;
+  const dim3 grid((unsigned)(((S + aq::PA_QB - 1) / aq::PA_QB) * Hq * B));
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const size_t lds = (size_t)(aq::PA_KB * (D + 8) + D * (aq::PA_KB + 4)) * sizeof(uint16_t);
+  if (D == 128)
+    hipLaunchKernelGGL((aq::prefill_attn_kernel<128, true>), grid, dim3(256), lds, st, a);
+  else
+    hipLaunchKernelGGL((aq::prefill_attn_kernel<64, true>), grid, dim3(256), lds, st, a);
   return (int)hipGetLastError();
 }

@@ -113,9 +113,11 @@ class AutoRegressiveLM(nn.Module):
             # a prompt from position 0 is causal without a mask tensor; later tokens attend to all
             # cached positions and causally among themselves
             mask = None
-            fused_step = (S == 1 and paged_cache is not None
+            # with the paged-cache kernels in every layer neither a single-token step nor a chunk on top of
+            # cached tokens takes a mask tensor: causality is by position inside the kernels
+            fused_step = (isinstance(paged_cache, PagedKV) and x.is_cuda and x.dtype == torch.bfloat16
                           and all(getattr(layer.attention, "_decode_attention", False) for layer in self.layers))
-            if start_pos > 0 and not fused_step:  # the fused single-token step takes no mask
+            if start_pos > 0 and not fused_step:
                 T = start_pos + S
                 mask = torch.zeros((B, 1, S, T), device=x.device, dtype=x.dtype)
                 if S > 1:

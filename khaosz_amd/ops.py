@@ -517,6 +517,42 @@ def prefill_attn_causal(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale
     return out
 
 
+def prefill_attn_paged(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, page_table: torch.Tensor,
+                       start: int, scale: Optional[float] = None) -> torch.Tensor:
+    """Attention of ``S`` new tokens at positions ``start .. start + S`` over everything cached:
+    ``q [B, S, Hq, D]`` against positions ``0 .. start + s`` of ``k_cache`` / ``v_cache
+    [n_pages, page, Hkv, D]`` read through ``page_table [B, P]`` in place (the new tokens' rows
+    written beforehand, ``rope_kv_write``) -> ``[B, S, Hq, D]``.  Unmapped pages are zero keys and
+    values.  bfloat16, D = 64 or 128."""
+    _need_gpu(q, k_cache, v_cache, page_table)
+    if q.dtype != torch.bfloat16 or k_cache.dtype != torch.bfloat16 or v_cache.dtype != torch.bfloat16:
+        raise ValueError("prefill_attn_paged takes bfloat16 tensors")
+    if q.dim() != 4 or k_cache.dim() != 4 or k_cache.shape != v_cache.shape or q.shape[3] != k_cache.shape[3]:
+        raise ValueError("q must be [B, S, Hq, D] and the caches [n_pages, page, Hkv, D]")
+    if page_table.dtype != torch.int64 or page_table.dim() != 2 or page_table.shape[0] != q.shape[0]:
+        raise ValueError("page_table must be int64 [B, P]")
+    B, S, Hq, D = q.shape
+    n_pages, page, Hkv, _ = k_cache.shape
+    if start < 0 or start + S > page_table.shape[1] * page:
+        raise ValueError(f"positions {start} .. {start + S} fall outside the page table")
+    if not (k_cache.is_contiguous() and v_cache.is_contiguous()):
+        raise ValueError("the caches must be contiguous")
+    page_table = page_table.contiguous()
+    if not (q.stride(3) == 1 and q.stride(2) == D and q.stride(0) == S * q.stride(1) and q.stride(1) % 8 == 0
+            and q.data_ptr() % 16 == 0):
+        q = q.contiguous()
+    out = torch.empty((B, S, Hq, D), dtype=torch.bfloat16, device=q.device)
+    if B and S:
+        with _OnDevice(q.device):
+            rc = _abi.load().aq_prefill_attn_paged(q.data_ptr(), q.stride(1), k_cache.data_ptr(), v_cache.data_ptr(),
+                                                   page_table.data_ptr(), page_table.shape[1], int(start), page,
+                                                   n_pages, out.data_ptr(),
+                                                   float(scale if scale is not None else D ** -0.5), B, S, Hq, Hkv, D,
+                                                   _stream(q))
+        _abi.check(rc, "aq_prefill_attn_paged")
+    return out
+
+
 def paged_attn_workspace_bytes(B: int, n_heads: int, n_kv_heads: int, total_len: int) -> int:
     """Bytes of device workspace ``paged_attn_decode`` needs for this shape (0: none)."""
     return int(_abi.load().aq_paged_attn_decode_workspace_bytes(B, n_heads, n_kv_heads, int(total_len)))

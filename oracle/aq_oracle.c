@@ -61,6 +61,10 @@
  *                         (enable_gqa and explicit repeats) within rounding, and on
  *                         closed forms (first position = its own value row; equal keys
  *                         = running mean of the values).
+ *   oq_prefill_attn_offset the same with the queries at positions start .. start + S over
+ *                         start + S keys; start = 0 must reproduce oq_prefill_attn_causal
+ *                         bit for bit, and it is pinned against torch's attention with the
+ *                         explicit position mask.
  *
  * Build: gcc -O3 -march=native -fopenmp -ffp-contract=off -fno-fast-math
  *        -shared -fPIC (oracle/build_oracle.py).  OpenMP only parallelises over
@@ -428,6 +432,41 @@ void oq_prefill_attn_causal(const uint16_t *q, const uint16_t *k, const uint16_t
           const float pt = expf(sc[t] - m);
           l += pt;
           const uint16_t *vr = v + ((b * S + t) * Hkv + kvh) * D;
+          for (int64_t i = 0; i < D; ++i) acc[i] += pt * oq_bf16_to_f32(vr[i]);
+        }
+        for (int64_t i = 0; i < D; ++i) out[((b * S + s) * Hq + h) * D + i] = oq_f32_to_bf16(acc[i] / l);
+        free(sc);
+        free(acc);
+      }
+}
+
+/* The same with the S queries at positions start .. start + S over T = start + S keys: query s attends to
+ * t <= start + s (the explicit position mask of transformer.py:17-46 for a chunk on top of cached tokens,
+ * executor.py:32-57 with start_pos > 0).  q: [B, S, Hq, D], k, v: [B, T, Hkv, D]. */
+void oq_prefill_attn_offset(const uint16_t *q, const uint16_t *k, const uint16_t *v, float scale, uint16_t *out,
+                            int64_t B, int64_t S, int64_t start, int64_t Hq, int64_t Hkv, int64_t D) {
+  const int64_t G = Hq / Hkv, T = start + S;
+#pragma omp parallel for schedule(dynamic) collapse(3)
+  for (int64_t b = 0; b < B; ++b)
+    for (int64_t h = 0; h < Hq; ++h)
+      for (int64_t s = 0; s < S; ++s) {
+        const int64_t kvh = h / G, last = start + s;
+        const uint16_t *qr = q + ((b * S + s) * Hq + h) * D;
+        float *sc = (float *)malloc((size_t)(last + 1) * sizeof(float));
+        float *acc = (float *)calloc((size_t)D, sizeof(float));
+        float m = -INFINITY;
+        for (int64_t t = 0; t <= last; ++t) {
+          const uint16_t *kr = k + ((b * T + t) * Hkv + kvh) * D;
+          float d = 0.0f;
+          for (int64_t i = 0; i < D; ++i) d += oq_bf16_to_f32(qr[i]) * oq_bf16_to_f32(kr[i]);
+          sc[t] = d * scale;
+          if (sc[t] > m) m = sc[t];
+        }
+        float l = 0.0f;
+        for (int64_t t = 0; t <= last; ++t) {
+          const float pt = expf(sc[t] - m);
+          l += pt;
+          const uint16_t *vr = v + ((b * T + t) * Hkv + kvh) * D;
           for (int64_t i = 0; i < D; ++i) acc[i] += pt * oq_bf16_to_f32(vr[i]);
         }
         for (int64_t i = 0; i < D; ++i) out[((b * S + s) * Hq + h) * D + i] = oq_f32_to_bf16(acc[i] / l);

@@ -230,6 +230,7 @@ def _load():
     lib.oq_rope_kv_write.argtypes = [vp, vp, vp, i64, i64, i64, vp, vp, i64, vp, i64, i64, i64, i64]
     lib.oq_paged_attn_decode.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, ctypes.c_float, vp, i64, i64, i64, i64]
     lib.oq_prefill_attn_causal.argtypes = [vp, vp, vp, ctypes.c_float, vp, i64, i64, i64, i64, i64]
+    lib.oq_prefill_attn_offset.argtypes = [vp, vp, vp, ctypes.c_float, vp, i64, i64, i64, i64, i64, i64]
     lib.oq_gemm_i8_i32.argtypes = [vp, vp, vp, i64, i64, i64]
     lib.oq_dequant_epilogue.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64]
     lib.oq_linear_w8a8_f32.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i64]
@@ -242,7 +243,8 @@ def _load():
         "oq_set_num_threads oq_quant_rowwise_i8_f32 oq_quant_rowwise_i8_bf16 oq_gemm_i8_i32 "
         "oq_dequant_epilogue oq_linear_w8a8_f32 oq_linear_w8a8_bf16 oq_quant_tensor_fp8_f32 "
         "oq_quant_tensor_fp8_bf16 oq_linear_fp8 oq_linear_f32 oq_rmsnorm_quant_i8_f32 oq_rmsnorm_quant_i8_bf16 "
-        "oq_swiglu_quant_i8_f32 oq_swiglu_quant_i8_bf16 oq_rope_kv_write oq_paged_attn_decode oq_prefill_attn_causal"
+        "oq_swiglu_quant_i8_f32 oq_swiglu_quant_i8_bf16 oq_rope_kv_write oq_paged_attn_decode oq_prefill_attn_causal "
+        "oq_prefill_attn_offset"
     ).split():
         getattr(lib, name).restype = None
     _lib = lib
@@ -356,6 +358,18 @@ def c_prefill_attn_causal(q, k, v, scale):
     Hkv = k.shape[2]
     out = np.empty((B, S, Hq, D), np.uint16)
     lib.oq_prefill_attn_causal(_p(q), _p(k), _p(v), ctypes.c_float(scale), _p(out), B, S, Hq, Hkv, D)
+    return out
+
+
+def c_prefill_attn_offset(q, k, v, start, scale):
+    """q [B, S, Hq, D] at positions start .. start + S, k / v [B, start + S, Hkv, D] (uint16 bf16 patterns)
+    -> out [B, S, Hq, D] (uint16)."""
+    lib = _load()
+    q, k, v = _c(q, np.uint16), _c(k, np.uint16), _c(v, np.uint16)
+    B, S, Hq, D = q.shape
+    assert k.shape[1] == start + S and k.shape == v.shape
+    out = np.empty((B, S, Hq, D), np.uint16)
+    lib.oq_prefill_attn_offset(_p(q), _p(k), _p(v), ctypes.c_float(scale), _p(out), B, S, int(start), Hq, k.shape[2], D)
     return out
 
 

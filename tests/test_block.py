@@ -499,3 +499,50 @@ def test_gated_attention_block_quantized_and_fused_paths_agree():
             ya = a(x[:, pos:pos + 1], _freqs(tab, B, pos, 1), mask, ca.bind(table, pos + 1))
             yb = b(x[:, pos:pos + 1], _freqs(tab, B, pos, 1), mask, cb.bind(table, pos + 1))
             assert rel(yb, ya) < 1e-2, (t, rel(yb, ya))
+
+
+@pytest.mark.gpu
+def test_chunked_prefill_on_cached_tokens_uses_the_paged_kernel_and_tracks_the_masked_attention():
+    """A second chunk of a prompt on top of cached tokens (a prefix-cache hit, executor.py:32-57 with
+    start_pos > 0): the fused block reads K / V through the page table with causality by position; the
+    plain quantized block runs gather + the stock attention under the explicit mask.  Outputs agree
+    within bf16 rounding, the caches hold the same rows, and prefill in two chunks equals one pass."""
+    from khaosz_amd import fuse_shared_inputs, ops
+
+    dev, dt = "cuda:0", torch.bfloat16
+    torch.manual_seed(21)
+    a = DecoderBlock(512, 8, 1408, 2)
+    a.reset_parameters()
+    a = a.to(dev).to(dt)
+    b = DecoderBlock(512, 8, 1408, 2).to(dev).to(dt)
+    b.load_state_dict(a.state_dict())
+    quantize_model(a), quantize_model(b)
+    fuse_shared_inputs(a)
+    fuse_shared_inputs(b, norms=False, decode_attention=True)
+    B, S1, S2, page = 2, 150, 90, 32
+    T = S1 + S2
+    P = (T + page - 1) // page
+    tab = rotary_table(64, 512, device=dev)
+    table = torch.randperm(B * P, device=dev).view(B, P)
+    ca, cb, cc = (PagedKV(B * P, page, 2, 64, dev, dt) for _ in range(3))
+    x = torch.randn(B, T, 512, device=dev).to(dt)
+    mask = torch.zeros(B, 1, S2, T, device=dev, dtype=dt)
+    mask[:, :, :, S1:] = torch.full((S2, S2), float("-inf"), device=dev, dtype=dt).triu(1)
+    rel = lambda u, w: ((u.float() - w.float()).norm() / w.float().norm()).item()
+    calls = []
+    real = ops.prefill_attn_paged
+    ops.prefill_attn_paged = lambda *args, **kw: (calls.append(1), real(*args, **kw))[1]
+    try:
+        with torch.inference_mode():
+            a(x[:, :S1], _freqs(tab, B, 0, S1), None, ca.bind(table, S1))
+            b(x[:, :S1], _freqs(tab, B, 0, S1), None, cb.bind(table, S1))
+            assert not calls                                       # an empty cache: the direct kernel
+            ya = a(x[:, S1:], _freqs(tab, B, S1, S2), mask, ca.bind(table, T))
+            yb = b(x[:, S1:], _freqs(tab, B, S1, S2), None, cb.bind(table, T))
+            assert len(calls) == 1
+            assert rel(yb, ya) < 1e-2
+            assert torch.allclose(ca.k.float(), cb.k.float(), rtol=1e-2, atol=1e-2) and torch.equal(ca.v, cb.v)
+            one = b(x, _freqs(tab, B, 0, T), None, cc.bind(table, T))
+            assert rel(yb, one[:, S1:]) < 1e-2
+    finally:
+        ops.prefill_attn_paged = real

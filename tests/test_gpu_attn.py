@@ -271,3 +271,57 @@ def test_attention_partials_entry_points_check_their_arguments():
     rc = lib.aq_paged_attn_decode_partials(q.data_ptr(), kc.data_ptr(), kc.data_ptr(), tb.data_ptr(), 1, 10, 16, 2, 0.125,
                                            1, 2, 1, 64, buf.data_ptr(), 64, None)
     assert rc == -5                         # AQ_E_WORKSPACE
+
+
+@pytest.mark.parametrize("B,S,start,Hq,Hkv,page", [(1, 1, 0, 1, 1, 4), (2, 37, 0, 6, 2, 16), (2, 40, 100, 8, 2, 16), (3, 130, 257, 4, 1, 64),
+                                                    (4, 200, 312, 24, 4, 128), (1, 300, 5, 4, 4, 32), (2, 64, 64, 3, 1, 8)])
+@pytest.mark.parametrize("D", [128, 64])
+def test_prefill_attn_paged_within_bf16_rounding(oracle, B, S, start, Hq, Hkv, page, D):
+    """A chunk of S new tokens over start cached ones, K / V read through the page table (one sequence
+    with an unmapped page: zero keys and values there), against the oracle on the gathered rows."""
+    _say("prefill_attn_paged", B, S, start, Hq, Hkv, page, D)
+    T = start + S
+    P = (T + page - 1) // page + 1
+    n_pages = B * P + 2
+    g = torch.Generator().manual_seed(S + start + D)
+    q = (torch.randn(B, S, Hq, D, generator=g) * 1.5).to(torch.bfloat16)
+    kc = torch.randn(n_pages, page, Hkv, D, generator=g).to(torch.bfloat16)
+    vc = torch.randn(n_pages, page, Hkv, D, generator=g).to(torch.bfloat16)
+    table = torch.randperm(n_pages, generator=g)[:B * P].view(B, P)
+    if B > 1 and T > page:
+        table[1, 0] = -1
+    # what gather gives: [B, T, Hkv, D], zeros where unmapped
+    idx = torch.arange(T)
+    rows = []
+    for b in range(B):
+        phys = table[b, idx // page]
+        kk, vv = kc[phys.clamp(min=0), idx % page], vc[phys.clamp(min=0), idx % page]
+        kk[phys < 0], vv[phys < 0] = 0, 0
+        rows.append((kk, vv))
+    k = torch.stack([r[0] for r in rows])
+    v = torch.stack([r[1] for r in rows])
+    want = torch.from_numpy(oracle.c_prefill_attn_offset(_bits(q), _bits(k), _bits(v), start, D ** -0.5)
+                            .view(np.int16)).view(torch.bfloat16).float()
+    out = ops.prefill_attn_paged(q.to(DEV), kc.to(DEV), vc.to(DEV), table.to(DEV), start).cpu().float()
+    assert torch.allclose(out, want, rtol=1e-2, atol=1e-2)      # stated tolerance for bf16 outputs
+    assert ((out - want).norm() / want.norm()).item() < 5e-3
+    if start == 0 and not (table < 0).any():                     # on an empty cache: the contiguous kernel's bits
+        same = ops.prefill_attn_causal(q.to(DEV), k.to(DEV), v.to(DEV)).cpu().float()
+        assert torch.equal(out, same)
+
+
+def test_prefill_attn_paged_checks_its_arguments():
+    from khaosz_amd import _abi
+    lib = _abi.load()
+    q = torch.zeros(1, 4, 2, 64, dtype=torch.bfloat16, device=DEV)
+    kc = torch.zeros(3, 16, 1, 64, dtype=torch.bfloat16, device=DEV)
+    tb = torch.zeros(1, 2, dtype=torch.int64, device=DEV)
+    out = torch.zeros_like(q)
+    call = lambda start, S, P=2, D=64: lib.aq_prefill_attn_paged(q.data_ptr(), 128, kc.data_ptr(), kc.data_ptr(), tb.data_ptr(),
+                                                                 P, start, 16, 3, out.data_ptr(), 0.125, 1, S, 2, 1, D, None)
+    assert call(0, 4) == 0
+    assert call(29, 4) == -2        # positions past the page table: AQ_E_SHAPE
+    assert call(-1, 4) == -2
+    assert call(0, 4, D=96) == -2
+    with pytest.raises(ValueError):
+        ops.prefill_attn_paged(q, kc, kc, tb, 30)

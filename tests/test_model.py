@@ -104,3 +104,38 @@ def test_quantized_fused_model_tracks_the_float_model_and_replays_in_a_graph():
                 g.replay()
                 torch.cuda.synchronize()
                 assert torch.equal(got, want)
+
+
+@pytest.mark.gpu
+def test_prompt_prefilled_in_two_chunks_matches_one_pass_on_the_quantized_fused_model():
+    """The second chunk starts on top of cached tokens (start_pos > 0, what a prefix-cache hit gives
+    the reference's executor): no mask tensor is built, the layers read the cache through the page
+    table.  Logits of the chunk agree with the one-pass prefill within bf16 rounding through the layers,
+    and the float model fed the same chunks (explicit mask, stock attention) stays within the
+    quantisation error."""
+    dev, dt = "cuda:0", torch.bfloat16
+    cfg = LMConfig(vocab_size=512, dim=768, n_layers=2, n_heads=12, n_kv_heads=2, dim_ffn=2048, max_len=640)
+    torch.manual_seed(4)
+    f = AutoRegressiveLM(cfg).to(dev).to(dt).eval()
+    q = AutoRegressiveLM(cfg).to(dev).to(dt).eval()
+    q.load_state_dict(f.state_dict())
+    quantize_model(q)
+    fuse_shared_inputs(q, norms=True, decode_attention=True, residuals=True)
+    B, S1, S2, page = 3, 200, 130, 64
+    T = S1 + S2
+    P = (T + page - 1) // page
+    ids = torch.randint(0, 512, (B, T), device=dev)
+    table = _table(B, P).to(dev)
+    c1, c2, cf = q.new_cache(B * P, page), q.new_cache(B * P, page), f.new_cache(B * P, page)
+
+    def rel(a, b):
+        return ((a.float() - b.float()).norm() / b.float().norm()).item()
+
+    with torch.inference_mode():
+        one = q(ids, paged_cache=c1.bind(table, T))["logits"]
+        q(ids[:, :S1], paged_cache=c2.bind(table, S1))
+        two = q(ids[:, S1:], paged_cache=c2.bind(table, T), start_pos=S1)["logits"]
+        assert rel(two, one[:, S1:]) < 2e-2
+        f(ids[:, :S1], paged_cache=cf.bind(table, S1))
+        ref = f(ids[:, S1:], paged_cache=cf.bind(table, T), start_pos=S1)["logits"]
+        assert rel(two, ref) < 6e-2

@@ -92,3 +92,27 @@ def test_prefill_attention_matches_torch_sdpa_and_closed_forms(oracle):
     out = _bf16(oracle.c_prefill_attn_causal(_bits(q), _bits(k), _bits(v), 0.125)).float()
     mean = v.float().cumsum(1) / torch.arange(1, S + 1).view(1, S, 1, 1)
     assert torch.allclose(out, mean.expand(B, S, Hq, D), rtol=1e-2, atol=1e-2)
+
+
+def test_prefill_attention_with_a_position_offset_matches_the_masked_torch_attention(oracle):
+    """A chunk of new tokens on top of cached ones: start = 0 is the causal oracle bit for bit; a
+    later chunk is the tail of the full causal result, and agrees with torch's attention under the
+    explicit position mask the reference builds (transformer.py:17-46)."""
+    for (B, S, start, Hq, Hkv, D) in [(2, 11, 0, 4, 2, 64), (2, 9, 30, 6, 2, 64), (1, 33, 70, 4, 4, 128), (2, 1, 17, 3, 1, 64)]:
+        g = torch.Generator().manual_seed(S + start)
+        T = start + S
+        qf = torch.randn(B, T, Hq, D, generator=g).to(torch.bfloat16)     # queries of every position
+        k = torch.randn(B, T, Hkv, D, generator=g).to(torch.bfloat16)
+        v = torch.randn(B, T, Hkv, D, generator=g).to(torch.bfloat16)
+        q = qf[:, start:].contiguous()
+        out = oracle.c_prefill_attn_offset(_bits(q), _bits(k), _bits(v), start, D ** -0.5)
+        full = oracle.c_prefill_attn_causal(_bits(qf), _bits(k), _bits(v), D ** -0.5)
+        assert np.array_equal(out, full[:, start:])                      # same arithmetic, same bits
+        rep = Hq // Hkv
+        pos = torch.arange(start, T)
+        mask = torch.zeros(S, T).masked_fill_(pos.view(S, 1) < torch.arange(T).view(1, T), float("-inf"))
+        want = F.scaled_dot_product_attention(q.float().transpose(1, 2), k.float().transpose(1, 2).repeat_interleave(rep, 1),
+                                              v.float().transpose(1, 2).repeat_interleave(rep, 1), mask).transpose(1, 2)
+        got = _bf16(out).float()
+        assert torch.allclose(got, want, rtol=1e-2, atol=1e-2)
+        assert ((got - want).norm() / want.norm()).item() < 4e-3

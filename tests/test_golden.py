@@ -93,3 +93,76 @@ def test_hip_reproduces_config1_hashes(config1):
     got = {"xq": sha(xq.cpu().numpy()), "sx": sha(sx.cpu().numpy()), "wq": sha(wq.cpu().numpy()),
            "sw": sha(sw.cpu().numpy()), "acc": sha(acc.cpu().numpy()), "y_f32": sha(y.cpu().numpy())}
     assert got == {k: want[k] for k in got}
+
+
+@pytest.fixture(scope="module")
+def fused():
+    return dict(np.load(os.path.join(G, "fused_small.npz")))
+
+
+def _bf16_close(a_bits, b_bits, ulps=2):
+    """bf16 bit patterns within a few units in the last place (libm's expf may differ between hosts)."""
+    a = torch.from_numpy(a_bits.view(np.int16).copy()).view(torch.bfloat16).float()
+    b = torch.from_numpy(b_bits.view(np.int16).copy()).view(torch.bfloat16).float()
+    return bool(((a - b).abs() <= ulps * 2.0 ** -8 * b.abs().clamp(min=2.0 ** -6)).all())
+
+
+def test_oracle_reproduces_fused_fixture(oracle, fused):
+    f = fused
+    q, s = oracle.c_rmsnorm_quant_i8(f["norm_x"], f["norm_gamma"], 1e-5, bf16_bits=True)
+    assert np.array_equal(q, f["norm_codes"]) and np.array_equal(s, f["norm_scale"])
+    q, s = oracle.c_swiglu_quant_i8(f["swiglu_ug"], bf16_bits=True)
+    assert np.array_equal(q, f["swiglu_codes"]) and np.array_equal(s, f["swiglu_scale"])
+    kc, vc = f["kc"].copy(), f["vc"].copy()
+    qr = oracle.c_rope_kv_write(f["rope_qkv"], f["rope_freqs"], f["table"], int(f["pos"]), kc, vc, 4, 2)
+    assert np.array_equal(qr, f["q_rot"]) and np.array_equal(kc, f["kc_after"]) and np.array_equal(vc, f["vc_after"])
+    # position 37 = slot 5 of logical page 2: pages 7 (sequence 0) and 4 (sequence 1) took the new rows, nothing else
+    changed = {(int(p), int(sl)) for p, sl in zip(*np.nonzero((kc != f["kc"]).any(axis=(2, 3))))}
+    assert changed == {(7, 5), (4, 5)}
+    out = oracle.c_paged_attn_decode(f["q_rot"], f["kc_after"], f["vc_after"], f["table"], int(f["pos"]) + 1, 0.125)
+    assert _bf16_close(out, f["attn_decode"])
+    assert _bf16_close(oracle.c_prefill_attn_causal(f["pre_q"], f["pre_k"], f["pre_v"], 0.125), f["pre_out"])
+    assert _bf16_close(oracle.c_prefill_attn_offset(f["chunk_q"], f["chunk_k"], f["chunk_v"], int(f["chunk_start"]), 0.125),
+                       f["chunk_out"])
+
+
+@pytest.mark.gpu
+def test_hip_reproduces_fused_fixture(fused):
+    from khaosz_amd import ops
+
+    f, dev = fused, "cuda:0"
+    bf = lambda a: torch.from_numpy(a.view(np.int16).copy()).view(torch.bfloat16).to(dev)
+    bits = lambda t: t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+    q, s = ops.rmsnorm_quant_rowwise_i8(bf(f["norm_x"]), bf(f["norm_gamma"]), 1e-5)
+    assert np.array_equal(q.cpu().numpy(), f["norm_codes"]) and np.array_equal(s.cpu().numpy(), f["norm_scale"])
+    q, s = ops.swiglu_quant_rowwise_i8(bf(f["swiglu_ug"]))
+    assert np.array_equal(q.cpu().numpy(), f["swiglu_codes"]) and np.array_equal(s.cpu().numpy(), f["swiglu_scale"])
+    kc, vc = bf(f["kc"]), bf(f["vc"])
+    fr = torch.from_numpy(f["rope_freqs"].copy())
+    freqs = torch.view_as_complex(fr).to(dev)
+    table = torch.from_numpy(f["table"].copy()).to(dev)
+    pos = int(f["pos"])
+    qr = ops.rope_kv_write(bf(f["rope_qkv"]), freqs, table, pos, kc, vc, 4, 2)
+    assert np.array_equal(bits(qr), f["q_rot"]) and np.array_equal(bits(kc), f["kc_after"])
+    assert np.array_equal(bits(vc), f["vc_after"])
+    out = ops.paged_attn_decode(qr, kc, vc, table, pos + 1)
+    tol = lambda t, want: torch.allclose(t.float().cpu(), torch.from_numpy(want.view(np.int16).copy()).view(torch.bfloat16).float(),
+                                         rtol=1e-2, atol=1e-2)   # the stated tolerance of the attention kernels
+    assert tol(out, f["attn_decode"])
+    kc2, vc2 = bf(f["kc"]), bf(f["vc"])
+    fused_out = ops.rope_paged_attn_decode(bf(f["rope_qkv"]), freqs, table, pos + 1, kc2, vc2, 4, 2)
+    assert torch.equal(fused_out, out) and np.array_equal(bits(kc2), f["kc_after"])
+    pre = ops.prefill_attn_causal(bf(f["pre_q"]), bf(f["pre_k"]), bf(f["pre_v"]))
+    assert tol(pre, f["pre_out"])
+    # the chunk on top of cached tokens: its keys and values laid into pages first
+    ck, cv, start = bf(f["chunk_k"]), bf(f["chunk_v"]), int(f["chunk_start"])
+    B, T, Hkv, D = ck.shape
+    page, P = 8, (T + 7) // 8
+    kp = torch.zeros(B * P, page, Hkv, D, dtype=torch.bfloat16, device=dev)
+    vp = torch.zeros_like(kp)
+    tb = torch.arange(B * P, device=dev).view(B, P).flip(1).contiguous()
+    for b in range(B):
+        for t in range(T):
+            kp[tb[b, t // page], t % page], vp[tb[b, t // page], t % page] = ck[b, t], cv[b, t]
+    got = ops.prefill_attn_paged(bf(f["chunk_q"]), kp, vp, tb, start)
+    assert tol(got, f["chunk_out"])

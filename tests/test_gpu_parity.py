@@ -233,6 +233,34 @@ def test_gemm_i8_i32_bit_exact(oracle, tile, M, N, K):
     assert np.array_equal(to_np(acc), want)
 
 
+def test_gemm_with_more_tiles_than_compute_units(oracle, tile):
+    """Beyond 256 tiles a workgroup walks several of them, reusing its LDS stages: 8200 x 1300 is 363
+    tiles of 256 rows (two passes, the second partial) or 715 of 128 (three).  int32 sums, the fused
+    epilogue with bias and residual, and the FP8 product, each against the oracle."""
+    M, N, K = 8200, 1300, 144
+    _say("gemm many tiles", M, N, K, tile)
+    xq, wq = rand_codes(M, K, 11), rand_codes(N, K, 12)
+    want = oracle.c_gemm_i8_i32(xq.numpy(), wq.numpy())
+    assert np.array_equal(to_np(ops.gemm_i8_i32(xq.to(DEV), wq.to(DEV))), want)
+    g = torch.Generator().manual_seed(13)
+    sx, sw = torch.rand(M, generator=g) + 0.01, torch.rand(N, generator=g) * 0.01 + 1e-4
+    bias = torch.randn(N, generator=g) * 0.01
+    res = (torch.randn(M, N, generator=g) * 2).to(torch.bfloat16)
+    y = ops.linear_w8a8(xq.to(DEV), sx.to(DEV), wq.to(DEV), sw.to(DEV), bias.to(DEV), out_dtype=torch.bfloat16)
+    assert np.array_equal(bf16_bits(y), oracle.c_dequant_epilogue(want, sx.numpy(), sw.numpy(), bias.numpy(), bf16_out=True))
+    y2 = ops.linear_w8a8(xq.to(DEV), sx.to(DEV), wq.to(DEV), sw.to(DEV), bias.to(DEV), out_dtype=torch.bfloat16,
+                         residual=res.to(DEV))
+    assert torch.equal(y2, y + res.to(DEV))
+    # FP8 codes from two binades: every product and partial sum is exact in fp32, so the result does not
+    # depend on the summation order or on the tile walk
+    a8 = torch.randint(0x30, 0x40, (M, K), generator=g, dtype=torch.uint8)     # e4m3 values 0.5 .. 1.875
+    b8 = torch.randint(0x30, 0x40, (N, K), generator=g, dtype=torch.uint8)
+    one = torch.ones(1, device=DEV)
+    y8 = ops.linear_fp8(a8.to(DEV), one, b8.to(DEV), one, out_dtype=torch.float32)
+    ref = a8.view(torch.float8_e4m3fn).float() @ b8.view(torch.float8_e4m3fn).float().T
+    assert torch.equal(y8.cpu(), ref)
+
+
 def test_gemm_i8_extremes(oracle, tile):
     K = 8192
     xq = torch.full((40, K), 127, dtype=torch.int8)

@@ -57,9 +57,11 @@ def parse():
     return ap.parse_args()
 
 
-def graph_time_ms(torch, step, steps, warmup):
+def graph_time_ms(torch, step, steps, warmup, dist=None):
     """Warm up eagerly, capture `steps` calls of step(i) into one HIP graph, replay it once
-    untimed, then time one replay with events on the launching stream.  Returns ms per step."""
+    untimed, then time one replay with events on the launching stream.  Returns ms per step.
+    dist: a list that receives [p10, p50, p90] of the ms per step of 11 further replays, each timed
+    on its own (the spread between replays; not part of the timed region)."""
     for i in range(warmup):
         step(i)
     torch.cuda.synchronize()
@@ -79,7 +81,17 @@ def graph_time_ms(torch, step, steps, warmup):
     g.replay()
     e1.record()
     torch.cuda.synchronize()
-    return e0.elapsed_time(e1) / steps
+    ms = e0.elapsed_time(e1) / steps
+    if dist is not None:
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(11)]
+        for a, b in evs:
+            a.record()
+            g.replay()
+            b.record()
+        torch.cuda.synchronize()
+        t = sorted(a.elapsed_time(b) / steps for a, b in evs)
+        dist[:] = [t[1], t[5], t[9]]
+    return ms
 
 
 def eager_time_ms(torch, step, steps, warmup):
@@ -129,19 +141,21 @@ def bench_decode(torch, ops, args, dev):
         ys[0] = ops.gemv_w8a8_codes(xq, sx, wq, sw, None, out_dtype=torch.bfloat16)
 
     bytes_alg = N * K + 4 * N + 2 * M * K + 2 * M * N
-    ms = graph_time_ms(torch, step, args.steps, args.warmup)
+    d_step, d_k = [], []
+    ms = graph_time_ms(torch, step, args.steps, args.warmup, d_step)
     ms_eager = eager_time_ms(torch, step, args.steps, args.warmup)
-    ms_k = graph_time_ms(torch, kernel_only, args.steps, args.warmup)
+    ms_k = graph_time_ms(torch, kernel_only, args.steps, args.warmup, d_k)
     ms_res = graph_time_ms(torch, resident, args.steps, args.warmup)
     gbs = bytes_alg / (ms * 1e-3) / 1e9
     gbs_k = bytes_alg / (ms_k * 1e-3) / 1e9
     return {
         "workload": f"decode_gemv_w8a8 M={M} K={K} N={N} bf16->int8 per-token, W int8 per-channel, bf16 out",
         "value": gbs, "unit": "GB/s", "ms_per_step": ms, "eager_ms_per_step": ms_eager,
-        "bytes_per_step": bytes_alg, "dtype": "int8",
+        "ms_per_step_p10_p50_p90": d_step, "bytes_per_step": bytes_alg, "dtype": "int8",
         "roofline": {"bound": "hbm", "kernel": "gemv_mfma_kernel" if M > 8 else "gemv_w8a8_kernel", "achieved": gbs_k, "peak": PEAK_HBM_GBS,
                      "unit": "GB/s", "frac": gbs_k / PEAK_HBM_GBS, "traffic": MEASURED_TRAFFIC["decode"].get(M),
-                     "kernel_us": ms_k * 1e3, "algorithmic_bytes": bytes_alg,
+                     "kernel_us": ms_k * 1e3, "kernel_us_p10_p50_p90": [v * 1e3 for v in d_k],
+                     "algorithmic_bytes": bytes_alg,
                      "llc_resident_gbs": bytes_alg / (ms_res * 1e-3) / 1e9, "weight_buffers": nbuf},
         "shape": (M, N, K),
     }
@@ -183,8 +197,9 @@ def bench_prefill(torch, ops, args, dev):
 
     ops_alg = 2.0 * M * N * K
     steps = max(10, min(args.steps, 100))
-    ms = graph_time_ms(torch, step, steps, args.warmup)
-    ms_k = graph_time_ms(torch, kernel_only, steps, args.warmup)
+    d_step, d_k = [], []
+    ms = graph_time_ms(torch, step, steps, args.warmup, d_step)
+    ms_k = graph_time_ms(torch, kernel_only, steps, args.warmup, d_k)
     ms_q = graph_time_ms(torch, quant_only, steps, args.warmup)
     ms_nq = graph_time_ms(torch, norm_quant_only, steps, args.warmup)
     tops = ops_alg / (ms * 1e-3) / 1e12
@@ -192,10 +207,12 @@ def bench_prefill(torch, ops, args, dev):
     qbytes = 2 * M * K + M * K + 4 * M
     return {
         "workload": f"prefill_linear_w8a8 M={M} K={K} N={N} quantise + int8 MFMA GEMM + scale/bias epilogue, bf16 out",
-        "value": tops, "unit": "TOPS", "ms_per_step": ms, "ops_per_step": ops_alg, "dtype": "int8",
+        "value": tops, "unit": "TOPS", "ms_per_step": ms, "ms_per_step_p10_p50_p90": d_step, "ops_per_step": ops_alg,
+        "dtype": "int8",
         "roofline": {"bound": "mfma", "kernel": "gemm_kernel<int8,bf16>", "achieved": tops_k, "peak": PEAK_INT8_TOPS,
                      "unit": "TOP/s", "frac": tops_k / PEAK_INT8_TOPS, "traffic": MEASURED_TRAFFIC["prefill"],
-                     "kernel_us": ms_k * 1e3, "algorithmic_ops": ops_alg},
+                     "kernel_us": ms_k * 1e3, "kernel_us_p10_p50_p90": [v * 1e3 for v in d_k],
+                     "algorithmic_ops": ops_alg},
         "quantise_kernel": {"us": ms_q * 1e3, "gbs": qbytes / (ms_q * 1e-3) / 1e9, "frac_hbm": qbytes / (ms_q * 1e-3) / 1e9 / PEAK_HBM_GBS,
                             "algorithmic_bytes": qbytes},
         "rmsnorm_quantise_kernel": {"us": ms_nq * 1e3, "gbs": (qbytes + 2 * K) / (ms_nq * 1e-3) / 1e9,
@@ -587,6 +604,7 @@ def main():
         "higher_is_better": main_res["unit"] != "ms", "scaling": "weak", "vs_baseline": None, "dtype": main_res["dtype"],
         "data": "synthetic", "config": {"workload": main_res["workload"], "timing": "HIP graph replay of the timed steps",
                                         "eager_ms_per_step": main_res.get("eager_ms_per_step"),
+                                        "replay_ms_per_step_p10_p50_p90": main_res.get("ms_per_step_p10_p50_p90"),
                                         **({"detail": detail} if detail else {})},
         "roofline": main_res["roofline"], "cpu_baseline": cpu, "measured_ceilings": ceilings,
         "also": {k: {kk: vv for kk, vv in v.items()} for k, v in extra.items()},

@@ -427,15 +427,36 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void paged_attn_decode_kernel(AttnA
 __global__ __launch_bounds__(ATT_MAX_D / 2) void attn_merge_kernel(const float* ws, uint16_t* out, int NS, int D) {
   const int d = threadIdx.x * 2, part_sz = D + 4;
   const float* part = ws + (int64_t)blockIdx.x * NS * part_sz;
+  // Slices are taken eight at a time, all loads of a group requested before any is used: with one slice per
+  // loop turn every load waited for the one before it (32 slices: two passes of 32 round trips).  The sums
+  // still run in slice order.
+  constexpr int GRP = 8;
   float mm = -INFINITY;
-  for (int s = 0; s < NS; ++s) mm = fmaxf(mm, part[s * part_sz + D]);  // slice 0 always holds a position
+  for (int s0 = 0; s0 < NS; s0 += GRP) {  // slice 0 always holds a position
+    float mv[GRP];
+#pragma unroll
+    for (int i = 0; i < GRP; ++i) mv[i] = s0 + i < NS ? part[(s0 + i) * part_sz + D] : -INFINITY;
+#pragma unroll
+    for (int i = 0; i < GRP; ++i) mm = fmaxf(mm, mv[i]);
+  }
   float n0 = 0.0f, n1 = 0.0f, den = 0.0f;
-  for (int s = 0; s < NS; ++s) {
-    const float a = attn_slice_weight(part[s * part_sz + D], mm);
-    const float2 v = *reinterpret_cast<const float2*>(part + s * part_sz + d);
-    n0 = __builtin_fmaf(v.x, a, n0);
-    n1 = __builtin_fmaf(v.y, a, n1);
-    den = __builtin_fmaf(part[s * part_sz + D + 1], a, den);
+  for (int s0 = 0; s0 < NS; s0 += GRP) {
+    float2 md[GRP], v[GRP];
+#pragma unroll
+    for (int i = 0; i < GRP; ++i) {
+      const bool ok = s0 + i < NS;  // uniform
+      md[i] = ok ? *reinterpret_cast<const float2*>(part + (s0 + i) * part_sz + D) : make_float2(0.0f, 0.0f);
+      v[i] = ok ? *reinterpret_cast<const float2*>(part + (s0 + i) * part_sz + d) : make_float2(0.0f, 0.0f);
+    }
+#pragma unroll
+    for (int i = 0; i < GRP; ++i) {
+      if (s0 + i < NS) {
+        const float a = attn_slice_weight(md[i].x, mm);
+        n0 = __builtin_fmaf(v[i].x, a, n0);
+        n1 = __builtin_fmaf(v[i].y, a, n1);
+        den = __builtin_fmaf(md[i].y, a, den);
+      }
+    }
   }
   const float r = attn_inv_denominator(den);
   store_wt(reinterpret_cast<uint32_t*>(out + (int64_t)blockIdx.x * D + d), pack_bf16x2(__fmul_rn(n0, r), __fmul_rn(n1, r)));

@@ -331,8 +331,8 @@ __global__ __launch_bounds__(1024) void swiglu_quant_wg_kernel(const void* __res
   const float wm = wave_max(vec_amax<EPV>(h));
   if (lane == 0) wmax[wave] = wm;
   __syncthreads();
-  float amax = 0.0f;
-  for (int w = 0; w < nwaves; ++w) amax = fmaxf(amax, wmax[w]);
+  // one LDS read per lane and a wavefront maximum, not a loop of dependent reads (at most 16 wavefronts)
+  const float amax = wave_max(lane < nwaves ? wmax[lane] : 0.0f);
   const RowScale rsc = row_scale(amax);
   if (v == 0) scale[row] = rsc.s;
   if (v < nvec) {

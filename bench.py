@@ -431,12 +431,20 @@ def bench_model(torch, ops, args, dev):
 
 
 def measure_ceilings(torch, ops, dev):
-    """What this part delivers on trivial kernels: an MFMA-only loop (constant operands, so the
-    clock is not power-limited: an upper bound), a 1 GiB streaming read, and a one-shot 16 MiB
-    read (the size of the decode weight), which no kernel of that size can beat."""
-    lib = ops._abi.load()
+    """What this part delivers on trivial kernels (the lab library's probes, csrc/aq_lab.h):
+      * an MFMA-only loop with constant operands (no bit toggling: the clock stays at its maximum) and with random
+        operands that change every instruction (what a GEMM feeds the matrix cores), each with the shader clock
+        the loop ran at: under matrix-core load with real data this part runs against its power limit;
+      * a 1 GiB streaming read;
+      * ONE launch reading 16 MiB (the size of the decode weight) from HBM, as a grid-stride loop and with every
+        load of a lane issued before any is used (1 .. 16 loads of 16 bytes per lane, plain and streaming), over
+        40 distinct buffers so that no launch finds its buffer in the last-level cache: no kernel of that size
+        can beat the best of these;
+      * an empty kernel: what a launch costs inside a replayed graph."""
+    lab = ops._abi.load_lab()
     st = torch.cuda.current_stream().cuda_stream
     sink = torch.zeros(4, dtype=torch.int32, device=dev)
+    clocks = torch.zeros(2, dtype=torch.int64, device=dev)
 
     def timed(fn, n):
         fn()
@@ -449,42 +457,59 @@ def measure_ceilings(torch, ops, dev):
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) * 1e-3 / n
 
+    def graph_us(launch, n=40):
+        """n launches captured in one graph, replayed once untimed and once timed: us per launch."""
+        for i in range(n):
+            launch(i, st)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(g, stream=side):
+                for i in range(n):
+                    launch(i, side.cuda_stream)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        best = None
+        for _ in range(3):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            g.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            t = e0.elapsed_time(e1) * 1e3 / n
+            best = t if best is None else min(best, t)
+        return best
+
     out = {}
-    iters = 4000
-    for kind, name, ops_per in ((0, "mfma_i8_32x32x32_tops", 65536), (2, "mfma_fp8_32x32x64_tflops", 131072)):
-        t = timed(lambda i=0: lib.aq_probe_mfma(kind, 1024, iters, sink.data_ptr(), st), 3)
-        out[name] = 1024 * 4 * iters * 8 * ops_per / t / 1e12
+    iters = 20000  # a few ms per probe: long enough for the clock to settle under the load
+    for kind, name, ops_per in ((0, "mfma_i8_32x32x32", 65536), (2, "mfma_fp8_32x32x64", 131072)):
+        unit = "tops" if kind == 0 else "tflops"
+        for data, tag in ((0, "constant_operands"), (1, "random_operands")):
+            t = timed(lambda i=0: lab.aq_lab_probe_mfma(kind, data, 256, iters, sink.data_ptr(), clocks.data_ptr(), st), 2)
+            c = clocks.tolist()
+            out[f"{name}_{tag}_{unit}"] = 256 * 4 * iters * 8 * ops_per / t / 1e12
+            out[f"{name}_{tag}_clock_mhz"] = c[0] / max(c[1], 1) * 100.0
     big = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
-    t = timed(lambda i=0: lib.aq_probe_read(big.data_ptr(), big.numel(), 2048, sink.data_ptr(), st), 3)
+    t = timed(lambda i=0: lab.aq_lab_probe_read(big.data_ptr(), big.numel(), 0, 2048, 0, sink.data_ptr(), st), 3)
     out["hbm_stream_read_gbs"] = big.numel() / t / 1e9
     del big
     small = [torch.empty(16 << 20, dtype=torch.uint8, device=dev) for _ in range(40)]
-
-    def one_shot(i=0):
-        lib.aq_probe_read(small[i % 40].data_ptr(), 16 << 20, 2048, sink.data_ptr(), st)
-
-    for i in range(40):
-        one_shot(i)
-    torch.cuda.synchronize()
-    g = torch.cuda.CUDAGraph()
-    side = torch.cuda.Stream()
-    side.wait_stream(torch.cuda.current_stream())
-    with torch.cuda.stream(side):
-        st2 = side.cuda_stream
-        with torch.cuda.graph(g, stream=side):
-            for i in range(40):
-                lib.aq_probe_read(small[i].data_ptr(), 16 << 20, 2048, sink.data_ptr(), st2)
-    torch.cuda.current_stream().wait_stream(side)
-    torch.cuda.synchronize()
-    g.replay()
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    g.replay()
-    e1.record()
-    torch.cuda.synchronize()
-    out["one_shot_16mib_read_us"] = e0.elapsed_time(e1) * 1e3 / 40
-    out["one_shot_16mib_read_gbs"] = (16 << 20) / (out["one_shot_16mib_read_us"] * 1e-6) / 1e9
+    shots = {}
+    for label, lpl, nt in (("grid_stride_2048_workgroups", 0, 0), ("upfront_1_load_per_lane", 1, 0),
+                           ("upfront_4_loads_per_lane", 4, 0), ("upfront_8_loads_per_lane", 8, 0),
+                           ("upfront_16_loads_per_lane", 16, 0), ("upfront_8_streaming_loads_per_lane", 8, 1),
+                           ("upfront_16_streaming_loads_per_lane", 16, 1)):
+        shots[label] = graph_us(lambda i, s, lpl=lpl, nt=nt: lab.aq_lab_probe_read(small[i % 40].data_ptr(), 16 << 20, lpl,
+                                                                                   2048, nt, sink.data_ptr(), s))
+    out["one_shot_16mib_read_us_by_variant"] = shots
+    best = min(shots.values())
+    out["one_shot_16mib_read_us"] = best
+    out["one_shot_16mib_read_gbs"] = (16 << 20) / (best * 1e-6) / 1e9
+    out["empty_kernel_in_graph_us"] = graph_us(lambda i, s: lab.aq_lab_probe_empty(sink.data_ptr(), s))
     return out
 
 

@@ -18,8 +18,9 @@
  *  - dtype codes: AQ_F32 = 0, AQ_BF16 = 1.
  *  - Return value: 0 on success, a negative AQ_E_* for a rejected argument, or
  *    a positive hipError_t from the launch.  aq_error_string() names either.
- *  - Re-entrant: no global mutable state.  (The reference calls Linear from its
- *    scheduler's daemon thread, astrai/inference/core/scheduler.py:191-196.)
+ *  - Re-entrant: no mutable state outlives a call except where an entry point says so (the
+ *    no-allocation variant's scratch).  (The reference calls Linear from its scheduler's
+ *    daemon thread, astrai/inference/core/scheduler.py:191-196.)
  */
 #ifndef ASTRAI_Q_H
 #define ASTRAI_Q_H
@@ -59,7 +60,10 @@ int aq_quant_rowwise_i8(const void *x, int x_dtype, int64_t M, int64_t K, int64_
 /* Per-tensor FP8 (OCP e4m3fn): scale[0] = amax / 448 (1 when all zero),
  * q = e4m3fn_rne(clamp(x / scale, -448, 448)).  Stands in for the operands of
  * the same F.linear call (linear.py:21) in the FP8 variant.
- * amax_ws: 4 bytes of device scratch the call overwrites. */
+ * amax_ws: AQ_FP8_AMAX_WS_BYTES of device scratch (partial maxima, one per workgroup of the
+ * first pass).  It needs no initial value and carries nothing from one call to the next; two
+ * calls that overlap in time must not share it.  Two launches: maximum, then scale + cast. */
+#define AQ_FP8_AMAX_WS_BYTES 1024
 int aq_quant_tensor_fp8(const void *x, int x_dtype, int64_t numel, uint8_t *q, float *scale,
                         uint32_t *amax_ws, void *stream);
 
@@ -287,28 +291,6 @@ int aq_prefill_attn_paged(const void *q, int64_t q_stride, const void *k_cache, 
                           const int64_t *page_table, int64_t P, int64_t start, int64_t page_size,
                           int64_t n_pages, void *out, float scale, int64_t B, int64_t S, int64_t Hq,
                           int64_t Hkv, int64_t D, void *stream);
-
-/* Tuning and test hook, no counterpart in the reference: the GEMM entry points
- * pick their workgroup tile (256 x 128, or 128 x 128 with a split K step when
- * the larger one would leave compute units idle) from M and N.  rows = 128 or
- * 256 forces one of them for every later call of this process, 0 restores the
- * choice by shape; anything else is AQ_E_SHAPE.  Results never depend on it
- * for the int8 path (exact int32 sums); FP8 outputs may differ in the last
- * bits of the fp32 accumulation.  Process-wide and unsynchronised: set it
- * while no GEMM call is in progress on another thread. */
-int aq_set_gemm_tile(int rows);
-
-/* ---- measurement probes: no counterpart in the reference, not on the Linear
- * path.  They measure what this part's matrix cores and HBM deliver so that the
- * benchmark can quote kernels against measured as well as published ceilings.
- * aq_probe_mfma: `workgroups` x 4 wavefronts each issue iters x 8 independent
- *   MFMAs; kind 0 = i32_32x32x32_i8 (65536 ops each), 1 = i32_16x16x64_i8
- *   (32768 ops), 2 = f32_32x32x64 e4m3 (131072 flops).
- * aq_probe_copy / aq_probe_read: grid-stride 16-byte streaming copy / read of
- *   `bytes` (a multiple of 16). */
-int aq_probe_mfma(int kind, int workgroups, int iters, int *sink, void *stream);
-int aq_probe_copy(const void *src, void *dst, int64_t bytes, int workgroups, void *stream);
-int aq_probe_read(const void *src, int64_t bytes, int workgroups, int *sink, void *stream);
 
 #ifdef __cplusplus
 }

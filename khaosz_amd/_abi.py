@@ -10,6 +10,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("ASTRAI_Q_LIB") or os.path.join(_HERE, "lib", "libastrai_q.so")
 
 AQ_F32, AQ_BF16 = 0, 1
+AQ_FP8_AMAX_WS_BYTES = 1024  # include/astrai_q.h
 
 # every symbol include/astrai_q.h declares: name -> (restype, argtypes)
 _i64, _vp, _int, _sz = ctypes.c_int64, ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
@@ -50,13 +51,20 @@ SYMBOLS = {
     "aq_gemv_w8a8_decode_attn": (_int, [_vp, _i64, _i64, _vp, _vp, _vp, _int, _vp, _vp, _int, _i64, _i64, _i64, _vp]),
     "aq_prefill_attn_paged": (_int, [_vp, _i64, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, ctypes.c_float, _i64, _i64, _i64,
                                      _i64, _i64, _vp]),
-    "aq_probe_mfma": (_int, [_int, _int, _int, _vp, _vp]),
-    "aq_probe_copy": (_int, [_vp, _vp, _i64, _int, _vp]),
-    "aq_probe_read": (_int, [_vp, _i64, _int, _vp, _vp]),
-    "aq_set_gemm_tile": (_int, [_int]),
+}
+
+# csrc/aq_lab.h: the lab library's additions (measurement probes, the tile-forcing test hook)
+LAB_LIB_PATH = os.path.join(_HERE, "lib", "libastrai_q_lab.so")
+LAB_SYMBOLS = {
+    "aq_lab_set_gemm_tile": (_int, [_int]),
+    "aq_lab_probe_mfma": (_int, [_int, _int, _int, _int, _vp, _vp, _vp]),
+    "aq_lab_probe_copy": (_int, [_vp, _vp, _i64, _int, _vp]),
+    "aq_lab_probe_read": (_int, [_vp, _i64, _int, _int, _int, _vp, _vp]),
+    "aq_lab_probe_empty": (_int, [_vp, _vp]),
 }
 
 _lib = None
+_lab = None
 
 
 def load() -> ctypes.CDLL:
@@ -76,6 +84,40 @@ def load() -> ctypes.CDLL:
         fn.argtypes = args
     _lib = lib
     return lib
+
+
+def load_lab() -> ctypes.CDLL:
+    """The lab library: every product symbol (from the same objects) plus LAB_SYMBOLS.  For the benchmark's
+    ceiling probes and for tests; the product path never loads it."""
+    global _lab
+    if _lab is not None:
+        return _lab
+    if not os.path.exists(LAB_LIB_PATH):
+        raise RuntimeError(f"{LAB_LIB_PATH} is missing: build it with `python -m khaosz_amd.build`")
+    lib = ctypes.CDLL(LAB_LIB_PATH)
+    for name, (res, args) in {**SYMBOLS, **LAB_SYMBOLS}.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    _lab = lib
+    return lib
+
+
+class lab_library:
+    """Context manager for tests: inside it ``load()`` hands out the lab library, so that the host module's
+    operators run the lab build (whose GEMM tile can be forced).  Not thread-safe; never used by the product."""
+
+    def __enter__(self):
+        global _lib
+        self._saved = _lib
+        _lib = load_lab()
+        return _lib
+
+    def __exit__(self, *exc):
+        global _lib
+        _lib.aq_lab_set_gemm_tile(0)
+        _lib = self._saved
+        return False
 
 
 def check(code: int, what: str) -> None:

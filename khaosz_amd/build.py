@@ -1,7 +1,11 @@
-"""Compile the HIP sources in csrc/ into khaosz_amd/lib/libastrai_q.so for gfx950.
+"""Compile the HIP sources in csrc/ for gfx950 into
 
-hipcc cross-compiles without a GPU.  The library depends on the HIP runtime
-only (no torch, no Python): it is the C ABI declared in include/astrai_q.h.
+  khaosz_amd/lib/libastrai_q.so      the product: the C ABI declared in include/astrai_q.h, nothing else;
+  khaosz_amd/lib/libastrai_q_lab.so  the same objects plus the measurement probes and the tile-forcing hook
+                                     of csrc/aq_lab.h (the GEMM source rebuilt with -DAQ_LAB), for the
+                                     benchmark's ceilings and for tests that pin a tile shape.
+
+hipcc cross-compiles without a GPU.  Both depend on the HIP runtime only (no torch, no Python).
 """
 import os
 import subprocess
@@ -12,7 +16,10 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(HERE, "lib", "obj")
 LIB = os.path.join(HERE, "lib", "libastrai_q.so")
-SOURCES = ["abi.hip", "quant.hip", "gemm_mfma.hip", "gemv.hip", "attn_decode.hip", "attn_prefill.hip", "probe.hip"]
+LAB_LIB = os.path.join(HERE, "lib", "libastrai_q_lab.so")
+SOURCES = ["abi.hip", "quant.hip", "gemm_mfma.hip", "gemv.hip", "attn_decode.hip", "attn_prefill.hip"]
+# (source, object, extra flags) of the lab library's own objects; the other product objects are shared
+LAB_SOURCES = [("gemm_mfma.hip", "gemm_mfma_lab.o", ["-DAQ_LAB"]), ("lab.hip", "lab.o", [])]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -34,13 +41,15 @@ def _stale(out, deps):
 
 def build(force: bool = True, verbose: bool = False) -> str:
     os.makedirs(OBJ_DIR, exist_ok=True)
-    headers = [os.path.join(CSRC, "aq_common.h"), os.path.join(CSRC, "aq_rows.h"), os.path.join(HERE, "..", "include", "astrai_q.h")]
+    headers = [os.path.join(CSRC, "aq_common.h"), os.path.join(CSRC, "aq_rows.h"), os.path.join(CSRC, "aq_lab.h"),
+               os.path.join(HERE, "..", "include", "astrai_q.h")]
 
-    def compile_one(src):
+    def compile_one(job):
+        src, obj, extra = job if isinstance(job, tuple) else (job, job.replace(".hip", ".o"), [])
         s = os.path.join(CSRC, src)
-        o = os.path.join(OBJ_DIR, src.replace(".hip", ".o"))
+        o = os.path.join(OBJ_DIR, obj)
         if force or _stale(o, [s] + headers):
-            cmd = [HIPCC, *FLAGS, "-c", s, "-o", o]
+            cmd = [HIPCC, *FLAGS, *extra, "-c", s, "-o", o]
             r = subprocess.run(cmd, capture_output=True, text=True)
             if r.returncode != 0:
                 raise RuntimeError(f"hipcc failed for {src}:\n{r.stderr}")
@@ -50,12 +59,15 @@ def build(force: bool = True, verbose: bool = False) -> str:
         return o
 
     with ThreadPoolExecutor(max_workers=4) as ex:
-        objs = list(ex.map(compile_one, SOURCES))
-    if force or _stale(LIB, objs):
-        cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]
-        r = subprocess.run(cmd, capture_output=True, text=True)
-        if r.returncode != 0:
-            raise RuntimeError(f"link failed:\n{r.stderr}")
+        all_objs = list(ex.map(compile_one, SOURCES + LAB_SOURCES))
+    objs, lab_only = all_objs[:len(SOURCES)], all_objs[len(SOURCES):]
+    lab_objs = [o for o in objs if not o.endswith("gemm_mfma.o")] + lab_only
+    for lib, members in ((LIB, objs), (LAB_LIB, lab_objs)):
+        if force or _stale(lib, members):
+            cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib, *members]
+            r = subprocess.run(cmd, capture_output=True, text=True)
+            if r.returncode != 0:
+                raise RuntimeError(f"link failed:\n{r.stderr}")
     return LIB
 
 

@@ -172,5 +172,21 @@ __device__ __forceinline__ void store_wt(uint2* p, uint2 v) {
 }
 
 inline int check_ptr16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ? AQ_E_ALIGN : AQ_OK; }
+inline int check_ptr(const void* p, unsigned align) { return (reinterpret_cast<uintptr_t>(p) & (align - 1u)) ? AQ_E_ALIGN : AQ_OK; }
+
+// Compute units of the current device, asked of the runtime once per device (launch shapes are
+// sized by it: a partition mode that exposes fewer compute units per device gets fewer workgroups).
+// The cache is written with the same value by whichever thread comes first: a benign race.
+inline int device_cus() {
+  static int cached[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  int v = cached[dev];
+  if (v <= 0) {
+    if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) v = 256;
+    cached[dev] = v;
+  }
+  return v;
+}
 
 }  // namespace aq

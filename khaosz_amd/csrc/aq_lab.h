@@ -1,0 +1,45 @@
+/*
+ * Measurement and test entry points of libastrai_q_lab.so.  NOT part of the product ABI
+ * (include/astrai_q.h) and not linked into libastrai_q.so: the lab library is the product's
+ * objects plus these, built for the benchmark's ceiling probes and for the tests that force
+ * a GEMM tile shape.  None of them has a counterpart in the reference.
+ */
+#ifndef AQ_LAB_H
+#define AQ_LAB_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Forces the GEMM workgroup tile for every later GEMM call of this process through the lab
+ * library: 128 (128 x 128, split K step), 256 (256 x 128), 0 = by shape.  Process-wide and
+ * unsynchronised -- which is why it does not exist in the product library. */
+int aq_lab_set_gemm_tile(int rows);
+
+/* `workgroups` x 4 wavefronts each issue iters x 8 independent MFMAs.
+ * kind 0 = i32_32x32x32_i8 (65536 ops each), 1 = i32_16x16x64_i8 (32768), 2 = f32_32x32x64 e4m3 (131072 flops).
+ * data 0 = constant operands (no toggling: the clock stays at its maximum), 1 = random bytes, four operand
+ * sets cycled between consecutive instructions (what a GEMM's operand stream does to the power budget).
+ * clocks (may be NULL): device int64[2] receiving the shader-clock and 100 MHz reference-clock ticks that
+ * wavefront 0 spent in the loop -- their ratio x 100 MHz is the clock the loop ran at. */
+int aq_lab_probe_mfma(int kind, int data, int workgroups, int iters, int *sink, long long *clocks, void *stream);
+
+/* Streaming copy, 16 bytes per lane, grid-stride: the known-size kernel HBM counters are scaled against. */
+int aq_lab_probe_copy(const void *src, void *dst, int64_t bytes, int workgroups, void *stream);
+
+/* Read `bytes` once.  loads_per_lane = 0: grid-stride loop over `workgroups` workgroups of 256 (each lane's
+ * loads are serialised by their use).  loads_per_lane = 1, 2, 4, 8, 16: every lane issues that many 16-byte
+ * loads before using any; the launch is sized to cover `bytes` exactly (which must divide evenly) and
+ * `workgroups` is ignored.  nontemporal != 0 marks the loads as streaming. */
+int aq_lab_probe_read(const void *src, int64_t bytes, int loads_per_lane, int workgroups, int nontemporal,
+                      int *sink, void *stream);
+
+/* One wavefront that does nothing: the cost of a launch. */
+int aq_lab_probe_empty(int *sink, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AQ_LAB_H */

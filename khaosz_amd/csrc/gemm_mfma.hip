@@ -24,21 +24,39 @@
 
 namespace aq {
 
-// Shapes of workgroup, all 8 wavefronts (two per SIMD), WM x 2 x WK of them, each
-// accumulating a (32 TM) x 64 sub-tile:
-//   WM = 4, TM = 2, WK = 1: 256 x 128 tile, 3 LDS stages of 48 KiB;
-//   WM = 2, TM = 2, WK = 2: 128 x 128 tile, 4 LDS stages of 32 KiB, the two wavefronts of a
-//                           sub-tile split every K step.
-// With WK = 2 the pair exchanges half of its accumulators through LDS at the end, so that
-// each wavefront finishes (and stores) 16 TM x 64 of the sums.
-// (WM = 2, TM = 4, WK = 2 -- a 256 x 128 tile of 128 x 64 sub-tiles, 6 fragment reads per
-// 8 MFMAs instead of 8 -- also builds, and measures 10 % slower than the first shape.)
-constexpr int BN = 128, BK = 128;
-constexpr int WAVES_N = 2, NWAVES = 8, NTHREADS = NWAVES * 64;
-constexpr int WAVE_N = BN / WAVES_N;
-constexpr int TN = WAVE_N / 32;
-constexpr int B_LOADS = BN * BK / 16 / NTHREADS;  // 16-byte vectors per thread per K step
-constexpr int BM_MAX = 256;
+// Shape of a workgroup: WM x WN x WK wavefronts, each accumulating a (32 TM) x (32 TN) sub-tile
+// (TM x TN MFMA 32x32 accumulators); K walked in BK-byte steps through NSTAGE LDS stages.
+//   <4, 2, 2, 2, 1, 128, 3>  256 x 128 tile, 8 wavefronts (two per SIMD) of 64 x 64, 3 stages of 48 KiB;
+//   <2, 2, 2, 2, 2, 128, 4>  128 x 128 tile, 8 wavefronts: the two that share a 64 x 64 sub-tile split every
+//                            K step and exchange half of their accumulators through LDS at the end, so that
+//                            each finishes (and stores) 32 x 64 of the sums; 4 stages of 32 KiB;
+// Shapes that only the lab build instantiates (measured, none faster: under a matrix-core load with real
+// operand data this part runs against its power limit, and fewer LDS reads per MFMA buy clock, not rate):
+//   <2, 2, 4, 4, 1, 64, 4>   256 x 256 tile, 4 wavefronts (one per SIMD) of 128 x 128: 256 accumulator
+//                            registers per lane (the AGPR half of the register file), 8 fragment reads per
+//                            16 MFMAs instead of 16, half the LDS fill per MFMA; 4 stages of 32 KiB;
+//   <4, 2, 2, 4, 1, 64, 4>   256 x 256 tile, 8 wavefronts of 64 x 128: 6 fragment reads per 8 MFMAs;
+//   <2, 2, 4, 2, 1, 128, 3>  256 x 128 tile, 4 wavefronts of 128 x 64.
+template <int WM_, int WN_, int TM_, int TN_, int WK_, int BK_, int NSTAGE_>
+struct Shape {
+  static constexpr int WM = WM_, WN = WN_, TM = TM_, TN = TN_, WK = WK_, BK = BK_, NSTAGE = NSTAGE_;
+  static constexpr int NWAVES = WM * WN * WK, NTHREADS = NWAVES * 64;
+  static constexpr int WAVE_M = 32 * TM, WAVE_N = 32 * TN;
+  static constexpr int BM = WM * WAVE_M, BN = WN * WAVE_N;
+  static constexpr int STAGE = (BM + BN) * BK;
+  static constexpr int LDS_BYTES = NSTAGE * STAGE;
+  static_assert(BK == 64 || BK == 128, "K bytes per stage");
+  static_assert(NWAVES % 2 == 0, "the piece permutation assumes a wavefront's row groups share parity");
+  static_assert((BM * BK / 1024) % NWAVES == 0 && (BN * BK / 1024) % NWAVES == 0, "whole 1 KiB loads per wavefront");
+  static_assert(LDS_BYTES <= 160 * 1024, "LDS of one compute unit");
+};
+using ShapeLarge = Shape<4, 2, 2, 2, 1, 128, 3>;
+using ShapeSmall = Shape<2, 2, 2, 2, 2, 128, 4>;
+#ifdef AQ_LAB
+using ShapeHuge = Shape<2, 2, 4, 4, 1, 64, 4>;
+using ShapeTall = Shape<2, 2, 4, 2, 1, 128, 3>;
+using ShapeHuge8 = Shape<4, 2, 2, 4, 1, 64, 4>;
+#endif
 constexpr int NUM_XCD = 8;
 constexpr int GROUP_M = 4;
 
@@ -137,29 +155,31 @@ __device__ __forceinline__ void sched_pattern() {
   }
 }
 
-template <bool FP8, int OUT, int WM, int TM, int WK>
+template <bool FP8, int OUT, class S>
 __device__ __forceinline__ void gemm_tile(const GemmArgs& p, uint8_t* smem, int pid) {
-  static_assert(WM * WAVES_N * WK == NWAVES, "8 wavefronts per workgroup");
+  constexpr int WM = S::WM, WN = S::WN, TM = S::TM, TN = S::TN, WK = S::WK, BK = S::BK, NSTAGE = S::NSTAGE;
+  constexpr int NWAVES = S::NWAVES, NTHREADS = S::NTHREADS, WAVE_M = S::WAVE_M, WAVE_N = S::WAVE_N;
+  constexpr int BM = S::BM, BN = S::BN, STAGE = S::STAGE;
   static_assert(TM % WK == 0, "the K-split pair divides the sub-tile's row blocks");
-  constexpr int WAVE_M = 32 * TM;
-  constexpr int BM = WM * WAVE_M;
   constexpr int TME = TM / WK;  // row blocks a wavefront finishes and stores
-  constexpr int NSTAGE = BM == 256 ? 3 : 4;
-  constexpr int A_LOADS = BM * BK / 16 / NTHREADS;
-  // NSTAGE stages of [A tile BM x 128 B][B tile 128 x 128 B], rows unpadded.
-  // Global->LDS loads land 64 lanes x 16 B contiguously (8 rows of 128 B), so
-  // the bank-conflict-free layout is obtained by permuting which 16-byte piece
-  // of its row each lane fetches: piece c of row r is stored at slot
-  // c ^ ((r / 2) % 8).  LDS has 64 banks here (two 128-byte rows per bank
+  constexpr int A_LOADS = BM * BK / 16 / NTHREADS;  // 16-byte vectors per thread per K step
+  constexpr int B_LOADS = BN * BK / 16 / NTHREADS;
+  // NSTAGE stages of [A tile BM x BK bytes][B tile BN x BK bytes], rows unpadded.
+  // Global->LDS loads land 64 lanes x 16 B contiguously (1 KiB: RPG = 8 rows of
+  // 128 B or 16 rows of 64 B), so the bank-conflict-free layout is obtained by
+  // permuting which 16-byte piece of its row each lane fetches: piece c of row r
+  // is stored at slot c ^ ((r / RPL) % PPR), with PPR = BK / 16 pieces per row and
+  // RPL = 256 / BK rows per bank line.  LDS has 64 banks here (256 bytes per bank
   // line) and a 16-byte-per-lane read is served 16 lanes at a time, so 16
-  // consecutive rows reading the same piece must land on 16 distinct slots.
-  constexpr int STAGE = (BM + BN) * BK;
+  // consecutive rows reading the same piece must land on 16 distinct slots:
+  // r % RPL picks the part of the bank line, the permuted piece the slot in it.
+  constexpr int PPR = BK / 16, RPL = 256 / BK, RPG = 1024 / BK;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wave_k = WK == 1 ? 0 : wave / (WM * WAVES_N), wave_mn = WK == 1 ? wave : wave % (WM * WAVES_N);
-  const int wave_m = wave_mn / WAVES_N, wave_n = wave_mn % WAVES_N;
+  const int wave_k = WK == 1 ? 0 : wave / (WM * WN), wave_mn = WK == 1 ? wave : wave % (WM * WN);
+  const int wave_m = wave_mn / WN, wave_n = wave_mn % WN;
 
   int tile_m, tile_n;
   tile_of_block(pid, p.tiles_m, p.tiles_n, tile_m, tile_n);
@@ -177,15 +197,15 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, uint8_t* smem, int 
   // first row of the part of the sub-tile this wavefront finishes (wavefront-uniform: kept scalar)
   const int mw = __builtin_amdgcn_readfirstlane(m0 + wave_m * WAVE_M + wave_k * (32 * TME));
 
-  // One load instruction of a wavefront fills 1 KiB = 8 tile rows.  Wavefront w
-  // owns the 8-row groups w, w+NWAVES, w+2*NWAVES, ... of A and of B.
-  // Row of lane l in group j: 8j + l/8, so (row/2) % 8 = 4*(w & 1) + l/16
-  // (NWAVES is even, so j and w have the same parity).
-  static_assert(NWAVES % 2 == 0, "the piece permutation assumes group and wavefront share parity");
-  const int ld_row = wave * 8 + (lane >> 3);  // + 8*NWAVES*i
-  const int ld_piece = ((lane & 7) ^ (4 * (wave & 1) + (lane >> 4))) * 16;  // piece this lane fetches
+  // One load instruction of a wavefront fills 1 KiB = RPG tile rows.  Wavefront w
+  // owns the row groups w, w+NWAVES, w+2*NWAVES, ... of A and of B.
+  // Row of lane l in group j: RPG j + l / PPR; (row / RPL) % PPR is the same for every
+  // group of a wavefront because RPG NWAVES / RPL is a multiple of PPR.
+  static_assert((RPG * NWAVES / RPL) % PPR == 0, "the piece permutation is the same for all row groups of a wavefront");
+  const int ld_row = wave * RPG + lane / PPR;  // + RPG*NWAVES*i
+  const int ld_piece = ((lane % PPR) ^ ((ld_row / RPL) % PPR)) * 16;  // piece this lane fetches
   const uint32_t ld_off = (uint32_t)ld_row * (uint32_t)K + ld_piece;
-  const uint32_t row32 = (uint32_t)(8 * NWAVES) * (uint32_t)K;  // byte distance between a wavefront's row groups
+  const uint32_t row32 = (uint32_t)(RPG * NWAVES) * (uint32_t)K;  // byte distance between a wavefront's row groups
   constexpr int NLOADS = A_LOADS + B_LOADS;
   // load number `idx` (0..NLOADS-1) of K step kt into stage buffer `buf`
   auto issue_load = [&](int kt, int buf, int idx) {
@@ -212,12 +232,13 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, uint8_t* smem, int 
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
-  // Fragment reads: lane -> tile row lane%32; its K pieces within a 128-byte row
+  // Fragment reads: lane -> tile row lane%32; its K pieces within a row
   // are (ks*2 + lane/32) for int8 (16 B per MFMA) and (ks*4 + (lane/32)*2 + {0,1})
-  // for FP8 (32 B per MFMA); slot = piece ^ ((row/2) % 8) and (row/2) % 8 == (lane/2) % 8.
+  // for FP8 (32 B per MFMA); slot = piece ^ ((row / RPL) % PPR), which depends on lane%32 only
+  // (sub-tile rows start at multiples of 32).
   const int fr_a = (wave_m * WAVE_M + (lane & 31)) * BK;
   const int fr_b = BM * BK + (wave_n * WAVE_N + (lane & 31)) * BK;
-  const int fsw = (lane >> 1) & 7;
+  const int fsw = ((lane & 31) / RPL) % PPR;
   constexpr int KSUB = FP8 ? 64 : 32;  // K per MFMA
   constexpr int NKS = BK / KSUB / WK;  // MFMA sub-steps per stage and wavefront: 4 or 2 (int8), 2 or 1 (FP8)
   // this wavefront's sub-steps of a stage start at piece wave_k * NKS * KSUB / 16; NKS is a power
@@ -254,28 +275,46 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, uint8_t* smem, int 
   // one on its SIMD) never queues a burst of memory instructions in front of
   // the matrix core.
   frag_t af[2][TM], bf[2][TN];
-  // slot number Q (0 = slot A .. NKS-1) issues loads [Q*NLOADS/NKS, (Q+1)*NLOADS/NKS) of its stage
+  // fragment number f of a sub-step, in the order the next sub-step's MFMAs need them: A0, B0 .. B(TN-1), A1 ..
+  auto load_frag = [&](const uint8_t* st, int ks, int f, frag_t (&a)[TM], frag_t (&b)[TN]) {
+    const bool is_a = f == 0 || f > TN;
+    const int idx = f == 0 ? 0 : f <= TN ? f - 1 : f - TN;
+    const uint8_t* base = st + (is_a ? fr_a : fr_b) + idx * 32 * BK;
+    if constexpr (!FP8) {
+      const v4i v = *reinterpret_cast<const v4i*>(base + (((ks * 2) << 4) ^ swz));
+      if (is_a) a[idx] = v; else b[idx] = v;
+    } else {
+      const int o0 = ((ks * 4) << 4) ^ swz;
+      const v4i lo = *reinterpret_cast<const v4i*>(base + o0);
+      const v4i hi = *reinterpret_cast<const v4i*>(base + (o0 ^ 16));
+      const v8i v = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+      if (is_a) a[idx] = v; else b[idx] = v;
+    }
+  };
+  // slot number Q (0 = slot A .. NKS-1) issues loads [Q*NLOADS/NKS, (Q+1)*NLOADS/NKS) of its stage.
+  // The order is written out and fenced: MFMA, then the fragment read(s) and at most a global load that
+  // it covers, so that every memory instruction is issued in the shadow of a running MFMA and no fragment is
+  // read right in front of its first use (left to itself the scheduler bunches the reads before the MFMAs
+  // that need them).  The last MFMAs of a slot carry no reads: the fragments have landed when the next slot starts.
   auto slot = [&](auto cur_c, const uint8_t* st_next, int ks_next, auto loads_c, int kt_ld, int buf_ld,
                   auto q_c) {
     constexpr int CUR = decltype(cur_c)::value;
     constexpr bool LOADS = decltype(loads_c)::value;
     constexpr int Q = decltype(q_c)::value;
-    constexpr int LD0 = (Q * NLOADS) / NKS, LPS = ((Q + 1) * NLOADS) / NKS - LD0;
-    load_frags(st_next, ks_next, af[CUR ^ 1], bf[CUR ^ 1]);
-    if constexpr (LOADS) {
+    constexpr int LD0 = (Q * NLOADS) / NKS, LPS = LOADS ? ((Q + 1) * NLOADS) / NKS - LD0 : 0;
+    constexpr int NMMA = TM * TN, NFR = TM + TN;
+    constexpr int GROUPS = NMMA > 4 ? NMMA - 2 : NMMA;  // MFMAs that carry memory instructions
 #pragma unroll
-      for (int q = 0; q < LPS; ++q) issue_load(kt_ld, buf_ld, LD0 + q);
+    for (int m = 0; m < NMMA; ++m) {
+      acc[m / TN][m % TN] = mma<FP8>(af[CUR][m / TN], bf[CUR][m % TN], acc[m / TN][m % TN]);
+      if (m < GROUPS) {
+#pragma unroll
+        for (int f = (m * NFR) / GROUPS; f < ((m + 1) * NFR) / GROUPS; ++f) load_frag(st_next, ks_next, f, af[CUR ^ 1], bf[CUR ^ 1]);
+#pragma unroll
+        for (int q = (m * LPS) / GROUPS; q < ((m + 1) * LPS) / GROUPS; ++q) issue_load(kt_ld, buf_ld, LD0 + q);
+      }
+      __builtin_amdgcn_sched_barrier(0);
     }
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-      for (int j = 0; j < TN; ++j) acc[i][j] = mma<FP8>(af[CUR][i], bf[CUR][j], acc[i][j]);
-    // issue order: one MFMA, then the LDS reads (and at most one global load) it covers
-    constexpr int NMMA = TM * TN;
-    constexpr int NDS = (TM + TN) * (FP8 ? 2 : 1);
-    constexpr int GROUPS = NMMA > 4 ? NMMA - 2 : NMMA;
-    sched_pattern<0, GROUPS, (NDS + GROUPS - 1) / GROUPS, LOADS ? LPS : 0>();
-    if constexpr (GROUPS < NMMA) __builtin_amdgcn_sched_group_barrier(0x008, NMMA - GROUPS, 0);
   };
   using std::integral_constant;
   using k0 = integral_constant<int, 0>;
@@ -499,9 +538,9 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, uint8_t* smem, int 
     // The residual elements a lane will add, requested ahead of the arithmetic: all columns at once on
     // the paired bf16 path (32 registers; the stores of one column would otherwise sit between the
     // loads of the next and their use), column by column on the others.
-    constexpr int RPG = PAIR ? 2 : 4;  // loads per 4-row group: packed row pairs, or single elements
-    constexpr bool HOIST = PAIR;
-    uint32_t rr[TN][TME][4][RPG];
+    constexpr int RLD = PAIR ? 2 : 4;  // loads per 4-row group: packed row pairs, or single elements
+    constexpr bool HOIST = PAIR && TN * TME <= 4;
+    uint32_t rr[HOIST ? TN : 1][TME][4][RLD];
     auto load_residual = [&](int j) {
       const uint32_t vbase = lane_offset(j);
 #pragma unroll
@@ -509,15 +548,15 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, uint8_t* smem, int 
 #pragma unroll
         for (int g = 0; g < 4; ++g)
 #pragma unroll
-          for (int q = 0; q < RPG; ++q) {
+          for (int q = 0; q < RLD; ++q) {
             const int r0 = i * 32 + g * 8;
             const int rowq = PAIR ? 2 * q : q;
             uint32_t vo = vbase;
             if (CHECK_M && mw + r0 + rq + rowq + (PAIR && odd ? 1 : 0) >= M) vo = OOB_OFFSET;
             if constexpr (OUT == OUT_F32 || PAIR)
-              rr[j][i][g][q] = __builtin_amdgcn_raw_buffer_load_b32(Rr, vo, (r0 + rowq) * rowb, 0);
+              rr[HOIST ? j : 0][i][g][q] = __builtin_amdgcn_raw_buffer_load_b32(Rr, vo, (r0 + rowq) * rowb, 0);
             else
-              rr[j][i][g][q] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(Rr, vo, (r0 + rowq) * rowb, 0);
+              rr[HOIST ? j : 0][i][g][q] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(Rr, vo, (r0 + rowq) * rowb, 0);
           }
     };
     if constexpr (OUT != OUT_I32 && HOIST) {
@@ -565,7 +604,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, uint8_t* smem, int 
               for (int q = 0; q < 4; ++q) {
                 uint32_t vo = vbase;
                 if (CHECK_M && mw + r0 + rq + q >= M) vo = OOB_OFFSET;
-                if (has_res) y[q] = __fadd_rn(y[q], __uint_as_float(rr[j][i][g][q]));
+                if (has_res) y[q] = __fadd_rn(y[q], __uint_as_float(rr[HOIST ? j : 0][i][g][q]));
                 __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(y[q]), Cr, vo, (r0 + q) * rowb, STORE_WT);
               }
             } else if constexpr (PAIR) {
@@ -578,7 +617,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, uint8_t* smem, int 
                 // odd lane:  {other.hi, mine.hi} = row 2h+1, columns (c-1, c)
                 uint32_t pk = __builtin_amdgcn_perm(other, mine, perm_sel);
                 if (has_res) {  // rounded output + residual, rounded again: what a separate add gives
-                  const uint32_t r = rr[j][i][g][h];
+                  const uint32_t r = rr[HOIST ? j : 0][i][g][h];
                   pk = pack_bf16x2(__fadd_rn(__uint_as_float(pk << 16), __uint_as_float(r << 16)),
                                    __fadd_rn(__uint_as_float(pk & 0xffff0000u), __uint_as_float(r & 0xffff0000u)));
                 }
@@ -592,7 +631,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, uint8_t* smem, int 
                 uint32_t vo = vbase;
                 if (CHECK_M && mw + r0 + rq + q >= M) vo = OOB_OFFSET;
                 uint32_t ob = f32_to_bf16_bits(y[q]);
-                if (has_res) ob = f32_to_bf16_bits(__fadd_rn(__uint_as_float(ob << 16), __uint_as_float(rr[j][i][g][q] << 16)));
+                if (has_res) ob = f32_to_bf16_bits(__fadd_rn(__uint_as_float(ob << 16), __uint_as_float(rr[HOIST ? j : 0][i][g][q] << 16)));
                 __builtin_amdgcn_raw_buffer_store_b16((uint16_t)ob, Cr, vo, (r0 + q) * rowb, STORE_WT);
               }
             }
@@ -611,51 +650,77 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, uint8_t* smem, int 
 
 // A workgroup walks tiles pid, pid + gridDim.x, ...: with more tiles than compute units the launch is one
 // resident workgroup per compute unit instead of a queue of short-lived ones (the LDS stages allow one at a time).
-template <bool FP8, int OUT, int WM, int TM, int WK>
-__global__ __launch_bounds__(NTHREADS) void gemm_kernel(GemmArgs p) {
-  constexpr int BM = WM * 32 * TM;
-  constexpr int NSTAGE = BM == 256 ? 3 : 4;
-  __shared__ __attribute__((aligned(1024))) uint8_t smem[NSTAGE * (BM + BN) * BK];
+#ifdef AQ_LAB
+__device__ long long aq_lab_clock[4];
+#endif
+template <bool FP8, int OUT, class S>
+__global__ __launch_bounds__(S::NTHREADS) void gemm_kernel(GemmArgs p) {
+  __shared__ __attribute__((aligned(1024))) uint8_t smem[S::LDS_BYTES];
   const int nt = p.tiles_m * p.tiles_n;
+#ifdef AQ_LAB
+  struct Clk {
+    long long c0, w0;
+    __device__ Clk() : c0(clock64()), w0(wall_clock64()) {}
+    __device__ ~Clk() {
+      if (blockIdx.x == 0 && threadIdx.x == 0) {
+        aq_lab_clock[0] = clock64() - c0;
+        aq_lab_clock[1] = wall_clock64() - w0;
+      }
+    }
+  } clk;
+#endif
   for (int pid = blockIdx.x; pid < nt; pid += gridDim.x) {
-    gemm_tile<FP8, OUT, WM, TM, WK>(p, smem, pid);
+    gemm_tile<FP8, OUT, S>(p, smem, pid);
     if (pid + (int)gridDim.x < nt) __syncthreads();  // every wavefront is done with the stages before they are refilled
   }
 }
 
-// 256-row tiles unless they leave much of the device idle: a workgroup per compute unit at a
-// time, so the cost of a launch is its number of rounds over the 256 compute units.  Measured:
+// Tile shape by the number of rounds over the compute units a launch needs: a workgroup per
+// compute unit at a time, so the cost of a launch is its number of rounds.  Measured:
 // a round of 128-row tiles costs 0.72 of a round of 256-row ones, and a last round that fills
 // only part of the device costs about half a round plus half its fill (384 large tiles, 1.5
 // rounds, take 1.74 times as long as 256).
-static int g_forced_tile = 0;  // 0: by shape; 128 / 256: forced (tuning and tests)
+enum TileKind { TILE_AUTO = 0, TILE_SMALL = 128, TILE_LARGE = 256, TILE_TALL = 257, TILE_HUGE = 512, TILE_HUGE8 = 513 };
+#ifdef AQ_LAB
+static int g_forced_tile = 0;  // lab build only: TILE_AUTO = by shape, otherwise forced (tuning and tests)
+#endif
 
-static bool use_small_tile(int64_t M, int64_t N) {
-  if (g_forced_tile) return g_forced_tile == 128;
-  constexpr int64_t CUS = 256;
-  const int64_t tn = (N + BN - 1) / BN;
-  auto rounds = [](int64_t tiles) {
-    const int64_t full = tiles / CUS, rest = tiles % CUS;
-    return (double)full + (rest ? 0.5 + 0.5 * (double)rest / CUS : 0.0);
+static int choose_tile(int64_t M, int64_t N) {
+#ifdef AQ_LAB
+  if (g_forced_tile) return g_forced_tile;
+#endif
+  const int64_t cus = device_cus();
+  const int64_t tn = (N + 127) / 128;
+  auto rounds = [cus](int64_t tiles) {
+    const int64_t full = tiles / cus, rest = tiles % cus;
+    return (double)full + (rest ? 0.5 + 0.5 * (double)rest / cus : 0.0);
   };
-  return 0.72 * rounds((M + 127) / 128 * tn) < rounds((M + 255) / 256 * tn);
+  return 0.72 * rounds((M + 127) / 128 * tn) < rounds((M + 255) / 256 * tn) ? TILE_SMALL : TILE_LARGE;
+}
+
+template <bool FP8, int OUT, class S>
+static int launch_shape(GemmArgs& a, hipStream_t st) {
+  a.tiles_m = (a.M + S::BM - 1) / S::BM;
+  a.tiles_n = (a.N + S::BN - 1) / S::BN;
+  // one resident workgroup per compute unit walks the tiles (a workgroup's LDS stages fill a compute unit):
+  // 3-5 % faster than queueing a workgroup per tile once there are more tiles than compute units
+  const int64_t ntiles = (int64_t)a.tiles_m * a.tiles_n, cus = device_cus();
+  const unsigned grid = (unsigned)(ntiles < cus ? ntiles : cus);
+  hipLaunchKernelGGL((gemm_kernel<FP8, OUT, S>), dim3(grid), dim3(S::NTHREADS), 0, st, a);
+  return (int)hipGetLastError();
 }
 
 template <bool FP8, int OUT>
 static int launch(GemmArgs& a, hipStream_t st) {
-  const bool small = use_small_tile(a.M, a.N);
-  const int bm = small ? 128 : 256;
-  a.tiles_m = (a.M + bm - 1) / bm;
-  a.tiles_n = (a.N + BN - 1) / BN;
-  // one resident workgroup per compute unit walks the tiles (a workgroup's LDS stages fill a compute unit):
-  // 3-5 % faster than queueing a workgroup per tile once there are more tiles than compute units
-  const int64_t ntiles = (int64_t)a.tiles_m * a.tiles_n;
-  const unsigned grid = (unsigned)(ntiles < 256 ? ntiles : 256);
-  if (small)
-    hipLaunchKernelGGL((gemm_kernel<FP8, OUT, 2, 2, 2>), dim3(grid), dim3(NTHREADS), 0, st, a);
-  else
-    hipLaunchKernelGGL((gemm_kernel<FP8, OUT, 4, 2, 1>), dim3(grid), dim3(NTHREADS), 0, st, a);
-  return (int)hipGetLastError();
+  switch (choose_tile(a.M, a.N)) {
+    case TILE_SMALL: return launch_shape<FP8, OUT, ShapeSmall>(a, st);
+#ifdef AQ_LAB
+    case TILE_TALL: return launch_shape<FP8, OUT, ShapeTall>(a, st);
+    case TILE_HUGE: return launch_shape<FP8, OUT, ShapeHuge>(a, st);
+    case TILE_HUGE8: return launch_shape<FP8, OUT, ShapeHuge8>(a, st);
+#endif
+    default: return launch_shape<FP8, OUT, ShapeLarge>(a, st);
+  }
 }
 
 static int check_gemm(const void* A, const void* B, const void* C, int64_t M, int64_t N, int64_t K) {
@@ -663,9 +728,10 @@ static int check_gemm(const void* A, const void* B, const void* C, int64_t M, in
   if (M == 0 || N == 0) return AQ_OK;
   if (!A || !B || !C) return AQ_E_NULL;
   if (check_ptr16(A) || check_ptr16(B) || check_ptr16(C)) return AQ_E_ALIGN;
-  // 32-bit tile-relative offsets: 256 rows * K bytes must fit an int
-  if (K > (1 << 22) || M > (1 << 30) || N > (1 << 30)) return AQ_E_RANGE;
-  if (((M + 127) / 128) * ((N + BN - 1) / BN) > (int64_t)0x7fffffff) return AQ_E_RANGE;
+  // 32-bit tile-relative offsets: 256 rows * K bytes of an operand and 256 rows * N * 4 bytes of the
+  // output window of a workgroup must fit 31 bits
+  if (K > (1 << 22) || M > (1 << 30) || N > (1 << 20)) return AQ_E_RANGE;
+  if (((M + 127) / 128) * ((N + 127) / 128) > (int64_t)0x7fffffff) return AQ_E_RANGE;
   return AQ_OK;
 }
 
@@ -682,11 +748,16 @@ static GemmArgs make_args(const void* A, const void* B, void* C, int64_t M, int6
 
 }  // namespace aq
 
-extern "C" int aq_set_gemm_tile(int rows) {
-  if (rows != 0 && rows != 128 && rows != 256) return AQ_E_SHAPE;
+#ifdef AQ_LAB
+extern "C" int aq_lab_read_clock(long long* host2) {
+  return (int)hipMemcpyFromSymbol(host2, HIP_SYMBOL(aq::aq_lab_clock), 16);
+}
+extern "C" int aq_lab_set_gemm_tile(int rows) {
+  if (rows != 0 && rows != 128 && rows != 256 && rows != 257 && rows != 512 && rows != 513) return AQ_E_SHAPE;
   aq::g_forced_tile = rows;
   return AQ_OK;
 }
+#endif
 
 extern "C" int aq_gemm_i8_i32(const int8_t* xq, const int8_t* wq, int32_t* acc, int64_t M, int64_t N,
                               int64_t K, void* stream) {
@@ -710,6 +781,9 @@ extern "C" int aq_linear_w8a8_residual(const int8_t* xq, const float* sx, const 
   int rc = aq::check_gemm(xq, wq, y, M, N, K);
   if (rc || M == 0 || N == 0) return rc;
   if (!sx || !sw) return AQ_E_NULL;
+  if (aq::check_ptr(sx, 4) || aq::check_ptr(sw, 4) || aq::check_ptr(bias, bias_dtype == AQ_BF16 ? 2 : 4) ||
+      aq::check_ptr(residual, 4))
+    return AQ_E_ALIGN;
   aq::GemmArgs a = aq::make_args(xq, wq, y, M, N, K);
   a.sx = sx;
   a.sw = sw;

@@ -283,13 +283,30 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_w8a8_kernel(GemvArgs p) {
 struct GemvShape {
   int waves, ksplit;
 };
+
+// A kernel whose dynamic LDS may exceed 64 KiB is opted in to the whole 160 KiB of a compute unit the first
+// time a launch on a device needs it (one attribute call per kernel and device instead of one per launch).
+// Two threads racing here both make the idempotent call.
+struct LdsOptIn {
+  bool done[64] = {};
+  int ensure(const void* fn) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = -1;
+    if (dev >= 0 && done[dev]) return 0;
+    const hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (e != hipSuccess) return (int)e;
+    if (dev >= 0) done[dev] = true;
+    return 0;
+  }
+};
 static GemvShape gemv_shape(int N, int K, bool fused) {
   GemvShape sh{GV_WAVES, 1};
   if (fused) return sh;
+  const int cus = device_cus();
   const int groups = (N + GV_ROWS - 1) / GV_ROWS, nchunk = (K + GV_CHUNK - 1) / GV_CHUNK;
-  while (nchunk >= 4 && sh.ksplit < 4 && groups * sh.ksplit < 1024 && nchunk >= 2 * sh.ksplit) sh.ksplit *= 2;
+  while (nchunk >= 4 && sh.ksplit < 4 && groups * sh.ksplit < 4 * cus && nchunk >= 2 * sh.ksplit) sh.ksplit *= 2;
   int per_wg = GV_WAVES / sh.ksplit;  // row groups per workgroup
-  while (per_wg > 1 && (groups + per_wg - 1) / per_wg < 256) per_wg >>= 1;
+  while (per_wg > 1 && (groups + per_wg - 1) / per_wg < cus) per_wg >>= 1;
   if (sh.ksplit == 1 && per_wg < 2) per_wg = 2;
   sh.waves = per_wg * sh.ksplit;
   return sh;
@@ -303,10 +320,10 @@ static int launch_gemv_fw(GemvArgs a, hipStream_t st) {
   const int rows_per_wg = GV_ROWS * (sh.waves / sh.ksplit);
   const unsigned grid = (unsigned)((a.N + rows_per_wg - 1) / rows_per_wg);
   const size_t lds = (size_t)MT * a.K + MT * sizeof(float) + (sh.ksplit > 1 ? (size_t)sh.waves * 64 * sizeof(int) : 0);
-  if (lds > 64 * 1024) {  // beyond the default dynamic-LDS limit: opt this kernel in (idempotent)
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_w8a8_kernel<MT, FUSED, VPL, NORM, MERGE, FW>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return (int)e;
+  if (lds > 64 * 1024) {  // beyond the default dynamic-LDS limit: opt this kernel in, once per device
+    static LdsOptIn opted;
+    const int e = opted.ensure(reinterpret_cast<const void*>(&gemv_w8a8_kernel<MT, FUSED, VPL, NORM, MERGE, FW>));
+    if (e) return e;
   }
   hipLaunchKernelGGL((gemv_w8a8_kernel<MT, FUSED, VPL, NORM, MERGE, FW>), dim3(grid), dim3(sh.waves * 64), lds, st, a);
   return (int)hipGetLastError();
@@ -519,9 +536,10 @@ static int launch_gemv_mfma(GemvArgs a, hipStream_t st) {
   // compute unit a workgroup, one row group per workgroup and up to 8 K parts
   a.ksplit = 2;
   a.groups = 2;
-  if ((a.N + 31) / 32 < 256) {
+  const int cus = device_cus();
+  if ((a.N + 31) / 32 < cus) {
     a.groups = 1;
-    while (a.ksplit < GM_MAX_WAVES && (a.N + 15) / 16 * (a.ksplit / 2) < 256 && a.K % (128 * a.ksplit) == 0 &&
+    while (a.ksplit < GM_MAX_WAVES && (a.N + 15) / 16 * (a.ksplit / 2) < cus && a.K % (128 * a.ksplit) == 0 &&
            a.K / (2 * a.ksplit) >= 512)
       a.ksplit *= 2;
   }
@@ -533,8 +551,9 @@ static int launch_gemv_mfma(GemvArgs a, hipStream_t st) {
                          : (res ? reinterpret_cast<const void*>(&gemv_mfma_kernel<0, 0, true>)
                                 : reinterpret_cast<const void*>(&gemv_mfma_kernel<0, 0, false>));
   if (lds > 64 * 1024) {
-    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return (int)e;
+    static LdsOptIn opted[4];
+    const int e = opted[(fixed ? 0 : 2) + (res ? 1 : 0)].ensure(fn);
+    if (e) return e;
   }
   const dim3 g(grid), b(a.ksplit * a.groups * 64);
   if (fixed && res) hipLaunchKernelGGL((gemv_mfma_kernel<2, 2, true>), g, b, lds, st, a);
@@ -553,18 +572,22 @@ extern "C" size_t aq_gemv_w8a8_workspace_bytes(int64_t M, int64_t K) {
   return aq::align256((size_t)(M * K)) + aq::align256((size_t)M * sizeof(float));
 }
 
-static int gemv_check(const int8_t* wq, const float* sw, const void* bias, int bias_dtype, const void* y,
-                      int y_dtype, int64_t M, int64_t N, int64_t K, int* mt_out) {
+// *mt_out: the token-count bucket of the GEMV kernels, or -1 when the activation codes of that bucket do
+// not fit the LDS of a compute unit (rows longer than 10 096 bytes at 9..16 tokens, 20 208 at 5..8, ...):
+// such a call is served by the tiled MFMA GEMM, which takes any M (same integer sums, same epilogue: same bits).
+static int gemv_check(const int8_t* wq, const float* sw, const void* bias, int bias_dtype, const void* residual,
+                      const void* y, int y_dtype, int64_t M, int64_t N, int64_t K, int* mt_out) {
   if (y_dtype != AQ_F32 && y_dtype != AQ_BF16) return AQ_E_DTYPE;
   if (bias && bias_dtype != AQ_F32 && bias_dtype != AQ_BF16) return AQ_E_DTYPE;
   if (M < 0 || M > 16 || N < 0 || K <= 0 || (K % 16) != 0) return AQ_E_SHAPE;
   if (M == 0 || N == 0) return AQ_OK;
   if (!wq || !sw || !y) return AQ_E_NULL;
-  if (aq::check_ptr16(wq)) return AQ_E_ALIGN;
-  if (N > (1 << 30)) return AQ_E_RANGE;
+  // matrices on 16 bytes (vector loads and stores), scale and bias vectors on their element size
+  if (aq::check_ptr16(wq) || aq::check_ptr16(y) || aq::check_ptr16(residual)) return AQ_E_ALIGN;
+  if (aq::check_ptr(sw, 4) || aq::check_ptr(bias, bias_dtype == AQ_BF16 ? 2 : 4)) return AQ_E_ALIGN;
+  if (N > (1 << 30) || K > (1 << 22)) return AQ_E_RANGE;
   const int mt = M <= 1 ? 1 : M <= 2 ? 2 : M <= 4 ? 4 : M <= 8 ? 8 : 16;
-  if ((int64_t)mt * K + 64 + 2048 > aq::GV_MAX_LDS) return AQ_E_RANGE;  // codes, scales, K-part sums
-  *mt_out = mt;
+  *mt_out = (int64_t)mt * K + 64 + 2048 > aq::GV_MAX_LDS ? -1 : mt;  // codes, scales, K-part sums
   return AQ_OK;
 }
 
@@ -608,10 +631,11 @@ extern "C" int aq_gemv_w8a8_codes_residual(const int8_t* xq, const float* sx, co
                                            const void* bias, int bias_dtype, const void* residual,
                                            void* y, int y_dtype, int64_t M, int64_t N, int64_t K, void* stream) {
   int mt = 0;
-  int rc = gemv_check(wq, sw, bias, bias_dtype, y, y_dtype, M, N, K, &mt);
+  int rc = gemv_check(wq, sw, bias, bias_dtype, residual, y, y_dtype, M, N, K, &mt);
   if (rc || M == 0 || N == 0) return rc;
   if (!xq || !sx) return AQ_E_NULL;
-  if (aq::check_ptr16(xq)) return AQ_E_ALIGN;
+  if (aq::check_ptr16(xq) || aq::check_ptr(sx, 4)) return AQ_E_ALIGN;
+  if (mt < 0) return aq_linear_w8a8_residual(xq, sx, wq, sw, bias, bias_dtype, residual, y, y_dtype, M, N, K, stream);
   aq::GemvArgs a{};
   a.xq = xq;
   a.sx = sx;
@@ -641,12 +665,12 @@ extern "C" int aq_gemv_w8a8_decode_residual(const void* x, int x_dtype, const in
                                             size_t ws_bytes, void* stream) {
   if (x_dtype != AQ_F32 && x_dtype != AQ_BF16) return AQ_E_DTYPE;
   int mt = 0;
-  int rc = gemv_check(wq, sw, bias, bias_dtype, y, y_dtype, M, N, K, &mt);
+  int rc = gemv_check(wq, sw, bias, bias_dtype, residual, y, y_dtype, M, N, K, &mt);
   if (rc || M == 0 || N == 0) return rc;
   if (!x || !ws) return AQ_E_NULL;
   if (aq::check_ptr16(x) || aq::check_ptr16(ws)) return AQ_E_ALIGN;
   if (ws_bytes < aq_gemv_w8a8_workspace_bytes(M, K)) return AQ_E_WORKSPACE;
-  if (x_dtype == AQ_BF16) {  // one launch: the GEMV kernel quantises the rows itself
+  if (x_dtype == AQ_BF16 && mt > 0) {  // one launch: the GEMV kernel quantises the rows itself
     aq::GemvArgs a{};
     a.x = x;
     a.wq = wq;
@@ -674,7 +698,7 @@ extern "C" int aq_gemv_w8a8_decode_attn(const float* partials, int64_t n_slices,
                                         const float* sw, const void* bias, int bias_dtype, const void* residual,
                                         void* y, int y_dtype, int64_t M, int64_t N, int64_t K, void* stream) {
   int mt = 0;
-  int rc = gemv_check(wq, sw, bias, bias_dtype, y, y_dtype, M, N, K, &mt);
+  int rc = gemv_check(wq, sw, bias, bias_dtype, residual, y, y_dtype, M, N, K, &mt);
   if (rc) return rc;
   if ((head_dim != 64 && head_dim != 128) || (K % head_dim) != 0 || n_slices <= 0) return AQ_E_SHAPE;
   // the in-kernel merge keeps every slice of a lane's vectors in registers
@@ -713,12 +737,12 @@ extern "C" int aq_gemv_w8a8_decode_rmsnorm(const void* x, int x_dtype, const voi
                                            size_t ws_bytes, void* stream) {
   if (x_dtype != AQ_F32 && x_dtype != AQ_BF16) return AQ_E_DTYPE;
   int mt = 0;
-  int rc = gemv_check(wq, sw, bias, bias_dtype, y, y_dtype, M, N, K, &mt);
+  int rc = gemv_check(wq, sw, bias, bias_dtype, residual, y, y_dtype, M, N, K, &mt);
   if (rc || M == 0 || N == 0) return rc;
   if (!x || !gamma || !ws) return AQ_E_NULL;
   if (aq::check_ptr16(x) || aq::check_ptr16(gamma) || aq::check_ptr16(ws)) return AQ_E_ALIGN;
   if (ws_bytes < aq_gemv_w8a8_workspace_bytes(M, K)) return AQ_E_WORKSPACE;
-  if (x_dtype == AQ_BF16) {  // one launch: the GEMV kernel normalises and quantises the rows itself
+  if (x_dtype == AQ_BF16 && mt > 0) {  // one launch: the GEMV kernel normalises and quantises the rows itself
     aq::GemvArgs a{};
     a.x = x;
     a.gamma = gamma;

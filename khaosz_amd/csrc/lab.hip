@@ -1,0 +1,213 @@
+// Measurement probes and test hooks of the lab library (libastrai_q_lab.so): what the matrix cores
+// and HBM of this particular part deliver, so that kernel figures can be read against measured
+// ceilings as well as the published ones.  Not on the Linear path and not in the product library.
+#include "aq_common.h"
+#include "aq_lab.h"
+
+namespace aq {
+
+__device__ __forceinline__ uint32_t lab_hash(uint32_t h) {
+  h ^= h >> 15;
+  h *= 2246822519u;
+  h ^= h >> 13;
+  h *= 3266489917u;
+  h ^= h >> 16;
+  return h;
+}
+
+// Every wavefront issues `iters` rounds of 8 independent MFMAs (no memory traffic, no
+// dependencies closer than 8 instructions apart).  DATA 0: one constant operand pair;
+// DATA 1: four random operand sets per lane, cycled so that consecutive instructions see
+// different bits on the operand buses, as a GEMM's fragment stream does.
+template <int KIND, int DATA>
+__global__ __launch_bounds__(256) void probe_mfma_kernel(int iters, int* sink, long long* clocks) {
+  const int lane = threadIdx.x & 63;
+  const uint32_t gid = blockIdx.x * 256 + threadIdx.x;
+  v4i a[4], b[4];
+#pragma unroll
+  for (int s = 0; s < 4; ++s) {
+    if constexpr (DATA == 0) {
+      a[s] = v4i{lane, lane + 1, lane + 2, lane + 3};
+      b[s] = v4i{lane * 3, 1, 2, 3};
+    } else {
+      // FP8: exponents kept low (no NaN, no overflow of the fp32 sums)
+      const uint32_t mask = KIND == 2 ? 0x77777777u : 0xffffffffu;
+      a[s] = v4i{(int)(lab_hash(gid * 32 + s * 8 + 0) & mask), (int)(lab_hash(gid * 32 + s * 8 + 1) & mask),
+                 (int)(lab_hash(gid * 32 + s * 8 + 2) & mask), (int)(lab_hash(gid * 32 + s * 8 + 3) & mask)};
+      b[s] = v4i{(int)(lab_hash(gid * 32 + s * 8 + 4) & mask), (int)(lab_hash(gid * 32 + s * 8 + 5) & mask),
+                 (int)(lab_hash(gid * 32 + s * 8 + 6) & mask), (int)(lab_hash(gid * 32 + s * 8 + 7) & mask)};
+    }
+  }
+  long long c0 = 0, w0 = 0;
+  if (clocks && gid == 0) {
+    c0 = clock64();
+    w0 = wall_clock64();
+  }
+  if constexpr (KIND == 0) {  // v_mfma_i32_32x32x32_i8
+    v16i c[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) c[i][r] = 0;
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        c[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i & 3], b[(i + (i >> 2)) & 3], c[i], 0, 0, 0);
+    }
+    int s = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) s += c[i][0] + c[i][15];
+    if (s == 0x12345678) sink[0] = s;
+  } else if constexpr (KIND == 1) {  // v_mfma_i32_16x16x64_i8
+    v4i c[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) c[i] = v4i{0, 0, 0, 0};
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        c[i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[i & 3], b[(i + (i >> 2)) & 3], c[i], 0, 0, 0);
+    }
+    int s = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) s += c[i][0] + c[i][3];
+    if (s == 0x12345678) sink[0] = s;
+  } else {  // v_mfma_scale_f32_32x32x64_f8f6f4, e4m3 x e4m3, unit scales
+    v16f c[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) c[i][r] = 0.0f;
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const v4i x = a[i & 3], y = a[(i + 1) & 3], u = b[(i + (i >> 2)) & 3], w = b[(i + 2) & 3];
+        const v8i aa = {x.x, x.y, x.z, x.w, y.x, y.y, y.z, y.w}, bb = {u.x, u.y, u.z, u.w, w.x, w.y, w.z, w.w};
+        c[i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(aa, bb, c[i], 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
+      }
+    }
+    float s = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) s += c[i][0] + c[i][15];
+    if (s == 1.2345f) sink[0] = 1;
+  }
+  if (clocks && gid == 0) {
+    clocks[0] = clock64() - c0;
+    clocks[1] = wall_clock64() - w0;
+  }
+}
+
+// Plain streaming copy, 16 bytes per lane, grid-stride: the known-size kernel
+// that HBM counters and achieved bandwidth are calibrated against.
+__global__ __launch_bounds__(256) void probe_copy_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst,
+                                                         int64_t nvec) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < nvec; i += stride) dst[i] = src[i];
+}
+
+// Read-only stream: sums every 16-byte vector (keeps the loads alive).
+__global__ __launch_bounds__(256) void probe_read_kernel(const uint4* __restrict__ src, int64_t nvec, int* sink) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  uint32_t s = 0;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < nvec; i += stride) {
+    const uint4 v = src[i];
+    s += v.x ^ v.y ^ v.z ^ v.w;
+  }
+  if (s == 0x12345678u) sink[0] = 1;
+}
+
+// The same read with every load of a lane issued before any is used: a wavefront owns L KiB contiguous
+// (its L loads are 1 KiB apart), so the whole buffer is requested at once and the kernel is one memory
+// latency plus the stream -- the shape of the decode GEMV's weight read.
+template <int L, bool NT>
+__global__ __launch_bounds__(256) void probe_read_upfront_kernel(const uint4* __restrict__ src, int* sink) {
+  const int lane = threadIdx.x & 63;
+  const int64_t wave = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 6;
+  uint4 v[L];
+#pragma unroll
+  for (int j = 0; j < L; ++j) {
+    const uint4* p = src + (wave * L + j) * 64 + lane;
+    if constexpr (NT) {
+      const uint32_t* q = reinterpret_cast<const uint32_t*>(p);
+      v[j] = make_uint4(__builtin_nontemporal_load(q), __builtin_nontemporal_load(q + 1), __builtin_nontemporal_load(q + 2),
+                        __builtin_nontemporal_load(q + 3));
+    } else {
+      v[j] = *p;
+    }
+  }
+  uint32_t s = 0;
+#pragma unroll
+  for (int j = 0; j < L; ++j) s += v[j].x ^ v[j].y ^ v[j].z ^ v[j].w;
+  if (s == 0x12345678u) sink[0] = 1;
+}
+
+__global__ void probe_empty_kernel(int* sink) {
+  if (threadIdx.x == 9999) sink[0] = 1;
+}
+
+template <int L>
+static int launch_read_upfront(const void* src, int64_t bytes, bool nt, int* sink, hipStream_t st) {
+  const int64_t per_wg = (int64_t)256 * 16 * L;
+  if (bytes % per_wg) return AQ_E_SHAPE;
+  const unsigned grid = (unsigned)(bytes / per_wg);
+  if (nt)
+    hipLaunchKernelGGL((probe_read_upfront_kernel<L, true>), dim3(grid), dim3(256), 0, st, static_cast<const uint4*>(src), sink);
+  else
+    hipLaunchKernelGGL((probe_read_upfront_kernel<L, false>), dim3(grid), dim3(256), 0, st, static_cast<const uint4*>(src), sink);
+  return (int)hipGetLastError();
+}
+
+}  // namespace aq
+
+extern "C" int aq_lab_probe_mfma(int kind, int data, int workgroups, int iters, int* sink, long long* clocks, void* stream) {
+  if (kind < 0 || kind > 2 || data < 0 || data > 1 || workgroups <= 0 || iters < 0) return AQ_E_SHAPE;
+  if (!sink) return AQ_E_NULL;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const dim3 g(workgroups), b(256);
+#define AQ_LAB_MFMA(K, D) hipLaunchKernelGGL((aq::probe_mfma_kernel<K, D>), g, b, 0, st, iters, sink, clocks)
+  if (kind == 0 && data == 0) AQ_LAB_MFMA(0, 0);
+  else if (kind == 0) AQ_LAB_MFMA(0, 1);
+  else if (kind == 1 && data == 0) AQ_LAB_MFMA(1, 0);
+  else if (kind == 1) AQ_LAB_MFMA(1, 1);
+  else if (data == 0) AQ_LAB_MFMA(2, 0);
+  else AQ_LAB_MFMA(2, 1);
+#undef AQ_LAB_MFMA
+  return (int)hipGetLastError();
+}
+
+extern "C" int aq_lab_probe_copy(const void* src, void* dst, int64_t bytes, int workgroups, void* stream) {
+  if (bytes < 0 || (bytes % 16) != 0 || workgroups <= 0) return AQ_E_SHAPE;
+  if (bytes == 0) return AQ_OK;
+  if (!src || !dst) return AQ_E_NULL;
+  if (aq::check_ptr16(src) || aq::check_ptr16(dst)) return AQ_E_ALIGN;
+  hipLaunchKernelGGL(aq::probe_copy_kernel, dim3(workgroups), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const uint4*>(src), static_cast<uint4*>(dst), bytes / 16);
+  return (int)hipGetLastError();
+}
+
+extern "C" int aq_lab_probe_read(const void* src, int64_t bytes, int loads_per_lane, int workgroups, int nontemporal,
+                                 int* sink, void* stream) {
+  if (bytes < 0 || (bytes % 16) != 0) return AQ_E_SHAPE;
+  if (bytes == 0) return AQ_OK;
+  if (!src || !sink) return AQ_E_NULL;
+  if (aq::check_ptr16(src)) return AQ_E_ALIGN;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  switch (loads_per_lane) {
+    case 0:
+      if (workgroups <= 0) return AQ_E_SHAPE;
+      hipLaunchKernelGGL(aq::probe_read_kernel, dim3(workgroups), dim3(256), 0, st, static_cast<const uint4*>(src),
+                         bytes / 16, sink);
+      return (int)hipGetLastError();
+    case 1: return aq::launch_read_upfront<1>(src, bytes, nontemporal != 0, sink, st);
+    case 2: return aq::launch_read_upfront<2>(src, bytes, nontemporal != 0, sink, st);
+    case 4: return aq::launch_read_upfront<4>(src, bytes, nontemporal != 0, sink, st);
+    case 8: return aq::launch_read_upfront<8>(src, bytes, nontemporal != 0, sink, st);
+    case 16: return aq::launch_read_upfront<16>(src, bytes, nontemporal != 0, sink, st);
+    default: return AQ_E_SHAPE;
+  }
+}
+
+extern "C" int aq_lab_probe_empty(int* sink, void* stream) {
+  if (!sink) return AQ_E_NULL;
+  hipLaunchKernelGGL(aq::probe_empty_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream), sink);
+  return (int)hipGetLastError();
+}

@@ -353,15 +353,17 @@ __global__ __launch_bounds__(1024) void swiglu_quant_wg_kernel(const void* __res
 // ---------------------------------------------------------------- FP8 tensor
 
 constexpr int FP8_BATCH = 4;  // 16-byte loads a thread keeps in flight in the per-tensor passes
-constexpr int AMAX_THREADS = 1024;  // few, large workgroups: the pass ends with one atomic per workgroup
+constexpr int AMAX_THREADS = 1024;  // few, large workgroups: the pass ends with one partial maximum per workgroup
+constexpr int AMAX_SLOTS = AQ_FP8_AMAX_WS_BYTES / 4;  // partial maxima in the workspace
 
-__global__ void fill_u32_kernel(uint32_t* p, uint32_t v) {
-  if (threadIdx.x == 0 && blockIdx.x == 0) *p = v;
-}
-
+// Pass 1: every workgroup leaves the maximum of its share in its own workspace slot (the launcher fills
+// all AMAX_SLOTS slots: workgroups past the data write 0).  No atomics and nothing to reset: the
+// workspace needs no initial value and a call leaves no state behind, so the whole quantisation is two
+// launches.  (A single slot updated with atomicMax needed a third launch to clear it, and same-address
+// atomics from 8 XCDs serialise at about 15 ns each.)
 template <bool BF16>
 __global__ __launch_bounds__(AMAX_THREADS) void amax_kernel(const void* __restrict__ x, int64_t nvec,
-                                                    uint32_t* __restrict__ amax_bits) {
+                                                    uint32_t* __restrict__ amax_slots) {
   constexpr int EPV = RowIn<BF16>::EPV;
   const uint4* src = reinterpret_cast<const uint4*>(x);
   float amax = 0.0f;
@@ -391,13 +393,7 @@ __global__ __launch_bounds__(AMAX_THREADS) void amax_kernel(const void* __restri
     float m = 0.0f;
 #pragma unroll
     for (int w = 0; w < AMAX_THREADS / 64; ++w) m = fmaxf(m, wmax[w]);
-    // |x| >= 0, so the IEEE bit patterns order like unsigned integers.  Same-address atomics
-    // from 8 XCDs serialise at about 15 ns each (2048 of them cost 30 us), so look first (a device-scope load; a stale
-    // value only costs an atomic that was not needed): after the first few workgroups hardly
-    // any partial maximum still exceeds the running one.
-    const uint32_t mb = __float_as_uint(m);
-    if (m > 0.0f && mb > __hip_atomic_load(amax_bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
-      atomicMax(amax_bits, mb);
+    amax_slots[blockIdx.x] = __float_as_uint(m);
   }
 }
 
@@ -408,11 +404,21 @@ __device__ __forceinline__ float fp8_prescale(float a, float s) {
 
 template <bool BF16>
 __global__ __launch_bounds__(256) void cast_fp8_kernel(const void* __restrict__ x, int64_t nvec,
-                                                        const uint32_t* __restrict__ amax_bits,
+                                                        const uint32_t* __restrict__ amax_slots,
                                                         uint8_t* __restrict__ q,
                                                         float* __restrict__ scale) {
   constexpr int EPV = RowIn<BF16>::EPV;
-  const float amax = __uint_as_float(*amax_bits);
+  // Pass 2 starts by combining the partial maxima: one slot per thread (1 KiB, served by the L2), a
+  // wavefront maximum, and the four wavefront results through LDS.  A maximum has no order: same bits
+  // whatever the grouping.
+  static_assert(AMAX_SLOTS == 256, "one slot per thread of the 256-thread workgroup");
+  __shared__ float part[4];
+  {
+    const float m = wave_max(__uint_as_float(amax_slots[threadIdx.x]));
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = m;
+  }
+  __syncthreads();
+  const float amax = fmaxf(fmaxf(part[0], part[1]), fmaxf(part[2], part[3]));
   float s = __fdiv_rn(amax, 448.0f);
   if (amax == 0.0f) s = 1.0f;
   if (blockIdx.x == 0 && threadIdx.x == 0) *scale = s;
@@ -605,7 +611,7 @@ extern "C" int aq_quant_tensor_fp8(const void* x, int x_dtype, int64_t numel, ui
   if (numel < 0 || (numel % 16) != 0) return AQ_E_SHAPE;
   if (!scale || !amax_ws) return AQ_E_NULL;
   if (numel > 0 && (!x || !q)) return AQ_E_NULL;
-  if (aq::check_ptr16(x) || aq::check_ptr16(q)) return AQ_E_ALIGN;
+  if (aq::check_ptr16(x) || aq::check_ptr16(q) || aq::check_ptr(amax_ws, 4) || aq::check_ptr(scale, 4)) return AQ_E_ALIGN;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const int epv = x_dtype == AQ_BF16 ? 8 : 4;
   const int64_t nvec = numel / epv;
@@ -613,9 +619,10 @@ extern "C" int aq_quant_tensor_fp8(const void* x, int x_dtype, int64_t numel, ui
   if (blocks > 2048) blocks = 2048;  // 8 workgroups per CU, grid-stride beyond
   if (blocks < 1) blocks = 1;
   int64_t ablocks = (nvec + aq::AMAX_THREADS * aq::FP8_BATCH - 1) / (aq::AMAX_THREADS * aq::FP8_BATCH);
-  if (ablocks > 256) ablocks = 256;  // one per CU
-  if (ablocks < 1) ablocks = 1;
-  hipLaunchKernelGGL(aq::fill_u32_kernel, dim3(1), dim3(64), 0, st, amax_ws, 0u);
+  // every slot is written each call: the grid is always AMAX_SLOTS workgroups (about one per compute unit;
+  // those past the data leave 0, which cannot change a maximum of magnitudes)
+  (void)ablocks;
+  ablocks = aq::AMAX_SLOTS;
   if (x_dtype == AQ_BF16) {
     hipLaunchKernelGGL((aq::amax_kernel<true>), dim3((unsigned)ablocks), dim3(aq::AMAX_THREADS), 0, st, x, nvec, amax_ws);
     hipLaunchKernelGGL((aq::cast_fp8_kernel<true>), dim3((unsigned)blocks), dim3(256), 0, st, x, nvec,

@@ -154,7 +154,7 @@ def quant_tensor_fp8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
         raise ValueError(f"numel must be a multiple of 16, got {n}")
     q = torch.empty(xc.shape, dtype=torch.uint8, device=x.device)
     s = torch.empty((1,), dtype=torch.float32, device=x.device)
-    ws = torch.empty((1,), dtype=torch.int32, device=x.device)
+    ws = torch.empty((_abi.AQ_FP8_AMAX_WS_BYTES // 4,), dtype=torch.int32, device=x.device)  # partial maxima, stateless
     with _OnDevice(x.device):
         rc = _abi.load().aq_quant_tensor_fp8(xc.data_ptr(), _dt(xc, "x"), n, q.data_ptr(), s.data_ptr(),
                                              ws.data_ptr(), _stream(x))
@@ -593,11 +593,6 @@ def paged_attn_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
                                                   B, Hq, Hkv, D, ws_ptr, ws_bytes, _stream(q))
         _abi.check(rc, "aq_paged_attn_decode")
     return out
-
-
-def set_gemm_tile(rows: int) -> None:
-    """Force the GEMM workgroup tile to 128 or 256 rows for this process (0: choose by shape)."""
-    _abi.check(_abi.load().aq_set_gemm_tile(int(rows)), "aq_set_gemm_tile")
 
 
 def linear_fp8(xq, sx, wq, sw, out_dtype=torch.bfloat16) -> torch.Tensor:

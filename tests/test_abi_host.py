@@ -26,6 +26,21 @@ def test_library_exports_every_declared_symbol():
     assert lib.aq_version() == 100
 
 
+def test_lab_library_holds_the_product_and_the_lab_symbols():
+    """The probes and the tile-forcing hook live in a second library built from the same objects:
+    the product library exports none of them."""
+    lab_header = open(os.path.join(ROOT, "khaosz_amd", "csrc", "aq_lab.h")).read()
+    declared = set(re.findall(r"\b(aq_lab_[a-z0-9_]+)\s*\(", lab_header))
+    assert declared == set(_abi.LAB_SYMBOLS), declared ^ set(_abi.LAB_SYMBOLS)
+    lab, lib = _abi.load_lab(), _abi.load()
+    for name in declared:
+        assert hasattr(lab, name), name
+        assert not hasattr(lib, name), f"{name} leaked into the product library"
+    for name in _abi.SYMBOLS:
+        assert hasattr(lab, name), name
+    assert lab.aq_lab_set_gemm_tile(3) == -2 and lab.aq_lab_set_gemm_tile(0) == 0
+
+
 def test_argument_validation_happens_before_any_launch():
     lib = _abi.load()
     P = 1 << 20  # a 16-byte aligned fake pointer; never dereferenced on these paths
@@ -43,7 +58,9 @@ def test_argument_validation_happens_before_any_launch():
     assert lib.aq_linear_fp8(P, P, P, P, P, 9, 4, 4, 32, None) == -3
     assert lib.aq_gemv_w8a8_decode(P, 1, P, P, None, 0, P, 1, 17, 8, 32, P, 1 << 20, None) == -2  # M > 16
     assert lib.aq_gemv_w8a8_decode(P, 1, P, P, None, 0, P, 1, 4, 8, 32, P, 8, None) == -5         # workspace
-    assert lib.aq_gemv_w8a8_decode(P, 1, P, P, None, 0, P, 1, 16, 8, 16384, P, 1 << 30, None) == -6  # LDS
+    assert lib.aq_gemv_w8a8_decode(P, 1, P, P, None, 0, P + 2, 1, 4, 8, 32, P, 1 << 20, None) == -4  # y alignment
+    assert lib.aq_gemv_w8a8_codes(P, P, P, P + 1, None, 0, P, 1, 4, 8, 32, None) == -4            # scale alignment
+    assert lib.aq_linear_w8a8(P, P, P, P, None, 0, P, 1, 4, 1 << 21, 32, None) == -6              # N beyond the epilogue's offsets
     assert lib.aq_gemv_w8a8_workspace_bytes(16, 2048) >= 16 * 2048 + 64
     assert b"multiple of 16" in lib.aq_error_string(-2)
     with pytest.raises(ValueError):

@@ -12,7 +12,7 @@ import torch
 
 pytestmark = pytest.mark.gpu
 
-from khaosz_amd import ops  # noqa: E402
+from khaosz_amd import _abi, ops  # noqa: E402
 from khaosz_amd.linear import Fp8Linear, Linear, QuantLinear, quantize_model  # noqa: E402
 
 DEV = "cuda:0"
@@ -214,9 +214,9 @@ GEMM_SHAPES = [(1, 1, 16), (37, 91, 48), (17, 5, 2048), (256, 128, 128), (257, 1
 @pytest.fixture(params=[128, 256])
 def tile(request):
     """Run a GEMM test once per workgroup tile shape (the library would pick one by shape)."""
-    ops.set_gemm_tile(request.param)
-    yield request.param
-    ops.set_gemm_tile(0)
+    with _abi.lab_library() as lab:  # the lab build of the same sources: its tile can be forced
+        assert lab.aq_lab_set_gemm_tile(request.param) == 0
+        yield request.param
 
 
 def rand_codes(M, K, seed):
@@ -379,6 +379,35 @@ def test_gemv_with_the_norm_folded_in_equals_norm_quantise_then_gemv(oracle, M, 
         want = ops.gemv_w8a8_codes(xq, sx, wqd, swd, out_dtype=torch.bfloat16, residual=res)
         got = ops.gemv_w8a8_decode(x, wqd, swd, out_dtype=torch.bfloat16, residual=res, norm=(gamma, 1e-5))
         assert torch.equal(got, want)
+
+
+@pytest.mark.parametrize("M,K", [(12, 11008), (16, 14336), (7, 22016)])
+def test_decode_rows_too_long_for_the_gemv_take_the_tiled_gemm(oracle, M, K):
+    """Activation codes of 9..16 tokens fit a compute unit's LDS up to K = 10 096 (5..8 tokens: 20 208).
+    Longer rows (FFN down projections of 11 008 or 14 336) must still work at decode batch sizes:
+    the decode entry points hand them to the MFMA GEMM.  Same bits as the oracle, with bias and residual,
+    through the drop-in module as well."""
+    N = 200
+    _say("gemv long K", M, N, K)
+    x = make_x(M, K, 41 + M).to(torch.bfloat16)
+    w = make_x(N, K, 42) * 0.02
+    wq, sw = oracle.c_quant_rowwise_i8(w.numpy())
+    b = torch.randn(N, generator=torch.Generator().manual_seed(43)) * 0.01
+    wqd, swd = torch.from_numpy(wq).to(DEV), torch.from_numpy(sw).to(DEV)
+    want = oracle.c_linear_w8a8(bf16_bits(x), wq, sw, b.numpy(), x_bf16_bits=True, bf16_out=True)
+    y = ops.gemv_w8a8_decode(x.to(DEV), wqd, swd, b.to(DEV), out_dtype=torch.bfloat16)
+    assert np.array_equal(bf16_bits(y), want)
+    r = torch.randn(M, N, generator=torch.Generator().manual_seed(44)).to(DEV, torch.bfloat16)
+    assert torch.equal(ops.gemv_w8a8_decode(x.to(DEV), wqd, swd, b.to(DEV), out_dtype=torch.bfloat16, residual=r), y + r)
+    xq, sx = ops.quant_rowwise_i8(x.to(DEV))
+    assert torch.equal(ops.gemv_w8a8_codes(xq, sx, wqd, swd, b.to(DEV), out_dtype=torch.bfloat16), y)
+    lin = Linear(K, N, bias=True)
+    with torch.no_grad():
+        lin.weight.copy_(w)
+        lin.bias.copy_(b)
+    q = QuantLinear.from_linear(lin.to(DEV))
+    with torch.inference_mode():
+        assert np.array_equal(bf16_bits(q(x.to(DEV))), want)
 
 
 def test_gemv_f32_in_out_and_agrees_with_gemm_path(oracle):

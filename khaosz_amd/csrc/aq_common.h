@@ -143,6 +143,11 @@ __device__ __forceinline__ uint4 buffer_load_16(__amdgpu_buffer_rsrc_t r, uint32
   v4i v = __builtin_amdgcn_raw_buffer_load_b128(r, (int)byte_off, 0, 0);
   return make_uint4((uint32_t)v.x, (uint32_t)v.y, (uint32_t)v.z, (uint32_t)v.w);
 }
+// the same load marked as streaming (nt): data that is read exactly once, such as a decode step's weights
+__device__ __forceinline__ uint4 buffer_load_16_stream(__amdgpu_buffer_rsrc_t r, uint32_t byte_off) {
+  v4i v = __builtin_amdgcn_raw_buffer_load_b128(r, (int)byte_off, 0, 2);
+  return make_uint4((uint32_t)v.x, (uint32_t)v.y, (uint32_t)v.z, (uint32_t)v.w);
+}
 constexpr uint32_t OOB_OFFSET = 0x7ffffff0u;  // beyond every descriptor built here
 
 // Write-through stores for bulk outputs.  With the default write-back policy

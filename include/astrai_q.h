@@ -115,6 +115,20 @@ int aq_gemv_w8a8_decode_residual(const void *x, int x_dtype, const int8_t *wq, c
                                  const void *bias, int bias_dtype, const void *residual, void *y,
                                  int y_dtype, int64_t M, int64_t N, int64_t K, void *ws,
                                  size_t ws_bytes, void *stream);
+
+/* The same call for callers that cannot allocate.  No counterpart in the reference: it is for code under
+ * HIP graph capture, tight serving loops and harnesses that forbid hipMalloc, which cannot provide the
+ * workspace of the entry point above.  The workspace (activation codes and scales between the row quantiser
+ * and the GEMV) is a device array that the library owns: AQ_GEMV_NOALLOC_MAX_MK + 256 bytes on every GPU the
+ * library runs on, held until the process ends.  M * K beyond AQ_GEMV_NOALLOC_MAX_MK (16 rows of 16384) is
+ * AQ_E_RANGE.  Allocates nothing and calls no allocating routine; the array's address is looked up on the first
+ * call on each device (make that call outside a graph capture).  Every call on a GPU uses that GPU's one array:
+ * calls that overlap in time on the same GPU (two streams, two threads) race on it -- serialise them or
+ * use aq_gemv_w8a8_decode_residual with a workspace per stream.  Results are bit-identical to that entry point. */
+#define AQ_GEMV_NOALLOC_MAX_MK 262144
+int aq_gemv_w8a8_decode_noalloc(const void *x, int x_dtype, const int8_t *wq, const float *sw,
+                                const void *bias, int bias_dtype, const void *residual, void *y,
+                                int y_dtype, int64_t M, int64_t N, int64_t K, void *stream);
 int aq_gemv_w8a8_codes_residual(const int8_t *xq, const float *sx, const int8_t *wq, const float *sw,
                                 const void *bias, int bias_dtype, const void *residual, void *y,
                                 int y_dtype, int64_t M, int64_t N, int64_t K, void *stream);

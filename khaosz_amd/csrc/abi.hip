@@ -11,7 +11,7 @@ extern "C" const char* aq_error_string(int code) {
     case AQ_E_DTYPE: return "unknown dtype code";
     case AQ_E_ALIGN: return "pointer or leading dimension is not 16-byte aligned";
     case AQ_E_WORKSPACE: return "workspace too small";
-    case AQ_E_RANGE: return "size beyond what the kernels index";
+    case AQ_E_RANGE: return "size beyond what the kernels index, or beyond the array of the no-allocation entry point";
     default: break;
   }
   if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));

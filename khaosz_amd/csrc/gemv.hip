@@ -773,6 +773,53 @@ extern "C" int aq_gemv_w8a8_decode_residual(const void* x, int x_dtype, const in
   return aq_gemv_w8a8_codes_residual(xq, sx, wq, sw, bias, bias_dtype, residual, y, y_dtype, M, N, K, stream);
 }
 
+// ---------------------------------------------------------------------------
+// The decode entry point for callers that cannot allocate (code under HIP graph capture, serving loops and
+// harnesses that forbid hipMalloc): the workspace of aq_gemv_w8a8_decode_residual -- the activation codes and
+// scales that the row quantiser hands to the GEMV when the rows are not quantised inside the GEMV kernel --
+// lives in device memory that the library itself owns, one copy per GPU, for the life of the process.
+namespace aq {
+
+constexpr size_t NOALLOC_SCRATCH_BYTES = AQ_GEMV_NOALLOC_MAX_MK + 256;  // codes [M, K] then scales [M]
+static_assert(AQ_GEMV_NOALLOC_MAX_MK % 256 == 0, "the scales start 256-byte aligned");
+static __device__ __align__(256) uint8_t scratch[NOALLOC_SCRATCH_BYTES];
+
+// In host code `scratch` is only a handle: the array's device address is asked of the runtime, once per
+// device (each GPU holds its own copy at its own address) with that device current, and kept.  Two threads
+// that come first at the same time both store the same address.
+static int scratch_of_current_device(void** out) {
+  static void* ptrs[64] = {};
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= 64) return AQ_E_RANGE;
+  void* p = __atomic_load_n(&ptrs[dev], __ATOMIC_ACQUIRE);
+  if (!p) {
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return (int)e;
+    if (!p) return AQ_E_NULL;
+    __atomic_store_n(&ptrs[dev], p, __ATOMIC_RELEASE);
+  }
+  *out = p;
+  return AQ_OK;
+}
+
+}  // namespace aq
+
+extern "C" int aq_gemv_w8a8_decode_noalloc(const void* x, int x_dtype, const int8_t* wq, const float* sw,
+                                           const void* bias, int bias_dtype, const void* residual, void* y,
+                                           int y_dtype, int64_t M, int64_t N, int64_t K, void* stream) {
+  // sizes beyond the scratch are rejected before anything else is looked at: AQ_E_RANGE, "size beyond ..."
+  if (M > 0 && K > 0 && (M > 16 || M * K > (int64_t)AQ_GEMV_NOALLOC_MAX_MK)) return M > 16 ? AQ_E_SHAPE : AQ_E_RANGE;
+  void* ws = nullptr;
+  const int rc = aq::scratch_of_current_device(&ws);
+  if (rc) return rc;
+  // The scratch keeps the previous call's contents; nothing in it has to start at zero: the quantiser
+  // writes all M rows of codes and all M scales before the GEMV reads exactly those.
+  return aq_gemv_w8a8_decode_residual(x, x_dtype, wq, sw, bias, bias_dtype, residual, y, y_dtype, M, N, K, ws,
+                                      aq::NOALLOC_SCRATCH_BYTES, stream);
+}
+
 extern "C" int aq_gemv_w8a8_decode_attn(const float* partials, int64_t n_slices, int64_t head_dim, const int8_t* wq,
                                         const float* sw, const void* bias, int bias_dtype, const void* residual,
                                         void* y, int y_dtype, int64_t M, int64_t N, int64_t K, void* stream) {

@@ -278,7 +278,11 @@ def bench_block(torch, ops, args, dev):
     # physical pages dealt out in a fixed shuffled order, as after some allocation history
     table = torch.randperm(B * pages_per_seq, generator=torch.Generator().manual_seed(8)).view(B, pages_per_seq).to(dev)
     fr = lambda a, n: tab[a:a + n].unsqueeze(0).expand(B, -1, -1)
-    masks = [decode_mask(B, S + t + 1, dev, dt) for t in range(steps)]
+    # the reference passes an all-zero mask tensor to a step whose sequences sit at one position; the paged
+    # kernels take no mask tensor (a tensor would send the step to the stock attention), so once they are
+    # switched on the steps pass None
+    zero_masks = [decode_mask(B, S + t + 1, dev, dt) for t in range(steps)]
+    masks = list(zero_masks)
 
     def prefill(i=0):
         return blk(x, fr(0, S), None, cache.bind(table, S))
@@ -304,6 +308,7 @@ def bench_block(torch, ops, args, dev):
     # and the paged-cache kernels: rotary + page writes in one launch at prefill, rotary + page
     # write + in-place attention in one launch for the single-token steps
     fuse_shared_inputs(blk, norms=True, decode_attention=True)
+    masks[:] = [None] * steps
     ms_pre_att = graph_time_ms(torch, prefill, 10, 3)
     prefill()
     ms_dec_att = graph_time_ms(torch, decode_all, 3, 2) / steps

@@ -214,14 +214,21 @@ int aq_swiglu_quant_rowwise_i8(const void *ug, int dtype, int64_t M, int64_t F, 
  * when one slice suffices -- then workspace may be NULL) and a second, small
  * kernel combines them.  A workspace that is too small is AQ_E_WORKSPACE.  The size
  * grows with total_len: a caller that sizes it once uses the longest sequence
- * it will serve. */
+ * it will serve.
+ * seq_lens (device int64 [B], or NULL: every sequence attends to all total_len positions): sequence b
+ * attends to positions t < seq_lens[b] only.  This is the reference's position mask for a decode batch whose
+ * sequences sit at different positions (execute_decode, executor.py:67-71, binds total_len = max position + 1
+ * and process_attention_mask, transformer.py:40-46, masks t > position_ids[b]: seq_lens[b] = position_ids[b]
+ * + 1); as in the reference the new token still goes to slot total_len - 1 of every sequence.  The same
+ * argument has the same meaning in the three entry points below. */
 int aq_rope_kv_write(const void *qkv, const float *freqs, int64_t freqs_stride,
                      const int64_t *page_table, int64_t P, int64_t pos, int64_t S,
                      int64_t page_size, void *k_cache, void *v_cache, int64_t n_pages,
                      void *q_out, void *k_out, int64_t B, int64_t Hq, int64_t Hkv, int64_t D,
                      void *stream);
 int aq_paged_attn_decode(const void *q, const void *k_cache, const void *v_cache,
-                         const int64_t *page_table, int64_t P, int64_t total_len, int64_t page_size,
+                         const int64_t *page_table, int64_t P, int64_t total_len,
+                         const int64_t *seq_lens, int64_t page_size,
                          int64_t n_pages, float scale, void *out, int64_t B, int64_t Hq, int64_t Hkv,
                          int64_t D, void *workspace, int64_t workspace_bytes, void *stream);
 int64_t aq_paged_attn_decode_workspace_bytes(int64_t B, int64_t Hq, int64_t Hkv, int64_t total_len);
@@ -235,7 +242,7 @@ int64_t aq_paged_attn_decode_workspace_bytes(int64_t B, int64_t Hq, int64_t Hkv,
  * aq_paged_attn_decode. */
 int aq_rope_paged_attn_decode(const void *qkv, const float *freqs, int64_t freqs_stride,
                               const int64_t *page_table, int64_t P, int64_t total_len,
-                              int64_t page_size, void *k_cache, void *v_cache, int64_t n_pages,
+                              const int64_t *seq_lens, int64_t page_size, void *k_cache, void *v_cache, int64_t n_pages,
                               float scale, void *out, int64_t B, int64_t Hq, int64_t Hkv, int64_t D,
                               void *workspace, int64_t workspace_bytes, void *stream);
 
@@ -261,12 +268,12 @@ int64_t aq_paged_attn_decode_slices(int64_t total_len);
 int64_t aq_paged_attn_decode_partials_bytes(int64_t B, int64_t Hq, int64_t total_len);
 int aq_paged_attn_decode_partials(const void *q, const void *k_cache, const void *v_cache,
                                   const int64_t *page_table, int64_t P, int64_t total_len,
-                                  int64_t page_size, int64_t n_pages, float scale, int64_t B,
+                                  const int64_t *seq_lens, int64_t page_size, int64_t n_pages, float scale, int64_t B,
                                   int64_t Hq, int64_t Hkv, int64_t D, void *partials,
                                   int64_t partials_bytes, void *stream);
 int aq_rope_paged_attn_decode_partials(const void *qkv, const float *freqs, int64_t freqs_stride,
                                        const int64_t *page_table, int64_t P, int64_t total_len,
-                                       int64_t page_size, void *k_cache, void *v_cache,
+                                       const int64_t *seq_lens, int64_t page_size, void *k_cache, void *v_cache,
                                        int64_t n_pages, float scale, int64_t B, int64_t Hq,
                                        int64_t Hkv, int64_t D, void *partials,
                                        int64_t partials_bytes, void *stream);

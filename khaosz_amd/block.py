@@ -83,7 +83,13 @@ class PagedKV:
     ``gather`` materialises ``[B, total_len, Hkv, D]`` through the table, zeros where unmapped.
     Which table entries are mapped is decided on a host copy of the table made at bind time,
     so neither method synchronises with the device (the reference tests the device tensor,
-    ``cache.py:233,262``) and both can be captured in a HIP graph."""
+    ``cache.py:233,262``) and both can be captured in a HIP graph.  That host copy is made when a
+    table tensor is first bound: a table that was changed in place (a page mapped as a sequence grew)
+    must be bound again with ``refresh=True`` -- or be a new tensor, as the reference's
+    ``make_table_tensor`` produces for every step.
+    ``seq_lens`` (int64 ``[B]`` on the device, optional): the positions each sequence may attend to
+    in a single-token step whose sequences sit at different positions; the attention kernels apply it as
+    the reference's position mask (transformer.py:40-46)."""
 
     def __init__(self, n_pages: int, page_size: int, n_kv_heads: int, head_dim: int, device, dtype,
                  n_layers: int = 1):
@@ -96,9 +102,11 @@ class PagedKV:
         self._safe = None        # device table with -1 replaced by 0
         self._invalid = None     # device bool [B, P * page_size] or None when everything is mapped
         self.total_len = 0
+        self.seq_lens: Optional[Tensor] = None
 
-    def bind(self, page_table: Optional[Tensor] = None, total_len: int = 0) -> "PagedKV":
-        if page_table is not None and page_table is not self.page_table:
+    def bind(self, page_table: Optional[Tensor] = None, total_len: int = 0, seq_lens: Optional[Tensor] = None,
+             refresh: bool = False) -> "PagedKV":
+        if page_table is not None and (refresh or page_table is not self.page_table):
             host = page_table.detach().cpu()
             self.page_table = page_table
             self._mapped = host >= 0
@@ -110,6 +118,7 @@ class PagedKV:
         if self.page_table is None:
             raise ValueError("bind() needs a page table")
         self.total_len = total_len
+        self.seq_lens = seq_lens
         return self
 
     def attn_workspace(self, n_heads: int) -> Optional[Tensor]:
@@ -261,7 +270,11 @@ class GQA(nn.Module):
         B, S, _ = x.shape
         if norm is not None and self._qkv is None:
             x, norm = F.rms_norm(x, (x.shape[-1],), norm[0], norm[1]), None
-        if (self._decode_attention and S == 1 and isinstance(cache, PagedKV) and x.is_cuda
+        # The paged decode kernels know two masks: none, and per-sequence lengths (``cache.seq_lens``).  Any
+        # mask TENSOR -- padding, or a caller's own -- goes to the stock attention below: the kernels would
+        # ignore it.  (A step whose sequences all sit at the same position needs no mask tensor at all; for
+        # different positions the caller binds ``seq_lens`` instead, as ``AutoRegressiveLM.forward`` does.)
+        if (self._decode_attention and S == 1 and attn_mask is None and isinstance(cache, PagedKV) and x.is_cuda
                 and x.dtype == torch.bfloat16):
             qkv = self._project_qkv(x, codes, norm)
             # the output projection combines the attention's position slices itself when the step is small
@@ -271,7 +284,8 @@ class GQA(nn.Module):
             out = ops.rope_paged_attn_decode(qkv.view(B, -1), rotary_emb.reshape(B, -1), cache.page_table,
                                              cache.total_len, cache.k_layers[self.layer_id],
                                              cache.v_layers[self.layer_id], self.n_heads, self.n_kv_heads,
-                                             workspace=cache.attn_workspace(self.n_heads), partials=split)
+                                             workspace=cache.attn_workspace(self.n_heads), partials=split,
+                                             seq_lens=cache.seq_lens)
             if split:
                 return self.o_proj.forward_attn(out, x.dtype, residual).view(B, 1, -1)
             return self._out(self._gated(out.view(B, 1, -1), x, norm, codes), residual)

@@ -99,6 +99,7 @@ struct AttnArgs {
   const uint16_t* kc;    // [n_pages, page, Hkv, D]
   const uint16_t* vc;
   const int64_t* table;  // [B, P]
+  const int64_t* lens;   // [B] positions each sequence may attend to (its own length), or null: all T
   uint16_t* out;         // [B, Hq, D]
   float* ws;             // partial results [B, Hq, NS, D + 4] when NS > 1
   const uint16_t* qkv;   // ROPE kernels: [B, (Hq + 2 Hkv) * D] projections of the new token (position T - 1)
@@ -115,6 +116,7 @@ constexpr int ATT_WAVES = 4;
 constexpr int ATT_KPW = 64;                  // positions per wavefront
 constexpr int ATT_KPG = ATT_WAVES * ATT_KPW; // positions per workgroup
 constexpr int ATT_MAX_D = 128;
+constexpr float ATT_MASKED = -1.0e30f;  // score (exp2 domain) of a cached position the sequence may not attend to
 
 // maximum / sum over each row of 16 consecutive lanes, result in all of them
 __device__ __forceinline__ float row16_max(float v) {
@@ -183,6 +185,14 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void paged_attn_decode_kernel(AttnA
   const int split = bs % p.NS, b = bs / p.NS;
   const int64_t T = p.T;
   const int64_t t0 = (int64_t)split * KPG + wave * KPW;  // first position of this wavefront
+  // A sequence shorter than T (a decode batch of sequences at different positions): positions from its own
+  // length on are masked, as the additive mask of the reference's forward does.  The mask value is finite, so
+  // a wavefront or slice whose positions are all masked leaves a partial result that later merges weigh with 0.
+  int64_t vis = T;
+  if (p.lens) {
+    const int64_t l = p.lens[b];
+    vis = l < T ? (l > 0 ? l : 0) : T;
+  }
 
   constexpr int KS = D / 32;                  // matrix-core steps over the head dimension
   const int col = lane & 15, kq = lane >> 4;  // operand row / column, group of 8 dimensions inside a step
@@ -312,7 +322,8 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void paged_attn_decode_kernel(AttnA
       float sv[4], mx = -INFINITY;
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
-        sv[t] = t0 + t * 16 + col < T ? sc[t][r] * p.scale_log2e : -INFINITY;
+        const int64_t pos = t0 + t * 16 + col;
+        sv[t] = pos < T ? (pos < vis ? sc[t][r] * p.scale_log2e : ATT_MASKED) : -INFINITY;
         mx = fmaxf(mx, sv[t]);
       }
       mx = row16_max(mx);  // finite: position t0 is valid
@@ -524,7 +535,8 @@ static void attn_launch(bool rope, dim3 grid, dim3 block, hipStream_t st, const 
 // q == nullptr: the fused form, queries and the new token come from qkv / freqs.
 // partials: stop after the slices' partial results (no merge launch, `out` unused).
 static int attn_decode(const void* q, const void* qkv, const float* freqs, int64_t freqs_stride, void* k_cache,
-                       void* v_cache, const int64_t* page_table, int64_t P, int64_t total_len, int64_t page_size,
+                       void* v_cache, const int64_t* page_table, int64_t P, int64_t total_len,
+                       const int64_t* seq_lens, int64_t page_size,
                        int64_t n_pages, float scale, void* out, int64_t B, int64_t Hq, int64_t Hkv, int64_t D,
                        void* workspace, int64_t workspace_bytes, void* stream, bool partials = false) {
   const bool rope = q == nullptr;
@@ -560,6 +572,7 @@ static int attn_decode(const void* q, const void* qkv, const float* freqs, int64
   a.kc_w = static_cast<uint16_t*>(k_cache);
   a.vc_w = static_cast<uint16_t*>(v_cache);
   a.table = page_table;
+  a.lens = seq_lens;
   a.out = partials ? nullptr : static_cast<uint16_t*>(out);
   a.ws = static_cast<float*>(workspace);
   a.P = P;
@@ -595,21 +608,23 @@ static int attn_decode(const void* q, const void* qkv, const float* freqs, int64
 }
 
 extern "C" int aq_paged_attn_decode(const void* q, const void* k_cache, const void* v_cache,
-                                    const int64_t* page_table, int64_t P, int64_t total_len, int64_t page_size,
+                                    const int64_t* page_table, int64_t P, int64_t total_len,
+                                    const int64_t* seq_lens, int64_t page_size,
                                     int64_t n_pages, float scale, void* out, int64_t B, int64_t Hq, int64_t Hkv,
                                     int64_t D, void* workspace, int64_t workspace_bytes, void* stream) {
   if (!q && B > 0) return AQ_E_NULL;
   return attn_decode(q, nullptr, nullptr, 0, const_cast<void*>(k_cache), const_cast<void*>(v_cache), page_table, P,
-                     total_len, page_size, n_pages, scale, out, B, Hq, Hkv, D, workspace, workspace_bytes, stream);
+                     total_len, seq_lens, page_size, n_pages, scale, out, B, Hq, Hkv, D, workspace, workspace_bytes, stream);
 }
 
 extern "C" int aq_rope_paged_attn_decode(const void* qkv, const float* freqs, int64_t freqs_stride,
-                                         const int64_t* page_table, int64_t P, int64_t total_len, int64_t page_size,
+                                         const int64_t* page_table, int64_t P, int64_t total_len,
+                                         const int64_t* seq_lens, int64_t page_size,
                                          void* k_cache, void* v_cache, int64_t n_pages, float scale, void* out,
                                          int64_t B, int64_t Hq, int64_t Hkv, int64_t D, void* workspace,
                                          int64_t workspace_bytes, void* stream) {
   if ((!qkv || !freqs) && B > 0) return AQ_E_NULL;
-  return attn_decode(nullptr, qkv, freqs, freqs_stride, k_cache, v_cache, page_table, P, total_len, page_size, n_pages,
+  return attn_decode(nullptr, qkv, freqs, freqs_stride, k_cache, v_cache, page_table, P, total_len, seq_lens, page_size, n_pages,
                      scale, out, B, Hq, Hkv, D, workspace, workspace_bytes, stream);
 }
 
@@ -622,21 +637,23 @@ extern "C" int64_t aq_paged_attn_decode_partials_bytes(int64_t B, int64_t Hq, in
 
 extern "C" int aq_paged_attn_decode_partials(const void* q, const void* k_cache, const void* v_cache,
                                              const int64_t* page_table, int64_t P, int64_t total_len,
+                                             const int64_t* seq_lens,
                                              int64_t page_size, int64_t n_pages, float scale, int64_t B, int64_t Hq,
                                              int64_t Hkv, int64_t D, void* partials, int64_t partials_bytes,
                                              void* stream) {
   if (!q && B > 0) return AQ_E_NULL;
   return attn_decode(q, nullptr, nullptr, 0, const_cast<void*>(k_cache), const_cast<void*>(v_cache), page_table, P,
-                     total_len, page_size, n_pages, scale, nullptr, B, Hq, Hkv, D, partials, partials_bytes, stream,
+                     total_len, seq_lens, page_size, n_pages, scale, nullptr, B, Hq, Hkv, D, partials, partials_bytes, stream,
                      true);
 }
 
 extern "C" int aq_rope_paged_attn_decode_partials(const void* qkv, const float* freqs, int64_t freqs_stride,
                                                   const int64_t* page_table, int64_t P, int64_t total_len,
+                                                  const int64_t* seq_lens,
                                                   int64_t page_size, void* k_cache, void* v_cache, int64_t n_pages,
                                                   float scale, int64_t B, int64_t Hq, int64_t Hkv, int64_t D,
                                                   void* partials, int64_t partials_bytes, void* stream) {
   if ((!qkv || !freqs) && B > 0) return AQ_E_NULL;
-  return attn_decode(nullptr, qkv, freqs, freqs_stride, k_cache, v_cache, page_table, P, total_len, page_size, n_pages,
+  return attn_decode(nullptr, qkv, freqs, freqs_stride, k_cache, v_cache, page_table, P, total_len, seq_lens, page_size, n_pages,
                      scale, nullptr, B, Hq, Hkv, D, partials, partials_bytes, stream, true);
 }

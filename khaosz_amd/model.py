@@ -125,7 +125,17 @@ class AutoRegressiveLM(nn.Module):
                                                            dtype=x.dtype).triu(1)
         else:
             rotary = self._freqs[position_ids]
-            mask = _attention_mask(x, position_ids, input_mask)
+            fused_step = (S == 1 and input_mask is None and isinstance(paged_cache, PagedKV) and x.is_cuda
+                          and x.dtype == torch.bfloat16
+                          and all(getattr(layer.attention, "_decode_attention", False) for layer in self.layers))
+            if fused_step:
+                # a decode step of sequences at possibly different positions (executor.py:59-94): the reference's
+                # mask lets sequence b attend to positions <= position_ids[b]; the paged kernels take that as
+                # per-sequence lengths, without a mask tensor and without reading the positions back to the host
+                mask = None
+                paged_cache.seq_lens = (position_ids[:, 0] + 1).to(torch.int64).contiguous()
+            else:
+                mask = _attention_mask(x, position_ids, input_mask)
         for layer in self.layers:
             x = layer(x, rotary, mask, paged_cache)
         hidden = self.norm(x)

@@ -411,11 +411,12 @@ def attn_gemv_fusable(B: int, n_heads: int, head_dim: int, total_len: int) -> bo
 def rope_paged_attn_decode(qkv: torch.Tensor, freqs: torch.Tensor, page_table: torch.Tensor, total_len: int,
                            k_cache: torch.Tensor, v_cache: torch.Tensor, n_heads: int, n_kv_heads: int,
                            scale: Optional[float] = None, workspace: Optional[torch.Tensor] = None,
-                           partials: bool = False):
+                           partials: bool = False, seq_lens: Optional[torch.Tensor] = None):
     """``rope_kv_write`` at position ``total_len - 1`` and ``paged_attn_decode`` over ``total_len``
     positions as one launch (plus the small merge launch for long sequences): same caches and
     outputs, bit for bit.  Returns the attention output ``[B, Hq, D]`` -- or, with ``partials``,
-    the slices' partial results (no merge launch) for ``gemv_w8a8_attn`` to combine."""
+    the slices' partial results (no merge launch) for ``gemv_w8a8_attn`` to combine.
+    ``seq_lens`` (int64 ``[B]`` on the device): sequence b attends to its first ``seq_lens[b]`` positions only."""
     if qkv.dim() != 2:
         raise ValueError(f"one new token per sequence: qkv must be [B, W], got {tuple(qkv.shape)}")
     qkv, fr, fr_stride, page_table = _rope_args(qkv, freqs, page_table, k_cache, v_cache, n_heads, n_kv_heads,
@@ -425,6 +426,7 @@ def rope_paged_attn_decode(qkv: torch.Tensor, freqs: torch.Tensor, page_table: t
         raise ValueError("total_len counts the new token: at least 1")
     lib = _abi.load()
     scale = float(scale if scale is not None else D ** -0.5)
+    lens_ptr = _seq_lens_ptr(seq_lens, B, qkv.device)
     if partials:
         if not B:
             raise ValueError("partial results need at least one sequence")
@@ -434,7 +436,7 @@ def rope_paged_attn_decode(qkv: torch.Tensor, freqs: torch.Tensor, page_table: t
             workspace = torch.empty(need // 4, dtype=torch.float32, device=qkv.device)
         with _OnDevice(qkv.device):
             rc = lib.aq_rope_paged_attn_decode_partials(qkv.data_ptr(), fr.data_ptr(), fr_stride, page_table.data_ptr(),
-                                                        page_table.shape[1], int(total_len), k_cache.shape[1],
+                                                        page_table.shape[1], int(total_len), lens_ptr, k_cache.shape[1],
                                                         k_cache.data_ptr(), v_cache.data_ptr(), k_cache.shape[0],
                                                         scale, B, n_heads, n_kv_heads, D, workspace.data_ptr(),
                                                         workspace.numel() * 4, _stream(qkv))
@@ -446,7 +448,7 @@ def rope_paged_attn_decode(qkv: torch.Tensor, freqs: torch.Tensor, page_table: t
                                            qkv.device)
         with _OnDevice(qkv.device):
             rc = lib.aq_rope_paged_attn_decode(qkv.data_ptr(), fr.data_ptr(), fr_stride, page_table.data_ptr(),
-                                               page_table.shape[1], int(total_len), k_cache.shape[1],
+                                               page_table.shape[1], int(total_len), lens_ptr, k_cache.shape[1],
                                                k_cache.data_ptr(), v_cache.data_ptr(), k_cache.shape[0], scale,
                                                out.data_ptr(), B, n_heads, n_kv_heads, D, ws_ptr, ws_bytes,
                                                _stream(qkv))
@@ -563,9 +565,17 @@ def paged_attn_partials_bytes(B: int, n_heads: int, total_len: int) -> int:
     return int(_abi.load().aq_paged_attn_decode_partials_bytes(B, n_heads, int(total_len)))
 
 
+def _seq_lens_ptr(seq_lens: Optional[torch.Tensor], B: int, device) -> Optional[int]:
+    if seq_lens is None:
+        return None
+    if seq_lens.dtype != torch.int64 or seq_lens.shape != (B,) or seq_lens.device != device or not seq_lens.is_contiguous():
+        raise ValueError(f"seq_lens must be a contiguous int64 [{B}] tensor on {device}")
+    return seq_lens.data_ptr()
+
+
 def paged_attn_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, page_table: torch.Tensor,
                       total_len: int, scale: Optional[float] = None,
-                      workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+                      workspace: Optional[torch.Tensor] = None, seq_lens: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``softmax(scale * q K^T) V`` for one query token per sequence over the first ``total_len``
     positions of each sequence's pages: ``q [B, Hq, D]`` -> ``[B, Hq, D]`` (bfloat16, D = 64 or 128).
     ``workspace``: a contiguous device tensor of at least ``paged_attn_workspace_bytes`` bytes
@@ -588,7 +598,7 @@ def paged_attn_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
         with _OnDevice(q.device):
             rc = _abi.load().aq_paged_attn_decode(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                                                   page_table.data_ptr(), page_table.shape[1], int(total_len),
-                                                  k_cache.shape[1], k_cache.shape[0],
+                                                  _seq_lens_ptr(seq_lens, B, q.device), k_cache.shape[1], k_cache.shape[0],
                                                   float(scale if scale is not None else D ** -0.5), out.data_ptr(),
                                                   B, Hq, Hkv, D, ws_ptr, ws_bytes, _stream(q))
         _abi.check(rc, "aq_paged_attn_decode")

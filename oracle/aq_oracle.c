@@ -364,10 +364,13 @@ void oq_rope_kv_write(const uint16_t *qkv, const float *freqs, const int64_t *ta
 
 /* out[b, h, :] = softmax_t(scale * q[b,h] . K[b,t,h/G]) V[b,t,h/G], t < T, read through
  * the page table; unmapped pages are zero keys and values (cache.py:254-274 zero
- * fill).  fp32, t and d ascending, libm expf. */
+ * fill).  lens (may be NULL): positions t >= lens[b] of sequence b carry the mask value that
+ * process_attention_mask (transformer.py:17-46) puts on positions past position_ids[b]
+ * (lens[b] = position_ids[b] + 1).  fp32, t and d ascending, libm expf. */
 void oq_paged_attn_decode(const uint16_t *q, const uint16_t *kc, const uint16_t *vc,
-                          const int64_t *table, int64_t P, int64_t T, int64_t page, int64_t n_pages,
-                          float scale, uint16_t *out, int64_t B, int64_t Hq, int64_t Hkv, int64_t D) {
+                          const int64_t *table, int64_t P, int64_t T, const int64_t *lens, int64_t page,
+                          int64_t n_pages, float scale, uint16_t *out, int64_t B, int64_t Hq, int64_t Hkv,
+                          int64_t D) {
   const int64_t G = Hq / Hkv;
 #pragma omp parallel for schedule(static) collapse(2)
   for (int64_t b = 0; b < B; ++b)
@@ -385,6 +388,9 @@ void oq_paged_attn_decode(const uint16_t *q, const uint16_t *kc, const uint16_t 
           for (int64_t i = 0; i < D; ++i) d += oq_bf16_to_f32(q[(b * Hq + h) * D + i]) * oq_bf16_to_f32(k[i]);
         }
         s[t] = d * scale;
+        /* a sequence shorter than T: the additive mask of transformer.py:40-46, -finfo(bfloat16).max / 2
+         * on every position past the sequence's own */
+        if (lens && t >= lens[b]) s[t] += -1.6947656946257676e38f;
         if (s[t] > m) m = s[t];
       }
       float l = 0.0f;

@@ -228,7 +228,7 @@ def _load():
     lib.oq_exp_repro.argtypes = [ctypes.c_float]
     lib.oq_exp_repro.restype = ctypes.c_float
     lib.oq_rope_kv_write.argtypes = [vp, vp, vp, i64, i64, i64, vp, vp, i64, vp, i64, i64, i64, i64]
-    lib.oq_paged_attn_decode.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, ctypes.c_float, vp, i64, i64, i64, i64]
+    lib.oq_paged_attn_decode.argtypes = [vp, vp, vp, vp, i64, i64, vp, i64, i64, ctypes.c_float, vp, i64, i64, i64, i64]
     lib.oq_prefill_attn_causal.argtypes = [vp, vp, vp, ctypes.c_float, vp, i64, i64, i64, i64, i64]
     lib.oq_prefill_attn_offset.argtypes = [vp, vp, vp, ctypes.c_float, vp, i64, i64, i64, i64, i64, i64]
     lib.oq_gemm_i8_i32.argtypes = [vp, vp, vp, i64, i64, i64]
@@ -339,13 +339,17 @@ def c_rope_kv_write(qkv, freqs, table, pos, kc, vc, Hq, Hkv):
     return q
 
 
-def c_paged_attn_decode(q, kc, vc, table, total_len, scale):
+def c_paged_attn_decode(q, kc, vc, table, total_len, scale, seq_lens=None):
+    """seq_lens [B] (optional): positions at and past seq_lens[b] are masked for sequence b as the reference's
+    position mask does (transformer.py:40-46)."""
     lib = _load()
     q, kc, vc, table = _c(q, np.uint16), _c(kc, np.uint16), _c(vc, np.uint16), _c(table, np.int64)
     B, Hq, D = q.shape
     n_pages, page, Hkv, _ = kc.shape
     out = np.empty((B, Hq, D), np.uint16)
-    lib.oq_paged_attn_decode(_p(q), _p(kc), _p(vc), _p(table), table.shape[1], total_len, page, n_pages,
+    lens = None if seq_lens is None else _c(seq_lens, np.int64)
+    lib.oq_paged_attn_decode(_p(q), _p(kc), _p(vc), _p(table), table.shape[1], total_len,
+                             None if lens is None else _p(lens), page, n_pages,
                              ctypes.c_float(scale), _p(out), B, Hq, Hkv, D)
     return out
 

@@ -104,6 +104,40 @@ def test_paged_attn_decode_within_bf16_rounding(oracle, B, Hq, Hkv, page, T, D):
     assert ((out - want).norm() / want.norm()).item() < 4e-3
 
 
+@pytest.mark.parametrize("B,Hq,Hkv,page,T,D,lens", [
+    (3, 4, 2, 16, 61, 64, [61, 1, 33]),
+    (4, 16, 4, 64, 700, 128, [700, 5, 256, 513]),       # three slices: one sequence ends inside the first, one on a boundary
+    (2, 8, 8, 32, 300, 128, [0, 299]),                  # nothing visible: the reference's uniform average
+])
+def test_paged_attn_decode_sequences_at_different_positions(oracle, B, Hq, Hkv, page, T, D, lens):
+    """seq_lens: sequence b attends to its first lens[b] positions (the reference's position mask for a decode
+    batch at mixed positions), against the oracle; slices that lie wholly past a sequence's length drop out of
+    the merge.  Both the plain kernel and the one that also rotates and writes the new token."""
+    _say("paged_attn_decode lens", B, Hq, Hkv, page, T, D, lens)
+    P = (T + page - 1) // page
+    n_pages = B * P + 2
+    g = torch.Generator().manual_seed(T + 1)
+    q = (torch.randn(B, Hq, D, generator=g) * 1.5).to(torch.bfloat16)
+    kc = torch.randn(n_pages, page, Hkv, D, generator=g).to(torch.bfloat16)
+    vc = torch.randn(n_pages, page, Hkv, D, generator=g).to(torch.bfloat16)
+    table = torch.randperm(n_pages, generator=g)[:B * P].view(B, P)
+    lens_t = torch.tensor(lens, dtype=torch.int64)
+    want = torch.from_numpy(oracle.c_paged_attn_decode(_bits(q), _bits(kc), _bits(vc), table.numpy(), T, D ** -0.5,
+                                                       seq_lens=lens_t.numpy()).view(np.int16)).view(torch.bfloat16).float()
+    out = ops.paged_attn_decode(q.to(DEV), kc.to(DEV), vc.to(DEV), table.to(DEV), T, seq_lens=lens_t.to(DEV)).cpu().float()
+    assert torch.allclose(out, want, rtol=1e-2, atol=1e-2)
+    assert ((out - want).norm() / want.norm()).item() < 4e-3
+    # the fused form (rotation + write of the new token at T - 1 + attention) against rope_kv_write + the plain kernel
+    qkv = torch.randn(B, (Hq + 2 * Hkv) * D, generator=g).to(torch.bfloat16).to(DEV)
+    ang = torch.rand(B, D // 2, generator=g) * 6.28
+    freqs = torch.polar(torch.ones_like(ang), ang).to(DEV)
+    k1, v1, k2, v2 = kc.to(DEV), vc.to(DEV), kc.to(DEV), vc.to(DEV)
+    q1 = ops.rope_kv_write(qkv, freqs, table.to(DEV), T - 1, k1, v1, Hq, Hkv)
+    a = ops.paged_attn_decode(q1.view(B, Hq, D), k1, v1, table.to(DEV), T, seq_lens=lens_t.to(DEV))
+    b = ops.rope_paged_attn_decode(qkv, freqs, table.to(DEV), T, k2, v2, Hq, Hkv, seq_lens=lens_t.to(DEV))
+    assert torch.equal(a, b) and torch.equal(k1, k2) and torch.equal(v1, v2)
+
+
 def test_paged_attn_workspace_reuse_and_checks(oracle):
     """A caller-owned workspace gives the same bits as a per-call one; a short one is refused."""
     _say("paged_attn_workspace")
@@ -125,8 +159,8 @@ def test_paged_attn_workspace_reuse_and_checks(oracle):
     assert torch.equal(a, b) and torch.equal(a, c)
     out = torch.empty_like(q)
     lib = _abi.load()
-    args = (q.data_ptr(), kc.data_ptr(), vc.data_ptr(), table.data_ptr(), P, T, page, B * P, D ** -0.5, out.data_ptr(),
-            B, Hq, Hkv, D)
+    args = (q.data_ptr(), kc.data_ptr(), vc.data_ptr(), table.data_ptr(), P, T, None, page, B * P, D ** -0.5,
+            out.data_ptr(), B, Hq, Hkv, D)
     assert lib.aq_paged_attn_decode(*args, ws.data_ptr(), need - 16, None) == -5    # AQ_E_WORKSPACE
     assert lib.aq_paged_attn_decode(*args, None, 0, None) == -1                  # AQ_E_NULL
     torch.cuda.synchronize()
@@ -265,10 +299,10 @@ def test_attention_partials_entry_points_check_their_arguments():
     q = torch.zeros(1, 2, 64, dtype=torch.bfloat16, device=DEV)
     kc = torch.zeros(2, 16, 1, 64, dtype=torch.bfloat16, device=DEV)
     tb = torch.zeros(1, 1, dtype=torch.int64, device=DEV)
-    rc = lib.aq_paged_attn_decode_partials(q.data_ptr(), kc.data_ptr(), kc.data_ptr(), tb.data_ptr(), 1, 10, 16, 2, 0.125,
+    rc = lib.aq_paged_attn_decode_partials(q.data_ptr(), kc.data_ptr(), kc.data_ptr(), tb.data_ptr(), 1, 10, None, 16, 2, 0.125,
                                            1, 2, 1, 64, None, 0, None)
     assert rc == -1                         # AQ_E_NULL
-    rc = lib.aq_paged_attn_decode_partials(q.data_ptr(), kc.data_ptr(), kc.data_ptr(), tb.data_ptr(), 1, 10, 16, 2, 0.125,
+    rc = lib.aq_paged_attn_decode_partials(q.data_ptr(), kc.data_ptr(), kc.data_ptr(), tb.data_ptr(), 1, 10, None, 16, 2, 0.125,
                                            1, 2, 1, 64, buf.data_ptr(), 64, None)
     assert rc == -5                         # AQ_E_WORKSPACE
 

@@ -139,3 +139,45 @@ def test_prompt_prefilled_in_two_chunks_matches_one_pass_on_the_quantized_fused_
         f(ids[:, :S1], paged_cache=cf.bind(table, S1))
         ref = f(ids[:, S1:], paged_cache=cf.bind(table, T), start_pos=S1)["logits"]
         assert rel(two, ref) < 6e-2
+
+
+@pytest.mark.gpu
+def test_decode_step_with_sequences_at_different_positions_follows_the_reference_mask():
+    """``position_ids`` of a decode batch at mixed positions, as execute_decode passes them
+    (executor.py:59-94): total_len is the largest position + 1, every new token lands in slot total_len - 1
+    and sequence b attends to positions <= position_ids[b] (transformer.py:40-46).  The quantized model with
+    the paged kernels (per-sequence lengths, no mask tensor, no host reads) must agree with the same quantized
+    model on the stock attention under the explicit mask tensor; a mask tensor given to the fused blocks sends
+    them to the stock attention too."""
+    dev, dt = "cuda:0", torch.bfloat16
+    cfg = LMConfig(vocab_size=512, dim=768, n_layers=2, n_heads=12, n_kv_heads=2, dim_ffn=2048, max_len=640)
+    torch.manual_seed(6)
+    a = AutoRegressiveLM(cfg).to(dev).to(dt).eval()
+    b = AutoRegressiveLM(cfg).to(dev).to(dt).eval()
+    b.load_state_dict(a.state_dict())
+    quantize_model(a), quantize_model(b)
+    fuse_shared_inputs(a, norms=True, residuals=True)                          # same fusions, torch attention
+    fuse_shared_inputs(b, norms=True, decode_attention=True, residuals=True)   # paged kernels
+    B, S, page = 3, 300, 64
+    P = (S + 2 + page - 1) // page
+    ids = torch.randint(0, 512, (B, S + 1), device=dev)
+    table = _table(B, P).to(dev)
+    ca, cb = a.new_cache(B * P, page), b.new_cache(B * P, page)
+
+    def rel(u, w):
+        return ((u.float() - w.float()).norm() / w.float().norm()).item()
+
+    with torch.inference_mode():
+        a(ids[:, :S], paged_cache=ca.bind(table, S))
+        b(ids[:, :S], paged_cache=cb.bind(table, S))
+        pos = torch.tensor([[S], [17], [S - 40]], device=dev)                 # three sequences, three positions
+        la = a(ids[:, S:], paged_cache=ca.bind(table, S + 1), position_ids=pos)["logits"]
+        lb = b(ids[:, S:], paged_cache=cb.bind(table, S + 1), position_ids=pos)["logits"]
+        assert cb.seq_lens is not None and cb.seq_lens.tolist() == [S + 1, 18, S - 39]
+        # every sequence on its own: W8A8 logits through two layers move by about 2 % when the attention
+        # numerics change (kernel against stock attention, also in the prefill that filled the caches)
+        for i in range(B):
+            assert rel(lb[i], la[i]) < 4e-2, i
+        # the short sequences must NOT see what the long one sees: same step without lengths differs for them
+        lc = b(ids[:, S:], paged_cache=cb.bind(table, S + 1), start_pos=S)["logits"]
+        assert rel(lc[0], lb[0]) < 2e-2 and rel(lc[1], lb[1]) > 5e-2

@@ -63,6 +63,37 @@ def test_paged_attention_matches_torch_sdpa(oracle):
     assert (out - ref).norm() / ref.norm() < 3e-3
 
 
+def test_paged_attention_with_sequence_lengths_matches_torch_under_the_position_mask(oracle):
+    """A decode batch whose sequences sit at different positions: the oracle's seq_lens against torch's attention
+    under the additive mask the reference builds from position_ids (transformer.py:40-46: 0 where
+    t <= position, -finfo.max / 2 elsewhere), and against the closed form for a sequence of length 1 (its
+    output is the first value row)."""
+    B, Hq, Hkv, D, page, n_pages, T = 3, 4, 2, 64, 16, 12, 61
+    g = torch.Generator().manual_seed(2)
+    q = torch.randn(B, Hq, D, generator=g).to(torch.bfloat16)
+    kc = torch.randn(n_pages, page, Hkv, D, generator=g).to(torch.bfloat16)
+    vc = torch.randn(n_pages, page, Hkv, D, generator=g).to(torch.bfloat16)
+    table = torch.tensor([[4, 0, 7, 2], [1, 8, 11, 3], [5, 9, 10, 6]])
+    lens = torch.tensor([61, 1, 33])
+    out = _bf16(oracle.c_paged_attn_decode(_bits(q), _bits(kc), _bits(vc), table.numpy(), T, D ** -0.5,
+                                           seq_lens=lens.numpy())).float()
+    k = kc[table].flatten(1, 2).float()[:, :T].repeat_interleave(Hq // Hkv, dim=2)
+    v = vc[table].flatten(1, 2).float()[:, :T].repeat_interleave(Hq // Hkv, dim=2)
+    pos = (lens - 1).view(B, 1)
+    attend = pos >= torch.arange(T)                                       # [B, T]
+    mask = torch.full((B, 1, 1, T), -torch.finfo(torch.bfloat16).max / 2).masked_fill_(attend.view(B, 1, 1, T), 0.0)
+    ref = F.scaled_dot_product_attention(q.float().unsqueeze(2), k.transpose(1, 2), v.transpose(1, 2), mask)[:, :, 0]
+    assert torch.allclose(out, ref, rtol=1e-2, atol=1e-2)
+    assert (out - ref).norm() / ref.norm() < 3e-3
+    first_v = vc[table[1, 0], 0].float().repeat_interleave(Hq // Hkv, dim=0)  # sequence 1 sees position 0 only
+    assert torch.equal(out[1], first_v)
+    # lengths equal to T change nothing
+    full = _bf16(oracle.c_paged_attn_decode(_bits(q), _bits(kc), _bits(vc), table.numpy(), T, D ** -0.5)).float()
+    same = _bf16(oracle.c_paged_attn_decode(_bits(q), _bits(kc), _bits(vc), table.numpy(), T, D ** -0.5,
+                                            seq_lens=np.full(B, T))).float()
+    assert torch.equal(full, same) and torch.equal(full[0], out[0])
+
+
 def test_prefill_attention_matches_torch_sdpa_and_closed_forms(oracle):
     """Causal attention over a prompt: against torch's scaled_dot_product_attention in fp32, with
     enable_gqa and with explicitly repeated KV heads (the reference's repeat_kv), and on inputs

@@ -76,7 +76,9 @@ class QuantLinear(Linear):
         self.register_buffer("qweight", torch.zeros((out_dim, in_dim), dtype=torch.int8, device=device))
         self.register_buffer("w_scale", torch.ones((out_dim,), dtype=torch.float32, device=device))
         self.bias = nn.Parameter(torch.zeros(out_dim, device=device), requires_grad=False) if bias else None
-        self._workspace: Optional[Tensor] = None
+        # decode workspaces (activation codes between the row quantiser and the GEMV), one per (device, stream):
+        # the same module called from two streams or threads must not share one
+        self._workspaces: dict = {}
 
     # -- construction -----------------------------------------------------
     @classmethod
@@ -176,10 +178,12 @@ class QuantLinear(Linear):
         if x2.dtype not in (torch.float32, torch.bfloat16):
             raise ValueError(f"activation dtype {x2.dtype} is not supported (float32 or bfloat16)")
         if M <= self.DECODE_MAX_ROWS:
+            ops._need_gpu(x, self.qweight)
             need = 16 * self.qweight.shape[1] + 512
-            ws = self._workspace
-            if ws is None or ws.device != x.device or ws.numel() < need:
-                ws = self._workspace = torch.empty((need,), dtype=torch.uint8, device=x.device)
+            key = (x.device, torch.cuda.current_stream(x.device).cuda_stream)
+            ws = self._workspaces.get(key)
+            if ws is None or ws.numel() < need:
+                ws = self._workspaces[key] = torch.empty((need,), dtype=torch.uint8, device=x.device)
             y = ops.gemv_w8a8_decode(x2, self.qweight, self.w_scale, self.bias, out_dtype=x.dtype, workspace=ws,
                                      residual=residual, norm=norm)
         else:
@@ -262,7 +266,12 @@ class Fp8Linear(Linear):
         return y.reshape(*lead, self.qweight.shape[0])
 
 
-TARGET_MODULES_ATTN = {"q_proj", "k_proj", "v_proj", "o_proj"}
+# Child names quantized by default: the projections of GQA (attention.py:57-67, `gate` is its optional output
+# gate), of MLA (attention.py:140-156: q_proj, kv_a_proj, kv_b_proj, o_proj, gate) and of every MLP, the experts of
+# DeepSeekMoE included (mlp.py:20-22,48-55).  Left in floating point unless named explicitly: `lm_head` (it may
+# alias the embedding, transformer.py:95-96) and DeepSeekMoE's `router` (mlp.py:48): its few outputs feed a top-k,
+# where int8 noise on near-equal logits changes which experts run, for under 0.1 % of a layer's weight bytes.
+TARGET_MODULES_ATTN = {"q_proj", "k_proj", "v_proj", "o_proj", "kv_a_proj", "kv_b_proj"}
 TARGET_MODULES_FFN = {"up", "gate", "down"}
 
 
@@ -336,6 +345,12 @@ def quantize_model(model: nn.Module, target_modules: Optional[Set[str]] = None, 
         parent_name, _, child_name = name.rpartition(".")
         seen.append(child_name)
         if child_name not in target_modules:
+            continue
+        if module.weight.shape[1] % 16:
+            # the kernels walk the reduction in 16-byte vectors; such a layer (the reference's dim-8 test
+            # models) stays in floating point rather than failing at its first call
+            logger.warning("Linear %s left in floating point: in_dim %d is not a multiple of 16", name,
+                           module.weight.shape[1])
             continue
         parent = model.get_submodule(parent_name) if parent_name else model
         setattr(parent, child_name, cls.from_linear(module))

@@ -145,5 +145,76 @@ def test_quantize_model_walks_like_inject_lora_and_skips_untargeted(monkeypatch)
         quantize_model(m, mode="int4")
 
 
+def _reference_linear_class():
+    """A class that looks, to code that never imports the reference, exactly like the reference's
+    own Linear (astrai/model/components/linear.py:7-21): same name, same module path, same attributes
+    and forward -- and no relation to this package's Linear."""
+
+    class RefLinear(nn.Module):
+        def __init__(self, in_dim, out_dim, bias=False):
+            super().__init__()
+            self.weight = nn.Parameter(torch.randn(out_dim, in_dim) * 0.05)
+            self.bias = nn.Parameter(torch.zeros(out_dim)) if bias else None
+
+        def forward(self, x):
+            return nn.functional.linear(x, self.weight, self.bias)
+
+    RefLinear.__name__ = RefLinear.__qualname__ = "Linear"
+    RefLinear.__module__ = "astrai.model.components.linear"
+    return RefLinear
+
+
+def test_the_reference_class_is_recognised_by_name_without_importing_it(monkeypatch):
+    from khaosz_amd.linear import _is_float_linear
+
+    Ref = _reference_linear_class()
+    assert not issubclass(Ref, Linear)
+    assert _is_float_linear(Ref(16, 8), ())
+    # the same class under another module path, or another name, is somebody else's layer
+    Other = _reference_linear_class()
+    Other.__module__ = "somewhere.else"
+    assert not _is_float_linear(Other(16, 8), ())
+    assert _is_float_linear(Other(16, 8), (Other,))  # unless the caller names its type
+    Renamed = _reference_linear_class()
+    Renamed.__name__ = "Dense"
+    assert not _is_float_linear(Renamed(16, 8), ())
+    assert not _is_float_linear(nn.Linear(16, 8), ())
+
+    made = []
+
+    def fake(cls, base):
+        made.append(base)
+        return QuantLinear(base.weight.shape[1], base.weight.shape[0], bias=base.bias is not None)
+
+    monkeypatch.setattr(QuantLinear, "from_linear", classmethod(fake))
+
+    class MLABlock(nn.Module):  # child names of the reference's MLA and DeepSeekMoE (attention.py:140-156, mlp.py:48-55)
+        def __init__(self):
+            super().__init__()
+            self.q_proj, self.kv_a_proj, self.kv_b_proj, self.o_proj = Ref(32, 48), Ref(32, 16), Ref(16, 96), Ref(32, 32)
+            self.router = Ref(32, 8)
+            self.routed_experts = nn.ModuleList([_RefMLP(Ref) for _ in range(2)])
+
+    class _Holder(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.attn = MLABlock()
+            self.up = Ref(8, 32)   # the reference's dim-8 test models: in_dim not a multiple of 16
+
+    m = _Holder()
+    n = quantize_model(m)
+    # q/kv_a/kv_b/o + 2 experts x (up, gate, down); router stays float by default, `up` with in_dim 8 is skipped
+    assert n == 4 + 6 and len(made) == n
+    assert type(m.attn.router) is Ref and type(m.up) is Ref
+    assert isinstance(m.attn.kv_a_proj, QuantLinear) and isinstance(m.attn.routed_experts[1].down, QuantLinear)
+    assert quantize_model(m, target_modules={"router"}) == 1 and isinstance(m.attn.router, QuantLinear)
+
+
+class _RefMLP(nn.Module):
+    def __init__(self, L):
+        super().__init__()
+        self.up, self.gate, self.down = L(32, 64), L(32, 64), L(64, 32)
+
+
 def test_package_exports():
     assert {"Linear", "QuantLinear", "Fp8Linear", "quantize_model"} <= set(dir(khaosz_amd))

@@ -546,3 +546,99 @@ def test_chunked_prefill_on_cached_tokens_uses_the_paged_kernel_and_tracks_the_m
             assert rel(yb, one[:, S1:]) < 1e-2
     finally:
         ops.prefill_attn_paged = real
+
+
+@pytest.mark.gpu
+def test_config5_full_size_fused_block_against_the_unfused_block_and_an_oracle_composition(oracle):
+    """Benchmark configuration 5 at its own size on the path the benchmark times: hidden 2048, 16 query /
+    4 KV heads of 128, FFN 5632, every fusion on, 8 x 512 prefill through a shuffled table of 64-token pages,
+    then decode steps of 8 tokens past 512 cached positions (position slices, merge inside o_proj).
+    (i) every step against the same weights in the unfused quantized block; (ii) one decode step against the
+    decoder block (decoder_block.py:43-59) composed on the CPU from the oracle's functions: the q/k/v
+    projection, the rotated queries and the cache contents bit for bit, everything behind the attention
+    within the stated bf16 tolerance, and the MLP half bit for bit on the attention half's own output."""
+    import numpy as np
+
+    from khaosz_amd import fuse_shared_inputs
+
+    def bits(t):
+        return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16).copy()
+
+    def from_bits(a):
+        return torch.from_numpy(np.ascontiguousarray(a).view(np.int16)).view(torch.bfloat16)
+
+    def add_bf16(a_bits, b_bits):  # the bits of a separate bf16 add
+        return bits((from_bits(a_bits).float() + from_bits(b_bits).float()).to(torch.bfloat16))
+
+    dev, dt = "cuda:0", torch.bfloat16
+    dim, Hq, Hkv, D, ffn, B, S, steps, page = 2048, 16, 4, 128, 5632, 8, 512, 4, 64
+    torch.manual_seed(55)
+    plain = DecoderBlock(dim, Hq, ffn, Hkv)
+    plain.reset_parameters()
+    with torch.no_grad():
+        plain.input_norm.weight.copy_(1 + 0.1 * torch.randn(dim))
+        plain.post_attention_norm.weight.copy_(1 + 0.1 * torch.randn(dim))
+    plain = plain.to(dev).to(dt)
+    fused = DecoderBlock(dim, Hq, ffn, Hkv).to(dev).to(dt)
+    fused.load_state_dict(plain.state_dict())
+    assert quantize_model(plain) == 7 and quantize_model(fused) == 7
+    fuse_shared_inputs(fused, norms=True, decode_attention=True, residuals=True)
+    assert fused._norm_quant and fused._residual_adds and fused.attention._decode_attention
+
+    P = (S + steps + page - 1) // page
+    n_pages = B * P + 5
+    table = torch.randperm(n_pages)[:B * P].view(B, P).to(dev)
+    ca, cb = PagedKV(n_pages, page, Hkv, D, dev, dt), PagedKV(n_pages, page, Hkv, D, dev, dt)
+    tab = rotary_table(D, 1024, device=dev)
+    x = torch.randn(B, S + steps, dim, device=dev).to(dt)
+    rel = lambda a, b: ((a.float() - b.float()).norm() / b.float().norm()).item()
+    att, mlp = fused.attention, fused.mlp
+    n1, n2 = fused.input_norm, fused.post_attention_norm
+    with torch.inference_mode():
+        pa = plain(x[:, :S], _freqs(tab, B, 0, S), None, ca.bind(table, S))
+        pb = fused(x[:, :S], _freqs(tab, B, 0, S), None, cb.bind(table, S))
+        assert rel(pb, pa) < 1e-2                      # stated bf16 tolerance
+        assert rel(cb.k, ca.k) < 1e-2 and rel(cb.v, ca.v) < 1e-2
+        for t in range(steps):
+            pos = S + t
+            xt, fr = x[:, pos:pos + 1], _freqs(tab, B, pos, 1)
+            da = plain(xt, fr, decode_mask(B, pos + 1, dev, dt), ca.bind(table, pos + 1))
+            if t == steps - 1:                         # state the oracle step starts from
+                k0, v0 = bits(cb.k), bits(cb.v)
+            db = fused(xt, fr, None, cb.bind(table, pos + 1))
+            assert db.shape == (B, 1, dim) and rel(db, da) < 1e-2, (t, rel(db, da))
+        # the last step once more in its two halves (an idempotent rewrite of the same cache slots)
+        h_gpu = att(xt, fr, None, cb.bind(table, pos + 1), norm=(n1.weight, n1.norm_eps), residual=xt)
+        out_gpu = mlp(h_gpu, norm=(n2.weight, n2.norm_eps), residual=h_gpu)
+        assert torch.equal(out_gpu, db)
+        qkv_gpu = att._qkv(xt, norm=(n1.weight, n1.norm_eps))
+
+    # ---- the same step on the CPU, from the oracle's functions
+    T = pos + 1
+    xb = bits(xt.reshape(B, dim))
+    qkv_w, qkv_s = att._qkv.qweight.cpu().numpy(), att._qkv.w_scale.cpu().numpy()
+    xq, sx = oracle.c_rmsnorm_quant_i8(xb, bits(n1.weight), n1.norm_eps, bf16_bits=True)
+    qkv = oracle.c_dequant_epilogue(oracle.c_gemm_i8_i32(xq, qkv_w), sx, qkv_s, bf16_out=True)
+    assert np.array_equal(bits(qkv_gpu.reshape(B, -1)), qkv)                      # bit for bit
+    fr_np = np.ascontiguousarray(torch.view_as_real(fr.reshape(B, D // 2)).cpu().numpy())
+    q_rot = oracle.c_rope_kv_write(qkv, fr_np, table.cpu().numpy(), pos, k0, v0, Hq, Hkv)
+    assert np.array_equal(bits(cb.k), k0) and np.array_equal(bits(cb.v), v0)      # the cache after the step, bit for bit
+    attn = oracle.c_paged_attn_decode(q_rot, k0, v0, table.cpu().numpy(), T, D ** -0.5)
+    o = oracle.c_linear_w8a8(attn.reshape(B, Hq * D), att.o_proj.qweight.cpu().numpy(), att.o_proj.w_scale.cpu().numpy(),
+                             x_bf16_bits=True, bf16_out=True)
+    h = add_bf16(o, xb)
+    assert rel(h_gpu.reshape(B, dim).cpu(), from_bits(h)) < 1e-2                  # behind the attention: stated tolerance
+
+    def mlp_half(h_bits):
+        hq, hs = oracle.c_rmsnorm_quant_i8(h_bits, bits(n2.weight), n2.norm_eps, bf16_bits=True)
+        ug = oracle.c_dequant_epilogue(oracle.c_gemm_i8_i32(hq, mlp._upgate.qweight.cpu().numpy()), hs,
+                                       mlp._upgate.w_scale.cpu().numpy(), bf16_out=True)
+        aq, asc = oracle.c_swiglu_quant_i8(ug, bf16_bits=True)
+        d = oracle.c_dequant_epilogue(oracle.c_gemm_i8_i32(aq, mlp.down.qweight.cpu().numpy()), asc,
+                                      mlp.down.w_scale.cpu().numpy(), bf16_out=True)
+        return add_bf16(d, h_bits)
+
+    assert rel(out_gpu.reshape(B, dim).cpu(), from_bits(mlp_half(h))) < 1e-2      # whole step, oracle end to end
+    # the MLP half on the bits the GPU's attention half produced: norm + quantise, up/gate, SwiGLU + quantise,
+    # down and the residual add, bit for bit
+    assert np.array_equal(bits(out_gpu.reshape(B, dim)), mlp_half(bits(h_gpu.reshape(B, dim))))

@@ -31,7 +31,11 @@ namespace aq {
 //                            K step and exchange half of their accumulators through LDS at the end, so that
 //                            each finishes (and stores) 32 x 64 of the sums; 4 stages of 32 KiB;
 // Shapes that only the lab build instantiates (measured, none faster: under a matrix-core load with real
-// operand data this part runs against its power limit, and fewer LDS reads per MFMA buy clock, not rate):
+// operand data this part runs against its power limit, and fewer LDS reads per MFMA buy clock, not rate;
+// with one wavefront per SIMD every fragment read also delays that SIMD's next MFMA, which a second
+// wavefront otherwise covers.  Two independent 4-wavefront workgroups per compute unit, 256 x 128 or
+// 128 x 128 tiles with 64-byte stages, were measured too: 8192^3 in 459 and 556 us against 310 us with
+// all-zero operands):
 //   <2, 2, 4, 4, 1, 64, 4>   256 x 256 tile, 4 wavefronts (one per SIMD) of 128 x 128: 256 accumulator
 //                            registers per lane (the AGPR half of the register file), 8 fragment reads per
 //                            16 MFMAs instead of 16, half the LDS fill per MFMA; 4 stages of 32 KiB;
@@ -155,6 +159,9 @@ __device__ __forceinline__ void sched_pattern() {
   }
 }
 
+#ifdef AQ_LAB
+__device__ long long aq_lab_clock[4];
+#endif
 template <bool FP8, int OUT, class S>
 __device__ __forceinline__ void gemm_tile(const GemmArgs& p, uint8_t* smem, int pid) {
   constexpr int WM = S::WM, WN = S::WN, TM = S::TM, TN = S::TN, WK = S::WK, BK = S::BK, NSTAGE = S::NSTAGE;
@@ -428,14 +435,26 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, uint8_t* smem, int 
   // slot A of stage 0: its buffer (0) is free now and takes stage NSTAGE
   slot(last_of(k0{}), smem + STAGE, 0, yes{}, NSTAGE, 0, q0{});
   int b_prev = 0;  // buffer of stage s-1
+#ifdef AQ_LAB_STALL
+  long long st_t0 = 0, st_t1 = 0, st_sum = 0;
+  const long long st_begin = clock64();
+#endif
   auto stage = [&](int s, auto c0_c) {
     const int b_cur = b_prev == NSTAGE - 1 ? 0 : b_prev + 1;
     const int b_next = b_cur == NSTAGE - 1 ? 0 : b_cur + 1;
     // sub-steps 0 .. NKS-2 of stage s; the rest of stage s-1+NSTAGE's loads go into stage s-1's buffer
     middle_slots(c0_c, smem + b_cur * STAGE, yes{}, s - 1 + NSTAGE, b_prev);
+#ifdef AQ_LAB_STALL
+    const long long st_now = clock64();
+#endif
     __builtin_amdgcn_s_waitcnt(0xc07f);        // lgkmcnt(0): the last fragments of stage s are in registers
     AQ_WAIT_VMCNT((NSTAGE - 2) * NLOADS);  // stage s+1 has landed (later ones may still be in flight)
     AQ_BARRIER();
+#ifdef AQ_LAB_STALL
+    st_sum += st_t1 - st_t0;  // the previous step's wait: both of its clock reads have returned by now
+    st_t0 = st_now;
+    st_t1 = clock64();
+#endif
     // slot A: last sub-step of stage s | first fragments of stage s+1 | first loads of stage s+NSTAGE
     slot(last_of(c0_c), smem + b_next * STAGE, 0, yes{}, s + NSTAGE, b_cur, q0{});
     b_prev = b_cur;
@@ -451,6 +470,12 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, uint8_t* smem, int 
     if (s < nk) stage(s, k1{});
   }
   AQ_WAIT_VMCNT(0);  // drain the padding loads before the workgroup's LDS can be released or reused
+#ifdef AQ_LAB_STALL
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    aq_lab_clock[2] = st_sum + (st_t1 - st_t0);
+    aq_lab_clock[3] = clock64() - st_begin;
+  }
+#endif
 
   if constexpr (WK == 2) {
     // The two wavefronts of a sub-tile hold the sums over their halves of every K step.  Each
@@ -650,9 +675,6 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, uint8_t* smem, int 
 
 // A workgroup walks tiles pid, pid + gridDim.x, ...: with more tiles than compute units the launch is one
 // resident workgroup per compute unit instead of a queue of short-lived ones (the LDS stages allow one at a time).
-#ifdef AQ_LAB
-__device__ long long aq_lab_clock[4];
-#endif
 template <bool FP8, int OUT, class S>
 __global__ __launch_bounds__(S::NTHREADS) void gemm_kernel(GemmArgs p) {
   __shared__ __attribute__((aligned(1024))) uint8_t smem[S::LDS_BYTES];
@@ -750,7 +772,7 @@ static GemmArgs make_args(const void* A, const void* B, void* C, int64_t M, int6
 
 #ifdef AQ_LAB
 extern "C" int aq_lab_read_clock(long long* host2) {
-  return (int)hipMemcpyFromSymbol(host2, HIP_SYMBOL(aq::aq_lab_clock), 16);
+  return (int)hipMemcpyFromSymbol(host2, HIP_SYMBOL(aq::aq_lab_clock), 32);
 }
 extern "C" int aq_lab_set_gemm_tile(int rows) {
   if (rows != 0 && rows != 128 && rows != 256 && rows != 257 && rows != 512 && rows != 513) return AQ_E_SHAPE;

@@ -410,8 +410,13 @@ constexpr int GM_BATCH = 8;    // MFMA steps (64 K bytes each) per register batc
 // compiler drain the weight loads at the join, 0.4 us of a 6.5 us launch).
 // XR: rounds of token-code vectors (8 per thread each) requested ahead of the weight stream; rows too long for
 // XR rounds copy the rest afterwards, which waits for the weight loads in flight.
-template <int KS, int GR, bool RES, int XR>
+// FQ > 0: the kernel quantises up to FQ (8 or 16) bf16 token rows of at most 2048 elements itself, one or two
+// rows per wavefront of a KS x GR = 8 wavefront workgroup, while its weight loads are in flight (the row
+// arithmetic of the stand-alone quantiser, shared through aq_rows.h: same codes and scales); NORM: after
+// RMS-normalising them with the gain p.gamma.  One launch per decode step instead of two.
+template <int KS, int GR, bool RES, int XR, int FQ = 0, bool NORM = false>
 __global__ __launch_bounds__(GM_MAX_WAVES * 64) void gemv_mfma_kernel(GemvArgs p) {
+  static_assert(FQ == 0 || (KS > 0 && GR > 0), "the in-kernel quantiser deals rows to a fixed number of wavefronts");
   extern __shared__ __attribute__((aligned(16))) uint8_t xs[];  // [16][K + 16] token codes, [16] scales, 16 spare bytes; later the partial sums
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -432,8 +437,8 @@ __global__ __launch_bounds__(GM_MAX_WAVES * 64) void gemv_mfma_kernel(GemvArgs p
   // only the first K part's wavefront writes outputs: the others get empty descriptors.  Requested first:
   // measured 0.2 us faster than behind the weight stream (loads return in request order, and these few come
   // back quickly, while behind the weights the epilogue would wait for the whole stream to drain).
-  const EpiOperands epi(p, kh == 0, true, RES);
-  const float sxv = epi.load_sx(tok, tok < M);
+  const EpiOperands epi(p, kh == 0, FQ == 0, RES);
+  float sxv = epi.load_sx(tok, tok < M);
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
     const int n = rbase + r;
@@ -468,7 +473,21 @@ __global__ __launch_bounds__(GM_MAX_WAVES * 64) void gemv_mfma_kernel(GemvArgs p
   // token codes -> LDS (padded rows; tokens >= M are zero).  Their loads are
   // issued before the weight loads, so they return first and the LDS fill
   // overlaps the weight stream's flight time.
-  {
+  float* const sx_lds = reinterpret_cast<float*>(xs + 16 * pitch);
+  if constexpr (FQ > 0) {
+    // produced here: every wavefront requests its bf16 rows, then its weights, then rounds the rows while the
+    // weights are in flight.  Rows >= M are not written: the lanes of those tokens read row 0 and their
+    // products are never stored.
+    constexpr int WAVES = KS * GR, RPW = (FQ + WAVES - 1) / WAVES;
+    RowsToLds<true, RPW, 4> xrows;
+    xrows.issue(p.x, M, K, K, wave, WAVES, lane);
+    if constexpr (NORM) xrows.issue_gamma(p.gamma, K, lane);
+    asm volatile("" ::: "memory");  // request order: token rows, then the weight stream
+    wload(0, wa);
+    wload(GM_LINES, wb);
+    asm volatile("" ::: "memory");
+    xrows.template finish<NORM>(M, M, K, xs, pitch, sx_lds, wave, WAVES, lane, p.eps);
+  } else {
     const __amdgpu_buffer_rsrc_t Xr = make_rsrc(p.xq, (uint32_t)M * (uint32_t)K);
     const int nvec_row = K / 16;
     const int nvec = 16 * nvec_row;
@@ -512,6 +531,7 @@ __global__ __launch_bounds__(GM_MAX_WAVES * 64) void gemv_mfma_kernel(GemvArgs p
   asm volatile("" ::: "memory");
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
+  if constexpr (FQ > 0) sxv = sx_lds[tok < M ? tok : 0];
 
   // Four independent accumulators (summed at the end: int32, exact in any order) and a batch's token
   // fragments read from LDS up front: one chain of 16 dependent read -> MFMA steps took 0.6 us after the
@@ -525,7 +545,7 @@ __global__ __launch_bounds__(GM_MAX_WAVES * 64) void gemv_mfma_kernel(GemvArgs p
   // row l % 8 (register lo) and of row 8 + l % 8 (register hi), so lanes 0..7 of each row of 16 lanes have
   // their operand of step e = 0 in lo, and lanes 8..15 find theirs in hi of lane l - 8; for e = 1 it is lo of
   // lane l + 8 and the own hi: one rotation by 8 within the row of 16 lanes, written into half of the lanes.
-  const uint8_t* xl = xs + tok * pitch + kh * khalf + (lane >> 4) * 32;
+  const uint8_t* xl = xs + (FQ > 0 && tok >= M ? 0 : tok) * pitch + kh * khalf + (lane >> 4) * 32;
   auto consume = [&](int line0, const uint4 (&wc)[GM_BATCH]) {
     v4i x[GM_BATCH];
 #pragma unroll
@@ -642,6 +662,40 @@ static int launch_gemv_mfma(GemvArgs a, hipStream_t st) {
   return (int)hipGetLastError();
 }
 
+// The matrix-core variant that quantises its token rows itself (8 wavefronts per workgroup, a row -- two above
+// 8 tokens -- per wavefront), where it measured faster than the alternatives (bf16 rows of K = 2048, one launch):
+//   9..16 tokens: always (N = 8192: 7.6 us against 8.4 us for row quantiser + GEMV; N = 2048: 6.6 against 7.1);
+//   5..8 tokens: from N = 8192 on (6.45 us against 7.4 us for the dot-product kernel, which is bound by its
+//                vector ALU there; at N = 4096 the dot-product kernel still wins, 4.8 against 5.2 us);
+//   3..4 tokens: only for matrices with more 32-row blocks than compute units (N = 11264: 7.0 against 7.6 us).
+static bool gemv_mfma_fq_ok(int64_t M, int64_t N, int64_t K) {
+  if (K > 2048 || (K % 512) != 0) return false;
+  const bool wide = (N + 31) / 32 > device_cus();
+  return M >= 9 || (M >= 5 && N >= 8192) || (M >= 3 && wide);
+}
+
+static int launch_gemv_mfma_fq(GemvArgs a, hipStream_t st) {
+  // 32 weight rows per workgroup (2 row groups x 4 K parts) while that gives every workgroup a compute unit
+  // of its own; beyond that 64 rows (4 row groups x 2 K parts): a second round of workgroups would repeat
+  // the row quantisation behind the first (N = 11264, 8 tokens: 9.9 -> 7.1 us).
+  const bool wide = (a.N + 31) / 32 > device_cus();
+  a.ksplit = wide ? 2 : 4;
+  a.groups = wide ? 4 : 2;
+  const unsigned grid = (unsigned)((a.N + GM_ROWS * a.groups - 1) / (GM_ROWS * a.groups));
+  const size_t lds = (size_t)16 * (a.K + 16) + 16 * sizeof(float) + 16;
+  const bool res = a.res != nullptr, many = a.M > 8, norm = a.gamma != nullptr;
+  using kern_t = void (*)(GemvArgs);
+#define AQ_FQ_TABLE(KS, GR)                                                                                  \
+  {{{gemv_mfma_kernel<KS, GR, false, 1, 8, false>, gemv_mfma_kernel<KS, GR, false, 1, 8, true>},             \
+    {gemv_mfma_kernel<KS, GR, false, 1, 16, false>, gemv_mfma_kernel<KS, GR, false, 1, 16, true>}},          \
+   {{gemv_mfma_kernel<KS, GR, true, 1, 8, false>, gemv_mfma_kernel<KS, GR, true, 1, 8, true>},               \
+    {gemv_mfma_kernel<KS, GR, true, 1, 16, false>, gemv_mfma_kernel<KS, GR, true, 1, 16, true>}}}
+  static const kern_t table[2][2][2][2] = {AQ_FQ_TABLE(4, 2), AQ_FQ_TABLE(2, 4)};
+#undef AQ_FQ_TABLE
+  hipLaunchKernelGGL(table[wide][res][many][norm], dim3(grid), dim3(8 * 64), lds, st, a);
+  return (int)hipGetLastError();
+}
+
 static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 }  // namespace aq
@@ -686,6 +740,7 @@ static int gemv_dispatch(const aq::GemvArgs& a, int mt, hipStream_t st) {
 // than 8 rows every workgroup would repeat 2+ row quantisations per wavefront
 // on its critical path, which measures no faster than the separate launch.
 static int gemv_dispatch_fused(const aq::GemvArgs& a, int mt, hipStream_t st) {
+  if (aq::gemv_mfma_fq_ok(a.M, a.N, a.K)) return aq::launch_gemv_mfma_fq(a, st);
   const int64_t vpl = (a.K / 8 + 63) / 64;  // 16-byte vectors per lane per bf16 row
   if (mt > 8 || vpl > 16) return -1;
   const bool small = vpl <= 4;

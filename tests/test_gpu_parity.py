@@ -339,8 +339,11 @@ def test_linear_residual_may_alias_the_output(tile):
 # ------------------------------------------------------------------- decode
 
 @pytest.mark.parametrize("M", [1, 2, 3, 4, 5, 8, 11, 16])
-@pytest.mark.parametrize("N,K", [(8192, 2048), (50, 16), (130, 1040), (2048, 5632)])
+@pytest.mark.parametrize("N,K", [(8192, 2048), (50, 16), (130, 1040), (2048, 5632), (11264, 2048), (8200, 512), (77, 1536)])
 def test_gemv_decode_bit_exact(oracle, M, N, K):
+    """(11264, 2048), (8200, 512) and 9+ rows of (77, 1536) take the matrix-core kernel that quantises its rows
+    itself: 64-row workgroups on the first (more 32-row blocks than compute units), a ragged last block on the
+    second, a single partly filled workgroup on the third."""
     _say("gemv", M, N, K)
     x = make_x(M, K, 11 + M).to(torch.bfloat16)
     w = make_x(N, K, 12) * 0.02
@@ -358,8 +361,8 @@ def test_gemv_decode_bit_exact(oracle, M, N, K):
         assert torch.equal(y2, y + r)
 
 
-@pytest.mark.parametrize("M", [1, 3, 4, 8, 12])
-@pytest.mark.parametrize("N,K", [(3072, 2048), (130, 1536), (2048, 4096), (50, 16)])
+@pytest.mark.parametrize("M", [1, 3, 4, 8, 12, 16])
+@pytest.mark.parametrize("N,K", [(3072, 2048), (130, 1536), (2048, 4096), (50, 16), (11264, 2048), (8192, 1024)])
 def test_gemv_with_the_norm_folded_in_equals_norm_quantise_then_gemv(oracle, M, N, K):
     """RMSNorm inside the decode GEMV (one launch for M <= 8, K <= 2048; two launches through the
     workspace otherwise): the codes are those of the stand-alone norm-and-quantise kernel, which is

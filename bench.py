@@ -35,14 +35,29 @@ PEAK_HBM_GBS = 8000.0        # MI355X HBM3E, published
 PEAK_INT8_TOPS = 5000.0      # dense int8 MFMA, published (no sparsity)
 PEAK_FP8_TFLOPS = 5000.0     # dense FP8 MFMA, published
 
-# Bytes per launch that the dominant kernel moves past the L2 (FETCH_SIZE + WRITE_SIZE from two
-# rocprofv3 --pmc runs of this script, each scaled by what the same counter reads for kernels of
-# known size in the same run: 2048 B per FETCH_SIZE unit, 1024 B per WRITE_SIZE unit).
-MEASURED_TRAFFIC = {
-    "decode": {1: 16.87e6 + 0.02e6, 4: 16.96e6 + 0.07e6, 16: 17.19e6 + 0.26e6},
-    "prefill": 33.76e6 + 16.80e6,  # the fetch side is L2 fills by 8 XCDs (12.58 MB of distinct input)
-    "fp8": 100.76e6 + 8.39e6,
-}
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic_fetch_write_size.txt")
+
+
+def measured_traffic(key):
+    """Bytes per launch that the dominant kernel of workload `key` moves past the L2: FETCH_SIZE + WRITE_SIZE of
+    two rocprofv3 --pmc runs of this script, scaled by what the same counters read for kernels of known size.
+    Counters cannot be read from inside a timed run, so the figure comes from the committed summary of those runs
+    (its `traffic` lines), which names the kernel's source file and that file's SHA-256 at the time of the
+    measurement: when the source has changed since, the figure is stale and None is reported instead."""
+    import hashlib
+
+    try:
+        for line in open(TRAFFIC_FILE):
+            f = line.split()
+            if len(f) >= 2 and f[0] == "traffic" and f[1] == key:
+                kv = dict(x.split("=", 1) for x in f[2:])
+                src = os.path.join(ROOT, kv["source"])
+                if hashlib.sha256(open(src, "rb").read()).hexdigest() != kv["sha256"]:
+                    return None, f"stale: {kv['source']} changed since the counters were read"
+                return float(kv["fetch_bytes"]) + float(kv["write_bytes"]), f"{os.path.basename(TRAFFIC_FILE)}: {kv['kernel']}"
+    except (OSError, KeyError, ValueError) as e:
+        return None, f"unreadable: {e}"
+    return None, "no counter run recorded for this workload"
 
 
 def parse():
@@ -140,6 +155,9 @@ def bench_decode(torch, ops, args, dev):
         wq, sw = weights[0]
         ys[0] = ops.gemv_w8a8_codes(xq, sx, wq, sw, None, out_dtype=torch.bfloat16)
 
+    # The step is ONE launch: the GEMV kernel quantises its token rows itself (dot-product kernel up to 4 rows,
+    # matrix-core kernel from 5 rows on at this N), so the step's time is the dominant kernel's duration.
+    # Bytes: the weight once, its scales, the bf16 rows in, the bf16 outputs.
     bytes_alg = N * K + 4 * N + 2 * M * K + 2 * M * N
     d_step, d_k = [], []
     ms = graph_time_ms(torch, step, args.steps, args.warmup, d_step)
@@ -147,16 +165,22 @@ def bench_decode(torch, ops, args, dev):
     ms_k = graph_time_ms(torch, kernel_only, args.steps, args.warmup, d_k)
     ms_res = graph_time_ms(torch, resident, args.steps, args.warmup)
     gbs = bytes_alg / (ms * 1e-3) / 1e9
-    gbs_k = bytes_alg / (ms_k * 1e-3) / 1e9
+    traffic, traffic_src = measured_traffic(f"decode_m{M}")
     return {
         "workload": f"decode_gemv_w8a8 M={M} K={K} N={N} bf16->int8 per-token, W int8 per-channel, bf16 out",
         "value": gbs, "unit": "GB/s", "ms_per_step": ms, "eager_ms_per_step": ms_eager,
         "ms_per_step_p10_p50_p90": d_step, "bytes_per_step": bytes_alg, "dtype": "int8",
-        "roofline": {"bound": "hbm", "kernel": "gemv_mfma_kernel" if M > 8 else "gemv_w8a8_kernel", "achieved": gbs_k, "peak": PEAK_HBM_GBS,
-                     "unit": "GB/s", "frac": gbs_k / PEAK_HBM_GBS, "traffic": MEASURED_TRAFFIC["decode"].get(M),
-                     "kernel_us": ms_k * 1e3, "kernel_us_p10_p50_p90": [v * 1e3 for v in d_k],
-                     "algorithmic_bytes": bytes_alg,
-                     "llc_resident_gbs": bytes_alg / (ms_res * 1e-3) / 1e9, "weight_buffers": nbuf},
+        "roofline": {"bound": "hbm", "kernel": ("gemv_mfma_kernel<.., FQ>" if M > 4 else "gemv_w8a8_kernel<.., FUSED>")
+                     + " (quantises its rows itself: the whole step)",
+                     "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
+                     "traffic": traffic, "traffic_source": traffic_src,
+                     "kernel_us": ms * 1e3, "kernel_us_p10_p50_p90": [v * 1e3 for v in d_step],
+                     "algorithmic_bytes": bytes_alg, "weight_buffers": nbuf,
+                     # the same GEMV on codes that a separate launch (or a producer kernel) has already made
+                     "gemv_on_codes": {"kernel_us": ms_k * 1e3, "kernel_us_p10_p50_p90": [v * 1e3 for v in d_k],
+                                       "gbs": (bytes_alg - M * K) / (ms_k * 1e-3) / 1e9,
+                                       "frac": (bytes_alg - M * K) / (ms_k * 1e-3) / 1e9 / PEAK_HBM_GBS,
+                                       "llc_resident_gbs": (bytes_alg - M * K) / (ms_res * 1e-3) / 1e9}},
         "shape": (M, N, K),
     }
 
@@ -204,13 +228,14 @@ def bench_prefill(torch, ops, args, dev):
     ms_nq = graph_time_ms(torch, norm_quant_only, steps, args.warmup)
     tops = ops_alg / (ms * 1e-3) / 1e12
     tops_k = ops_alg / (ms_k * 1e-3) / 1e12
+    traffic, traffic_src = measured_traffic("prefill")
     qbytes = 2 * M * K + M * K + 4 * M
     return {
         "workload": f"prefill_linear_w8a8 M={M} K={K} N={N} quantise + int8 MFMA GEMM + scale/bias epilogue, bf16 out",
         "value": tops, "unit": "TOPS", "ms_per_step": ms, "ms_per_step_p10_p50_p90": d_step, "ops_per_step": ops_alg,
         "dtype": "int8",
         "roofline": {"bound": "mfma", "kernel": "gemm_kernel<int8,bf16>", "achieved": tops_k, "peak": PEAK_INT8_TOPS,
-                     "unit": "TOP/s", "frac": tops_k / PEAK_INT8_TOPS, "traffic": MEASURED_TRAFFIC["prefill"],
+                     "unit": "TOP/s", "frac": tops_k / PEAK_INT8_TOPS, "traffic": traffic, "traffic_source": traffic_src,
                      "kernel_us": ms_k * 1e3, "kernel_us_p10_p50_p90": [v * 1e3 for v in d_k],
                      "algorithmic_ops": ops_alg},
         "quantise_kernel": {"us": ms_q * 1e3, "gbs": qbytes / (ms_q * 1e-3) / 1e9, "frac_hbm": qbytes / (ms_q * 1e-3) / 1e9 / PEAK_HBM_GBS,
@@ -247,11 +272,12 @@ def bench_fp8(torch, ops, args, dev):
     ms_k = graph_time_ms(torch, kernel_only, steps, args.warmup)
     t = flops / (ms * 1e-3) / 1e12
     tk = flops / (ms_k * 1e-3) / 1e12
+    traffic, traffic_src = measured_traffic("fp8")
     return {
         "workload": f"fp8_linear M={M} K={K} N={N} per-tensor e4m3 quantise + FP8 MFMA GEMM, bf16 out",
         "value": t, "unit": "TFLOP/s", "ms_per_step": ms, "flops_per_step": flops, "dtype": "fp8_e4m3",
         "roofline": {"bound": "mfma", "kernel": "gemm_kernel<fp8,bf16>", "achieved": tk, "peak": PEAK_FP8_TFLOPS,
-                     "unit": "TFLOP/s", "frac": tk / PEAK_FP8_TFLOPS, "traffic": MEASURED_TRAFFIC["fp8"],
+                     "unit": "TFLOP/s", "frac": tk / PEAK_FP8_TFLOPS, "traffic": traffic, "traffic_source": traffic_src,
                      "kernel_us": ms_k * 1e3, "algorithmic_flops": flops},
         "shape": (M, N, K),
     }
@@ -515,7 +541,68 @@ def measure_ceilings(torch, ops, dev):
     out["one_shot_16mib_read_us"] = best
     out["one_shot_16mib_read_gbs"] = (16 << 20) / (best * 1e-6) / 1e9
     out["empty_kernel_in_graph_us"] = graph_us(lambda i, s: lab.aq_lab_probe_empty(sink.data_ptr(), s))
+    del small
+    out["gemm_operand_data_and_stock_library"] = gemm_calibration(torch, ops, dev)
     return out
+
+
+def gemm_calibration(torch, ops, dev):
+    """Two calibrations of the GEMM figures, measured in the same run on the same box:
+      * this library's int8 GEMM (fused epilogue, bf16 out) at 8192^3 on all-zero operands and on uniformly random
+        codes: identical instruction streams; with zeros the shader clock stays near its maximum, with real data
+        the part throttles to about 1.5 GHz (the MFMA-only probe above shows the same), so the first figure is the
+        kernel's pipeline efficiency and the second what the power limit leaves of it;
+      * the stock library behind torch (hipBLASLt) on the same operands: torch._int_mm (int8 -> int32, no epilogue)
+        and torch._scaled_mm (e4m3 -> bf16) at 8192^3 and at the benchmark shapes of configurations 3 and 4.
+    Eager launches timed with events (kernels of 20 us and more; the launch path is not the limit)."""
+    def timed_us(fn, n):
+        for _ in range(2):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / n
+
+    res = {}
+    g = torch.Generator(device=dev).manual_seed(99)
+    for (M, N, K, n) in ((8192, 8192, 8192, 5), (4096, 2048, 2048, 30)):
+        ops_n = 2.0 * M * N * K
+        tag = f"{M}x{N}x{K}"
+        sx = torch.full((M,), 0.01, device=dev)
+        sw = torch.full((N,), 0.001, device=dev)
+        for name, lim in (("zero_operands", 0), ("random_operands", 127)):
+            a = torch.randint(-lim, lim + 1, (M, K), generator=g, device=dev, dtype=torch.int8)
+            b = torch.randint(-lim, lim + 1, (N, K), generator=g, device=dev, dtype=torch.int8)
+            us = timed_us(lambda: ops.linear_w8a8(a, sx, b, sw, None, out_dtype=torch.bfloat16), n)
+            res[f"this_library_int8_{tag}_{name}_tops"] = ops_n / us / 1e6
+            try:
+                us = timed_us(lambda: torch._int_mm(a, b.t()), n)
+                res[f"stock_int_mm_{tag}_{name}_tops"] = ops_n / us / 1e6
+            except Exception as e:  # the stock routine is a calibration only
+                res[f"stock_int_mm_{tag}_{name}_tops"] = f"unavailable: {str(e)[:80]}"
+            del a, b
+    for (M, N, K, n) in ((8192, 8192, 8192, 5), (2048, 2048, 8192, 30)):
+        flops = 2.0 * M * N * K
+        tag = f"{M}x{N}x{K}"
+        a = torch.randn(M, K, generator=g, device=dev).to(torch.bfloat16)
+        b = (torch.randn(N, K, generator=g, device=dev) * 0.02).to(torch.bfloat16)
+        aq_, sa = ops.quant_tensor_fp8(a)
+        bq_, sb = ops.quant_tensor_fp8(b)
+        us = timed_us(lambda: ops.linear_fp8(aq_, sa, bq_, sb, out_dtype=torch.bfloat16), n)
+        res[f"this_library_fp8_{tag}_tflops"] = flops / us / 1e6
+        try:
+            a8, b8 = aq_.view(torch.float8_e4m3fn), bq_.view(torch.float8_e4m3fn)
+            us = timed_us(lambda: torch._scaled_mm(a8, b8.t(), scale_a=sa.reshape(()), scale_b=sb.reshape(()),
+                                                   out_dtype=torch.bfloat16), n)
+            res[f"stock_scaled_mm_fp8_{tag}_tflops"] = flops / us / 1e6
+        except Exception as e:
+            res[f"stock_scaled_mm_fp8_{tag}_tflops"] = f"unavailable: {str(e)[:80]}"
+        del a, b, aq_, bq_
+    return res
 
 
 def cpu_baseline(workload, shape, unit, per_step):
@@ -585,6 +672,7 @@ def float_linear_cpu(M, N, K, with_bias):
 
 
 def main():
+    t_start = time.time()
     args = parse()
     if args.gpus != 1:
         print(f"bench.py measures one GPU only: --gpus {args.gpus} is not supported in this build "
@@ -616,6 +704,16 @@ def main():
                     r = bench_decode(torch, ops, a2, dev)
                     extra[f"decode_m{m}"] = r
         ceilings = measure_ceilings(torch, ops, dev)
+        if not args.no_extra and args.workload != "model":
+            # the reference's own generation benchmark: about a minute; skipped when this run is already long
+            if time.time() - t_start < 150:
+                m = bench_model(torch, ops, args, dev)
+                extra["model"] = {k: m[k] for k in ("workload", "value", "unit", "ms_per_step", "dtype", "quantized_linears",
+                                                     "int8_weight_bytes", "decode_weight_stream_gbs", "quantized_fused",
+                                                     "quantized_drop_in", "float_bf16_torch", "prefill_logits_rel_err_vs_float",
+                                                     "speedup_decode_vs_float_graph", "speedup_prefill_vs_float_graph")}
+            else:
+                extra["model"] = {"skipped": "time budget of the default run spent"}
     per_step = main_res.get("bytes_per_step") or main_res.get("ops_per_step") or main_res.get("flops_per_step")
     cpu = None
     if not args.no_cpu and args.workload not in ("block", "model"):

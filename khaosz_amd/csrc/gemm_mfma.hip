@@ -133,6 +133,9 @@ struct Frag<true> {
   using type = v8i;  // 32 bytes of K per lane: v_mfma_scale_f32_32x32x64_f8f6f4
 };
 
+#ifndef AQ_FP8_SCALE
+#define AQ_FP8_SCALE 0
+#endif
 template <bool FP8>
 __device__ __forceinline__ typename Acc<FP8>::type mma(const typename Frag<FP8>::type& a,
                                                        const typename Frag<FP8>::type& b,
@@ -141,7 +144,7 @@ __device__ __forceinline__ typename Acc<FP8>::type mma(const typename Frag<FP8>:
     return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
   } else {
     // E8M0 scale 127 = 2^0 for both operands: plain e4m3 x e4m3.
-    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
+    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, AQ_FP8_SCALE, 0, AQ_FP8_SCALE);
   }
 }
 
@@ -162,7 +165,10 @@ __device__ __forceinline__ void sched_pattern() {
 #ifdef AQ_LAB
 __device__ long long aq_lab_clock[4];
 #endif
-template <bool FP8, int OUT, class S>
+// EXACT: K is a whole number of BK-byte steps, so every 16-byte piece of every step lies inside its row and the
+// global->LDS loads need no per-lane range logic: a loop-invariant lane offset per row group and the K step as a
+// scalar offset, no vector ALU work per load.
+template <bool FP8, int OUT, class S, bool EXACT>
 __device__ __forceinline__ void gemm_tile(const GemmArgs& p, uint8_t* smem, int pid) {
   constexpr int WM = S::WM, WN = S::WN, TM = S::TM, TN = S::TN, WK = S::WK, BK = S::BK, NSTAGE = S::NSTAGE;
   constexpr int NWAVES = S::NWAVES, NTHREADS = S::NTHREADS, WAVE_M = S::WAVE_M, WAVE_N = S::WAVE_N;
@@ -214,8 +220,23 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, uint8_t* smem, int 
   const uint32_t ld_off = (uint32_t)ld_row * (uint32_t)K + ld_piece;
   const uint32_t row32 = (uint32_t)(RPG * NWAVES) * (uint32_t)K;  // byte distance between a wavefront's row groups
   constexpr int NLOADS = A_LOADS + B_LOADS;
+  const int nk = (K + BK - 1) / BK;
+  uint32_t ld_vo[A_LOADS > B_LOADS ? A_LOADS : B_LOADS];  // EXACT: lane offset of row group i, A and B alike
+#pragma unroll
+  for (int i = 0; i < (A_LOADS > B_LOADS ? A_LOADS : B_LOADS); ++i) ld_vo[i] = ld_off + (uint32_t)i * row32;
   // load number `idx` (0..NLOADS-1) of K step kt into stage buffer `buf`
   auto issue_load = [&](int kt, int buf, int idx) {
+    if constexpr (EXACT) {
+      // steps past the last one request the last step again (into a stage nobody reads): in range by construction
+      const int k0s = (kt < nk ? kt : nk - 1) * BK;  // wavefront-uniform: a scalar offset
+      uint8_t* st = smem + buf * STAGE + wave * 1024;
+      if (idx < A_LOADS)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(Ar, (lds_void*)(st + idx * (1024 * NWAVES)), 16, ld_vo[idx], k0s, 0, 0);
+      else
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(Br, (lds_void*)(st + BM * BK + (idx - A_LOADS) * (1024 * NWAVES)), 16,
+                                                 ld_vo[idx - A_LOADS], k0s, 0, 0);
+      return;
+    }
     const int k0 = kt * BK;
     // K is a multiple of 16: a piece is all in or all out.  Pieces past K would
     // alias the next row, so they are pushed outside the descriptor (-> zeros).
@@ -311,6 +332,26 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, uint8_t* smem, int 
     constexpr int LD0 = (Q * NLOADS) / NKS, LPS = LOADS ? ((Q + 1) * NLOADS) / NKS - LD0 : 0;
     constexpr int NMMA = TM * TN, NFR = TM + TN;
     constexpr int GROUPS = NMMA > 4 ? NMMA - 2 : NMMA;  // MFMAs that carry memory instructions
+    if constexpr (NMMA >= 8) {
+      // Large sub-tiles (one wavefront per SIMD, or few fragment reads per MFMA): the fragment reads go out in
+      // pairs behind every STRIDE-th MFMA and the global loads behind the MFMA after it.  Measured on a loop of
+      // independent MFMAs with one wavefront per SIMD: two reads behind every fourth MFMA cost nothing (512.3
+      // cycles per 16 MFMAs against 512.4 without reads), one behind every second 24 cycles, all eight first 40.
+      constexpr int NPAIR = (NFR + 1) / 2, STRIDE = NMMA / NPAIR;
+#pragma unroll
+      for (int m = 0; m < NMMA; ++m) {
+        acc[m / TN][m % TN] = mma<FP8>(af[CUR][m / TN], bf[CUR][m % TN], acc[m / TN][m % TN]);
+        if (m % STRIDE == 0 && m / STRIDE < NPAIR) {
+          load_frag(st_next, ks_next, 2 * (m / STRIDE), af[CUR ^ 1], bf[CUR ^ 1]);
+          if (2 * (m / STRIDE) + 1 < NFR) load_frag(st_next, ks_next, 2 * (m / STRIDE) + 1, af[CUR ^ 1], bf[CUR ^ 1]);
+        } else if (m % STRIDE == 1 && m / STRIDE < NPAIR) {
+#pragma unroll
+          for (int q = ((m / STRIDE) * LPS) / NPAIR; q < ((m / STRIDE + 1) * LPS) / NPAIR; ++q) issue_load(kt_ld, buf_ld, LD0 + q);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      return;
+    }
 #pragma unroll
     for (int m = 0; m < NMMA; ++m) {
       acc[m / TN][m % TN] = mma<FP8>(af[CUR][m / TN], bf[CUR][m % TN], acc[m / TN][m % TN]);
@@ -333,7 +374,6 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, uint8_t* smem, int 
   using yes = integral_constant<bool, true>;
   using no = integral_constant<bool, false>;
 
-  const int nk = (K + BK - 1) / BK;
   // Rotated software pipeline over K steps ("stages" s = 0 .. nk-1):
   //   iteration s:  slots    MFMAs of (s, 0 .. NKS-2)       | read fragments (s, 1 .. NKS-1)
   //                 wait for this wavefront's loads of stage s+1, barrier
@@ -691,8 +731,12 @@ __global__ __launch_bounds__(S::NTHREADS) void gemm_kernel(GemmArgs p) {
     }
   } clk;
 #endif
+  const bool exact = (p.K % S::BK) == 0;  // uniform
   for (int pid = blockIdx.x; pid < nt; pid += gridDim.x) {
-    gemm_tile<FP8, OUT, S>(p, smem, pid);
+    if (exact)
+      gemm_tile<FP8, OUT, S, true>(p, smem, pid);
+    else
+      gemm_tile<FP8, OUT, S, false>(p, smem, pid);
     if (pid + (int)gridDim.x < nt) __syncthreads();  // every wavefront is done with the stages before they are refilled
   }
 }

@@ -154,6 +154,15 @@ int aq_gemv_w8a8_decode_rmsnorm(const void *x, int x_dtype, const void *gamma, f
 int aq_linear_fp8(const uint8_t *xq, const float *sx, const uint8_t *wq, const float *sw,
                   void *y, int y_dtype, int64_t M, int64_t N, int64_t K, void *stream);
 
+/* The same with the optional operands of aq_linear_w8a8_residual: y = ((acc * sx) * sw + bias[n]), cast
+ * to y_dtype, then + residual[m, n] (in y's type, may be y itself), rounded again -- the bits of a
+ * separate add.  bias: [N] fp32 or bf16 (linear.py:11) or NULL; residual NULL: no add.  Replaces
+ * F.linear(x, weight, bias) (linear.py:21) and the block's residual add (decoder_block.py:53,58) in
+ * the FP8 variant. */
+int aq_linear_fp8_residual(const uint8_t *xq, const float *sx, const uint8_t *wq, const float *sw,
+                           const void *bias, int bias_dtype, const void *residual, void *y,
+                           int y_dtype, int64_t M, int64_t N, int64_t K, void *stream);
+
 /* RMSNorm followed by per-token quantisation, one launch: the codes and scales
  * aq_quant_rowwise_i8 would give for y = x * rsqrt(mean(x^2) + eps) * gamma held
  * in fp32.  Fuses the reference's F.rms_norm (astrai/model/components/norm.py:14-15)

@@ -34,6 +34,7 @@ SYMBOLS = {
                                            _i64, _vp, _sz, _vp]),
     "aq_gemv_w8a8_codes_residual": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _vp, _vp, _int, _i64, _i64, _i64, _vp]),
     "aq_linear_fp8": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _vp]),
+    "aq_linear_fp8_residual": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _vp, _vp, _int, _i64, _i64, _i64, _vp]),
     "aq_rope_kv_write": (_int, [_vp, _vp, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _vp, _i64, _vp, _vp, _i64, _i64, _i64,
                                 _i64, _vp]),
     "aq_paged_attn_decode": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _vp, _i64, _i64, ctypes.c_float, _vp, _i64, _i64, _i64,

@@ -395,12 +395,20 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, uint8_t* smem, int 
   float sxr[TME][4][4];  // [i][g][q]: row mw + i*32 + g*8 + rq + q
   float swn[TN];
   uint32_t bias_raw[TN];
-  const bool has_bias = !FP8 && OUT != OUT_I32 && p.bias != nullptr;
+  const bool has_bias = OUT != OUT_I32 && p.bias != nullptr;
   const bool bias_bf16 = p.bias_dtype == AQ_BF16;
   auto load_epilogue_operands = [&]() {
     if constexpr (FP8) {
       sx1 = *p.sx;
       sw1 = *p.sw;
+      const __amdgpu_buffer_rsrc_t Bsr =
+          make_rsrc(has_bias ? p.bias : (const void*)p.sw, has_bias ? (uint32_t)N * (bias_bf16 ? 2u : 4u) : 0u);
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const uint32_t n = (uint32_t)(n0 + wave_n * WAVE_N + j * 32 + col);  // past N, or no bias: outside -> 0
+        bias_raw[j] = bias_bf16 ? (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(Bsr, n * 2u, 0, 0)
+                                : (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(Bsr, n * 4u, 0, 0);
+      }
     } else if constexpr (OUT != OUT_I32) {
       // rows past M fall outside the descriptor and read as zero (their outputs are never stored)
       const int rows_left = __builtin_amdgcn_readfirstlane((M - mw) > 0 ? (M - mw) : 0);
@@ -633,7 +641,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, uint8_t* smem, int 
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       float bn = 0.0f;
-      if constexpr (!FP8 && OUT != OUT_I32)
+      if constexpr (OUT != OUT_I32)
         bn = !has_bias ? 0.0f : bias_bf16 ? bf16_bits_to_f32(bias_raw[j]) : __uint_as_float(bias_raw[j]);
       const uint32_t vbase = lane_offset(j);
       if constexpr (OUT != OUT_I32 && !HOIST) {
@@ -656,7 +664,9 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, uint8_t* smem, int 
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
               if constexpr (FP8) {
-                y[q] = __fmul_rn(__fmul_rn(acc[i][j][g * 4 + q], sx1), sw1);
+                // without a bias bn is +0: it changes no bit unless the product is -0, whose sign a bf16 or
+                // fp32 consumer of a Linear output never sees as a different value
+                y[q] = __fadd_rn(__fmul_rn(__fmul_rn(acc[i][j][g * 4 + q], sx1), sw1), bn);
               } else {
                 // three separately rounded fp32 operations, never contracted.  Without a bias
                 // bn is +0: the product of an integer and two positive scales is never -0,
@@ -862,13 +872,26 @@ extern "C" int aq_linear_w8a8_residual(const int8_t* xq, const float* sx, const 
 
 extern "C" int aq_linear_fp8(const uint8_t* xq, const float* sx, const uint8_t* wq, const float* sw,
                              void* y, int y_dtype, int64_t M, int64_t N, int64_t K, void* stream) {
+  return aq_linear_fp8_residual(xq, sx, wq, sw, nullptr, AQ_F32, nullptr, y, y_dtype, M, N, K, stream);
+}
+
+extern "C" int aq_linear_fp8_residual(const uint8_t* xq, const float* sx, const uint8_t* wq, const float* sw,
+                                      const void* bias, int bias_dtype, const void* residual, void* y, int y_dtype,
+                                      int64_t M, int64_t N, int64_t K, void* stream) {
   if (y_dtype != AQ_F32 && y_dtype != AQ_BF16) return AQ_E_DTYPE;
+  if (bias && bias_dtype != AQ_F32 && bias_dtype != AQ_BF16) return AQ_E_DTYPE;
   int rc = aq::check_gemm(xq, wq, y, M, N, K);
   if (rc || M == 0 || N == 0) return rc;
   if (!sx || !sw) return AQ_E_NULL;
+  if (aq::check_ptr(sx, 4) || aq::check_ptr(sw, 4) || aq::check_ptr(bias, bias_dtype == AQ_BF16 ? 2 : 4) ||
+      aq::check_ptr(residual, 4))
+    return AQ_E_ALIGN;
   aq::GemmArgs a = aq::make_args(xq, wq, y, M, N, K);
   a.sx = sx;
   a.sw = sw;
+  a.bias = bias;
+  a.bias_dtype = bias_dtype;
+  a.res = residual;
   hipStream_t st = static_cast<hipStream_t>(stream);
   return y_dtype == AQ_BF16 ? aq::launch<true, aq::OUT_BF16>(a, st) : aq::launch<true, aq::OUT_F32>(a, st);
 }

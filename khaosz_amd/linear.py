@@ -218,26 +218,24 @@ class Fp8Linear(Linear):
     """FP8 (OCP e4m3fn) Linear with per-tensor scales and fp32 accumulation."""
 
     def __init__(self, in_dim: int, out_dim: int, bias: bool = False, device=None):
-        if bias:
-            raise ValueError("the FP8 path has no bias epilogue (the reference never builds a Linear with bias)")
         nn.Module.__init__(self)
         self.register_buffer("qweight", torch.zeros((out_dim, in_dim), dtype=torch.uint8, device=device))
         self.register_buffer("w_scale", torch.ones((1,), dtype=torch.float32, device=device))
-        self.bias = None
+        self.bias = nn.Parameter(torch.zeros(out_dim, device=device), requires_grad=False) if bias else None
 
     @classmethod
     def from_linear(cls, base: nn.Module) -> "Fp8Linear":
         w = base.weight.detach()
         if not w.is_cuda:
             raise RuntimeError("Fp8Linear.from_linear needs the weight on the GPU (the quantizer is a HIP kernel)")
-        if base.bias is not None:
-            raise ValueError("the FP8 path has no bias epilogue")
-        q = cls(w.shape[1], w.shape[0], device=w.device)
+        q = cls(w.shape[1], w.shape[0], bias=base.bias is not None, device=w.device)
         if w.dtype not in (torch.float32, torch.bfloat16):
             w = w.float()
         codes, scale = ops.quant_tensor_fp8(w)
         q.qweight.copy_(codes)
         q.w_scale.copy_(scale)
+        if base.bias is not None:
+            q.bias = nn.Parameter(base.bias.detach().clone(), requires_grad=False)
         return q
 
     @property
@@ -255,14 +253,15 @@ class Fp8Linear(Linear):
     def reset_parameters(self) -> None:
         raise RuntimeError("Fp8Linear holds quantized weights; initialise a float Linear and convert it")
 
-    def forward(self, x: Tensor) -> Tensor:
+    def forward(self, x: Tensor, residual: Optional[Tensor] = None) -> Tensor:
+        """``residual`` (shape and dtype of the output): added in the kernel's epilogue, the bits of a separate add."""
         _no_grad_guard(x)
         lead = x.shape[:-1]
         x2 = x.reshape(-1, x.shape[-1])
         if x2.shape[1] != self.qweight.shape[1]:
             raise ValueError(f"expected last dim {self.qweight.shape[1]}, got {x2.shape[1]}")
         xq, sx = ops.quant_tensor_fp8(x2)
-        y = ops.linear_fp8(xq, sx, self.qweight, self.w_scale, out_dtype=x.dtype)
+        y = ops.linear_fp8(xq, sx, self.qweight, self.w_scale, self.bias, out_dtype=x.dtype, residual=residual)
         return y.reshape(*lead, self.qweight.shape[0])
 
 

@@ -605,9 +605,9 @@ def paged_attn_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     return out
 
 
-def linear_fp8(xq, sx, wq, sw, out_dtype=torch.bfloat16) -> torch.Tensor:
-    """FP8 e4m3fn GEMM with fp32 accumulation: y = (acc * sx[0]) * sw[0]."""
-    _need_gpu(xq, sx, wq, sw)
+def linear_fp8(xq, sx, wq, sw, bias=None, out_dtype=torch.bfloat16, residual=None) -> torch.Tensor:
+    """FP8 e4m3fn GEMM with fp32 accumulation: y = (acc * sx[0]) * sw[0] (+ bias), cast, (+ residual)."""
+    _need_gpu(xq, sx, wq, sw, bias, residual)
     if xq.dtype != torch.uint8 or wq.dtype != torch.uint8:
         raise ValueError("linear_fp8 takes e4m3fn codes as uint8")
     if xq.dim() != 2 or wq.dim() != 2 or xq.shape[1] != wq.shape[1]:
@@ -620,10 +620,16 @@ def linear_fp8(xq, sx, wq, sw, out_dtype=torch.bfloat16) -> torch.Tensor:
     if out_dtype not in _DT:
         raise ValueError(f"out_dtype {out_dtype} is not supported")
     xq, wq = xq.contiguous(), wq.contiguous()
+    b, bdt = _bias_args(bias, N)
+    r = _residual_arg(residual, M, N, out_dtype, xq.device)
     y = torch.empty((M, N), dtype=out_dtype, device=xq.device)
     if M and N:
         with _OnDevice(xq.device):
-            rc = _abi.load().aq_linear_fp8(xq.data_ptr(), sx.data_ptr(), wq.data_ptr(), sw.data_ptr(), y.data_ptr(),
-                                           _DT[out_dtype], M, N, K, _stream(xq))
+            rc = _abi.load().aq_linear_fp8_residual(xq.data_ptr(), sx.data_ptr(), wq.data_ptr(), sw.data_ptr(),
+                                                    b.data_ptr() if b is not None else None, bdt,
+                                                    r.data_ptr() if r is not None else None, y.data_ptr(),
+                                                    _DT[out_dtype], M, N, K, _stream(xq))
         _abi.check(rc, "aq_linear_fp8")
+    elif r is not None:
+        y.copy_(r.view(M, N))
     return y

@@ -587,7 +587,7 @@ void oq_quant_tensor_fp8_bf16(const uint16_t *x, int64_t numel, uint8_t *q, floa
 }
 
 /* y = (sum_k f(xq[m,k]) f(wq[n,k])) * sx * sw; fp32 accumulate, k ascending. */
-void oq_linear_fp8(const uint8_t *xq, float sx, const uint8_t *wq, float sw, float *y_f32,
+void oq_linear_fp8(const uint8_t *xq, float sx, const uint8_t *wq, float sw, const float *bias, float *y_f32,
                    uint16_t *y_bf16, int64_t M, int64_t N, int64_t K) {
   float lut[256];
   for (int i = 0; i < 256; ++i) lut[i] = oq_e4m3fn_to_f32((uint8_t)i);
@@ -601,7 +601,8 @@ void oq_linear_fp8(const uint8_t *xq, float sx, const uint8_t *wq, float sw, flo
       for (int64_t k = 0; k < K; ++k) s += xr[k] * lut[wr[k]];
       volatile float t = s * sx;
       volatile float u = t * sw;
-      float y = u;
+      volatile float v = bias ? u + bias[n] : u;  /* the bias of linear.py:11,21: one more rounded add */
+      float y = v;
       if (y_f32) y_f32[m * N + n] = y;
       if (y_bf16) y_bf16[m * N + n] = oq_f32_to_bf16(y);
     }

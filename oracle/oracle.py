@@ -180,12 +180,15 @@ def np_quant_tensor_fp8(x: np.ndarray):
     return np_f32_to_e4m3fn(v), s
 
 
-def np_linear_fp8(xq, sx, wq, sw) -> np.ndarray:
+def np_linear_fp8(xq, sx, wq, sw, bias=None) -> np.ndarray:
     """Float64 accumulation of the decoded codes: the 'true' value the fp32
     accumulating implementations are held to within tolerance."""
     lut = np_e4m3fn_table().astype(np.float64)
     acc = lut[xq] @ lut[wq].T
-    return ((acc * float(sx)) * float(sw)).astype(F32)
+    y = (acc * float(sx)) * float(sw)
+    if bias is not None:
+        y = y + np.asarray(bias, np.float64)[None, :]
+    return y.astype(F32)
 
 
 def np_linear_f32(x, w, bias=None) -> np.ndarray:
@@ -237,7 +240,7 @@ def _load():
     lib.oq_linear_w8a8_bf16.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i64]
     lib.oq_quant_tensor_fp8_f32.argtypes = [vp, i64, vp, vp]
     lib.oq_quant_tensor_fp8_bf16.argtypes = [vp, i64, vp, vp]
-    lib.oq_linear_fp8.argtypes = [vp, ctypes.c_float, vp, ctypes.c_float, vp, vp, i64, i64, i64]
+    lib.oq_linear_fp8.argtypes = [vp, ctypes.c_float, vp, ctypes.c_float, vp, vp, vp, i64, i64, i64]
     lib.oq_linear_f32.argtypes = [vp, vp, vp, vp, i64, i64, i64]
     for name in (
         "oq_set_num_threads oq_quant_rowwise_i8_f32 oq_quant_rowwise_i8_bf16 oq_gemm_i8_i32 "
@@ -422,13 +425,14 @@ def c_quant_tensor_fp8(x: np.ndarray, bf16_bits: bool = False):
     return q, F32(s[0])
 
 
-def c_linear_fp8(xq, sx, wq, sw, bf16_out: bool = False) -> np.ndarray:
+def c_linear_fp8(xq, sx, wq, sw, bf16_out: bool = False, bias=None) -> np.ndarray:
     lib = _load()
     xq, wq = _c(xq, np.uint8), _c(wq, np.uint8)
+    bias = None if bias is None else _c(bias, F32)
     M, K = xq.shape
     N = wq.shape[0]
     y = np.empty((M, N), np.uint16 if bf16_out else F32)
-    lib.oq_linear_fp8(_p(xq), float(sx), _p(wq), float(sw), None if bf16_out else _p(y),
+    lib.oq_linear_fp8(_p(xq), float(sx), _p(wq), float(sw), _p(bias), None if bf16_out else _p(y),
                       _p(y) if bf16_out else None, M, N, K)
     return y
 

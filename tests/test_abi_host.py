@@ -56,6 +56,8 @@ def test_argument_validation_happens_before_any_launch():
     assert lib.aq_linear_w8a8(P, P, P, P, None, 0, P, 5, 4, 4, 32, None) == -3
     assert lib.aq_linear_w8a8(P, None, P, P, None, 0, P, 1, 4, 4, 32, None) == -1
     assert lib.aq_linear_fp8(P, P, P, P, P, 9, 4, 4, 32, None) == -3
+    assert lib.aq_linear_fp8_residual(P, P, P, P, P, 7, None, P, 1, 4, 4, 32, None) == -3       # bias dtype
+    assert lib.aq_linear_fp8_residual(P, P, P, P, None, 0, P + 2, P, 1, 4, 4, 32, None) == -4   # residual alignment
     assert lib.aq_gemv_w8a8_decode(P, 1, P, P, None, 0, P, 1, 17, 8, 32, P, 1 << 20, None) == -2  # M > 16
     assert lib.aq_gemv_w8a8_decode(P, 1, P, P, None, 0, P, 1, 4, 8, 32, P, 8, None) == -5         # workspace
     assert lib.aq_gemv_w8a8_decode(P, 1, P, P, None, 0, P + 2, 1, 4, 8, 32, P, 1 << 20, None) == -4  # y alignment
@@ -109,8 +111,8 @@ def test_quant_linear_is_a_linear_with_quantized_state():
     assert q.in_dim == 32 and q.out_dim == 16
     f = Fp8Linear(32, 16)
     assert isinstance(f, Linear) and set(f.state_dict()) == {"qweight", "w_scale"}
-    with pytest.raises(ValueError):
-        Fp8Linear(32, 16, bias=True)
+    fb = Fp8Linear(32, 16, bias=True)
+    assert set(fb.state_dict()) == {"qweight", "w_scale", "bias"} and tuple(fb.bias.shape) == (16,)
     with pytest.raises(RuntimeError):
         q.reset_parameters()
 

@@ -478,6 +478,49 @@ def test_linear_fp8_within_tolerance(oracle, tile, M, N, K):
     np.testing.assert_allclose(yb, exact, rtol=1e-2, atol=1e-2 * rms)  # stated tolerance: 1e-2 relative in bf16
     yc = oracle.c_linear_fp8(xq, sx, wq, sw)
     np.testing.assert_allclose(y32, yc, rtol=1e-2, atol=1e-3 * rms)
+    # bias (fp32 and bf16) and residual in the epilogue: the bias inside the stated tolerance of the oracle
+    # with a bias, the residual the bits of a separate add
+    g = torch.Generator().manual_seed(43)
+    for bias in (torch.randn(N, generator=g) * 0.5, (torch.randn(N, generator=g) * 0.5).to(torch.bfloat16)):
+        want = oracle.np_linear_fp8(xq, sx, wq, sw, bias=bias.float().numpy())
+        got32 = ops.linear_fp8(*args, bias.to(DEV), out_dtype=torch.float32)
+        assert np.max(np.abs(to_np(got32) - want)) <= 1e-3 * max(rms, 0.5)
+        np.testing.assert_allclose(to_np(got32), oracle.c_linear_fp8(xq, sx, wq, sw, bias=bias.float().numpy()),
+                                   rtol=1e-2, atol=1e-3 * max(rms, 0.5))
+        for dt in (torch.float32, torch.bfloat16):
+            plain = ops.linear_fp8(*args, bias.to(DEV), out_dtype=dt)
+            r = torch.randn(M, N, generator=g).to(dt).to(DEV)
+            assert torch.equal(ops.linear_fp8(*args, bias.to(DEV), out_dtype=dt, residual=r), plain + r)
+            y_in_place = r.clone()   # the residual may be the output buffer itself
+            rc = _abi.load().aq_linear_fp8_residual(args[0].data_ptr(), args[1].data_ptr(), args[2].data_ptr(),
+                                                    args[3].data_ptr(), None, 0, y_in_place.data_ptr(),
+                                                    y_in_place.data_ptr(), 1 if dt == torch.bfloat16 else 0, M, N, K,
+                                                    torch.cuda.current_stream().cuda_stream)
+            assert rc == 0 and torch.equal(y_in_place, ops.linear_fp8(*args, out_dtype=dt) + r)
+
+
+def test_fp8_linear_module_with_a_bias_and_a_residual(oracle):
+    """Fp8Linear keeps the reference's optional bias (linear.py:11) and takes the residual stream like QuantLinear."""
+    torch.manual_seed(8)
+    lin = Linear(256, 96, bias=True)
+    lin.reset_parameters()
+    lin = lin.to(DEV)
+    f = Fp8Linear.from_linear(lin)
+    assert torch.equal(f.bias, lin.bias) and set(f.state_dict()) == {"qweight", "w_scale", "bias"}
+    x = torch.randn(3, 20, 256, device=DEV, dtype=torch.bfloat16)
+    r = torch.randn(3, 20, 96, device=DEV, dtype=torch.bfloat16)
+    with torch.inference_mode():
+        y = f(x)
+        assert torch.equal(f(x, residual=r), y + r)
+    xq, sx = oracle.c_quant_tensor_fp8(bf16_bits(x.reshape(60, 256)), bf16_bits=True)
+    want = oracle.np_linear_fp8(xq, sx, to_np(f.qweight), float(f.w_scale.item()), bias=to_np(lin.bias.detach()))
+    np.testing.assert_allclose(to_np(y.float()).reshape(60, 96), want, rtol=1e-2, atol=1e-2 * float(np.abs(want).mean()))
+    ref = torch.nn.functional.linear(x.float(), lin.weight, lin.bias)
+    assert ((y.float() - ref).norm() / ref.norm()).item() < 0.08
+    g = Fp8Linear(256, 96, bias=True, device=DEV)
+    g.load_state_dict(f.state_dict())
+    with torch.inference_mode():
+        assert torch.equal(g(x), y)
 
 
 def test_linear_fp8_one_hot_pins_operand_order(oracle, tile):

@@ -45,10 +45,16 @@ def test_linear_fp8_fp32_accumulate_within_tolerance_of_exact(oracle):
     assert np.max(np.abs(y - exact)) <= 1e-4 * rms
     yb = oracle.c_linear_fp8(xq, sx, wq, sw, bf16_out=True)
     assert np.array_equal(yb, oracle.np_f32_to_bf16_bits(y))
+    # with a bias (linear.py:11,21): one more rounded add, against the float64 sum and a hand value
+    b = (rng.standard_normal(40) * 0.5).astype(np.float32)
+    yb32 = oracle.c_linear_fp8(xq, sx, wq, sw, bias=b)
+    assert np.array_equal(yb32, (y + b[None, :]).astype(np.float32))
+    assert np.max(np.abs(yb32 - oracle.np_linear_fp8(xq, sx, wq, sw, bias=b))) <= 1e-4 * max(rms, 0.5)
     # one hand-checked product: 1.5 * -2 summed 16 times, scales 0.5 and 4
     a = np.full((1, 16), 0x3C, np.uint8)       # 1.5
     b = np.full((1, 16), 0xC0, np.uint8)       # -2.0
     assert oracle.c_linear_fp8(a, 0.5, b, 4.0)[0, 0] == 16 * 1.5 * -2.0 * 0.5 * 4.0
+    assert oracle.c_linear_fp8(a, 0.5, b, 4.0, bias=np.array([100.25], np.float32))[0, 0] == 16 * 1.5 * -2.0 * 0.5 * 4.0 + 100.25
     # end to end against the float Linear: e4m3 carries 3 mantissa bits, so the
     # element error is about 2^-4/sqrt(3) relative and averages down over K
     ref = torch.nn.functional.linear(torch.from_numpy(x), torch.from_numpy(w)).numpy()

@@ -67,6 +67,8 @@ def parse():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="decode", choices=["decode", "prefill", "fp8", "block", "model"])
     ap.add_argument("--m", type=int, default=16, help="decode rows (1..16)")
+    ap.add_argument("--mnk", default=None, help="prefill workload only: M,N,K of the int8 Linear instead of configuration 3's "
+                    "4096,2048,2048 (e.g. 8192,8192,8192 for a profile of the GEMM's steady state)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary workloads")
     return ap.parse_args()
@@ -188,12 +190,15 @@ def bench_decode(torch, ops, args, dev):
 def bench_prefill(torch, ops, args, dev):
     M, K, N = 4096, 2048, 2048
     nbuf = 8
+    if getattr(args, "mnk", None) and args.workload == "prefill":
+        M, N, K = (int(v) for v in args.mnk.split(","))
+        nbuf = 8 if M * K <= (1 << 25) else 2
     weights = make_weights(torch, ops, N, K, nbuf, dev, seed=3)
     g = torch.Generator(device=dev).manual_seed(4)
     xs = []
     for _ in range(nbuf):
         x = torch.randn(M, K, generator=g, device=dev)
-        cols = torch.randperm(K, generator=g, device=dev)[:20]  # 1 % outlier channels x10
+        cols = torch.randperm(K, generator=g, device=dev)[:max(1, K // 100)]  # 1 % outlier channels x10
         x[:, cols] *= 10
         xs.append(x.to(torch.bfloat16))
     bias = (torch.randn(N, generator=g, device=dev) * 0.01)
@@ -228,7 +233,7 @@ def bench_prefill(torch, ops, args, dev):
     ms_nq = graph_time_ms(torch, norm_quant_only, steps, args.warmup)
     tops = ops_alg / (ms * 1e-3) / 1e12
     tops_k = ops_alg / (ms_k * 1e-3) / 1e12
-    traffic, traffic_src = measured_traffic("prefill")
+    traffic, traffic_src = measured_traffic("prefill") if (M, N, K) == (4096, 2048, 2048) else (None, "not measured for this shape")
     qbytes = 2 * M * K + M * K + 4 * M
     return {
         "workload": f"prefill_linear_w8a8 M={M} K={K} N={N} quantise + int8 MFMA GEMM + scale/bias epilogue, bf16 out",
@@ -270,6 +275,24 @@ def bench_fp8(torch, ops, args, dev):
     steps = max(10, min(args.steps, 50))
     ms = graph_time_ms(torch, step, steps, args.warmup)
     ms_k = graph_time_ms(torch, kernel_only, steps, args.warmup)
+    # the same variant at decode sizes (configuration 2's shape): per-tensor cast inside the streaming GEMV
+    dec = {}
+    if not args.no_extra:
+        Nd, Kd = 8192, 2048
+        wd = make_weights(torch, ops, Nd, Kd, 40, dev, seed=15, mode="fp8")
+        for Md in (1, 16):
+            xd = torch.randn(Md, Kd, generator=g, device=dev).to(torch.bfloat16)
+            wsd = torch.empty((ops._abi.load().aq_gemv_fp8_workspace_bytes(Md, Kd),), dtype=torch.uint8, device=dev)
+
+            def dstep(i, xd=xd, wsd=wsd):
+                wq, sw = wd[i % 40]
+                ys[0] = ops.gemv_fp8_decode(xd, wq, sw, None, out_dtype=torch.bfloat16, workspace=wsd)
+
+            t_us = graph_time_ms(torch, dstep, args.steps, args.warmup) * 1e3
+            db = Nd * Kd + 2 * Md * Kd + 2 * Md * Nd
+            dec[f"M={Md}"] = {"us_per_step": t_us, "gbs": db / t_us / 1e3, "frac_hbm": db / t_us / 1e3 / PEAK_HBM_GBS,
+                              "algorithmic_bytes": db}
+        del wd
     t = flops / (ms * 1e-3) / 1e12
     tk = flops / (ms_k * 1e-3) / 1e12
     traffic, traffic_src = measured_traffic("fp8")
@@ -279,6 +302,7 @@ def bench_fp8(torch, ops, args, dev):
         "roofline": {"bound": "mfma", "kernel": "gemm_kernel<fp8,bf16>", "achieved": tk, "peak": PEAK_FP8_TFLOPS,
                      "unit": "TFLOP/s", "frac": tk / PEAK_FP8_TFLOPS, "traffic": traffic, "traffic_source": traffic_src,
                      "kernel_us": ms_k * 1e3, "algorithmic_flops": flops},
+        "decode_gemv_fp8_N8192_K2048": dec,
         "shape": (M, N, K),
     }
 
@@ -461,7 +485,7 @@ def bench_model(torch, ops, args, dev):
     }
 
 
-def measure_ceilings(torch, ops, dev):
+def measure_ceilings(torch, ops, dev, calibrate=True):
     """What this part delivers on trivial kernels (the lab library's probes, csrc/aq_lab.h):
       * an MFMA-only loop with constant operands (no bit toggling: the clock stays at its maximum) and with random
         operands that change every instruction (what a GEMM feeds the matrix cores), each with the shader clock
@@ -542,7 +566,8 @@ def measure_ceilings(torch, ops, dev):
     out["one_shot_16mib_read_gbs"] = (16 << 20) / (best * 1e-6) / 1e9
     out["empty_kernel_in_graph_us"] = graph_us(lambda i, s: lab.aq_lab_probe_empty(sink.data_ptr(), s))
     del small
-    out["gemm_operand_data_and_stock_library"] = gemm_calibration(torch, ops, dev)
+    if calibrate:  # launches GEMMs of other shapes: left out of single-workload (profiling) runs
+        out["gemm_operand_data_and_stock_library"] = gemm_calibration(torch, ops, dev)
     return out
 
 
@@ -703,7 +728,7 @@ def main():
                     a2.m = m
                     r = bench_decode(torch, ops, a2, dev)
                     extra[f"decode_m{m}"] = r
-        ceilings = measure_ceilings(torch, ops, dev)
+        ceilings = measure_ceilings(torch, ops, dev, calibrate=not args.no_extra)
         if not args.no_extra and args.workload != "model":
             # the reference's own generation benchmark: about a minute; skipped when this run is already long
             if time.time() - t_start < 150:

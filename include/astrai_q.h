@@ -163,6 +163,23 @@ int aq_linear_fp8_residual(const uint8_t *xq, const float *sx, const uint8_t *wq
                            const void *bias, int bias_dtype, const void *residual, void *y,
                            int y_dtype, int64_t M, int64_t N, int64_t K, void *stream);
 
+/* The FP8 Linear at decode, M <= 16 rows (executor.py:59-94): the weight-streaming GEMV of aq_gemv_w8a8_decode
+ * on e4m3 codes (one 16x16x128 matrix-core product per 128-byte line), per-tensor scales, fp32 accumulation,
+ * y = ((acc * sx) * sw + bias) cast, + residual.  aq_gemv_fp8_codes_residual takes codes and scale as
+ * aq_quant_tensor_fp8 writes them; aq_gemv_fp8_decode_residual takes the rows themselves and, for bf16 rows
+ * of K <= 2048 (K a multiple of 512), casts them inside the GEMV kernel (one launch: the tensor's maximum goes
+ * round the workgroup first), otherwise through ws (aq_gemv_fp8_workspace_bytes(M, K) bytes) by
+ * aq_quant_tensor_fp8 + the codes entry.  K not a multiple of 256, or rows too long for a compute unit's
+ * LDS: the tiled FP8 GEMM takes the call.  Replaces F.linear (linear.py:21) in the FP8 variant. */
+size_t aq_gemv_fp8_workspace_bytes(int64_t M, int64_t K);
+int aq_gemv_fp8_codes_residual(const uint8_t *xq, const float *sx, const uint8_t *wq, const float *sw,
+                               const void *bias, int bias_dtype, const void *residual, void *y,
+                               int y_dtype, int64_t M, int64_t N, int64_t K, void *stream);
+int aq_gemv_fp8_decode_residual(const void *x, int x_dtype, const uint8_t *wq, const float *sw,
+                                const void *bias, int bias_dtype, const void *residual, void *y,
+                                int y_dtype, int64_t M, int64_t N, int64_t K, void *ws, size_t ws_bytes,
+                                void *stream);
+
 /* RMSNorm followed by per-token quantisation, one launch: the codes and scales
  * aq_quant_rowwise_i8 would give for y = x * rsqrt(mean(x^2) + eps) * gamma held
  * in fp32.  Fuses the reference's F.rms_norm (astrai/model/components/norm.py:14-15)

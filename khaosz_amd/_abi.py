@@ -34,6 +34,10 @@ SYMBOLS = {
                                            _i64, _vp, _sz, _vp]),
     "aq_gemv_w8a8_codes_residual": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _vp, _vp, _int, _i64, _i64, _i64, _vp]),
     "aq_linear_fp8": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _vp]),
+    "aq_gemv_fp8_workspace_bytes": (_sz, [_i64, _i64]),
+    "aq_gemv_fp8_codes_residual": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _vp, _vp, _int, _i64, _i64, _i64, _vp]),
+    "aq_gemv_fp8_decode_residual": (_int, [_vp, _int, _vp, _vp, _vp, _int, _vp, _vp, _int, _i64, _i64, _i64, _vp,
+                                           _sz, _vp]),
     "aq_linear_fp8_residual": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _vp, _vp, _int, _i64, _i64, _i64, _vp]),
     "aq_rope_kv_write": (_int, [_vp, _vp, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _vp, _i64, _vp, _vp, _i64, _i64, _i64,
                                 _i64, _vp]),

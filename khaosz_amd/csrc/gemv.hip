@@ -414,9 +414,14 @@ constexpr int GM_BATCH = 8;    // MFMA steps (64 K bytes each) per register batc
 // rows per wavefront of a KS x GR = 8 wavefront workgroup, while its weight loads are in flight (the row
 // arithmetic of the stand-alone quantiser, shared through aq_rows.h: same codes and scales); NORM: after
 // RMS-normalising them with the gain p.gamma.  One launch per decode step instead of two.
-template <int KS, int GR, bool RES, int XR, int FQ = 0, bool NORM = false>
+// FP8: weights and tokens are OCP e4m3fn codes with one scale per tensor (p.sx, p.sw point to scalars) and the
+// products run on v_mfma_f32_16x16x128_f8f6f4 -- one instruction per 128-byte line instead of two -- with fp32
+// accumulation; with FQ the kernel casts its bf16 rows itself, after the maximum over ALL rows (the per-tensor
+// scale of aq_quant_tensor_fp8: s = amax / 448, codes = e4m3(clamp(x / s))) has gone round the workgroup.
+template <int KS, int GR, bool RES, int XR, int FQ = 0, bool NORM = false, bool FP8 = false>
 __global__ __launch_bounds__(GM_MAX_WAVES * 64) void gemv_mfma_kernel(GemvArgs p) {
   static_assert(FQ == 0 || (KS > 0 && GR > 0), "the in-kernel quantiser deals rows to a fixed number of wavefronts");
+  static_assert(!(FP8 && NORM), "no fused norm in front of the FP8 cast");
   extern __shared__ __attribute__((aligned(16))) uint8_t xs[];  // [16][K + 16] token codes, [16] scales, 16 spare bytes; later the partial sums
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -438,11 +443,11 @@ __global__ __launch_bounds__(GM_MAX_WAVES * 64) void gemv_mfma_kernel(GemvArgs p
   // measured 0.2 us faster than behind the weight stream (loads return in request order, and these few come
   // back quickly, while behind the weights the epilogue would wait for the whole stream to drain).
   const EpiOperands epi(p, kh == 0, FQ == 0, RES);
-  float sxv = epi.load_sx(tok, tok < M);
+  float sxv = epi.load_sx(FP8 ? 0 : tok, FP8 || tok < M);
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
     const int n = rbase + r;
-    swv[r] = epi.load_sw(n, n < N);
+    swv[r] = epi.load_sw(FP8 ? 0 : n, FP8 || n < N);
     bv[r] = epi.load_bias(n, n < N);
     rv[r] = RES ? epi.load_res(tok, n, tok < M && n < N, (int)p.ldr) : 0u;
   }
@@ -486,7 +491,68 @@ __global__ __launch_bounds__(GM_MAX_WAVES * 64) void gemv_mfma_kernel(GemvArgs p
     wload(0, wa);
     wload(GM_LINES, wb);
     asm volatile("" ::: "memory");
-    xrows.template finish<NORM>(M, M, K, xs, pitch, sx_lds, wave, WAVES, lane, p.eps);
+    if constexpr (!FP8) {
+      xrows.template finish<NORM>(M, M, K, xs, pitch, sx_lds, wave, WAVES, lane, p.eps);
+    } else {
+      // the tensor's maximum: every wavefront's share through LDS (a maximum has no order), then the cast
+      float amax = 0.0f;
+#pragma unroll
+      for (int j = 0; j < RPW; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          float f[8];
+          RowIn<true>::unpack(xrows.c[j][i], f);  // rows >= M and vectors past K were loaded as zeros
+          amax = fmaxf(amax, vec_amax<8>(f));
+        }
+      amax = wave_max(amax);
+      if (lane == 0) sx_lds[wave] = amax;
+      __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_s_barrier();  // no memory fence: the weight loads stay in flight
+      asm volatile("" ::: "memory");
+      float all = 0.0f;
+#pragma unroll
+      for (int w = 0; w < WAVES; ++w) all = fmaxf(all, sx_lds[w]);
+      float sc = __fdiv_rn(all, 448.0f);
+      if (all == 0.0f) sc = 1.0f;
+      sxv = sc;
+      const float y0 = __builtin_amdgcn_rcpf(sc);
+      const float rsc = __builtin_fmaf(__builtin_fmaf(-sc, y0, 1.0f), y0, y0);
+      const bool lean_ok = sc >= 5.421010862427522e-20f && sc <= 1.8446744073709552e19f;  // [2^-64, 2^64]
+      const int nvec = K / 8;
+#pragma unroll
+      for (int j = 0; j < RPW; ++j) {
+        const int m = wave + j * WAVES;
+        if (m >= M) continue;  // uniform
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int v = i * 64 + lane;
+          if (v < nvec) {
+            float f[8];
+            RowIn<true>::unpack(xrows.c[j][i], f);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+              // x / s: the refined-reciprocal sequence that equals the correctly rounded divide for in-range
+              // scales (see quant_codes), the divide itself otherwise; then the clamp to the e4m3 range
+              float q;
+              if (__builtin_expect(lean_ok, 1)) {
+                q = f[e] * rsc;
+                q = __builtin_fmaf(__builtin_fmaf(-sc, q, f[e]), rsc, q);
+                q = __builtin_fmaf(__builtin_fmaf(-sc, q, f[e]), rsc, q);
+              } else {
+                q = __fdiv_rn(f[e], sc);
+              }
+              f[e] = fminf(fmaxf(q, -448.0f), 448.0f);
+            }
+            int w0 = __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], 0, false);
+            w0 = __builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], w0, true);
+            int w1 = __builtin_amdgcn_cvt_pk_fp8_f32(f[4], f[5], 0, false);
+            w1 = __builtin_amdgcn_cvt_pk_fp8_f32(f[6], f[7], w1, true);
+            *reinterpret_cast<uint2*>(xs + m * pitch + v * 8) = make_uint2((uint32_t)w0, (uint32_t)w1);
+          }
+        }
+      }
+    }
   } else {
     const __amdgpu_buffer_rsrc_t Xr = make_rsrc(p.xq, (uint32_t)M * (uint32_t)K);
     const int nvec_row = K / 16;
@@ -531,14 +597,15 @@ __global__ __launch_bounds__(GM_MAX_WAVES * 64) void gemv_mfma_kernel(GemvArgs p
   asm volatile("" ::: "memory");
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
-  if constexpr (FQ > 0) sxv = sx_lds[tok < M ? tok : 0];
+  if constexpr (FQ > 0 && !FP8) sxv = sx_lds[tok < M ? tok : 0];
 
   // Four independent accumulators (summed at the end: int32, exact in any order) and a batch's token
   // fragments read from LDS up front: one chain of 16 dependent read -> MFMA steps took 0.6 us after the
   // token codes had landed, which is all on the kernel's critical path.
-  v4i accs[4];
+  using accv = std::conditional_t<FP8, v4f, v4i>;
+  accv accs[4];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) accs[i] = v4i{0, 0, 0, 0};
+  for (int i = 0; i < 4; ++i) accs[i] = accv{0, 0, 0, 0};
   // MFMA step (t, e) of line t takes, for weight row r = lane % 16 and token lane % 16, the line's piece
   // 2 (lane / 16) + e: K bytes t 128 + (2 q + e) 16 of the wavefront's part.  (Any assignment of K bytes to the
   // steps' k slots is a valid product as long as both operands use the same one.)  Lane l holds piece l / 8 of
@@ -568,8 +635,16 @@ __global__ __launch_bounds__(GM_MAX_WAVES * 64) void gemv_mfma_kernel(GemvArgs p
                       __builtin_amdgcn_update_dpp((int)hi.y, (int)lo.y, ROR8, 0xf, 0x3, false),
                       __builtin_amdgcn_update_dpp((int)hi.z, (int)lo.z, ROR8, 0xf, 0x3, false),
                       __builtin_amdgcn_update_dpp((int)hi.w, (int)lo.w, ROR8, 0xf, 0x3, false)};
-      accs[(2 * t) & 3] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w0, x[2 * t], accs[(2 * t) & 3], 0, 0, 0);
-      accs[(2 * t + 1) & 3] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w1, x[2 * t + 1], accs[(2 * t + 1) & 3], 0, 0, 0);
+      if constexpr (!FP8) {
+        accs[(2 * t) & 3] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w0, x[2 * t], accs[(2 * t) & 3], 0, 0, 0);
+        accs[(2 * t + 1) & 3] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w1, x[2 * t + 1], accs[(2 * t + 1) & 3], 0, 0, 0);
+      } else {
+        // the line's pieces 2q and 2q + 1 are the 32 K bytes lane (row, q) feeds one 16x16x128 product
+        const v8i wl = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+        const v4i xa = x[2 * t], xb = x[2 * t + 1];
+        const v8i xl8 = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
+        accs[t & 3] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wl, xl8, accs[t & 3], 0, 0, 0, 0, 0, 0);
+      }
     }
   };
   for (int l0 = 0; l0 < nline; l0 += 2 * GM_LINES) {
@@ -579,16 +654,16 @@ __global__ __launch_bounds__(GM_MAX_WAVES * 64) void gemv_mfma_kernel(GemvArgs p
     if (l0 + 3 * GM_LINES < nline) wload(l0 + 3 * GM_LINES, wb);
   }
 
-  v4i acc = (accs[0] + accs[1]) + (accs[2] + accs[3]);
+  accv acc = (accs[0] + accs[1]) + (accs[2] + accs[3]);
   // sum the K parts: all but the first wavefront of each group park their 4 sums in LDS
   __syncthreads();  // everyone is done reading the token codes: the buffer is reused
   int* part = reinterpret_cast<int*>(xs) + grp * (ksplit - 1) * 256;
   if (kh != 0) {
-    *reinterpret_cast<v4i*>(part + (kh - 1) * 256 + lane * 4) = acc;
+    *reinterpret_cast<accv*>(part + (kh - 1) * 256 + lane * 4) = acc;
   }
   __syncthreads();
   if (kh != 0) return;
-  for (int k = 0; k < ksplit - 1; ++k) acc += *reinterpret_cast<const v4i*>(part + k * 256 + lane * 4);
+  for (int k = 0; k < ksplit - 1; ++k) acc += *reinterpret_cast<const accv*>(part + k * 256 + lane * 4);  // fp32: a fixed order
 
   if (tok >= M) return;
   float y[4];
@@ -629,7 +704,7 @@ static bool gemv_mfma_ok(int64_t M, int64_t K) {
   return M > GV_MFMA_MIN_M && (K % 256) == 0 && 16 * (K + 16) + 64 + 16 <= GV_MAX_LDS;
 }
 
-static int launch_gemv_mfma(GemvArgs a, hipStream_t st) {
+static int launch_gemv_mfma(GemvArgs a, hipStream_t st, bool fp8 = false) {
   // 2 row groups x 2 K parts per workgroup by default; with too few rows for that to give every
   // compute unit a workgroup, one row group per workgroup and up to 8 K parts
   a.ksplit = 2;
@@ -647,15 +722,19 @@ static int launch_gemv_mfma(GemvArgs a, hipStream_t st) {
   // one round of token-code loads ahead of the weights covers 8 vectors per thread; longer rows take three
   const bool long_rows = (int64_t)16 * (a.K / 16) > (int64_t)8 * a.ksplit * a.groups * 64;
   using kern_t = void (*)(GemvArgs);
-  static const kern_t table[2][2][2] = {
-      {{gemv_mfma_kernel<0, 0, false, 1>, gemv_mfma_kernel<0, 0, false, 3>},
-       {gemv_mfma_kernel<0, 0, true, 1>, gemv_mfma_kernel<0, 0, true, 3>}},
-      {{gemv_mfma_kernel<2, 2, false, 1>, gemv_mfma_kernel<2, 2, false, 3>},
-       {gemv_mfma_kernel<2, 2, true, 1>, gemv_mfma_kernel<2, 2, true, 3>}}};
-  const kern_t fn = table[fixed][res][long_rows];
+  static const kern_t table[2][2][2][2] = {
+      {{{gemv_mfma_kernel<0, 0, false, 1>, gemv_mfma_kernel<0, 0, false, 3>},
+        {gemv_mfma_kernel<0, 0, true, 1>, gemv_mfma_kernel<0, 0, true, 3>}},
+       {{gemv_mfma_kernel<2, 2, false, 1>, gemv_mfma_kernel<2, 2, false, 3>},
+        {gemv_mfma_kernel<2, 2, true, 1>, gemv_mfma_kernel<2, 2, true, 3>}}},
+      {{{gemv_mfma_kernel<0, 0, false, 1, 0, false, true>, gemv_mfma_kernel<0, 0, false, 3, 0, false, true>},
+        {gemv_mfma_kernel<0, 0, true, 1, 0, false, true>, gemv_mfma_kernel<0, 0, true, 3, 0, false, true>}},
+       {{gemv_mfma_kernel<2, 2, false, 1, 0, false, true>, gemv_mfma_kernel<2, 2, false, 3, 0, false, true>},
+        {gemv_mfma_kernel<2, 2, true, 1, 0, false, true>, gemv_mfma_kernel<2, 2, true, 3, 0, false, true>}}}};
+  const kern_t fn = table[fp8][fixed][res][long_rows];
   if (lds > 64 * 1024) {
-    static LdsOptIn opted[8];
-    const int e = opted[fixed * 4 + res * 2 + long_rows].ensure(reinterpret_cast<const void*>(fn));
+    static LdsOptIn opted[16];
+    const int e = opted[fp8 * 8 + fixed * 4 + res * 2 + long_rows].ensure(reinterpret_cast<const void*>(fn));
     if (e) return e;
   }
   hipLaunchKernelGGL(fn, dim3(grid), dim3(a.ksplit * a.groups * 64), lds, st, a);
@@ -674,7 +753,7 @@ static bool gemv_mfma_fq_ok(int64_t M, int64_t N, int64_t K) {
   return M >= 9 || (M >= 5 && N >= 8192) || (M >= 3 && wide);
 }
 
-static int launch_gemv_mfma_fq(GemvArgs a, hipStream_t st) {
+static int launch_gemv_mfma_fq(GemvArgs a, hipStream_t st, bool fp8 = false) {
   // 32 weight rows per workgroup (2 row groups x 4 K parts) while that gives every workgroup a compute unit
   // of its own; beyond that 64 rows (4 row groups x 2 K parts): a second round of workgroups would repeat
   // the row quantisation behind the first (N = 11264, 8 tokens: 9.9 -> 7.1 us).
@@ -692,7 +771,13 @@ static int launch_gemv_mfma_fq(GemvArgs a, hipStream_t st) {
     {gemv_mfma_kernel<KS, GR, true, 1, 16, false>, gemv_mfma_kernel<KS, GR, true, 1, 16, true>}}}
   static const kern_t table[2][2][2][2] = {AQ_FQ_TABLE(4, 2), AQ_FQ_TABLE(2, 4)};
 #undef AQ_FQ_TABLE
-  hipLaunchKernelGGL(table[wide][res][many][norm], dim3(grid), dim3(8 * 64), lds, st, a);
+#define AQ_FQ8_TABLE(KS, GR)                                                                                       \
+  {{gemv_mfma_kernel<KS, GR, false, 1, 8, false, true>, gemv_mfma_kernel<KS, GR, false, 1, 16, false, true>},      \
+   {gemv_mfma_kernel<KS, GR, true, 1, 8, false, true>, gemv_mfma_kernel<KS, GR, true, 1, 16, false, true>}}
+  static const kern_t table8[2][2][2] = {AQ_FQ8_TABLE(4, 2), AQ_FQ8_TABLE(2, 4)};
+#undef AQ_FQ8_TABLE
+  const kern_t fn = fp8 ? table8[wide][res][many] : table[wide][res][many][norm];
+  hipLaunchKernelGGL(fn, dim3(grid), dim3(8 * 64), lds, st, a);
   return (int)hipGetLastError();
 }
 
@@ -826,6 +911,82 @@ extern "C" int aq_gemv_w8a8_decode_residual(const void* x, int x_dtype, const in
   rc = aq_quant_rowwise_i8(x, x_dtype, M, K, K, xq, sx, stream);
   if (rc) return rc;
   return aq_gemv_w8a8_codes_residual(xq, sx, wq, sw, bias, bias_dtype, residual, y, y_dtype, M, N, K, stream);
+}
+
+// ---------------------------------------------------------------------------
+// FP8 decode: the same streaming GEMV on e4m3 codes with per-tensor scales.  Shapes the kernel does not take
+// (K not in whole 256-byte steps, rows too long for the LDS) go to the tiled FP8 GEMM, which takes any M.
+extern "C" size_t aq_gemv_fp8_workspace_bytes(int64_t M, int64_t K) {
+  if (M < 0 || K < 0) return 0;
+  return aq::align256((size_t)(M * K)) + 256 + AQ_FP8_AMAX_WS_BYTES;  // codes, the scale, the quantiser's partial maxima
+}
+
+static int gemv_fp8_check(const uint8_t* wq, const float* sw, const void* bias, int bias_dtype, const void* residual,
+                          const void* y, int y_dtype, int64_t M, int64_t N, int64_t K) {
+  if (y_dtype != AQ_F32 && y_dtype != AQ_BF16) return AQ_E_DTYPE;
+  if (bias && bias_dtype != AQ_F32 && bias_dtype != AQ_BF16) return AQ_E_DTYPE;
+  if (M < 0 || M > 16 || N < 0 || K <= 0 || (K % 16) != 0) return AQ_E_SHAPE;
+  if (M == 0 || N == 0) return AQ_OK;
+  if (!wq || !sw || !y) return AQ_E_NULL;
+  if (aq::check_ptr16(wq) || aq::check_ptr16(y) || aq::check_ptr16(residual)) return AQ_E_ALIGN;
+  if (aq::check_ptr(sw, 4) || aq::check_ptr(bias, bias_dtype == AQ_BF16 ? 2 : 4)) return AQ_E_ALIGN;
+  if (N > (1 << 25) || K > (1 << 22)) return AQ_E_RANGE;
+  return AQ_OK;
+}
+
+static aq::GemvArgs gemv_fp8_args(const uint8_t* wq, const float* sw, const void* bias, int bias_dtype,
+                                  const void* residual, void* y, int y_dtype, int64_t M, int64_t N, int64_t K) {
+  aq::GemvArgs a{};
+  a.wq = reinterpret_cast<const int8_t*>(wq);
+  a.sw = sw;
+  a.bias = bias;
+  a.res = residual;
+  a.ldr = N;
+  a.y = y;
+  a.M = (int)M;
+  a.N = (int)N;
+  a.K = (int)K;
+  a.bias_dtype = bias_dtype;
+  a.y_dtype = y_dtype;
+  return a;
+}
+
+static bool gemv_fp8_ok(int64_t K) { return (K % 256) == 0 && 16 * (K + 16) + 64 + 16 <= aq::GV_MAX_LDS; }
+
+extern "C" int aq_gemv_fp8_codes_residual(const uint8_t* xq, const float* sx, const uint8_t* wq, const float* sw,
+                                          const void* bias, int bias_dtype, const void* residual, void* y, int y_dtype,
+                                          int64_t M, int64_t N, int64_t K, void* stream) {
+  int rc = gemv_fp8_check(wq, sw, bias, bias_dtype, residual, y, y_dtype, M, N, K);
+  if (rc || M == 0 || N == 0) return rc;
+  if (!xq || !sx) return AQ_E_NULL;
+  if (aq::check_ptr16(xq) || aq::check_ptr(sx, 4)) return AQ_E_ALIGN;
+  if (!gemv_fp8_ok(K)) return aq_linear_fp8_residual(xq, sx, wq, sw, bias, bias_dtype, residual, y, y_dtype, M, N, K, stream);
+  aq::GemvArgs a = gemv_fp8_args(wq, sw, bias, bias_dtype, residual, y, y_dtype, M, N, K);
+  a.xq = reinterpret_cast<const int8_t*>(xq);
+  a.sx = sx;
+  return aq::launch_gemv_mfma(a, static_cast<hipStream_t>(stream), true);
+}
+
+extern "C" int aq_gemv_fp8_decode_residual(const void* x, int x_dtype, const uint8_t* wq, const float* sw,
+                                           const void* bias, int bias_dtype, const void* residual, void* y, int y_dtype,
+                                           int64_t M, int64_t N, int64_t K, void* ws, size_t ws_bytes, void* stream) {
+  if (x_dtype != AQ_F32 && x_dtype != AQ_BF16) return AQ_E_DTYPE;
+  int rc = gemv_fp8_check(wq, sw, bias, bias_dtype, residual, y, y_dtype, M, N, K);
+  if (rc || M == 0 || N == 0) return rc;
+  if (!x || !ws) return AQ_E_NULL;
+  if (aq::check_ptr16(x) || aq::check_ptr16(ws)) return AQ_E_ALIGN;
+  if (ws_bytes < aq_gemv_fp8_workspace_bytes(M, K)) return AQ_E_WORKSPACE;
+  if (x_dtype == AQ_BF16 && K <= 2048 && (K % 512) == 0) {  // one launch: the kernel casts the rows itself
+    aq::GemvArgs a = gemv_fp8_args(wq, sw, bias, bias_dtype, residual, y, y_dtype, M, N, K);
+    a.x = x;
+    return aq::launch_gemv_mfma_fq(a, static_cast<hipStream_t>(stream), true);
+  }
+  uint8_t* xq = static_cast<uint8_t*>(ws);
+  float* sx = reinterpret_cast<float*>(static_cast<char*>(ws) + aq::align256((size_t)(M * K)));
+  uint32_t* amax_ws = reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(sx) + 256);
+  rc = aq_quant_tensor_fp8(x, x_dtype, M * K, xq, sx, amax_ws, stream);
+  if (rc) return rc;
+  return aq_gemv_fp8_codes_residual(xq, sx, wq, sw, bias, bias_dtype, residual, y, y_dtype, M, N, K, stream);
 }
 
 // ---------------------------------------------------------------------------

@@ -222,6 +222,9 @@ class Fp8Linear(Linear):
         self.register_buffer("qweight", torch.zeros((out_dim, in_dim), dtype=torch.uint8, device=device))
         self.register_buffer("w_scale", torch.ones((1,), dtype=torch.float32, device=device))
         self.bias = nn.Parameter(torch.zeros(out_dim, device=device), requires_grad=False) if bias else None
+        self._workspaces: dict = {}  # decode workspaces, one per (device, stream), as in QuantLinear
+
+    DECODE_MAX_ROWS = 16
 
     @classmethod
     def from_linear(cls, base: nn.Module) -> "Fp8Linear":
@@ -260,8 +263,18 @@ class Fp8Linear(Linear):
         x2 = x.reshape(-1, x.shape[-1])
         if x2.shape[1] != self.qweight.shape[1]:
             raise ValueError(f"expected last dim {self.qweight.shape[1]}, got {x2.shape[1]}")
-        xq, sx = ops.quant_tensor_fp8(x2)
-        y = ops.linear_fp8(xq, sx, self.qweight, self.w_scale, self.bias, out_dtype=x.dtype, residual=residual)
+        if x2.shape[0] <= self.DECODE_MAX_ROWS:  # decode step: the weight-streaming GEMV
+            ops._need_gpu(x, self.qweight)
+            need = 16 * self.qweight.shape[1] + 2048
+            key = (x.device, torch.cuda.current_stream(x.device).cuda_stream)
+            ws = self._workspaces.get(key)
+            if ws is None or ws.numel() < need:
+                ws = self._workspaces[key] = torch.empty((need,), dtype=torch.uint8, device=x.device)
+            y = ops.gemv_fp8_decode(x2, self.qweight, self.w_scale, self.bias, out_dtype=x.dtype, workspace=ws,
+                                    residual=residual)
+        else:
+            xq, sx = ops.quant_tensor_fp8(x2)
+            y = ops.linear_fp8(xq, sx, self.qweight, self.w_scale, self.bias, out_dtype=x.dtype, residual=residual)
         return y.reshape(*lead, self.qweight.shape[0])
 
 

@@ -633,3 +633,74 @@ def linear_fp8(xq, sx, wq, sw, bias=None, out_dtype=torch.bfloat16, residual=Non
     elif r is not None:
         y.copy_(r.view(M, N))
     return y
+
+
+def gemv_fp8_codes(xq, sx, wq, sw, bias=None, out_dtype=torch.bfloat16, residual=None) -> torch.Tensor:
+    """The FP8 decode GEMV on codes the caller already holds (at most 16 rows; ``sx``, ``sw`` device scalars)."""
+    _need_gpu(xq, sx, wq, sw, bias, residual)
+    if xq.dtype != torch.uint8 or wq.dtype != torch.uint8 or xq.dim() != 2 or wq.dim() != 2 or xq.shape[1] != wq.shape[1]:
+        raise ValueError(f"gemv_fp8_codes takes e4m3fn codes as uint8 [M, K] and [N, K], got {tuple(xq.shape)} / {tuple(wq.shape)}")
+    M, K = xq.shape
+    N = wq.shape[0]
+    if M > 16:
+        raise ValueError(f"the decode path takes at most 16 rows, got {M}")
+    _check_k(K)
+    if sx.dtype != torch.float32 or sw.dtype != torch.float32 or sx.numel() != 1 or sw.numel() != 1:
+        raise ValueError("sx and sw must be float32 device scalars")
+    if out_dtype not in _DT:
+        raise ValueError(f"out_dtype {out_dtype} is not supported")
+    xq, wq = xq.contiguous(), wq.contiguous()
+    b, bdt = _bias_args(bias, N)
+    r = _residual_arg(residual, M, N, out_dtype, xq.device)
+    y = torch.empty((M, N), dtype=out_dtype, device=xq.device)
+    if M and N:
+        with _OnDevice(xq.device):
+            rc = _abi.load().aq_gemv_fp8_codes_residual(xq.data_ptr(), sx.data_ptr(), wq.data_ptr(), sw.data_ptr(),
+                                                        b.data_ptr() if b is not None else None, bdt,
+                                                        r.data_ptr() if r is not None else None, y.data_ptr(),
+                                                        _DT[out_dtype], M, N, K, _stream(xq))
+        _abi.check(rc, "aq_gemv_fp8_codes")
+    elif r is not None:
+        y.copy_(r.view(M, N))
+    return y
+
+
+def gemv_fp8_decode(x, wq, sw, bias=None, out_dtype=None, workspace: Optional[torch.Tensor] = None,
+                    residual=None) -> torch.Tensor:
+    """FP8 decode path for at most 16 rows of ``x [M, K]``: per-tensor e4m3 cast + GEMV + epilogue, one launch for
+    bfloat16 rows of at most 2048 elements."""
+    _need_gpu(x, wq, sw, bias, workspace, residual)
+    x2 = _rows(x, "gemv_fp8_decode")
+    M, K = x2.shape
+    N = wq.shape[0]
+    if M > 16:
+        raise ValueError(f"the decode path takes at most 16 rows, got {M}")
+    if wq.dtype != torch.uint8 or wq.dim() != 2 or wq.shape[1] != K:
+        raise ValueError(f"wq must be uint8 (e4m3fn codes) [N, {K}], got {wq.dtype} {tuple(wq.shape)}")
+    _check_k(K)
+    if sw.dtype != torch.float32 or sw.numel() != 1:
+        raise ValueError("sw must be a float32 device scalar")
+    out_dtype = out_dtype or x.dtype
+    if out_dtype not in _DT:
+        raise ValueError(f"out_dtype {out_dtype} is not supported")
+    wq = wq.contiguous()
+    b, bdt = _bias_args(bias, N)
+    lib = _abi.load()
+    need = lib.aq_gemv_fp8_workspace_bytes(M, K)
+    if workspace is None:
+        workspace = torch.empty((max(need, 16),), dtype=torch.uint8, device=x.device)
+    elif workspace.numel() * workspace.element_size() < need:
+        raise ValueError(f"workspace holds {workspace.numel() * workspace.element_size()} bytes, {need} needed")
+    r = _residual_arg(residual, M, N, out_dtype, x.device)
+    y = torch.empty((M, N), dtype=out_dtype, device=x.device)
+    if M and N:
+        with _OnDevice(x.device):
+            rc = lib.aq_gemv_fp8_decode_residual(x2.data_ptr(), _dt(x2, "x"), wq.data_ptr(), sw.data_ptr(),
+                                                 b.data_ptr() if b is not None else None, bdt,
+                                                 r.data_ptr() if r is not None else None, y.data_ptr(), _DT[out_dtype],
+                                                 M, N, K, workspace.data_ptr(),
+                                                 workspace.numel() * workspace.element_size(), _stream(x))
+        _abi.check(rc, "aq_gemv_fp8_decode")
+    elif r is not None:
+        y.copy_(r.view(M, N))
+    return y

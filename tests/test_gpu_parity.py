@@ -499,6 +499,54 @@ def test_linear_fp8_within_tolerance(oracle, tile, M, N, K):
             assert rc == 0 and torch.equal(y_in_place, ops.linear_fp8(*args, out_dtype=dt) + r)
 
 
+@pytest.mark.parametrize("M", [1, 3, 8, 9, 16])
+@pytest.mark.parametrize("N,K", [(8192, 2048), (77, 512), (11264, 1024), (300, 4096), (130, 1040)])
+def test_gemv_fp8_decode_within_tolerance(oracle, M, N, K):
+    """The FP8 Linear at decode sizes: (8192, 2048), (77, 512) and (11264, 1024) cast their bf16 rows inside the
+    GEMV kernel (32- and 64-row workgroups, a ragged single workgroup); (300, 4096) goes through the workspace
+    (quantiser + GEMV on codes); (130, 1040) is handed to the tiled GEMM.  All against the float64 sum of the
+    oracle's codes, and the fused cast against the codes path (a wrong code would move an output by far more
+    than a change of summation order)."""
+    _say("gemv_fp8", M, N, K)
+    g = torch.Generator().manual_seed(M * 13 + N)
+    x = (torch.randn(M, K, generator=g) * (0.2 + 3 * torch.rand(M, 1, generator=g))).to(torch.bfloat16)
+    w = make_x(N, K, 52) * 0.02
+    xq, sx = oracle.c_quant_tensor_fp8(bf16_bits(x), bf16_bits=True)
+    wq, sw = oracle.c_quant_tensor_fp8(w.numpy())
+    bias = torch.randn(N, generator=g) * 0.3
+    wqd, swd = torch.from_numpy(wq).to(DEV), torch.tensor([sw], device=DEV)
+    exact = oracle.np_linear_fp8(xq, sx, wq, sw, bias=bias.numpy())
+    rms = float(np.sqrt(np.mean(exact.astype(np.float64) ** 2)))
+    y32 = ops.gemv_fp8_decode(x.to(DEV), wqd, swd, bias.to(DEV), out_dtype=torch.float32)
+    assert np.max(np.abs(to_np(y32) - exact)) <= 1e-3 * rms
+    yb = ops.gemv_fp8_decode(x.to(DEV), wqd, swd, bias.to(DEV), out_dtype=torch.bfloat16)
+    np.testing.assert_allclose(to_np(yb.float()), exact, rtol=1e-2, atol=1e-2 * rms)   # stated tolerance
+    # the library's own quantiser gives the oracle's codes; the GEMV on them agrees with the fused launch
+    xqd, sxd = ops.quant_tensor_fp8(x.to(DEV))
+    assert np.array_equal(to_np(xqd), xq) and float(sxd.item()) == float(sx)
+    yc = ops.gemv_fp8_codes(xqd, sxd, wqd, swd, bias.to(DEV), out_dtype=torch.float32)
+    assert np.max(np.abs(to_np(yc) - to_np(y32))) <= 2e-5 * rms
+    # and with the tiled GEMM on the same codes
+    yg = ops.linear_fp8(xqd, sxd, wqd, swd, bias.to(DEV), out_dtype=torch.float32)
+    assert np.max(np.abs(to_np(yg) - to_np(y32))) <= 2e-5 * rms
+    r = torch.randn(M, N, generator=g).to(torch.bfloat16).to(DEV)
+    assert torch.equal(ops.gemv_fp8_decode(x.to(DEV), wqd, swd, bias.to(DEV), out_dtype=torch.bfloat16, residual=r), yb + r)
+
+
+def test_fp8_linear_module_decode_rows_take_the_gemv_and_match_the_prefill_path():
+    torch.manual_seed(9)
+    lin = Linear(2048, 512)
+    lin.reset_parameters()
+    f = Fp8Linear.from_linear(lin.to(DEV))
+    x = torch.randn(40, 2048, device=DEV, dtype=torch.bfloat16)
+    with torch.inference_mode():
+        big = f(x)                                   # 40 rows: quantiser + tiled GEMM, one scale for all 40
+        small = f(x[:16])                            # 16 rows: the GEMV, one scale for these 16
+    ref = torch.nn.functional.linear(x.float(), lin.weight)
+    assert ((big.float() - ref).norm() / ref.norm()).item() < 0.08
+    assert ((small.float() - ref[:16]).norm() / ref[:16].norm()).item() < 0.08
+
+
 def test_fp8_linear_module_with_a_bias_and_a_residual(oracle):
     """Fp8Linear keeps the reference's optional bias (linear.py:11) and takes the residual stream like QuantLinear."""
     torch.manual_seed(8)

@@ -30,17 +30,23 @@ namespace aq {
 //   <2, 2, 2, 2, 2, 128, 4>  128 x 128 tile, 8 wavefronts: the two that share a 64 x 64 sub-tile split every
 //                            K step and exchange half of their accumulators through LDS at the end, so that
 //                            each finishes (and stores) 32 x 64 of the sums; 4 stages of 32 KiB;
-// Shapes that only the lab build instantiates (measured, none faster: under a matrix-core load with real
-// operand data this part runs against its power limit, and fewer LDS reads per MFMA buy clock, not rate;
-// with one wavefront per SIMD every fragment read also delays that SIMD's next MFMA, which a second
-// wavefront otherwise covers.  Two independent 4-wavefront workgroups per compute unit, 256 x 128 or
-// 128 x 128 tiles with 64-byte stages, were measured too: 8192^3 in 459 and 556 us against 310 us with
-// all-zero operands):
+// Shapes that only the lab build instantiates.  Measured, none faster on int8 with real operand data: under a
+// matrix-core load with toggling operands this part runs against its power limit, and fewer LDS reads per MFMA
+// buy clock, not rate (8192^3: 2.31-2.42 POP/s for every shape below and for the 256 x 128 tile alike, while the
+// clock moves between 1.47 and 1.65 GHz).  FP8, which is throttled less, gains 8 % from the first one at 8192^3
+// (2.6 against 2.4 PFLOP/s); no benchmark configuration has enough 256 x 256 tiles to use it.
 //   <2, 2, 4, 4, 1, 64, 4>   256 x 256 tile, 4 wavefronts (one per SIMD) of 128 x 128: 256 accumulator
 //                            registers per lane (the AGPR half of the register file), 8 fragment reads per
-//                            16 MFMAs instead of 16, half the LDS fill per MFMA; 4 stages of 32 KiB;
+//                            16 MFMAs instead of 16, half the LDS fill per MFMA; 4 stages of 32 KiB; whole K
+//                            steps, whole 256-row multiples, even N, no residual (one K-loop and one epilogue
+//                            variant: with all three epilogues and both K loops the kernel was 45 000 lines of
+//                            machine code whose spilled values came back from scratch one memory round trip at a
+//                            time, 45 k cycles of epilogue per tile; now 12-16 k);
 //   <4, 2, 2, 4, 1, 64, 4>   256 x 256 tile, 8 wavefronts of 64 x 128: 6 fragment reads per 8 MFMAs;
 //   <2, 2, 4, 2, 1, 128, 3>  256 x 128 tile, 4 wavefronts of 128 x 64.
+// Two independent 4-wavefront workgroups per compute unit (256 x 128 or 128 x 128 tiles with 64-byte stages, so
+// that one's epilogue overlaps the other's loop) were measured too: 8192^3 in 459 and 556 us against 310 us with
+// all-zero operands.
 template <int WM_, int WN_, int TM_, int TN_, int WK_, int BK_, int NSTAGE_>
 struct Shape {
   static constexpr int WM = WM_, WN = WN_, TM = TM_, TN = TN_, WK = WK_, BK = BK_, NSTAGE = NSTAGE_;
@@ -48,7 +54,12 @@ struct Shape {
   static constexpr int WAVE_M = 32 * TM, WAVE_N = 32 * TN;
   static constexpr int BM = WM * WAVE_M, BN = WN * WAVE_N;
   static constexpr int STAGE = (BM + BN) * BK;
-  static constexpr int LDS_BYTES = NSTAGE * STAGE;
+  // Sub-tiles of 16 accumulators (128 x 128 per wavefront): the 256 accumulator registers leave no room to hold a
+  // lane's 64 per-row scales through the K loop, so the tile's BM scales wait in LDS behind the stages instead;
+  // such shapes also compile one K-loop variant (whole K steps) and one epilogue variant only (see gemm_kernel).
+  static constexpr bool BIG = TM * TN >= 16;
+  static constexpr int SX_BYTES = BIG ? BM * 4 : 0;
+  static constexpr int LDS_BYTES = NSTAGE * STAGE + SX_BYTES;
   static_assert(BK == 64 || BK == 128, "K bytes per stage");
   static_assert(NWAVES % 2 == 0, "the piece permutation assumes a wavefront's row groups share parity");
   static_assert((BM * BK / 1024) % NWAVES == 0 && (BN * BK / 1024) % NWAVES == 0, "whole 1 KiB loads per wavefront");
@@ -163,7 +174,7 @@ __device__ __forceinline__ void sched_pattern() {
 }
 
 #ifdef AQ_LAB
-__device__ long long aq_lab_clock[4];
+__device__ long long aq_lab_clock[16];
 #endif
 // EXACT: K is a whole number of BK-byte steps, so every 16-byte piece of every step lies inside its row and the
 // global->LDS loads need no per-lane range logic: a loop-invariant lane offset per row group and the K step as a
@@ -173,7 +184,9 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, uint8_t* smem, int 
   constexpr int WM = S::WM, WN = S::WN, TM = S::TM, TN = S::TN, WK = S::WK, BK = S::BK, NSTAGE = S::NSTAGE;
   constexpr int NWAVES = S::NWAVES, NTHREADS = S::NTHREADS, WAVE_M = S::WAVE_M, WAVE_N = S::WAVE_N;
   constexpr int BM = S::BM, BN = S::BN, STAGE = S::STAGE;
+  constexpr bool BIG = S::BIG;
   static_assert(TM % WK == 0, "the K-split pair divides the sub-tile's row blocks");
+  static_assert(!BIG || (EXACT && WK == 1), "big sub-tiles: whole K steps, no K-split pair");
   constexpr int TME = TM / WK;  // row blocks a wavefront finishes and stores
   constexpr int A_LOADS = BM * BK / 16 / NTHREADS;  // 16-byte vectors per thread per K step
   constexpr int B_LOADS = BN * BK / 16 / NTHREADS;
@@ -251,6 +264,9 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, uint8_t* smem, int 
                                                0, 0, 0);
   };
 
+#ifdef AQ_LAB_STALL
+  const long long tl_start = clock64();
+#endif
   using acc_t = typename Acc<FP8>::type;
   acc_t acc[TM][TN];
 #pragma unroll
@@ -392,7 +408,8 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, uint8_t* smem, int 
   // as one scalar per 32x32 tile column.  Nothing is done with the values until
   // the epilogue (bias stays a raw bit pattern), so no wait is placed here.
   float sx1 = 1.0f, sw1 = 1.0f;
-  float sxr[TME][4][4];  // [i][g][q]: row mw + i*32 + g*8 + rq + q
+  float sxr[BIG ? 1 : TME][4][4];  // [i][g][q]: row mw + i*32 + g*8 + rq + q (big sub-tiles: in LDS instead)
+  float* const sx_lds = reinterpret_cast<float*>(smem + NSTAGE * STAGE);  // [BM], big sub-tiles only
   float swn[TN];
   uint32_t bias_raw[TN];
   const bool has_bias = OUT != OUT_I32 && p.bias != nullptr;
@@ -414,7 +431,14 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, uint8_t* smem, int 
       const int rows_left = __builtin_amdgcn_readfirstlane((M - mw) > 0 ? (M - mw) : 0);
       const __amdgpu_buffer_rsrc_t Sr =
           make_rsrc(p.sx + (rows_left ? mw : 0), (uint32_t)(rows_left < 32 * TME ? rows_left : 32 * TME) * 4u);
-      if ((M & 3) == 0) {  // uniform: the 4 rows of a float4 are all in or all out, and 16-byte aligned
+      if constexpr (BIG) {
+        // the tile's BM scales straight into LDS, 64 per load instruction; rows past M read as zero
+        const __amdgpu_buffer_rsrc_t Tr = make_rsrc(p.sx + m0, (uint32_t)rows_a * 4u);
+#pragma unroll
+        for (int r = 0; r < BM / 64 / NWAVES; ++r)
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(Tr, (lds_void*)(sx_lds + (r * NWAVES + wave) * 64), 4,
+                                                   (uint32_t)((r * NWAVES + wave) * 64 + lane) * 4u, 0, 0, 0);
+      } else if ((M & 3) == 0) {  // uniform: the 4 rows of a float4 are all in or all out, and 16-byte aligned
 #pragma unroll
         for (int i = 0; i < TME; ++i)
 #pragma unroll
@@ -475,6 +499,9 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, uint8_t* smem, int 
 
   AQ_WAIT_VMCNT((NSTAGE - 1) * NLOADS);  // all but the younger stages: stage 0 (and the operands) have landed
   AQ_BARRIER();
+#ifdef AQ_LAB_STALL
+  const long long tl_stage0 = clock64();
+#endif
   load_frags(smem, 0, af[0], bf[0]);
   middle_slots(k0{}, smem, no{}, 0, 0);  // no loads to issue yet: every stage buffer is in flight
   __builtin_amdgcn_s_waitcnt(0xc07f);        // lgkmcnt(0): the last fragments of stage 0 are in registers
@@ -519,9 +546,12 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, uint8_t* smem, int 
   }
   AQ_WAIT_VMCNT(0);  // drain the padding loads before the workgroup's LDS can be released or reused
 #ifdef AQ_LAB_STALL
+  const long long tl_loop_end = clock64();
   if (blockIdx.x == 0 && threadIdx.x == 0) {
     aq_lab_clock[2] = st_sum + (st_t1 - st_t0);
-    aq_lab_clock[3] = clock64() - st_begin;
+    aq_lab_clock[3] = tl_loop_end - st_begin;
+    aq_lab_clock[4] = tl_stage0 - tl_start;   // tile start -> first stage landed and visible
+    aq_lab_clock[5] = st_begin - tl_stage0;   // first K step without loads
   }
 #endif
 
@@ -590,7 +620,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, uint8_t* smem, int 
       make_rsrc(reinterpret_cast<uint8_t*>(p.C) + ((int64_t)mw * N + nw) * ESZ, 0x40000000u);
   // Residual: the same window over the tensor that is added to the rounded output; each lane
   // reads exactly the elements it then writes, so the residual may be the output itself.
-  const bool has_res = OUT != OUT_I32 && p.res != nullptr;  // uniform
+  const bool has_res = !BIG && OUT != OUT_I32 && p.res != nullptr;  // uniform (big sub-tiles are not launched with a residual)
   const __amdgpu_buffer_rsrc_t Rr = make_rsrc(
       reinterpret_cast<const uint8_t*>(has_res ? p.res : p.C) + ((int64_t)mw * N + nw) * ESZ, has_res ? 0x40000000u : 0u);
   const bool pair_ok = (N & 1) == 0;  // uniform: bf16 rows start dword-aligned, pairs never straddle N
@@ -661,6 +691,9 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, uint8_t* smem, int 
             }
           } else {
             float y[4];
+            v4f sxq = {0.0f, 0.0f, 0.0f, 0.0f};
+            if constexpr (BIG && !FP8)
+              sxq = *reinterpret_cast<const v4f*>(sx_lds + (mw - m0) + r0 + rq);
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
               if constexpr (FP8) {
@@ -671,7 +704,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, uint8_t* smem, int 
                 // three separately rounded fp32 operations, never contracted.  Without a bias
                 // bn is +0: the product of an integer and two positive scales is never -0,
                 // so adding it changes no bit.
-                y[q] = __fadd_rn(__fmul_rn(__fmul_rn((float)acc[i][j][g * 4 + q], sxr[i][g][q]), swn[j]), bn);
+                y[q] = __fadd_rn(__fmul_rn(__fmul_rn((float)acc[i][j][g * 4 + q], BIG ? sxq[q] : sxr[BIG ? 0 : i][g][q]), swn[j]), bn);
               }
             }
             if constexpr (OUT == OUT_F32) {
@@ -715,12 +748,22 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, uint8_t* smem, int 
       }
     }
   };
-  if (rows_inside && pair_ok)
-    store_all(no{}, yes{});   // interior tiles: straight-line, no per-row checks
-  else if (pair_ok)
-    store_all(yes{}, yes{});
-  else
-    store_all(yes{}, no{});
+  if constexpr (BIG) {
+    store_all(no{}, yes{});  // one variant (256 outputs per lane): the launcher sends ragged M and odd N to another shape
+  } else {
+    if (rows_inside && pair_ok)
+      store_all(no{}, yes{});   // interior tiles: straight-line, no per-row checks
+    else if (pair_ok)
+      store_all(yes{}, yes{});
+    else
+      store_all(yes{}, no{});
+  }
+#ifdef AQ_LAB_STALL
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    aq_lab_clock[6] = clock64() - tl_loop_end;  // accumulator exchange (split K steps) + epilogue issue
+    aq_lab_clock[7] = clock64() - tl_start;     // the whole tile as wavefront 0 sees it
+  }
+#endif
 }
 
 // A workgroup walks tiles pid, pid + gridDim.x, ...: with more tiles than compute units the launch is one
@@ -743,7 +786,9 @@ __global__ __launch_bounds__(S::NTHREADS) void gemm_kernel(GemmArgs p) {
 #endif
   const bool exact = (p.K % S::BK) == 0;  // uniform
   for (int pid = blockIdx.x; pid < nt; pid += gridDim.x) {
-    if (exact)
+    if constexpr (S::BIG)
+      gemm_tile<FP8, OUT, S, true>(p, smem, pid);  // launched for whole K steps and even N only
+    else if (exact)
       gemm_tile<FP8, OUT, S, true>(p, smem, pid);
     else
       gemm_tile<FP8, OUT, S, false>(p, smem, pid);
@@ -792,7 +837,10 @@ static int launch(GemmArgs& a, hipStream_t st) {
     case TILE_SMALL: return launch_shape<FP8, OUT, ShapeSmall>(a, st);
 #ifdef AQ_LAB
     case TILE_TALL: return launch_shape<FP8, OUT, ShapeTall>(a, st);
-    case TILE_HUGE: return launch_shape<FP8, OUT, ShapeHuge>(a, st);
+    case TILE_HUGE:
+      if ((a.K % ShapeHuge::BK) == 0 && (a.N % 2) == 0 && (a.M % ShapeHuge::BM) == 0 && a.res == nullptr)
+        return launch_shape<FP8, OUT, ShapeHuge>(a, st);
+      return launch_shape<FP8, OUT, ShapeLarge>(a, st);
     case TILE_HUGE8: return launch_shape<FP8, OUT, ShapeHuge8>(a, st);
 #endif
     default: return launch_shape<FP8, OUT, ShapeLarge>(a, st);
@@ -826,7 +874,7 @@ static GemmArgs make_args(const void* A, const void* B, void* C, int64_t M, int6
 
 #ifdef AQ_LAB
 extern "C" int aq_lab_read_clock(long long* host2) {
-  return (int)hipMemcpyFromSymbol(host2, HIP_SYMBOL(aq::aq_lab_clock), 32);
+  return (int)hipMemcpyFromSymbol(host2, HIP_SYMBOL(aq::aq_lab_clock), 64);
 }
 extern "C" int aq_lab_set_gemm_tile(int rows) {
   if (rows != 0 && rows != 128 && rows != 256 && rows != 257 && rows != 512 && rows != 513) return AQ_E_SHAPE;

@@ -261,6 +261,33 @@ def test_gemm_with_more_tiles_than_compute_units(oracle, tile):
     assert torch.equal(y8.cpu(), ref)
 
 
+def test_lab_tile_256x256_on_shapes_it_takes(oracle):
+    """The lab build's 256 x 256 tile (four wavefronts of 128 x 128, accumulators in AGPRs, per-row scales through
+    LDS) takes whole 256-row multiples, even N and whole 64-byte K steps without a residual; anything else falls
+    back to the 256 x 128 tile.  Same bits as the oracle on both routes, int8 sums, fused epilogue and FP8."""
+    with _abi.lab_library() as lab:
+        assert lab.aq_lab_set_gemm_tile(512) == 0
+        for (M, N, K) in ((512, 768, 320), (256, 130, 64), (300, 256, 128), (512, 256, 80)):
+            _say("tile 256x256", M, N, K)
+            xq, wq = rand_codes(M, K, 91).numpy(), rand_codes(N, K, 92).numpy()
+            acc = ops.gemm_i8_i32(torch.from_numpy(xq).to(DEV), torch.from_numpy(wq).to(DEV))
+            assert np.array_equal(to_np(acc), oracle.c_gemm_i8_i32(xq, wq))
+            g = np.random.default_rng(93)
+            sx = (g.random(M) * 0.02 + 0.001).astype(np.float32)
+            sw = (g.random(N) * 0.002 + 0.0001).astype(np.float32)
+            b = (g.standard_normal(N) * 0.01).astype(np.float32)
+            y = ops.linear_w8a8(torch.from_numpy(xq).to(DEV), torch.from_numpy(sx).to(DEV), torch.from_numpy(wq).to(DEV),
+                                torch.from_numpy(sw).to(DEV), torch.from_numpy(b).to(DEV), out_dtype=torch.bfloat16)
+            want = oracle.c_dequant_epilogue(oracle.c_gemm_i8_i32(xq, wq), sx, sw, b, bf16_out=True)
+            assert np.array_equal(bf16_bits(y), want)
+            x8, s8 = oracle.c_quant_tensor_fp8(make_x(M, K, 94).numpy())
+            w8, t8 = oracle.c_quant_tensor_fp8((make_x(N, K, 95) * 0.02).numpy())
+            y8 = ops.linear_fp8(torch.from_numpy(x8).to(DEV), torch.tensor([s8], device=DEV), torch.from_numpy(w8).to(DEV),
+                                torch.tensor([t8], device=DEV), torch.from_numpy(b).to(DEV), out_dtype=torch.float32)
+            exact = oracle.np_linear_fp8(x8, s8, w8, t8, bias=b)
+            assert np.max(np.abs(to_np(y8) - exact)) <= 1e-3 * float(np.sqrt(np.mean(exact.astype(np.float64) ** 2)))
+
+
 def test_gemm_i8_extremes(oracle, tile):
     K = 8192
     xq = torch.full((40, K), 127, dtype=torch.int8)

@@ -548,6 +548,16 @@ def measure_ceilings(torch, ops, dev, calibrate=True):
             c = clocks.tolist()
             out[f"{name}_{tag}_{unit}"] = 256 * 4 * iters * 8 * ops_per / t / 1e12
             out[f"{name}_{tag}_clock_mhz"] = c[0] / max(c[1], 1) * 100.0
+    # fragment reads against the matrix pipe with one wavefront per SIMD, by placement (cycles per 32 MFMAs; 1024 = free)
+    issue = {}
+    for variant, label in ((0, "mfma_only"), (1, "one_read_behind_every_2nd_mfma"), (2, "eight_reads_first"),
+                           (3, "pairs_behind_every_4th_mfma")):
+        n_it = 2000
+        lab.aq_lab_probe_mfma_lds_issue(variant, 256, 50, sink.data_ptr(), clocks.data_ptr(), st)
+        lab.aq_lab_probe_mfma_lds_issue(variant, 256, n_it, sink.data_ptr(), clocks.data_ptr(), st)
+        torch.cuda.synchronize()
+        issue[label] = clocks.tolist()[0] / n_it
+    out["cycles_per_32_mfma_with_16_ds_read_b128_one_wavefront_per_simd"] = issue
     big = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
     t = timed(lambda i=0: lab.aq_lab_probe_read(big.data_ptr(), big.numel(), 0, 2048, 0, sink.data_ptr(), st), 3)
     out["hbm_stream_read_gbs"] = big.numel() / t / 1e9

@@ -67,6 +67,7 @@ LAB_SYMBOLS = {
     "aq_lab_probe_copy": (_int, [_vp, _vp, _i64, _int, _vp]),
     "aq_lab_probe_read": (_int, [_vp, _i64, _int, _int, _int, _vp, _vp]),
     "aq_lab_probe_empty": (_int, [_vp, _vp]),
+    "aq_lab_probe_mfma_lds_issue": (_int, [_int, _int, _int, _vp, _vp, _vp]),
 }
 
 _lib = None

@@ -36,6 +36,14 @@ int aq_lab_probe_copy(const void *src, void *dst, int64_t bytes, int workgroups,
 int aq_lab_probe_read(const void *src, int64_t bytes, int loads_per_lane, int workgroups, int nontemporal,
                       int *sink, void *stream);
 
+/* What fragment reads cost the matrix pipe with one wavefront per SIMD (4 per workgroup), by where they are issued:
+ * `iters` iterations of 32 MFMAs (i32_32x32x32_i8) and 16 ds_read_b128 in a ping-pong of two register sets (the MFMAs
+ * of one half consume what the reads of the other half filled).  variant 0: MFMAs only; 1: one read behind every
+ * second MFMA; 2: a half's eight reads first; 3: reads in pairs behind every fourth MFMA.  clocks: device int64[1]
+ * receiving the shader-clock cycles wavefront 0 of workgroup 0 spent in the loop (1024 per iteration is the matrix
+ * pipe's own time). */
+int aq_lab_probe_mfma_lds_issue(int variant, int workgroups, int iters, int *sink, long long *clocks, void *stream);
+
 /* One wavefront that does nothing: the cost of a launch. */
 int aq_lab_probe_empty(int *sink, void *stream);
 

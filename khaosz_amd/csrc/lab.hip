@@ -156,6 +156,70 @@ static int launch_read_upfront(const void* src, int64_t bytes, bool nt, int* sin
   return (int)hipGetLastError();
 }
 
+
+// What fragment reads cost the matrix pipe with ONE wavefront per SIMD, by where they are issued.  Every wavefront
+// runs `iters` iterations of 32 MFMAs (v_mfma_i32_32x32x32_i8, 8 accumulators in AGPRs) and 16 ds_read_b128 in a
+// ping-pong of two register sets: the MFMAs of one half consume what the reads of the other half filled, as a
+// GEMM's K loop does.  The instruction order is fixed in inline assembly.
+//   variant 0: MFMAs only (1024 cycles per iteration is the matrix pipe's own time)
+//   variant 1: one read behind every second MFMA
+//   variant 2: the eight reads of a half first, then its sixteen MFMAs
+//   variant 3: reads in pairs behind every fourth MFMA
+// clocks[0] receives the shader-clock cycles wavefront 0 of workgroup 0 spent in the loop.
+#define AQ_MF(acc, a, b) asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b))
+#define AQ_DR(dst, off) asm volatile("ds_read_b128 %0, %1 offset:" #off : "=&v"(dst) : "v"(addr))
+#define AQ_LGKM0() asm volatile("s_waitcnt lgkmcnt(0)")
+template <int V>
+__global__ __launch_bounds__(256) void probe_issue_kernel(int iters, int* sink, long long* clocks) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int i = threadIdx.x; i < 32768 / 4; i += 256) reinterpret_cast<int*>(lds)[i] = 0;
+  __syncthreads();
+  const unsigned addr = (unsigned)(wave * 1024 + lane * 16);
+  v16i c0 = {}, c1 = {}, c2 = {}, c3 = {}, c4 = {}, c5 = {}, c6 = {}, c7 = {};
+  v4i a0 = {0, 0, 0, 0}, a1 = a0, a2 = a0, a3 = a0, b0 = a0, b1 = a0, b2 = a0, b3 = a0;
+  v4i n0 = a0, n1 = a0, n2 = a0, n3 = a0, n4 = a0, n5 = a0, n6 = a0, n7 = a0;
+  const long long t0 = clock64();
+  for (int it = 0; it < iters; ++it) {
+    if constexpr (V == 0) {
+      AQ_MF(c0, n0, n4); AQ_MF(c1, n0, n5); AQ_MF(c2, n0, n6); AQ_MF(c3, n0, n7); AQ_MF(c4, n1, n4); AQ_MF(c5, n1, n5); AQ_MF(c6, n1, n6); AQ_MF(c7, n1, n7);
+      AQ_MF(c0, n2, n4); AQ_MF(c1, n2, n5); AQ_MF(c2, n2, n6); AQ_MF(c3, n2, n7); AQ_MF(c4, n3, n4); AQ_MF(c5, n3, n5); AQ_MF(c6, n3, n6); AQ_MF(c7, n3, n7);
+      AQ_MF(c0, a0, b0); AQ_MF(c1, a0, b1); AQ_MF(c2, a0, b2); AQ_MF(c3, a0, b3); AQ_MF(c4, a1, b0); AQ_MF(c5, a1, b1); AQ_MF(c6, a1, b2); AQ_MF(c7, a1, b3);
+      AQ_MF(c0, a2, b0); AQ_MF(c1, a2, b1); AQ_MF(c2, a2, b2); AQ_MF(c3, a2, b3); AQ_MF(c4, a3, b0); AQ_MF(c5, a3, b1); AQ_MF(c6, a3, b2); AQ_MF(c7, a3, b3);
+    } else if constexpr (V == 1) {
+      AQ_MF(c0, n0, n4); AQ_DR(a0, 0); AQ_MF(c1, n0, n5); AQ_MF(c2, n0, n6); AQ_DR(b0, 16384); AQ_MF(c3, n0, n7); AQ_MF(c4, n1, n4); AQ_DR(a1, 4096); AQ_MF(c5, n1, n5); AQ_MF(c6, n1, n6); AQ_DR(b1, 20480); AQ_MF(c7, n1, n7);
+      AQ_MF(c0, n2, n4); AQ_DR(a2, 8192); AQ_MF(c1, n2, n5); AQ_MF(c2, n2, n6); AQ_DR(b2, 24576); AQ_MF(c3, n2, n7); AQ_MF(c4, n3, n4); AQ_DR(a3, 12288); AQ_MF(c5, n3, n5); AQ_MF(c6, n3, n6); AQ_DR(b3, 28672); AQ_MF(c7, n3, n7);
+      AQ_LGKM0();
+      AQ_MF(c0, a0, b0); AQ_DR(n0, 0); AQ_MF(c1, a0, b1); AQ_MF(c2, a0, b2); AQ_DR(n4, 16384); AQ_MF(c3, a0, b3); AQ_MF(c4, a1, b0); AQ_DR(n1, 4096); AQ_MF(c5, a1, b1); AQ_MF(c6, a1, b2); AQ_DR(n5, 20480); AQ_MF(c7, a1, b3);
+      AQ_MF(c0, a2, b0); AQ_DR(n2, 8192); AQ_MF(c1, a2, b1); AQ_MF(c2, a2, b2); AQ_DR(n6, 24576); AQ_MF(c3, a2, b3); AQ_MF(c4, a3, b0); AQ_DR(n3, 12288); AQ_MF(c5, a3, b1); AQ_MF(c6, a3, b2); AQ_DR(n7, 28672); AQ_MF(c7, a3, b3);
+    } else if constexpr (V == 2) {
+      AQ_DR(a0, 0); AQ_DR(b0, 16384); AQ_DR(a1, 4096); AQ_DR(b1, 20480); AQ_DR(a2, 8192); AQ_DR(b2, 24576); AQ_DR(a3, 12288); AQ_DR(b3, 28672);
+      AQ_MF(c0, n0, n4); AQ_MF(c1, n0, n5); AQ_MF(c2, n0, n6); AQ_MF(c3, n0, n7); AQ_MF(c4, n1, n4); AQ_MF(c5, n1, n5); AQ_MF(c6, n1, n6); AQ_MF(c7, n1, n7);
+      AQ_MF(c0, n2, n4); AQ_MF(c1, n2, n5); AQ_MF(c2, n2, n6); AQ_MF(c3, n2, n7); AQ_MF(c4, n3, n4); AQ_MF(c5, n3, n5); AQ_MF(c6, n3, n6); AQ_MF(c7, n3, n7);
+      AQ_LGKM0();
+      AQ_DR(n0, 0); AQ_DR(n4, 16384); AQ_DR(n1, 4096); AQ_DR(n5, 20480); AQ_DR(n2, 8192); AQ_DR(n6, 24576); AQ_DR(n3, 12288); AQ_DR(n7, 28672);
+      AQ_MF(c0, a0, b0); AQ_MF(c1, a0, b1); AQ_MF(c2, a0, b2); AQ_MF(c3, a0, b3); AQ_MF(c4, a1, b0); AQ_MF(c5, a1, b1); AQ_MF(c6, a1, b2); AQ_MF(c7, a1, b3);
+      AQ_MF(c0, a2, b0); AQ_MF(c1, a2, b1); AQ_MF(c2, a2, b2); AQ_MF(c3, a2, b3); AQ_MF(c4, a3, b0); AQ_MF(c5, a3, b1); AQ_MF(c6, a3, b2); AQ_MF(c7, a3, b3);
+    } else {
+      AQ_MF(c0, n0, n4); AQ_DR(a0, 0); AQ_DR(b0, 16384); AQ_MF(c1, n0, n5); AQ_MF(c2, n0, n6); AQ_MF(c3, n0, n7); AQ_MF(c4, n1, n4); AQ_DR(a1, 4096); AQ_DR(b1, 20480); AQ_MF(c5, n1, n5); AQ_MF(c6, n1, n6); AQ_MF(c7, n1, n7);
+      AQ_MF(c0, n2, n4); AQ_DR(a2, 8192); AQ_DR(b2, 24576); AQ_MF(c1, n2, n5); AQ_MF(c2, n2, n6); AQ_MF(c3, n2, n7); AQ_MF(c4, n3, n4); AQ_DR(a3, 12288); AQ_DR(b3, 28672); AQ_MF(c5, n3, n5); AQ_MF(c6, n3, n6); AQ_MF(c7, n3, n7);
+      AQ_LGKM0();
+      AQ_MF(c0, a0, b0); AQ_DR(n0, 0); AQ_DR(n4, 16384); AQ_MF(c1, a0, b1); AQ_MF(c2, a0, b2); AQ_MF(c3, a0, b3); AQ_MF(c4, a1, b0); AQ_DR(n1, 4096); AQ_DR(n5, 20480); AQ_MF(c5, a1, b1); AQ_MF(c6, a1, b2); AQ_MF(c7, a1, b3);
+      AQ_MF(c0, a2, b0); AQ_DR(n2, 8192); AQ_DR(n6, 24576); AQ_MF(c1, a2, b1); AQ_MF(c2, a2, b2); AQ_MF(c3, a2, b3); AQ_MF(c4, a3, b0); AQ_DR(n3, 12288); AQ_DR(n7, 28672); AQ_MF(c5, a3, b1); AQ_MF(c6, a3, b2); AQ_MF(c7, a3, b3);
+    }
+    AQ_LGKM0();
+  }
+  const long long t1 = clock64();
+  if (clocks && threadIdx.x == 0 && blockIdx.x == 0) clocks[0] = t1 - t0;
+  int s = n0[0] ^ n1[1] ^ n2[2] ^ n3[3] ^ n4[0] ^ n5[0] ^ n6[0] ^ n7[0] ^ a0[0] ^ a1[0] ^ a2[0] ^ a3[0] ^ b0[0] ^ b1[0] ^ b2[0] ^ b3[0];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) s ^= c0[i] ^ c1[i] ^ c2[i] ^ c3[i] ^ c4[i] ^ c5[i] ^ c6[i] ^ c7[i];
+  if (s == 0x12345678) sink[0] = s;
+}
+#undef AQ_MF
+#undef AQ_DR
+#undef AQ_LGKM0
+
 }  // namespace aq
 
 extern "C" int aq_lab_probe_mfma(int kind, int data, int workgroups, int iters, int* sink, long long* clocks, void* stream) {
@@ -209,5 +273,16 @@ extern "C" int aq_lab_probe_read(const void* src, int64_t bytes, int loads_per_l
 extern "C" int aq_lab_probe_empty(int* sink, void* stream) {
   if (!sink) return AQ_E_NULL;
   hipLaunchKernelGGL(aq::probe_empty_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream), sink);
+  return (int)hipGetLastError();
+}
+
+extern "C" int aq_lab_probe_mfma_lds_issue(int variant, int workgroups, int iters, int* sink, long long* clocks,
+                                           void* stream) {
+  if (variant < 0 || variant > 3 || workgroups <= 0 || iters <= 0 || !sink) return AQ_E_SHAPE;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  using kern_t = void (*)(int, int*, long long*);
+  static const kern_t table[4] = {aq::probe_issue_kernel<0>, aq::probe_issue_kernel<1>, aq::probe_issue_kernel<2>,
+                                  aq::probe_issue_kernel<3>};
+  hipLaunchKernelGGL(table[variant], dim3((unsigned)workgroups), dim3(256), 32768, st, iters, sink, clocks);
   return (int)hipGetLastError();
 }

@@ -41,21 +41,31 @@ __device__ __forceinline__ float vec_amax(const float* f) {
 }
 
 // Symmetric absmax scale of one row from its wavefront-wide maximum:
-// s = amax / 127 (1 for an all-zero row), rs = the once-refined reciprocal of s
-// that quant_codes expects, and whether s is in the range where it may be used.
+// s = amax / 127 (1 for an all-zero row), rs = the reciprocal of s in the form
+// quant_codes<N, STEPS> expects (STEPS = 2: the once-refined hardware reciprocal;
+// STEPS = 1, rows of bf16 numbers: the correctly rounded one, a full divide once
+// per row), and whether s is in the range where the short sequence may be used.
 struct RowScale {
   float s, rs;
   bool fast_ok;
 };
+template <int STEPS = 2>
 __device__ __forceinline__ RowScale row_scale(float amax) {
   RowScale r;
   r.s = __fdiv_rn(amax, 127.0f);
   if (amax == 0.0f) r.s = 1.0f;
-  const float y0 = __builtin_amdgcn_rcpf(r.s);
-  r.rs = __builtin_fmaf(__builtin_fmaf(-r.s, y0, 1.0f), y0, y0);
+  if constexpr (STEPS == 1) {
+    r.rs = __fdiv_rn(1.0f, r.s);
+  } else {
+    const float y0 = __builtin_amdgcn_rcpf(r.s);
+    r.rs = __builtin_fmaf(__builtin_fmaf(-r.s, y0, 1.0f), y0, y0);
+  }
   r.fast_ok = r.s >= 5.421010862427522e-20f && r.s <= 1.8446744073709552e19f;  // [2^-64, 2^64]
   return r;
 }
+// correction steps for rows that are read as they are (bf16 numbers: one) or computed in fp32 (two)
+template <bool BF16, bool COMPUTED>
+constexpr int quant_steps() { return BF16 && !COMPUTED ? 1 : 2; }
 
 // Sum across the wavefront in a fixed order: p[l] += p[l ^ 1], ^2, ^4, ^8, ^16, ^32, every add
 // rounded.  After the xor-1 and xor-2 steps a quad holds one value, after the half-row mirror a
@@ -159,7 +169,8 @@ struct RowsToLds {
         values<NORM>(j, i, r, f);
         amax = fmaxf(amax, vec_amax<EPV>(f));
       }
-      const RowScale rsc = row_scale(wave_max(amax));
+      constexpr int STEPS = quant_steps<BF16, NORM>();
+      const RowScale rsc = row_scale<STEPS>(wave_max(amax));
       if (lane == 0 && m < M) sx[m] = rsc.s;
 #pragma unroll
       for (int i = 0; i < VPL; ++i) {
@@ -168,7 +179,7 @@ struct RowsToLds {
           float f[EPV];
           uint32_t code[EPV];
           values<NORM>(j, i, r, f);
-          quant_codes<EPV>(f, rsc.s, rsc.rs, rsc.fast_ok, code);  // zero rows give zero codes
+          quant_codes<EPV, STEPS>(f, rsc.s, rsc.rs, rsc.fast_ok, code);  // zero rows give zero codes
           uint8_t* dst = xs + m * pitch + v * EPV;
           if constexpr (BF16) {
             uint2 o;

@@ -173,7 +173,9 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_w8a8_kernel(GemvArgs p) {
 
   // 0. After the reduction lane l owns output (row n0 + idx / MT, token idx % MT)
   // with idx = l >> (6 - log2(rows * MT)).  Its scales and bias are requested
-  // now, ahead of everything else, so the epilogue never waits on memory.
+  // ahead of the weight stream, so the epilogue never waits on memory, but behind
+  // the activation rows (step 1): loads return in request order, and these lines,
+  // which no other workgroup shares, come from HBM while the rows come from cache.
   constexpr int V = GV_ROWS * MT;
   constexpr int SH = 6 - ilog2(V);
   static_assert(V <= 64, "one output per lane at most");
@@ -182,10 +184,17 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_w8a8_kernel(GemvArgs p) {
   const bool out_lane = (lane & ((1 << SH) - 1)) == 0 && om < M && on < N;
   float* sx_lds = reinterpret_cast<float*>(xs + MT * K);
   const EpiOperands epi(p, true, !FUSED, true);
-  float sxv = epi.load_sx(om, out_lane);
-  const float swv = epi.load_sw(on, out_lane);
-  const float bv = epi.load_bias(on, out_lane);
-  const uint32_t rv = epi.load_res(om, on, out_lane, (int)p.ldr);  // residual element, raw bits
+  float sxv = 0.0f, swv, bv;
+  uint32_t rv;  // residual element, raw bits
+  auto load_epi = [&]() {
+    sxv = epi.load_sx(om, out_lane);
+    swv = epi.load_sw(on, out_lane);
+    bv = epi.load_bias(on, out_lane);
+    rv = epi.load_res(om, on, out_lane, (int)p.ldr);
+  };
+  // (the copy of ready-made codes goes straight to LDS and is waited for by counting the requests behind it:
+  // there the operands stay in front)
+  if constexpr (!FUSED) load_epi();
 
   // 1. activation codes -> LDS.  Either copied, 16 bytes per lane, straight from
   // global memory (rows m >= M lie outside the descriptor and arrive as zeros),
@@ -211,6 +220,10 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_w8a8_kernel(GemvArgs p) {
             (base + lane * 16) < xbytes ? (uint32_t)(base + lane * 16) : OOB_OFFSET, 0, 0, 0);
     }
   }
+
+  asm volatile("" ::: "memory");  // request order: activation rows, epilogue operands, the weight stream
+  if constexpr (FUSED) load_epi();
+  asm volatile("" ::: "memory");
 
   // 2. the first GV_DEPTH weight chunks of this wavefront's rows.  The
   // descriptor spans these rows only; rows past N and bytes past K fall
@@ -439,18 +452,24 @@ __global__ __launch_bounds__(GM_MAX_WAVES * 64) void gemv_mfma_kernel(GemvArgs p
   const int rbase = n0 + (lane >> 4) * 4;
   float swv[4], bv[4];
   uint32_t rv[4];  // residual elements, raw bits
-  // only the first K part's wavefront writes outputs: the others get empty descriptors.  Requested first:
-  // measured 0.2 us faster than behind the weight stream (loads return in request order, and these few come
-  // back quickly, while behind the weights the epilogue would wait for the whole stream to drain).
+  // only the first K part's wavefront writes outputs: the others get empty descriptors.  Requested (load_epi)
+  // between the token rows and the weight stream.  Loads return in request order: behind the weights the
+  // epilogue would wait for the whole stream to drain (0.2 us), and in front of the tokens these few lines, which
+  // no other workgroup shares and which therefore come from HBM, hold back the token rows that every workgroup
+  // reads and the caches serve (M = 16, N = 8192: 7.45 -> 7.2 us with the rows quantised here, 5.85 -> 5.65 us on
+  // codes).
   const EpiOperands epi(p, kh == 0, FQ == 0, RES);
-  float sxv = epi.load_sx(FP8 ? 0 : tok, FP8 || tok < M);
+  float sxv = 0.0f;
+  auto load_epi = [&]() {
+    sxv = epi.load_sx(FP8 ? 0 : tok, FP8 || tok < M);
 #pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    const int n = rbase + r;
-    swv[r] = epi.load_sw(FP8 ? 0 : n, FP8 || n < N);
-    bv[r] = epi.load_bias(n, n < N);
-    rv[r] = RES ? epi.load_res(tok, n, tok < M && n < N, (int)p.ldr) : 0u;
-  }
+    for (int r = 0; r < 4; ++r) {
+      const int n = rbase + r;
+      swv[r] = epi.load_sw(FP8 ? 0 : n, FP8 || n < N);
+      bv[r] = epi.load_bias(n, n < N);
+      rv[r] = RES ? epi.load_res(tok, n, tok < M && n < N, (int)p.ldr) : 0u;
+    }
+  };
 
   // weight stream: descriptor over this wavefront's 16 rows; rows past N read as zero
   const int rows = n0 < N ? ((N - n0) < GM_ROWS ? (N - n0) : GM_ROWS) : 0;
@@ -487,7 +506,9 @@ __global__ __launch_bounds__(GM_MAX_WAVES * 64) void gemv_mfma_kernel(GemvArgs p
     RowsToLds<true, RPW, 4> xrows;
     xrows.issue(p.x, M, K, K, wave, WAVES, lane);
     if constexpr (NORM) xrows.issue_gamma(p.gamma, K, lane);
-    asm volatile("" ::: "memory");  // request order: token rows, then the weight stream
+    asm volatile("" ::: "memory");  // request order: token rows, epilogue operands, the weight stream
+    load_epi();
+    asm volatile("" ::: "memory");
     wload(0, wa);
     wload(GM_LINES, wb);
     asm volatile("" ::: "memory");
@@ -516,8 +537,7 @@ __global__ __launch_bounds__(GM_MAX_WAVES * 64) void gemv_mfma_kernel(GemvArgs p
       float sc = __fdiv_rn(all, 448.0f);
       if (all == 0.0f) sc = 1.0f;
       sxv = sc;
-      const float y0 = __builtin_amdgcn_rcpf(sc);
-      const float rsc = __builtin_fmaf(__builtin_fmaf(-sc, y0, 1.0f), y0, y0);
+      const float rsc = __fdiv_rn(1.0f, sc);  // correctly rounded: what the one-step sequence below needs
       const bool lean_ok = sc >= 5.421010862427522e-20f && sc <= 1.8446744073709552e19f;  // [2^-64, 2^64]
       const int nvec = K / 8;
 #pragma unroll
@@ -532,12 +552,12 @@ __global__ __launch_bounds__(GM_MAX_WAVES * 64) void gemv_mfma_kernel(GemvArgs p
             RowIn<true>::unpack(xrows.c[j][i], f);
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-              // x / s: the refined-reciprocal sequence that equals the correctly rounded divide for in-range
-              // scales (see quant_codes), the divide itself otherwise; then the clamp to the e4m3 range
+              // x / s: the one-correction sequence that gives a bf16 number's e4m3 code exactly for in-range
+              // scales (see quant_codes; a -0.0 comes out as +0.0, which no product can tell apart), the
+              // divide itself otherwise; then the clamp to the e4m3 range
               float q;
               if (__builtin_expect(lean_ok, 1)) {
                 q = f[e] * rsc;
-                q = __builtin_fmaf(__builtin_fmaf(-sc, q, f[e]), rsc, q);
                 q = __builtin_fmaf(__builtin_fmaf(-sc, q, f[e]), rsc, q);
               } else {
                 q = __fdiv_rn(f[e], sc);
@@ -581,7 +601,9 @@ __global__ __launch_bounds__(GM_MAX_WAVES * 64) void gemv_mfma_kernel(GemvArgs p
     };
 #pragma unroll
     for (int r = 0; r < XR; ++r) xload(r * XV * nthreads, xvr[r]);
-    asm volatile("" ::: "memory");  // request order: token codes, then the weight stream
+    asm volatile("" ::: "memory");  // request order: token codes, epilogue operands, the weight stream
+    load_epi();
+    asm volatile("" ::: "memory");
     wload(0, wa);
     wload(GM_LINES, wb);
     asm volatile("" ::: "memory");

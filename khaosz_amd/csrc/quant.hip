@@ -15,7 +15,7 @@ __device__ __forceinline__ void quant_store(const uint4& v, float s, float rs, b
   float f[EPV];
   uint32_t c[EPV];
   RowIn<BF16>::unpack(v, f);
-  quant_codes<EPV>(f, s, rs, fast_ok, c);
+  quant_codes<EPV, quant_steps<BF16, false>()>(f, s, rs, fast_ok, c);
   if constexpr (BF16) {
     uint2 o;
     o.x = pack_low_bytes(c[0], c[1], c[2], c[3]);
@@ -76,7 +76,7 @@ __global__ __launch_bounds__(256) void quant_rowwise_i8_kernel(const void* __res
       }
     }
     amax = wave_max(amax);
-    const RowScale rsc = row_scale(amax);
+    const RowScale rsc = row_scale<quant_steps<BF16, false>()>(amax);
     const float s = rsc.s, rs = rsc.rs;
     const bool fast_ok = rsc.fast_ok;
     if (lane == 0) scale[r] = s;
@@ -147,7 +147,7 @@ __global__ __launch_bounds__(256) void quant_row_wg_kernel(const void* __restric
   if ((tid & 63) == 0) wmax[tid >> 6] = amax;
   __syncthreads();
   amax = fmaxf(fmaxf(wmax[0], wmax[1]), fmaxf(wmax[2], wmax[3]));
-  const RowScale rsc = row_scale(amax);
+  const RowScale rsc = row_scale<quant_steps<BF16, false>()>(amax);
   const float s = rsc.s, rs = rsc.rs;
   const bool fast_ok = rsc.fast_ok;
   if (tid == 0) scale[row] = s;
@@ -397,8 +397,31 @@ __global__ __launch_bounds__(AMAX_THREADS) void amax_kernel(const void* __restri
   }
 }
 
-__device__ __forceinline__ float fp8_prescale(float a, float s) {
-  float v = __fdiv_rn(a, s);
+// x / s clamped to the e4m3 range.  For scales in [2^-64, 2^64] the short sequences of quant_codes
+// (aq_common.h) stand in for the correctly rounded divide, whose vector operations had made this kernel
+// ALU-bound: with STEPS = 2, rs = the once-refined hardware reciprocal and the result is fl(x / s); with
+// STEPS = 1 (x a bf16 number), rs = fl(1 / s) and one correction gives fl(x / s) whenever the quotient is
+// above 2^-11 in magnitude, and something that still rounds to the code 0 below (every pair of bf16
+// maximum and value evaluated on the CPU, as for the int8 rows).  Other scales take the full divide.
+template <int STEPS>
+__device__ __forceinline__ float fp8_reciprocal(float s) {
+  if constexpr (STEPS == 1) return __fdiv_rn(1.0f, s);
+  const float y0 = __builtin_amdgcn_rcpf(s);
+  return __builtin_fmaf(__builtin_fmaf(-s, y0, 1.0f), y0, y0);
+}
+template <int STEPS>
+__device__ __forceinline__ float fp8_prescale(float a, float s, float rs, bool lean_ok) {
+  float v;
+  if (__builtin_expect(lean_ok, 1)) {
+    v = a * rs;
+    v = __builtin_fmaf(__builtin_fmaf(-s, v, a), rs, v);
+    if constexpr (STEPS == 2) v = __builtin_fmaf(__builtin_fmaf(-s, v, a), rs, v);
+    // a zero residual added to a quotient of -0 gives +0: the quotient takes the sign of a (s > 0), as the
+    // divide's does, so that -0.0 still becomes the code 0x80
+    v = __uint_as_float((__float_as_uint(v) & 0x7fffffffu) | (__float_as_uint(a) & 0x80000000u));
+  } else {
+    v = __fdiv_rn(a, s);
+  }
   return fminf(fmaxf(v, -448.0f), 448.0f);
 }
 
@@ -422,6 +445,9 @@ __global__ __launch_bounds__(256) void cast_fp8_kernel(const void* __restrict__ 
   float s = __fdiv_rn(amax, 448.0f);
   if (amax == 0.0f) s = 1.0f;
   if (blockIdx.x == 0 && threadIdx.x == 0) *scale = s;
+  constexpr int STEPS = BF16 ? 1 : 2;
+  const float rs = fp8_reciprocal<STEPS>(s);
+  const bool lean_ok = s >= 5.421010862427522e-20f && s <= 1.8446744073709552e19f;  // [2^-64, 2^64]
   const uint4* src = reinterpret_cast<const uint4*>(x);
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   for (int64_t v0 = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; v0 < nvec; v0 += FP8_BATCH * stride) {
@@ -438,7 +464,7 @@ __global__ __launch_bounds__(256) void cast_fp8_kernel(const void* __restrict__ 
       float f[EPV];
       RowIn<BF16>::unpack(t[u], f);
 #pragma unroll
-      for (int i = 0; i < EPV; ++i) f[i] = fp8_prescale(f[i], s);
+      for (int i = 0; i < EPV; ++i) f[i] = fp8_prescale<STEPS>(f[i], s, rs, lean_ok);
       // v_cvt_pk_fp8_f32: two fp32 -> two OCP e4m3fn codes, round to nearest even.
       int w0 = __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], 0, false);
       w0 = __builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], w0, true);

@@ -40,6 +40,9 @@
  *   oq_linear_fp8         restatement; accumulation order makes the GEMM a
  *                         tolerance (1e-2) comparison, never bit-exact.
  *
+ *   oq_one_step_divide_mismatches   not a restatement: an exhaustive evaluation of a shortcut
+ *                         the HIP quantisers take on bf16 rows, against the divide itself.
+ *
  *   oq_rmsnorm_quant_i8   the norm itself restates F.rms_norm (norm.py:14-15) with a
  *                         fixed summation order; pinned against float64 and torch's
  *                         F.rms_norm within rounding, against the numpy restatement
@@ -584,6 +587,58 @@ void oq_quant_tensor_fp8_bf16(const uint16_t *x, int64_t numel, uint8_t *q, floa
   for (int64_t i = 0; i < numel; ++i) tmp[i] = oq_bf16_to_f32(x[i]);
   oq_quant_tensor_fp8_f32(tmp, numel, q, scale);
   free(tmp);
+}
+
+/*
+ * Checker for a shortcut the HIP quantisers take on rows of bf16 numbers (not a restatement of anything in the
+ * reference).  The definition above divides, q = fl(a / s); the kernels compute, with rs = fl(1 / s),
+ *     q0 = fl(a * rs);  r = fma(-s, q0, a);  q1 = fma(r, rs, q0)
+ * (one correction step; in general two are needed) and claim the CODE of q1 equals the code of q whenever a and
+ * the maximum the scale comes from are bf16 numbers.  This function evaluates the claim for every bf16 maximum
+ * with bit pattern in [am_lo, am_hi) whose scale s = fl(amax / divisor) lies in [2^-64, 2^64] (the range in which
+ * the kernels use the shortcut) and every bf16 a with |a| <= amax, both signs, and returns the number of pairs
+ * whose codes differ (*pairs = the number evaluated).  divisor 127: code = clamp(rint(.), +-127); divisor 448:
+ * code = e4m3fn(clamp(., +-448)) with the quotient given the sign of a (the kernel does that too: a zero residual
+ * turns a quotient of -0 into +0).  steps = 0 evaluates q0 alone, which does differ: the check has teeth.
+ */
+int64_t oq_one_step_divide_mismatches(float divisor, int steps, uint32_t am_lo, uint32_t am_hi, int64_t *pairs) {
+  int64_t bad = 0, n = 0;
+  const int fp8 = divisor == 448.0f;
+#pragma omp parallel for schedule(dynamic, 16) reduction(+ : bad, n)
+  for (uint32_t am = am_lo; am < am_hi; ++am) {
+    if (am == 0 || am >= 0x7f80u) continue;
+    const float amax = oq_bf16_to_f32((uint16_t)am);
+    const float s = amax / divisor;
+    if (!(s >= 5.421010862427522e-20f && s <= 1.8446744073709552e19f)) continue;
+    const float rs = 1.0f / s;
+    for (uint32_t ab = 0; ab <= am; ++ab) {
+      for (int neg = 0; neg < 2; ++neg) {
+        const float a = oq_bf16_to_f32((uint16_t)(ab | (neg ? 0x8000u : 0u)));
+        const float q = a / s;
+        const float q0 = a * rs;
+        float q1 = steps ? fmaf(fmaf(-s, q0, a), rs, q0) : q0;
+        ++n;
+        if (fp8) {
+          q1 = copysignf(q1, a);
+          float c0 = q, c1 = q1;
+          if (c0 > 448.0f) c0 = 448.0f;
+          if (c0 < -448.0f) c0 = -448.0f;
+          if (c1 > 448.0f) c1 = 448.0f;
+          if (c1 < -448.0f) c1 = -448.0f;
+          bad += oq_f32_to_e4m3fn(c0) != oq_f32_to_e4m3fn(c1);
+        } else {
+          float c0 = rintf(q), c1 = rintf(q1);
+          if (c0 > 127.0f) c0 = 127.0f;
+          if (c0 < -127.0f) c0 = -127.0f;
+          if (c1 > 127.0f) c1 = 127.0f;
+          if (c1 < -127.0f) c1 = -127.0f;
+          bad += (int)c0 != (int)c1;
+        }
+      }
+    }
+  }
+  if (pairs) *pairs = n;
+  return bad;
 }
 
 /* y = (sum_k f(xq[m,k]) f(wq[n,k])) * sx * sw; fp32 accumulate, k ascending. */

@@ -240,6 +240,8 @@ def _load():
     lib.oq_linear_w8a8_bf16.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i64]
     lib.oq_quant_tensor_fp8_f32.argtypes = [vp, i64, vp, vp]
     lib.oq_quant_tensor_fp8_bf16.argtypes = [vp, i64, vp, vp]
+    lib.oq_one_step_divide_mismatches.argtypes = [ctypes.c_float, ctypes.c_int, ctypes.c_uint32, ctypes.c_uint32, vp]
+    lib.oq_one_step_divide_mismatches.restype = ctypes.c_int64
     lib.oq_linear_fp8.argtypes = [vp, ctypes.c_float, vp, ctypes.c_float, vp, vp, vp, i64, i64, i64]
     lib.oq_linear_f32.argtypes = [vp, vp, vp, vp, i64, i64, i64]
     for name in (
@@ -423,6 +425,14 @@ def c_quant_tensor_fp8(x: np.ndarray, bf16_bits: bool = False):
     fn = lib.oq_quant_tensor_fp8_bf16 if bf16_bits else lib.oq_quant_tensor_fp8_f32
     fn(_p(x), x.size, _p(q), _p(s))
     return q, F32(s[0])
+
+
+def c_one_step_divide_mismatches(divisor: float, am_lo: int = 0, am_hi: int = 0x7F80, steps: int = 1):
+    """(pairs whose code differs, pairs evaluated) for the one-correction divide on bf16 numbers: see the C source."""
+    lib = _load()
+    n = np.zeros((1,), np.int64)
+    bad = lib.oq_one_step_divide_mismatches(float(divisor), int(steps), int(am_lo), int(am_hi), _p(n))
+    return int(bad), int(n[0])
 
 
 def c_linear_fp8(xq, sx, wq, sw, bf16_out: bool = False, bias=None) -> np.ndarray:

@@ -485,6 +485,43 @@ def test_quant_tensor_fp8_codes_bit_exact(oracle):
     assert s0.item() == 1.0 and not to_np(q0).any()
 
 
+@pytest.mark.parametrize("scale", [1.0, 0.37, 3.3e-3, 7.7e5, 1e-21, 1e-30, 3e25, 1e36])
+def test_quant_tensor_fp8_scale_range_and_dense_midpoints(oracle, scale):
+    """The cast kernel divides by the scale with a refined-reciprocal sequence that must equal the correctly
+    rounded divide: inputs placed on and next to every e4m3 rounding midpoint (times the scale, one ulp either
+    side), scales across the fp32 range (those outside [2^-64, 2^64] take the full divide), small and subnormal
+    inputs.  Codes bit for bit against the oracle, fp32 and bf16 inputs; the GEMV's own cast gives the same codes."""
+    tab = oracle.np_e4m3fn_table()[:127].astype(np.float64)
+    mids = (tab[:-1] + tab[1:]) / 2
+    pts = np.concatenate([tab, mids, -tab, -mids])
+    s32 = np.float32(scale / 448.0) * np.float32(448.0)  # amax; the kernel's scale is amax / 448
+    base = (pts * float(s32) / 448.0).astype(np.float32)
+    near = np.concatenate([base, np.nextafter(base, np.float32(np.inf)), np.nextafter(base, np.float32(-np.inf))])
+    rng = np.random.default_rng(61)
+    rest = 4096 - near.size - 8
+    tiny = np.array([1e-45, -1e-45, 1e-39, -3e-39, 0.0, -0.0, 1e-38, -1e-38], np.float32)
+    x = np.concatenate([near, (rng.uniform(-1, 1, rest) * float(s32)).astype(np.float32), tiny]).astype(np.float32)
+    x[0] = s32  # pins amax
+    x = np.clip(x, -s32, s32)
+    xd = torch.from_numpy(x).to(DEV)
+    q, s = ops.quant_tensor_fp8(xd)
+    qo, so = oracle.c_quant_tensor_fp8(x)
+    assert np.float32(s.item()) == so
+    assert np.array_equal(to_np(q), qo), int((to_np(q) != qo).sum())
+    xb = xd.to(torch.bfloat16)
+    qb, sb = ops.quant_tensor_fp8(xb)
+    qbo, sbo = oracle.c_quant_tensor_fp8(bf16_bits(xb), bf16_bits=True)
+    assert np.float32(sb.item()) == sbo and np.array_equal(to_np(qb), qbo)
+    # the same rows through the GEMV that casts them itself: against the GEMV on the quantiser's codes
+    if 1e-15 < scale < 1e15:
+        rows = xb.view(2, 2048)
+        w8, t8 = ops.quant_tensor_fp8(torch.randn(96, 2048, device=DEV) * 0.02)
+        fused = ops.gemv_fp8_decode(rows, w8, t8, out_dtype=torch.float32)
+        codes = ops.gemv_fp8_codes(qb.view(2, 2048), sb, w8, t8, out_dtype=torch.float32)
+        ref = float(codes.abs().mean())
+        assert float((fused - codes).abs().max()) <= 2e-5 * max(ref, 1e-30)
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 1, 16), (33, 70, 144), (256, 128, 1024), (300, 260, 2048), (64, 96, 8192)])
 def test_linear_fp8_within_tolerance(oracle, tile, M, N, K):
     _say("linear_fp8", M, N, K)

@@ -193,3 +193,16 @@ def test_config1_linear_w8a8_vs_reference_float_linear(oracle):
     assert rel0 < 0.4 * rel and rel0 < 1.5e-2, (rel0, rel)
     # the oracle's own fp32 Linear agrees with torch's
     assert np.allclose(oracle.c_linear_f32(x.numpy(), w.numpy()), ref, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("divisor", [127.0, 448.0])
+def test_one_correction_divide_gives_the_code_of_the_divide_for_every_pair_of_bf16_numbers(oracle, divisor):
+    """The HIP quantisers round rows of bf16 numbers with one correction step on a correctly rounded
+    reciprocal instead of the divide of the definition.  Every pair (row maximum, value) of bf16 numbers the
+    shortcut can meet, 5.6e8 of them per code format, evaluated one by one with the same IEEE operations:
+    no pair's code differs.  The product with the reciprocal alone (no correction) does differ, so the
+    evaluation can tell."""
+    bad, pairs = oracle.c_one_step_divide_mismatches(divisor)
+    assert pairs > 5.5e8 and bad == 0
+    bad0, _ = oracle.c_one_step_divide_mismatches(divisor, am_lo=0x3F80, am_hi=0x4000, steps=0)
+    assert bad0 > 0

@@ -67,6 +67,19 @@ int aq_quant_rowwise_i8(const void *x, int x_dtype, int64_t M, int64_t K, int64_
 int aq_quant_tensor_fp8(const void *x, int x_dtype, int64_t numel, uint8_t *q, float *scale,
                         uint32_t *amax_ws, void *stream);
 
+/* The same result in ONE launch, for callers that can keep a small piece of device state: every workgroup holds
+ * its share of x in registers between the maximum and the cast (tensors up to 32 MiB on 256 compute units are read
+ * from HBM once instead of twice; what does not fit is read again), and the workgroups exchange their partial
+ * maxima through ws while the kernel runs.  ws: AQ_FP8_ONEPASS_WS_BYTES of device memory, 8-byte aligned, that
+ * must be ZERO-FILLED before its first use and is then left, after every call, in a state the next call accepts
+ * (so: fill once, reuse for every later call on that device); calls that overlap in time must not share one.
+ * The wait for the other workgroups is bounded: if they cannot all run at once (a busy or partitioned device) each
+ * takes the tensor's maximum itself after about a millisecond -- same codes and scale, much slower.
+ * Same definition and reference call site as aq_quant_tensor_fp8 (linear.py:21, FP8 variant). */
+#define AQ_FP8_ONEPASS_WS_BYTES 2048
+int aq_quant_tensor_fp8_onepass(const void *x, int x_dtype, int64_t numel, uint8_t *q, float *scale,
+                                void *ws, size_t ws_bytes, void *stream);
+
 /* acc[m, n] = sum_k xq[m, k] * wq[n, k], exact int32: the matrix product inside
  * F.linear (linear.py:21) on int8 codes.  xq: [M, K], wq: [N, K], acc: [M, N]. */
 int aq_gemm_i8_i32(const int8_t *xq, const int8_t *wq, int32_t *acc, int64_t M, int64_t N,

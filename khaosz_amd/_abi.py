@@ -11,6 +11,7 @@ LIB_PATH = os.environ.get("ASTRAI_Q_LIB") or os.path.join(_HERE, "lib", "libastr
 
 AQ_F32, AQ_BF16 = 0, 1
 AQ_FP8_AMAX_WS_BYTES = 1024  # include/astrai_q.h
+AQ_FP8_ONEPASS_WS_BYTES = 2048  # include/astrai_q.h
 
 # every symbol include/astrai_q.h declares: name -> (restype, argtypes)
 _i64, _vp, _int, _sz = ctypes.c_int64, ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
@@ -21,6 +22,7 @@ SYMBOLS = {
     "aq_rmsnorm_quant_rowwise_i8": (_int, [_vp, _int, _vp, _int, ctypes.c_float, _i64, _i64, _i64, _vp, _vp, _vp]),
     "aq_swiglu_quant_rowwise_i8": (_int, [_vp, _int, _i64, _i64, _i64, _vp, _vp, _vp]),
     "aq_quant_tensor_fp8": (_int, [_vp, _int, _i64, _vp, _vp, _vp, _vp]),
+    "aq_quant_tensor_fp8_onepass": (_int, [_vp, _int, _i64, _vp, _vp, _vp, _sz, _vp]),
     "aq_gemm_i8_i32": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "aq_linear_w8a8": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _vp, _int, _i64, _i64, _i64, _vp]),
     "aq_linear_w8a8_residual": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _vp, _vp, _int, _i64, _i64, _i64, _vp]),
@@ -68,6 +70,7 @@ LAB_SYMBOLS = {
     "aq_lab_probe_read": (_int, [_vp, _i64, _int, _int, _int, _vp, _vp]),
     "aq_lab_probe_empty": (_int, [_vp, _vp]),
     "aq_lab_probe_mfma_lds_issue": (_int, [_int, _int, _int, _vp, _vp, _vp]),
+    "aq_lab_quant_tensor_fp8_onepass_spin": (_int, [_vp, _int, _i64, _vp, _vp, _vp, _sz, _int, _vp]),
 }
 
 _lib = None

@@ -47,6 +47,12 @@ int aq_lab_probe_mfma_lds_issue(int variant, int workgroups, int iters, int *sin
 /* One wavefront that does nothing: the cost of a launch. */
 int aq_lab_probe_empty(int *sink, void *stream);
 
+/* aq_quant_tensor_fp8_onepass with the bound on its wait for the other workgroups (polls of their slots) given
+ * by the caller.  spin_limit 0: every workgroup gives up at once and takes the maximum of the whole tensor
+ * itself -- the path of a device too busy to run all workgroups together -- so a test can run it without one. */
+int aq_lab_quant_tensor_fp8_onepass_spin(const void *x, int x_dtype, int64_t numel, uint8_t *q, float *scale,
+                                         void *ws, size_t ws_bytes, int spin_limit, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -286,3 +286,16 @@ extern "C" int aq_lab_probe_mfma_lds_issue(int variant, int workgroups, int iter
   hipLaunchKernelGGL(table[variant], dim3((unsigned)workgroups), dim3(256), 32768, st, iters, sink, clocks);
   return (int)hipGetLastError();
 }
+
+// The one-launch FP8 quantiser with the bound on its wait for the other workgroups given by the caller: 0 makes
+// every workgroup give up at once and take the tensor's maximum itself, the path a busy device would take.
+namespace aq {
+int quant_tensor_fp8_onepass(const void* x, int x_dtype, int64_t numel, uint8_t* q, float* scale, void* ws,
+                             size_t ws_bytes, int spin_limit, hipStream_t st);
+}
+extern "C" int aq_lab_quant_tensor_fp8_onepass_spin(const void* x, int x_dtype, int64_t numel, uint8_t* q, float* scale,
+                                                    void* ws, size_t ws_bytes, int spin_limit, void* stream) {
+  if (spin_limit < 0) return AQ_E_RANGE;
+  return aq::quant_tensor_fp8_onepass(x, x_dtype, numel, q, scale, ws, ws_bytes, spin_limit,
+                                      static_cast<hipStream_t>(stream));
+}

@@ -409,20 +409,24 @@ __device__ __forceinline__ float fp8_reciprocal(float s) {
   const float y0 = __builtin_amdgcn_rcpf(s);
   return __builtin_fmaf(__builtin_fmaf(-s, y0, 1.0f), y0, y0);
 }
-template <int STEPS>
-__device__ __forceinline__ float fp8_prescale(float a, float s, float rs, bool lean_ok) {
-  float v;
-  if (__builtin_expect(lean_ok, 1)) {
-    v = a * rs;
-    v = __builtin_fmaf(__builtin_fmaf(-s, v, a), rs, v);
-    if constexpr (STEPS == 2) v = __builtin_fmaf(__builtin_fmaf(-s, v, a), rs, v);
-    // a zero residual added to a quotient of -0 gives +0: the quotient takes the sign of a (s > 0), as the
-    // divide's does, so that -0.0 still becomes the code 0x80
-    v = __uint_as_float((__float_as_uint(v) & 0x7fffffffu) | (__float_as_uint(a) & 0x80000000u));
+template <int STEPS, int N>
+__device__ __forceinline__ void fp8_prescale(float* f, float s, float rs, bool lean_ok) {
+  if (__builtin_expect(lean_ok, 1)) {  // one uniform branch around the whole vector
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const float a = f[i];
+      float v = a * rs;
+      v = __builtin_fmaf(__builtin_fmaf(-s, v, a), rs, v);
+      if constexpr (STEPS == 2) v = __builtin_fmaf(__builtin_fmaf(-s, v, a), rs, v);
+      // a zero residual added to a quotient of -0 gives +0: the quotient takes the sign of a (s > 0), as the
+      // divide's does, so that -0.0 still becomes the code 0x80
+      v = __uint_as_float((__float_as_uint(v) & 0x7fffffffu) | (__float_as_uint(a) & 0x80000000u));
+      f[i] = fminf(fmaxf(v, -448.0f), 448.0f);
+    }
   } else {
-    v = __fdiv_rn(a, s);
+#pragma unroll
+    for (int i = 0; i < N; ++i) f[i] = fminf(fmaxf(__fdiv_rn(f[i], s), -448.0f), 448.0f);
   }
-  return fminf(fmaxf(v, -448.0f), 448.0f);
 }
 
 template <bool BF16>
@@ -463,8 +467,7 @@ __global__ __launch_bounds__(256) void cast_fp8_kernel(const void* __restrict__ 
       if (v >= nvec) break;
       float f[EPV];
       RowIn<BF16>::unpack(t[u], f);
-#pragma unroll
-      for (int i = 0; i < EPV; ++i) f[i] = fp8_prescale<STEPS>(f[i], s, rs, lean_ok);
+      fp8_prescale<STEPS, EPV>(f, s, rs, lean_ok);
       // v_cvt_pk_fp8_f32: two fp32 -> two OCP e4m3fn codes, round to nearest even.
       int w0 = __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], 0, false);
       w0 = __builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], w0, true);
@@ -480,6 +483,136 @@ __global__ __launch_bounds__(256) void cast_fp8_kernel(const void* __restrict__ 
       }
     }
   }
+}
+
+// Both passes in ONE launch for tensors that fit the register files: a workgroup per compute unit keeps its share
+// of x in registers (ONEPASS_R 16-byte vectors per thread: 32 MiB over 256 workgroups of 1024 threads), takes the
+// maximum of it, exchanges the partial maxima with the other workgroups through `slots`, and casts from the
+// registers -- x is read from HBM once instead of twice.  What does not fit the registers is read again in the
+// second phase, as the two-launch form does.
+//
+// The exchange.  slots[b] = (tag << 32) | bits of workgroup b's maximum, one 8-byte device-scope store.  Every
+// launch leaves all G slots carrying the same tag, and that is the only state: a workgroup reads the tag T its own
+// slot holds, publishes T + 1 with its maximum, and polls until all G slots carry T + 1 (thread t watches slot t).
+// The slots must start out equal (zero-filled) and a workspace must always be used with the same G; overlapping
+// launches must not share one.  The wait is bounded: workgroups that cannot all be resident at once (another
+// kernel holding compute units, a device with fewer than G of them) would otherwise wait for each other forever.
+// After spin_limit polls a workgroup stops waiting and takes the maximum of the WHOLE tensor itself -- slow, the
+// same bits (a maximum has no order) -- and still publishes its slot, so the state stays consistent.
+constexpr int ONEPASS_THREADS = 1024;
+constexpr int ONEPASS_R = 8;
+
+template <bool BF16>
+__global__ __launch_bounds__(ONEPASS_THREADS) void quant_fp8_onepass_kernel(const void* __restrict__ x, int64_t nvec,
+                                                                            unsigned long long* __restrict__ slots,
+                                                                            uint8_t* __restrict__ q,
+                                                                            float* __restrict__ scale, int spin_limit) {
+  constexpr int EPV = RowIn<BF16>::EPV;
+  constexpr int NW = ONEPASS_THREADS / 64;
+  __shared__ float wmax[NW];
+  __shared__ uint32_t tag_lds;
+  const int tid = threadIdx.x, G = gridDim.x;
+  const uint4* src = reinterpret_cast<const uint4*>(x);
+  // vector index of (round k, this thread): workgroups interleaved per round, 16 KiB contiguous per workgroup
+  const int64_t round = (int64_t)G * ONEPASS_THREADS;
+  const int64_t v0 = (int64_t)blockIdx.x * ONEPASS_THREADS + tid;
+  uint4 c[ONEPASS_R];
+#pragma unroll
+  for (int k = 0; k < ONEPASS_R; ++k) {
+    const int64_t i = v0 + k * round;
+    c[k] = make_uint4(0, 0, 0, 0);
+    if (i < nvec) c[k] = src[i];
+  }
+  // the tag this launch publishes: one more than the one this workgroup's slot carries.  Requested behind the
+  // data (loads return in request order; the tag is not needed before the maximum is known)
+  asm volatile("" ::: "memory");
+  unsigned long long old_slot = 0;
+  if (tid == 0) old_slot = __hip_atomic_load(slots + blockIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  asm volatile("" ::: "memory");
+  float amax = 0.0f;
+#pragma unroll
+  for (int k = 0; k < ONEPASS_R; ++k) {
+    float f[EPV];
+    RowIn<BF16>::unpack(c[k], f);
+    amax = fmaxf(amax, vec_amax<EPV>(f));
+  }
+  for (int64_t i = v0 + ONEPASS_R * round; i < nvec; i += round) {  // the part that does not fit the registers
+    float f[EPV];
+    RowIn<BF16>::unpack(src[i], f);
+    amax = fmaxf(amax, vec_amax<EPV>(f));
+  }
+  amax = wave_max(amax);
+  if ((tid & 63) == 0) wmax[tid >> 6] = amax;
+  if (tid == 0) tag_lds = (uint32_t)(old_slot >> 32) + 1u;
+  __syncthreads();
+  const uint32_t tag = tag_lds;
+  if (tid == 0) {
+    float m = 0.0f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) m = fmaxf(m, wmax[w]);
+    __hip_atomic_store(slots + blockIdx.x, ((unsigned long long)tag << 32) | __float_as_uint(m), __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
+  }
+  // wait for the other workgroups' slots (bounded)
+  float seen = 0.0f;
+  bool mine = tid >= G;
+  int all = 0;
+  for (int spin = 0; spin < spin_limit; ++spin) {
+    if (!mine) {
+      const unsigned long long u = __hip_atomic_load(slots + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if ((uint32_t)(u >> 32) == tag) {
+        mine = true;
+        seen = __uint_as_float((uint32_t)u);
+      }
+    }
+    all = __syncthreads_and(mine ? 1 : 0);
+    if (all) break;
+    __builtin_amdgcn_s_sleep(4);
+  }
+  if (!all) {  // uniform: the others did not show up in time; the whole tensor's maximum, taken here
+    seen = 0.0f;
+    for (int64_t i = tid; i < nvec; i += ONEPASS_THREADS) {
+      float f[EPV];
+      RowIn<BF16>::unpack(src[i], f);
+      seen = fmaxf(seen, vec_amax<EPV>(f));
+    }
+  }
+  seen = wave_max(seen);
+  __syncthreads();  // wmax is reused
+  if ((tid & 63) == 0) wmax[tid >> 6] = seen;
+  __syncthreads();
+  float tmax = 0.0f;
+#pragma unroll
+  for (int w = 0; w < NW; ++w) tmax = fmaxf(tmax, wmax[w]);
+  float s = __fdiv_rn(tmax, 448.0f);
+  if (tmax == 0.0f) s = 1.0f;
+  if (blockIdx.x == 0 && tid == 0) *scale = s;
+  constexpr int STEPS = BF16 ? 1 : 2;
+  const float rs = fp8_reciprocal<STEPS>(s);
+  const bool lean_ok = s >= 5.421010862427522e-20f && s <= 1.8446744073709552e19f;  // [2^-64, 2^64]
+  auto cast_store = [&](const uint4& t, int64_t i) {
+    float f[EPV];
+    RowIn<BF16>::unpack(t, f);
+    fp8_prescale<STEPS, EPV>(f, s, rs, lean_ok);
+    int w0 = __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], 0, false);
+    w0 = __builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], w0, true);
+    if constexpr (BF16) {
+      int w1 = __builtin_amdgcn_cvt_pk_fp8_f32(f[4], f[5], 0, false);
+      w1 = __builtin_amdgcn_cvt_pk_fp8_f32(f[6], f[7], w1, true);
+      uint2 o;
+      o.x = (uint32_t)w0;
+      o.y = (uint32_t)w1;
+      store_wt(reinterpret_cast<uint2*>(q + i * EPV), o);
+    } else {
+      store_wt(reinterpret_cast<uint32_t*>(q + i * EPV), (uint32_t)w0);
+    }
+  };
+#pragma unroll
+  for (int k = 0; k < ONEPASS_R; ++k) {
+    const int64_t i = v0 + k * round;
+    if (i < nvec) cast_store(c[k], i);
+  }
+  for (int64_t i = v0 + ONEPASS_R * round; i < nvec; i += round) cast_store(src[i], i);
 }
 
 }  // namespace aq
@@ -629,6 +762,37 @@ extern "C" int aq_swiglu_quant_rowwise_i8(const void* ug, int dtype, int64_t M, 
   hipStream_t st = static_cast<hipStream_t>(stream);
   return dtype == AQ_BF16 ? launch_swiglu_quant<true>(ug, M, F, ld, q, scale, st)
                           : launch_swiglu_quant<false>(ug, M, F, ld, q, scale, st);
+}
+
+// (not static: the lab library's hook in lab.hip calls it with its own bound on the wait)
+namespace aq {
+int quant_tensor_fp8_onepass(const void* x, int x_dtype, int64_t numel, uint8_t* q, float* scale, void* ws,
+                             size_t ws_bytes, int spin_limit, hipStream_t st) {
+  if (x_dtype != AQ_F32 && x_dtype != AQ_BF16) return AQ_E_DTYPE;
+  if (numel < 0 || (numel % 16) != 0) return AQ_E_SHAPE;
+  if (!scale || !ws) return AQ_E_NULL;
+  if (numel > 0 && (!x || !q)) return AQ_E_NULL;
+  if (ws_bytes < AQ_FP8_ONEPASS_WS_BYTES) return AQ_E_WORKSPACE;
+  if (aq::check_ptr16(x) || aq::check_ptr16(q) || aq::check_ptr(ws, 8) || aq::check_ptr(scale, 4)) return AQ_E_ALIGN;
+  const int epv = x_dtype == AQ_BF16 ? 8 : 4;
+  const int64_t nvec = numel / epv;
+  // one workgroup per compute unit, at most one per slot; always the same count on a device, whatever the size
+  int g = aq::device_cus();
+  if (g > AQ_FP8_ONEPASS_WS_BYTES / 8) g = AQ_FP8_ONEPASS_WS_BYTES / 8;
+  if (x_dtype == AQ_BF16)
+    hipLaunchKernelGGL((aq::quant_fp8_onepass_kernel<true>), dim3((unsigned)g), dim3(aq::ONEPASS_THREADS), 0, st, x, nvec,
+                       static_cast<unsigned long long*>(ws), q, scale, spin_limit);
+  else
+    hipLaunchKernelGGL((aq::quant_fp8_onepass_kernel<false>), dim3((unsigned)g), dim3(aq::ONEPASS_THREADS), 0, st, x, nvec,
+                       static_cast<unsigned long long*>(ws), q, scale, spin_limit);
+  return (int)hipGetLastError();
+}
+}  // namespace aq
+
+extern "C" int aq_quant_tensor_fp8_onepass(const void* x, int x_dtype, int64_t numel, uint8_t* q, float* scale,
+                                           void* ws, size_t ws_bytes, void* stream) {
+  // 4096 polls of a few hundred nanoseconds each: a millisecond or two before a workgroup stops waiting
+  return aq::quant_tensor_fp8_onepass(x, x_dtype, numel, q, scale, ws, ws_bytes, 4096, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int aq_quant_tensor_fp8(const void* x, int x_dtype, int64_t numel, uint8_t* q,

@@ -223,6 +223,7 @@ class Fp8Linear(Linear):
         self.register_buffer("w_scale", torch.ones((1,), dtype=torch.float32, device=device))
         self.bias = nn.Parameter(torch.zeros(out_dim, device=device), requires_grad=False) if bias else None
         self._workspaces: dict = {}  # decode workspaces, one per (device, stream), as in QuantLinear
+        self._quant_states: dict = {}  # the one-launch activation quantiser's state, one per (device, stream)
 
     DECODE_MAX_ROWS = 16
 
@@ -273,7 +274,12 @@ class Fp8Linear(Linear):
             y = ops.gemv_fp8_decode(x2, self.qweight, self.w_scale, self.bias, out_dtype=x.dtype, workspace=ws,
                                     residual=residual)
         else:
-            xq, sx = ops.quant_tensor_fp8(x2)
+            ops._need_gpu(x, self.qweight)
+            key = (x.device, torch.cuda.current_stream(x.device).cuda_stream)
+            state = self._quant_states.get(key)
+            if state is None:
+                state = self._quant_states[key] = ops.fp8_onepass_state(x.device)
+            xq, sx = ops.quant_tensor_fp8(x2, state=state)  # one launch for large inputs
             y = ops.linear_fp8(xq, sx, self.qweight, self.w_scale, self.bias, out_dtype=x.dtype, residual=residual)
         return y.reshape(*lead, self.qweight.shape[0])
 

@@ -145,8 +145,23 @@ def swiglu_quant_rowwise_i8(ug: torch.Tensor) -> Tuple[torch.Tensor, torch.Tenso
     return q, s
 
 
-def quant_tensor_fp8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
-    """Per-tensor OCP e4m3fn -> (codes uint8 with x's shape, scale f32 [1])."""
+# From this many input bytes on, the one-launch form of the per-tensor quantiser is the faster one (below, its
+# exchange of partial maxima between workgroups costs more than the second launch: 6.9 against 4.6-5.2 us for small
+# tensors, level at 16 MiB, 13.0 against 16.5 us at 32 MiB).
+FP8_ONEPASS_MIN_BYTES = 16 << 20
+
+
+def fp8_onepass_state(device) -> torch.Tensor:
+    """The small piece of device state the one-launch per-tensor quantiser needs: zero-filled once, then reused
+    for every call on that device and stream (calls that overlap in time must not share one)."""
+    return torch.zeros((_abi.AQ_FP8_ONEPASS_WS_BYTES // 8,), dtype=torch.int64, device=device)
+
+
+def quant_tensor_fp8(x: torch.Tensor, state: Optional[torch.Tensor] = None,
+                     onepass: Optional[bool] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Per-tensor OCP e4m3fn -> (codes uint8 with x's shape, scale f32 [1]).
+    ``state`` (from ``fp8_onepass_state``): allows the one-launch form, which reads x from HBM once instead of
+    twice -- same codes and scale; taken for tensors of ``FP8_ONEPASS_MIN_BYTES`` and more, or as ``onepass`` says."""
     _need_gpu(x)
     xc = x.contiguous()
     n = xc.numel()
@@ -154,6 +169,20 @@ def quant_tensor_fp8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
         raise ValueError(f"numel must be a multiple of 16, got {n}")
     q = torch.empty(xc.shape, dtype=torch.uint8, device=x.device)
     s = torch.empty((1,), dtype=torch.float32, device=x.device)
+    if onepass is None:
+        onepass = state is not None and n * xc.element_size() >= FP8_ONEPASS_MIN_BYTES
+    if onepass:
+        if state is None:
+            raise ValueError("the one-launch form needs the state tensor of fp8_onepass_state()")
+        _need_gpu(state)
+        if state.dtype != torch.int64 or state.numel() * 8 < _abi.AQ_FP8_ONEPASS_WS_BYTES or not state.is_contiguous() \
+                or state.device != x.device:
+            raise ValueError("state must come from fp8_onepass_state() for x's device")
+        with _OnDevice(x.device):
+            rc = _abi.load().aq_quant_tensor_fp8_onepass(xc.data_ptr(), _dt(xc, "x"), n, q.data_ptr(), s.data_ptr(),
+                                                         state.data_ptr(), state.numel() * 8, _stream(x))
+        _abi.check(rc, "aq_quant_tensor_fp8_onepass")
+        return q, s
     ws = torch.empty((_abi.AQ_FP8_AMAX_WS_BYTES // 4,), dtype=torch.int32, device=x.device)  # partial maxima, stateless
     with _OnDevice(x.device):
         rc = _abi.load().aq_quant_tensor_fp8(xc.data_ptr(), _dt(xc, "x"), n, q.data_ptr(), s.data_ptr(),

@@ -522,6 +522,98 @@ def test_quant_tensor_fp8_scale_range_and_dense_midpoints(oracle, scale):
         assert float((fused - codes).abs().max()) <= 2e-5 * max(ref, 1e-30)
 
 
+def test_quant_tensor_fp8_one_launch_form_same_codes_and_scale(oracle):
+    """The one-launch per-tensor quantiser (partial maxima exchanged between the workgroups while the kernel runs,
+    the tensor held in registers in between) against the oracle and the two-launch form, bit for bit: sizes from
+    one vector to more than the registers hold (the rest is read again), both input types, calls in a row on ONE
+    state tensor with sizes going up and down (the state a call leaves is what the next one starts from), the
+    scale-setting element in the first, the last and a middle workgroup's share, a zero tensor."""
+    state = ops.fp8_onepass_state(DEV)
+    g = torch.Generator(device=DEV).manual_seed(77)
+    cases = [(16, torch.float32), (4096, torch.bfloat16), (1 << 20, torch.bfloat16), (48, torch.float32),
+             ((5 << 20) + 16 * 7, torch.float32), (20 << 20, torch.bfloat16), (256 * 1024 * 8 - 16, torch.bfloat16), (16, torch.bfloat16)]
+    for n, dt in cases:
+        x = (torch.randn(n, generator=g, device=DEV) * 0.3).to(dt)
+        for where in (0, n // 2 + 3, n - 1):
+            xx = x.clone()
+            xx[where] = -7.25  # the element that sets the scale: first, middle or last share
+            q, s = ops.quant_tensor_fp8(xx, state=state, onepass=True)
+            q2, s2 = ops.quant_tensor_fp8(xx)
+            assert s.item() == s2.item() == np.float32(7.25) / np.float32(448.0), (n, dt, where)
+            assert torch.equal(q, q2), (n, dt, where)
+        if n <= (1 << 20):
+            if dt == torch.bfloat16:
+                qo, so = oracle.c_quant_tensor_fp8(bf16_bits(xx), bf16_bits=True)
+            else:
+                qo, so = oracle.c_quant_tensor_fp8(to_np(xx))
+            assert np.float32(s.item()) == so and np.array_equal(to_np(q), qo)
+    q0, s0 = ops.quant_tensor_fp8(torch.zeros(64, 16, device=DEV), state=state, onepass=True)
+    assert s0.item() == 1.0 and not to_np(q0).any()
+    # the register-resident limit of this device: a tensor of 40 MiB takes the second-read path for its tail
+    big = (torch.randn(20 << 20, generator=g, device=DEV) * 2).to(torch.bfloat16)
+    q, s = ops.quant_tensor_fp8(big, state=state, onepass=True)
+    q2, s2 = ops.quant_tensor_fp8(big)
+    assert s.item() == s2.item() and torch.equal(q, q2)
+    with pytest.raises(ValueError):
+        ops.quant_tensor_fp8(big, onepass=True)  # no state
+    with pytest.raises(ValueError):
+        ops.quant_tensor_fp8(big, state=torch.zeros(8, dtype=torch.int64, device=DEV), onepass=True)  # too small
+
+
+def test_quant_tensor_fp8_one_launch_form_when_the_workgroups_do_not_wait(oracle):
+    """A device that cannot run all workgroups at once would leave them waiting for each other: the wait is bounded
+    and a workgroup that gives up takes the whole tensor's maximum itself.  Forced here from the host by a bound of
+    zero polls (lab build): same codes and scale, and the state it leaves is good for an ordinary call."""
+    from khaosz_amd import _abi
+    lab = _abi.load_lab()
+    state = ops.fp8_onepass_state(DEV)
+    g = torch.Generator(device=DEV).manual_seed(78)
+    st = torch.cuda.current_stream().cuda_stream
+    for n, dt, code in ((1 << 18, torch.bfloat16, _abi.AQ_BF16), (3 * 4096 + 16, torch.float32, _abi.AQ_F32)):
+        x = (torch.randn(n, generator=g, device=DEV) * 0.1).to(dt)
+        q = torch.empty(n, dtype=torch.uint8, device=DEV)
+        s = torch.empty(1, dtype=torch.float32, device=DEV)
+        for spin in (0, 1):
+            rc = lab.aq_lab_quant_tensor_fp8_onepass_spin(x.data_ptr(), code, n, q.data_ptr(), s.data_ptr(),
+                                                          state.data_ptr(), state.numel() * 8, spin, st)
+            assert rc == 0
+            q2, s2 = ops.quant_tensor_fp8(x)
+            assert s.item() == s2.item() and torch.equal(q, q2), (n, dt, spin)
+        q3, s3 = ops.quant_tensor_fp8(x, state=state, onepass=True)
+        assert s3.item() == s2.item() and torch.equal(q3, q2)
+
+
+def test_quant_tensor_fp8_one_launch_form_in_a_replayed_graph():
+    """Its state lives in device memory and moves on by itself, so a captured call can be replayed: three calls on
+    different inputs captured once, replayed five times with eager calls on the same state in between, every
+    replay's codes and scales equal to the two-launch form's."""
+    state = ops.fp8_onepass_state(DEV)
+    g = torch.Generator(device=DEV).manual_seed(79)
+    xs = [(torch.randn(512, 2048, generator=g, device=DEV) * (i + 1)).to(torch.bfloat16) for i in range(3)]
+    want = [ops.quant_tensor_fp8(x) for x in xs]
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for x in xs:
+            ops.quant_tensor_fp8(x, state=state, onepass=True)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            outs = [ops.quant_tensor_fp8(x, state=state, onepass=True) for x in xs]
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    for r in range(5):
+        for q, s in outs:
+            q.zero_()
+            s.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        for (q, s), (qw, sw) in zip(outs, want):
+            assert s.item() == sw.item() and torch.equal(q, qw), r
+        qe, se = ops.quant_tensor_fp8(xs[r % 3], state=state, onepass=True)  # eager work on the same state in between
+        assert se.item() == want[r % 3][1].item() and torch.equal(qe, want[r % 3][0])
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 1, 16), (33, 70, 144), (256, 128, 1024), (300, 260, 2048), (64, 96, 8192)])
 def test_linear_fp8_within_tolerance(oracle, tile, M, N, K):
     _say("linear_fp8", M, N, K)

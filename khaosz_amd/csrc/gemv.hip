@@ -507,10 +507,6 @@ __global__ __launch_bounds__(GM_MAX_WAVES * 64) void gemv_mfma_kernel(GemvArgs p
     xrows.issue(p.x, M, K, K, wave, WAVES, lane);
     if constexpr (NORM) xrows.issue_gamma(p.gamma, K, lane);
     asm volatile("" ::: "memory");  // request order: token rows, epilogue operands, the weight stream
-#ifdef AQ_GV_XWAIT
-    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
-    asm volatile("" ::: "memory");
-#endif
     load_epi();
     asm volatile("" ::: "memory");
     wload(0, wa);

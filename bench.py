@@ -277,6 +277,10 @@ def bench_fp8(torch, ops, args, dev):
     steps = max(10, min(args.steps, 50))
     ms = graph_time_ms(torch, step, steps, args.warmup)
     ms_k = graph_time_ms(torch, kernel_only, steps, args.warmup)
+    # the activation quantiser alone, in its one-launch form (what the step uses) and its stateless two-launch form
+    qbytes = 3 * M * K  # bf16 read once, codes written
+    us_q1 = graph_time_ms(torch, lambda i: ops.quant_tensor_fp8(xs[i % nbuf], state=qstate), steps, args.warmup) * 1e3
+    us_q2 = graph_time_ms(torch, lambda i: ops.quant_tensor_fp8(xs[i % nbuf]), steps, args.warmup) * 1e3
     # the same variant at decode sizes (configuration 2's shape): per-tensor cast inside the streaming GEMV
     dec = {}
     if not args.no_extra:
@@ -304,6 +308,8 @@ def bench_fp8(torch, ops, args, dev):
         "roofline": {"bound": "mfma", "kernel": "gemm_kernel<fp8,bf16>", "achieved": tk, "peak": PEAK_FP8_TFLOPS,
                      "unit": "TFLOP/s", "frac": tk / PEAK_FP8_TFLOPS, "traffic": traffic, "traffic_source": traffic_src,
                      "kernel_us": ms_k * 1e3, "algorithmic_flops": flops},
+        "quantise_kernel": {"us": us_q1, "gbs": qbytes / us_q1 / 1e3, "frac_hbm": qbytes / us_q1 / 1e3 / PEAK_HBM_GBS,
+                            "algorithmic_bytes": qbytes, "two_launch_form_us": us_q2},
         "decode_gemv_fp8_N8192_K2048": dec,
         "shape": (M, N, K),
     }

@@ -160,6 +160,20 @@ int aq_gemv_w8a8_decode_rmsnorm(const void *x, int x_dtype, const void *gamma, f
                                 int64_t M, int64_t N, int64_t K, void *ws, size_t ws_bytes,
                                 void *stream);
 
+/* An MLP's up and gate projections and its activation as one launch at decode (mlp.py:25-26:
+ * down(up(x) * silu(gate(x))), the part before `down`), with the norm in front folded in like
+ * aq_gemv_w8a8_decode_rmsnorm when gamma is not NULL (decoder_block.py:57).
+ * wq: [2F, K] codes, rows [0, F) the up projection and [F, 2F) the gate projection; sw, bias: [2F].
+ * h: [M, F] = u * (g / (1 + exp(-g))) with u, g the two projections as aq_gemv_w8a8_decode would have stored them
+ * in h_dtype (rounded to bf16 first for a bf16 h), the exponential and divide of aq_swiglu_quant_rowwise_i8, the
+ * product rounded to h_dtype: the [M, 2F] intermediate is never written and the separate activation launch
+ * disappears.  Served for bf16 x, 1 <= M <= 16, K <= 2048 a multiple of 512, F a multiple of 16
+ * (aq_gemv_w8a8_decode_swiglu_ok returns 1); otherwise AQ_E_RANGE and the caller takes the separate launches. */
+int aq_gemv_w8a8_decode_swiglu_ok(int x_dtype, int64_t M, int64_t F, int64_t K);
+int aq_gemv_w8a8_decode_swiglu(const void *x, int x_dtype, const void *gamma, float eps,
+                               const int8_t *wq, const float *sw, const void *bias, int bias_dtype,
+                               void *h, int h_dtype, int64_t M, int64_t F, int64_t K, void *stream);
+
 /* FP8 Linear: y[m, n] = (sum_k f(xq[m,k]) * f(wq[n,k])) * sx[0] * sw[0] with
  * fp32 accumulation, cast to y_dtype.  xq: [M, K], wq: [N, K] e4m3fn codes;
  * sx, sw: device scalars written by aq_quant_tensor_fp8.  Replaces F.linear

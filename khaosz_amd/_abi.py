@@ -32,6 +32,9 @@ SYMBOLS = {
     "aq_gemv_w8a8_decode_residual": (_int, [_vp, _int, _vp, _vp, _vp, _int, _vp, _vp, _int, _i64, _i64, _i64, _vp, _sz,
                                             _vp]),
     "aq_gemv_w8a8_decode_noalloc": (_int, [_vp, _int, _vp, _vp, _vp, _int, _vp, _vp, _int, _i64, _i64, _i64, _vp]),
+    "aq_gemv_w8a8_decode_swiglu_ok": (_int, [_int, _i64, _i64, _i64]),
+    "aq_gemv_w8a8_decode_swiglu": (_int, [_vp, _int, _vp, ctypes.c_float, _vp, _vp, _vp, _int, _vp, _int, _i64, _i64,
+                                          _i64, _vp]),
     "aq_gemv_w8a8_decode_rmsnorm": (_int, [_vp, _int, _vp, ctypes.c_float, _vp, _vp, _vp, _int, _vp, _vp, _int, _i64, _i64,
                                            _i64, _vp, _sz, _vp]),
     "aq_gemv_w8a8_codes_residual": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _vp, _vp, _int, _i64, _i64, _i64, _vp]),

@@ -367,6 +367,13 @@ class MLP(nn.Module):
             return self.forward(x, codes, norm=norm) + residual
         kw = {} if residual is None else {"residual": residual}
         if self._upgate is not None:
+            if (self._swiglu_quant and codes is None and isinstance(self.down, QuantLinear)
+                    and ops.gemv_swiglu_ok(x, self._upgate.qweight.shape[0] // 2)):
+                # decode step: up, gate and the activation in one launch (the [M, 2F] projections are never
+                # written), then `down`, which quantises the few rows of h itself
+                ug = self._upgate
+                h = ops.gemv_w8a8_decode_swiglu(x, ug.qweight, ug.w_scale, ug.bias, out_dtype=x.dtype, norm=norm)
+                return self.down(h.view(*x.shape[:-1], -1), **kw)
             if codes is not None:
                 ug = self._upgate.forward_codes(codes[0], codes[1], x.dtype).view(*x.shape[:-1], -1)
             else:

@@ -431,10 +431,17 @@ constexpr int GM_BATCH = 8;    // MFMA steps (64 K bytes each) per register batc
 // products run on v_mfma_f32_16x16x128_f8f6f4 -- one instruction per 128-byte line instead of two -- with fp32
 // accumulation; with FQ the kernel casts its bf16 rows itself, after the maximum over ALL rows (the per-tensor
 // scale of aq_quant_tensor_fp8: s = amax / 448, codes = e4m3(clamp(x / s))) has gone round the workgroup.
-template <int KS, int GR, bool RES, int XR, int FQ = 0, bool NORM = false, bool FP8 = false>
+// SWI: the weight is an MLP's up and gate projections stacked, rows [0, F) up and [F, 2F) gate with F = N / 2 (what
+// QuantLinear.concat([up, gate]) builds), and the kernel writes h = up * silu(gate), [M, F], instead of the 2F
+// projections: the first half of a workgroup's row groups takes 16-row blocks of up, the second half the same
+// blocks of gate, the gate sums cross to the up wavefronts through LDS, and the up wavefronts apply the activation
+// (the fixed-sequence exponential and correctly rounded divide of the stand-alone SwiGLU kernel) to the two
+// projections as the separate launch would have stored them (rounded to the output type first).
+template <int KS, int GR, bool RES, int XR, int FQ = 0, bool NORM = false, bool FP8 = false, bool SWI = false>
 __global__ __launch_bounds__(GM_MAX_WAVES * 64) void gemv_mfma_kernel(GemvArgs p) {
   static_assert(FQ == 0 || (KS > 0 && GR > 0), "the in-kernel quantiser deals rows to a fixed number of wavefronts");
   static_assert(!(FP8 && NORM), "no fused norm in front of the FP8 cast");
+  static_assert(!SWI || (FQ > 0 && !RES && !FP8 && GR % 2 == 0), "the SwiGLU epilogue exists for the int8 kernels that quantise their rows");
   extern __shared__ __attribute__((aligned(16))) uint8_t xs[];  // [16][K + 16] token codes, [16] scales, 16 spare bytes; later the partial sums
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -442,7 +449,12 @@ __global__ __launch_bounds__(GM_MAX_WAVES * 64) void gemv_mfma_kernel(GemvArgs p
   const int nthreads = ksplit * groups * 64;
   const int grp = wave / ksplit, kh = wave % ksplit;
   const int K = p.K, N = p.N, M = p.M;
-  const int n0 = __builtin_amdgcn_readfirstlane((blockIdx.x * groups + grp) * GM_ROWS);
+  // first weight row of this wavefront's group, and the end of the rows it may touch
+  const int FH = N >> 1;  // SWI: rows per half
+  const int hgroups = SWI ? groups >> 1 : groups;
+  const int ghalf = SWI ? grp / hgroups : 0, gsub = SWI ? grp - ghalf * hgroups : grp;
+  const int n0 = __builtin_amdgcn_readfirstlane((SWI ? ghalf * FH : 0) + (blockIdx.x * hgroups + gsub) * GM_ROWS);
+  const int nlim = SWI ? (ghalf + 1) * FH : N;
   const int pitch = K + 16;  // 16 token rows then start 4 banks apart: conflict-free 16-byte reads
   const int khalf = K / ksplit;  // a multiple of 128 (checked by the launcher)
   const int nline = khalf / 128;  // 128-byte lines of a row's K part: two MFMA steps each
@@ -465,16 +477,16 @@ __global__ __launch_bounds__(GM_MAX_WAVES * 64) void gemv_mfma_kernel(GemvArgs p
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const int n = rbase + r;
-      swv[r] = epi.load_sw(FP8 ? 0 : n, FP8 || n < N);
-      bv[r] = epi.load_bias(n, n < N);
-      rv[r] = RES ? epi.load_res(tok, n, tok < M && n < N, (int)p.ldr) : 0u;
+      swv[r] = epi.load_sw(FP8 ? 0 : n, FP8 || n < nlim);
+      bv[r] = epi.load_bias(n, n < nlim);
+      rv[r] = RES ? epi.load_res(tok, n, tok < M && n < nlim, (int)p.ldr) : 0u;
     }
   };
 
   // weight stream: descriptor over this wavefront's 16 rows; rows past N read as zero
-  const int rows = n0 < N ? ((N - n0) < GM_ROWS ? (N - n0) : GM_ROWS) : 0;
+  const int rows = n0 < nlim ? ((nlim - n0) < GM_ROWS ? (nlim - n0) : GM_ROWS) : 0;
   const __amdgpu_buffer_rsrc_t Wr =
-      make_rsrc(p.wq + (int64_t)(n0 < N ? n0 : 0) * K, (uint32_t)rows * (uint32_t)K);
+      make_rsrc(p.wq + (int64_t)(n0 < nlim ? n0 : 0) * K, (uint32_t)rows * (uint32_t)K);
   // Whole 128-byte lines per load: an instruction covers one line of 8 rows (lane l: row l % 8, 16-byte piece
   // l / 8), two instructions (rows 0..7 and 8..15) per line index.  In the MFMA's own operand order (lane l: row
   // l % 16, piece l / 16 of a 64-byte step) an instruction would cover 16 half lines, and a one-shot read of
@@ -684,6 +696,49 @@ __global__ __launch_bounds__(GM_MAX_WAVES * 64) void gemv_mfma_kernel(GemvArgs p
     *reinterpret_cast<accv*>(part + (kh - 1) * 256 + lane * 4) = acc;
   }
   __syncthreads();
+  if constexpr (SWI) {
+    // every wavefront stays for the exchange: gate sums -> LDS (behind the K-part area) -> the up wavefronts
+    float* const ex = reinterpret_cast<float*>(xs) + groups * (ksplit - 1) * 256 + (gsub * 64 + lane) * 4;
+    const bool live = kh == 0;
+    float u[4];
+    if (live) {
+      for (int k = 0; k < ksplit - 1; ++k) acc += *reinterpret_cast<const accv*>(part + k * 256 + lane * 4);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        u[r] = __fmul_rn(__fmul_rn((float)acc[r], sxv), swv[r]);
+        if (p.bias) u[r] = __fadd_rn(u[r], bv[r]);
+        if (p.y_dtype == AQ_BF16) u[r] = bf16_bits_to_f32(f32_to_bf16_bits(u[r]));  // as the projection would be stored
+      }
+      if (ghalf == 1) *reinterpret_cast<float4*>(ex) = make_float4(u[0], u[1], u[2], u[3]);
+    }
+    __syncthreads();
+    if (!live || ghalf == 1 || tok >= M) return;
+    const float4 g4 = *reinterpret_cast<const float4*>(ex);
+    const float g[4] = {g4.x, g4.y, g4.z, g4.w};
+    float h[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) h[r] = swiglu_repro(u[r], g[r]);
+    const int64_t o = (int64_t)tok * FH + rbase;  // rbase lies in the up half: the column of h
+    if (p.y_dtype == AQ_BF16) {
+      uint16_t* dst = reinterpret_cast<uint16_t*>(p.y) + o;
+      if ((FH & 3) == 0 && rbase + 3 < FH) {
+        uint2 pk;
+        pk.x = pack_bf16x2(h[0], h[1]);
+        pk.y = pack_bf16x2(h[2], h[3]);
+        *reinterpret_cast<uint2*>(dst) = pk;
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (rbase + r < FH) dst[r] = (uint16_t)f32_to_bf16_bits(h[r]);
+      }
+    } else {
+      float* dst = reinterpret_cast<float*>(p.y) + o;
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (rbase + r < FH) dst[r] = h[r];
+    }
+    return;
+  }
   if (kh != 0) return;
   for (int k = 0; k < ksplit - 1; ++k) acc += *reinterpret_cast<const accv*>(part + k * 256 + lane * 4);  // fp32: a fixed order
 
@@ -803,6 +858,32 @@ static int launch_gemv_mfma_fq(GemvArgs a, hipStream_t st, bool fp8 = false) {
   return (int)hipGetLastError();
 }
 
+// up/gate + SwiGLU in one launch: bf16 rows of K <= 2048 in whole 512-byte steps, F a multiple of 16.
+static bool gemv_mfma_swiglu_ok(int64_t M, int64_t F, int64_t K) {
+  return M >= 1 && M <= 16 && F > 0 && (F % 16) == 0 && K <= 2048 && (K % 512) == 0;
+}
+
+// a.N = 2 F.  A workgroup holds 16 (2 x 4 wavefronts: up block, gate block) or, once F has more 16-row blocks than the
+// device has compute units, 32 columns of h (4 x 2 wavefronts).
+static int launch_gemv_mfma_swiglu(GemvArgs a, hipStream_t st) {
+  const int F = a.N / 2;
+  const bool wide = (F + 15) / 16 > device_cus();
+  a.ksplit = wide ? 2 : 4;
+  a.groups = wide ? 4 : 2;
+  const int per_wg = GM_ROWS * (a.groups / 2);
+  const unsigned grid = (unsigned)((F + per_wg - 1) / per_wg);
+  const size_t lds = (size_t)16 * (a.K + 16) + 16 * sizeof(float) + 16;
+  const bool many = a.M > 8, norm = a.gamma != nullptr;
+  using kern_t = void (*)(GemvArgs);
+#define AQ_SWI_TABLE(KS, GR)                                                                                   \
+  {{gemv_mfma_kernel<KS, GR, false, 1, 8, false, false, true>, gemv_mfma_kernel<KS, GR, false, 1, 8, true, false, true>},   \
+   {gemv_mfma_kernel<KS, GR, false, 1, 16, false, false, true>, gemv_mfma_kernel<KS, GR, false, 1, 16, true, false, true>}}
+  static const kern_t table[2][2][2] = {AQ_SWI_TABLE(4, 2), AQ_SWI_TABLE(2, 4)};
+#undef AQ_SWI_TABLE
+  hipLaunchKernelGGL(table[wide][many][norm], dim3(grid), dim3(8 * 64), lds, st, a);
+  return (int)hipGetLastError();
+}
+
 static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 }  // namespace aq
@@ -850,6 +931,11 @@ static int gemv_dispatch_fused(const aq::GemvArgs& a, int mt, hipStream_t st) {
   if (aq::gemv_mfma_fq_ok(a.M, a.N, a.K)) return aq::launch_gemv_mfma_fq(a, st);
   const int64_t vpl = (a.K / 8 + 63) / 64;  // 16-byte vectors per lane per bf16 row
   if (mt > 8 || vpl > 16) return -1;
+  // A short matrix with long rows (an MLP's down projection): the fused kernel cannot cut rows into K parts, so
+  // its N / 32 workgroups leave most compute units without loads in flight, and the separate row quantiser + the
+  // K-split GEMV on codes is faster (N = 2048, K = 5632, 8 rows: 11.0 against 9.1 us; K = 8192: 13.3 against 10.5;
+  // from N = 4096 on the one launch wins again).
+  if ((a.N + 31) / 32 * 4 <= aq::device_cus() && (a.K > 4096 || (a.M > 4 && a.K >= 4096))) return -1;
   const bool small = vpl <= 4;
   if (a.gamma) {  // with the norm in front: short rows only (the gain's vectors stay in registers too)
     if (!small) return -1;
@@ -1130,6 +1216,37 @@ extern "C" int aq_gemv_w8a8_decode_rmsnorm(const void* x, int x_dtype, const voi
   rc = aq_rmsnorm_quant_rowwise_i8(x, x_dtype, gamma, x_dtype, eps, M, K, K, xq, sx, stream);
   if (rc) return rc;
   return aq_gemv_w8a8_codes_residual(xq, sx, wq, sw, bias, bias_dtype, residual, y, y_dtype, M, N, K, stream);
+}
+
+extern "C" int aq_gemv_w8a8_decode_swiglu_ok(int x_dtype, int64_t M, int64_t F, int64_t K) {
+  return x_dtype == AQ_BF16 && aq::gemv_mfma_swiglu_ok(M, F, K) ? 1 : 0;
+}
+
+extern "C" int aq_gemv_w8a8_decode_swiglu(const void* x, int x_dtype, const void* gamma, float eps, const int8_t* wq,
+                                          const float* sw, const void* bias, int bias_dtype, void* h, int h_dtype,
+                                          int64_t M, int64_t F, int64_t K, void* stream) {
+  if (x_dtype != AQ_F32 && x_dtype != AQ_BF16) return AQ_E_DTYPE;
+  if (F < 0 || F > (1 << 24)) return F < 0 ? AQ_E_SHAPE : AQ_E_RANGE;
+  int mt = 0;
+  int rc = gemv_check(wq, sw, bias, bias_dtype, nullptr, h, h_dtype, M, 2 * F, K, &mt);
+  if (rc || M == 0 || F == 0) return rc;
+  if (!x) return AQ_E_NULL;
+  if (aq::check_ptr16(x) || aq::check_ptr16(gamma)) return AQ_E_ALIGN;
+  if (!aq_gemv_w8a8_decode_swiglu_ok(x_dtype, M, F, K)) return AQ_E_RANGE;  // the caller takes the separate launches
+  aq::GemvArgs a{};
+  a.x = x;
+  a.gamma = gamma;
+  a.eps = eps;
+  a.wq = wq;
+  a.sw = sw;
+  a.bias = bias;
+  a.y = h;
+  a.M = (int)M;
+  a.N = (int)(2 * F);
+  a.K = (int)K;
+  a.bias_dtype = bias_dtype;
+  a.y_dtype = h_dtype;
+  return aq::launch_gemv_mfma_swiglu(a, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int aq_gemv_w8a8_decode(const void* x, int x_dtype, const int8_t* wq, const float* sw,

@@ -317,6 +317,53 @@ def gemv_w8a8_decode(x, wq, sw, bias=None, out_dtype=None, workspace: Optional[t
     return y
 
 
+def gemv_swiglu_ok(x: torch.Tensor, dim_ffn: int) -> bool:
+    """Whether ``gemv_w8a8_decode_swiglu`` serves these rows (bf16, at most 16 of them, K <= 2048 in whole
+    512-byte steps, dim_ffn a multiple of 16)."""
+    if not x.is_cuda or x.dtype not in _DT:
+        return False
+    rows = x.numel() // x.shape[-1] if x.shape[-1] else 0
+    return bool(_abi.load().aq_gemv_w8a8_decode_swiglu_ok(_DT[x.dtype], rows, dim_ffn, x.shape[-1]))
+
+
+def gemv_w8a8_decode_swiglu(x, wq, sw, bias=None, out_dtype=None, norm=None) -> torch.Tensor:
+    """``up(x) * silu(gate(x))`` of an MLP at decode in ONE launch: ``wq [2F, K]`` holds the up projection's rows and
+    then the gate projection's (``QuantLinear.concat([up, gate])``); returns ``h [M, F]``.  ``norm = (gamma, eps)``:
+    the RMSNorm in front, folded in as in ``gemv_w8a8_decode``.  Raises ``ValueError`` for shapes
+    ``gemv_swiglu_ok`` refuses."""
+    _need_gpu(x, wq, sw, bias, norm[0] if norm is not None else None)
+    x2 = _rows(x, "gemv_w8a8_decode_swiglu")
+    M, K = x2.shape
+    if wq.dtype != torch.int8 or wq.dim() != 2 or wq.shape[1] != K or wq.shape[0] % 2:
+        raise ValueError(f"wq must be int8 [2F, {K}], got {wq.dtype} {tuple(wq.shape)}")
+    N = wq.shape[0]
+    Fh = N // 2
+    _check_k(K)
+    if sw.dtype != torch.float32 or sw.numel() != N:
+        raise ValueError("sw must be float32 [2F]")
+    out_dtype = out_dtype or x.dtype
+    if out_dtype not in _DT:
+        raise ValueError(f"out_dtype {out_dtype} is not supported")
+    wq, sw = wq.contiguous(), sw.contiguous()
+    b, bdt = _bias_args(bias, N)
+    gamma, eps = (None, 0.0)
+    if norm is not None:
+        gamma, eps = norm
+        if gamma.dtype != x2.dtype or gamma.numel() != K:
+            raise ValueError(f"the norm's gain must be {x2.dtype} [{K}], got {gamma.dtype} {tuple(gamma.shape)}")
+        gamma = gamma.contiguous()
+    h = torch.empty((M, Fh), dtype=out_dtype, device=x.device)
+    if M and Fh:
+        with _OnDevice(x.device):
+            rc = _abi.load().aq_gemv_w8a8_decode_swiglu(x2.data_ptr(), _dt(x2, "x"),
+                                                        gamma.data_ptr() if gamma is not None else None, float(eps),
+                                                        wq.data_ptr(), sw.data_ptr(),
+                                                        b.data_ptr() if b is not None else None, bdt, h.data_ptr(),
+                                                        _DT[out_dtype], M, Fh, K, _stream(x))
+        _abi.check(rc, "aq_gemv_w8a8_decode_swiglu")
+    return h
+
+
 def gemv_w8a8_codes(xq, sx, wq, sw, bias=None, out_dtype=torch.bfloat16, residual=None) -> torch.Tensor:
     """The decode GEMV on activation codes the caller already holds (at most 16 rows)."""
     _need_gpu(xq, sx, wq, sw, bias, residual)

@@ -633,12 +633,15 @@ def test_config5_full_size_fused_block_against_the_unfused_block_and_an_oracle_c
         hq, hs = oracle.c_rmsnorm_quant_i8(h_bits, bits(n2.weight), n2.norm_eps, bf16_bits=True)
         ug = oracle.c_dequant_epilogue(oracle.c_gemm_i8_i32(hq, mlp._upgate.qweight.cpu().numpy()), hs,
                                        mlp._upgate.w_scale.cpu().numpy(), bf16_out=True)
-        aq, asc = oracle.c_swiglu_quant_i8(ug, bf16_bits=True)
+        # a decode step: up, gate and the activation are one launch that rounds h to bf16, and `down` quantises
+        # those bf16 rows itself (the prefill's activation kernel quantises h from fp32 instead)
+        _, _, hf = oracle.c_swiglu_quant_i8(ug, bf16_bits=True, want_h=True)
+        aq, asc = oracle.c_quant_rowwise_i8(oracle.np_f32_to_bf16_bits(hf), bf16_bits=True)
         d = oracle.c_dequant_epilogue(oracle.c_gemm_i8_i32(aq, mlp.down.qweight.cpu().numpy()), asc,
                                       mlp.down.w_scale.cpu().numpy(), bf16_out=True)
         return add_bf16(d, h_bits)
 
     assert rel(out_gpu.reshape(B, dim).cpu(), from_bits(mlp_half(h))) < 1e-2      # whole step, oracle end to end
-    # the MLP half on the bits the GPU's attention half produced: norm + quantise, up/gate, SwiGLU + quantise,
+    # the MLP half on the bits the GPU's attention half produced: norm + quantise, up/gate + SwiGLU, quantise,
     # down and the residual add, bit for bit
     assert np.array_equal(bits(out_gpu.reshape(B, dim)), mlp_half(bits(h_gpu.reshape(B, dim))))

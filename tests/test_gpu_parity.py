@@ -411,6 +411,55 @@ def test_gemv_with_the_norm_folded_in_equals_norm_quantise_then_gemv(oracle, M, 
         assert torch.equal(got, want)
 
 
+@pytest.mark.parametrize("M,F,K,norm", [(8, 5632, 2048, True), (4, 6912, 1536, True), (16, 5632, 2048, False),
+                                          (1, 48, 512, False), (11, 8208, 1024, True), (3, 2048, 2048, False)])
+def test_up_gate_gemv_with_the_activation_in_its_epilogue_against_an_oracle_composition(oracle, M, F, K, norm):
+    """up(x) * silu(gate(x)) as one launch at decode.  Composed on the CPU from the oracle's own functions: the
+    row quantiser (with the RMSNorm in front when folded in), the int8 GEMM and its epilogue rounded to bf16 for
+    both projections, the SwiGLU arithmetic on those bf16 values, one rounding to bf16.  Bit for bit, with and
+    without a bias, for F below and above the device's count of 16-row blocks (both workgroup shapes) and F not a
+    multiple of the workgroup's columns; and the same codes for `down` as the separate activation kernel would
+    give when h is quantised afterwards."""
+    _say("gemv+swiglu", M, F, K)
+    g = torch.Generator().manual_seed(M * 131 + F)
+    x = (torch.randn(M, K, generator=g) * (0.2 + 2 * torch.rand(M, 1, generator=g))).to(torch.bfloat16).to(DEV)
+    gamma = (1 + 0.2 * torch.randn(K, generator=g)).to(torch.bfloat16).to(DEV)
+    w = make_x(2 * F, K, 15) * 0.03
+    wq, sw = oracle.c_quant_rowwise_i8(w.numpy())
+    wqd, swd = torch.from_numpy(wq).to(DEV), torch.from_numpy(sw).to(DEV)
+    bias = (torch.randn(2 * F, generator=g) * 0.05)
+    if norm:
+        xq, sx = oracle.c_rmsnorm_quant_i8(bf16_bits(x), bf16_bits(gamma), 1e-5, bf16_bits=True)
+    else:
+        xq, sx = oracle.c_quant_rowwise_i8(bf16_bits(x), bf16_bits=True)
+    acc = oracle.c_gemm_i8_i32(xq, wq)
+    assert ops.gemv_swiglu_ok(x, F)
+    for b in (None, bias):
+        ug = oracle.c_dequant_epilogue(acc, sx, sw, None if b is None else b.numpy(), bf16_out=True)  # bf16 bits [M, 2F]
+        _, _, h = oracle.c_swiglu_quant_i8(ug, bf16_bits=True, want_h=True)
+        want = oracle.np_f32_to_bf16_bits(h)
+        got = ops.gemv_w8a8_decode_swiglu(x, wqd, swd, None if b is None else b.to(DEV), out_dtype=torch.bfloat16,
+                                          norm=(gamma, 1e-5) if norm else None)
+        assert got.shape == (M, F)
+        assert np.array_equal(bf16_bits(got), want), int((bf16_bits(got) != want).sum())
+    # fp32 output: the projections are not rounded in between
+    ugf = oracle.c_dequant_epilogue(acc, sx, sw, None, bf16_out=False)
+    _, _, hf = oracle.c_swiglu_quant_i8(ugf, want_h=True)
+    gotf = ops.gemv_w8a8_decode_swiglu(x, wqd, swd, None, out_dtype=torch.float32, norm=(gamma, 1e-5) if norm else None)
+    assert np.array_equal(to_np(gotf).view(np.uint32), hf.view(np.uint32))
+
+
+def test_up_gate_gemv_with_the_activation_refuses_what_it_does_not_serve():
+    x = torch.zeros(4, 4096, dtype=torch.bfloat16, device=DEV)  # rows too long for the in-kernel quantiser
+    assert not ops.gemv_swiglu_ok(x, 1024)
+    assert not ops.gemv_swiglu_ok(torch.zeros(4, 2048, dtype=torch.float32, device=DEV), 1024)  # fp32 rows
+    assert not ops.gemv_swiglu_ok(torch.zeros(17, 2048, dtype=torch.bfloat16, device=DEV), 1024)
+    assert not ops.gemv_swiglu_ok(torch.zeros(4, 2048, dtype=torch.bfloat16, device=DEV), 1000)  # F not a multiple of 16
+    with pytest.raises(ValueError):
+        ops.gemv_w8a8_decode_swiglu(x, torch.zeros(2048, 4096, dtype=torch.int8, device=DEV),
+                                    torch.ones(2048, device=DEV))
+
+
 @pytest.mark.parametrize("M,K", [(12, 11008), (16, 14336), (7, 22016)])
 def test_decode_rows_too_long_for_the_gemv_take_the_tiled_gemm(oracle, M, K):
     """Activation codes of 9..16 tokens fit a compute unit's LDS up to K = 10 096 (5..8 tokens: 20 208).

@@ -913,7 +913,12 @@ static int gemv_check(const int8_t* wq, const float* sw, const void* bias, int b
 }
 
 static int gemv_dispatch(const aq::GemvArgs& a, int mt, hipStream_t st) {
-  if (aq::gemv_mfma_ok(a.M, a.K)) return aq::launch_gemv_mfma(a, st);
+  // 9..16 rows go to the matrix-core variant, except on a short matrix with long rows (an MLP's down projection):
+  // its 16-row wavefronts make N / 16 workgroups, half the device or less, where the dot-product kernel's 4-row
+  // wavefronts still reach every compute unit (N = 2048, K = 5632: 7.6-8.0 against 8.5 us; N = 1536, K = 6912:
+  // 11.0 against 12.9 us; at K = 2048 or from N = 3072 on the matrix core wins, 4.7 against 5.6 us).
+  const bool short_long = (a.N + 15) / 16 * 2 <= aq::device_cus() && a.K >= 4096;
+  if (aq::gemv_mfma_ok(a.M, a.K) && !short_long) return aq::launch_gemv_mfma(a, st);
   switch (mt) {
     case 1: return aq::launch_gemv<1, false, 4>(a, st);
     case 2: return aq::launch_gemv<2, false, 4>(a, st);

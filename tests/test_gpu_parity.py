@@ -366,7 +366,7 @@ def test_linear_residual_may_alias_the_output(tile):
 # ------------------------------------------------------------------- decode
 
 @pytest.mark.parametrize("M", [1, 2, 3, 4, 5, 8, 11, 16])
-@pytest.mark.parametrize("N,K", [(8192, 2048), (50, 16), (130, 1040), (2048, 5632), (11264, 2048), (8200, 512), (77, 1536)])
+@pytest.mark.parametrize("N,K", [(8192, 2048), (50, 16), (130, 1040), (2048, 5632), (1536, 6912), (11264, 2048), (8200, 512), (77, 1536)])
 def test_gemv_decode_bit_exact(oracle, M, N, K):
     """(11264, 2048), (8200, 512) and 9+ rows of (77, 1536) take the matrix-core kernel that quantises its rows
     itself: 64-row workgroups on the first (more 32-row blocks than compute units), a ragged last block on the

@@ -350,12 +350,16 @@ struct LdsOptIn {
     return 0;
   }
 };
-static GemvShape gemv_shape(int N, int K, bool fused) {
+static GemvShape gemv_shape(int N, int K, bool fused, int mt) {
   GemvShape sh{GV_WAVES, 1};
   if (fused) return sh;
   const int cus = device_cus();
   const int groups = (N + GV_ROWS - 1) / GV_ROWS, nchunk = (K + GV_CHUNK - 1) / GV_CHUNK;
-  while (nchunk >= 4 && sh.ksplit < 4 && groups * sh.ksplit < 4 * cus && nchunk >= 2 * sh.ksplit) sh.ksplit *= 2;
+  // K parts until the device holds 4 wavefronts per compute unit -- 8 for up to 4 tokens, where the extra loads in
+  // flight pay (N = K = 4096, 1 token: 6.25 -> 5.5 us) and the token codes every workgroup copies are few; with 8
+  // tokens the same change costs 0.4 us
+  const int waves_per_cu = mt <= 4 ? 8 : 4;
+  while (nchunk >= 4 && sh.ksplit < 4 && groups * sh.ksplit < waves_per_cu * cus && nchunk >= 2 * sh.ksplit) sh.ksplit *= 2;
   int per_wg = GV_WAVES / sh.ksplit;  // row groups per workgroup
   while (per_wg > 1 && (groups + per_wg - 1) / per_wg < cus) per_wg >>= 1;
   if (sh.ksplit == 1 && per_wg < 2) per_wg = 2;
@@ -365,7 +369,7 @@ static GemvShape gemv_shape(int N, int K, bool fused) {
 
 template <int MT, bool FUSED, int VPL, bool NORM, int MERGE, int FW>
 static int launch_gemv_fw(GemvArgs a, hipStream_t st) {
-  GemvShape sh = gemv_shape(a.N, a.K, FUSED);
+  GemvShape sh = gemv_shape(a.N, a.K, FUSED, MT);
   if (FUSED) sh.waves = FW;
   a.ksplit = sh.ksplit;
   const int rows_per_wg = GV_ROWS * (sh.waves / sh.ksplit);
@@ -823,11 +827,13 @@ static int launch_gemv_mfma(GemvArgs a, hipStream_t st, bool fp8 = false) {
 //   9..16 tokens: always (N = 8192: 7.6 us against 8.4 us for row quantiser + GEMV; N = 2048: 6.6 against 7.1);
 //   5..8 tokens: from N = 8192 on (6.45 us against 7.4 us for the dot-product kernel, which is bound by its
 //                vector ALU there; at N = 4096 the dot-product kernel still wins, 4.8 against 5.2 us);
+//                with the norm folded in, whose arithmetic weighs on the dot-product kernel's fewer wavefronts,
+//                from N = 6144 on (7.2 -> 6.5 us there; level at N = 3072);
 //   3..4 tokens: only for matrices with more 32-row blocks than compute units (N = 11264: 7.0 against 7.6 us).
-static bool gemv_mfma_fq_ok(int64_t M, int64_t N, int64_t K) {
+static bool gemv_mfma_fq_ok(int64_t M, int64_t N, int64_t K, bool norm = false) {
   if (K > 2048 || (K % 512) != 0) return false;
   const bool wide = (N + 31) / 32 > device_cus();
-  return M >= 9 || (M >= 5 && N >= 8192) || (M >= 3 && wide);
+  return M >= 9 || (M >= 5 && N >= (norm ? 6144 : 8192)) || (M >= 3 && wide);
 }
 
 static int launch_gemv_mfma_fq(GemvArgs a, hipStream_t st, bool fp8 = false) {
@@ -933,7 +939,7 @@ static int gemv_dispatch(const aq::GemvArgs& a, int mt, hipStream_t st) {
 // than 8 rows every workgroup would repeat 2+ row quantisations per wavefront
 // on its critical path, which measures no faster than the separate launch.
 static int gemv_dispatch_fused(const aq::GemvArgs& a, int mt, hipStream_t st) {
-  if (aq::gemv_mfma_fq_ok(a.M, a.N, a.K)) return aq::launch_gemv_mfma_fq(a, st);
+  if (aq::gemv_mfma_fq_ok(a.M, a.N, a.K, a.gamma != nullptr)) return aq::launch_gemv_mfma_fq(a, st);
   const int64_t vpl = (a.K / 8 + 63) / 64;  // 16-byte vectors per lane per bf16 row
   if (mt > 8 || vpl > 16) return -1;
   // A short matrix with long rows (an MLP's down projection): the fused kernel cannot cut rows into K parts, so

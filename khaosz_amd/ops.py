@@ -480,8 +480,14 @@ def attn_gemv_fusable(B: int, n_heads: int, head_dim: int, total_len: int) -> bo
     """Whether ``gemv_w8a8_attn`` can, and should, combine this step's attention slices itself:
     within the kernel's limits, and more than one slice (a single slice has no merge launch to
     save, and the attention kernel's bf16 output is the smaller input)."""
-    return (0 < B <= GEMV_ATTN_MAX_ROWS and n_heads * head_dim <= GEMV_ATTN_MAX_K
-            and 256 < total_len <= GEMV_ATTN_MAX_SLICES * 256)
+    if not (0 < B <= GEMV_ATTN_MAX_ROWS and n_heads * head_dim <= GEMV_ATTN_MAX_K
+            and 256 < total_len <= GEMV_ATTN_MAX_SLICES * 256):
+        return False
+    # Every workgroup of the projection repeats the merge of all rows, so it pays only while that is little work
+    # (rows x row length x slices): 4 x 1536 x 3 saves 1.2 us per step over the separate merge launch, 8 x 2048 x 3
+    # loses 0.8 us.
+    slices = (total_len + 255) // 256
+    return B * n_heads * head_dim * slices <= 32768
 
 
 def rope_paged_attn_decode(qkv: torch.Tensor, freqs: torch.Tensor, page_table: torch.Tensor, total_len: int,

@@ -552,7 +552,7 @@ def test_chunked_prefill_on_cached_tokens_uses_the_paged_kernel_and_tracks_the_m
 def test_config5_full_size_fused_block_against_the_unfused_block_and_an_oracle_composition(oracle):
     """Benchmark configuration 5 at its own size on the path the benchmark times: hidden 2048, 16 query /
     4 KV heads of 128, FFN 5632, every fusion on, 8 x 512 prefill through a shuffled table of 64-token pages,
-    then decode steps of 8 tokens past 512 cached positions (position slices, merge inside o_proj).
+    then decode steps of 8 tokens past 512 cached positions (position slices combined by the merge launch: at this size the output projection leaves that to it).
     (i) every step against the same weights in the unfused quantized block; (ii) one decode step against the
     decoder block (decoder_block.py:43-59) composed on the CPU from the oracle's functions: the q/k/v
     projection, the rotated queries and the cache contents bit for bit, everything behind the attention

@@ -752,6 +752,33 @@ def test_fp8_linear_module_decode_rows_take_the_gemv_and_match_the_prefill_path(
     assert ((small.float() - ref[:16]).norm() / ref[:16].norm()).item() < 0.08
 
 
+def test_fp8_linear_module_large_input_takes_the_one_launch_quantiser_same_bits():
+    """From 16 MiB of activations Fp8Linear quantises them in one launch (its per-stream state is created on first
+    use and carried from call to call): the output must be the bits of the two-launch quantiser + the same GEMM,
+    call after call, and on a second stream with a state of its own."""
+    torch.manual_seed(10)
+    lin = Linear(2048, 256)
+    lin.reset_parameters()
+    f = Fp8Linear.from_linear(lin.to(DEV))
+    xs = [torch.randn(4096, 2048, device=DEV, dtype=torch.bfloat16) * (i + 1) for i in range(2)]  # 16 MiB each
+    assert xs[0].numel() * 2 >= ops.FP8_ONEPASS_MIN_BYTES
+    with torch.inference_mode():
+        want = []
+        for x in xs:
+            xq, sx = ops.quant_tensor_fp8(x)
+            want.append(ops.linear_fp8(xq, sx, f.qweight, f.w_scale, None, out_dtype=torch.bfloat16))
+        for rep in range(3):
+            for x, w in zip(xs, want):
+                assert torch.equal(f(x), w), rep
+        assert len(f._quant_states) == 1
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            got = f(xs[1])
+        side.synchronize()
+        assert torch.equal(got, want[1]) and len(f._quant_states) == 2
+
+
 def test_fp8_linear_module_with_a_bias_and_a_residual(oracle):
     """Fp8Linear keeps the reference's optional bias (linear.py:11) and takes the residual stream like QuantLinear."""
     torch.manual_seed(8)

@@ -513,13 +513,13 @@ __global__ __launch_bounds__(ONEPASS_THREADS) void quant_fp8_onepass_kernel(cons
   __shared__ uint32_t tag_lds;
   const int tid = threadIdx.x, G = gridDim.x;
   const uint4* src = reinterpret_cast<const uint4*>(x);
-  // vector index of (round k, this thread): workgroups interleaved per round, 16 KiB contiguous per workgroup
-  const int64_t round = (int64_t)G * ONEPASS_THREADS;
+  // vector index of (sweep k, this thread): workgroups interleaved per sweep, 16 KiB contiguous per workgroup
+  const int64_t sweep = (int64_t)G * ONEPASS_THREADS;
   const int64_t v0 = (int64_t)blockIdx.x * ONEPASS_THREADS + tid;
   uint4 c[ONEPASS_R];
 #pragma unroll
   for (int k = 0; k < ONEPASS_R; ++k) {
-    const int64_t i = v0 + k * round;
+    const int64_t i = v0 + k * sweep;
     c[k] = make_uint4(0, 0, 0, 0);
     if (i < nvec) c[k] = src[i];
   }
@@ -536,7 +536,7 @@ __global__ __launch_bounds__(ONEPASS_THREADS) void quant_fp8_onepass_kernel(cons
     RowIn<BF16>::unpack(c[k], f);
     amax = fmaxf(amax, vec_amax<EPV>(f));
   }
-  for (int64_t i = v0 + ONEPASS_R * round; i < nvec; i += round) {  // the part that does not fit the registers
+  for (int64_t i = v0 + ONEPASS_R * sweep; i < nvec; i += sweep) {  // the part that does not fit the registers
     float f[EPV];
     RowIn<BF16>::unpack(src[i], f);
     amax = fmaxf(amax, vec_amax<EPV>(f));
@@ -609,10 +609,10 @@ __global__ __launch_bounds__(ONEPASS_THREADS) void quant_fp8_onepass_kernel(cons
   };
 #pragma unroll
   for (int k = 0; k < ONEPASS_R; ++k) {
-    const int64_t i = v0 + k * round;
+    const int64_t i = v0 + k * sweep;
     if (i < nvec) cast_store(c[k], i);
   }
-  for (int64_t i = v0 + ONEPASS_R * round; i < nvec; i += round) cast_store(src[i], i);
+  for (int64_t i = v0 + ONEPASS_R * sweep; i < nvec; i += sweep) cast_store(src[i], i);
 }
 
 }  // namespace aq

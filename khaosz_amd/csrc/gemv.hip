@@ -890,6 +890,253 @@ static int launch_gemv_mfma_swiglu(GemvArgs a, hipStream_t st) {
   return (int)hipGetLastError();
 }
 
+// ---------------------------------------------------------------------------
+// 17..64 tokens on codes: the same weight stream (every weight byte HBM -> registers once, operands assembled by
+// one DPP rotation per dword) with TG groups of 16 tokens multiplied against each weight fragment.  Between the
+// decode batch sizes above and a prefill, the tiled GEMM has too few tiles to occupy the device (32 x 8192 x 2048:
+// 64 tiles of 128 x 128, 12.7 us); this kernel keeps it a bandwidth-bound launch.  Same integer sums, same
+// epilogue: the bits of the tiled GEMM.
+template <int TG, bool RES>
+__global__ __launch_bounds__(GM_MAX_WAVES * 64) void gemv_mfma_tokens_kernel(GemvArgs p) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t xs[];  // [16 TG][K + 16] token codes, 16 spare bytes; later the partial sums
+  constexpr int MTOK = 16 * TG;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int ksplit = p.ksplit, groups = p.groups;
+  const int nthreads = ksplit * groups * 64;
+  const int grp = wave / ksplit, kh = wave % ksplit;
+  const int K = p.K, N = p.N, M = p.M;
+  const int n0 = __builtin_amdgcn_readfirstlane((blockIdx.x * groups + grp) * GM_ROWS);
+  const int pitch = K + 16;
+  const int khalf = K / ksplit;   // a multiple of 128 (checked by the launcher)
+  const int nline = khalf / 128;
+
+  const int tok = lane & 15;
+  const int rbase = n0 + (lane >> 4) * 4;
+  float swv[4], bv[4], sxv[TG];
+  uint32_t rv[TG][4];
+  const EpiOperands epi(p, kh == 0, true, RES);
+
+  const int rows = n0 < N ? ((N - n0) < GM_ROWS ? (N - n0) : GM_ROWS) : 0;
+  const __amdgpu_buffer_rsrc_t Wr = make_rsrc(p.wq + (int64_t)(n0 < N ? n0 : 0) * K, (uint32_t)rows * (uint32_t)K);
+  const uint32_t woff = (uint32_t)(lane & 7) * (uint32_t)K + (uint32_t)(kh * khalf + (lane >> 3) * 16);
+  const uint32_t woff8 = 8u * (uint32_t)K;
+  constexpr int GM_LINES = GM_BATCH / 2;
+  uint4 wa[GM_BATCH], wb[GM_BATCH];
+  auto wload = [&](int line0, uint4 (&dst)[GM_BATCH]) {
+#pragma unroll
+    for (int t = 0; t < GM_LINES; ++t) {
+      const bool ok = (line0 + t) < nline;
+      const uint32_t o = woff + (uint32_t)(line0 + t) * 128u;
+      dst[2 * t] = GV_WLOAD(Wr, ok ? o : OOB_OFFSET);
+      dst[2 * t + 1] = GV_WLOAD(Wr, ok ? o + woff8 : OOB_OFFSET);
+    }
+  };
+
+  // token codes -> LDS: TG rounds of 8 vectors per thread are requested ahead of the weights (MTOK x 2048 codes
+  // with 256 threads), longer rows copy the rest behind them
+  const __amdgpu_buffer_rsrc_t Xr = make_rsrc(p.xq, (uint32_t)M * (uint32_t)K);
+  const int nvec_row = K / 16;
+  const int nvec = MTOK * nvec_row;
+  constexpr int XV = 8;
+  uint4 xvr[TG][XV];
+  auto xload = [&](int v0, uint4 (&xv)[XV]) {
+#pragma unroll
+    for (int i = 0; i < XV; ++i) {
+      const int v = v0 + i * nthreads + tid;
+      xv[i] = buffer_load_16(Xr, v < nvec ? (uint32_t)v * 16u : OOB_OFFSET);
+    }
+  };
+  uint8_t* const spare = xs + MTOK * pitch;
+  auto xstore = [&](int v0, const uint4 (&xv)[XV]) {
+#pragma unroll
+    for (int i = 0; i < XV; ++i) {
+      const int v = v0 + i * nthreads + tid;
+      const int m = v / nvec_row, c = v - m * nvec_row;
+      *reinterpret_cast<uint4*>(v < nvec ? xs + m * pitch + c * 16 : spare) = xv[i];
+    }
+  };
+#pragma unroll
+  for (int r = 0; r < TG; ++r) xload(r * XV * nthreads, xvr[r]);
+  asm volatile("" ::: "memory");  // request order: token codes, epilogue operands, the weight stream
+#pragma unroll
+  for (int g = 0; g < TG; ++g) sxv[g] = epi.load_sx(tok + 16 * g, tok + 16 * g < M);
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int n = rbase + r;
+    swv[r] = epi.load_sw(n, n < N);
+    bv[r] = epi.load_bias(n, n < N);
+#pragma unroll
+    for (int g = 0; g < TG; ++g) rv[g][r] = RES ? epi.load_res(tok + 16 * g, n, tok + 16 * g < M && n < N, (int)p.ldr) : 0u;
+  }
+  asm volatile("" ::: "memory");
+  wload(0, wa);
+  wload(GM_LINES, wb);
+  asm volatile("" ::: "memory");
+#pragma unroll
+  for (int r = 0; r < TG; ++r) xstore(r * XV * nthreads, xvr[r]);
+  for (int v0 = TG * XV * nthreads; v0 < nvec; v0 += XV * nthreads) {
+    xload(v0, xvr[0]);
+    xstore(v0, xvr[0]);
+  }
+  __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();  // no fence: the weight loads stay in flight
+  asm volatile("" ::: "memory");
+
+  v4i accs[TG][2];
+#pragma unroll
+  for (int g = 0; g < TG; ++g) accs[g][0] = accs[g][1] = v4i{0, 0, 0, 0};
+  const uint8_t* xl = xs + tok * pitch + kh * khalf + (lane >> 4) * 32;
+  auto consume = [&](int line0, const uint4 (&wc)[GM_BATCH]) {
+#pragma unroll
+    for (int t = 0; t < GM_LINES; ++t) {
+      const int ln = (line0 + t) < nline ? (line0 + t) : 0;  // lines past the end multiply zero weights
+      v4i x0[TG], x1[TG];
+#pragma unroll
+      for (int g = 0; g < TG; ++g) {
+        x0[g] = *reinterpret_cast<const v4i*>(xl + g * 16 * pitch + ln * 128);
+        x1[g] = *reinterpret_cast<const v4i*>(xl + g * 16 * pitch + ln * 128 + 16);
+      }
+      const uint4 lo = wc[2 * t], hi = wc[2 * t + 1];
+      constexpr int ROR8 = 0x128;  // DPP row_ror:8 (see gemv_mfma_kernel)
+      const v4i w0 = {__builtin_amdgcn_update_dpp((int)lo.x, (int)hi.x, ROR8, 0xf, 0xc, false),
+                      __builtin_amdgcn_update_dpp((int)lo.y, (int)hi.y, ROR8, 0xf, 0xc, false),
+                      __builtin_amdgcn_update_dpp((int)lo.z, (int)hi.z, ROR8, 0xf, 0xc, false),
+                      __builtin_amdgcn_update_dpp((int)lo.w, (int)hi.w, ROR8, 0xf, 0xc, false)};
+      const v4i w1 = {__builtin_amdgcn_update_dpp((int)hi.x, (int)lo.x, ROR8, 0xf, 0x3, false),
+                      __builtin_amdgcn_update_dpp((int)hi.y, (int)lo.y, ROR8, 0xf, 0x3, false),
+                      __builtin_amdgcn_update_dpp((int)hi.z, (int)lo.z, ROR8, 0xf, 0x3, false),
+                      __builtin_amdgcn_update_dpp((int)hi.w, (int)lo.w, ROR8, 0xf, 0x3, false)};
+#pragma unroll
+      for (int g = 0; g < TG; ++g) {
+        accs[g][0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w0, x0[g], accs[g][0], 0, 0, 0);
+        accs[g][1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w1, x1[g], accs[g][1], 0, 0, 0);
+      }
+    }
+  };
+  for (int l0 = 0; l0 < nline; l0 += 2 * GM_LINES) {
+    consume(l0, wa);
+    if (l0 + 2 * GM_LINES < nline) wload(l0 + 2 * GM_LINES, wa);
+    if (l0 + GM_LINES < nline) consume(l0 + GM_LINES, wb);
+    if (l0 + 3 * GM_LINES < nline) wload(l0 + 3 * GM_LINES, wb);
+  }
+
+  // sum the K parts through LDS (exact int32)
+  __syncthreads();  // everyone is done reading the token codes: the buffer is reused
+  int* part = reinterpret_cast<int*>(xs) + (grp * (ksplit - 1)) * TG * 256;
+  v4i acc[TG];
+#pragma unroll
+  for (int g = 0; g < TG; ++g) acc[g] = accs[g][0] + accs[g][1];
+  if (kh != 0) {
+#pragma unroll
+    for (int g = 0; g < TG; ++g) *reinterpret_cast<v4i*>(part + ((kh - 1) * TG + g) * 256 + lane * 4) = acc[g];
+  }
+  __syncthreads();
+  if (kh != 0) return;
+  for (int k = 0; k < ksplit - 1; ++k)
+#pragma unroll
+    for (int g = 0; g < TG; ++g) acc[g] += *reinterpret_cast<const v4i*>(part + (k * TG + g) * 256 + lane * 4);
+
+#pragma unroll
+  for (int g = 0; g < TG; ++g) {
+    const int tk = tok + 16 * g;
+    if (tk >= M) continue;
+    float y[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      y[r] = __fmul_rn(__fmul_rn((float)acc[g][r], sxv[g]), swv[r]);
+      if (p.bias) y[r] = __fadd_rn(y[r], bv[r]);
+      if constexpr (RES) y[r] = p.y_dtype == AQ_BF16 ? add_residual_bf16(y[r], rv[g][r]) : __fadd_rn(y[r], __uint_as_float(rv[g][r]));
+    }
+    const int64_t o = (int64_t)tk * N + rbase;
+    if (p.y_dtype == AQ_BF16) {
+      uint16_t* dst = reinterpret_cast<uint16_t*>(p.y) + o;
+      if ((N & 3) == 0 && rbase + 3 < N) {
+        uint2 pk;
+        pk.x = pack_bf16x2(y[0], y[1]);
+        pk.y = pack_bf16x2(y[2], y[3]);
+        *reinterpret_cast<uint2*>(dst) = pk;
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (rbase + r < N) dst[r] = (uint16_t)f32_to_bf16_bits(y[r]);
+      }
+    } else {
+      float* dst = reinterpret_cast<float*>(p.y) + o;
+      if ((N & 3) == 0 && rbase + 3 < N) {
+        *reinterpret_cast<float4*>(dst) = make_float4(y[0], y[1], y[2], y[3]);
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (rbase + r < N) dst[r] = y[r];
+      }
+    }
+  }
+}
+
+// Shapes the token-group kernel takes: 17..64 rows, K in whole 256-byte steps, the padded codes within a compute
+// unit's LDS.
+bool gemv_tokens_ok(int64_t M, int64_t N, int64_t K) {
+  if (M <= 16 || M > 64 || N <= 0 || (K % 256) != 0) return false;
+  const int64_t tg = (M + 15) / 16;
+  return 16 * tg * (K + 16) + 16 <= GV_MAX_LDS;
+}
+
+// (not static: the tiled GEMM's entry points in gemm_mfma.hip hand these shapes over)
+int launch_gemv_tokens(GemvArgs a, hipStream_t st) {
+  a.ksplit = 2;
+  a.groups = 2;
+  const int cus = device_cus();
+  if ((a.N + 31) / 32 < cus) {
+    a.groups = 1;
+    while (a.ksplit < GM_MAX_WAVES && (a.N + 15) / 16 * (a.ksplit / 2) < cus && a.K % (256 * a.ksplit) == 0 &&
+           a.K / (2 * a.ksplit) >= 512)
+      a.ksplit *= 2;
+  }
+  // more 32-row blocks than compute units: 64 rows per workgroup, so that a second round of workgroups does not
+  // copy the token codes (up to 128 KiB each) all over again
+  else if ((a.N + 31) / 32 > cus) {
+    a.groups = 4;
+  }
+  const int tg = (a.M + 15) / 16;
+  const unsigned grid = (unsigned)((a.N + GM_ROWS * a.groups - 1) / (GM_ROWS * a.groups));
+  const size_t lds = (size_t)16 * tg * (a.K + 16) + 16;
+  const bool res = a.res != nullptr;
+  using kern_t = void (*)(GemvArgs);
+  static const kern_t table[3][2] = {{gemv_mfma_tokens_kernel<2, false>, gemv_mfma_tokens_kernel<2, true>},
+                                     {gemv_mfma_tokens_kernel<3, false>, gemv_mfma_tokens_kernel<3, true>},
+                                     {gemv_mfma_tokens_kernel<4, false>, gemv_mfma_tokens_kernel<4, true>}};
+  const kern_t fn = table[tg - 2][res];
+  if (lds > 64 * 1024) {
+    static LdsOptIn opted[6];
+    const int e = opted[(tg - 2) * 2 + res].ensure(reinterpret_cast<const void*>(fn));
+    if (e) return e;
+  }
+  hipLaunchKernelGGL(fn, dim3(grid), dim3(a.ksplit * a.groups * 64), lds, st, a);
+  return (int)hipGetLastError();
+}
+
+int gemv_tokens_launch(const int8_t* xq, const float* sx, const int8_t* wq, const float* sw, const void* bias,
+                       int bias_dtype, const void* residual, void* y, int y_dtype, int64_t M, int64_t N, int64_t K,
+                       hipStream_t st) {
+  GemvArgs a{};
+  a.xq = xq;
+  a.sx = sx;
+  a.wq = wq;
+  a.sw = sw;
+  a.bias = bias;
+  a.res = residual;
+  a.ldr = N;
+  a.y = y;
+  a.M = (int)M;
+  a.N = (int)N;
+  a.K = (int)K;
+  a.bias_dtype = bias_dtype;
+  a.y_dtype = y_dtype;
+  return launch_gemv_tokens(a, st);
+}
+
 static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 }  // namespace aq

@@ -460,6 +460,37 @@ def test_up_gate_gemv_with_the_activation_refuses_what_it_does_not_serve():
                                     torch.ones(2048, device=DEV))
 
 
+@pytest.mark.parametrize("M", [17, 31, 32, 33, 48, 50, 64])
+@pytest.mark.parametrize("N,K", [(8192, 2048), (200, 256), (77, 1536), (2048, 2304), (3072, 4096), (130, 9984)])
+def test_a_few_dozen_rows_take_the_weight_streaming_kernel_same_bits_as_the_oracle(oracle, M, N, K):
+    """17..64 rows are too few for the tiled GEMM to fill the device: the Linear on codes hands them to the
+    weight-streaming matrix-core kernel with 2..4 groups of 16 tokens (where the padded codes fit a compute
+    unit's LDS; (130, 9984) at 33+ rows does not and stays on the tiles).  int32 sums and the frozen epilogue:
+    bit for bit against the oracle, bf16 and fp32 outputs, with bias and residual, odd N."""
+    _say("linear, few dozen rows", M, N, K)
+    x = make_x(M, K, 50 + M).to(torch.bfloat16)
+    w = make_x(N, K, 51) * 0.02
+    wq, sw = oracle.c_quant_rowwise_i8(w.numpy())
+    xq, sx = oracle.c_quant_rowwise_i8(bf16_bits(x), bf16_bits=True)
+    g = torch.Generator().manual_seed(52)
+    b = torch.randn(N, generator=g) * 0.01
+    wqd, swd = torch.from_numpy(wq).to(DEV), torch.from_numpy(sw).to(DEV)
+    xqd, sxd = torch.from_numpy(xq).to(DEV), torch.from_numpy(sx).to(DEV)
+    acc = oracle.c_gemm_i8_i32(xq, wq)
+    for bias in (None, b):
+        want = oracle.c_dequant_epilogue(acc, sx, sw, None if bias is None else bias.numpy(), bf16_out=True)
+        y = ops.linear_w8a8(xqd, sxd, wqd, swd, None if bias is None else bias.to(DEV), out_dtype=torch.bfloat16)
+        assert np.array_equal(bf16_bits(y), want)
+        r = torch.randn(M, N, generator=g).to(torch.bfloat16).to(DEV)
+        yr = ops.linear_w8a8(xqd, sxd, wqd, swd, None if bias is None else bias.to(DEV), out_dtype=torch.bfloat16, residual=r)
+        assert torch.equal(yr, y + r)
+    wantf = oracle.c_dequant_epilogue(acc, sx, sw, b.numpy(), bf16_out=False)
+    yf = ops.linear_w8a8(xqd, sxd, wqd, swd, b.to(DEV), out_dtype=torch.float32)
+    assert np.array_equal(to_np(yf).view(np.uint32), wantf.view(np.uint32))
+    rf = torch.randn(M, N, generator=g).to(DEV)
+    assert torch.equal(ops.linear_w8a8(xqd, sxd, wqd, swd, b.to(DEV), out_dtype=torch.float32, residual=rf), yf + rf)
+
+
 @pytest.mark.parametrize("M,K", [(12, 11008), (16, 14336), (7, 22016)])
 def test_decode_rows_too_long_for_the_gemv_take_the_tiled_gemm(oracle, M, K):
     """Activation codes of 9..16 tokens fit a compute unit's LDS up to K = 10 096 (5..8 tokens: 20 208).

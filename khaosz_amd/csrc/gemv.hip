@@ -1075,16 +1075,228 @@ __global__ __launch_bounds__(GM_MAX_WAVES * 64) void gemv_mfma_tokens_kernel(Gem
   }
 }
 
+// The same for 17..32 tokens whose rows are too long for their codes to sit in LDS all at once (an MLP's down
+// projection): K is walked in chunks of 1024 bytes per wavefront (KS wavefronts per row group: 2048- or 4096-byte
+// chunks per workgroup), the token codes of one chunk at a time in LDS.  A chunk's codes are requested into registers
+// while the chunk before is multiplied and stored between two barriers; the weight stream runs through the chunk
+// boundaries untouched (two register batches, each reloaded as soon as it has been consumed).  Two row groups per
+// workgroup; rows must be whole 128-byte lines (K % 128 == 0).
+template <int KS, bool RES>
+__global__ __launch_bounds__(KS * 2 * 64) void gemv_mfma_tokens_longk_kernel(GemvArgs p) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t xs[];  // [32][KC + 16] codes of one chunk, 16 spare bytes; later the partial sums
+  constexpr int TG = 2, MTOK = 32, GRP = 2, NTHREADS = KS * GRP * 64;
+  constexpr int KC = 1024 * KS;            // K bytes of a chunk
+  constexpr int PITCH = KC + 16;
+  constexpr int XV = MTOK * (KC / 16) / NTHREADS;  // 16-byte vectors of a chunk's codes per thread: 16
+  static_assert(XV == 16, "a chunk's codes are 16 vectors per thread");
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int grp = wave / KS, kh = wave % KS;
+  const int K = p.K, N = p.N, M = p.M;
+  const int n0 = __builtin_amdgcn_readfirstlane((blockIdx.x * GRP + grp) * GM_ROWS);
+  const int nchunk = (K + KC - 1) / KC;
+
+  const int tok = lane & 15;
+  const int rbase = n0 + (lane >> 4) * 4;
+  float swv[4], bv[4], sxv[TG];
+  uint32_t rv[TG][4];
+  const EpiOperands epi(p, kh == 0, true, RES);
+
+  const int rows = n0 < N ? ((N - n0) < GM_ROWS ? (N - n0) : GM_ROWS) : 0;
+  const __amdgpu_buffer_rsrc_t Wr = make_rsrc(p.wq + (int64_t)(n0 < N ? n0 : 0) * K, (uint32_t)rows * (uint32_t)K);
+  const uint32_t woff = (uint32_t)(lane & 7) * (uint32_t)K + (uint32_t)((lane >> 3) * 16);
+  const uint32_t woff8 = 8u * (uint32_t)K;
+  constexpr int GM_LINES = GM_BATCH / 2;
+  uint4 wa[GM_BATCH], wb[GM_BATCH];
+  // lines line0 .. line0+3 of this wavefront's 1024 bytes of chunk c (columns past K read zeros: an offset there
+  // would alias the next row, so it is pushed outside the descriptor)
+  auto wload = [&](int c, int line0, uint4 (&dst)[GM_BATCH]) {
+#pragma unroll
+    for (int t = 0; t < GM_LINES; ++t) {
+      const int col = c * KC + kh * 1024 + (line0 + t) * 128;
+      const bool ok = col < K;
+      const uint32_t o = woff + (uint32_t)col;
+      dst[2 * t] = GV_WLOAD(Wr, ok ? o : OOB_OFFSET);
+      dst[2 * t + 1] = GV_WLOAD(Wr, ok ? o + woff8 : OOB_OFFSET);
+    }
+  };
+  const __amdgpu_buffer_rsrc_t Xr = make_rsrc(p.xq, (uint32_t)M * (uint32_t)K);
+  uint4 xvr[XV];
+  auto xload = [&](int c) {
+#pragma unroll
+    for (int i = 0; i < XV; ++i) {
+      const int v = i * NTHREADS + tid;
+      const int m = v / (KC / 16), cc = v - m * (KC / 16);
+      const int col = c * KC + cc * 16;
+      xvr[i] = buffer_load_16(Xr, (m < M && col < K) ? (uint32_t)m * (uint32_t)K + (uint32_t)col : OOB_OFFSET);
+    }
+  };
+  auto xstore = [&]() {
+#pragma unroll
+    for (int i = 0; i < XV; ++i) {
+      const int v = i * NTHREADS + tid;
+      const int m = v / (KC / 16), cc = v - m * (KC / 16);
+      *reinterpret_cast<uint4*>(xs + m * PITCH + cc * 16) = xvr[i];
+    }
+  };
+
+  xload(0);
+  asm volatile("" ::: "memory");  // request order: token codes, epilogue operands, the weight stream
+#pragma unroll
+  for (int g = 0; g < TG; ++g) sxv[g] = epi.load_sx(tok + 16 * g, tok + 16 * g < M);
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int n = rbase + r;
+    swv[r] = epi.load_sw(n, n < N);
+    bv[r] = epi.load_bias(n, n < N);
+#pragma unroll
+    for (int g = 0; g < TG; ++g) rv[g][r] = RES ? epi.load_res(tok + 16 * g, n, tok + 16 * g < M && n < N, (int)p.ldr) : 0u;
+  }
+  asm volatile("" ::: "memory");
+  wload(0, 0, wa);
+  wload(0, GM_LINES, wb);
+  asm volatile("" ::: "memory");
+
+  v4i accs[TG][2];
+#pragma unroll
+  for (int g = 0; g < TG; ++g) accs[g][0] = accs[g][1] = v4i{0, 0, 0, 0};
+  const uint8_t* xl = xs + tok * PITCH + kh * 1024 + (lane >> 4) * 32;
+  auto consume = [&](int line0, const uint4 (&wc)[GM_BATCH]) {
+#pragma unroll
+    for (int t = 0; t < GM_LINES; ++t) {
+      v4i x0[TG], x1[TG];
+#pragma unroll
+      for (int g = 0; g < TG; ++g) {
+        x0[g] = *reinterpret_cast<const v4i*>(xl + g * 16 * PITCH + (line0 + t) * 128);
+        x1[g] = *reinterpret_cast<const v4i*>(xl + g * 16 * PITCH + (line0 + t) * 128 + 16);
+      }
+      const uint4 lo = wc[2 * t], hi = wc[2 * t + 1];
+      constexpr int ROR8 = 0x128;  // DPP row_ror:8 (see gemv_mfma_kernel)
+      const v4i w0 = {__builtin_amdgcn_update_dpp((int)lo.x, (int)hi.x, ROR8, 0xf, 0xc, false),
+                      __builtin_amdgcn_update_dpp((int)lo.y, (int)hi.y, ROR8, 0xf, 0xc, false),
+                      __builtin_amdgcn_update_dpp((int)lo.z, (int)hi.z, ROR8, 0xf, 0xc, false),
+                      __builtin_amdgcn_update_dpp((int)lo.w, (int)hi.w, ROR8, 0xf, 0xc, false)};
+      const v4i w1 = {__builtin_amdgcn_update_dpp((int)hi.x, (int)lo.x, ROR8, 0xf, 0x3, false),
+                      __builtin_amdgcn_update_dpp((int)hi.y, (int)lo.y, ROR8, 0xf, 0x3, false),
+                      __builtin_amdgcn_update_dpp((int)hi.z, (int)lo.z, ROR8, 0xf, 0x3, false),
+                      __builtin_amdgcn_update_dpp((int)hi.w, (int)lo.w, ROR8, 0xf, 0x3, false)};
+#pragma unroll
+      for (int g = 0; g < TG; ++g) {
+        accs[g][0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w0, x0[g], accs[g][0], 0, 0, 0);
+        accs[g][1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w1, x1[g], accs[g][1], 0, 0, 0);
+      }
+    }
+  };
+  // barriers without a memory fence (LDS traffic only has to be complete): the weight loads stay in flight
+  auto lds_barrier = [&]() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+  };
+  for (int c = 0; c < nchunk; ++c) {
+    if (c > 0) lds_barrier();  // every wavefront is done with the codes of the chunk before
+    xstore();                  // waits for this chunk's codes only: they are older than the weight loads in flight
+    lds_barrier();
+    if (c + 1 < nchunk) xload(c + 1);
+    consume(0, wa);
+    if (c + 1 < nchunk) wload(c + 1, 0, wa);
+    consume(GM_LINES, wb);
+    if (c + 1 < nchunk) wload(c + 1, GM_LINES, wb);
+  }
+
+  // sum the K parts through LDS (exact int32)
+  __syncthreads();
+  int* part = reinterpret_cast<int*>(xs) + (grp * (KS - 1)) * TG * 256;
+  v4i acc[TG];
+#pragma unroll
+  for (int g = 0; g < TG; ++g) acc[g] = accs[g][0] + accs[g][1];
+  if (kh != 0) {
+#pragma unroll
+    for (int g = 0; g < TG; ++g) *reinterpret_cast<v4i*>(part + ((kh - 1) * TG + g) * 256 + lane * 4) = acc[g];
+  }
+  __syncthreads();
+  if (kh != 0) return;
+  for (int k = 0; k < KS - 1; ++k)
+#pragma unroll
+    for (int g = 0; g < TG; ++g) acc[g] += *reinterpret_cast<const v4i*>(part + (k * TG + g) * 256 + lane * 4);
+
+#pragma unroll
+  for (int g = 0; g < TG; ++g) {
+    const int tk = tok + 16 * g;
+    if (tk >= M) continue;
+    float y[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      y[r] = __fmul_rn(__fmul_rn((float)acc[g][r], sxv[g]), swv[r]);
+      if (p.bias) y[r] = __fadd_rn(y[r], bv[r]);
+      if constexpr (RES) y[r] = p.y_dtype == AQ_BF16 ? add_residual_bf16(y[r], rv[g][r]) : __fadd_rn(y[r], __uint_as_float(rv[g][r]));
+    }
+    const int64_t o = (int64_t)tk * N + rbase;
+    if (p.y_dtype == AQ_BF16) {
+      uint16_t* dst = reinterpret_cast<uint16_t*>(p.y) + o;
+      if ((N & 3) == 0 && rbase + 3 < N) {
+        uint2 pk;
+        pk.x = pack_bf16x2(y[0], y[1]);
+        pk.y = pack_bf16x2(y[2], y[3]);
+        *reinterpret_cast<uint2*>(dst) = pk;
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (rbase + r < N) dst[r] = (uint16_t)f32_to_bf16_bits(y[r]);
+      }
+    } else {
+      float* dst = reinterpret_cast<float*>(p.y) + o;
+      if ((N & 3) == 0 && rbase + 3 < N) {
+        *reinterpret_cast<float4*>(dst) = make_float4(y[0], y[1], y[2], y[3]);
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (rbase + r < N) dst[r] = y[r];
+      }
+    }
+  }
+}
+
 // Shapes the token-group kernel takes: 17..64 rows, K in whole 256-byte steps, the padded codes within a compute
 // unit's LDS.
+static bool gemv_tokens_fit(int64_t M, int64_t K) {
+  return (K % 256) == 0 && 16 * ((M + 15) / 16) * (K + 16) + 16 <= GV_MAX_LDS;
+}
+// ... or, up to 32 rows of whole 128-byte lines, any length (the chunked kernel above)
+// -- which also takes the decode batch sizes whose rows are too long for the GEMV kernels' own LDS budget (9..16
+// rows beyond 10 096 bytes, 5..8 beyond 20 208, ...), where the tiles were the only path (12 x 4096 x 11008: 41 us
+// against 19 us).
 bool gemv_tokens_ok(int64_t M, int64_t N, int64_t K) {
-  if (M <= 16 || M > 64 || N <= 0 || (K % 256) != 0) return false;
-  const int64_t tg = (M + 15) / 16;
-  return 16 * tg * (K + 16) + 16 <= GV_MAX_LDS;
+  if (M < 1 || M > 64 || N <= 0) return false;
+  const bool chunked = (K % 128) == 0 && K <= (1 << 22);
+  if (M <= 16) {
+    const int64_t mt = M <= 1 ? 1 : M <= 2 ? 2 : M <= 4 ? 4 : M <= 8 ? 8 : 16;
+    return chunked && mt * K + 64 + 2048 > GV_MAX_LDS;  // the GEMV kernels' own limit (gemv_check)
+  }
+  return gemv_tokens_fit(M, K) || (M <= 32 && chunked);
 }
 
 // (not static: the tiled GEMM's entry points in gemm_mfma.hip hand these shapes over)
+template <int KS>
+static int launch_gemv_tokens_longk(const GemvArgs& a, hipStream_t st) {
+  const unsigned grid = (unsigned)((a.N + 2 * GM_ROWS - 1) / (2 * GM_ROWS));
+  const size_t lds = (size_t)32 * (1024 * KS + 16) + 16;
+  using kern_t = void (*)(GemvArgs);
+  const kern_t fn = a.res ? gemv_mfma_tokens_longk_kernel<KS, true> : gemv_mfma_tokens_longk_kernel<KS, false>;
+  static LdsOptIn opted[2];
+  const int e = opted[a.res ? 1 : 0].ensure(reinterpret_cast<const void*>(fn));
+  if (e) return e;
+  hipLaunchKernelGGL(fn, dim3(grid), dim3(KS * 2 * 64), lds, st, a);
+  return (int)hipGetLastError();
+}
+
 int launch_gemv_tokens(GemvArgs a, hipStream_t st) {
+  if (a.M <= 16 || !gemv_tokens_fit(a.M, a.K)) {
+    // 4096-byte chunks over 8 wavefronts while that still gives every compute unit a workgroup's worth of loads;
+    // 2048-byte chunks over 4 wavefronts for wide matrices
+    return (a.N + 31) / 32 > device_cus() ? launch_gemv_tokens_longk<2>(a, st) : launch_gemv_tokens_longk<4>(a, st);
+  }
   a.ksplit = 2;
   a.groups = 2;
   const int cus = device_cus();

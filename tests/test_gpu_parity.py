@@ -461,12 +461,14 @@ def test_up_gate_gemv_with_the_activation_refuses_what_it_does_not_serve():
 
 
 @pytest.mark.parametrize("M", [17, 31, 32, 33, 48, 50, 64])
-@pytest.mark.parametrize("N,K", [(8192, 2048), (200, 256), (77, 1536), (2048, 2304), (3072, 4096), (130, 9984)])
+@pytest.mark.parametrize("N,K", [(8192, 2048), (200, 256), (77, 1536), (2048, 2304), (3072, 4096), (130, 9984),
+                                 (2048, 5632), (8200, 6912), (77, 11008), (40, 128), (12000, 4224)])
 def test_a_few_dozen_rows_take_the_weight_streaming_kernel_same_bits_as_the_oracle(oracle, M, N, K):
     """17..64 rows are too few for the tiled GEMM to fill the device: the Linear on codes hands them to the
-    weight-streaming matrix-core kernel with 2..4 groups of 16 tokens (where the padded codes fit a compute
-    unit's LDS; (130, 9984) at 33+ rows does not and stays on the tiles).  int32 sums and the frozen epilogue:
-    bit for bit against the oracle, bf16 and fp32 outputs, with bias and residual, odd N."""
+    weight-streaming matrix-core kernel with 2..4 groups of 16 tokens where the padded codes fit a compute
+    unit's LDS, and up to 32 rows of any length to its variant that walks K in chunks (ragged last chunks, both
+    chunk sizes); what neither takes ((130, 9984) at 33+ rows) stays on the tiles.  int32 sums and the frozen
+    epilogue: bit for bit against the oracle, bf16 and fp32 outputs, with bias and residual, odd N."""
     _say("linear, few dozen rows", M, N, K)
     x = make_x(M, K, 50 + M).to(torch.bfloat16)
     w = make_x(N, K, 51) * 0.02
@@ -491,12 +493,13 @@ def test_a_few_dozen_rows_take_the_weight_streaming_kernel_same_bits_as_the_orac
     assert torch.equal(ops.linear_w8a8(xqd, sxd, wqd, swd, b.to(DEV), out_dtype=torch.float32, residual=rf), yf + rf)
 
 
-@pytest.mark.parametrize("M,K", [(12, 11008), (16, 14336), (7, 22016)])
-def test_decode_rows_too_long_for_the_gemv_take_the_tiled_gemm(oracle, M, K):
+@pytest.mark.parametrize("M,K", [(12, 11008), (16, 14336), (7, 22016), (9, 10160)])
+def test_decode_rows_too_long_for_the_gemv_take_the_kernel_that_walks_k_in_chunks(oracle, M, K):
     """Activation codes of 9..16 tokens fit a compute unit's LDS up to K = 10 096 (5..8 tokens: 20 208).
     Longer rows (FFN down projections of 11 008 or 14 336) must still work at decode batch sizes:
-    the decode entry points hand them to the MFMA GEMM.  Same bits as the oracle, with bias and residual,
-    through the drop-in module as well."""
+    the decode entry points hand them on to the Linear on codes, whose weight-streaming kernel walks such
+    rows in chunks (rows that are not whole 128-byte lines would take the tiles).  Same bits as the oracle,
+    with bias and residual, through the drop-in module as well."""
     N = 200
     _say("gemv long K", M, N, K)
     x = make_x(M, K, 41 + M).to(torch.bfloat16)

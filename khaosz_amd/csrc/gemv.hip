@@ -1075,20 +1075,20 @@ __global__ __launch_bounds__(GM_MAX_WAVES * 64) void gemv_mfma_tokens_kernel(Gem
   }
 }
 
-// The same for 17..32 tokens whose rows are too long for their codes to sit in LDS all at once (an MLP's down
-// projection): K is walked in chunks of 1024 bytes per wavefront (KS wavefronts per row group: 2048- or 4096-byte
-// chunks per workgroup), the token codes of one chunk at a time in LDS.  A chunk's codes are requested into registers
+// The same for tokens whose rows are too long for their codes to sit in LDS all at once (an MLP's down
+// projection): K is walked in chunks of 1024 bytes per wavefront (KS wavefronts per row group: 2048- or, for up to
+// 32 tokens, 4096-byte chunks per workgroup), the token codes of one chunk at a time in LDS.  A chunk's codes are requested into registers
 // while the chunk before is multiplied and stored between two barriers; the weight stream runs through the chunk
 // boundaries untouched (two register batches, each reloaded as soon as it has been consumed).  Two row groups per
 // workgroup; rows must be whole 128-byte lines (K % 128 == 0).
-template <int KS, bool RES>
+template <int TG, int KS, bool RES>
 __global__ __launch_bounds__(KS * 2 * 64) void gemv_mfma_tokens_longk_kernel(GemvArgs p) {
-  extern __shared__ __attribute__((aligned(16))) uint8_t xs[];  // [32][KC + 16] codes of one chunk, 16 spare bytes; later the partial sums
-  constexpr int TG = 2, MTOK = 32, GRP = 2, NTHREADS = KS * GRP * 64;
+  extern __shared__ __attribute__((aligned(16))) uint8_t xs[];  // [16 TG][KC + 16] codes of one chunk; later the partial sums
+  constexpr int MTOK = 16 * TG, GRP = 2, NTHREADS = KS * GRP * 64;
   constexpr int KC = 1024 * KS;            // K bytes of a chunk
   constexpr int PITCH = KC + 16;
-  constexpr int XV = MTOK * (KC / 16) / NTHREADS;  // 16-byte vectors of a chunk's codes per thread: 16
-  static_assert(XV == 16, "a chunk's codes are 16 vectors per thread");
+  constexpr int XV = MTOK * (KC / 16) / NTHREADS;  // 16-byte vectors of a chunk's codes per thread: 8 per token group
+  static_assert(XV == 8 * TG && MTOK * PITCH <= 150 * 1024, "a chunk's codes: 8 vectors per thread and token group, within LDS");
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int grp = wave / KS, kh = wave % KS;
@@ -1274,16 +1274,16 @@ bool gemv_tokens_ok(int64_t M, int64_t N, int64_t K) {
     const int64_t mt = M <= 1 ? 1 : M <= 2 ? 2 : M <= 4 ? 4 : M <= 8 ? 8 : 16;
     return chunked && mt * K + 64 + 2048 > GV_MAX_LDS;  // the GEMV kernels' own limit (gemv_check)
   }
-  return gemv_tokens_fit(M, K) || (M <= 32 && chunked);
+  return gemv_tokens_fit(M, K) || chunked;
 }
 
 // (not static: the tiled GEMM's entry points in gemm_mfma.hip hand these shapes over)
-template <int KS>
+template <int TG, int KS>
 static int launch_gemv_tokens_longk(const GemvArgs& a, hipStream_t st) {
   const unsigned grid = (unsigned)((a.N + 2 * GM_ROWS - 1) / (2 * GM_ROWS));
-  const size_t lds = (size_t)32 * (1024 * KS + 16) + 16;
+  const size_t lds = (size_t)16 * TG * (1024 * KS + 16) + 16;
   using kern_t = void (*)(GemvArgs);
-  const kern_t fn = a.res ? gemv_mfma_tokens_longk_kernel<KS, true> : gemv_mfma_tokens_longk_kernel<KS, false>;
+  const kern_t fn = a.res ? gemv_mfma_tokens_longk_kernel<TG, KS, true> : gemv_mfma_tokens_longk_kernel<TG, KS, false>;
   static LdsOptIn opted[2];
   const int e = opted[a.res ? 1 : 0].ensure(reinterpret_cast<const void*>(fn));
   if (e) return e;
@@ -1293,9 +1293,11 @@ static int launch_gemv_tokens_longk(const GemvArgs& a, hipStream_t st) {
 
 int launch_gemv_tokens(GemvArgs a, hipStream_t st) {
   if (a.M <= 16 || !gemv_tokens_fit(a.M, a.K)) {
-    // 4096-byte chunks over 8 wavefronts while that still gives every compute unit a workgroup's worth of loads;
-    // 2048-byte chunks over 4 wavefronts for wide matrices
-    return (a.N + 31) / 32 > device_cus() ? launch_gemv_tokens_longk<2>(a, st) : launch_gemv_tokens_longk<4>(a, st);
+    // up to 32 tokens: 4096-byte chunks over 8 wavefronts while that still gives every compute unit a workgroup's
+    // worth of loads, 2048-byte chunks over 4 wavefronts for wide matrices; more tokens: 2048-byte chunks (LDS)
+    if (a.M > 48) return launch_gemv_tokens_longk<4, 2>(a, st);
+    if (a.M > 32) return launch_gemv_tokens_longk<3, 2>(a, st);
+    return (a.N + 31) / 32 > device_cus() ? launch_gemv_tokens_longk<2, 2>(a, st) : launch_gemv_tokens_longk<2, 4>(a, st);
   }
   a.ksplit = 2;
   a.groups = 2;

@@ -466,8 +466,8 @@ def test_up_gate_gemv_with_the_activation_refuses_what_it_does_not_serve():
 def test_a_few_dozen_rows_take_the_weight_streaming_kernel_same_bits_as_the_oracle(oracle, M, N, K):
     """17..64 rows are too few for the tiled GEMM to fill the device: the Linear on codes hands them to the
     weight-streaming matrix-core kernel with 2..4 groups of 16 tokens where the padded codes fit a compute
-    unit's LDS, and up to 32 rows of any length to its variant that walks K in chunks (ragged last chunks, both
-    chunk sizes); what neither takes ((130, 9984) at 33+ rows) stays on the tiles.  int32 sums and the frozen
+    unit's LDS, and rows of any length (whole 128-byte lines) to its variant that walks K in chunks (ragged last
+    chunks, both chunk sizes, 2..4 token groups).  int32 sums and the frozen
     epilogue: bit for bit against the oracle, bf16 and fp32 outputs, with bias and residual, odd N."""
     _say("linear, few dozen rows", M, N, K)
     x = make_x(M, K, 50 + M).to(torch.bfloat16)

@@ -64,7 +64,7 @@ def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=1000)
     ap.add_argument("--workload", default="decode", choices=["decode", "prefill", "fp8", "block", "model"])
     ap.add_argument("--m", type=int, default=16, help="decode rows (1..16)")
     ap.add_argument("--mnk", default=None, help="prefill workload only: M,N,K of the int8 Linear instead of configuration 3's "
@@ -75,11 +75,15 @@ def parse():
 
 
 def graph_time_ms(torch, step, steps, warmup, dist=None):
-    """Warm up eagerly, capture `steps` calls of step(i) into one HIP graph, replay it once
-    untimed, then time one replay with events on the launching stream.  Returns ms per step.
+    """Warm up, capture `steps` calls of step(i) into one HIP graph, then time one replay with events on
+    the launching stream.  Returns ms per step.  The `warmup` untimed steps run the way the timed ones do: a
+    few eager calls first (allocations, lazy initialisation), then whole untimed replays of the graph until at
+    least `warmup` steps have gone by (at least one replay) -- the device reaches its steady clocks only
+    under the replayed load, and a replay timed straight after one warm-up replay reads 2-10 % slower than
+    the ones that follow.
     dist: a list that receives [p10, p50, p90] of the ms per step of 11 further replays, each timed
     on its own (the spread between replays; not part of the timed region)."""
-    for i in range(warmup):
+    for i in range(min(warmup, 20)):
         step(i)
     torch.cuda.synchronize()
     side = torch.cuda.Stream()
@@ -91,7 +95,8 @@ def graph_time_ms(torch, step, steps, warmup, dist=None):
                 step(i)
     torch.cuda.current_stream().wait_stream(side)
     torch.cuda.synchronize()
-    g.replay()
+    for _ in range(max(1, -(-warmup // steps))):
+        g.replay()
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
@@ -249,6 +254,36 @@ def bench_prefill(torch, ops, args, dev):
                                     "algorithmic_bytes": qbytes + 2 * K},
         "shape": (M, N, K),
     }
+
+
+def bench_few_dozen_rows(torch, ops, args, dev):
+    """The same Linear (configuration 2's weight, N = 8192, K = 2048) at batch sizes between the reference's default
+    decode batch (16) and a prefill: row quantiser + the Linear on codes, which runs these on the weight-streaming
+    kernel (a tiled GEMM has 64 tiles here and takes 12.6-13.3 us).  us per step, HIP-graph replay over 40 weights."""
+    N, K, nbuf = 8192, 2048, 40
+    weights = make_weights(torch, ops, N, K, nbuf, dev, seed=21, mode="int8")
+    g = torch.Generator(device=dev).manual_seed(22)
+    out = {"workload": f"linear_w8a8 K={K} N={N}, bf16 rows -> int8 per token, bf16 out; quantiser + Linear on codes"}
+    for M in (32, 64):
+        x = torch.randn(M, K, generator=g, device=dev).to(torch.bfloat16)
+
+        def step(i, x=x):
+            xq, sx = ops.quant_rowwise_i8(x)
+            wq, sw = weights[i % nbuf]
+            return ops.linear_w8a8(xq, sx, wq, sw, out_dtype=torch.bfloat16)
+
+        xq, sx = ops.quant_rowwise_i8(x)
+
+        def kern(i, xq=xq, sx=sx):
+            wq, sw = weights[i % nbuf]
+            return ops.linear_w8a8(xq, sx, wq, sw, out_dtype=torch.bfloat16)
+
+        t = graph_time_ms(torch, step, args.steps, args.warmup) * 1e3
+        tk = graph_time_ms(torch, kern, args.steps, args.warmup) * 1e3
+        nbytes = N * K + 4 * N + 2 * M * K + 2 * M * N
+        out[f"M={M}"] = {"us_per_step": t, "linear_on_codes_us": tk, "gbs": nbytes / t / 1e3,
+                         "frac_hbm_linear_on_codes": nbytes / tk / 1e3 / PEAK_HBM_GBS, "algorithmic_bytes": nbytes}
+    return out
 
 
 def bench_fp8(torch, ops, args, dev):
@@ -748,6 +783,7 @@ def main():
                     a2.m = m
                     r = bench_decode(torch, ops, a2, dev)
                     extra[f"decode_m{m}"] = r
+                extra["batch_32_to_64"] = bench_few_dozen_rows(torch, ops, args, dev)
         ceilings = measure_ceilings(torch, ops, dev, calibrate=not args.no_extra)
         if not args.no_extra and args.workload != "model":
             # the reference's own generation benchmark: about a minute; skipped when this run is already long

@@ -1263,10 +1263,9 @@ __global__ __launch_bounds__(KS * 2 * 64) void gemv_mfma_tokens_longk_kernel(Gem
 static bool gemv_tokens_fit(int64_t M, int64_t K) {
   return (K % 256) == 0 && 16 * ((M + 15) / 16) * (K + 16) + 16 <= GV_MAX_LDS;
 }
-// ... or, up to 32 rows of whole 128-byte lines, any length (the chunked kernel above)
-// -- which also takes the decode batch sizes whose rows are too long for the GEMV kernels' own LDS budget (9..16
-// rows beyond 10 096 bytes, 5..8 beyond 20 208, ...), where the tiles were the only path (12 x 4096 x 11008: 41 us
-// against 19 us).
+// ... or rows of whole 128-byte lines of any length (the chunked kernel above), which also takes the decode batch
+// sizes whose rows are too long for the GEMV kernels' own LDS budget (9..16 rows beyond 10 096 bytes, 5..8 beyond
+// 20 208, ...), where the tiles were the only path (12 x 4096 x 11008: 41 us against 19 us).
 bool gemv_tokens_ok(int64_t M, int64_t N, int64_t K) {
   if (M < 1 || M > 64 || N <= 0) return false;
   const bool chunked = (K % 128) == 0 && K <= (1 << 22);
@@ -1277,7 +1276,6 @@ bool gemv_tokens_ok(int64_t M, int64_t N, int64_t K) {
   return gemv_tokens_fit(M, K) || chunked;
 }
 
-// (not static: the tiled GEMM's entry points in gemm_mfma.hip hand these shapes over)
 template <int TG, int KS>
 static int launch_gemv_tokens_longk(const GemvArgs& a, hipStream_t st) {
   const unsigned grid = (unsigned)((a.N + 2 * GM_ROWS - 1) / (2 * GM_ROWS));
@@ -1291,6 +1289,8 @@ static int launch_gemv_tokens_longk(const GemvArgs& a, hipStream_t st) {
   return (int)hipGetLastError();
 }
 
+// (gemv_tokens_ok and gemv_tokens_launch are not static: the tiled GEMM's entry points in gemm_mfma.hip hand these
+// shapes over)
 int launch_gemv_tokens(GemvArgs a, hipStream_t st) {
   if (a.M <= 16 || !gemv_tokens_fit(a.M, a.K)) {
     // up to 32 tokens: 4096-byte chunks over 8 wavefronts while that still gives every compute unit a workgroup's

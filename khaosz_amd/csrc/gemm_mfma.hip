@@ -900,9 +900,10 @@ extern "C" int aq_linear_w8a8(const int8_t* xq, const float* sx, const int8_t* w
 namespace aq {
 // gemv.hip: the weight-streaming kernel for 17..64 rows (same sums, same epilogue: same bits)
 bool gemv_tokens_ok(int64_t M, int64_t N, int64_t K);
+bool gemv_tokens_fp8_ok(int64_t M, int64_t N, int64_t K);
 int gemv_tokens_launch(const int8_t* xq, const float* sx, const int8_t* wq, const float* sw, const void* bias,
                        int bias_dtype, const void* residual, void* y, int y_dtype, int64_t M, int64_t N, int64_t K,
-                       hipStream_t st);
+                       hipStream_t st, bool fp8);
 }  // namespace aq
 
 extern "C" int aq_linear_w8a8_residual(const int8_t* xq, const float* sx, const int8_t* wq, const float* sw,
@@ -925,7 +926,7 @@ extern "C" int aq_linear_w8a8_residual(const int8_t* xq, const float* sx, const 
   const bool tile_forced = false;
 #endif
   if (!tile_forced && aq::gemv_tokens_ok(M, N, K) && aq::check_ptr16(residual) == 0)
-    return aq::gemv_tokens_launch(xq, sx, wq, sw, bias, bias_dtype, residual, y, y_dtype, M, N, K, st);
+    return aq::gemv_tokens_launch(xq, sx, wq, sw, bias, bias_dtype, residual, y, y_dtype, M, N, K, st, false);
   aq::GemmArgs a = aq::make_args(xq, wq, y, M, N, K);
   a.sx = sx;
   a.sw = sw;
@@ -951,12 +952,21 @@ extern "C" int aq_linear_fp8_residual(const uint8_t* xq, const float* sx, const 
   if (aq::check_ptr(sx, 4) || aq::check_ptr(sw, 4) || aq::check_ptr(bias, bias_dtype == AQ_BF16 ? 2 : 4) ||
       aq::check_ptr(residual, 4))
     return AQ_E_ALIGN;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  // a few dozen rows: the weight-streaming kernel, as for int8 (fp32 sums in its own fixed order)
+#ifdef AQ_LAB
+  const bool tile_forced = aq::g_forced_tile != 0;
+#else
+  const bool tile_forced = false;
+#endif
+  if (!tile_forced && aq::gemv_tokens_fp8_ok(M, N, K) && aq::check_ptr16(residual) == 0)
+    return aq::gemv_tokens_launch(reinterpret_cast<const int8_t*>(xq), sx, reinterpret_cast<const int8_t*>(wq), sw, bias,
+                                  bias_dtype, residual, y, y_dtype, M, N, K, st, true);
   aq::GemmArgs a = aq::make_args(xq, wq, y, M, N, K);
   a.sx = sx;
   a.sw = sw;
   a.bias = bias;
   a.bias_dtype = bias_dtype;
   a.res = residual;
-  hipStream_t st = static_cast<hipStream_t>(stream);
   return y_dtype == AQ_BF16 ? aq::launch<true, aq::OUT_BF16>(a, st) : aq::launch<true, aq::OUT_F32>(a, st);
 }

@@ -896,7 +896,9 @@ static int launch_gemv_mfma_swiglu(GemvArgs a, hipStream_t st) {
 // decode batch sizes above and a prefill, the tiled GEMM has too few tiles to occupy the device (32 x 8192 x 2048:
 // 64 tiles of 128 x 128, 12.7 us); this kernel keeps it a bandwidth-bound launch.  Same integer sums, same
 // epilogue: the bits of the tiled GEMM.
-template <int TG, bool RES>
+// FP8: e4m3 codes with one scale per tensor and fp32 accumulation, as in gemv_mfma_kernel (K parts summed in a fixed
+// order).
+template <int TG, bool RES, bool FP8 = false>
 __global__ __launch_bounds__(GM_MAX_WAVES * 64) void gemv_mfma_tokens_kernel(GemvArgs p) {
   extern __shared__ __attribute__((aligned(16))) uint8_t xs[];  // [16 TG][K + 16] token codes, 16 spare bytes; later the partial sums
   constexpr int MTOK = 16 * TG;
@@ -960,11 +962,11 @@ __global__ __launch_bounds__(GM_MAX_WAVES * 64) void gemv_mfma_tokens_kernel(Gem
   for (int r = 0; r < TG; ++r) xload(r * XV * nthreads, xvr[r]);
   asm volatile("" ::: "memory");  // request order: token codes, epilogue operands, the weight stream
 #pragma unroll
-  for (int g = 0; g < TG; ++g) sxv[g] = epi.load_sx(tok + 16 * g, tok + 16 * g < M);
+  for (int g = 0; g < TG; ++g) sxv[g] = epi.load_sx(FP8 ? 0 : tok + 16 * g, FP8 || tok + 16 * g < M);
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
     const int n = rbase + r;
-    swv[r] = epi.load_sw(n, n < N);
+    swv[r] = epi.load_sw(FP8 ? 0 : n, FP8 || n < N);
     bv[r] = epi.load_bias(n, n < N);
 #pragma unroll
     for (int g = 0; g < TG; ++g) rv[g][r] = RES ? epi.load_res(tok + 16 * g, n, tok + 16 * g < M && n < N, (int)p.ldr) : 0u;
@@ -984,9 +986,10 @@ __global__ __launch_bounds__(GM_MAX_WAVES * 64) void gemv_mfma_tokens_kernel(Gem
   __builtin_amdgcn_s_barrier();  // no fence: the weight loads stay in flight
   asm volatile("" ::: "memory");
 
-  v4i accs[TG][2];
+  using accv = std::conditional_t<FP8, v4f, v4i>;
+  accv accs[TG][2];
 #pragma unroll
-  for (int g = 0; g < TG; ++g) accs[g][0] = accs[g][1] = v4i{0, 0, 0, 0};
+  for (int g = 0; g < TG; ++g) accs[g][0] = accs[g][1] = accv{0, 0, 0, 0};
   const uint8_t* xl = xs + tok * pitch + kh * khalf + (lane >> 4) * 32;
   auto consume = [&](int line0, const uint4 (&wc)[GM_BATCH]) {
 #pragma unroll
@@ -1010,8 +1013,14 @@ __global__ __launch_bounds__(GM_MAX_WAVES * 64) void gemv_mfma_tokens_kernel(Gem
                       __builtin_amdgcn_update_dpp((int)hi.w, (int)lo.w, ROR8, 0xf, 0x3, false)};
 #pragma unroll
       for (int g = 0; g < TG; ++g) {
-        accs[g][0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w0, x0[g], accs[g][0], 0, 0, 0);
-        accs[g][1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w1, x1[g], accs[g][1], 0, 0, 0);
+        if constexpr (!FP8) {
+          accs[g][0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w0, x0[g], accs[g][0], 0, 0, 0);
+          accs[g][1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w1, x1[g], accs[g][1], 0, 0, 0);
+        } else {  // the line's two pieces are the 32 K bytes a lane feeds one 16x16x128 product
+          const v8i wl = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+          const v8i xl8 = {x0[g].x, x0[g].y, x0[g].z, x0[g].w, x1[g].x, x1[g].y, x1[g].z, x1[g].w};
+          accs[g][t & 1] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wl, xl8, accs[g][t & 1], 0, 0, 0, 0, 0, 0);
+        }
       }
     }
   };
@@ -1022,21 +1031,21 @@ __global__ __launch_bounds__(GM_MAX_WAVES * 64) void gemv_mfma_tokens_kernel(Gem
     if (l0 + 3 * GM_LINES < nline) wload(l0 + 3 * GM_LINES, wb);
   }
 
-  // sum the K parts through LDS (exact int32)
+  // sum the K parts through LDS (int32: exact; fp32: in a fixed order)
   __syncthreads();  // everyone is done reading the token codes: the buffer is reused
   int* part = reinterpret_cast<int*>(xs) + (grp * (ksplit - 1)) * TG * 256;
-  v4i acc[TG];
+  accv acc[TG];
 #pragma unroll
   for (int g = 0; g < TG; ++g) acc[g] = accs[g][0] + accs[g][1];
   if (kh != 0) {
 #pragma unroll
-    for (int g = 0; g < TG; ++g) *reinterpret_cast<v4i*>(part + ((kh - 1) * TG + g) * 256 + lane * 4) = acc[g];
+    for (int g = 0; g < TG; ++g) *reinterpret_cast<accv*>(part + ((kh - 1) * TG + g) * 256 + lane * 4) = acc[g];
   }
   __syncthreads();
   if (kh != 0) return;
   for (int k = 0; k < ksplit - 1; ++k)
 #pragma unroll
-    for (int g = 0; g < TG; ++g) acc[g] += *reinterpret_cast<const v4i*>(part + (k * TG + g) * 256 + lane * 4);
+    for (int g = 0; g < TG; ++g) acc[g] += *reinterpret_cast<const accv*>(part + (k * TG + g) * 256 + lane * 4);
 
 #pragma unroll
   for (int g = 0; g < TG; ++g) {
@@ -1291,8 +1300,8 @@ static int launch_gemv_tokens_longk(const GemvArgs& a, hipStream_t st) {
 
 // (gemv_tokens_ok and gemv_tokens_launch are not static: the tiled GEMM's entry points in gemm_mfma.hip hand these
 // shapes over)
-int launch_gemv_tokens(GemvArgs a, hipStream_t st) {
-  if (a.M <= 16 || !gemv_tokens_fit(a.M, a.K)) {
+int launch_gemv_tokens(GemvArgs a, hipStream_t st, bool fp8 = false) {
+  if (!fp8 && (a.M <= 16 || !gemv_tokens_fit(a.M, a.K))) {
     // up to 32 tokens: 4096-byte chunks over 8 wavefronts while that still gives every compute unit a workgroup's
     // worth of loads, 2048-byte chunks over 4 wavefronts for wide matrices; more tokens: 2048-byte chunks (LDS)
     if (a.M > 48) return launch_gemv_tokens_longk<4, 2>(a, st);
@@ -1318,22 +1327,29 @@ int launch_gemv_tokens(GemvArgs a, hipStream_t st) {
   const size_t lds = (size_t)16 * tg * (a.K + 16) + 16;
   const bool res = a.res != nullptr;
   using kern_t = void (*)(GemvArgs);
-  static const kern_t table[3][2] = {{gemv_mfma_tokens_kernel<2, false>, gemv_mfma_tokens_kernel<2, true>},
-                                     {gemv_mfma_tokens_kernel<3, false>, gemv_mfma_tokens_kernel<3, true>},
-                                     {gemv_mfma_tokens_kernel<4, false>, gemv_mfma_tokens_kernel<4, true>}};
-  const kern_t fn = table[tg - 2][res];
+  static const kern_t table[2][3][2] = {
+      {{gemv_mfma_tokens_kernel<2, false>, gemv_mfma_tokens_kernel<2, true>},
+       {gemv_mfma_tokens_kernel<3, false>, gemv_mfma_tokens_kernel<3, true>},
+       {gemv_mfma_tokens_kernel<4, false>, gemv_mfma_tokens_kernel<4, true>}},
+      {{gemv_mfma_tokens_kernel<2, false, true>, gemv_mfma_tokens_kernel<2, true, true>},
+       {gemv_mfma_tokens_kernel<3, false, true>, gemv_mfma_tokens_kernel<3, true, true>},
+       {gemv_mfma_tokens_kernel<4, false, true>, gemv_mfma_tokens_kernel<4, true, true>}}};
+  const kern_t fn = table[fp8][tg - 2][res];
   if (lds > 64 * 1024) {
-    static LdsOptIn opted[6];
-    const int e = opted[(tg - 2) * 2 + res].ensure(reinterpret_cast<const void*>(fn));
+    static LdsOptIn opted[12];
+    const int e = opted[fp8 * 6 + (tg - 2) * 2 + res].ensure(reinterpret_cast<const void*>(fn));
     if (e) return e;
   }
   hipLaunchKernelGGL(fn, dim3(grid), dim3(a.ksplit * a.groups * 64), lds, st, a);
   return (int)hipGetLastError();
 }
 
+// the FP8 Linear's share of these shapes: 17..64 rows whose codes fit LDS (no chunked variant)
+bool gemv_tokens_fp8_ok(int64_t M, int64_t N, int64_t K) { return M > 16 && M <= 64 && N > 0 && gemv_tokens_fit(M, K); }
+
 int gemv_tokens_launch(const int8_t* xq, const float* sx, const int8_t* wq, const float* sw, const void* bias,
                        int bias_dtype, const void* residual, void* y, int y_dtype, int64_t M, int64_t N, int64_t K,
-                       hipStream_t st) {
+                       hipStream_t st, bool fp8) {
   GemvArgs a{};
   a.xq = xq;
   a.sx = sx;
@@ -1348,7 +1364,7 @@ int gemv_tokens_launch(const int8_t* xq, const float* sx, const int8_t* wq, cons
   a.K = (int)K;
   a.bias_dtype = bias_dtype;
   a.y_dtype = y_dtype;
-  return launch_gemv_tokens(a, st);
+  return launch_gemv_tokens(a, st, fp8);
 }
 
 static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }

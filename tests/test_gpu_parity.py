@@ -738,6 +738,43 @@ def test_linear_fp8_within_tolerance(oracle, tile, M, N, K):
             assert rc == 0 and torch.equal(y_in_place, ops.linear_fp8(*args, out_dtype=dt) + r)
 
 
+@pytest.mark.parametrize("M", [17, 32, 33, 50, 64])
+@pytest.mark.parametrize("N,K", [(8192, 2048), (77, 512), (3072, 1536), (200, 256), (8400, 2304), (130, 4096)])
+def test_linear_fp8_a_few_dozen_rows_take_the_weight_streaming_kernel(oracle, M, N, K):
+    """17..64 rows of FP8 codes that fit a compute unit's LDS go to the weight-streaming kernel (one 16x16x128
+    product per 128-byte line and token group, fp32 sums, K parts added in a fixed order); (130, 4096) fits up to
+    32 rows and stays on the tiles beyond.  Against the float64 sum of the oracle's codes inside the stated
+    tolerance, against the tiled GEMM on the same codes (a forced tile shape keeps it on the tiles) within the
+    change of summation order, with bias and residual, and the same bits on a second call."""
+    _say("linear_fp8, few dozen rows", M, N, K)
+    x = make_x(M, K, 61 + M).to(torch.bfloat16)
+    w = make_x(N, K, 62) * 0.02
+    xq, sx = oracle.c_quant_tensor_fp8(bf16_bits(x), bf16_bits=True)
+    wq, sw = oracle.c_quant_tensor_fp8(w.numpy())
+    g = torch.Generator().manual_seed(63)
+    bias = torch.randn(N, generator=g) * 0.3
+    args = (torch.from_numpy(xq).to(DEV), torch.tensor([sx], device=DEV), torch.from_numpy(wq).to(DEV),
+            torch.tensor([sw], device=DEV))
+    exact = oracle.np_linear_fp8(xq, sx, wq, sw, bias=bias.numpy())
+    rms = float(np.sqrt(np.mean(exact.astype(np.float64) ** 2)))
+    y32 = ops.linear_fp8(*args, bias.to(DEV), out_dtype=torch.float32)
+    assert np.max(np.abs(to_np(y32) - exact)) <= 1e-3 * rms
+    assert torch.equal(ops.linear_fp8(*args, bias.to(DEV), out_dtype=torch.float32), y32)
+    yb = ops.linear_fp8(*args, bias.to(DEV), out_dtype=torch.bfloat16)
+    np.testing.assert_allclose(to_np(yb.float()), exact, rtol=1e-2, atol=1e-2 * rms)   # stated tolerance
+    np.testing.assert_allclose(to_np(y32), oracle.c_linear_fp8(xq, sx, wq, sw, bias=bias.numpy()), rtol=1e-2,
+                               atol=1e-3 * rms)
+    nb = ops.linear_fp8(*args, out_dtype=torch.float32)
+    assert np.max(np.abs(to_np(nb) - oracle.np_linear_fp8(xq, sx, wq, sw))) <= 1e-3 * rms
+    for dt, plain in ((torch.float32, y32), (torch.bfloat16, yb)):
+        r = torch.randn(M, N, generator=g).to(dt).to(DEV)
+        assert torch.equal(ops.linear_fp8(*args, bias.to(DEV), out_dtype=dt, residual=r), plain + r)
+    with _abi.lab_library() as lab:
+        assert lab.aq_lab_set_gemm_tile(128) == 0
+        yt = ops.linear_fp8(*args, bias.to(DEV), out_dtype=torch.float32)
+    assert np.max(np.abs(to_np(yt) - to_np(y32))) <= 2e-5 * rms
+
+
 @pytest.mark.parametrize("M", [1, 3, 8, 9, 16])
 @pytest.mark.parametrize("N,K", [(8192, 2048), (77, 512), (11264, 1024), (300, 4096), (130, 1040)])
 def test_gemv_fp8_decode_within_tolerance(oracle, M, N, K):

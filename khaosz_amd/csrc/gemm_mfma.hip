@@ -900,7 +900,6 @@ extern "C" int aq_linear_w8a8(const int8_t* xq, const float* sx, const int8_t* w
 namespace aq {
 // gemv.hip: the weight-streaming kernel for 17..64 rows (same sums, same epilogue: same bits)
 bool gemv_tokens_ok(int64_t M, int64_t N, int64_t K);
-bool gemv_tokens_fp8_ok(int64_t M, int64_t N, int64_t K);
 int gemv_tokens_launch(const int8_t* xq, const float* sx, const int8_t* wq, const float* sw, const void* bias,
                        int bias_dtype, const void* residual, void* y, int y_dtype, int64_t M, int64_t N, int64_t K,
                        hipStream_t st, bool fp8);
@@ -959,7 +958,7 @@ extern "C" int aq_linear_fp8_residual(const uint8_t* xq, const float* sx, const 
 #else
   const bool tile_forced = false;
 #endif
-  if (!tile_forced && aq::gemv_tokens_fp8_ok(M, N, K) && aq::check_ptr16(residual) == 0)
+  if (!tile_forced && aq::gemv_tokens_ok(M, N, K) && aq::check_ptr16(residual) == 0)
     return aq::gemv_tokens_launch(reinterpret_cast<const int8_t*>(xq), sx, reinterpret_cast<const int8_t*>(wq), sw, bias,
                                   bias_dtype, residual, y, y_dtype, M, N, K, st, true);
   aq::GemmArgs a = aq::make_args(xq, wq, y, M, N, K);

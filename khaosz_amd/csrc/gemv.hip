@@ -894,210 +894,27 @@ static int launch_gemv_mfma_swiglu(GemvArgs a, hipStream_t st) {
 // 17..64 tokens on codes: the same weight stream (every weight byte HBM -> registers once, operands assembled by
 // one DPP rotation per dword) with TG groups of 16 tokens multiplied against each weight fragment.  Between the
 // decode batch sizes above and a prefill, the tiled GEMM has too few tiles to occupy the device (32 x 8192 x 2048:
-// 64 tiles of 128 x 128, 12.7 us); this kernel keeps it a bandwidth-bound launch.  Same integer sums, same
+// 64 tiles of 128 x 128, 9.3 us); this kernel keeps it a bandwidth-bound launch (5.2 us).  Same integer sums, same
 // epilogue: the bits of the tiled GEMM.
-// FP8: e4m3 codes with one scale per tensor and fp32 accumulation, as in gemv_mfma_kernel (K parts summed in a fixed
-// order).
-template <int TG, bool RES, bool FP8 = false>
-__global__ __launch_bounds__(GM_MAX_WAVES * 64) void gemv_mfma_tokens_kernel(GemvArgs p) {
-  extern __shared__ __attribute__((aligned(16))) uint8_t xs[];  // [16 TG][K + 16] token codes, 16 spare bytes; later the partial sums
-  constexpr int MTOK = 16 * TG;
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int ksplit = p.ksplit, groups = p.groups;
-  const int nthreads = ksplit * groups * 64;
-  const int grp = wave / ksplit, kh = wave % ksplit;
-  const int K = p.K, N = p.N, M = p.M;
-  const int n0 = __builtin_amdgcn_readfirstlane((blockIdx.x * groups + grp) * GM_ROWS);
-  const int pitch = K + 16;
-  const int khalf = K / ksplit;   // a multiple of 128 (checked by the launcher)
-  const int nline = khalf / 128;
-
-  const int tok = lane & 15;
-  const int rbase = n0 + (lane >> 4) * 4;
-  float swv[4], bv[4], sxv[TG];
-  uint32_t rv[TG][4];
-  const EpiOperands epi(p, kh == 0, true, RES);
-
-  const int rows = n0 < N ? ((N - n0) < GM_ROWS ? (N - n0) : GM_ROWS) : 0;
-  const __amdgpu_buffer_rsrc_t Wr = make_rsrc(p.wq + (int64_t)(n0 < N ? n0 : 0) * K, (uint32_t)rows * (uint32_t)K);
-  const uint32_t woff = (uint32_t)(lane & 7) * (uint32_t)K + (uint32_t)(kh * khalf + (lane >> 3) * 16);
-  const uint32_t woff8 = 8u * (uint32_t)K;
-  constexpr int GM_LINES = GM_BATCH / 2;
-  uint4 wa[GM_BATCH], wb[GM_BATCH];
-  auto wload = [&](int line0, uint4 (&dst)[GM_BATCH]) {
-#pragma unroll
-    for (int t = 0; t < GM_LINES; ++t) {
-      const bool ok = (line0 + t) < nline;
-      const uint32_t o = woff + (uint32_t)(line0 + t) * 128u;
-      dst[2 * t] = GV_WLOAD(Wr, ok ? o : OOB_OFFSET);
-      dst[2 * t + 1] = GV_WLOAD(Wr, ok ? o + woff8 : OOB_OFFSET);
-    }
-  };
-
-  // token codes -> LDS: TG rounds of 8 vectors per thread are requested ahead of the weights (MTOK x 2048 codes
-  // with 256 threads), longer rows copy the rest behind them
-  const __amdgpu_buffer_rsrc_t Xr = make_rsrc(p.xq, (uint32_t)M * (uint32_t)K);
-  const int nvec_row = K / 16;
-  const int nvec = MTOK * nvec_row;
-  constexpr int XV = 8;
-  uint4 xvr[TG][XV];
-  auto xload = [&](int v0, uint4 (&xv)[XV]) {
-#pragma unroll
-    for (int i = 0; i < XV; ++i) {
-      const int v = v0 + i * nthreads + tid;
-      xv[i] = buffer_load_16(Xr, v < nvec ? (uint32_t)v * 16u : OOB_OFFSET);
-    }
-  };
-  uint8_t* const spare = xs + MTOK * pitch;
-  auto xstore = [&](int v0, const uint4 (&xv)[XV]) {
-#pragma unroll
-    for (int i = 0; i < XV; ++i) {
-      const int v = v0 + i * nthreads + tid;
-      const int m = v / nvec_row, c = v - m * nvec_row;
-      *reinterpret_cast<uint4*>(v < nvec ? xs + m * pitch + c * 16 : spare) = xv[i];
-    }
-  };
-#pragma unroll
-  for (int r = 0; r < TG; ++r) xload(r * XV * nthreads, xvr[r]);
-  asm volatile("" ::: "memory");  // request order: token codes, epilogue operands, the weight stream
-#pragma unroll
-  for (int g = 0; g < TG; ++g) sxv[g] = epi.load_sx(FP8 ? 0 : tok + 16 * g, FP8 || tok + 16 * g < M);
-#pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    const int n = rbase + r;
-    swv[r] = epi.load_sw(FP8 ? 0 : n, FP8 || n < N);
-    bv[r] = epi.load_bias(n, n < N);
-#pragma unroll
-    for (int g = 0; g < TG; ++g) rv[g][r] = RES ? epi.load_res(tok + 16 * g, n, tok + 16 * g < M && n < N, (int)p.ldr) : 0u;
-  }
-  asm volatile("" ::: "memory");
-  wload(0, wa);
-  wload(GM_LINES, wb);
-  asm volatile("" ::: "memory");
-#pragma unroll
-  for (int r = 0; r < TG; ++r) xstore(r * XV * nthreads, xvr[r]);
-  for (int v0 = TG * XV * nthreads; v0 < nvec; v0 += XV * nthreads) {
-    xload(v0, xvr[0]);
-    xstore(v0, xvr[0]);
-  }
-  __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
-  asm volatile("" ::: "memory");
-  __builtin_amdgcn_s_barrier();  // no fence: the weight loads stay in flight
-  asm volatile("" ::: "memory");
-
-  using accv = std::conditional_t<FP8, v4f, v4i>;
-  accv accs[TG][2];
-#pragma unroll
-  for (int g = 0; g < TG; ++g) accs[g][0] = accs[g][1] = accv{0, 0, 0, 0};
-  const uint8_t* xl = xs + tok * pitch + kh * khalf + (lane >> 4) * 32;
-  auto consume = [&](int line0, const uint4 (&wc)[GM_BATCH]) {
-#pragma unroll
-    for (int t = 0; t < GM_LINES; ++t) {
-      const int ln = (line0 + t) < nline ? (line0 + t) : 0;  // lines past the end multiply zero weights
-      v4i x0[TG], x1[TG];
-#pragma unroll
-      for (int g = 0; g < TG; ++g) {
-        x0[g] = *reinterpret_cast<const v4i*>(xl + g * 16 * pitch + ln * 128);
-        x1[g] = *reinterpret_cast<const v4i*>(xl + g * 16 * pitch + ln * 128 + 16);
-      }
-      const uint4 lo = wc[2 * t], hi = wc[2 * t + 1];
-      constexpr int ROR8 = 0x128;  // DPP row_ror:8 (see gemv_mfma_kernel)
-      const v4i w0 = {__builtin_amdgcn_update_dpp((int)lo.x, (int)hi.x, ROR8, 0xf, 0xc, false),
-                      __builtin_amdgcn_update_dpp((int)lo.y, (int)hi.y, ROR8, 0xf, 0xc, false),
-                      __builtin_amdgcn_update_dpp((int)lo.z, (int)hi.z, ROR8, 0xf, 0xc, false),
-                      __builtin_amdgcn_update_dpp((int)lo.w, (int)hi.w, ROR8, 0xf, 0xc, false)};
-      const v4i w1 = {__builtin_amdgcn_update_dpp((int)hi.x, (int)lo.x, ROR8, 0xf, 0x3, false),
-                      __builtin_amdgcn_update_dpp((int)hi.y, (int)lo.y, ROR8, 0xf, 0x3, false),
-                      __builtin_amdgcn_update_dpp((int)hi.z, (int)lo.z, ROR8, 0xf, 0x3, false),
-                      __builtin_amdgcn_update_dpp((int)hi.w, (int)lo.w, ROR8, 0xf, 0x3, false)};
-#pragma unroll
-      for (int g = 0; g < TG; ++g) {
-        if constexpr (!FP8) {
-          accs[g][0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w0, x0[g], accs[g][0], 0, 0, 0);
-          accs[g][1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w1, x1[g], accs[g][1], 0, 0, 0);
-        } else {  // the line's two pieces are the 32 K bytes a lane feeds one 16x16x128 product
-          const v8i wl = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
-          const v8i xl8 = {x0[g].x, x0[g].y, x0[g].z, x0[g].w, x1[g].x, x1[g].y, x1[g].z, x1[g].w};
-          accs[g][t & 1] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wl, xl8, accs[g][t & 1], 0, 0, 0, 0, 0, 0);
-        }
-      }
-    }
-  };
-  for (int l0 = 0; l0 < nline; l0 += 2 * GM_LINES) {
-    consume(l0, wa);
-    if (l0 + 2 * GM_LINES < nline) wload(l0 + 2 * GM_LINES, wa);
-    if (l0 + GM_LINES < nline) consume(l0 + GM_LINES, wb);
-    if (l0 + 3 * GM_LINES < nline) wload(l0 + 3 * GM_LINES, wb);
-  }
-
-  // sum the K parts through LDS (int32: exact; fp32: in a fixed order)
-  __syncthreads();  // everyone is done reading the token codes: the buffer is reused
-  int* part = reinterpret_cast<int*>(xs) + (grp * (ksplit - 1)) * TG * 256;
-  accv acc[TG];
-#pragma unroll
-  for (int g = 0; g < TG; ++g) acc[g] = accs[g][0] + accs[g][1];
-  if (kh != 0) {
-#pragma unroll
-    for (int g = 0; g < TG; ++g) *reinterpret_cast<accv*>(part + ((kh - 1) * TG + g) * 256 + lane * 4) = acc[g];
-  }
-  __syncthreads();
-  if (kh != 0) return;
-  for (int k = 0; k < ksplit - 1; ++k)
-#pragma unroll
-    for (int g = 0; g < TG; ++g) acc[g] += *reinterpret_cast<const accv*>(part + (k * TG + g) * 256 + lane * 4);
-
-#pragma unroll
-  for (int g = 0; g < TG; ++g) {
-    const int tk = tok + 16 * g;
-    if (tk >= M) continue;
-    float y[4];
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      y[r] = __fmul_rn(__fmul_rn((float)acc[g][r], sxv[g]), swv[r]);
-      if (p.bias) y[r] = __fadd_rn(y[r], bv[r]);
-      if constexpr (RES) y[r] = p.y_dtype == AQ_BF16 ? add_residual_bf16(y[r], rv[g][r]) : __fadd_rn(y[r], __uint_as_float(rv[g][r]));
-    }
-    const int64_t o = (int64_t)tk * N + rbase;
-    if (p.y_dtype == AQ_BF16) {
-      uint16_t* dst = reinterpret_cast<uint16_t*>(p.y) + o;
-      if ((N & 3) == 0 && rbase + 3 < N) {
-        uint2 pk;
-        pk.x = pack_bf16x2(y[0], y[1]);
-        pk.y = pack_bf16x2(y[2], y[3]);
-        *reinterpret_cast<uint2*>(dst) = pk;
-      } else {
-#pragma unroll
-        for (int r = 0; r < 4; ++r)
-          if (rbase + r < N) dst[r] = (uint16_t)f32_to_bf16_bits(y[r]);
-      }
-    } else {
-      float* dst = reinterpret_cast<float*>(p.y) + o;
-      if ((N & 3) == 0 && rbase + 3 < N) {
-        *reinterpret_cast<float4*>(dst) = make_float4(y[0], y[1], y[2], y[3]);
-      } else {
-#pragma unroll
-        for (int r = 0; r < 4; ++r)
-          if (rbase + r < N) dst[r] = y[r];
-      }
-    }
-  }
-}
-
-// The same for tokens whose rows are too long for their codes to sit in LDS all at once (an MLP's down
-// projection): K is walked in chunks of 1024 bytes per wavefront (KS wavefronts per row group: 2048- or, for up to
-// 32 tokens, 4096-byte chunks per workgroup), the token codes of one chunk at a time in LDS.  A chunk's codes are requested into registers
-// while the chunk before is multiplied and stored between two barriers; the weight stream runs through the chunk
-// boundaries untouched (two register batches, each reloaded as soon as it has been consumed).  Two row groups per
-// workgroup; rows must be whole 128-byte lines (K % 128 == 0).
-template <int TG, int KS, bool RES>
-__global__ __launch_bounds__(KS * 2 * 64) void gemv_mfma_tokens_longk_kernel(GemvArgs p) {
+// K is walked in chunks of 1024 bytes per wavefront (KS wavefronts per row group: 1024-, 2048- or 4096-byte chunks
+// per workgroup), the token codes of one chunk at a time in LDS, so that rows of any length are taken (an MLP's
+// down projection) and the LDS of a compute unit holds several workgroups.  A chunk's codes are requested into
+// registers while the chunk before is multiplied and stored between two barriers; the weight stream runs through
+// the chunk boundaries untouched (two register batches, each reloaded as soon as it has been consumed).  GRP row
+// groups of 16 rows per workgroup (every workgroup copies all token codes from L2: more rows per workgroup for
+// matrices of more 32-row blocks than compute units); rows must be whole 128-byte lines (K % 128 == 0).
+// FP8: e4m3 codes with one scale per tensor and fp32 accumulation, as in gemv_mfma_kernel (chunks and K parts
+// summed in a fixed order).
+template <int TG, int KS, bool RES, int GRP = 2, bool FP8 = false>
+__global__ __launch_bounds__(KS * GRP * 64) void gemv_mfma_tokens_kernel(GemvArgs p) {
   extern __shared__ __attribute__((aligned(16))) uint8_t xs[];  // [16 TG][KC + 16] codes of one chunk; later the partial sums
-  constexpr int MTOK = 16 * TG, GRP = 2, NTHREADS = KS * GRP * 64;
+  constexpr int MTOK = 16 * TG, NTHREADS = KS * GRP * 64;
   constexpr int KC = 1024 * KS;            // K bytes of a chunk
   constexpr int PITCH = KC + 16;
-  constexpr int XV = MTOK * (KC / 16) / NTHREADS;  // 16-byte vectors of a chunk's codes per thread: 8 per token group
-  static_assert(XV == 8 * TG && MTOK * PITCH <= 150 * 1024, "a chunk's codes: 8 vectors per thread and token group, within LDS");
+  constexpr int XV = MTOK * (KC / 16) / NTHREADS;  // 16-byte vectors of a chunk's codes per thread: 16 / GRP per token group
+  static_assert(XV * NTHREADS == MTOK * (KC / 16) && MTOK * PITCH <= 150 * 1024 && KS * GRP <= GM_MAX_WAVES,
+                "a chunk's codes: whole vectors per thread, within LDS");
+  static_assert(GRP * (KS - 1) * TG * 1024 <= MTOK * PITCH, "the partial sums reuse the codes' LDS");
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int grp = wave / KS, kh = wave % KS;
@@ -1152,11 +969,11 @@ __global__ __launch_bounds__(KS * 2 * 64) void gemv_mfma_tokens_longk_kernel(Gem
   xload(0);
   asm volatile("" ::: "memory");  // request order: token codes, epilogue operands, the weight stream
 #pragma unroll
-  for (int g = 0; g < TG; ++g) sxv[g] = epi.load_sx(tok + 16 * g, tok + 16 * g < M);
+  for (int g = 0; g < TG; ++g) sxv[g] = epi.load_sx(FP8 ? 0 : tok + 16 * g, FP8 || tok + 16 * g < M);
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
     const int n = rbase + r;
-    swv[r] = epi.load_sw(n, n < N);
+    swv[r] = epi.load_sw(FP8 ? 0 : n, FP8 || n < N);
     bv[r] = epi.load_bias(n, n < N);
 #pragma unroll
     for (int g = 0; g < TG; ++g) rv[g][r] = RES ? epi.load_res(tok + 16 * g, n, tok + 16 * g < M && n < N, (int)p.ldr) : 0u;
@@ -1166,9 +983,10 @@ __global__ __launch_bounds__(KS * 2 * 64) void gemv_mfma_tokens_longk_kernel(Gem
   wload(0, GM_LINES, wb);
   asm volatile("" ::: "memory");
 
-  v4i accs[TG][2];
+  using accv = std::conditional_t<FP8, v4f, v4i>;
+  accv accs[TG][2];
 #pragma unroll
-  for (int g = 0; g < TG; ++g) accs[g][0] = accs[g][1] = v4i{0, 0, 0, 0};
+  for (int g = 0; g < TG; ++g) accs[g][0] = accs[g][1] = accv{0, 0, 0, 0};
   const uint8_t* xl = xs + tok * PITCH + kh * 1024 + (lane >> 4) * 32;
   auto consume = [&](int line0, const uint4 (&wc)[GM_BATCH]) {
 #pragma unroll
@@ -1191,8 +1009,14 @@ __global__ __launch_bounds__(KS * 2 * 64) void gemv_mfma_tokens_longk_kernel(Gem
                       __builtin_amdgcn_update_dpp((int)hi.w, (int)lo.w, ROR8, 0xf, 0x3, false)};
 #pragma unroll
       for (int g = 0; g < TG; ++g) {
-        accs[g][0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w0, x0[g], accs[g][0], 0, 0, 0);
-        accs[g][1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w1, x1[g], accs[g][1], 0, 0, 0);
+        if constexpr (!FP8) {
+          accs[g][0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w0, x0[g], accs[g][0], 0, 0, 0);
+          accs[g][1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w1, x1[g], accs[g][1], 0, 0, 0);
+        } else {  // the line's two pieces are the 32 K bytes a lane feeds one 16x16x128 product
+          const v8i wl = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+          const v8i xl8 = {x0[g].x, x0[g].y, x0[g].z, x0[g].w, x1[g].x, x1[g].y, x1[g].z, x1[g].w};
+          accs[g][t & 1] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wl, xl8, accs[g][t & 1], 0, 0, 0, 0, 0, 0);
+        }
       }
     }
   };
@@ -1214,21 +1038,21 @@ __global__ __launch_bounds__(KS * 2 * 64) void gemv_mfma_tokens_longk_kernel(Gem
     if (c + 1 < nchunk) wload(c + 1, GM_LINES, wb);
   }
 
-  // sum the K parts through LDS (exact int32)
+  // sum the K parts through LDS (int32: exact; fp32: in a fixed order)
   __syncthreads();
   int* part = reinterpret_cast<int*>(xs) + (grp * (KS - 1)) * TG * 256;
-  v4i acc[TG];
+  accv acc[TG];
 #pragma unroll
   for (int g = 0; g < TG; ++g) acc[g] = accs[g][0] + accs[g][1];
   if (kh != 0) {
 #pragma unroll
-    for (int g = 0; g < TG; ++g) *reinterpret_cast<v4i*>(part + ((kh - 1) * TG + g) * 256 + lane * 4) = acc[g];
+    for (int g = 0; g < TG; ++g) *reinterpret_cast<accv*>(part + ((kh - 1) * TG + g) * 256 + lane * 4) = acc[g];
   }
   __syncthreads();
   if (kh != 0) return;
   for (int k = 0; k < KS - 1; ++k)
 #pragma unroll
-    for (int g = 0; g < TG; ++g) acc[g] += *reinterpret_cast<const v4i*>(part + (k * TG + g) * 256 + lane * 4);
+    for (int g = 0; g < TG; ++g) acc[g] += *reinterpret_cast<const accv*>(part + (k * TG + g) * 256 + lane * 4);
 
 #pragma unroll
   for (int g = 0; g < TG; ++g) {
@@ -1267,85 +1091,59 @@ __global__ __launch_bounds__(KS * 2 * 64) void gemv_mfma_tokens_longk_kernel(Gem
   }
 }
 
-// Shapes the token-group kernel takes: 17..64 rows, K in whole 256-byte steps, the padded codes within a compute
-// unit's LDS.
-static bool gemv_tokens_fit(int64_t M, int64_t K) {
-  return (K % 256) == 0 && 16 * ((M + 15) / 16) * (K + 16) + 16 <= GV_MAX_LDS;
-}
-// ... or rows of whole 128-byte lines of any length (the chunked kernel above), which also takes the decode batch
-// sizes whose rows are too long for the GEMV kernels' own LDS budget (9..16 rows beyond 10 096 bytes, 5..8 beyond
-// 20 208, ...), where the tiles were the only path (12 x 4096 x 11008: 41 us against 19 us).
+// Shapes the token-group kernel takes: 17..64 rows of whole 128-byte lines, and the decode batch sizes whose rows
+// are too long for the GEMV kernels' own LDS budget (9..16 rows beyond 10 096 bytes, 5..8 beyond 20 208, ...),
+// where the tiles were the only path (12 x 4096 x 11008: 41 us against 19 us).  int8 and FP8 codes alike.
 bool gemv_tokens_ok(int64_t M, int64_t N, int64_t K) {
-  if (M < 1 || M > 64 || N <= 0) return false;
-  const bool chunked = (K % 128) == 0 && K <= (1 << 22);
+  if (M < 1 || M > 64 || N <= 0 || (K % 128) != 0 || K > (1 << 22)) return false;
   if (M <= 16) {
     const int64_t mt = M <= 1 ? 1 : M <= 2 ? 2 : M <= 4 ? 4 : M <= 8 ? 8 : 16;
-    return chunked && mt * K + 64 + 2048 > GV_MAX_LDS;  // the GEMV kernels' own limit (gemv_check)
+    return mt * K + 64 + 2048 > GV_MAX_LDS;  // the GEMV kernels' own limit (gemv_check)
   }
-  return gemv_tokens_fit(M, K) || chunked;
+  return true;
 }
 
-template <int TG, int KS>
-static int launch_gemv_tokens_longk(const GemvArgs& a, hipStream_t st) {
-  const unsigned grid = (unsigned)((a.N + 2 * GM_ROWS - 1) / (2 * GM_ROWS));
+template <int TG, int KS, int GRP>
+static int launch_gemv_tokens_shape(const GemvArgs& a, hipStream_t st, bool fp8) {
+  const unsigned grid = (unsigned)((a.N + GRP * GM_ROWS - 1) / (GRP * GM_ROWS));
   const size_t lds = (size_t)16 * TG * (1024 * KS + 16) + 16;
   using kern_t = void (*)(GemvArgs);
-  const kern_t fn = a.res ? gemv_mfma_tokens_longk_kernel<TG, KS, true> : gemv_mfma_tokens_longk_kernel<TG, KS, false>;
-  static LdsOptIn opted[2];
-  const int e = opted[a.res ? 1 : 0].ensure(reinterpret_cast<const void*>(fn));
+  const kern_t fn = fp8 ? (a.res ? gemv_mfma_tokens_kernel<TG, KS, true, GRP, true> : gemv_mfma_tokens_kernel<TG, KS, false, GRP, true>)
+                        : (a.res ? gemv_mfma_tokens_kernel<TG, KS, true, GRP> : gemv_mfma_tokens_kernel<TG, KS, false, GRP>);
+  static LdsOptIn opted[4];
+  const int e = opted[(fp8 ? 2 : 0) + (a.res ? 1 : 0)].ensure(reinterpret_cast<const void*>(fn));
   if (e) return e;
-  hipLaunchKernelGGL(fn, dim3(grid), dim3(KS * 2 * 64), lds, st, a);
+  hipLaunchKernelGGL(fn, dim3(grid), dim3(KS * GRP * 64), lds, st, a);
   return (int)hipGetLastError();
 }
 
+// Chunk and workgroup shapes, from timings of 17..64 rows over N = 256..16384, K = 512..4096 (the tiles take 9.3 us
+// at K = 2048 whatever N up to 16384, 13.7 us at K = 4096):
+//   * chunks no longer than the rows, or wavefronts idle: 1024 bytes up to K = 1024, else 2048; 4096 over 8
+//     wavefronts for up to 32 tokens and K >= 4096 while every compute unit gets at most one workgroup
+//     (32 x 6144 x 4096: 7.5 us against 8.5 us);
+//   * 32 rows per workgroup while there are no more 32-row blocks than compute units (32 x 8192 x 2048: 5.2 us, 64
+//     rows 6.8 us), 64 rows beyond (48 x 16384 x 2048: 7.9 us against 11.3 us: half the copies of the token codes),
+//     with 1024-byte chunks for 49..64 tokens, whose 2048-byte chunks leave LDS for one workgroup per compute unit
+//     (64 x 16384 x 2048: 9.8 us against 13.0 us);
+//   * short rows (K <= 1024): 64 rows per workgroup also for 49..64 tokens (64 x 4096 x 1024: 5.6 us against 6.1 us).
 // (gemv_tokens_ok and gemv_tokens_launch are not static: the tiled GEMM's entry points in gemm_mfma.hip hand these
 // shapes over)
-int launch_gemv_tokens(GemvArgs a, hipStream_t st, bool fp8 = false) {
-  if (!fp8 && (a.M <= 16 || !gemv_tokens_fit(a.M, a.K))) {
-    // up to 32 tokens: 4096-byte chunks over 8 wavefronts while that still gives every compute unit a workgroup's
-    // worth of loads, 2048-byte chunks over 4 wavefronts for wide matrices; more tokens: 2048-byte chunks (LDS)
-    if (a.M > 48) return launch_gemv_tokens_longk<4, 2>(a, st);
-    if (a.M > 32) return launch_gemv_tokens_longk<3, 2>(a, st);
-    return (a.N + 31) / 32 > device_cus() ? launch_gemv_tokens_longk<2, 2>(a, st) : launch_gemv_tokens_longk<2, 4>(a, st);
-  }
-  a.ksplit = 2;
-  a.groups = 2;
-  const int cus = device_cus();
-  if ((a.N + 31) / 32 < cus) {
-    a.groups = 1;
-    while (a.ksplit < GM_MAX_WAVES && (a.N + 15) / 16 * (a.ksplit / 2) < cus && a.K % (256 * a.ksplit) == 0 &&
-           a.K / (2 * a.ksplit) >= 512)
-      a.ksplit *= 2;
-  }
-  // more 32-row blocks than compute units: 64 rows per workgroup, so that a second round of workgroups does not
-  // copy the token codes (up to 128 KiB each) all over again
-  else if ((a.N + 31) / 32 > cus) {
-    a.groups = 4;
-  }
-  const int tg = (a.M + 15) / 16;
-  const unsigned grid = (unsigned)((a.N + GM_ROWS * a.groups - 1) / (GM_ROWS * a.groups));
-  const size_t lds = (size_t)16 * tg * (a.K + 16) + 16;
-  const bool res = a.res != nullptr;
-  using kern_t = void (*)(GemvArgs);
-  static const kern_t table[2][3][2] = {
-      {{gemv_mfma_tokens_kernel<2, false>, gemv_mfma_tokens_kernel<2, true>},
-       {gemv_mfma_tokens_kernel<3, false>, gemv_mfma_tokens_kernel<3, true>},
-       {gemv_mfma_tokens_kernel<4, false>, gemv_mfma_tokens_kernel<4, true>}},
-      {{gemv_mfma_tokens_kernel<2, false, true>, gemv_mfma_tokens_kernel<2, true, true>},
-       {gemv_mfma_tokens_kernel<3, false, true>, gemv_mfma_tokens_kernel<3, true, true>},
-       {gemv_mfma_tokens_kernel<4, false, true>, gemv_mfma_tokens_kernel<4, true, true>}}};
-  const kern_t fn = table[fp8][tg - 2][res];
-  if (lds > 64 * 1024) {
-    static LdsOptIn opted[12];
-    const int e = opted[fp8 * 6 + (tg - 2) * 2 + res].ensure(reinterpret_cast<const void*>(fn));
-    if (e) return e;
-  }
-  hipLaunchKernelGGL(fn, dim3(grid), dim3(a.ksplit * a.groups * 64), lds, st, a);
-  return (int)hipGetLastError();
+int launch_gemv_tokens(const GemvArgs& a, hipStream_t st, bool fp8) {
+  const int tg = a.M > 48 ? 4 : a.M > 32 ? 3 : 2;
+  const bool wide = (a.N + 31) / 32 > device_cus();
+#define AQ_TOKENS(KS, GRP)                                                        \
+  (tg == 4 ? launch_gemv_tokens_shape<4, KS, GRP>(a, st, fp8)                     \
+           : tg == 3 ? launch_gemv_tokens_shape<3, KS, GRP>(a, st, fp8) : launch_gemv_tokens_shape<2, KS, GRP>(a, st, fp8))
+#define AQ_TOKENS23(KS, GRP) \
+  (tg == 3 ? launch_gemv_tokens_shape<3, KS, GRP>(a, st, fp8) : launch_gemv_tokens_shape<2, KS, GRP>(a, st, fp8))
+  if (a.K <= 1024) return (wide || tg == 4) ? AQ_TOKENS(1, 4) : AQ_TOKENS23(1, 2);
+  if (wide) return tg == 4 ? launch_gemv_tokens_shape<4, 1, 4>(a, st, fp8) : AQ_TOKENS23(2, 4);
+  if (tg == 2 && a.K >= 4096) return launch_gemv_tokens_shape<2, 4, 2>(a, st, fp8);
+  return AQ_TOKENS(2, 2);
+#undef AQ_TOKENS
+#undef AQ_TOKENS23
 }
-
-// the FP8 Linear's share of these shapes: 17..64 rows whose codes fit LDS (no chunked variant)
-bool gemv_tokens_fp8_ok(int64_t M, int64_t N, int64_t K) { return M > 16 && M <= 64 && N > 0 && gemv_tokens_fit(M, K); }
 
 int gemv_tokens_launch(const int8_t* xq, const float* sx, const int8_t* wq, const float* sw, const void* bias,
                        int bias_dtype, const void* residual, void* y, int y_dtype, int64_t M, int64_t N, int64_t K,

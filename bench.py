@@ -258,13 +258,14 @@ def bench_prefill(torch, ops, args, dev):
 
 def bench_few_dozen_rows(torch, ops, args, dev):
     """The same Linear (configuration 2's weight, N = 8192, K = 2048) at batch sizes between the reference's default
-    decode batch (16) and a prefill: row quantiser + the Linear on codes, which runs these on the weight-streaming
-    kernel (a tiled GEMM has 64 tiles here and takes 12.6-13.3 us).  us per step, HIP-graph replay over 40 weights."""
+    decode batch (16) and a prefill: row quantiser + the Linear on codes, which runs up to 32 rows on the
+    weight-streaming kernel and the rest on 128 x 32 or 128 x 64 tiles (128 x 128 tiles: 64 of them here, 9.4 us
+    whatever M).  us per step, HIP-graph replay over 40 weights."""
     N, K, nbuf = 8192, 2048, 40
     weights = make_weights(torch, ops, N, K, nbuf, dev, seed=21, mode="int8")
     g = torch.Generator(device=dev).manual_seed(22)
     out = {"workload": f"linear_w8a8 K={K} N={N}, bf16 rows -> int8 per token, bf16 out; quantiser + Linear on codes"}
-    for M in (32, 64):
+    for M in (32, 64, 128, 256):
         x = torch.randn(M, K, generator=g, device=dev).to(torch.bfloat16)
 
         def step(i, x=x):
@@ -783,7 +784,7 @@ def main():
                     a2.m = m
                     r = bench_decode(torch, ops, a2, dev)
                     extra[f"decode_m{m}"] = r
-                extra["batch_32_to_64"] = bench_few_dozen_rows(torch, ops, args, dev)
+                extra["batch_32_to_256"] = bench_few_dozen_rows(torch, ops, args, dev)
         ceilings = measure_ceilings(torch, ops, dev, calibrate=not args.no_extra)
         if not args.no_extra and args.workload != "model":
             # the reference's own generation benchmark: about a minute; skipped when this run is already long

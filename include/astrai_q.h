@@ -90,9 +90,9 @@ int aq_gemm_i8_i32(const int8_t *xq, const int8_t *wq, int32_t *acc, int64_t M, 
  * fp32, then one round-to-nearest-even cast to y_dtype.  Replaces the whole
  * F.linear(x, weight, bias) of linear.py:21 for M > 16.
  * bias may be NULL (the reference never constructs a Linear with bias=True).
- * Any M: a tiled matrix-core GEMM, except that a few dozen rows (17..64, K a multiple of 128) run on
- * the weight-streaming kernel of the decode path instead -- the tiles would leave most of the device
- * idle -- with the same bits. */
+ * Any M: a tiled matrix-core GEMM whose tile is chosen by shape (128 x 32 up to 256 x 128), except
+ * that 17..32 rows (K a multiple of 128) run on the weight-streaming kernel of the decode path
+ * instead, with the same bits. */
 int aq_linear_w8a8(const int8_t *xq, const float *sx, const int8_t *wq, const float *sw,
                    const void *bias, int bias_dtype, void *y, int y_dtype, int64_t M,
                    int64_t N, int64_t K, void *stream);

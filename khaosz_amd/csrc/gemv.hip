@@ -891,11 +891,12 @@ static int launch_gemv_mfma_swiglu(GemvArgs a, hipStream_t st) {
 }
 
 // ---------------------------------------------------------------------------
-// 17..64 tokens on codes: the same weight stream (every weight byte HBM -> registers once, operands assembled by
-// one DPP rotation per dword) with TG groups of 16 tokens multiplied against each weight fragment.  Between the
-// decode batch sizes above and a prefill, the tiled GEMM has too few tiles to occupy the device (32 x 8192 x 2048:
-// 64 tiles of 128 x 128, 9.3 us); this kernel keeps it a bandwidth-bound launch (5.2 us).  Same integer sums, same
-// epilogue: the bits of the tiled GEMM.
+// 17..32 tokens on codes: the same weight stream (every weight byte HBM -> registers once, operands assembled by
+// one DPP rotation per dword) with TG = 2 groups of 16 tokens multiplied against each weight fragment.  Between the
+// decode batch sizes above and the tiled GEMM (whose smallest tile, 128 x 32, spends the matrix-core time of 128
+// rows whatever M is: 32 x 8192 x 2048 in 5.9 us) this kernel stays a bandwidth-bound launch (5.2 us); from 33
+// tokens on, with a third and fourth token group, it was the slower one (48 rows: 6.1 us, 64 rows: 7.6 us against
+// 5.8 us), so those go to the tiles.  Same integer sums, same epilogue: the bits of the tiled GEMM.
 // K is walked in chunks of 1024 bytes per wavefront (KS wavefronts per row group: 1024-, 2048- or 4096-byte chunks
 // per workgroup), the token codes of one chunk at a time in LDS, so that rows of any length are taken (an MLP's
 // down projection) and the LDS of a compute unit holds several workgroups.  A chunk's codes are requested into
@@ -1091,11 +1092,11 @@ __global__ __launch_bounds__(KS * GRP * 64) void gemv_mfma_tokens_kernel(GemvArg
   }
 }
 
-// Shapes the token-group kernel takes: 17..64 rows of whole 128-byte lines, and the decode batch sizes whose rows
+// Shapes the token-group kernel takes: 17..32 rows of whole 128-byte lines, and the decode batch sizes whose rows
 // are too long for the GEMV kernels' own LDS budget (9..16 rows beyond 10 096 bytes, 5..8 beyond 20 208, ...),
 // where the tiles were the only path (12 x 4096 x 11008: 41 us against 19 us).  int8 and FP8 codes alike.
 bool gemv_tokens_ok(int64_t M, int64_t N, int64_t K) {
-  if (M < 1 || M > 64 || N <= 0 || (K % 128) != 0 || K > (1 << 22)) return false;
+  if (M < 1 || M > 32 || N <= 0 || (K % 128) != 0 || K > (1 << 22)) return false;
   if (M <= 16) {
     const int64_t mt = M <= 1 ? 1 : M <= 2 ? 2 : M <= 4 ? 4 : M <= 8 ? 8 : 16;
     return mt * K + 64 + 2048 > GV_MAX_LDS;  // the GEMV kernels' own limit (gemv_check)
@@ -1103,8 +1104,9 @@ bool gemv_tokens_ok(int64_t M, int64_t N, int64_t K) {
   return true;
 }
 
-template <int TG, int KS, int GRP>
+template <int KS, int GRP>
 static int launch_gemv_tokens_shape(const GemvArgs& a, hipStream_t st, bool fp8) {
+  constexpr int TG = 2;
   const unsigned grid = (unsigned)((a.N + GRP * GM_ROWS - 1) / (GRP * GM_ROWS));
   const size_t lds = (size_t)16 * TG * (1024 * KS + 16) + 16;
   using kern_t = void (*)(GemvArgs);
@@ -1117,32 +1119,21 @@ static int launch_gemv_tokens_shape(const GemvArgs& a, hipStream_t st, bool fp8)
   return (int)hipGetLastError();
 }
 
-// Chunk and workgroup shapes, from timings of 17..64 rows over N = 256..16384, K = 512..4096 (the tiles take 9.3 us
-// at K = 2048 whatever N up to 16384, 13.7 us at K = 4096):
+// Chunk and workgroup shapes, from timings of 17..32 rows over N = 256..16384, K = 512..4096:
 //   * chunks no longer than the rows, or wavefronts idle: 1024 bytes up to K = 1024, else 2048; 4096 over 8
-//     wavefronts for up to 32 tokens and K >= 4096 while every compute unit gets at most one workgroup
-//     (32 x 6144 x 4096: 7.5 us against 8.5 us);
+//     wavefronts for K >= 4096 while every compute unit gets at most one workgroup (32 x 6144 x 4096: 7.5 us
+//     against 8.5 us), on 16 rows per workgroup while that still gives no compute unit a second one (32 x 2048 x
+//     5632: 9.5 us against 11.1 us; x 11008: 13.4 us against 16.6 us);
 //   * 32 rows per workgroup while there are no more 32-row blocks than compute units (32 x 8192 x 2048: 5.2 us, 64
-//     rows 6.8 us), 64 rows beyond (48 x 16384 x 2048: 7.9 us against 11.3 us: half the copies of the token codes),
-//     with 1024-byte chunks for 49..64 tokens, whose 2048-byte chunks leave LDS for one workgroup per compute unit
-//     (64 x 16384 x 2048: 9.8 us against 13.0 us);
-//   * short rows (K <= 1024): 64 rows per workgroup also for 49..64 tokens (64 x 4096 x 1024: 5.6 us against 6.1 us).
+//     rows 6.8 us), 64 rows beyond (32 x 16384 x 2048: 7.0 us against 7.4 us: half the copies of the token codes).
 // (gemv_tokens_ok and gemv_tokens_launch are not static: the tiled GEMM's entry points in gemm_mfma.hip hand these
 // shapes over)
 int launch_gemv_tokens(const GemvArgs& a, hipStream_t st, bool fp8) {
-  const int tg = a.M > 48 ? 4 : a.M > 32 ? 3 : 2;
   const bool wide = (a.N + 31) / 32 > device_cus();
-#define AQ_TOKENS(KS, GRP)                                                        \
-  (tg == 4 ? launch_gemv_tokens_shape<4, KS, GRP>(a, st, fp8)                     \
-           : tg == 3 ? launch_gemv_tokens_shape<3, KS, GRP>(a, st, fp8) : launch_gemv_tokens_shape<2, KS, GRP>(a, st, fp8))
-#define AQ_TOKENS23(KS, GRP) \
-  (tg == 3 ? launch_gemv_tokens_shape<3, KS, GRP>(a, st, fp8) : launch_gemv_tokens_shape<2, KS, GRP>(a, st, fp8))
-  if (a.K <= 1024) return (wide || tg == 4) ? AQ_TOKENS(1, 4) : AQ_TOKENS23(1, 2);
-  if (wide) return tg == 4 ? launch_gemv_tokens_shape<4, 1, 4>(a, st, fp8) : AQ_TOKENS23(2, 4);
-  if (tg == 2 && a.K >= 4096) return launch_gemv_tokens_shape<2, 4, 2>(a, st, fp8);
-  return AQ_TOKENS(2, 2);
-#undef AQ_TOKENS
-#undef AQ_TOKENS23
+  if (a.K <= 1024) return wide ? launch_gemv_tokens_shape<1, 4>(a, st, fp8) : launch_gemv_tokens_shape<1, 2>(a, st, fp8);
+  if (wide) return launch_gemv_tokens_shape<2, 4>(a, st, fp8);
+  if (a.K >= 4096) return (a.N + 15) / 16 <= device_cus() ? launch_gemv_tokens_shape<4, 1>(a, st, fp8) : launch_gemv_tokens_shape<4, 2>(a, st, fp8);
+  return launch_gemv_tokens_shape<2, 2>(a, st, fp8);
 }
 
 int gemv_tokens_launch(const int8_t* xq, const float* sx, const int8_t* wq, const float* sw, const void* bias,

@@ -211,7 +211,7 @@ GEMM_SHAPES = [(1, 1, 16), (37, 91, 48), (17, 5, 2048), (256, 128, 128), (257, 1
                (512, 384, 5632), (1000, 520, 1024)]
 
 
-@pytest.fixture(params=[128, 256])
+@pytest.fixture(params=[32, 64, 128, 256])
 def tile(request):
     """Run a GEMM test once per workgroup tile shape (the library would pick one by shape)."""
     with _abi.lab_library() as lab:  # the lab build of the same sources: its tile can be forced
@@ -462,14 +462,15 @@ def test_up_gate_gemv_with_the_activation_refuses_what_it_does_not_serve():
 
 @pytest.mark.parametrize("M", [17, 31, 32, 33, 48, 50, 64])
 @pytest.mark.parametrize("N,K", [(8192, 2048), (200, 256), (77, 1536), (2048, 2304), (3072, 4096), (130, 9984),
-                                 (2048, 5632), (8200, 6912), (77, 11008), (40, 128), (12000, 4224), (8400, 1024)])
-def test_a_few_dozen_rows_take_the_weight_streaming_kernel_same_bits_as_the_oracle(oracle, M, N, K):
-    """17..64 rows are too few for the tiled GEMM to fill the device: the Linear on codes hands them to the
-    weight-streaming matrix-core kernel with 2..4 groups of 16 tokens, which walks rows of any length (whole
-    128-byte lines) in chunks: 1024-byte chunks for short rows, 2048 otherwise, 4096 for up to 32 tokens and
-    K >= 4096; 32 rows per workgroup, 64 for matrices of more 32-row blocks than compute units; ragged last
-    chunks, rows shorter than a chunk.  int32 sums and the frozen epilogue: bit for bit against the oracle,
-    bf16 and fp32 outputs, with bias and residual, odd N."""
+                                 (2048, 5632), (8200, 6912), (77, 11008), (40, 128), (12000, 4224), (8400, 1024),
+                                 (4200, 4224)])
+def test_a_few_dozen_rows_same_bits_as_the_oracle(oracle, M, N, K):
+    """17..32 rows: the Linear on codes hands them to the weight-streaming matrix-core kernel with 2 groups of
+    16 tokens, which walks rows of any length (whole 128-byte lines) in chunks: 1024-byte chunks for short rows,
+    2048 otherwise, 4096 for K >= 4096; 16, 32 or 64 rows per workgroup by the number of row blocks against the
+    compute units; ragged last chunks, rows shorter than a chunk.  33..64 rows: the tiled GEMM, whose tile
+    narrows to 128 x 64 or 128 x 32 for so few rows.  int32 sums and the frozen epilogue: bit for bit against the
+    oracle, bf16 and fp32 outputs, with bias and residual, odd N."""
     _say("linear, few dozen rows", M, N, K)
     x = make_x(M, K, 50 + M).to(torch.bfloat16)
     w = make_x(N, K, 51) * 0.02
@@ -741,11 +742,11 @@ def test_linear_fp8_within_tolerance(oracle, tile, M, N, K):
 
 @pytest.mark.parametrize("M", [17, 32, 33, 50, 64])
 @pytest.mark.parametrize("N,K", [(8192, 2048), (77, 512), (3072, 1536), (200, 256), (8400, 2304), (130, 4096),
-                                 (8400, 1024), (300, 5632)])
-def test_linear_fp8_a_few_dozen_rows_take_the_weight_streaming_kernel(oracle, M, N, K):
-    """17..64 rows of FP8 codes (whole 128-byte lines) go to the weight-streaming kernel (one 16x16x128 product
+                                 (8400, 1024), (300, 5632), (4200, 4224)])
+def test_linear_fp8_a_few_dozen_rows(oracle, M, N, K):
+    """17..32 rows of FP8 codes (whole 128-byte lines) go to the weight-streaming kernel (one 16x16x128 product
     per 128-byte line and token group, fp32 sums, chunks and K parts added in a fixed order), in every chunk and
-    workgroup shape of its dispatch.  Against the float64 sum of the oracle's codes inside the stated
+    workgroup shape of its dispatch; 33..64 rows to the narrow tiles.  Against the float64 sum of the oracle's codes inside the stated
     tolerance, against the tiled GEMM on the same codes (a forced tile shape keeps it on the tiles) within the
     change of summation order, with bias and residual, and the same bits on a second call."""
     _say("linear_fp8, few dozen rows", M, N, K)

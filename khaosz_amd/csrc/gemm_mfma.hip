@@ -9,9 +9,9 @@
 // materialised.  A workgroup of 8 wavefronts (two per SIMD) owns a 256 x 128
 // tile of C; each wavefront a 64 x 64 sub-tile held as 2 x 2 MFMA 32x32
 // accumulators.  (When that gives too few tiles to occupy the device, the
-// tile is 128 x 128, 128 x 64 or 128 x 32 instead and the two wavefronts that
-// share a sub-tile each take half of every K step; their accumulators are
-// summed through LDS at the end.)  K is walked in 128-byte steps through three (four) LDS stages that
+// tile is 128 x 128, 128 x 64, 128 x 32, 64 x 64 or 64 x 32 instead and the
+// two wavefronts that share a sub-tile each take half of every K step; their
+// accumulators are summed through LDS at the end.)  K is walked in 128-byte steps through three (four) LDS stages that
 // are filled by direct global->LDS loads (no register staging), with an XOR
 // permutation of 16-byte pieces that makes the fragment reads bank-conflict
 // free; the loop is software-pipelined so that LDS reads and global loads of
@@ -30,13 +30,15 @@ namespace aq {
 //   <2, 2, 2, 2, 2, 128, 4>  128 x 128 tile, 8 wavefronts: the two that share a 64 x 64 sub-tile split every
 //                            K step and exchange half of their accumulators through LDS at the end, so that
 //                            each finishes (and stores) 32 x 64 of the sums; 4 stages of 32 KiB;
-//   <2, 1, 2, 2, 2, 128, 4>  128 x 64 tile and
-//   <2, 1, 2, 1, 2, 128, 4>  128 x 32 tile, 4 wavefronts as two K-split pairs: for a few hundred rows, where wider
-//                            tiles leave most compute units without one.  A workgroup's time is the matrix-core
-//                            time of its whole tile, rows past M included (128 x 128 x 2048: 16 K steps of 16
-//                            MFMAs, 3.9 us per compute unit), so with tiles to spare the narrower tile is the
-//                            faster launch (128 x 2048 x 2048: 9.6 us on 16 tiles of 128 x 128, 5.6 us on 64 of
-//                            128 x 32);
+//   <2, 1, 2, 2, 2, 128, 4>  128 x 64 tile,
+//   <2, 1, 2, 1, 2, 128, 4>  128 x 32 tile (4 wavefronts as two K-split pairs),
+//   <1, 2, 2, 1, 2, 128, 4>  64 x 64 tile (the same, side by side) and
+//   <1, 1, 2, 1, 2, 128, 4>  64 x 32 tile (one K-split pair): for a few hundred rows, where wider tiles leave
+//                            most compute units without one.  A workgroup's time is the matrix-core time of its
+//                            whole tile, rows past M included (128 x 128 x 2048: 16 K steps of 16 MFMAs, 3.9 us
+//                            per compute unit), so with tiles to spare the smaller tile is the faster launch
+//                            (128 x 2048 x 2048, weights from HBM: 12.4 us on 16 tiles of 128 x 128, 8.7 us on 64
+//                            of 128 x 32, 7.0 us on 128 of 64 x 32);
 // Shapes that only the lab build instantiates.  Measured, none faster on int8 with real operand data: under a
 // matrix-core load with toggling operands this part runs against its power limit, and fewer LDS reads per MFMA
 // buy clock, not rate (8192^3: 2.31-2.42 POP/s for every shape below and for the 256 x 128 tile alike, while the
@@ -76,6 +78,8 @@ using ShapeLarge = Shape<4, 2, 2, 2, 1, 128, 3>;
 using ShapeSmall = Shape<2, 2, 2, 2, 2, 128, 4>;
 using ShapeN64 = Shape<2, 1, 2, 2, 2, 128, 4>;
 using ShapeN32 = Shape<2, 1, 2, 1, 2, 128, 4>;
+using ShapeM64N64 = Shape<1, 2, 2, 1, 2, 128, 4>;
+using ShapeM64N32 = Shape<1, 1, 2, 1, 2, 128, 4>;
 #ifdef AQ_LAB
 using ShapeHuge = Shape<2, 2, 4, 4, 1, 64, 4>;
 using ShapeTall = Shape<2, 2, 4, 2, 1, 128, 3>;
@@ -805,19 +809,20 @@ __global__ __launch_bounds__(S::NTHREADS) void gemm_kernel(GemmArgs p) {
   }
 }
 
-// Tile shape by the number of rounds over the compute units a launch needs: a workgroup per
-// compute unit at a time, so the cost of a launch is its number of rounds times the cost of a round of that
-// shape.  Measured: a round of 128 x 128 tiles costs 0.72 of a round of 256 x 128 ones, of 128 x 64 tiles 0.42, of
-// 128 x 32 tiles 0.30, and a last round that fills only part of the device costs about half a round plus half its
-// fill (384 large tiles, 1.5 rounds, take 1.74 times as long as 256).  Fitted on 65..1024 rows against N = 2048..
-// 11264 and K = 2048..5632, where the rule picks the fastest shape of the four or one within 6 % of it (a full
-// round of 128 x 128 tiles against half a round of 256 x 128 ones goes either way by 10-15 % from one device to
-// the next).  The
-// narrow tiles are for launches of a few rounds only (with many, their weights above are too high, and the wide
-// tiles win regardless).
+// Tile shape by the number of rounds over the compute units a launch needs: a workgroup per compute unit at a
+// time, so the cost of a launch is its number of rounds times the cost of a round of that shape (us at K = 2048
+// with the weights streamed from HBM, on top of 4 us of launch and pipeline fill; every term scales with K alike):
+//   256 x 128: 15.0   128 x 128: 10.8   128 x 64: 7.0   128 x 32: 5.0   64 x 64: 4.6   64 x 32: 3.5
+// After a full round, a last round of the two wide shapes that fills only part of the device costs about half a
+// round plus half its fill (384 large tiles, 1.5 rounds, take 1.74 times as long as 256); a first round runs at the
+// latency of its K loop whatever the fill (128 x 128: 64 tiles 12.3-14.8 us, 256 tiles 14.5 us), and so does every
+// round of the small shapes (64 x 32: 64 tiles 6.9 us, 256 tiles 7.0 us, 352 tiles 12.0 us), whose rounds count
+// whole.  Fitted on
+// 33..2048 rows against N = 1024..16384 and K = 1024..5632, where the rule picks the fastest shape or one within
+// 6 % of it.  The small tiles are for launches of a few rounds only.
 enum TileKind {
-  TILE_AUTO = 0, TILE_N32 = 32, TILE_N64 = 64, TILE_SMALL = 128, TILE_LARGE = 256, TILE_TALL = 257, TILE_HUGE = 512,
-  TILE_HUGE8 = 513
+  TILE_AUTO = 0, TILE_N32 = 32, TILE_M64N32 = 33, TILE_N64 = 64, TILE_M64N64 = 65, TILE_SMALL = 128, TILE_LARGE = 256,
+  TILE_TALL = 257, TILE_HUGE = 512, TILE_HUGE8 = 513
 };
 #ifdef AQ_LAB
 static int g_forced_tile = 0;  // lab build only: TILE_AUTO = by shape, otherwise forced (tuning and tests)
@@ -830,19 +835,28 @@ static int choose_tile(int64_t M, int64_t N) {
   const int64_t cus = device_cus();
   auto rounds = [cus](int64_t tiles) {
     const int64_t full = tiles / cus, rest = tiles % cus;
+    if (full == 0) return 1.0;
     return (double)full + (rest ? 0.5 + 0.5 * (double)rest / cus : 0.0);
   };
-  const int64_t tm = (M + 127) / 128;
-  int best = TILE_LARGE;
-  double cost = rounds((M + 255) / 256 * ((N + 127) / 128));
-  auto consider = [&](int kind, int64_t tiles, double weight, bool few_rounds_only) {
-    if (few_rounds_only && tiles > 4 * cus) return;
-    const double c = weight * rounds(tiles);
-    if (c < cost) { cost = c; best = kind; }
+  struct Cand {
+    int kind, bm, bn;
+    double round_us;
+    bool small;
   };
-  consider(TILE_SMALL, tm * ((N + 127) / 128), 0.72, false);
-  consider(TILE_N64, tm * ((N + 63) / 64), 0.42, true);
-  consider(TILE_N32, tm * ((N + 31) / 32), 0.30, true);
+  static const Cand cands[] = {{TILE_LARGE, 256, 128, 15.0, false}, {TILE_SMALL, 128, 128, 10.8, false},
+                               {TILE_N64, 128, 64, 7.0, true},      {TILE_N32, 128, 32, 5.0, true},
+                               {TILE_M64N64, 64, 64, 4.6, true},    {TILE_M64N32, 64, 32, 3.5, true}};
+  int best = TILE_LARGE;
+  double cost = 0.0;
+  for (const Cand& c : cands) {
+    const int64_t tiles = ((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn);
+    if (c.small && tiles > 4 * cus) continue;
+    const double us = c.round_us * (c.small ? (double)((tiles + cus - 1) / cus) : rounds(tiles));
+    if (c.kind == TILE_LARGE || us < cost) {
+      cost = us;
+      best = c.kind;
+    }
+  }
   return best;
 }
 
@@ -864,6 +878,8 @@ static int launch(GemmArgs& a, hipStream_t st) {
     case TILE_SMALL: return launch_shape<FP8, OUT, ShapeSmall>(a, st);
     case TILE_N64: return launch_shape<FP8, OUT, ShapeN64>(a, st);
     case TILE_N32: return launch_shape<FP8, OUT, ShapeN32>(a, st);
+    case TILE_M64N64: return launch_shape<FP8, OUT, ShapeM64N64>(a, st);
+    case TILE_M64N32: return launch_shape<FP8, OUT, ShapeM64N32>(a, st);
 #ifdef AQ_LAB
     case TILE_TALL: return launch_shape<FP8, OUT, ShapeTall>(a, st);
     case TILE_HUGE:
@@ -906,7 +922,7 @@ extern "C" int aq_lab_read_clock(long long* host2) {
   return (int)hipMemcpyFromSymbol(host2, HIP_SYMBOL(aq::aq_lab_clock), 64);
 }
 extern "C" int aq_lab_set_gemm_tile(int rows) {
-  if (rows != 0 && rows != 64 && rows != 32 && rows != 128 && rows != 256 && rows != 257 && rows != 512 && rows != 513) return AQ_E_SHAPE;
+  if (rows != 0 && rows != 33 && rows != 65 && rows != 64 && rows != 32 && rows != 128 && rows != 256 && rows != 257 && rows != 512 && rows != 513) return AQ_E_SHAPE;
   aq::g_forced_tile = rows;
   return AQ_OK;
 }

@@ -33,12 +33,14 @@ namespace aq {
 //   <2, 1, 2, 2, 2, 128, 4>  128 x 64 tile,
 //   <2, 1, 2, 1, 2, 128, 4>  128 x 32 tile (4 wavefronts as two K-split pairs),
 //   <1, 2, 2, 1, 2, 128, 4>  64 x 64 tile (the same, side by side) and
-//   <1, 1, 2, 1, 2, 128, 4>  64 x 32 tile (one K-split pair): for a few hundred rows, where wider tiles leave
-//                            most compute units without one.  A workgroup's time is the matrix-core time of its
-//                            whole tile, rows past M included (128 x 128 x 2048: 16 K steps of 16 MFMAs, 3.9 us
-//                            per compute unit), so with tiles to spare the smaller tile is the faster launch
-//                            (128 x 2048 x 2048, weights from HBM: 12.4 us on 16 tiles of 128 x 128, 8.7 us on 64
-//                            of 128 x 32, 7.0 us on 128 of 64 x 32);
+//   <1, 1, 2, 1, 2, 128, 6>  64 x 32 tile (one K-split pair; six stages of 12 KiB: 2-20 % faster than four,
+//                            while the other three were fastest with four of the 4..8 that fit): for a few
+//                            hundred rows, where wider tiles leave most compute units without one.  A
+//                            workgroup's time is the matrix-core time of its whole tile, rows past M included
+//                            (128 x 128 x 2048: 16 K steps of 16 MFMAs, 3.9 us per compute unit), so with tiles
+//                            to spare the smaller tile is the faster launch (128 x 2048 x 2048, weights from
+//                            HBM: 12.4 us on 16 tiles of 128 x 128, 8.7 us on 64 of 128 x 32, 6.9 us on 128 of
+//                            64 x 32);
 // Shapes that only the lab build instantiates.  Measured, none faster on int8 with real operand data: under a
 // matrix-core load with toggling operands this part runs against its power limit, and fewer LDS reads per MFMA
 // buy clock, not rate (8192^3: 2.31-2.42 POP/s for every shape below and for the 256 x 128 tile alike, while the
@@ -73,13 +75,14 @@ struct Shape {
   static_assert(NWAVES % 2 == 0, "the piece permutation assumes a wavefront's row groups share parity");
   static_assert((BM * BK / 1024) % NWAVES == 0 && (BN * BK / 1024) % NWAVES == 0, "whole 1 KiB loads per wavefront");
   static_assert(LDS_BYTES <= 160 * 1024, "LDS of one compute unit");
+  static_assert((NSTAGE - 1) * ((BM + BN) * BK / 16 / NTHREADS) <= 63, "the loads in flight fit the 6-bit counter");
 };
 using ShapeLarge = Shape<4, 2, 2, 2, 1, 128, 3>;
 using ShapeSmall = Shape<2, 2, 2, 2, 2, 128, 4>;
 using ShapeN64 = Shape<2, 1, 2, 2, 2, 128, 4>;
 using ShapeN32 = Shape<2, 1, 2, 1, 2, 128, 4>;
 using ShapeM64N64 = Shape<1, 2, 2, 1, 2, 128, 4>;
-using ShapeM64N32 = Shape<1, 1, 2, 1, 2, 128, 4>;
+using ShapeM64N32 = Shape<1, 1, 2, 1, 2, 128, 6>;
 #ifdef AQ_LAB
 using ShapeHuge = Shape<2, 2, 4, 4, 1, 64, 4>;
 using ShapeTall = Shape<2, 2, 4, 2, 1, 128, 3>;

@@ -180,7 +180,9 @@ int aq_gemv_w8a8_decode_swiglu(const void *x, int x_dtype, const void *gamma, fl
 /* FP8 Linear: y[m, n] = (sum_k f(xq[m,k]) * f(wq[n,k])) * sx[0] * sw[0] with
  * fp32 accumulation, cast to y_dtype.  xq: [M, K], wq: [N, K] e4m3fn codes;
  * sx, sw: device scalars written by aq_quant_tensor_fp8.  Replaces F.linear
- * (linear.py:21) in the FP8 variant. */
+ * (linear.py:21) in the FP8 variant.  Tiles chosen by shape and 17..32 rows on the
+ * weight-streaming kernel, as for aq_linear_w8a8 (the order of the fp32 sums, fixed for a
+ * given shape, differs between the kernels). */
 int aq_linear_fp8(const uint8_t *xq, const float *sx, const uint8_t *wq, const float *sw,
                   void *y, int y_dtype, int64_t M, int64_t N, int64_t K, void *stream);
 

@@ -68,6 +68,7 @@ SYMBOLS = {
 LAB_LIB_PATH = os.path.join(_HERE, "lib", "libastrai_q_lab.so")
 LAB_SYMBOLS = {
     "aq_lab_set_gemm_tile": (_int, [_int]),
+    "aq_lab_choose_gemm_tile": (_int, [_i64, _i64, _int]),
     "aq_lab_probe_mfma": (_int, [_int, _int, _int, _int, _vp, _vp, _vp]),
     "aq_lab_probe_copy": (_int, [_vp, _vp, _i64, _int, _vp]),
     "aq_lab_probe_read": (_int, [_vp, _i64, _int, _int, _int, _vp, _vp]),

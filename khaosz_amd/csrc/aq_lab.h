@@ -19,6 +19,10 @@ extern "C" {
  * unsynchronised -- which is why it does not exist in the product library. */
 int aq_lab_set_gemm_tile(int rows);
 
+/* The tile the library would pick for an M x N output on a device of `compute_units` compute units, in the
+ * numbering above (a pure function of its arguments: no device is touched). */
+int aq_lab_choose_gemm_tile(int64_t M, int64_t N, int compute_units);
+
 /* `workgroups` x 4 wavefronts each issue iters x 8 independent MFMAs.
  * kind 0 = i32_32x32x32_i8 (65536 ops each), 1 = i32_16x16x64_i8 (32768), 2 = f32_32x32x64 e4m3 (131072 flops).
  * data 0 = constant operands (no toggling: the clock stays at its maximum), 1 = random bytes, four operand

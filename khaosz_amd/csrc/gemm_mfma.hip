@@ -831,11 +831,7 @@ enum TileKind {
 static int g_forced_tile = 0;  // lab build only: TILE_AUTO = by shape, otherwise forced (tuning and tests)
 #endif
 
-static int choose_tile(int64_t M, int64_t N) {
-#ifdef AQ_LAB
-  if (g_forced_tile) return g_forced_tile;
-#endif
-  const int64_t cus = device_cus();
+static int choose_tile_for(int64_t M, int64_t N, int64_t cus) {
   auto rounds = [cus](int64_t tiles) {
     const int64_t full = tiles / cus, rest = tiles % cus;
     if (full == 0) return 1.0;
@@ -861,6 +857,13 @@ static int choose_tile(int64_t M, int64_t N) {
     }
   }
   return best;
+}
+
+static int choose_tile(int64_t M, int64_t N) {
+#ifdef AQ_LAB
+  if (g_forced_tile) return g_forced_tile;
+#endif
+  return choose_tile_for(M, N, device_cus());
 }
 
 template <bool FP8, int OUT, class S>
@@ -928,6 +931,10 @@ extern "C" int aq_lab_set_gemm_tile(int rows) {
   if (rows != 0 && rows != 33 && rows != 65 && rows != 64 && rows != 32 && rows != 128 && rows != 256 && rows != 257 && rows != 512 && rows != 513) return AQ_E_SHAPE;
   aq::g_forced_tile = rows;
   return AQ_OK;
+}
+extern "C" int aq_lab_choose_gemm_tile(int64_t M, int64_t N, int compute_units) {
+  if (M <= 0 || N <= 0 || compute_units <= 0) return AQ_E_SHAPE;
+  return aq::choose_tile_for(M, N, compute_units);
 }
 #endif
 

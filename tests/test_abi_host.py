@@ -220,3 +220,28 @@ class _RefMLP(nn.Module):
 
 def test_package_exports():
     assert {"Linear", "QuantLinear", "Fp8Linear", "quantize_model"} <= set(dir(khaosz_amd))
+
+
+def test_gemm_tile_choice_for_the_benchmark_shapes_and_a_few_hundred_rows():
+    """The tile shape is picked on the host from M, N and the number of compute units alone.  Pinned here for
+    256 compute units: the benchmark configurations keep the wide tiles (one round of 256 tiles of 256 x 128
+    for the prefill configuration, 256 tiles of 128 x 128 for the FP8 one), a few hundred rows get the small
+    tiles that still give every compute unit at most one tile, and a launch of many rounds never takes a small
+    tile."""
+    lab = _abi.load_lab()
+    pick = lambda M, N: lab.aq_lab_choose_gemm_tile(M, N, 256)
+    assert pick(4096, 2048) == 256          # configuration 3: 256 tiles of 256 x 128, one round
+    assert pick(2048, 2048) == 128          # configuration 4: 256 tiles of 128 x 128
+    assert pick(8192, 8192) == 256
+    assert pick(4096, 3072) == 256 and pick(4096, 11264) == 256   # block prefill: q/k/v, up/gate
+    assert pick(2048, 13824) == 256         # model prefill, up/gate
+    assert pick(64, 8192) == 33 and pick(48, 2048) == 33          # 64 x 32: 256 and 64 tiles
+    assert pick(128, 8192) == 65            # 64 x 64: 256 tiles (64 x 32 would need two rounds)
+    assert pick(256, 8192) == 64            # 128 x 64
+    assert pick(128, 11264) == 64 and pick(64, 11264) == 65
+    assert pick(384, 8192) == 128 and pick(512, 8192) == 128
+    assert pick(768, 8192) == 256 and pick(1024, 8192) == 256
+    assert pick(512, 2048) == 65 and pick(1024, 2048) == 64 and pick(256, 2048) == 33
+    for M, N in ((8192, 8192), (100000, 4096), (1 << 20, 1 << 20)):
+        assert pick(M, N) in (128, 256)
+    assert lab.aq_lab_choose_gemm_tile(0, 8, 256) == -2 and lab.aq_lab_choose_gemm_tile(8, 8, 0) == -2

@@ -27,14 +27,17 @@ namespace aq {
 // Shape of a workgroup: WM x WN x WK wavefronts, each accumulating a (32 TM) x (32 TN) sub-tile
 // (TM x TN MFMA 32x32 accumulators); K walked in BK-byte steps through NSTAGE LDS stages.
 //   <4, 2, 2, 2, 1, 128, 3>  256 x 128 tile, 8 wavefronts (two per SIMD) of 64 x 64, 3 stages of 48 KiB;
-//   <2, 2, 2, 2, 2, 128, 4>  128 x 128 tile, 8 wavefronts: the two that share a 64 x 64 sub-tile split every
+//   <2, 2, 2, 2, 2, 128, 3>  128 x 128 tile, 8 wavefronts: the two that share a 64 x 64 sub-tile split every
 //                            K step and exchange half of their accumulators through LDS at the end, so that
-//                            each finishes (and stores) 32 x 64 of the sums; 4 stages of 32 KiB;
+//                            each finishes (and stores) 32 x 64 of the sums; 3 stages of 32 KiB (4 and 5 fit and
+//                            were 1-5 % and 2-10 % slower on this tile's shapes: 2048 x 2048 x 2048 17.9 / 18.2-
+//                            19.2 / 20.0 us with the row quantiser in front);
 //   <2, 1, 2, 2, 2, 128, 4>  128 x 64 tile,
 //   <2, 1, 2, 1, 2, 128, 4>  128 x 32 tile (4 wavefronts as two K-split pairs),
 //   <1, 2, 2, 1, 2, 128, 4>  64 x 64 tile (the same, side by side) and
 //   <1, 1, 2, 1, 2, 128, 6>  64 x 32 tile (one K-split pair; six stages of 12 KiB: 2-20 % faster than four,
-//                            while the other three were fastest with four of the 4..8 that fit): for a few
+//                            while the other three were fastest with four of the 3..8 that fit, three costing
+//                            them 5-25 %: their K loop runs at the latency of its loads): for a few
 //                            hundred rows, where wider tiles leave most compute units without one.  A
 //                            workgroup's time is the matrix-core time of its whole tile, rows past M included
 //                            (128 x 128 x 2048: 16 K steps of 16 MFMAs, 3.9 us per compute unit), so with tiles
@@ -78,7 +81,7 @@ struct Shape {
   static_assert((NSTAGE - 1) * ((BM + BN) * BK / 16 / NTHREADS) <= 63, "the loads in flight fit the 6-bit counter");
 };
 using ShapeLarge = Shape<4, 2, 2, 2, 1, 128, 3>;
-using ShapeSmall = Shape<2, 2, 2, 2, 2, 128, 4>;
+using ShapeSmall = Shape<2, 2, 2, 2, 2, 128, 3>;
 using ShapeN64 = Shape<2, 1, 2, 2, 2, 128, 4>;
 using ShapeN32 = Shape<2, 1, 2, 1, 2, 128, 4>;
 using ShapeM64N64 = Shape<1, 2, 2, 1, 2, 128, 4>;

@@ -779,11 +779,12 @@ def test_linear_fp8_a_few_dozen_rows(oracle, M, N, K):
 
 
 @pytest.mark.parametrize("M", [1, 3, 8, 9, 16])
-@pytest.mark.parametrize("N,K", [(8192, 2048), (77, 512), (11264, 1024), (300, 4096), (130, 1040)])
+@pytest.mark.parametrize("N,K", [(8192, 2048), (77, 512), (11264, 1024), (300, 4096), (130, 1040), (200, 11008)])
 def test_gemv_fp8_decode_within_tolerance(oracle, M, N, K):
     """The FP8 Linear at decode sizes: (8192, 2048), (77, 512) and (11264, 1024) cast their bf16 rows inside the
     GEMV kernel (32- and 64-row workgroups, a ragged single workgroup); (300, 4096) goes through the workspace
-    (quantiser + GEMV on codes); (130, 1040) is handed to the tiled GEMM.  All against the float64 sum of the
+    (quantiser + GEMV on codes); (130, 1040) is handed to the tiled GEMM; rows of 11008 codes are too long for the
+    GEMV's LDS and go to the Linear on codes (its weight-streaming kernel from 9 rows on).  All against the float64 sum of the
     oracle's codes, and the fused cast against the codes path (a wrong code would move an output by far more
     than a change of summation order)."""
     _say("gemv_fp8", M, N, K)

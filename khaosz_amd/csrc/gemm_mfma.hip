@@ -956,7 +956,7 @@ extern "C" int aq_linear_w8a8(const int8_t* xq, const float* sx, const int8_t* w
 }
 
 namespace aq {
-// gemv.hip: the weight-streaming kernel for 17..64 rows (same sums, same epilogue: same bits)
+// gemv.hip: the weight-streaming kernel for 17..32 rows (same sums, same epilogue: same bits)
 bool gemv_tokens_ok(int64_t M, int64_t N, int64_t K);
 int gemv_tokens_launch(const int8_t* xq, const float* sx, const int8_t* wq, const float* sw, const void* bias,
                        int bias_dtype, const void* residual, void* y, int y_dtype, int64_t M, int64_t N, int64_t K,

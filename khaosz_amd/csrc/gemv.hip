@@ -893,10 +893,11 @@ static int launch_gemv_mfma_swiglu(GemvArgs a, hipStream_t st) {
 // ---------------------------------------------------------------------------
 // 17..32 tokens on codes: the same weight stream (every weight byte HBM -> registers once, operands assembled by
 // one DPP rotation per dword) with TG = 2 groups of 16 tokens multiplied against each weight fragment.  Between the
-// decode batch sizes above and the tiled GEMM (whose smallest tile, 128 x 32, spends the matrix-core time of 128
-// rows whatever M is: 32 x 8192 x 2048 in 5.9 us) this kernel stays a bandwidth-bound launch (5.2 us); from 33
-// tokens on, with a third and fourth token group, it was the slower one (48 rows: 6.1 us, 64 rows: 7.6 us against
-// 5.8 us), so those go to the tiles.  Same integer sums, same epilogue: the bits of the tiled GEMM.
+// decode batch sizes above and the tiled GEMM (whose smallest tile, 64 x 32, spends the matrix-core time of 64
+// rows whatever M is: 32 x 8192 x 2048 in 6.9 us with the weights streamed from HBM) this kernel stays a
+// bandwidth-bound launch (6.0 us); from 33 tokens on, with a third and fourth token group, it was the slower one
+// (48 rows: 6.1 us, 64 rows: 7.6 us with the weights in the last-level cache, where a 128 x 32 tile took 5.8 us),
+// so those go to the tiles.  Same integer sums, same epilogue: the bits of the tiled GEMM.
 // K is walked in chunks of 1024 bytes per wavefront (KS wavefronts per row group: 1024-, 2048- or 4096-byte chunks
 // per workgroup), the token codes of one chunk at a time in LDS, so that rows of any length are taken (an MLP's
 // down projection) and the LDS of a compute unit holds several workgroups.  A chunk's codes are requested into

@@ -14,8 +14,8 @@ extern "C" {
 #endif
 
 /* Forces the GEMM workgroup tile for every later GEMM call of this process through the lab
- * library: 32 (128 x 32), 33 (64 x 32), 64 (128 x 64), 65 (64 x 64), 128 (128 x 128; all five with a split
- * K step), 256 (256 x 128), 0 = by shape.  Process-wide and
+ * library: 32 (128 x 32), 33 (64 x 32), 64 (128 x 64), 65 (64 x 64), 128 (128 x 128), 129 (128 x 128 on
+ * wavefront pairs that split every K step: lab build only), 256 (256 x 128), 0 = by shape.  Process-wide and
  * unsynchronised -- which is why it does not exist in the product library. */
 int aq_lab_set_gemm_tile(int rows);
 

@@ -9,10 +9,9 @@
 // materialised.  A workgroup of 8 wavefronts (two per SIMD) owns a 256 x 128
 // tile of C; each wavefront a 64 x 64 sub-tile held as 2 x 2 MFMA 32x32
 // accumulators.  (When that gives too few tiles to occupy the device, the
-// tile is 128 x 128, 128 x 64, 128 x 32, 64 x 64 or 64 x 32 instead and the
-// two wavefronts that share a sub-tile each take half of every K step; their
-// accumulators are summed through LDS at the end.)  K is walked in 128-byte steps through three (four) LDS stages that
-// are filled by direct global->LDS loads (no register staging), with an XOR
+// tile is 128 x 128, 128 x 64, 128 x 32, 64 x 64 or 64 x 32 instead, on four or
+// two wavefronts.)  K is walked in 128-byte steps through three to six LDS
+// stages that are filled by direct global->LDS loads (no register staging), with an XOR
 // permutation of 16-byte pieces that makes the fragment reads bank-conflict
 // free; the loop is software-pipelined so that LDS reads and global loads of
 // later sub-steps are issued between the MFMAs of the current one, with one
@@ -27,15 +26,12 @@ namespace aq {
 // Shape of a workgroup: WM x WN x WK wavefronts, each accumulating a (32 TM) x (32 TN) sub-tile
 // (TM x TN MFMA 32x32 accumulators); K walked in BK-byte steps through NSTAGE LDS stages.
 //   <4, 2, 2, 2, 1, 128, 3>  256 x 128 tile, 8 wavefronts (two per SIMD) of 64 x 64, 3 stages of 48 KiB;
-//   <2, 2, 2, 2, 2, 128, 3>  128 x 128 tile, 8 wavefronts: the two that share a 64 x 64 sub-tile split every
-//                            K step and exchange half of their accumulators through LDS at the end, so that
-//                            each finishes (and stores) 32 x 64 of the sums; 3 stages of 32 KiB (4 and 5 fit and
-//                            were 1-5 % and 2-10 % slower on this tile's shapes: 2048 x 2048 x 2048 17.9 / 18.2-
-//                            19.2 / 20.0 us with the row quantiser in front);
-//   <2, 1, 2, 2, 2, 128, 4>  128 x 64 tile,
-//   <2, 1, 2, 1, 2, 128, 4>  128 x 32 tile (4 wavefronts as two K-split pairs),
-//   <1, 2, 2, 1, 2, 128, 4>  64 x 64 tile (the same, side by side) and
-//   <1, 1, 2, 1, 2, 128, 6>  64 x 32 tile (one K-split pair; six stages of 12 KiB: 2-20 % faster than four,
+//   <2, 2, 2, 2, 1, 128, 3>  128 x 128 tile, 4 wavefronts (one per SIMD) of 64 x 64, 3 stages of 32 KiB (4 fit
+//                            and were 1-5 % slower on this tile's shapes);
+//   <2, 2, 2, 1, 1, 128, 4>  128 x 64 tile, 4 wavefronts of 64 x 32,
+//   <4, 1, 1, 1, 1, 128, 4>  128 x 32 tile, 4 wavefronts of 32 x 32,
+//   <2, 2, 1, 1, 1, 128, 4>  64 x 64 tile, 4 wavefronts of 32 x 32, and
+//   <2, 1, 1, 1, 1, 128, 6>  64 x 32 tile, 2 wavefronts of 32 x 32 (six stages of 12 KiB: 2-20 % faster than four,
 //                            while the other three were fastest with four of the 3..8 that fit, three costing
 //                            them 5-25 %: their K loop runs at the latency of its loads): for a few
 //                            hundred rows, where wider tiles leave most compute units without one.  A
@@ -44,6 +40,12 @@ namespace aq {
 //                            to spare the smaller tile is the faster launch (128 x 2048 x 2048, weights from
 //                            HBM: 12.4 us on 16 tiles of 128 x 128, 8.7 us on 64 of 128 x 32, 6.9 us on 128 of
 //                            64 x 32);
+// The same five tiles on twice the wavefronts, the two that share a sub-tile each taking half of every K step
+// and exchanging half of their accumulators through LDS at the end (WK = 2, so that each finishes and stores
+// half of the sub-tile), were measured against these in one process over 48..512 rows and four weight shapes:
+// 2-6 % slower every time (128 x 128 at 512 x 8192 x 2048: 15.0 against 14.1 us; 64 x 64 at 128 x 8192 x 2048:
+// 8.8 against 8.4 us).  The lab build keeps the 128 x 128 one (<2, 2, 2, 2, 2, 128, 3>) so that the K-split
+// code stays compiled and tested.
 // Shapes that only the lab build instantiates.  Measured, none faster on int8 with real operand data: under a
 // matrix-core load with toggling operands this part runs against its power limit, and fewer LDS reads per MFMA
 // buy clock, not rate (8192^3: 2.31-2.42 POP/s for every shape below and for the 256 x 128 tile alike, while the
@@ -81,15 +83,16 @@ struct Shape {
   static_assert((NSTAGE - 1) * ((BM + BN) * BK / 16 / NTHREADS) <= 63, "the loads in flight fit the 6-bit counter");
 };
 using ShapeLarge = Shape<4, 2, 2, 2, 1, 128, 3>;
-using ShapeSmall = Shape<2, 2, 2, 2, 2, 128, 3>;
-using ShapeN64 = Shape<2, 1, 2, 2, 2, 128, 4>;
-using ShapeN32 = Shape<2, 1, 2, 1, 2, 128, 4>;
-using ShapeM64N64 = Shape<1, 2, 2, 1, 2, 128, 4>;
-using ShapeM64N32 = Shape<1, 1, 2, 1, 2, 128, 6>;
+using ShapeSmall = Shape<2, 2, 2, 2, 1, 128, 3>;
+using ShapeN64 = Shape<2, 2, 2, 1, 1, 128, 4>;
+using ShapeN32 = Shape<4, 1, 1, 1, 1, 128, 4>;
+using ShapeM64N64 = Shape<2, 2, 1, 1, 1, 128, 4>;
+using ShapeM64N32 = Shape<2, 1, 1, 1, 1, 128, 6>;
 #ifdef AQ_LAB
 using ShapeHuge = Shape<2, 2, 4, 4, 1, 64, 4>;
 using ShapeTall = Shape<2, 2, 4, 2, 1, 128, 3>;
 using ShapeHuge8 = Shape<4, 2, 2, 4, 1, 64, 4>;
+using ShapePair = Shape<2, 2, 2, 2, 2, 128, 3>;
 #endif
 constexpr int NUM_XCD = 8;
 constexpr int GROUP_M = 4;
@@ -827,8 +830,8 @@ __global__ __launch_bounds__(S::NTHREADS) void gemm_kernel(GemmArgs p) {
 // 33..2048 rows against N = 1024..16384 and K = 1024..5632, where the rule picks the fastest shape or one within
 // 6 % of it.  The small tiles are for launches of a few rounds only.
 enum TileKind {
-  TILE_AUTO = 0, TILE_N32 = 32, TILE_M64N32 = 33, TILE_N64 = 64, TILE_M64N64 = 65, TILE_SMALL = 128, TILE_LARGE = 256,
-  TILE_TALL = 257, TILE_HUGE = 512, TILE_HUGE8 = 513
+  TILE_AUTO = 0, TILE_N32 = 32, TILE_M64N32 = 33, TILE_N64 = 64, TILE_M64N64 = 65, TILE_SMALL = 128, TILE_PAIR = 129,
+  TILE_LARGE = 256, TILE_TALL = 257, TILE_HUGE = 512, TILE_HUGE8 = 513
 };
 #ifdef AQ_LAB
 static int g_forced_tile = 0;  // lab build only: TILE_AUTO = by shape, otherwise forced (tuning and tests)
@@ -896,6 +899,7 @@ static int launch(GemmArgs& a, hipStream_t st) {
         return launch_shape<FP8, OUT, ShapeHuge>(a, st);
       return launch_shape<FP8, OUT, ShapeLarge>(a, st);
     case TILE_HUGE8: return launch_shape<FP8, OUT, ShapeHuge8>(a, st);
+    case TILE_PAIR: return launch_shape<FP8, OUT, ShapePair>(a, st);
 #endif
     default: return launch_shape<FP8, OUT, ShapeLarge>(a, st);
   }
@@ -931,7 +935,7 @@ extern "C" int aq_lab_read_clock(long long* host2) {
   return (int)hipMemcpyFromSymbol(host2, HIP_SYMBOL(aq::aq_lab_clock), 64);
 }
 extern "C" int aq_lab_set_gemm_tile(int rows) {
-  if (rows != 0 && rows != 33 && rows != 65 && rows != 64 && rows != 32 && rows != 128 && rows != 256 && rows != 257 && rows != 512 && rows != 513) return AQ_E_SHAPE;
+  if (rows != 0 && rows != 129 && rows != 33 && rows != 65 && rows != 64 && rows != 32 && rows != 128 && rows != 256 && rows != 257 && rows != 512 && rows != 513) return AQ_E_SHAPE;
   aq::g_forced_tile = rows;
   return AQ_OK;
 }

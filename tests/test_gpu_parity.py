@@ -211,7 +211,7 @@ GEMM_SHAPES = [(1, 1, 16), (37, 91, 48), (17, 5, 2048), (256, 128, 128), (257, 1
                (512, 384, 5632), (1000, 520, 1024)]
 
 
-@pytest.fixture(params=[32, 33, 64, 65, 128, 256])
+@pytest.fixture(params=[32, 33, 64, 65, 128, 129, 256])
 def tile(request):
     """Run a GEMM test once per workgroup tile shape (the library would pick one by shape)."""
     with _abi.lab_library() as lab:  # the lab build of the same sources: its tile can be forced

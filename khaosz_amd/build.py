@@ -2,7 +2,7 @@
 
   khaosz_amd/lib/libastrai_q.so      the product: the C ABI declared in include/astrai_q.h, nothing else;
   khaosz_amd/lib/libastrai_q_lab.so  the same objects plus the measurement probes and the tile-forcing hook
-                                     of csrc/aq_lab.h (the GEMM source rebuilt with -DAQ_LAB), for the
+                                     of csrc/aq_lab.h (the GEMM and GEMV sources rebuilt with -DAQ_LAB), for the
                                      benchmark's ceilings and for tests that pin a tile shape.
 
 hipcc cross-compiles without a GPU.  Both depend on the HIP runtime only (no torch, no Python).
@@ -19,7 +19,8 @@ LIB = os.path.join(HERE, "lib", "libastrai_q.so")
 LAB_LIB = os.path.join(HERE, "lib", "libastrai_q_lab.so")
 SOURCES = ["abi.hip", "quant.hip", "gemm_mfma.hip", "gemv.hip", "attn_decode.hip", "attn_prefill.hip"]
 # (source, object, extra flags) of the lab library's own objects; the other product objects are shared
-LAB_SOURCES = [("gemm_mfma.hip", "gemm_mfma_lab.o", ["-DAQ_LAB"]), ("lab.hip", "lab.o", [])]
+LAB_SOURCES = [("gemm_mfma.hip", "gemm_mfma_lab.o", ["-DAQ_LAB"]), ("gemv.hip", "gemv_lab.o", ["-DAQ_LAB"]),
+               ("lab.hip", "lab.o", [])]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -61,7 +62,7 @@ def build(force: bool = True, verbose: bool = False) -> str:
     with ThreadPoolExecutor(max_workers=4) as ex:
         all_objs = list(ex.map(compile_one, SOURCES + LAB_SOURCES))
     objs, lab_only = all_objs[:len(SOURCES)], all_objs[len(SOURCES):]
-    lab_objs = [o for o in objs if not o.endswith("gemm_mfma.o")] + lab_only
+    lab_objs = [o for o in objs if not o.endswith(("gemm_mfma.o", "gemv.o"))] + lab_only
     for lib, members in ((LIB, objs), (LAB_LIB, lab_objs)):
         if force or _stale(lib, members):
             cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib, *members]

@@ -58,6 +58,17 @@ int aq_lab_probe_empty(int *sink, void *stream);
 int aq_lab_quant_tensor_fp8_onepass_spin(const void *x, int x_dtype, int64_t numel, uint8_t *q, float *scale,
                                          void *ws, size_t ws_bytes, int spin_limit, void *stream);
 
+/* Where the wavefronts of the matrix-core decode GEMV that quantises its rows leave time stamps (NULL: nowhere,
+ * the default): device int64 [workgroup][16 wavefronts][8], 100 MHz ticks.  Slots: 0 rows and epilogue operands
+ * requested, 3 rows rounded into LDS, 4 past the barrier, 5 products done, 6 outputs stored.  Process-wide and
+ * unsynchronised: lab only.  (The lab library's GEMV is its own compile of gemv.hip with these stamps in it.) */
+int aq_lab_set_gemv_timeline(long long *buf);
+
+/* on != 0: the matrix-core decode GEMV that quantises its rows requests no weight bytes at all (its products
+ * then multiply zeros): what the launch costs with the token rows, their rounding, the barrier, the products and
+ * the stores but WITHOUT the weight stream -- the floor the rounding sets.  Results are wrong while it is on. */
+int aq_lab_set_gemv_skip_weights(int on);
+
 #ifdef __cplusplus
 }
 #endif

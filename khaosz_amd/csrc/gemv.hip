@@ -418,6 +418,21 @@ constexpr int GV_MFMA_MIN_M = AQ_GV_MFMA_MIN_M;  // more tokens than this take t
 // summed through LDS (exact int32).  A workgroup holds `groups` row groups:
 // 2 x 2 wavefronts when N fills the device that way, fewer rows per workgroup
 // and more K parts when it does not.
+#ifdef AQ_LAB
+// Lab build only (csrc/aq_lab.h, aq_lab_set_gemv_timeline): where the wavefronts of the matrix-core GEMV leave
+// time stamps of the 100 MHz counter, 8 per wavefront.  Expands to nothing in the product library.
+__device__ long long* gv_timeline = nullptr;
+__device__ int gv_skip_weights = 0;  // != 0: the kernel that quantises its rows requests no weight bytes (products of zeros)
+#define GV_STAMP(slot)                                                                                          \
+  do {                                                                                                          \
+    if (gv_timeline && lane == 0) gv_timeline[((size_t)blockIdx.x * 16 + wave) * 8 + (slot)] = wall_clock64(); \
+  } while (0)
+#else
+#define GV_STAMP(slot) \
+  do {                 \
+  } while (0)
+#endif
+
 constexpr int GM_ROWS = 16;    // weight rows per wavefront
 constexpr int GM_MAX_WAVES = 8;
 constexpr int GM_BATCH = 8;    // MFMA steps (64 K bytes each) per register batch
@@ -489,8 +504,13 @@ __global__ __launch_bounds__(GM_MAX_WAVES * 64) void gemv_mfma_kernel(GemvArgs p
 
   // weight stream: descriptor over this wavefront's 16 rows; rows past N read as zero
   const int rows = n0 < nlim ? ((nlim - n0) < GM_ROWS ? (nlim - n0) : GM_ROWS) : 0;
+#ifdef AQ_LAB
+  const __amdgpu_buffer_rsrc_t Wr = make_rsrc(p.wq + (int64_t)(n0 < nlim ? n0 : 0) * K,
+                                              FQ > 0 && gv_skip_weights ? 0u : (uint32_t)rows * (uint32_t)K);
+#else
   const __amdgpu_buffer_rsrc_t Wr =
       make_rsrc(p.wq + (int64_t)(n0 < nlim ? n0 : 0) * K, (uint32_t)rows * (uint32_t)K);
+#endif
   // Whole 128-byte lines per load: an instruction covers one line of 8 rows (lane l: row l % 8, 16-byte piece
   // l / 8), two instructions (rows 0..7 and 8..15) per line index.  In the MFMA's own operand order (lane l: row
   // l % 16, piece l / 16 of a 64-byte step) an instruction would cover 16 half lines, and a one-shot read of
@@ -525,11 +545,13 @@ __global__ __launch_bounds__(GM_MAX_WAVES * 64) void gemv_mfma_kernel(GemvArgs p
     asm volatile("" ::: "memory");  // request order: token rows, epilogue operands, the weight stream
     load_epi();
     asm volatile("" ::: "memory");
+    GV_STAMP(0);
     wload(0, wa);
     wload(GM_LINES, wb);
     asm volatile("" ::: "memory");
     if constexpr (!FP8) {
       xrows.template finish<NORM>(M, M, K, xs, pitch, sx_lds, wave, WAVES, lane, p.eps);
+      GV_STAMP(3);
     } else {
       // the tensor's maximum: every wavefront's share through LDS (a maximum has no order), then the cast
       float amax = 0.0f;
@@ -636,6 +658,7 @@ __global__ __launch_bounds__(GM_MAX_WAVES * 64) void gemv_mfma_kernel(GemvArgs p
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
   if constexpr (FQ > 0 && !FP8) sxv = sx_lds[tok < M ? tok : 0];
+  GV_STAMP(4);
 
   // Four independent accumulators (summed at the end: int32, exact in any order) and a batch's token
   // fragments read from LDS up front: one chain of 16 dependent read -> MFMA steps took 0.6 us after the
@@ -693,6 +716,7 @@ __global__ __launch_bounds__(GM_MAX_WAVES * 64) void gemv_mfma_kernel(GemvArgs p
   }
 
   accv acc = (accs[0] + accs[1]) + (accs[2] + accs[3]);
+  GV_STAMP(5);
   // sum the K parts: all but the first wavefront of each group park their 4 sums in LDS
   __syncthreads();  // everyone is done reading the token codes: the buffer is reused
   int* part = reinterpret_cast<int*>(xs) + grp * (ksplit - 1) * 256;
@@ -777,6 +801,7 @@ __global__ __launch_bounds__(GM_MAX_WAVES * 64) void gemv_mfma_kernel(GemvArgs p
         if (rbase + r < N) dst[r] = y[r];
     }
   }
+  GV_STAMP(6);
 }
 
 // the streaming MFMA variant needs K in whole 256-byte steps (two K parts of whole 128-byte lines)
@@ -1533,3 +1558,13 @@ extern "C" int aq_gemv_w8a8_decode(const void* x, int x_dtype, const int8_t* wq,
   return aq_gemv_w8a8_decode_residual(x, x_dtype, wq, sw, bias, bias_dtype, nullptr, y, y_dtype, M, N, K, ws, ws_bytes,
                                       stream);
 }
+
+#ifdef AQ_LAB
+// Lab build only (see aq_lab.h): the buffer the matrix-core GEMV's wavefronts leave their time stamps in.
+extern "C" int aq_lab_set_gemv_timeline(long long* buf) {
+  return (int)hipMemcpyToSymbol(HIP_SYMBOL(aq::gv_timeline), &buf, sizeof(buf));
+}
+extern "C" int aq_lab_set_gemv_skip_weights(int on) {
+  return (int)hipMemcpyToSymbol(HIP_SYMBOL(aq::gv_skip_weights), &on, sizeof(on));
+}
+#endif

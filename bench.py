@@ -37,6 +37,50 @@ PEAK_FP8_TFLOPS = 5000.0     # dense FP8 MFMA, published
 
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic_fetch_write_size.txt")
 
+# What the part delivers on trivial kernels, measured at the start of this run (measure_ceilings): the roofline
+# objects quote the kernel against these next to the published peaks.
+CEIL = {}
+
+
+def hbm_ceiling_fields(kernel_us):
+    """Same-run ceiling of a decode-sized HBM kernel: the fastest ONE launch that reads 16 MiB once."""
+    floor = CEIL.get("one_shot_16mib_read_us")
+    if not floor:
+        return {}
+    return {"floor_us_one_shot_read": floor, "frac_of_floor": floor / kernel_us,
+            "empty_kernel_in_graph_us": CEIL.get("empty_kernel_in_graph_us")}
+
+
+def mfma_ceiling_fields(achieved, fp8, clock_mhz):
+    """Same-run ceiling of a matrix-core kernel: an MFMA-only loop on random operands (no memory traffic), the
+    clock that loop ran at, and the clock the kernel itself ran at (lab build of the same source, see gemm_clock_mhz)."""
+    name = "mfma_fp8_32x32x64_random_operands" if fp8 else "mfma_i8_32x32x32_random_operands"
+    unit = "tflops" if fp8 else "tops"
+    loop = CEIL.get(f"{name}_{unit}")
+    if not loop:
+        return {}
+    return {"mfma_loop_random_operands_" + unit: loop, "mfma_loop_random_operands_clock_mhz": CEIL.get(f"{name}_clock_mhz"),
+            "mfma_loop_constant_operands_" + unit: CEIL.get(name.replace("random", "constant") + "_" + unit),
+            "mfma_loop_constant_operands_clock_mhz": CEIL.get(name.replace("random", "constant") + "_clock_mhz"),
+            "shader_clock_mhz_during_kernel": clock_mhz, "frac_of_measured_loop": achieved / loop}
+
+
+def gemm_clock_mhz(torch, ops, kernel_only, steps):
+    """The shader clock the tiled GEMM runs at under this workload: the lab library's compile of the same source
+    has wavefront 0 of workgroup 0 read the shader-clock and the 100 MHz reference counters at its start and end
+    (aq_lab_read_clock); their ratio over a conditioned graph replay of the same calls is the clock."""
+    import ctypes
+
+    try:
+        with ops._abi.lab_library() as lab:
+            graph_time_ms(torch, kernel_only, steps, steps)
+            buf = (ctypes.c_longlong * 8)()
+            if lab.aq_lab_read_clock(buf) != 0 or buf[1] <= 0:
+                return None
+            return buf[0] / buf[1] * 100.0
+    except Exception as e:  # a probe: never fails the run
+        return f"unavailable: {str(e)[:80]}"
+
 
 def measured_traffic(key):
     """Bytes per launch that the dominant kernel of workload `key` moves past the L2: FETCH_SIZE + WRITE_SIZE of
@@ -74,15 +118,19 @@ def parse():
     return ap.parse_args()
 
 
-def graph_time_ms(torch, step, steps, warmup, dist=None):
+CONDITION_MS = 200.0  # untimed replays in front of every timed one, by time (the clocks settle under the load itself)
+
+
+def graph_time_ms(torch, step, steps, warmup, dist=None, info=None):
     """Warm up, capture `steps` calls of step(i) into one HIP graph, then time one replay with events on
-    the launching stream.  Returns ms per step.  The `warmup` untimed steps run the way the timed ones do: a
-    few eager calls first (allocations, lazy initialisation), then whole untimed replays of the graph until at
-    least `warmup` steps have gone by (at least one replay) -- the device reaches its steady clocks only
-    under the replayed load, and a replay timed straight after one warm-up replay reads 2-10 % slower than
-    the ones that follow.
-    dist: a list that receives [p10, p50, p90] of the ms per step of 11 further replays, each timed
-    on its own (the spread between replays; not part of the timed region)."""
+    the launching stream.  Returns ms per step.  The untimed part runs the way the timed one does: a few eager
+    calls first (allocations, lazy initialisation), then whole untimed replays of the graph for at least
+    CONDITION_MS milliseconds and at least `warmup` steps -- the device reaches its steady clocks only under the
+    replayed load, and a replay timed straight after a single warm-up replay reads 2-10 % slower than the ones
+    that follow, whatever the number of steps in it.  The K timed steps are one replay between two events.
+    dist: a list that receives [p10, p50, p90] of the ms per step of 11 further replays, each timed on its own
+    (the spread between replays; not part of the timed region).
+    info: a dict that receives conditioning_ms / conditioning_replays of this measurement."""
     for i in range(min(warmup, 20)):
         step(i)
     torch.cuda.synchronize()
@@ -95,22 +143,38 @@ def graph_time_ms(torch, step, steps, warmup, dist=None):
                 step(i)
     torch.cuda.current_stream().wait_stream(side)
     torch.cuda.synchronize()
-    for _ in range(max(1, -(-warmup // steps))):
+    # how long one replay takes, roughly: sizes the conditioning
+    t0 = time.perf_counter()
+    for _ in range(4):
         g.replay()
     torch.cuda.synchronize()
+    per_replay_ms = max((time.perf_counter() - t0) * 1e3 / 4, 1e-3)
+    replays = max(1, -(-warmup // steps), int(CONDITION_MS / per_replay_ms) + 1)
+    t0 = time.perf_counter()
+    for _ in range(replays):
+        g.replay()
+    torch.cuda.synchronize()
+    cond_ms = (time.perf_counter() - t0) * 1e3
+    # The timed replay follows two untimed ones on the stream without a gap: the first launch after the device
+    # has sat idle in a synchronize() pays for waking up (a fixed 5-10 us here, 2-5 % of a 20-step replay),
+    # which is the host's pause and no part of a step.
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(11 if dist is not None else 0)]
+    g.replay()
+    g.replay()
     e0.record()
     g.replay()
     e1.record()
+    for a, b in evs:  # the spread: further replays behind the timed one, each between its own events
+        a.record()
+        g.replay()
+        b.record()
     torch.cuda.synchronize()
     ms = e0.elapsed_time(e1) / steps
+    if info is not None:
+        info["conditioning_ms"] = cond_ms
+        info["conditioning_replays"] = replays
     if dist is not None:
-        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(11)]
-        for a, b in evs:
-            a.record()
-            g.replay()
-            b.record()
-        torch.cuda.synchronize()
         t = sorted(a.elapsed_time(b) / steps for a, b in evs)
         dist[:] = [t[1], t[5], t[9]]
     return ms
@@ -166,13 +230,26 @@ def bench_decode(torch, ops, args, dev):
     # matrix-core kernel from 5 rows on at this N), so the step's time is the dominant kernel's duration.
     # Bytes: the weight once, its scales, the bf16 rows in, the bf16 outputs.
     bytes_alg = N * K + 4 * N + 2 * M * K + 2 * M * N
-    d_step, d_k = [], []
-    ms = graph_time_ms(torch, step, args.steps, args.warmup, d_step)
+    d_step, d_k, cond = [], [], {}
+    ms = graph_time_ms(torch, step, args.steps, args.warmup, d_step, cond)
     ms_eager = eager_time_ms(torch, step, args.steps, args.warmup)
     ms_k = graph_time_ms(torch, kernel_only, args.steps, args.warmup, d_k)
     ms_res = graph_time_ms(torch, resident, args.steps, args.warmup)
     gbs = bytes_alg / (ms * 1e-3) / 1e9
     traffic, traffic_src = measured_traffic(f"decode_m{M}")
+    # The same launch WITHOUT its weight stream (lab build of the same source: token rows requested, rounded,
+    # barrier, products of zeros, stores): what the rounding that every workgroup repeats costs on its own.
+    no_w_us = None
+    if M > 8:
+        try:
+            with ops._abi.lab_library() as lab:
+                lab.aq_lab_set_gemv_skip_weights(1)
+                try:
+                    no_w_us = graph_time_ms(torch, step, args.steps, args.warmup) * 1e3
+                finally:
+                    lab.aq_lab_set_gemv_skip_weights(0)
+        except Exception as e:
+            no_w_us = f"unavailable: {str(e)[:80]}"
     return {
         "workload": f"decode_gemv_w8a8 M={M} K={K} N={N} bf16->int8 per-token, W int8 per-channel, bf16 out",
         "value": gbs, "unit": "GB/s", "ms_per_step": ms, "eager_ms_per_step": ms_eager,
@@ -182,9 +259,11 @@ def bench_decode(torch, ops, args, dev):
                      "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
                      "traffic": traffic, "traffic_source": traffic_src,
                      "kernel_us": ms * 1e3, "kernel_us_p10_p50_p90": [v * 1e3 for v in d_step],
-                     "algorithmic_bytes": bytes_alg, "weight_buffers": nbuf,
+                     "algorithmic_bytes": bytes_alg, "weight_buffers": nbuf, **cond, **hbm_ceiling_fields(ms * 1e3),
+                     "same_launch_without_weight_stream_us": no_w_us,
                      # the same GEMV on codes that a separate launch (or a producer kernel) has already made
                      "gemv_on_codes": {"kernel_us": ms_k * 1e3, "kernel_us_p10_p50_p90": [v * 1e3 for v in d_k],
+                                       **hbm_ceiling_fields(ms_k * 1e3),
                                        "gbs": (bytes_alg - M * K) / (ms_k * 1e-3) / 1e9,
                                        "frac": (bytes_alg - M * K) / (ms_k * 1e-3) / 1e9 / PEAK_HBM_GBS,
                                        "llc_resident_gbs": (bytes_alg - M * K) / (ms_res * 1e-3) / 1e9}},
@@ -231,9 +310,10 @@ def bench_prefill(torch, ops, args, dev):
 
     ops_alg = 2.0 * M * N * K
     steps = max(10, min(args.steps, 100))
-    d_step, d_k = [], []
+    d_step, d_k, cond = [], [], {}
     ms = graph_time_ms(torch, step, steps, args.warmup, d_step)
-    ms_k = graph_time_ms(torch, kernel_only, steps, args.warmup, d_k)
+    ms_k = graph_time_ms(torch, kernel_only, steps, args.warmup, d_k, cond)
+    clock_mhz = gemm_clock_mhz(torch, ops, kernel_only, steps)
     ms_q = graph_time_ms(torch, quant_only, steps, args.warmup)
     ms_nq = graph_time_ms(torch, norm_quant_only, steps, args.warmup)
     tops = ops_alg / (ms * 1e-3) / 1e12
@@ -247,7 +327,7 @@ def bench_prefill(torch, ops, args, dev):
         "roofline": {"bound": "mfma", "kernel": "gemm_kernel<int8,bf16>", "achieved": tops_k, "peak": PEAK_INT8_TOPS,
                      "unit": "TOP/s", "frac": tops_k / PEAK_INT8_TOPS, "traffic": traffic, "traffic_source": traffic_src,
                      "kernel_us": ms_k * 1e3, "kernel_us_p10_p50_p90": [v * 1e3 for v in d_k],
-                     "algorithmic_ops": ops_alg},
+                     "algorithmic_ops": ops_alg, **cond, **mfma_ceiling_fields(tops_k, False, clock_mhz)},
         "quantise_kernel": {"us": ms_q * 1e3, "gbs": qbytes / (ms_q * 1e-3) / 1e9, "frac_hbm": qbytes / (ms_q * 1e-3) / 1e9 / PEAK_HBM_GBS,
                             "algorithmic_bytes": qbytes},
         "rmsnorm_quantise_kernel": {"us": ms_nq * 1e3, "gbs": (qbytes + 2 * K) / (ms_nq * 1e-3) / 1e9,
@@ -311,8 +391,10 @@ def bench_fp8(torch, ops, args, dev):
 
     flops = 2.0 * M * N * K
     steps = max(10, min(args.steps, 50))
+    d_k, cond = [], {}
     ms = graph_time_ms(torch, step, steps, args.warmup)
-    ms_k = graph_time_ms(torch, kernel_only, steps, args.warmup)
+    ms_k = graph_time_ms(torch, kernel_only, steps, args.warmup, d_k, cond)
+    clock_mhz = gemm_clock_mhz(torch, ops, kernel_only, steps)
     # the activation quantiser alone, in its one-launch form (what the step uses) and its stateless two-launch form
     qbytes = 3 * M * K  # bf16 read once, codes written
     us_q1 = graph_time_ms(torch, lambda i: ops.quant_tensor_fp8(xs[i % nbuf], state=qstate), steps, args.warmup) * 1e3
@@ -343,7 +425,8 @@ def bench_fp8(torch, ops, args, dev):
         "value": t, "unit": "TFLOP/s", "ms_per_step": ms, "flops_per_step": flops, "dtype": "fp8_e4m3",
         "roofline": {"bound": "mfma", "kernel": "gemm_kernel<fp8,bf16>", "achieved": tk, "peak": PEAK_FP8_TFLOPS,
                      "unit": "TFLOP/s", "frac": tk / PEAK_FP8_TFLOPS, "traffic": traffic, "traffic_source": traffic_src,
-                     "kernel_us": ms_k * 1e3, "algorithmic_flops": flops},
+                     "kernel_us": ms_k * 1e3, "kernel_us_p10_p50_p90": [v * 1e3 for v in d_k], "algorithmic_flops": flops,
+                     **cond, **mfma_ceiling_fields(tk, True, clock_mhz)},
         "quantise_kernel": {"us": us_q1, "gbs": qbytes / us_q1 / 1e3, "frac_hbm": qbytes / us_q1 / 1e3 / PEAK_HBM_GBS,
                             "algorithmic_bytes": qbytes, "two_launch_form_us": us_q2},
         "decode_gemv_fp8_N8192_K2048": dec,
@@ -464,7 +547,24 @@ def bench_block(torch, ops, args, dev):
         "linears_prefill_ms": ms_lin_pre, "linears_prefill_tops": lin_ops / (ms_lin_pre * 1e-3) / 1e12,
         "linears_decode_ms_per_step": ms_lin_dec, "linears_decode_gbs": lin_bytes / (ms_lin_dec * 1e-3) / 1e9,
         "non_linear_prefill_ms": ms_pre - ms_lin_pre, "non_linear_decode_ms_per_step": ms_dec - ms_lin_dec,
-        "dtype": "int8", "ms_per_step": ms_pre + steps * ms_dec, "roofline": {}, "shape": (B * S, 0, 0),
+        "dtype": "int8", "ms_per_step": ms_pre + steps * ms_dec,
+        # the Linear kernels of the block against the published peaks (algorithmic work: 2 * rows * 45 088 768
+        # operations at prefill, 45 088 768 weight bytes per decode step), and what is left outside them
+        "roofline": {"bound": "hbm", "kernel": "the block's four Linear launches of a decode step (q/k/v, o, up/gate + SwiGLU, down)",
+                     "achieved": lin_bytes / (ms_lin_dec * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": lin_bytes / (ms_lin_dec * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": None,
+                     "kernel_us": ms_lin_dec * 1e3, "algorithmic_bytes": lin_bytes,
+                     "empty_kernel_in_graph_us": CEIL.get("empty_kernel_in_graph_us"),
+                     "prefill_linears": {"bound": "mfma", "achieved": lin_ops / (ms_lin_pre * 1e-3) / 1e12,
+                                         "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
+                                         "frac": lin_ops / (ms_lin_pre * 1e-3) / 1e12 / PEAK_INT8_TOPS,
+                                         "kernel_us": ms_lin_pre * 1e3, "algorithmic_ops": lin_ops,
+                                         **{k: v for k, v in mfma_ceiling_fields(lin_ops / (ms_lin_pre * 1e-3) / 1e12, False, None).items()
+                                            if k != "shader_clock_mhz_during_kernel"}},
+                     "non_linear_residue": {"prefill_ms": ms_pre - ms_lin_pre, "decode_ms_per_step": ms_dec - ms_lin_dec,
+                                            "prefill_frac_of_block": (ms_pre - ms_lin_pre) / ms_pre,
+                                            "decode_frac_of_step": (ms_dec - ms_lin_dec) / ms_dec}},
+        "shape": (B * S, 0, 0),
     }
 
 
@@ -772,6 +872,8 @@ def main():
     fns = {"decode": bench_decode, "prefill": bench_prefill, "fp8": bench_fp8, "block": bench_block,
            "model": bench_model}
     with torch.inference_mode():
+        # the part's own ceilings first: the roofline objects of the workloads quote them
+        CEIL.update(measure_ceilings(torch, ops, dev, calibrate=False))
         main_res = fns[args.workload](torch, ops, args, dev)
         extra = {}
         if not args.no_extra:
@@ -785,7 +887,9 @@ def main():
                     r = bench_decode(torch, ops, a2, dev)
                     extra[f"decode_m{m}"] = r
                 extra["batch_32_to_256"] = bench_few_dozen_rows(torch, ops, args, dev)
-        ceilings = measure_ceilings(torch, ops, dev, calibrate=not args.no_extra)
+        ceilings = dict(CEIL)
+        if not args.no_extra:  # launches GEMMs of other shapes: left out of single-workload (profiling) runs
+            ceilings["gemm_operand_data_and_stock_library"] = gemm_calibration(torch, ops, dev)
         if not args.no_extra and args.workload != "model":
             # the reference's own generation benchmark: about a minute; skipped when this run is already long
             if time.time() - t_start < 150:

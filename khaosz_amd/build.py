@@ -6,6 +6,12 @@
                                      benchmark's ceilings and for tests that pin a tile shape.
 
 hipcc cross-compiles without a GPU.  Both depend on the HIP runtime only (no torch, no Python).
+
+    python -m khaosz_amd.build [--if-stale] [--stall-counters]
+
+--stall-counters builds the lab library's GEMM object with -DAQ_LAB_STALL as well: cycle counters inside the K
+loop (waits at the stage barriers, loop, prologue, epilogue; read with aq_lab_read_clock).  They cost a few clock
+reads per K step, so the default lab build leaves them out; the product library never has them.
 """
 import os
 import subprocess
@@ -40,8 +46,10 @@ def _stale(out, deps):
     return any(os.path.getmtime(d) > t for d in deps)
 
 
-def build(force: bool = True, verbose: bool = False) -> str:
+def build(force: bool = True, verbose: bool = False, stall_counters: bool = False) -> str:
     os.makedirs(OBJ_DIR, exist_ok=True)
+    lab_sources = [(src, obj, extra + (["-DAQ_LAB_STALL"] if stall_counters and src == "gemm_mfma.hip" else []))
+                   for src, obj, extra in LAB_SOURCES]
     headers = [os.path.join(CSRC, "aq_common.h"), os.path.join(CSRC, "aq_rows.h"), os.path.join(CSRC, "aq_lab.h"),
                os.path.join(HERE, "..", "include", "astrai_q.h")]
 
@@ -60,7 +68,7 @@ def build(force: bool = True, verbose: bool = False) -> str:
         return o
 
     with ThreadPoolExecutor(max_workers=4) as ex:
-        all_objs = list(ex.map(compile_one, SOURCES + LAB_SOURCES))
+        all_objs = list(ex.map(compile_one, SOURCES + lab_sources))
     objs, lab_only = all_objs[:len(SOURCES)], all_objs[len(SOURCES):]
     lab_objs = [o for o in objs if not o.endswith(("gemm_mfma.o", "gemv.o"))] + lab_only
     for lib, members in ((LIB, objs), (LAB_LIB, lab_objs)):
@@ -73,4 +81,5 @@ def build(force: bool = True, verbose: bool = False) -> str:
 
 
 if __name__ == "__main__":
-    print(build(force="--if-stale" not in sys.argv, verbose=True))
+    stall = "--stall-counters" in sys.argv
+    print(build(force=stall or "--if-stale" not in sys.argv, verbose=True, stall_counters=stall))

@@ -23,6 +23,14 @@ int aq_lab_set_gemm_tile(int rows);
  * numbering above (a pure function of its arguments: no device is touched). */
 int aq_lab_choose_gemm_tile(int64_t M, int64_t N, int compute_units);
 
+/* Clock counters the lab build's tiled GEMM leaves behind (wavefront 0 of workgroup 0 of the LAST GEMM launch that
+ * completed): host int64[8].  [0] shader-clock cycles and [1] 100 MHz reference ticks between the kernel's first and
+ * last instruction -- their ratio x 100 MHz is the clock the kernel ran at.  [2..7] are filled only by a build with
+ * the K-loop stall counters (python -m khaosz_amd.build --stall-counters, which adds -DAQ_LAB_STALL to the lab
+ * library's GEMM object): [2] cycles waited at the stage barriers, [3] cycles of the K loop, [4] tile start ->
+ * first stage landed, [5] the first K step, [6] accumulator exchange + epilogue, [7] the whole tile. */
+int aq_lab_read_clock(long long *host8);
+
 /* `workgroups` x 4 wavefronts each issue iters x 8 independent MFMAs.
  * kind 0 = i32_32x32x32_i8 (65536 ops each), 1 = i32_16x16x64_i8 (32768), 2 = f32_32x32x64 e4m3 (131072 flops).
  * data 0 = constant operands (no toggling: the clock stays at its maximum), 1 = random bytes, four operand

@@ -133,6 +133,70 @@ __device__ __forceinline__ float swiglu_repro(float u, float g) {
   return __fmul_rn(u, __fdiv_rn(g, __fadd_rn(1.0f, exp_repro(-g))));
 }
 
+// n / d, correctly rounded, for operands in the middle of the range: the compiler's own sequence for an fp32
+// divide (hardware reciprocal, one refinement, quotient, two residual corrections) without the scaling of
+// extreme operands in front (v_div_scale) and the special-case selection behind (v_div_fixup) -- both the
+// identity when 2^-62 <= |n|, |d| <= 2^62, where no intermediate leaves the normal range.  11 instead of 14
+// operation slots (the reciprocal counts four).
+__device__ __forceinline__ float div_midrange(float n, float d) {
+  const float y0 = __builtin_amdgcn_rcpf(d);
+  const float y = __builtin_fmaf(__builtin_fmaf(-d, y0, 1.0f), y0, y0);
+  float q = n * y;
+  q = __builtin_fmaf(__builtin_fmaf(-d, q, n), y, q);
+  return __builtin_fmaf(__builtin_fmaf(-d, q, n), y, q);
+}
+
+// The gates div_midrange may be used for: zero (0 / d = 0, with a sign that no code and no maximum depends on) or
+// 2^-62 <= |g| <= 80, so that 1 + exp(-g) < 2^116 and every intermediate of the short divide stays a normal
+// number.  Exact zeros must pass: rows of real bf16 activations hold a few per ten million values, and a row sent
+// through the general divide takes three times as long as its neighbours and holds up the launch.
+// For bf16 gates the test runs on the raw pairs with packed 16-bit integer operations, two gates per operation:
+// |g| as a 16-bit pattern orders like the number; pattern - 1 wraps a zero to 0xffff, above every bound.
+struct GateRangeBf16 {
+  typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+  u16x2 lo = {0xffff, 0xffff}, hi = {0, 0};
+  __device__ __forceinline__ void add(uint32_t pair) {
+    const uint32_t a = pair & 0x7fff7fffu;
+    const u16x2 av = __builtin_bit_cast(u16x2, a);
+    lo = __builtin_elementwise_min(lo, av - (u16x2){1, 1});
+    hi = __builtin_elementwise_max(hi, av);
+  }
+  __device__ __forceinline__ void add(const uint4& v) {
+    add(v.x);
+    add(v.y);
+    add(v.z);
+    add(v.w);
+  }
+  __device__ __forceinline__ bool ok() const {
+    const unsigned l = lo.x < lo.y ? lo.x : lo.y, h = hi.x > hi.y ? hi.x : hi.y;
+    return l >= 0x2080u - 1u && h <= 0x42a0u;  // bf16 patterns of 2^-62 and 80
+  }
+};
+// the same test on fp32 gates
+template <int N>
+__device__ __forceinline__ bool gates_midrange(const float* g) {
+  float lo = 1.0f, hi = 0.0f;
+#pragma unroll
+  for (int i = 0; i < N; ++i) {
+    const float a = fabsf(g[i]);
+    lo = fminf(lo, a == 0.0f ? 1.0f : a);
+    hi = fmaxf(hi, a);
+  }
+  return lo >= 2.168404344971009e-19f && hi <= 80.0f;  // 2^-62
+}
+
+// SwiGLU of N pairs with div_midrange: the bits of swiglu_repro when the gates pass the test above (zeros aside).
+// Four chains at a time: enough to cover the arithmetic's latency, few enough temporaries for a caller to keep a
+// whole row of h in registers next to them.
+template <int N>
+__device__ __forceinline__ void swiglu_group_midrange(const float* u, const float* g, float* h) {
+#pragma unroll
+  for (int i = 0; i < N; ++i) {
+    if (i > 0 && (i & 3) == 0) __builtin_amdgcn_sched_barrier(0);
+    h[i] = __fmul_rn(u[i], div_midrange(g[i], __fadd_rn(1.0f, exp_repro(-g[i]))));
+  }
+}
+
 // low bytes of four 32-bit patterns -> one dword (a in bits 7:0 .. d in bits 31:24)
 __device__ __forceinline__ uint32_t pack_low_bytes(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
   const uint32_t ab = __builtin_amdgcn_perm(b, a, 0x0c0c0400u);  // {a.b0, b.b0, 0, 0}

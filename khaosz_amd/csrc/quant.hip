@@ -2,6 +2,8 @@
 // per row and per-tensor FP8 (OCP e4m3fn).  Both are HBM-bound streaming
 // kernels: 16-byte loads per lane, one wavefront per row, wavefront-wide
 // absmax through cross-lane shuffles, no LDS.
+#include <type_traits>
+
 #include "aq_common.h"
 #include "aq_rows.h"
 
@@ -256,51 +258,126 @@ __global__ __launch_bounds__(256) void rmsnorm_quant_kernel(const void* __restri
 // the quantiser launches (three passes over [M, F]) by one.  A lane first turns
 // its NC vector pairs into h (fp32, kept in registers; the inputs die as it goes),
 // then reduces the absmax and rounds.
+//
+// The kernel is bound by its vector arithmetic (about 34 operations per element: the exponential's polynomial, a
+// correctly rounded divide, the two-correction rounding; 4096 x 5632 is 20 us of it at 2.4 GHz), so the work went
+// into keeping the vector ALUs fed and into the operation count:
+//  * every load of a row is requested up front, pair by pair (up vector, gate vector), and the arithmetic walks
+//    the pairs in that order, waiting for one pair at a time (loads return in request order).  A row's first pair
+//    arrives within a microsecond and the rest streams in behind the arithmetic.  (Left to itself the compiler
+//    waited for the whole row before the first operation; with only a few pairs requested ahead, a wavefront's
+//    time was the memory latency times its pairs.)
+//  * the divide is div_midrange (11 instead of 14 operation slots) whenever the row's gates allow it, which is
+//    tested on the raw bf16 pairs with packed 16-bit operations; a row with a gate outside is done again with
+//    the general divide, out of line.
+//  * NC is the row's own number of vector pairs per lane (a pair past the row would cost its full arithmetic).
+// Four wavefronts fit a SIMD (128 registers: a row's h is 88 of them at F = 5632); the SIMD serves the oldest
+// first, so a compute unit's 16 rows finish one after the other, 4096 x 5632 bf16 in 28 us (before: 31.5).
 template <bool BF16, int NC>
-__global__ __launch_bounds__(256) void swiglu_quant_kernel(const void* __restrict__ ug, int64_t M, int F, int64_t ld,
-                                                           int8_t* __restrict__ q, float* __restrict__ scale) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void swiglu_quant_kernel(
+    const void* __restrict__ ug, int64_t M, int F, int64_t ld, int8_t* __restrict__ q, float* __restrict__ scale) {
   constexpr int EPV = RowIn<BF16>::EPV;
   const int lane = threadIdx.x & 63;
   const int64_t stride = (int64_t)gridDim.x * 4;
   const int nvec = F / EPV;
-  for (int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6); row < M; row += stride) {
-    const uint4* up = reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(ug) + row * ld * (BF16 ? 2 : 4));
-    const uint4* gate = up + nvec;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // scalar: the row's descriptors live in SGPRs
+  for (int64_t row = (int64_t)blockIdx.x * 4 + wave; row < M; row += stride) {
+    // descriptors over the row's two halves: vectors past the row read as zeros.  (Buffer loads also stay where
+    // they are written, between the scheduling barriers below: plain loads of read-only memory moved freely.)
+    const char* up = reinterpret_cast<const char*>(ug) + row * ld * (BF16 ? 2 : 4);
+    const uint32_t half_bytes = (uint32_t)F * (BF16 ? 2u : 4u);
+    const __amdgpu_buffer_rsrc_t Ur = make_rsrc(up, half_bytes), Gr = make_rsrc(up + half_bytes, half_bytes);
     uint4 cu[NC], cg[NC];
 #pragma unroll
     for (int i = 0; i < NC; ++i) {
-      const int v = i * 64 + lane;
-      cu[i] = v < nvec ? up[v] : make_uint4(0, 0, 0, 0);
-      cg[i] = v < nvec ? gate[v] : make_uint4(0, 0, 0, 0);
+      const uint32_t off = (uint32_t)(i * 64 + lane) * 16u;
+      cu[i] = buffer_load_16(Ur, off);
+      cg[i] = buffer_load_16(Gr, off);
+      __builtin_amdgcn_sched_barrier(0);  // pair by pair (the scheduler would put all up halves in front of all gate halves)
     }
+    asm volatile("" ::: "memory");
     float h[NC][EPV];
     float amax = 0.0f;
+    bool ok = true;
+    GateRangeBf16 range;
 #pragma unroll
     for (int i = 0; i < NC; ++i) {
       float u[EPV], g[EPV];
       RowIn<BF16>::unpack(cu[i], u);
       RowIn<BF16>::unpack(cg[i], g);
-#pragma unroll
-      for (int e = 0; e < EPV; ++e) h[i][e] = swiglu_repro(u[e], g[e]);  // 0 * silu(0) = 0 past the row
+      // (a last pair that lies partly past the row's end reads zeros there: h = 0 * silu(0) = 0)
+      if constexpr (BF16)
+        range.add(cg[i]);
+      else
+        ok &= gates_midrange<EPV>(g);
+      swiglu_group_midrange<EPV>(u, g, h[i]);
       amax = fmaxf(amax, vec_amax<EPV>(h[i]));
+      // h is wanted HERE: left to itself the compiler takes the range checks of all pairs (which need the gates only)
+      // and the branch on them first, and requests each pair's up half inside the branch, one by one
+      if constexpr (BF16)
+        asm volatile("" ::"v"(h[i][0]), "v"(h[i][1]), "v"(h[i][2]), "v"(h[i][3]), "v"(h[i][4]), "v"(h[i][5]), "v"(h[i][6]), "v"(h[i][7]));
+      else
+        asm volatile("" ::"v"(h[i][0]), "v"(h[i][1]), "v"(h[i][2]), "v"(h[i][3]));
+      __builtin_amdgcn_sched_barrier(0);  // pairs in the order they were requested, which is the order they arrive in
+    }
+    int8_t* dst = q + row * (int64_t)F;
+    if constexpr (BF16) ok = range.ok();
+    if (__builtin_amdgcn_ballot_w64(!ok) != 0) {
+      // Some gate of the row lies outside the range of the short divide (an outlier beyond +-80, a denormal):
+      // rare, so the row is simply done again with the general divide, in two rolled loops that keep nothing in
+      // registers (maximum, then codes) and leave the main path's register budget alone.
+      float am = 0.0f;
+      for (int i = 0; i < NC; ++i) {
+        const uint32_t off = (uint32_t)(i * 64 + lane) * 16u;
+        float u[EPV], g[EPV];
+        RowIn<BF16>::unpack(buffer_load_16(Ur, off), u);
+        RowIn<BF16>::unpack(buffer_load_16(Gr, off), g);
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) am = fmaxf(am, fabsf(swiglu_repro(u[e], g[e])));
+      }
+      const RowScale rsc = row_scale(wave_max(am));
+      if (lane == 0) scale[row] = rsc.s;
+      for (int i = 0; i < NC; ++i) {
+        const int v = i * 64 + lane;
+        const uint32_t off = (uint32_t)v * 16u;
+        float u[EPV], g[EPV], hh[EPV];
+        uint32_t code[EPV];
+        RowIn<BF16>::unpack(buffer_load_16(Ur, off), u);
+        RowIn<BF16>::unpack(buffer_load_16(Gr, off), g);
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) hh[e] = swiglu_repro(u[e], g[e]);
+        quant_codes<EPV>(hh, rsc.s, rsc.rs, rsc.fast_ok, code);
+        if (v < nvec) {
+          if constexpr (BF16) {
+            uint2 o;
+            o.x = pack_low_bytes(code[0], code[1], code[2], code[3]);
+            o.y = pack_low_bytes(code[4], code[5], code[6], code[7]);
+            store_wt(reinterpret_cast<uint2*>(dst + (int64_t)v * EPV), o);
+          } else {
+            store_wt(reinterpret_cast<uint32_t*>(dst + (int64_t)v * EPV), pack_low_bytes(code[0], code[1], code[2], code[3]));
+          }
+        }
+      }
+      continue;
     }
     const RowScale rsc = row_scale(wave_max(amax));
     if (lane == 0) scale[row] = rsc.s;
-    int8_t* dst = q + row * (int64_t)F;
+    // codes through a descriptor over the row (written through, like store_wt): one lane offset for the whole
+    // row and the vector's position as a constant, instead of a 64-bit address per store; what lies past the
+    // row falls outside the descriptor and is dropped
+    const __amdgpu_buffer_rsrc_t Qr = make_rsrc(dst, (uint32_t)F);
 #pragma unroll
     for (int i = 0; i < NC; ++i) {
-      const int v = i * 64 + lane;
-      if (v < nvec) {
-        uint32_t code[EPV];
-        quant_codes<EPV>(h[i], rsc.s, rsc.rs, rsc.fast_ok, code);
-        if constexpr (BF16) {
-          uint2 o;
-          o.x = pack_low_bytes(code[0], code[1], code[2], code[3]);
-          o.y = pack_low_bytes(code[4], code[5], code[6], code[7]);
-          store_wt(reinterpret_cast<uint2*>(dst + (int64_t)v * EPV), o);
-        } else {
-          store_wt(reinterpret_cast<uint32_t*>(dst + (int64_t)v * EPV), pack_low_bytes(code[0], code[1], code[2], code[3]));
-        }
+      uint32_t code[EPV];
+      quant_codes<EPV>(h[i], rsc.s, rsc.rs, rsc.fast_ok, code);
+      if constexpr (BF16) {
+        typedef int v2i_t __attribute__((ext_vector_type(2)));
+        const v2i_t o = {(int)pack_low_bytes(code[0], code[1], code[2], code[3]),
+                         (int)pack_low_bytes(code[4], code[5], code[6], code[7])};
+        __builtin_amdgcn_raw_buffer_store_b64(o, Qr, lane * 8, i * 512, STORE_WT);
+      } else {
+        __builtin_amdgcn_raw_buffer_store_b32((int)pack_low_bytes(code[0], code[1], code[2], code[3]), Qr, lane * 4,
+                                              i * 256, STORE_WT);
       }
     }
   }
@@ -326,8 +403,11 @@ __global__ __launch_bounds__(1024) void swiglu_quant_wg_kernel(const void* __res
   float u[EPV], g[EPV], h[EPV];
   RowIn<BF16>::unpack(cu, u);
   RowIn<BF16>::unpack(cg, g);
+  swiglu_group_midrange<EPV>(u, g, h);
+  if (__builtin_amdgcn_ballot_w64(!gates_midrange<EPV>(g)) != 0) {  // a gate outside the short divide's range: again
 #pragma unroll
-  for (int e = 0; e < EPV; ++e) h[e] = swiglu_repro(u[e], g[e]);
+    for (int e = 0; e < EPV; ++e) h[e] = swiglu_repro(u[e], g[e]);
+  }
   const float wm = wave_max(vec_amax<EPV>(h));
   if (lane == 0) wmax[wave] = wm;
   __syncthreads();
@@ -738,15 +818,22 @@ static int launch_swiglu_quant(const void* ug, int64_t M, int64_t F, int64_t ld,
                        ld, q, scale);
     return (int)hipGetLastError();
   }
+  // four wavefronts of this kernel fit a SIMD (128 registers each): 16 rows at a time per compute unit, and
+  // wavefronts walk the rows beyond that
   int64_t wgs = (M + 3) / 4;
-  if (wgs > 1024) wgs = 1024;
+  const int64_t cap = (int64_t)aq::device_cus() * 4;
+  if (wgs > cap) wgs = cap;
   const dim3 g((unsigned)wgs), b(256);
-  if (vpl <= 4)
-    hipLaunchKernelGGL((aq::swiglu_quant_kernel<BF16, 4>), g, b, 0, st, ug, M, (int)F, ld, q, scale);
-  else if (vpl <= 12)
-    hipLaunchKernelGGL((aq::swiglu_quant_kernel<BF16, 12>), g, b, 0, st, ug, M, (int)F, ld, q, scale);
-  else
-    return AQ_E_RANGE;
+  // as many vector pairs per lane as the row has (a slot past the row costs its full arithmetic: a 5632-wide row
+  // is 11 pairs per lane, and a 12th would be 8 % more work)
+  switch (vpl) {
+#define AQ_SWIGLU_CASE(nc)                                                                                   \
+  case nc: hipLaunchKernelGGL((aq::swiglu_quant_kernel<BF16, nc>), g, b, 0, st, ug, M, (int)F, ld, q, scale); break;
+    AQ_SWIGLU_CASE(1) AQ_SWIGLU_CASE(2) AQ_SWIGLU_CASE(3) AQ_SWIGLU_CASE(4) AQ_SWIGLU_CASE(5) AQ_SWIGLU_CASE(6)
+    AQ_SWIGLU_CASE(7) AQ_SWIGLU_CASE(8) AQ_SWIGLU_CASE(9) AQ_SWIGLU_CASE(10) AQ_SWIGLU_CASE(11) AQ_SWIGLU_CASE(12)
+#undef AQ_SWIGLU_CASE
+    default: return AQ_E_RANGE;
+  }
   return (int)hipGetLastError();
 }
 
@@ -824,3 +911,4 @@ extern "C" int aq_quant_tensor_fp8(const void* x, int x_dtype, int64_t numel, ui
   }
   return (int)hipGetLastError();
 }
+

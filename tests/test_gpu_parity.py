@@ -188,6 +188,35 @@ def test_swiglu_quant_bit_exact(oracle, M, F, dtype):
     assert bad.size == 0, f"first mismatches (row, col): {bad[:5].tolist()}"
 
 
+@pytest.mark.parametrize("M,F", [(40, 5632), (40, 1040), (1100, 704)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_swiglu_quant_divide_range_edges(oracle, M, F, dtype):
+    """The kernels take a short divide for rows whose gates are zero or in 2^-62 .. 80 and the general one for the
+    rest: one special gate per row on either side of each bound (and zeros of both signs, a denormal, gates past
+    the exponential's clamp), among ordinary values, must give the oracle's bits on both paths."""
+    if dtype == torch.float32 and F > 4096:
+        pytest.skip("fp32 rows longer than 4096 are outside the kernel's limit")
+    _say("swiglu_quant edges", M, F, dtype)
+    g = torch.Generator().manual_seed(M + F)
+    ug = torch.randn(M, 2 * F, generator=g) * 1.5
+    specials = [0.0, -0.0, 2.0 ** -62, -(2.0 ** -62), 2.0 ** -63, -(2.0 ** -63), 2.0 ** -100, 1e-39, -1e-39, 80.0, -80.0,
+                80.5, -80.5, 31.9, 32.0, 88.0, -88.0, 1e30, -1e30, 2.0 ** -126, 3.0 * 2.0 ** -64]
+    cols = torch.randint(0, F, (len(specials),), generator=g)
+    for r, (v, c) in enumerate(zip(specials, cols.tolist())):
+        ug[r, F + c] = v
+    ug[len(specials), F:F + 64] = 0.0          # a run of zero gates
+    ug[len(specials) + 1, :F] = 0.0            # up all zero: h = 0 whatever the gates
+    ud = ug.to(DEV, dtype)
+    q, s = ops.swiglu_quant_rowwise_i8(ud)
+    if dtype == torch.bfloat16:
+        qo, so = oracle.c_swiglu_quant_i8(bf16_bits(ud), bf16_bits=True)
+    else:
+        qo, so = oracle.c_swiglu_quant_i8(to_np(ud))
+    assert np.array_equal(to_np(s).view(np.uint32), so.view(np.uint32))
+    bad = np.argwhere(to_np(q) != qo)
+    assert bad.size == 0, f"first mismatches (row, col): {bad[:5].tolist()}"
+
+
 def test_swiglu_quant_tracks_the_unfused_flow():
     """Against silu, product and row quantiser as three launches (mlp.py:25-26 in bf16): the fused
     kernel keeps the product in fp32, so codes may differ by one step."""

@@ -46,11 +46,15 @@ namespace aq {
 // 2-6 % slower every time (128 x 128 at 512 x 8192 x 2048: 15.0 against 14.1 us; 64 x 64 at 128 x 8192 x 2048:
 // 8.8 against 8.4 us).  The lab build keeps the 128 x 128 one (<2, 2, 2, 2, 2, 128, 3>) so that the K-split
 // code stays compiled and tested.
-// Shapes that only the lab build instantiates.  Measured, none faster on int8 with real operand data: under a
-// matrix-core load with toggling operands this part runs against its power limit, and fewer LDS reads per MFMA
-// buy clock, not rate (8192^3: 2.31-2.42 POP/s for every shape below and for the 256 x 128 tile alike, while the
-// clock moves between 1.47 and 1.65 GHz).  FP8, which is throttled less, gains 8 % from the first one at 8192^3
-// (2.6 against 2.4 PFLOP/s); no benchmark configuration has enough 256 x 256 tiles to use it.
+// Shapes that (but for the first one on FP8) only the lab build instantiates.  Measured, none faster on int8 with
+// real operand data: under a matrix-core load with toggling operands this part runs against its power limit, and
+// fewer LDS reads per MFMA buy clock, not rate (8192^3: 2.31-2.42 POP/s for every shape below and for the
+// 256 x 128 tile alike, while the clock moves between 1.47 and 1.65 GHz).  FP8, which is throttled less, gains 5 %
+// from the first one at 8192^3 (417 against 438 us: its K loop runs at 84 % of the matrix cores' own time with 6 %
+// of it waited at the stage barriers, where the 256 x 128 tile waits 40 %; a 64 x 64 sub-tile reads 32 bytes of
+// fragments per wavefront and cycle, 128 per compute unit, which is all the LDS delivers, before the fills'
+// writes; the 128 x 128 sub-tile needs half); the product takes it for FP8 launches of at least two rounds of
+// 256 x 256 tiles.
 //   <2, 2, 4, 4, 1, 64, 4>   256 x 256 tile, 4 wavefronts (one per SIMD) of 128 x 128: 256 accumulator
 //                            registers per lane (the AGPR half of the register file), 8 fragment reads per
 //                            16 MFMAs instead of 16, half the LDS fill per MFMA; 4 stages of 32 KiB; whole K
@@ -88,8 +92,8 @@ using ShapeN64 = Shape<2, 2, 2, 1, 1, 128, 4>;
 using ShapeN32 = Shape<4, 1, 1, 1, 1, 128, 4>;
 using ShapeM64N64 = Shape<2, 2, 1, 1, 1, 128, 4>;
 using ShapeM64N32 = Shape<2, 1, 1, 1, 1, 128, 6>;
+using ShapeHuge = Shape<2, 2, 4, 4, 1, 64, 4>;  // product: FP8 launches of two rounds or more (see huge_fp8_ok)
 #ifdef AQ_LAB
-using ShapeHuge = Shape<2, 2, 4, 4, 1, 64, 4>;
 using ShapeTall = Shape<2, 2, 4, 2, 1, 128, 3>;
 using ShapeHuge8 = Shape<4, 2, 2, 4, 1, 64, 4>;
 using ShapePair = Shape<2, 2, 2, 2, 2, 128, 3>;
@@ -884,8 +888,25 @@ static int launch_shape(GemmArgs& a, hipStream_t st) {
   return (int)hipGetLastError();
 }
 
+// FP8 launches the 256 x 256 tile serves and gains on: whole 256-row multiples, even N, whole 64-byte K steps, no
+// residual (the tile's one K-loop and epilogue variant), and at least two rounds of such tiles over the compute
+// units (one round -- 4096^3 -- measured level with the 256 x 128 tile, 57.0 against 57.7 us).
+static bool huge_fp8_ok(const GemmArgs& a) {
+  if ((a.K % ShapeHuge::BK) != 0 || (a.N % 2) != 0 || (a.M % ShapeHuge::BM) != 0 || a.res != nullptr) return false;
+  const int64_t tiles = (int64_t)(a.M / ShapeHuge::BM) * ((a.N + ShapeHuge::BN - 1) / ShapeHuge::BN);
+  return tiles >= 2 * (int64_t)device_cus();
+}
+
 template <bool FP8, int OUT>
 static int launch(GemmArgs& a, hipStream_t st) {
+#ifdef AQ_LAB
+  const bool forced = g_forced_tile != 0;
+#else
+  const bool forced = false;
+#endif
+  if constexpr (FP8 && OUT != OUT_I32) {
+    if (!forced && huge_fp8_ok(a)) return launch_shape<FP8, OUT, ShapeHuge>(a, st);
+  }
   switch (choose_tile(a.M, a.N)) {
     case TILE_SMALL: return launch_shape<FP8, OUT, ShapeSmall>(a, st);
     case TILE_N64: return launch_shape<FP8, OUT, ShapeN64>(a, st);

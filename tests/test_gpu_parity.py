@@ -290,6 +290,93 @@ def test_gemm_with_more_tiles_than_compute_units(oracle, tile):
     assert torch.equal(y8.cpu(), ref)
 
 
+PRODUCT_TILES = {256: "256 x 128", 128: "128 x 128", 64: "128 x 64", 32: "128 x 32", 65: "64 x 64", 33: "64 x 32"}
+
+
+def _smallest_shape_for_tile(kind, cus):
+    """The (M, N) of fewest outputs for which the library's own rule (a pure function, asked of the lab library;
+    no GEMM runs there) picks tile `kind` on a device of `cus` compute units."""
+    lab = _abi.load_lab()
+    best = None
+    for M in range(33, 2100, 7):
+        for N in list(range(32, 2100, 32)) + [3072, 4096, 8192]:
+            if lab.aq_lab_choose_gemm_tile(M, N, cus) == kind and (best is None or M * N < best[0] * best[1]):
+                best = (M, N)
+    return best
+
+
+@pytest.mark.parametrize("kind", sorted(PRODUCT_TILES))
+def test_every_product_tile_on_the_shipped_library(oracle, kind):
+    """Each of the six tile shapes of libastrai_q.so (the tests above force tiles in the lab library, a separate
+    compile of the same source): a shape for which the shipped library's rule picks that tile, run through the
+    shipped library, int32 sums, fused epilogue and FP8 product against the oracle."""
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    shape = _smallest_shape_for_tile(kind, cus)
+    assert shape is not None, f"no shape found for which the rule picks the {PRODUCT_TILES[kind]} tile"
+    M, N = shape
+    lib = _abi.load()
+    assert lib is not _abi.load_lab() and not hasattr(lib, "aq_lab_set_gemm_tile")  # the product object does the work
+    for K in (144, 256):  # ragged K steps, whole K steps
+        _say("product tile", PRODUCT_TILES[kind], M, N, K)
+        xq, wq = rand_codes(M, K, 301).numpy(), rand_codes(N, K, 302).numpy()
+        want = oracle.c_gemm_i8_i32(xq, wq)
+        acc = ops.gemm_i8_i32(torch.from_numpy(xq).to(DEV), torch.from_numpy(wq).to(DEV))
+        assert np.array_equal(to_np(acc), want)
+        g = np.random.default_rng(303)
+        sx = (g.random(M) * 0.02 + 0.001).astype(np.float32)
+        sw = (g.random(N) * 0.002 + 0.0001).astype(np.float32)
+        b = (g.standard_normal(N) * 0.01).astype(np.float32)
+        y = ops.linear_w8a8(torch.from_numpy(xq).to(DEV), torch.from_numpy(sx).to(DEV), torch.from_numpy(wq).to(DEV),
+                            torch.from_numpy(sw).to(DEV), torch.from_numpy(b).to(DEV), out_dtype=torch.bfloat16)
+        assert np.array_equal(bf16_bits(y), oracle.c_dequant_epilogue(want, sx, sw, b, bf16_out=True))
+        yf = ops.linear_w8a8(torch.from_numpy(xq).to(DEV), torch.from_numpy(sx).to(DEV), torch.from_numpy(wq).to(DEV),
+                             torch.from_numpy(sw).to(DEV), None, out_dtype=torch.float32)
+        assert np.array_equal(to_np(yf).view(np.uint32),
+                              oracle.c_dequant_epilogue(want, sx, sw, None, bf16_out=False).view(np.uint32))
+        # FP8 codes from two binades: every product and partial sum is exact in fp32 (no order dependence)
+        gt = torch.Generator().manual_seed(304)
+        a8 = torch.randint(0x30, 0x40, (M, K), generator=gt, dtype=torch.uint8)
+        b8 = torch.randint(0x30, 0x40, (N, K), generator=gt, dtype=torch.uint8)
+        one = torch.ones(1, device=DEV)
+        y8 = ops.linear_fp8(a8.to(DEV), one, b8.to(DEV), one, out_dtype=torch.float32)
+        ref = a8.view(torch.float8_e4m3fn).float() @ b8.view(torch.float8_e4m3fn).float().T
+        assert torch.equal(y8.cpu(), ref)
+
+
+def test_product_fp8_256x256_tile(oracle):
+    """FP8 launches of two rounds or more of 256 x 256 tiles take that tile in the shipped library (whole 256-row
+    multiples, even N, whole 64-byte K steps, no residual).  Exact-in-fp32 operands against a float product, a
+    random-data slab against the oracle within the FP8 tolerance, and the neighbouring shapes that must NOT take it
+    (ragged M, a residual) against the same references."""
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    N, K = 2048 + 130, 192                      # ragged N (even), three K steps
+    M = 256 * ((2 * cus + (N + 255) // 256 - 1) // ((N + 255) // 256))
+    assert (M // 256) * ((N + 255) // 256) >= 2 * cus
+    _say("product fp8 256x256", M, N, K)
+    gt = torch.Generator().manual_seed(305)
+    b8 = torch.randint(0x30, 0x40, (N, K), generator=gt, dtype=torch.uint8)
+    one = torch.ones(1, device=DEV)
+    for rows in (M, M + 3):                     # the 256 x 256 tile, and a ragged M that goes to another tile
+        a8 = torch.randint(0x30, 0x40, (rows, K), generator=gt, dtype=torch.uint8)
+        y8 = ops.linear_fp8(a8.to(DEV), one, b8.to(DEV), one, out_dtype=torch.float32)
+        ref = a8.view(torch.float8_e4m3fn).float() @ b8.view(torch.float8_e4m3fn).float().T
+        assert torch.equal(y8.cpu(), ref)
+        yb = ops.linear_fp8(a8.to(DEV), one, b8.to(DEV), one, out_dtype=torch.bfloat16)
+        assert torch.equal(yb.cpu(), ref.to(torch.bfloat16))
+    # random data with real scales, a bias and bf16 output: a slab of rows against the oracle
+    x = make_x(M, K, 306)
+    w = make_x(N, K, 307) * 0.02
+    xq, sx = ops.quant_tensor_fp8(x.to(DEV))
+    wq, sw = ops.quant_tensor_fp8(w.to(DEV))
+    bias = (torch.randn(N, generator=gt) * 0.01)
+    y = ops.linear_fp8(xq, sx, wq, sw, out_dtype=torch.bfloat16, bias=bias.to(DEV))
+    rows = slice(M - 40, M)
+    want = oracle.c_linear_fp8(to_np(xq)[rows], float(to_np(sx)[0]), to_np(wq), float(to_np(sw)[0]), bf16_out=False,
+                               bias=bias.numpy())
+    got = y[rows].float().cpu().numpy()
+    assert np.allclose(got, want, rtol=1e-2, atol=1e-2 * float(np.sqrt((want ** 2).mean())))
+
+
 def test_lab_tile_256x256_on_shapes_it_takes(oracle):
     """The lab build's 256 x 256 tile (four wavefronts of 128 x 128, accumulators in AGPRs, per-row scales through
     LDS) takes whole 256-row multiples, even N and whole 64-byte K steps without a residual; anything else falls

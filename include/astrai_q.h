@@ -60,12 +60,14 @@ int aq_quant_rowwise_i8(const void *x, int x_dtype, int64_t M, int64_t K, int64_
 /* Per-tensor FP8 (OCP e4m3fn): scale[0] = amax / 448 (1 when all zero),
  * q = e4m3fn_rne(clamp(x / scale, -448, 448)).  Stands in for the operands of
  * the same F.linear call (linear.py:21) in the FP8 variant.
- * amax_ws: AQ_FP8_AMAX_WS_BYTES of device scratch (partial maxima, one per workgroup of the
- * first pass).  It needs no initial value and carries nothing from one call to the next; two
- * calls that overlap in time must not share it.  Two launches: maximum, then scale + cast. */
+ * amax_ws: device scratch of ws_bytes >= AQ_FP8_AMAX_WS_BYTES (partial maxima, one per workgroup of the first
+ * pass; a smaller one is AQ_E_WORKSPACE: the size is an argument so that a buffer of a single word is refused
+ * instead of written past).  It needs no initial value and carries
+ * nothing from one call to the next; two calls that overlap in time must not share it.  Two launches: maximum,
+ * then scale + cast. */
 #define AQ_FP8_AMAX_WS_BYTES 1024
 int aq_quant_tensor_fp8(const void *x, int x_dtype, int64_t numel, uint8_t *q, float *scale,
-                        uint32_t *amax_ws, void *stream);
+                        uint32_t *amax_ws, size_t ws_bytes, void *stream);
 
 /* The same result in ONE launch, for callers that can keep a small piece of device state: every workgroup holds
  * its share of x in registers between the maximum and the cast (tensors up to 32 MiB on 256 compute units are read

@@ -21,7 +21,7 @@ SYMBOLS = {
     "aq_quant_rowwise_i8": (_int, [_vp, _int, _i64, _i64, _i64, _vp, _vp, _vp]),
     "aq_rmsnorm_quant_rowwise_i8": (_int, [_vp, _int, _vp, _int, ctypes.c_float, _i64, _i64, _i64, _vp, _vp, _vp]),
     "aq_swiglu_quant_rowwise_i8": (_int, [_vp, _int, _i64, _i64, _i64, _vp, _vp, _vp]),
-    "aq_quant_tensor_fp8": (_int, [_vp, _int, _i64, _vp, _vp, _vp, _vp]),
+    "aq_quant_tensor_fp8": (_int, [_vp, _int, _i64, _vp, _vp, _vp, _sz, _vp]),
     "aq_quant_tensor_fp8_onepass": (_int, [_vp, _int, _i64, _vp, _vp, _vp, _sz, _vp]),
     "aq_gemm_i8_i32": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "aq_linear_w8a8": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _vp, _int, _i64, _i64, _i64, _vp]),

@@ -1395,7 +1395,7 @@ extern "C" int aq_gemv_fp8_decode_residual(const void* x, int x_dtype, const uin
   uint8_t* xq = static_cast<uint8_t*>(ws);
   float* sx = reinterpret_cast<float*>(static_cast<char*>(ws) + aq::align256((size_t)(M * K)));
   uint32_t* amax_ws = reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(sx) + 256);
-  rc = aq_quant_tensor_fp8(x, x_dtype, M * K, xq, sx, amax_ws, stream);
+  rc = aq_quant_tensor_fp8(x, x_dtype, M * K, xq, sx, amax_ws, AQ_FP8_AMAX_WS_BYTES, stream);
   if (rc) return rc;
   return aq_gemv_fp8_codes_residual(xq, sx, wq, sw, bias, bias_dtype, residual, y, y_dtype, M, N, K, stream);
 }

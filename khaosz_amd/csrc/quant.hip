@@ -883,10 +883,11 @@ extern "C" int aq_quant_tensor_fp8_onepass(const void* x, int x_dtype, int64_t n
 }
 
 extern "C" int aq_quant_tensor_fp8(const void* x, int x_dtype, int64_t numel, uint8_t* q,
-                                   float* scale, uint32_t* amax_ws, void* stream) {
+                                   float* scale, uint32_t* amax_ws, size_t ws_bytes, void* stream) {
   if (x_dtype != AQ_F32 && x_dtype != AQ_BF16) return AQ_E_DTYPE;
   if (numel < 0 || (numel % 16) != 0) return AQ_E_SHAPE;
   if (!scale || !amax_ws) return AQ_E_NULL;
+  if (ws_bytes < AQ_FP8_AMAX_WS_BYTES) return AQ_E_WORKSPACE;  // every call writes all of its partial-maximum slots
   if (numel > 0 && (!x || !q)) return AQ_E_NULL;
   if (aq::check_ptr16(x) || aq::check_ptr16(q) || aq::check_ptr(amax_ws, 4) || aq::check_ptr(scale, 4)) return AQ_E_ALIGN;
   hipStream_t st = static_cast<hipStream_t>(stream);

@@ -53,6 +53,32 @@ class Linear(nn.Module):
         return F.linear(x, self.weight, self.bias)
 
 
+class _PerStream:
+    """Scratch tensors a module keeps per (device, stream): the decode workspace, the one-launch quantiser's state.
+    Bounded: the most recently used ``keep`` streams stay, older entries are dropped (a module called from ever
+    new side or capture streams would otherwise grow by a workspace per stream for the life of the model).
+    Keys are raw stream handles, which the runtime may hand out again for a new stream: harmless for a stateless
+    workspace, and for the quantiser's state too, because what it needs is only that calls sharing it do not
+    overlap in time -- which launches on one stream never do -- and every call leaves it in the state the next
+    one accepts."""
+
+    def __init__(self, keep: int = 8):
+        self._keep, self._items = keep, {}
+
+    def get(self, device, make, fits=lambda t: True):
+        key = (device, torch.cuda.current_stream(device).cuda_stream)
+        t = self._items.pop(key, None)
+        if t is None or not fits(t):
+            t = make()
+        self._items[key] = t  # most recently used last
+        while len(self._items) > self._keep:
+            self._items.pop(next(iter(self._items)))
+        return t
+
+    def __len__(self):
+        return len(self._items)
+
+
 def _no_grad_guard(x: Tensor) -> None:
     if torch.is_grad_enabled() and x.requires_grad:
         raise RuntimeError("the quantized Linear is forward-only; call it under torch.no_grad()/inference_mode()")
@@ -78,7 +104,7 @@ class QuantLinear(Linear):
         self.bias = nn.Parameter(torch.zeros(out_dim, device=device), requires_grad=False) if bias else None
         # decode workspaces (activation codes between the row quantiser and the GEMV), one per (device, stream):
         # the same module called from two streams or threads must not share one
-        self._workspaces: dict = {}
+        self._workspaces = _PerStream()
 
     # -- construction -----------------------------------------------------
     @classmethod
@@ -180,10 +206,8 @@ class QuantLinear(Linear):
         if M <= self.DECODE_MAX_ROWS:
             ops._need_gpu(x, self.qweight)
             need = 16 * self.qweight.shape[1] + 512
-            key = (x.device, torch.cuda.current_stream(x.device).cuda_stream)
-            ws = self._workspaces.get(key)
-            if ws is None or ws.numel() < need:
-                ws = self._workspaces[key] = torch.empty((need,), dtype=torch.uint8, device=x.device)
+            ws = self._workspaces.get(x.device, lambda: torch.empty((need,), dtype=torch.uint8, device=x.device),
+                                      lambda t: t.numel() >= need)
             y = ops.gemv_w8a8_decode(x2, self.qweight, self.w_scale, self.bias, out_dtype=x.dtype, workspace=ws,
                                      residual=residual, norm=norm)
         else:
@@ -222,8 +246,8 @@ class Fp8Linear(Linear):
         self.register_buffer("qweight", torch.zeros((out_dim, in_dim), dtype=torch.uint8, device=device))
         self.register_buffer("w_scale", torch.ones((1,), dtype=torch.float32, device=device))
         self.bias = nn.Parameter(torch.zeros(out_dim, device=device), requires_grad=False) if bias else None
-        self._workspaces: dict = {}  # decode workspaces, one per (device, stream), as in QuantLinear
-        self._quant_states: dict = {}  # the one-launch activation quantiser's state, one per (device, stream)
+        self._workspaces = _PerStream()    # decode workspaces, one per (device, stream), as in QuantLinear
+        self._quant_states = _PerStream()  # the one-launch activation quantiser's state, one per (device, stream)
 
     DECODE_MAX_ROWS = 16
 
@@ -267,18 +291,13 @@ class Fp8Linear(Linear):
         if x2.shape[0] <= self.DECODE_MAX_ROWS:  # decode step: the weight-streaming GEMV
             ops._need_gpu(x, self.qweight)
             need = 16 * self.qweight.shape[1] + 2048
-            key = (x.device, torch.cuda.current_stream(x.device).cuda_stream)
-            ws = self._workspaces.get(key)
-            if ws is None or ws.numel() < need:
-                ws = self._workspaces[key] = torch.empty((need,), dtype=torch.uint8, device=x.device)
+            ws = self._workspaces.get(x.device, lambda: torch.empty((need,), dtype=torch.uint8, device=x.device),
+                                      lambda t: t.numel() >= need)
             y = ops.gemv_fp8_decode(x2, self.qweight, self.w_scale, self.bias, out_dtype=x.dtype, workspace=ws,
                                     residual=residual)
         else:
             ops._need_gpu(x, self.qweight)
-            key = (x.device, torch.cuda.current_stream(x.device).cuda_stream)
-            state = self._quant_states.get(key)
-            if state is None:
-                state = self._quant_states[key] = ops.fp8_onepass_state(x.device)
+            state = self._quant_states.get(x.device, lambda: ops.fp8_onepass_state(x.device))
             xq, sx = ops.quant_tensor_fp8(x2, state=state)  # one launch for large inputs
             y = ops.linear_fp8(xq, sx, self.qweight, self.w_scale, self.bias, out_dtype=x.dtype, residual=residual)
         return y.reshape(*lead, self.qweight.shape[0])

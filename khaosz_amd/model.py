@@ -136,8 +136,16 @@ class AutoRegressiveLM(nn.Module):
                 paged_cache.seq_lens = (position_ids[:, 0] + 1).to(torch.int64).contiguous()
             else:
                 mask = _attention_mask(x, position_ids, input_mask)
-        for layer in self.layers:
-            x = layer(x, rotary, mask, paged_cache)
+        if start_pos is not None and isinstance(paged_cache, PagedKV):
+            paged_cache.seq_lens = None  # lengths of an earlier mixed-position step do not apply to this call
+        try:
+            for layer in self.layers:
+                x = layer(x, rotary, mask, paged_cache)
+        finally:
+            # the per-sequence lengths belong to this step only: a later call on the same cache object (a block or
+            # an attention module used directly, another forward) must not find them
+            if isinstance(paged_cache, PagedKV):
+                paged_cache.seq_lens = None
         hidden = self.norm(x)
         return {"logits": self.lm_head(hidden), "hidden_states": hidden}
 

@@ -186,7 +186,7 @@ def quant_tensor_fp8(x: torch.Tensor, state: Optional[torch.Tensor] = None,
     ws = torch.empty((_abi.AQ_FP8_AMAX_WS_BYTES // 4,), dtype=torch.int32, device=x.device)  # partial maxima, stateless
     with _OnDevice(x.device):
         rc = _abi.load().aq_quant_tensor_fp8(xc.data_ptr(), _dt(xc, "x"), n, q.data_ptr(), s.data_ptr(),
-                                             ws.data_ptr(), _stream(x))
+                                             ws.data_ptr(), ws.numel() * 4, _stream(x))
     _abi.check(rc, "aq_quant_tensor_fp8")
     return q, s
 

@@ -245,3 +245,13 @@ def test_gemm_tile_choice_for_the_benchmark_shapes_and_a_few_hundred_rows():
     for M, N in ((8192, 8192), (100000, 4096), (1 << 20, 1 << 20)):
         assert pick(M, N) in (128, 256)
     assert lab.aq_lab_choose_gemm_tile(0, 8, 256) == -2 and lab.aq_lab_choose_gemm_tile(8, 8, 0) == -2
+
+
+def test_quant_tensor_fp8_refuses_a_workspace_smaller_than_its_slots():
+    """aq_quant_tensor_fp8 writes AQ_FP8_AMAX_WS_BYTES of partial maxima: a smaller workspace is refused before
+    anything is launched (argument checks only: runs without a GPU)."""
+    lib = _abi.load()
+    dummy = 4096  # never dereferenced: the size check comes first
+    assert lib.aq_quant_tensor_fp8(dummy, 1, 64, dummy, dummy, dummy, 4, None) == -5
+    assert lib.aq_quant_tensor_fp8(dummy, 1, 64, dummy, dummy, dummy, _abi.AQ_FP8_AMAX_WS_BYTES - 1, None) == -5
+    assert b"workspace" in lib.aq_error_string(-5).lower()

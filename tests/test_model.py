@@ -3,6 +3,7 @@ quantized and fused model against the float one on the GPU."""
 import pytest
 import torch
 
+from khaosz_amd import ops  # noqa: E402
 from khaosz_amd import AutoRegressiveLM, LMConfig, fuse_shared_inputs, quantize_model
 
 TINY = LMConfig(vocab_size=97, dim=64, n_layers=3, n_heads=4, n_kv_heads=2, dim_ffn=176, max_len=64)
@@ -173,7 +174,7 @@ def test_decode_step_with_sequences_at_different_positions_follows_the_reference
         pos = torch.tensor([[S], [17], [S - 40]], device=dev)                 # three sequences, three positions
         la = a(ids[:, S:], paged_cache=ca.bind(table, S + 1), position_ids=pos)["logits"]
         lb = b(ids[:, S:], paged_cache=cb.bind(table, S + 1), position_ids=pos)["logits"]
-        assert cb.seq_lens is not None and cb.seq_lens.tolist() == [S + 1, 18, S - 39]
+        assert cb.seq_lens is None  # the step's per-sequence lengths do not stay behind on the caller's cache
         # every sequence on its own: W8A8 logits through two layers move by about 2 % when the attention
         # numerics change (kernel against stock attention, also in the prefill that filled the caches)
         for i in range(B):
@@ -181,3 +182,30 @@ def test_decode_step_with_sequences_at_different_positions_follows_the_reference
         # the short sequences must NOT see what the long one sees: same step without lengths differs for them
         lc = b(ids[:, S:], paged_cache=cb.bind(table, S + 1), start_pos=S)["logits"]
         assert rel(lc[0], lb[0]) < 2e-2 and rel(lc[1], lb[1]) > 5e-2
+        # Where codes cannot flip -- one layer's attention on the cache this model filled, the same q/k/v for
+        # both sides -- the kernel with per-sequence lengths must match attention under the reference's mask
+        # (transformer.py:40-46) within bf16 rounding, and be far from it without the lengths.
+        att = b.layers[0].attention
+        Hq, Hkv, D = att.n_heads, att.n_kv_heads, att.head_dim
+        T = S + 1
+        lens = (pos[:, 0] + 1).to(torch.int64)
+        g = torch.Generator().manual_seed(61)
+        qkv = torch.randn(B, (Hq + 2 * Hkv) * D, generator=g).to(dt).to(dev)
+        freqs = b._freqs[pos[:, 0]]                                                        # the rotary table rows of the three positions
+        kc, vc = cb.k_layers[0].clone(), cb.v_layers[0].clone()
+        out = ops.rope_paged_attn_decode(qkv, freqs.reshape(B, -1), table, T, kc, vc, Hq, Hkv, seq_lens=lens).float()
+        out_all = ops.rope_paged_attn_decode(qkv, freqs.reshape(B, -1), table, T, kc.clone(), vc.clone(), Hq, Hkv).float()
+        # the reference flow on the same tensors: rotated q, keys / values gathered from the pages (the kernel has
+        # written the new token's into slot T - 1), attention in fp32 under the position mask
+        qr = ops.rope_kv_write(qkv.view(B, 1, -1), freqs.unsqueeze(1), table, T - 1, kc.clone(), vc.clone(), Hq, Hkv)
+        slots = (table[:, :, None] * page + torch.arange(page, device=dev)[None, None, :]).view(B, -1)[:, :T]
+        k = kc.view(-1, Hkv, D)[slots].float().repeat_interleave(Hq // Hkv, dim=2)           # [B, T, Hq, D]
+        v = vc.view(-1, Hkv, D)[slots].float().repeat_interleave(Hq // Hkv, dim=2)
+        allowed = torch.arange(T, device=dev)[None, :] < lens[:, None]
+        mask = torch.zeros(B, 1, 1, T, device=dev).masked_fill_(~allowed[:, None, None, :], float("-inf"))
+        want = torch.nn.functional.scaled_dot_product_attention(qr.view(B, Hq, 1, D).float(), k.transpose(1, 2),
+                                                                v.transpose(1, 2), mask).view(B, Hq, D)
+        for i in range(B):
+            assert rel(out[i], want[i]) < 1e-2, i          # bf16 rounding of the outputs: 2^-9 relative
+        assert rel(out_all[0], want[0]) < 1e-2             # the longest sequence attends to everything anyway
+        assert rel(out_all[1], want[1]) > 0.3              # 18 of 301 positions: without the lengths, another result

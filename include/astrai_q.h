@@ -306,6 +306,26 @@ int aq_rope_paged_attn_decode(const void *qkv, const float *freqs, int64_t freqs
                               float scale, void *out, int64_t B, int64_t Hq, int64_t Hkv, int64_t D,
                               void *workspace, int64_t workspace_bytes, void *stream);
 
+/* The three rotating entry points above for attention with qk-norm (use_qk_norm: RMSNorm modules q_norm / k_norm
+ * over the head dimension, applied to the rotated query and key before the key is cached and the scores are
+ * taken: astrai/model/components/attention.py:62-64, 86-89).  q_gain, k_gain: the two norms' weights, bf16 [D],
+ * 16-byte aligned; eps their epsilon.  The rotated head (as it would be stored, rounded to bf16) is normalised as
+ * y = bf16((x * r) * gain), r = 1 / sqrt(mean(x^2) + eps), with the squares summed in a fixed order (per 8
+ * elements in memory order, the chunk sums by a butterfly over the chunk index) so that the prefill and the decode
+ * kernels store the same bits.  What is cached is the NORMALISED key, as in the reference; a cache filled with
+ * these entry points must be read with them too.  Everything else as in the entry points without the suffix. */
+int aq_rope_kv_write_qknorm(const void *qkv, const float *freqs, int64_t freqs_stride,
+                            const int64_t *page_table, int64_t P, int64_t pos, int64_t S,
+                            int64_t page_size, void *k_cache, void *v_cache, int64_t n_pages,
+                            void *q_out, void *k_out, int64_t B, int64_t Hq, int64_t Hkv, int64_t D,
+                            const void *q_gain, const void *k_gain, float eps, void *stream);
+int aq_rope_paged_attn_decode_qknorm(const void *qkv, const float *freqs, int64_t freqs_stride,
+                                     const int64_t *page_table, int64_t P, int64_t total_len,
+                                     const int64_t *seq_lens, int64_t page_size, void *k_cache, void *v_cache,
+                                     int64_t n_pages, float scale, void *out, int64_t B, int64_t Hq, int64_t Hkv,
+                                     int64_t D, const void *q_gain, const void *k_gain, float eps,
+                                     void *workspace, int64_t workspace_bytes, void *stream);
+
 /* The decode step's attention and output projection without the merge launch
  * in between.  aq_paged_attn_decode_partials / aq_rope_paged_attn_decode_partials
  * are the two calls above stopped before their slices are combined: `partials`
@@ -337,6 +357,13 @@ int aq_rope_paged_attn_decode_partials(const void *qkv, const float *freqs, int6
                                        int64_t n_pages, float scale, int64_t B, int64_t Hq,
                                        int64_t Hkv, int64_t D, void *partials,
                                        int64_t partials_bytes, void *stream);
+/* aq_rope_paged_attn_decode_partials with qk-norm (see aq_rope_paged_attn_decode_qknorm). */
+int aq_rope_paged_attn_decode_partials_qknorm(const void *qkv, const float *freqs, int64_t freqs_stride,
+                                              const int64_t *page_table, int64_t P, int64_t total_len,
+                                              const int64_t *seq_lens, int64_t page_size, void *k_cache,
+                                              void *v_cache, int64_t n_pages, float scale, int64_t B, int64_t Hq,
+                                              int64_t Hkv, int64_t D, const void *q_gain, const void *k_gain,
+                                              float eps, void *partials, int64_t partials_bytes, void *stream);
 int aq_gemv_w8a8_decode_attn(const float *partials, int64_t n_slices, int64_t head_dim,
                              const int8_t *wq, const float *sw, const void *bias, int bias_dtype,
                              const void *residual, void *y, int y_dtype, int64_t M, int64_t N,

@@ -59,6 +59,13 @@ SYMBOLS = {
                                              _i64, _i64, _vp, _i64, _vp]),
     "aq_rope_paged_attn_decode_partials": (_int, [_vp, _vp, _i64, _vp, _i64, _i64, _vp, _i64, _vp, _vp, _i64, ctypes.c_float,
                                                   _i64, _i64, _i64, _i64, _vp, _i64, _vp]),
+    "aq_rope_kv_write_qknorm": (_int, [_vp, _vp, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _vp, _i64, _vp, _vp, _i64, _i64,
+                                       _i64, _i64, _vp, _vp, ctypes.c_float, _vp]),
+    "aq_rope_paged_attn_decode_qknorm": (_int, [_vp, _vp, _i64, _vp, _i64, _i64, _vp, _i64, _vp, _vp, _i64, ctypes.c_float,
+                                                _vp, _i64, _i64, _i64, _i64, _vp, _vp, ctypes.c_float, _vp, _i64, _vp]),
+    "aq_rope_paged_attn_decode_partials_qknorm": (_int, [_vp, _vp, _i64, _vp, _i64, _i64, _vp, _i64, _vp, _vp, _i64,
+                                                         ctypes.c_float, _i64, _i64, _i64, _i64, _vp, _vp, ctypes.c_float,
+                                                         _vp, _i64, _vp]),
     "aq_gemv_w8a8_decode_attn": (_int, [_vp, _i64, _i64, _vp, _vp, _vp, _int, _vp, _vp, _int, _i64, _i64, _i64, _vp]),
     "aq_prefill_attn_paged": (_int, [_vp, _i64, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, ctypes.c_float, _i64, _i64, _i64,
                                      _i64, _i64, _vp]),

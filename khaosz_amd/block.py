@@ -183,8 +183,8 @@ class GQA(nn.Module):
     options: RMSNorm over the head dimension of q and k after the rotation (``use_qk_norm``,
     attention.py:62-64,88-89) and a sigmoid output gate computed from the block input by a fifth
     Linear (``use_gated_attention``, attention.py:66-67,105-106).  Benchmark configuration 5
-    leaves both off; with qk-norm the paged-cache kernels are not used (they store the rotated,
-    un-normalised key)."""
+    leaves both off.  With qk-norm the paged-cache kernels normalise the rotated heads themselves and
+    cache the normalised key, as the reference does."""
 
     def __init__(self, dim: int, n_heads: int, n_kv_heads: int, layer_id: int = 0, use_qk_norm: bool = False,
                  norm_eps: float = 1e-5, use_gated_attention: bool = False):
@@ -225,10 +225,17 @@ class GQA(nn.Module):
         repeating them.  Needs the fused q/k/v projection, bf16, head dimension 64 or 128 and
         1, 2, 3, 4, 6 or 8 query heads per KV head.
         Outputs agree within bf16 rounding."""
-        if (self._qkv is not None and self.head_dim in (64, 128) and not self.use_qk_norm
+        if (self._qkv is not None and self.head_dim in (64, 128)
                 and self.n_heads // self.n_kv_heads in (1, 2, 3, 4, 6, 8)):
             self._decode_attention = True
         return self._decode_attention
+
+    def _qk_norm(self) -> Optional[ops.QkNorm]:
+        """The two head norms for the paged-cache kernels (which compute in bf16 activations)."""
+        if not self.use_qk_norm:
+            return None
+        return ops.QkNorm(self.q_norm.weight.detach().to(torch.bfloat16), self.k_norm.weight.detach().to(torch.bfloat16),
+                          self.q_norm.norm_eps)
 
     def _gated(self, out: Tensor, x: Tensor, norm, codes=None) -> Tensor:
         """``out * sigmoid(gate(x))`` (attention.py:105-106); ``x`` is the attention input, still to
@@ -285,7 +292,7 @@ class GQA(nn.Module):
                                              cache.total_len, cache.k_layers[self.layer_id],
                                              cache.v_layers[self.layer_id], self.n_heads, self.n_kv_heads,
                                              workspace=cache.attn_workspace(self.n_heads), partials=split,
-                                             seq_lens=cache.seq_lens)
+                                             seq_lens=cache.seq_lens, qk_norm=self._qk_norm())
             if split:
                 return self.o_proj.forward_attn(out, x.dtype, residual).view(B, 1, -1)
             return self._out(self._gated(out.view(B, 1, -1), x, norm, codes), residual)
@@ -302,11 +309,12 @@ class GQA(nn.Module):
             direct = start == 0 and cache.all_mapped
             kc, vc = cache.k_layers[self.layer_id], cache.v_layers[self.layer_id]
             if attn_mask is None and not direct:
-                q = ops.rope_kv_write(qkv, rotary_emb, cache.page_table, start, kc, vc, self.n_heads, self.n_kv_heads)
+                q = ops.rope_kv_write(qkv, rotary_emb, cache.page_table, start, kc, vc, self.n_heads, self.n_kv_heads,
+                                      qk_norm=self._qk_norm())
                 out = ops.prefill_attn_paged(q, kc, vc, cache.page_table, start)
                 return self._out(self._gated(out.view(B, S, -1), x, norm, codes), residual)
             q, k = ops.rope_kv_write(qkv, rotary_emb, cache.page_table, start, kc, vc, self.n_heads, self.n_kv_heads,
-                                     return_k=True)
+                                     return_k=True, qk_norm=self._qk_norm())
             if direct:
                 v = qkv[..., nq + nkv:].view(B, S, self.n_kv_heads, self.head_dim)
                 if attn_mask is None:

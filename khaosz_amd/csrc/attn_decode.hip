@@ -55,6 +55,35 @@ __device__ __forceinline__ uint4 rope8(uint4 x, float4 a, float4 b) {
   return make_uint4(o[0], o[1], o[2], o[3]);
 }
 
+// RMSNorm over the head dimension of a rotated query or key (attention.py:62-64, 86-89: after the rotation, before
+// the key goes into the cache).  The rotated values are taken as they are stored, rounded to bf16.  Sum of squares
+// in a fixed order that does not depend on which kernel holds the vector how: per 8-element chunk the rounded
+// squares are added in memory order, then the D / 8 chunk sums are combined by a butterfly over the chunk index
+// (chunk c with c ^ 1, then ^ 2, ^ 4, ^ 8; fl(a + b) is the same whichever partner computes it).  Then
+// r = 1 / sqrt(ss / D + eps) (every operation correctly rounded) and y = bf16((x * r) * gain).
+__device__ __forceinline__ float chunk_sumsq(uint4 x) {
+  const uint32_t in[4] = {x.x, x.y, x.z, x.w};
+  float s = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float x0 = __uint_as_float(in[i] << 16), x1 = __uint_as_float(in[i] & 0xffff0000u);
+    s = __fadd_rn(s, __fmul_rn(x0, x0));
+    s = __fadd_rn(s, __fmul_rn(x1, x1));
+  }
+  return s;
+}
+__device__ __forceinline__ uint4 chunk_normed(uint4 x, float r, uint4 gain) {
+  const uint32_t in[4] = {x.x, x.y, x.z, x.w}, gn[4] = {gain.x, gain.y, gain.z, gain.w};
+  uint32_t o[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float x0 = __uint_as_float(in[i] << 16), x1 = __uint_as_float(in[i] & 0xffff0000u);
+    const float g0 = __uint_as_float(gn[i] << 16), g1 = __uint_as_float(gn[i] & 0xffff0000u);
+    o[i] = pack_bf16x2(__fmul_rn(__fmul_rn(x0, r), g0), __fmul_rn(__fmul_rn(x1, r), g1));
+  }
+  return make_uint4(o[0], o[1], o[2], o[3]);
+}
+
 struct RopeArgs {
   const uint16_t* qkv;   // [B, S, (Hq + 2 Hkv) * D]
   const float* freqs;    // [S, D/2, 2] (cos, sin) per sequence; sequences freqs_stride floats apart (0: shared)
@@ -66,6 +95,9 @@ struct RopeArgs {
   uint16_t* k_out;       // [B, S, Hkv, D] rotated keys, or null
   int64_t P, pos, page, n_pages, S;
   int B, Hq, Hkv, D;
+  const uint16_t* q_gain;  // [D] RMSNorm gains of the rotated q / k heads, or null: no qk-norm
+  const uint16_t* k_gain;
+  float eps;
 };
 
 // one thread per 16-byte chunk (8 elements) of a head vector of a token
@@ -80,6 +112,18 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(RopeArgs p) {
   const int64_t b = tokn / p.S, s = tokn % p.S;
   uint4 x = *reinterpret_cast<const uint4*>(p.qkv + hv * p.D + ch * 8);
   if (h < p.Hq + p.Hkv) x = rope8(x, p.freqs + b * p.freqs_stride + s * p.D + ch * 8);  // v heads do not rotate
+  if (p.q_gain) {  // uniform: qk-norm.  A head vector's D / 8 chunks sit in neighbouring lanes of one DPP row.
+    float ss = chunk_sumsq(x);
+    ss = __fadd_rn(ss, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(ss), 0xB1, 0xf, 0xf, false)));   // c ^ 1
+    ss = __fadd_rn(ss, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(ss), 0x4E, 0xf, 0xf, false)));   // c ^ 2
+    ss = __fadd_rn(ss, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(ss), 0x141, 0xf, 0xf, false)));  // the other quad of the half row: c ^ 4
+    if (p.D == 128)
+      ss = __fadd_rn(ss, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(ss), 0x140, 0xf, 0xf, false)));  // the other half row: c ^ 8
+    if (h < p.Hq + p.Hkv) {
+      const uint16_t* gain = h < p.Hq ? p.q_gain : p.k_gain;
+      x = chunk_normed(x, rms_scale(ss, (float)p.D, p.eps), *reinterpret_cast<const uint4*>(gain + ch * 8));
+    }
+  }
   if (h < p.Hq) {
     *reinterpret_cast<uint4*>(p.q_out + (tokn * p.Hq + h) * p.D + ch * 8) = x;
     return;
@@ -110,6 +154,9 @@ struct AttnArgs {
   int64_t P, T, page, n_pages;
   float scale_log2e;     // softmax scale times log2(e): scores live in the exp2 domain
   int B, Hq, Hkv, NS;
+  const uint16_t* q_gain;  // QKN kernels: [D] RMSNorm gains of the rotated q / k heads
+  const uint16_t* k_gain;
+  float eps;
 };
 
 constexpr int ATT_WAVES = 4;
@@ -164,8 +211,12 @@ typedef float attn_f32x4 __attribute__((ext_vector_type(4)));
 // new key, stores it and the new value into their page slot and uses them from
 // registers instead of what it read from the cache.  Same roundings, so caches
 // and outputs are the bits the two separate launches give.
-template <int G, int D, bool ROPE>
+// QKN (with ROPE): the rotated queries and the rotated new key are RMS-normalised over the head dimension (see
+// chunk_sumsq) before they are used and stored: what rope_kv_write_kernel does with gains, same bits.  A head
+// vector's chunk c = 4 ks + kq sits in register ks of the lane with that kq.
+template <int G, int D, bool ROPE, bool QKN = false>
 __global__ __launch_bounds__(ATT_WAVES * 64) void paged_attn_decode_kernel(AttnArgs p) {
+  static_assert(!QKN || ROPE, "qk-norm belongs to the kernels that rotate");
   constexpr int CPR = D / 8;     // 16-byte chunks per row: 16 or 8
   constexpr int RPL = 64 / CPR;  // rows per load instruction: 4 or 8
   constexpr int NL = 64 / RPL;   // loads per wavefront (= CPR)
@@ -218,6 +269,31 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void paged_attn_decode_kernel(AttnA
         fb[ks] = *reinterpret_cast<const float4*>(cs + 4);
       } else {
         qraw[ks] = *reinterpret_cast<const uint4*>(p.q + ((int64_t)b * p.Hq + kvh * G + hq) * D + d0);
+      }
+    }
+  }
+  // RMSNorm of a rotated head vector held as KS chunks per lane (chunk 4 ks + kq), gains requested by the caller
+  auto head_norm = [&](uint4 (&v)[KS], const uint4 (&gain)[KS]) {
+    float ss[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      ss[ks] = chunk_sumsq(v[ks]);
+      ss[ks] = __fadd_rn(ss[ks], __shfl_xor(ss[ks], 16, 64));  // c ^ 1
+      ss[ks] = __fadd_rn(ss[ks], __shfl_xor(ss[ks], 32, 64));  // c ^ 2
+    }
+    float tot = __fadd_rn(ss[0], ss[1]);                            // c ^ 4
+    if constexpr (KS == 4) tot = __fadd_rn(tot, __fadd_rn(ss[2], ss[3]));  // c ^ 8
+    const float r = rms_scale(tot, (float)D, p.eps);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) v[ks] = chunk_normed(v[ks], r, gain[ks]);
+  };
+  uint4 qgain[KS], kgain[KS];
+  if constexpr (QKN) {
+    if (t0 < T) {
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        qgain[ks] = *reinterpret_cast<const uint4*>(p.q_gain + ks * 32 + kq * 8);
+        kgain[ks] = *reinterpret_cast<const uint4*>(p.k_gain + ks * 32 + kq * 8);
       }
     }
   }
@@ -277,14 +353,18 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void paged_attn_decode_kernel(AttnA
       const int64_t rn = row_of((int)(T - 1 - t0));  // the same in every lane; -1: its page is unmapped
       if (rn >= 0) {
         const int tn = (int)(T - 1 - t0) >> 4, cn = (int)(T - 1 - t0) & 15;  // tile and column of the new key
+        uint4 kn[KS];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+          kn[ks] = rope8(*reinterpret_cast<const uint4*>(tok + (int64_t)(p.Hq + kvh) * D + ks * 32 + kq * 8), fa[ks], fb[ks]);
+        if constexpr (QKN) head_norm(kn, kgain);  // (every column holds the same new key: all lanes take part)
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
           const int d0 = ks * 32 + kq * 8;
-          const uint4 kn = rope8(*reinterpret_cast<const uint4*>(tok + (int64_t)(p.Hq + kvh) * D + d0), fa[ks], fb[ks]);
-          if (col == cn) *reinterpret_cast<uint4*>(p.kc_w + rn + d0) = kn;
+          if (col == cn) *reinterpret_cast<uint4*>(p.kc_w + rn + d0) = kn[ks];
 #pragma unroll
           for (int t = 0; t < 4; ++t)
-            if (t == tn && col == cn) kb[t][ks] = kn;
+            if (t == tn && col == cn) kb[t][ks] = kn[ks];
         }
         const uint4 vn = *reinterpret_cast<const uint4*>(tok + (int64_t)(p.Hq + p.Hkv + kvh) * D + ch * 8);
         const int in = (int)(T - 1 - t0) / RPL, sn = (int)(T - 1 - t0) % RPL;  // load and key group of the new value
@@ -302,6 +382,10 @@ __global__ __launch_bounds__(ATT_WAVES * 64) void paged_attn_decode_kernel(AttnA
         qa[ks] = rope8(qraw[ks], fa[ks], fb[ks]);
       else
         qa[ks] = qraw[ks];
+    }
+    if constexpr (QKN) head_norm(qa, qgain);  // (columns past G normalise a copy of head 0 and are zeroed below)
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
       if (col >= G) qa[ks] = make_uint4(0, 0, 0, 0);
     }
     // ---- scores: S[head][key] per tile; this lane gets key col of the tile, heads 4 kq .. + 4
@@ -481,11 +565,14 @@ inline int64_t attn_workspace_bytes(int64_t B, int64_t Hq, int64_t ns) {
 
 }  // namespace aq
 
-extern "C" int aq_rope_kv_write(const void* qkv, const float* freqs, int64_t freqs_stride, const int64_t* page_table,
-                                int64_t P, int64_t pos, int64_t S, int64_t page_size, void* k_cache, void* v_cache,
-                                int64_t n_pages, void* q_out, void* k_out, int64_t B, int64_t Hq, int64_t Hkv, int64_t D,
-                                void* stream) {
+// q_gain == nullptr: no qk-norm (then k_gain and eps are not looked at)
+static int rope_kv_write(const void* qkv, const float* freqs, int64_t freqs_stride, const int64_t* page_table,
+                         int64_t P, int64_t pos, int64_t S, int64_t page_size, void* k_cache, void* v_cache,
+                         int64_t n_pages, void* q_out, void* k_out, int64_t B, int64_t Hq, int64_t Hkv, int64_t D,
+                         const void* q_gain, const void* k_gain, float eps, void* stream) {
   if (D != 64 && D != 128) return AQ_E_SHAPE;
+  if (q_gain && (!k_gain || !(eps >= 0.0f))) return k_gain ? AQ_E_SHAPE : AQ_E_NULL;
+  if (aq::check_ptr16(q_gain) || (q_gain && aq::check_ptr16(k_gain))) return AQ_E_ALIGN;
   if (B < 0 || S < 0 || Hq <= 0 || Hkv <= 0 || P <= 0 || pos < 0 || page_size <= 0 || n_pages <= 0) return AQ_E_SHAPE;
   if (freqs_stride != 0 && freqs_stride < S * D) return AQ_E_SHAPE;
   if (B == 0 || S == 0) return AQ_OK;
@@ -513,9 +600,30 @@ extern "C" int aq_rope_kv_write(const void* qkv, const float* freqs, int64_t fre
   a.Hq = (int)Hq;
   a.Hkv = (int)Hkv;
   a.D = (int)D;
+  a.q_gain = static_cast<const uint16_t*>(q_gain);
+  a.k_gain = static_cast<const uint16_t*>(k_gain);
+  a.eps = eps;
   hipLaunchKernelGGL(aq::rope_kv_write_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0,
                      static_cast<hipStream_t>(stream), a);
   return (int)hipGetLastError();
+}
+
+extern "C" int aq_rope_kv_write(const void* qkv, const float* freqs, int64_t freqs_stride, const int64_t* page_table,
+                                int64_t P, int64_t pos, int64_t S, int64_t page_size, void* k_cache, void* v_cache,
+                                int64_t n_pages, void* q_out, void* k_out, int64_t B, int64_t Hq, int64_t Hkv, int64_t D,
+                                void* stream) {
+  return rope_kv_write(qkv, freqs, freqs_stride, page_table, P, pos, S, page_size, k_cache, v_cache, n_pages, q_out, k_out,
+                       B, Hq, Hkv, D, nullptr, nullptr, 0.0f, stream);
+}
+
+extern "C" int aq_rope_kv_write_qknorm(const void* qkv, const float* freqs, int64_t freqs_stride,
+                                       const int64_t* page_table, int64_t P, int64_t pos, int64_t S, int64_t page_size,
+                                       void* k_cache, void* v_cache, int64_t n_pages, void* q_out, void* k_out, int64_t B,
+                                       int64_t Hq, int64_t Hkv, int64_t D, const void* q_gain, const void* k_gain,
+                                       float eps, void* stream) {
+  if (!q_gain || !k_gain) return AQ_E_NULL;
+  return rope_kv_write(qkv, freqs, freqs_stride, page_table, P, pos, S, page_size, k_cache, v_cache, n_pages, q_out, k_out,
+                       B, Hq, Hkv, D, q_gain, k_gain, eps, stream);
 }
 
 extern "C" int64_t aq_paged_attn_decode_workspace_bytes(int64_t B, int64_t Hq, int64_t Hkv, int64_t total_len) {
@@ -526,7 +634,9 @@ extern "C" int64_t aq_paged_attn_decode_workspace_bytes(int64_t B, int64_t Hq, i
 
 template <int G, int D>
 static void attn_launch(bool rope, dim3 grid, dim3 block, hipStream_t st, const aq::AttnArgs& a) {
-  if (rope)
+  if (rope && a.q_gain)
+    hipLaunchKernelGGL((aq::paged_attn_decode_kernel<G, D, true, true>), grid, block, 0, st, a);
+  else if (rope)
     hipLaunchKernelGGL((aq::paged_attn_decode_kernel<G, D, true>), grid, block, 0, st, a);
   else
     hipLaunchKernelGGL((aq::paged_attn_decode_kernel<G, D, false>), grid, block, 0, st, a);
@@ -538,9 +648,13 @@ static int attn_decode(const void* q, const void* qkv, const float* freqs, int64
                        void* v_cache, const int64_t* page_table, int64_t P, int64_t total_len,
                        const int64_t* seq_lens, int64_t page_size,
                        int64_t n_pages, float scale, void* out, int64_t B, int64_t Hq, int64_t Hkv, int64_t D,
-                       void* workspace, int64_t workspace_bytes, void* stream, bool partials = false) {
+                       void* workspace, int64_t workspace_bytes, void* stream, bool partials = false,
+                       const void* q_gain = nullptr, const void* k_gain = nullptr, float eps = 0.0f) {
   const bool rope = q == nullptr;
   if (D != 64 && D != 128) return AQ_E_SHAPE;
+  if (q_gain && (!rope || !k_gain)) return AQ_E_NULL;  // qk-norm belongs to the forms that rotate
+  if (q_gain && !(eps >= 0.0f)) return AQ_E_SHAPE;
+  if (aq::check_ptr16(q_gain) || (q_gain && aq::check_ptr16(k_gain))) return AQ_E_ALIGN;
   if (B < 0 || Hq <= 0 || Hkv <= 0 || (Hq % Hkv) != 0 || P <= 0 || total_len <= 0 || page_size <= 0 ||
       n_pages <= 0 || !(scale > 0.0f))
     return AQ_E_SHAPE;
@@ -584,6 +698,9 @@ static int attn_decode(const void* q, const void* qkv, const float* freqs, int64
   a.Hq = (int)Hq;
   a.Hkv = (int)Hkv;
   a.NS = (int)ns;
+  a.q_gain = static_cast<const uint16_t*>(q_gain);
+  a.k_gain = static_cast<const uint16_t*>(k_gain);
+  a.eps = eps;
   const dim3 grid((unsigned)(B * Hkv * ns)), block(aq::ATT_WAVES * 64);
   hipStream_t st = static_cast<hipStream_t>(stream);
 #define AQ_ATTN_CASE(G_)                                            \
@@ -656,4 +773,29 @@ extern "C" int aq_rope_paged_attn_decode_partials(const void* qkv, const float* 
   if ((!qkv || !freqs) && B > 0) return AQ_E_NULL;
   return attn_decode(nullptr, qkv, freqs, freqs_stride, k_cache, v_cache, page_table, P, total_len, seq_lens, page_size, n_pages,
                      scale, nullptr, B, Hq, Hkv, D, partials, partials_bytes, stream, true);
+}
+
+extern "C" int aq_rope_paged_attn_decode_qknorm(const void* qkv, const float* freqs, int64_t freqs_stride,
+                                                const int64_t* page_table, int64_t P, int64_t total_len,
+                                                const int64_t* seq_lens, int64_t page_size, void* k_cache, void* v_cache,
+                                                int64_t n_pages, float scale, void* out, int64_t B, int64_t Hq,
+                                                int64_t Hkv, int64_t D, const void* q_gain, const void* k_gain, float eps,
+                                                void* workspace, int64_t workspace_bytes, void* stream) {
+  if ((!qkv || !freqs) && B > 0) return AQ_E_NULL;
+  if (!q_gain || !k_gain) return AQ_E_NULL;
+  return attn_decode(nullptr, qkv, freqs, freqs_stride, k_cache, v_cache, page_table, P, total_len, seq_lens, page_size, n_pages,
+                     scale, out, B, Hq, Hkv, D, workspace, workspace_bytes, stream, false, q_gain, k_gain, eps);
+}
+
+extern "C" int aq_rope_paged_attn_decode_partials_qknorm(const void* qkv, const float* freqs, int64_t freqs_stride,
+                                                         const int64_t* page_table, int64_t P, int64_t total_len,
+                                                         const int64_t* seq_lens, int64_t page_size, void* k_cache,
+                                                         void* v_cache, int64_t n_pages, float scale, int64_t B,
+                                                         int64_t Hq, int64_t Hkv, int64_t D, const void* q_gain,
+                                                         const void* k_gain, float eps, void* partials,
+                                                         int64_t partials_bytes, void* stream) {
+  if ((!qkv || !freqs) && B > 0) return AQ_E_NULL;
+  if (!q_gain || !k_gain) return AQ_E_NULL;
+  return attn_decode(nullptr, qkv, freqs, freqs_stride, k_cache, v_cache, page_table, P, total_len, seq_lens, page_size, n_pages,
+                     scale, nullptr, B, Hq, Hkv, D, partials, partials_bytes, stream, true, q_gain, k_gain, eps);
 }

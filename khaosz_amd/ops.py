@@ -428,27 +428,57 @@ def _rope_args(qkv, freqs, page_table, k_cache, v_cache, n_heads, n_kv_heads, wh
     return qkv.contiguous(), fr, fr_stride, page_table.contiguous()
 
 
+class QkNorm(NamedTuple):
+    """Attention's qk-norm (``use_qk_norm``, astrai/model/components/attention.py:62-64, 86-89): the weights of the
+    RMSNorm modules over the head dimension that follow the rotation of q and of k, and their epsilon."""
+    q_gain: torch.Tensor
+    k_gain: torch.Tensor
+    eps: float
+
+
+def _qk_norm_args(qk_norm, D: int, dev):
+    """``(q_gain, k_gain, eps)`` checked for the kernels: bfloat16 ``[D]`` on ``dev``, 16-byte aligned."""
+    if qk_norm is None:
+        return None
+    qg, kg, eps = qk_norm
+    out = []
+    for g in (qg, kg):
+        if g.dtype != torch.bfloat16 or g.numel() != D or g.device != dev:
+            raise ValueError(f"qk-norm gains must be bfloat16 [{D}] on {dev}, got {g.dtype} {tuple(g.shape)} on {g.device}")
+        g = g.reshape(D).contiguous()
+        out.append(g if g.data_ptr() % 16 == 0 else g.clone())
+    if not eps >= 0.0:
+        raise ValueError("qk-norm eps must not be negative")
+    return out[0], out[1], float(eps)
+
+
 def rope_kv_write(qkv: torch.Tensor, freqs: torch.Tensor, page_table: torch.Tensor, pos: int, k_cache: torch.Tensor,
-                  v_cache: torch.Tensor, n_heads: int, n_kv_heads: int, return_k: bool = False):
+                  v_cache: torch.Tensor, n_heads: int, n_kv_heads: int, return_k: bool = False,
+                  qk_norm: Optional[QkNorm] = None):
     """New tokens of every sequence -- ``qkv [B, (Hq + 2 Hkv) * D]`` (one each, D = 64 or 128) or ``[B, S, ...]``:
     rotate q and k by ``freqs`` (complex64 ``[B, (S,) 64]`` or float32 ``[B, (S,) 64, 2]``), write k and
     v into the paged caches ``[n_pages, page, Hkv, D]`` at logical positions ``pos .. pos + S - 1``;
     returns the rotated ``q [B, (S,) Hq, D]``, and with ``return_k`` also the rotated
-    ``k [B, (S,) Hkv, D]``."""
+    ``k [B, (S,) Hkv, D]``.  With ``qk_norm`` the rotated q and k heads are RMS-normalised over D before they are
+    returned and cached."""
     one = qkv.dim() == 2
     qkv, fr, fr_stride, page_table = _rope_args(qkv, freqs, page_table, k_cache, v_cache, n_heads, n_kv_heads,
                                                 "rope_kv_write")
     B, S, D = qkv.shape[0], qkv.shape[1], k_cache.shape[-1]
     q = torch.empty((B, S, n_heads, D), dtype=torch.bfloat16, device=qkv.device)
     k = torch.empty((B, S, n_kv_heads, D), dtype=torch.bfloat16, device=qkv.device) if return_k else None
+    norm = _qk_norm_args(qk_norm, D, qkv.device)
     if B and S:
+        head = (qkv.data_ptr(), fr.data_ptr(), fr_stride, page_table.data_ptr(), page_table.shape[1], int(pos), S,
+                k_cache.shape[1], k_cache.data_ptr(), v_cache.data_ptr(), k_cache.shape[0], q.data_ptr(),
+                k.data_ptr() if return_k else None, B, n_heads, n_kv_heads, D)
         with _OnDevice(qkv.device):
-            rc = _abi.load().aq_rope_kv_write(qkv.data_ptr(), fr.data_ptr(), fr_stride, page_table.data_ptr(),
-                                              page_table.shape[1], int(pos), S, k_cache.shape[1], k_cache.data_ptr(),
-                                              v_cache.data_ptr(), k_cache.shape[0], q.data_ptr(),
-                                              k.data_ptr() if return_k else None, B, n_heads, n_kv_heads, D,
-                                              _stream(qkv))
-        _abi.check(rc, "aq_rope_kv_write")
+            if norm is None:
+                rc = _abi.load().aq_rope_kv_write(*head, _stream(qkv))
+            else:
+                rc = _abi.load().aq_rope_kv_write_qknorm(*head, norm[0].data_ptr(), norm[1].data_ptr(), norm[2],
+                                                         _stream(qkv))
+        _abi.check(rc, "aq_rope_kv_write" if norm is None else "aq_rope_kv_write_qknorm")
     if one:
         q, k = q.squeeze(1), (k.squeeze(1) if return_k else None)
     return (q, k) if return_k else q
@@ -493,12 +523,14 @@ def attn_gemv_fusable(B: int, n_heads: int, head_dim: int, total_len: int) -> bo
 def rope_paged_attn_decode(qkv: torch.Tensor, freqs: torch.Tensor, page_table: torch.Tensor, total_len: int,
                            k_cache: torch.Tensor, v_cache: torch.Tensor, n_heads: int, n_kv_heads: int,
                            scale: Optional[float] = None, workspace: Optional[torch.Tensor] = None,
-                           partials: bool = False, seq_lens: Optional[torch.Tensor] = None):
+                           partials: bool = False, seq_lens: Optional[torch.Tensor] = None,
+                           qk_norm: Optional[QkNorm] = None):
     """``rope_kv_write`` at position ``total_len - 1`` and ``paged_attn_decode`` over ``total_len``
     positions as one launch (plus the small merge launch for long sequences): same caches and
     outputs, bit for bit.  Returns the attention output ``[B, Hq, D]`` -- or, with ``partials``,
     the slices' partial results (no merge launch) for ``gemv_w8a8_attn`` to combine.
-    ``seq_lens`` (int64 ``[B]`` on the device): sequence b attends to its first ``seq_lens[b]`` positions only."""
+    ``seq_lens`` (int64 ``[B]`` on the device): sequence b attends to its first ``seq_lens[b]`` positions only.
+    ``qk_norm``: as in ``rope_kv_write``, same bits."""
     if qkv.dim() != 2:
         raise ValueError(f"one new token per sequence: qkv must be [B, W], got {tuple(qkv.shape)}")
     qkv, fr, fr_stride, page_table = _rope_args(qkv, freqs, page_table, k_cache, v_cache, n_heads, n_kv_heads,
@@ -509,6 +541,9 @@ def rope_paged_attn_decode(qkv: torch.Tensor, freqs: torch.Tensor, page_table: t
     lib = _abi.load()
     scale = float(scale if scale is not None else D ** -0.5)
     lens_ptr = _seq_lens_ptr(seq_lens, B, qkv.device)
+    norm = _qk_norm_args(qk_norm, D, qkv.device)
+    tail = () if norm is None else (norm[0].data_ptr(), norm[1].data_ptr(), norm[2])
+    suffix = "" if norm is None else "_qknorm"
     if partials:
         if not B:
             raise ValueError("partial results need at least one sequence")
@@ -516,25 +551,27 @@ def rope_paged_attn_decode(qkv: torch.Tensor, freqs: torch.Tensor, page_table: t
         if (workspace is None or not workspace.is_contiguous() or workspace.device != qkv.device
                 or workspace.dtype != torch.float32 or workspace.numel() * 4 < need or workspace.data_ptr() % 16):
             workspace = torch.empty(need // 4, dtype=torch.float32, device=qkv.device)
+        entry = "aq_rope_paged_attn_decode_partials" + suffix
         with _OnDevice(qkv.device):
-            rc = lib.aq_rope_paged_attn_decode_partials(qkv.data_ptr(), fr.data_ptr(), fr_stride, page_table.data_ptr(),
-                                                        page_table.shape[1], int(total_len), lens_ptr, k_cache.shape[1],
-                                                        k_cache.data_ptr(), v_cache.data_ptr(), k_cache.shape[0],
-                                                        scale, B, n_heads, n_kv_heads, D, workspace.data_ptr(),
-                                                        workspace.numel() * 4, _stream(qkv))
-        _abi.check(rc, "aq_rope_paged_attn_decode_partials")
+            rc = getattr(lib, entry)(qkv.data_ptr(), fr.data_ptr(), fr_stride, page_table.data_ptr(),
+                                     page_table.shape[1], int(total_len), lens_ptr, k_cache.shape[1],
+                                     k_cache.data_ptr(), v_cache.data_ptr(), k_cache.shape[0],
+                                     scale, B, n_heads, n_kv_heads, D, *tail, workspace.data_ptr(),
+                                     workspace.numel() * 4, _stream(qkv))
+        _abi.check(rc, entry)
         return AttnPartials(workspace, int(lib.aq_paged_attn_decode_slices(int(total_len))), B, n_heads, D)
     out = torch.empty((B, n_heads, D), dtype=torch.bfloat16, device=qkv.device)
     if B:
         ws_ptr, ws_bytes = _attn_workspace(workspace, paged_attn_workspace_bytes(B, n_heads, n_kv_heads, total_len),
                                            qkv.device)
+        entry = "aq_rope_paged_attn_decode" + suffix
         with _OnDevice(qkv.device):
-            rc = lib.aq_rope_paged_attn_decode(qkv.data_ptr(), fr.data_ptr(), fr_stride, page_table.data_ptr(),
-                                               page_table.shape[1], int(total_len), lens_ptr, k_cache.shape[1],
-                                               k_cache.data_ptr(), v_cache.data_ptr(), k_cache.shape[0], scale,
-                                               out.data_ptr(), B, n_heads, n_kv_heads, D, ws_ptr, ws_bytes,
-                                               _stream(qkv))
-        _abi.check(rc, "aq_rope_paged_attn_decode")
+            rc = getattr(lib, entry)(qkv.data_ptr(), fr.data_ptr(), fr_stride, page_table.data_ptr(),
+                                     page_table.shape[1], int(total_len), lens_ptr, k_cache.shape[1],
+                                     k_cache.data_ptr(), v_cache.data_ptr(), k_cache.shape[0], scale,
+                                     out.data_ptr(), B, n_heads, n_kv_heads, D, *tail, ws_ptr, ws_bytes,
+                                     _stream(qkv))
+        _abi.check(rc, entry)
     return out
 
 

@@ -54,6 +54,10 @@
  *                         restatement bit for bit (numpy has no fma: the comparison
  *                         runs the polynomial in float64 products rounded once, which
  *                         is what an fma is), and on closed forms (g = 0, large |g|).
+ *   oq_rope_kv_write_qknorm  the RMSNorm of the rotated heads (attention.py:86-89), pinned against
+ *                         F.rms_norm applied to oq_rope_kv_write's heads (within one bf16
+ *                         step), against an independent numpy restatement bit for bit,
+ *                         and on closed forms (constant heads, unit gain, v untouched).
  *   oq_rope_kv_write,     restate apply_rotary_emb (rope.py:26-33), Storage.write / gather
  *   oq_paged_attn_decode  (cache.py:216-274), repeat_kv and softmax attention
  *                         (attention.py:15-23,93-103) for one new token per sequence;
@@ -331,9 +335,10 @@ void oq_swiglu_quant_i8_bf16(const uint16_t *ug, int64_t M, int64_t F, int64_t l
  * and v go to slot pos % page of page table[b, pos / page] of the caches
  * [n_pages, page, Hkv, D]; sequences whose page is unmapped are skipped
  * (cache.py:216-252). */
-void oq_rope_kv_write(const uint16_t *qkv, const float *freqs, const int64_t *table, int64_t P,
-                      int64_t pos, int64_t page, uint16_t *kc, uint16_t *vc, int64_t n_pages,
-                      uint16_t *q_out, int64_t B, int64_t Hq, int64_t Hkv, int64_t D) {
+static void rope_kv_write(const uint16_t *qkv, const float *freqs, const int64_t *table, int64_t P,
+                          int64_t pos, int64_t page, uint16_t *kc, uint16_t *vc, int64_t n_pages,
+                          uint16_t *q_out, int64_t B, int64_t Hq, int64_t Hkv, int64_t D,
+                          const uint16_t *q_gain, const uint16_t *k_gain, float eps) {
   const int64_t heads = Hq + 2 * Hkv;
   for (int64_t b = 0; b < B; ++b) {
     const int64_t lp = pos / page;
@@ -353,6 +358,31 @@ void oq_rope_kv_write(const uint16_t *qkv, const float *freqs, const int64_t *ta
           tmp[2 * i + 1] = src[2 * i + 1];
         }
       }
+      if (q_gain && h < Hq + Hkv) {
+        /* RMSNorm over the head (attention.py:62-64, 86-89; norm.py:14-15), on the rotated head as bf16 holds
+         * it: y = bf16((x * r) * gain), r = 1 / sqrt(sum / D + eps).  The squares are summed per 8 elements in
+         * memory order, those sums pairwise over the chunk index (c, c ^ 1, then ^ 2, ^ 4, ^ 8). */
+        const uint16_t *gain = h < Hq ? q_gain : k_gain;
+        float part[128];
+        int64_t n = D / 8;
+        for (int64_t c = 0; c < n; ++c) {
+          float acc = 0.0f;
+          for (int64_t e = 0; e < 8; ++e) {
+            const float x = oq_bf16_to_f32(tmp[c * 8 + e]);
+            const float sq = x * x;
+            acc = acc + sq;
+          }
+          part[c] = acc;
+        }
+        for (; n > 1; n /= 2)
+          for (int64_t c = 0; c < n / 2; ++c) part[c] = part[2 * c] + part[2 * c + 1];
+        const float mean = part[0] / (float)D;
+        const float r = 1.0f / sqrtf(mean + eps);
+        for (int64_t i = 0; i < D; ++i) {
+          const float xr = oq_bf16_to_f32(tmp[i]) * r;
+          tmp[i] = oq_f32_to_bf16(xr * oq_bf16_to_f32(gain[i]));
+        }
+      }
       if (h < Hq) {
         memcpy(q_out + (b * Hq + h) * D, tmp, (size_t)D * 2);
       } else if (phys >= 0 && phys < n_pages) {
@@ -363,6 +393,21 @@ void oq_rope_kv_write(const uint16_t *qkv, const float *freqs, const int64_t *ta
       }
     }
   }
+}
+
+void oq_rope_kv_write(const uint16_t *qkv, const float *freqs, const int64_t *table, int64_t P,
+                      int64_t pos, int64_t page, uint16_t *kc, uint16_t *vc, int64_t n_pages,
+                      uint16_t *q_out, int64_t B, int64_t Hq, int64_t Hkv, int64_t D) {
+  rope_kv_write(qkv, freqs, table, P, pos, page, kc, vc, n_pages, q_out, B, Hq, Hkv, D, NULL, NULL, 0.0f);
+}
+
+/* oq_rope_kv_write for attention with qk-norm: the rotated q and k heads go through RMSNorm modules over D
+ * (gains bf16 [D]) before q is returned and k is cached; v is untouched. */
+void oq_rope_kv_write_qknorm(const uint16_t *qkv, const float *freqs, const int64_t *table, int64_t P,
+                             int64_t pos, int64_t page, uint16_t *kc, uint16_t *vc, int64_t n_pages,
+                             uint16_t *q_out, int64_t B, int64_t Hq, int64_t Hkv, int64_t D,
+                             const uint16_t *q_gain, const uint16_t *k_gain, float eps) {
+  rope_kv_write(qkv, freqs, table, P, pos, page, kc, vc, n_pages, q_out, B, Hq, Hkv, D, q_gain, k_gain, eps);
 }
 
 /* out[b, h, :] = softmax_t(scale * q[b,h] . K[b,t,h/G]) V[b,t,h/G], t < T, read through

@@ -231,6 +231,8 @@ def _load():
     lib.oq_exp_repro.argtypes = [ctypes.c_float]
     lib.oq_exp_repro.restype = ctypes.c_float
     lib.oq_rope_kv_write.argtypes = [vp, vp, vp, i64, i64, i64, vp, vp, i64, vp, i64, i64, i64, i64]
+    lib.oq_rope_kv_write_qknorm.argtypes = [vp, vp, vp, i64, i64, i64, vp, vp, i64, vp, i64, i64, i64, i64, vp, vp,
+                                            ctypes.c_float]
     lib.oq_paged_attn_decode.argtypes = [vp, vp, vp, vp, i64, i64, vp, i64, i64, ctypes.c_float, vp, i64, i64, i64, i64]
     lib.oq_prefill_attn_causal.argtypes = [vp, vp, vp, ctypes.c_float, vp, i64, i64, i64, i64, i64]
     lib.oq_prefill_attn_offset.argtypes = [vp, vp, vp, ctypes.c_float, vp, i64, i64, i64, i64, i64, i64]
@@ -249,6 +251,7 @@ def _load():
         "oq_dequant_epilogue oq_linear_w8a8_f32 oq_linear_w8a8_bf16 oq_quant_tensor_fp8_f32 "
         "oq_quant_tensor_fp8_bf16 oq_linear_fp8 oq_linear_f32 oq_rmsnorm_quant_i8_f32 oq_rmsnorm_quant_i8_bf16 "
         "oq_swiglu_quant_i8_f32 oq_swiglu_quant_i8_bf16 oq_rope_kv_write oq_paged_attn_decode oq_prefill_attn_causal "
+        "oq_rope_kv_write_qknorm "
         "oq_prefill_attn_offset"
     ).split():
         getattr(lib, name).restype = None
@@ -330,17 +333,42 @@ def c_swiglu_quant_i8(ug: np.ndarray, bf16_bits: bool = False, want_h: bool = Fa
     return (q, s, h) if want_h else (q, s)
 
 
-def c_rope_kv_write(qkv, freqs, table, pos, kc, vc, Hq, Hkv):
+def np_head_rmsnorm_bits(x_bits: np.ndarray, gain_bits: np.ndarray, eps: float) -> np.ndarray:
+    """RMSNorm over the last axis of bf16 head vectors ``[..., D]`` (D a power of two times 8) as the
+    qk-norm kernels do it: squares summed per 8 elements in memory order, the chunk sums pairwise over
+    the chunk index; ``bf16((x * r) * gain)``.  Bit patterns in and out."""
+    x = np_bf16_bits_to_f32(x_bits)
+    D = x.shape[-1]
+    sq = (x * x).astype(F32).reshape(*x.shape[:-1], D // 8, 8)
+    part = np.zeros(sq.shape[:-1], F32)
+    for e in range(8):
+        part = (part + sq[..., e]).astype(F32)
+    while part.shape[-1] > 1:
+        part = (part[..., 0::2] + part[..., 1::2]).astype(F32)
+    mean = (part / F32(D)).astype(F32)
+    r = (F32(1.0) / np.sqrt((mean + F32(eps)).astype(F32)).astype(F32)).astype(F32)
+    y = ((x * r).astype(F32) * np_bf16_bits_to_f32(gain_bits)).astype(F32)
+    return np_f32_to_bf16_bits(y)
+
+
+def c_rope_kv_write(qkv, freqs, table, pos, kc, vc, Hq, Hkv, qk_norm=None):
     """bf16 bit patterns (uint16) throughout; kc / vc [n_pages, page, Hkv, D] are updated in place.
-    Returns the rotated q [B, Hq, D]."""
+    Returns the rotated q [B, Hq, D].  ``qk_norm = (q_gain bits [D], k_gain bits [D], eps)``: the
+    rotated q and k heads are RMS-normalised over D (attention.py:86-89)."""
     lib = _load()
     qkv, freqs, table = _c(qkv, np.uint16), _c(freqs, F32), _c(table, np.int64)
     assert kc.dtype == np.uint16 and vc.dtype == np.uint16 and kc.flags.c_contiguous and vc.flags.c_contiguous
     B = qkv.shape[0]
     n_pages, page, _, D = kc.shape
     q = np.empty((B, Hq, D), np.uint16)
-    lib.oq_rope_kv_write(_p(qkv), _p(freqs), _p(table), table.shape[1], pos, page, _p(kc), _p(vc), n_pages, _p(q),
-                         B, Hq, Hkv, D)
+    if qk_norm is None:
+        lib.oq_rope_kv_write(_p(qkv), _p(freqs), _p(table), table.shape[1], pos, page, _p(kc), _p(vc), n_pages, _p(q),
+                             B, Hq, Hkv, D)
+    else:
+        qg, kg = _c(qk_norm[0], np.uint16), _c(qk_norm[1], np.uint16)
+        assert qg.shape == (D,) and kg.shape == (D,)
+        lib.oq_rope_kv_write_qknorm(_p(qkv), _p(freqs), _p(table), table.shape[1], pos, page, _p(kc), _p(vc), n_pages,
+                                    _p(q), B, Hq, Hkv, D, _p(qg), _p(kg), float(qk_norm[2]))
     return q
 
 

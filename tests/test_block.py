@@ -115,7 +115,7 @@ def test_gqa_options_qk_norm_and_output_gate_by_hand():
     blk(xs[:, :S], _freqs(tab, B, 0, S), None, cache.bind(S))
     step = blk(xs[:, S:], _freqs(tab, B, S, 1), decode_mask(B, S + 1, "cpu", torch.float32), cache.bind(S + 1))
     assert torch.allclose(step[:, 0], full[:, S], atol=1e-5)
-    assert not blk.attention.fuse_decode_attention()           # never with qk-norm
+    assert not blk.attention.fuse_decode_attention()           # needs the fused, quantized q/k/v projection
 
 
 def _block(dim=64, heads=4, kv=2, ffn=176, seed=0):
@@ -686,3 +686,59 @@ def test_config5_full_size_fused_block_against_the_unfused_block_and_an_oracle_c
     # the MLP half on the bits the GPU's attention half produced: norm + quantise, up/gate + SwiGLU, quantise,
     # down and the residual add, bit for bit
     assert np.array_equal(bits(out_gpu.reshape(B, dim)), mlp_half(bits(h_gpu.reshape(B, dim))))
+
+
+@pytest.mark.gpu
+def test_qk_norm_block_through_the_paged_cache_kernels_tracks_the_stock_path():
+    """use_qk_norm with the paged-cache kernels: they normalise the rotated heads and cache the normalised
+    key (attention.py:86-92).  Against the same quantized block on gather / repeat_kv / stock attention:
+    prompt, a chunk on top of cached tokens, decode steps in one slice and in several; cache contents
+    within one bf16 step, outputs within bf16 rounding."""
+    from khaosz_amd import fuse_shared_inputs
+
+    dev, dt = "cuda:0", torch.bfloat16
+    for dim, heads, kv, S in ((512, 4, 2, 70), (512, 8, 2, 290)):       # head dimension 128 and 64
+        torch.manual_seed(11)
+        a = DecoderBlock(dim, heads, 1408, kv, use_qk_norm=True)
+        a.reset_parameters()
+        with torch.no_grad():
+            a.attention.q_norm.weight.add_(0.3 * torch.randn_like(a.attention.q_norm.weight))
+            a.attention.k_norm.weight.add_(0.3 * torch.randn_like(a.attention.k_norm.weight))
+        a = a.to(dev).to(dt)
+        b = DecoderBlock(dim, heads, 1408, kv, use_qk_norm=True).to(dev).to(dt)
+        b.load_state_dict(a.state_dict())
+        quantize_model(a), quantize_model(b)
+        fuse_shared_inputs(a)
+        fuse_shared_inputs(b, decode_attention=True)
+        assert b.attention._decode_attention and not a.attention._decode_attention
+        D = dim // heads
+        B, steps, page = 3, 3, 16
+        P = (S + steps + 5 + page - 1) // page
+        tab = rotary_table(D, 512, device=dev)
+        table = torch.randperm(B * P, device=dev).view(B, P)
+        ca, cb = PagedKV(B * P, page, kv, D, dev, dt), PagedKV(B * P, page, kv, D, dev, dt)
+        x = torch.randn(B, S + steps, dim, device=dev).to(dt)
+        with torch.inference_mode():
+            pa = a(x[:, :S], _freqs(tab, B, 0, S), None, ca.bind(table, S))
+            pb = b(x[:, :S], _freqs(tab, B, 0, S), None, cb.bind(table, S))
+            assert ((pa.float() - pb.float()).norm() / pa.float().norm()).item() < 1e-2
+            assert torch.allclose(ca.k.float(), cb.k.float(), rtol=1e-2, atol=1e-2) and torch.equal(ca.v, cb.v)
+            # the keys in the cache are unit-RMS times the gain: nothing like the un-normalised ones
+            rms = cb.k[table[0, 0], 0, 0].float().div(b.attention.k_norm.weight.float()).pow(2).mean().sqrt().item()
+            assert abs(rms - 1.0) < 2e-2
+            for t in range(steps):
+                pos = S + t
+                mask = decode_mask(B, pos + 1, dev, dt)
+                ya = a(x[:, pos:pos + 1], _freqs(tab, B, pos, 1), mask, ca.bind(table, pos + 1))
+                yb = b(x[:, pos:pos + 1], _freqs(tab, B, pos, 1), None, cb.bind(table, pos + 1))
+                rel = ((ya.float() - yb.float()).norm() / ya.float().norm()).item()
+                assert rel < 1e-2, (dim, heads, t, rel)
+            assert torch.allclose(ca.k.float(), cb.k.float(), rtol=1e-2, atol=1e-2) and torch.equal(ca.v, cb.v)
+            more = torch.randn(B, 5, dim, device=dev).to(dt)           # a chunk on top of the cached tokens
+            T = S + steps + 5
+            cm = torch.zeros(B, 1, 5, T, device=dev, dtype=dt)
+            cm[:, :, :, T - 5:] = torch.full((5, 5), float("-inf"), device=dev, dtype=dt).triu(1)
+            ya = a(more, _freqs(tab, B, S + steps, 5), cm, ca.bind(table, T))
+            yb = b(more, _freqs(tab, B, S + steps, 5), None, cb.bind(table, T))
+            assert ((ya.float() - yb.float()).norm() / ya.float().norm()).item() < 1e-2
+            assert torch.allclose(ca.k.float(), cb.k.float(), rtol=1e-2, atol=1e-2)

@@ -360,3 +360,113 @@ def test_prefill_attn_paged_checks_its_arguments():
     assert call(0, 4, D=96) == -2
     with pytest.raises(ValueError):
         ops.prefill_attn_paged(q, kc, kc, tb, 30)
+
+
+def _gains(D, g):
+    return ((1.0 + 0.3 * torch.randn(D, generator=g)).to(torch.bfloat16),
+            (1.0 + 0.3 * torch.randn(D, generator=g)).to(torch.bfloat16))
+
+
+@pytest.mark.parametrize("D", [128, 64])
+@pytest.mark.parametrize("B,S,Hq,Hkv,page,pos", [(1, 1, 1, 1, 4, 0), (3, 1, 4, 2, 8, 13), (3, 21, 4, 2, 8, 13),
+                                                 (2, 130, 16, 4, 64, 0), (5, 1, 8, 1, 16, 31)])
+def test_rope_kv_write_qknorm_bit_exact(oracle, B, S, Hq, Hkv, page, pos, D):
+    """Rotation, RMSNorm of the rotated q and k heads, page writes: q, the cached keys and values bit for bit
+    against the oracle applied token by token (attention.py:86-92: the normalised key is what is cached)."""
+    _say("rope_kv_write_qknorm", B, S, Hq, Hkv, page, pos, D)
+    P = (pos + S + page - 1) // page + 1
+    n_pages = B * P + 3
+    g = torch.Generator().manual_seed(B * 100 + S + D)
+    qkv = (torch.randn(B, S, (Hq + 2 * Hkv) * D, generator=g) * 1.5).to(torch.bfloat16)
+    ang = torch.rand(B, S, D // 2, generator=g) * 6.28
+    freqs = torch.polar(torch.ones_like(ang), ang)
+    qg, kg = _gains(D, g)
+    eps = 1e-5
+    table = torch.randperm(n_pages, generator=g)[:B * P].view(B, P)
+    if B > 2:
+        table[1, (pos + S // 2) // page] = -1
+    kc = torch.randn(n_pages, page, Hkv, D, generator=g).to(torch.bfloat16)
+    vc = torch.randn(n_pages, page, Hkv, D, generator=g).to(torch.bfloat16)
+    kb, vb = _bits(kc), _bits(vc)
+    fr = torch.view_as_real(freqs).numpy()
+    qo = np.stack([oracle.c_rope_kv_write(_bits(qkv[:, s]), np.ascontiguousarray(fr[:, s]), table.numpy(), pos + s,
+                                          kb, vb, Hq, Hkv, qk_norm=(_bits(qg), _bits(kg), eps)) for s in range(S)], 1)
+    kd, vd = kc.to(DEV), vc.to(DEV)
+    norm = ops.QkNorm(qg.to(DEV), kg.to(DEV), eps)
+    q, k = ops.rope_kv_write(qkv.to(DEV), freqs.to(DEV), table.to(DEV), pos, kd, vd, Hq, Hkv, return_k=True,
+                             qk_norm=norm)
+    assert np.array_equal(_bits(q), qo)
+    assert np.array_equal(_bits(kd), kb) and np.array_equal(_bits(vd), vb)
+    # the returned keys are the cached ones
+    for b in range(B):
+        for s in range(S):
+            phys = int(table[b, (pos + s) // page])
+            if phys >= 0:
+                assert torch.equal(k[b, s], kd[phys, (pos + s) % page])
+    # without the norm the same call stores other bits: the argument is not ignored
+    k2, v2 = kc.to(DEV), vc.to(DEV)
+    q2 = ops.rope_kv_write(qkv.to(DEV), freqs.to(DEV), table.to(DEV), pos, k2, v2, Hq, Hkv)
+    assert not torch.equal(q2, q)
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,page,T,D", [(1, 1, 1, 4, 1, 128), (3, 4, 2, 8, 14, 128), (3, 8, 2, 16, 300, 64),
+                                               (2, 16, 4, 64, 700, 128), (5, 8, 1, 16, 32, 64), (2, 6, 2, 16, 90, 128),
+                                               (4, 12, 4, 32, 260, 64)])
+def test_rope_paged_attn_decode_qknorm_equals_the_two_launches(oracle, B, Hq, Hkv, page, T, D):
+    """The decode step with qk-norm in one launch against rope_kv_write with qk-norm followed by the plain
+    attention kernel: same cache bits (hence the oracle's), same output bits; partial results likewise.
+    Per-sequence lengths included."""
+    _say("rope_paged_attn_decode_qknorm", B, Hq, Hkv, page, T, D)
+    P = (T + page - 1) // page
+    n_pages = B * P + 2
+    g = torch.Generator().manual_seed(T + D)
+    qkv = (torch.randn(B, (Hq + 2 * Hkv) * D, generator=g) * 1.5).to(torch.bfloat16).to(DEV)
+    ang = torch.rand(B, D // 2, generator=g) * 6.28
+    freqs = torch.polar(torch.ones_like(ang), ang).to(DEV)
+    qg, kg = _gains(D, g)
+    norm = ops.QkNorm(qg.to(DEV), kg.to(DEV), 1e-6)
+    table = torch.randperm(n_pages, generator=g)[:B * P].view(B, P).to(DEV)
+    kc = torch.randn(n_pages, page, Hkv, D, generator=g).to(torch.bfloat16).to(DEV)
+    vc = torch.randn(n_pages, page, Hkv, D, generator=g).to(torch.bfloat16).to(DEV)
+    k1, v1, k2, v2, k3, v3 = kc.clone(), vc.clone(), kc.clone(), vc.clone(), kc.clone(), vc.clone()
+    q = ops.rope_kv_write(qkv, freqs, table, T - 1, k1, v1, Hq, Hkv, qk_norm=norm)
+    want = ops.paged_attn_decode(q, k1, v1, table, T)
+    out = ops.rope_paged_attn_decode(qkv, freqs, table, T, k2, v2, Hq, Hkv, qk_norm=norm)
+    assert torch.equal(k1, k2) and torch.equal(v1, v2)
+    assert torch.equal(out, want)
+    # and the cache row is the oracle's
+    kb, vb = _bits(kc), _bits(vc)
+    oracle.c_rope_kv_write(_bits(qkv), torch.view_as_real(freqs).cpu().numpy(), table.cpu().numpy(), T - 1, kb, vb, Hq, Hkv,
+                           qk_norm=(_bits(qg), _bits(kg), 1e-6))
+    assert np.array_equal(_bits(k2), kb) and np.array_equal(_bits(v2), vb)
+    parts = ops.rope_paged_attn_decode(qkv, freqs, table, T, k3, v3, Hq, Hkv, partials=True, qk_norm=norm)
+    assert torch.equal(k3, k1)
+    if T > 1:
+        lens = torch.randint(1, T + 1, (B,), generator=g)
+        lens[0] = T
+        k4, v4, k5, v5 = kc.clone(), vc.clone(), kc.clone(), vc.clone()
+        q = ops.rope_kv_write(qkv, freqs, table, T - 1, k4, v4, Hq, Hkv, qk_norm=norm)
+        a = ops.paged_attn_decode(q, k4, v4, table, T, seq_lens=lens.to(DEV))
+        b = ops.rope_paged_attn_decode(qkv, freqs, table, T, k5, v5, Hq, Hkv, seq_lens=lens.to(DEV), qk_norm=norm)
+        assert torch.equal(a, b) and torch.equal(k4, k5)
+    # the partial results, combined by the output projection, against the projection of the merged output
+    K, N = Hq * D, 72
+    if B <= ops.GEMV_ATTN_MAX_ROWS and K <= ops.GEMV_ATTN_MAX_K and parts.n_slices <= ops.GEMV_ATTN_MAX_SLICES:
+        wq = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8).to(DEV)
+        sw = (torch.rand(N, generator=g) * 0.01 + 1e-3).to(DEV)
+        assert torch.equal(ops.gemv_w8a8_attn(parts, wq, sw), ops.gemv_w8a8_decode(want.view(B, K), wq, sw))
+
+
+def test_qknorm_arguments_are_checked():
+    D, Hq, Hkv = 64, 2, 1
+    qkv = torch.zeros(1, (Hq + 2 * Hkv) * D, dtype=torch.bfloat16, device=DEV)
+    freqs = torch.ones(1, D // 2, dtype=torch.complex64, device=DEV)
+    table = torch.zeros(1, 1, dtype=torch.int64, device=DEV)
+    kc = torch.zeros(1, 4, Hkv, D, dtype=torch.bfloat16, device=DEV)
+    g = torch.ones(D, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(ValueError):
+        ops.rope_kv_write(qkv, freqs, table, 0, kc, kc.clone(), Hq, Hkv, qk_norm=ops.QkNorm(g.float(), g, 1e-5))
+    with pytest.raises(ValueError):
+        ops.rope_kv_write(qkv, freqs, table, 0, kc, kc.clone(), Hq, Hkv, qk_norm=ops.QkNorm(g[:32], g, 1e-5))
+    with pytest.raises(ValueError):
+        ops.rope_paged_attn_decode(qkv, freqs, table, 1, kc, kc.clone(), Hq, Hkv, qk_norm=ops.QkNorm(g, g, -1.0))

@@ -147,3 +147,101 @@ def test_prefill_attention_with_a_position_offset_matches_the_masked_torch_atten
         got = _bf16(out).float()
         assert torch.allclose(got, want, rtol=1e-2, atol=1e-2)
         assert ((got - want).norm() / want.norm()).item() < 4e-3
+
+
+def _qknorm_case(D, seed, gains="random"):
+    B, Hq, Hkv, page, n_pages, pos = 3, 4, 2, 8, 12, 13
+    g = torch.Generator().manual_seed(seed)
+    qkv = (torch.randn(B, (Hq + 2 * Hkv) * D, generator=g) * 1.7).to(torch.bfloat16)
+    ang = torch.rand(B, D // 2, generator=g) * 6.28
+    freqs = torch.view_as_real(torch.polar(torch.ones_like(ang), ang)).numpy()
+    table = torch.tensor([[5, 2, 9], [0, -1, 11], [3, 7, 1]])
+    if gains == "random":
+        qg = (1.0 + 0.3 * torch.randn(D, generator=g)).to(torch.bfloat16)
+        kg = (1.0 + 0.3 * torch.randn(D, generator=g)).to(torch.bfloat16)
+    else:
+        qg = kg = torch.ones(D, dtype=torch.bfloat16)
+    return B, Hq, Hkv, page, n_pages, pos, qkv, freqs, table, qg, kg
+
+
+def test_qknorm_of_the_rotated_heads_matches_rms_norm_and_numpy(oracle):
+    """oq_rope_kv_write_qknorm against (a) F.rms_norm applied to the heads that oq_rope_kv_write stores -- the
+    reference's order, rotation then q_norm / k_norm (attention.py:86-89) -- within one bf16 step; (b) the
+    numpy restatement of the fixed summation order bit for bit; (c) v and the pages of unmapped sequences
+    untouched."""
+    eps = 1e-5
+    for D, seed in ((128, 3), (64, 4)):
+        B, Hq, Hkv, page, n_pages, pos, qkv, freqs, table, qg, kg = _qknorm_case(D, seed)
+        k0, v0 = np.zeros((n_pages, page, Hkv, D), np.uint16), np.zeros((n_pages, page, Hkv, D), np.uint16)
+        k1, v1 = k0.copy(), v0.copy()
+        q_plain = oracle.c_rope_kv_write(_bits(qkv), freqs, table.numpy(), pos, k0, v0, Hq, Hkv)
+        q_norm = oracle.c_rope_kv_write(_bits(qkv), freqs, table.numpy(), pos, k1, v1, Hq, Hkv,
+                                        qk_norm=(_bits(qg), _bits(kg), eps))
+        assert np.array_equal(v0, v1)
+        # (b) bit for bit against numpy on the un-normalised heads
+        assert np.array_equal(q_norm, oracle.np_head_rmsnorm_bits(q_plain, _bits(qg), eps))
+        assert np.array_equal(k1, np.where((k0 != 0).any(-1, keepdims=True),
+                                           oracle.np_head_rmsnorm_bits(k0, _bits(kg), eps), 0))
+        # (a) torch's rms_norm on the same heads, fp32 arithmetic, then rounded once
+        want_q = F.rms_norm(_bf16(q_plain).float(), (D,), qg.float(), eps)
+        got_q = _bf16(q_norm).float()
+        step = torch.maximum(want_q.abs(), torch.tensor(1e-30)) * 2.0 ** -7     # one bf16 step, generously
+        assert ((got_q - want_q).abs() <= step).all()
+        assert (got_q == want_q.to(torch.bfloat16).float()).float().mean() > 0.97
+        want_k = F.rms_norm(_bf16(k0).float(), (D,), kg.float(), eps)
+        assert ((_bf16(k1).float() - want_k).abs() <= want_k.abs() * 2.0 ** -7 + 1e-30).all()
+        # a plausible mistake -- the norm before the rotation, or the other head's gain -- does not pass (a)
+        swapped = oracle.np_head_rmsnorm_bits(q_plain, _bits(kg), eps)
+        assert not np.array_equal(swapped, q_norm)
+
+
+def test_qknorm_closed_forms(oracle):
+    """Unit gains and a head of equal magnitudes +-a: the mean square is a^2 exactly, so every element becomes
+    +-a / sqrt(a^2 + eps); with eps = 0 exactly +-1.  A rotation by angle 0 keeps the head."""
+    D, Hq, Hkv, page = 64, 2, 1, 4
+    a = 0.75
+    sign = np.where(np.arange((Hq + 2 * Hkv) * D) % 3 == 0, -1.0, 1.0).astype(np.float32)
+    qkv = torch.from_numpy(sign * a).to(torch.bfloat16).view(1, -1)
+    freqs = np.zeros((1, D // 2, 2), np.float32)
+    freqs[..., 0] = 1.0
+    table = np.array([[0]], np.int64)
+    ones = _bits(torch.ones(D, dtype=torch.bfloat16))
+    for eps, want in ((0.0, 1.0), (0.4375, a / np.sqrt(np.float32(a * a + 0.4375)))):
+        kc, vc = np.zeros((1, page, Hkv, D), np.uint16), np.zeros((1, page, Hkv, D), np.uint16)
+        q = oracle.c_rope_kv_write(_bits(qkv), freqs, table, 2, kc, vc, Hq, Hkv, qk_norm=(ones, ones, eps))
+        got = _bf16(q).float().view(-1)
+        want_t = torch.tensor(float(want)).to(torch.bfloat16).float()
+        assert torch.equal(got, torch.from_numpy(sign[:Hq * D]) * want_t)
+        assert torch.equal(_bf16(kc)[0, 2].float().view(-1), torch.from_numpy(sign[Hq * D:(Hq + Hkv) * D]) * want_t)
+        assert torch.equal(_bf16(vc)[0, 2].view(-1), qkv[0, (Hq + Hkv) * D:])
+
+
+def test_qknorm_then_attention_matches_the_reference_sequence_in_torch(oracle):
+    """Decode steps of an attention with use_qk_norm written as the reference does (rotate, norm, cache the
+    normed key, attend: attention.py:83-103) in torch fp32 against the oracle's qk-norm write + paged attention."""
+    D, Hq, Hkv, page, n_pages, B = 64, 4, 2, 4, 8, 2
+    g = torch.Generator().manual_seed(9)
+    qg = (1.0 + 0.3 * torch.randn(D, generator=g)).to(torch.bfloat16)
+    kg = (1.0 + 0.3 * torch.randn(D, generator=g)).to(torch.bfloat16)
+    table = torch.tensor([[3, 0, 6], [5, 1, 2]])
+    kc, vc = np.zeros((n_pages, page, Hkv, D), np.uint16), np.zeros((n_pages, page, Hkv, D), np.uint16)
+    ks, vs = [], []
+    for pos in range(9):
+        qkv = torch.randn(B, (Hq + 2 * Hkv) * D, generator=g).to(torch.bfloat16)
+        ang = torch.rand(B, D // 2, generator=g) * 6.28
+        fr = torch.polar(torch.ones_like(ang), ang)
+        q = oracle.c_rope_kv_write(_bits(qkv), torch.view_as_real(fr).numpy(), table.numpy(), pos, kc, vc, Hq, Hkv,
+                                   qk_norm=(_bits(qg), _bits(kg), 1e-6))
+        out = _bf16(oracle.c_paged_attn_decode(q, kc, vc, table.numpy(), pos + 1, D ** -0.5)).float()
+        x = qkv.view(B, 1, Hq + 2 * Hkv, D)
+        rot = torch.view_as_real(torch.view_as_complex(x[:, :, :Hq + Hkv].float().reshape(B, 1, -1, D // 2, 2)) *
+                                 fr.view(B, 1, 1, D // 2)).flatten(-2).to(torch.bfloat16)
+        qn = F.rms_norm(rot[:, :, :Hq], (D,), qg, 1e-6)
+        kn = F.rms_norm(rot[:, :, Hq:], (D,), kg, 1e-6)
+        ks.append(kn)
+        vs.append(x[:, :, Hq + Hkv:])
+        k_all = torch.cat(ks, 1).float().repeat_interleave(Hq // Hkv, dim=2)
+        v_all = torch.cat(vs, 1).float().repeat_interleave(Hq // Hkv, dim=2)
+        ref = F.scaled_dot_product_attention(qn.float().transpose(1, 2), k_all.transpose(1, 2), v_all.transpose(1, 2))
+        assert torch.allclose(out, ref[:, :, 0], rtol=2e-2, atol=2e-2)
+        assert (out - ref[:, :, 0]).norm() / ref.norm() < 8e-3

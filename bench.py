@@ -239,8 +239,10 @@ def bench_decode(torch, ops, args, dev):
     traffic, traffic_src = measured_traffic(f"decode_m{M}")
     # The same launch WITHOUT its weight stream (lab build of the same source: token rows requested, rounded,
     # barrier, products of zeros, stores): what the rounding that every workgroup repeats costs on its own.
+    # Left out of single-workload (profiling) runs: the lab kernel carries the product kernel's name and would be
+    # averaged into its counters.
     no_w_us = None
-    if M > 8:
+    if M > 8 and not args.no_extra:
         try:
             with ops._abi.lab_library() as lab:
                 lab.aq_lab_set_gemv_skip_weights(1)

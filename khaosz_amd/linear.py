@@ -14,7 +14,7 @@ from __future__ import annotations
 
 import logging
 import math
-from typing import Iterable, Optional, Sequence, Set
+from typing import Iterable, Optional, Sequence, Set, Tuple
 
 import torch
 import torch.nn as nn
@@ -84,6 +84,43 @@ def _no_grad_guard(x: Tensor) -> None:
         raise RuntimeError("the quantized Linear is forward-only; call it under torch.no_grad()/inference_mode()")
 
 
+class _SharedInput:
+    """Sibling projections that a module's forward applies to ONE input tensor, run as one concatenated
+    projection (``QuantLinear.concat``: one activation quantisation, one launch, bit-identical columns)
+    without touching that forward: the first sibling called with a tensor computes all columns, every
+    sibling returns its column slice.  The input is recognised by identity (and, where torch tracks one,
+    by its version counter), and both it and the result are dropped as soon as every sibling has taken
+    its slice, so nothing outlives the forward that used it.  Not for concurrent calls of one module from
+    several threads.  For modules whose forward is known to hand
+    the same, unmodified tensor to all siblings (the reference's GQA, MLA and MLP: attention.py:83-85,
+    105-106, 166-170, 205-206; mlp.py:25)."""
+
+    def __init__(self, fused: "QuantLinear", bounds: Sequence[Tuple[int, int]]):
+        self.fused, self.bounds = fused, list(bounds)
+        self._x = self._y = None
+        self._version = None
+        self._served: set = set()
+
+    @staticmethod
+    def _version_of(x: Tensor):
+        try:
+            return x._version
+        except RuntimeError:  # inference tensors carry no version counter
+            return None
+
+    def output(self, x: Tensor, index: int) -> Tensor:
+        if self._x is not x or self._version != self._version_of(x) or index in self._served:
+            self._y = self.fused(x)
+            self._x, self._version, self._served = x, self._version_of(x), set()
+        lo, hi = self.bounds[index]
+        y = self._y[..., lo:hi]
+        self._served.add(index)
+        if len(self._served) == len(self.bounds):
+            self._x = self._y = None
+            self._served = set()
+        return y
+
+
 class QuantLinear(Linear):
     """W8A8 Linear: per-channel int8 weight, per-token int8 activation.
 
@@ -105,6 +142,7 @@ class QuantLinear(Linear):
         # decode workspaces (activation codes between the row quantiser and the GEMV), one per (device, stream):
         # the same module called from two streams or threads must not share one
         self._workspaces = _PerStream()
+        self._shared: Optional[Tuple[_SharedInput, int]] = None  # set by share_inputs(): (group, index in it)
 
     # -- construction -----------------------------------------------------
     @classmethod
@@ -196,6 +234,8 @@ class QuantLinear(Linear):
         into the activation quantisation (the normalised activations are never written; see
         ``ops.rmsnorm_quant_rowwise_i8``)."""
         _no_grad_guard(x)
+        if self._shared is not None and residual is None and norm is None:
+            return self._shared[0].output(x, self._shared[1])
         lead = x.shape[:-1]
         x2 = x.reshape(-1, x.shape[-1])
         M = x2.shape[0]
@@ -312,12 +352,47 @@ TARGET_MODULES_ATTN = {"q_proj", "k_proj", "v_proj", "o_proj", "kv_a_proj", "kv_
 TARGET_MODULES_FFN = {"up", "gate", "down"}
 
 
+def share_inputs(parent: nn.Module, names: Sequence[str]) -> bool:
+    """Run the quantized children ``names`` of ``parent`` -- projections its forward applies to one and
+    the same tensor -- as one concatenated projection behind their own ``forward`` (see ``_SharedInput``);
+    ``parent``'s code and state-dict keys stay as they are.  Returns False (and changes nothing) unless at
+    least two of the named children exist and all of those are ``QuantLinear`` with one input width and
+    alike in having a bias."""
+    parts = [getattr(parent, n, None) for n in names]
+    parts = [p for p in parts if p is not None]
+    if len(parts) < 2 or any(not isinstance(p, QuantLinear) or p._shared is not None for p in parts):
+        return False
+    if len({p.in_dim for p in parts}) != 1 or len({p.bias is None for p in parts}) != 1:
+        return False
+    bounds, row = [], 0
+    for p in parts:
+        bounds.append((row, row + p.out_dim))
+        row += p.out_dim
+    group = _SharedInput(QuantLinear.concat(parts), bounds)
+    for i, p in enumerate(parts):
+        p._shared = (group, i)
+    return True
+
+
+# Modules of the reference whose forward hands one tensor to several projections, by class (module path, name)
+# -- matched by name so that this package never imports the reference: GQA (attention.py:83-85; the output gate
+# reads the same x, attention.py:105-106), MLA (attention.py:166-170, 205-206) and MLP, the experts of DeepSeekMoE
+# included (mlp.py:25).
+REFERENCE_SHARED_INPUTS = {
+    ("astrai.model.components.attention", "GQA"): ("q_proj", "k_proj", "v_proj", "gate"),
+    ("astrai.model.components.attention", "MLA"): ("q_proj", "kv_a_proj", "gate"),
+    ("astrai.model.components.mlp", "MLP"): ("up", "gate"),
+}
+
+
 def fuse_shared_inputs(model: nn.Module, norms: bool = False, decode_attention: bool = False,
                        residuals: bool = False) -> int:
     """Call ``fuse_projections()`` on every module that offers it (attention and MLP blocks whose
     projections read one input); returns how many fused modules were built.  Run it after
     ``quantize_model`` and after loading weights: the fused module owns the weight storage from
-    then on.  Outputs stay bit-identical.  ``norms=True`` additionally lets blocks compute
+    then on.  Outputs stay bit-identical.  Modules of the reference itself (its GQA, MLA and MLP classes,
+    recognised by name) get the same single launch behind their own unchanged forward (``share_inputs``).
+    ``norms=True`` additionally lets blocks compute
     RMSNorm and the quantisation of its output in one launch (``fuse_norm_quant()``), which
     drops the bf16 rounding of the normalised activations: not bit-identical, inside the
     quantisation noise.  ``decode_attention=True`` lets attention modules with a fused q/k/v
@@ -330,6 +405,11 @@ def fuse_shared_inputs(model: nn.Module, norms: bool = False, decode_attention: 
         f = getattr(m, "fuse_projections", None)
         if callable(f):
             n += int(f())
+            continue
+        names = REFERENCE_SHARED_INPUTS.get((type(m).__module__, type(m).__name__))
+        if names is not None:  # the reference's own module: its forward is untouched
+            # (the output gate joins the group only if it matches the others in having a bias)
+            n += int(share_inputs(m, names) or share_inputs(m, [x for x in names if x != "gate" or "up" in names]))
     if norms:
         for m in model.modules():
             f = getattr(m, "fuse_norm_quant", None)

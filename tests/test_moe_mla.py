@@ -51,6 +51,10 @@ class RefMLP(nn.Module):  # mlp.py:17-27
         return self.down(F.silu(self.gate(x)) * self.up(x))
 
 
+RefMLP.__name__ = RefMLP.__qualname__ = "MLP"
+RefMLP.__module__ = "astrai.model.components.mlp"
+
+
 class RefMoE(nn.Module):
     """The routed half of DeepSeekMoE (mlp.py:72-93): top-k of a softmax over the router's logits, each
     expert run on the rows routed to it."""
@@ -183,3 +187,116 @@ def test_reference_class_with_a_bias_and_this_packages_linear_quantize_alike(ora
         a, b = holder["up"](x), holder["down"](x)
     assert torch.equal(a, b)
     assert np.array_equal(bf16_bits(a), _oracle_linear(oracle, holder["up"], x))
+
+
+class RefGQAProjections(nn.Module):
+    """The Linear calls of the reference's GQA.forward in its order (attention.py:83-85, 105-108), under its
+    class name; what lies between them is replaced by a fixed mixing of q, k and v."""
+
+    def __init__(self, dim, n_heads, n_kv_heads, gated):
+        super().__init__()
+        hd = dim // n_heads
+        self.q_proj, self.k_proj, self.v_proj = RefLinear(dim, dim), RefLinear(dim, n_kv_heads * hd), RefLinear(dim, n_kv_heads * hd)
+        self.o_proj = RefLinear(dim, dim)
+        self.rep = n_heads // n_kv_heads
+        if gated:
+            self.gate = RefLinear(dim, dim)
+        self.gated = gated
+
+    def forward(self, x):
+        B, S, _ = x.shape
+        q = self.q_proj(x).reshape(B, S, -1, 32)
+        k = self.k_proj(x).reshape(B, S, -1, 32)
+        v = self.v_proj(x).reshape(B, S, -1, 32)
+        out = (q + k.repeat_interleave(self.rep, 2) * v.repeat_interleave(self.rep, 2)).flatten(2)
+        if self.gated:
+            out = out * torch.sigmoid(self.gate(x))
+        return self.o_proj(out)
+
+
+RefGQAProjections.__name__ = RefGQAProjections.__qualname__ = "GQA"
+RefGQAProjections.__module__ = "astrai.model.components.attention"
+
+
+class RefMLA(RefMLAProjections):
+    """MLA.forward's Linear calls in order (attention.py:166-176, 205-209): q_proj(x), kv_a_proj(x), a norm,
+    kv_b_proj, the gate on x, o_proj."""
+
+    def forward(self, x):
+        B, S, _ = x.shape
+        q = self.q_proj(x)
+        q = q.view(B, S, 8, -1)                              # a view, as the reference takes it
+        c = self.kv_a_proj(x)
+        c = F.rms_norm(c, (c.shape[-1],))
+        kv = self.kv_b_proj(c).view(B, S, 2, -1)
+        mixed = q.flatten(2)[..., :x.shape[-1]] * kv.flatten(2).mean(-1, keepdim=True)
+        return self.o_proj(mixed * torch.sigmoid(self.gate(x)))
+
+
+RefMLA.__name__ = RefMLA.__qualname__ = "MLA"
+RefMLA.__module__ = "astrai.model.components.attention"
+
+
+def _count_launches(monkeypatch):
+    from khaosz_amd import ops
+    calls = []
+    for name in ("gemv_w8a8_decode", "linear_w8a8", "quant_rowwise_i8"):
+        real = getattr(ops, name)
+        monkeypatch.setattr(ops, name, (lambda real, name: lambda *a, **k: (calls.append(name), real(*a, **k))[1])(real, name))
+    return calls
+
+
+@pytest.mark.parametrize("tokens", [(2, 1), (3, 4), (2, 48)])
+def test_reference_modules_share_one_launch_behind_their_own_forward(monkeypatch, tokens):
+    """fuse_shared_inputs on modules that carry the reference's class names (GQA, MLA, MLP and the experts of a
+    routed layer): their forward is untouched, the projections of one input run as one concatenated launch
+    (one activation quantisation), outputs and state-dict keys are what they were, bit for bit -- at decode
+    sizes, where the GEMV quantises its rows itself, and at prefill sizes."""
+    from khaosz_amd import fuse_shared_inputs
+    _say("shared inputs of reference modules", tokens)
+    torch.manual_seed(11)
+    B, S = tokens
+    dim = 256
+    mods = {"gqa": RefGQAProjections(dim, 8, 2, gated=True), "gqa_plain": RefGQAProjections(dim, 8, 4, gated=False),
+            "mla": RefMLA(dim, 8, 2, 128, 96), "mlp": RefMLP(dim, 704)}
+    x = torch.randn(B, S, dim, device=DEV, dtype=torch.bfloat16)
+    for name, m in mods.items():
+        m = m.to(DEV)
+        assert quantize_model(m) > 0
+        keys = sorted(m.state_dict().keys())
+        calls = _count_launches(monkeypatch)
+        with torch.inference_mode():
+            want = m(x)
+        before = calls.count("gemv_w8a8_decode") + calls.count("linear_w8a8")
+        assert fuse_shared_inputs(m) == 1, name
+        assert sorted(m.state_dict().keys()) == keys
+        del calls[:]
+        with torch.inference_mode():
+            got = m(x)
+            again = m(x)                                     # nothing stale is served on a second pass
+        after = (calls.count("gemv_w8a8_decode") + calls.count("linear_w8a8")) // 2
+        saved = {"gqa": 3, "gqa_plain": 2, "mla": 2, "mlp": 1}[name]
+        assert before - after == saved, (name, before, after)
+        assert torch.equal(got, want) and torch.equal(again, want), name
+        # a tensor modified in place between two calls is a new input (where torch tracks versions)
+        y = x.clone()
+        first = m.q_proj(y) if hasattr(m, "q_proj") else m.up(y)
+        y.mul_(2.0)
+        second = m.q_proj(y) if hasattr(m, "q_proj") else m.up(y)
+        assert not torch.equal(first, second)
+        monkeypatch.undo()
+
+
+def test_routed_experts_share_up_and_gate(monkeypatch):
+    """Every expert of a routed layer is an MLP of the reference (mlp.py:17-27, 53-55): up and gate of an expert
+    read the same gathered rows x[token_idx] and become one launch; the layer's output keeps its bits."""
+    from khaosz_amd import fuse_shared_inputs
+    torch.manual_seed(5)
+    moe = RefMoE(256, 352, 8, 2).to(DEV).to(torch.bfloat16)
+    x = torch.randn(40, 256, device=DEV, dtype=torch.bfloat16)
+    assert quantize_model(moe) == 24
+    with torch.inference_mode():
+        want = moe(x)
+    assert fuse_shared_inputs(moe) == 8
+    with torch.inference_mode():
+        assert torch.equal(moe(x), want)

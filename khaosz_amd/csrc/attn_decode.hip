@@ -527,29 +527,52 @@ __global__ __launch_bounds__(ATT_MAX_D / 2) void attn_merge_kernel(const float* 
   // still run in slice order.
   constexpr int GRP = 8;
   float mm = -INFINITY;
-  for (int s0 = 0; s0 < NS; s0 += GRP) {  // slice 0 always holds a position
-    float mv[GRP];
-#pragma unroll
-    for (int i = 0; i < GRP; ++i) mv[i] = s0 + i < NS ? part[(s0 + i) * part_sz + D] : -INFINITY;
-#pragma unroll
-    for (int i = 0; i < GRP; ++i) mm = fmaxf(mm, mv[i]);
-  }
   float n0 = 0.0f, n1 = 0.0f, den = 0.0f;
-  for (int s0 = 0; s0 < NS; s0 += GRP) {
+  if (NS <= GRP) {
+    // The usual case (up to 2048 positions): (maximum, denominator) and the numerators of every slice are
+    // requested together, so the launch is one memory round trip instead of two (maxima first, then values).
     float2 md[GRP], v[GRP];
 #pragma unroll
     for (int i = 0; i < GRP; ++i) {
-      const bool ok = s0 + i < NS;  // uniform
-      md[i] = ok ? *reinterpret_cast<const float2*>(part + (s0 + i) * part_sz + D) : make_float2(0.0f, 0.0f);
-      v[i] = ok ? *reinterpret_cast<const float2*>(part + (s0 + i) * part_sz + d) : make_float2(0.0f, 0.0f);
+      const bool ok = i < NS;  // uniform
+      md[i] = ok ? *reinterpret_cast<const float2*>(part + i * part_sz + D) : make_float2(-INFINITY, 0.0f);
+      v[i] = ok ? *reinterpret_cast<const float2*>(part + i * part_sz + d) : make_float2(0.0f, 0.0f);
     }
 #pragma unroll
+    for (int i = 0; i < GRP; ++i) mm = fmaxf(mm, md[i].x);
+#pragma unroll
     for (int i = 0; i < GRP; ++i) {
-      if (s0 + i < NS) {
+      if (i < NS) {
         const float a = attn_slice_weight(md[i].x, mm);
         n0 = __builtin_fmaf(v[i].x, a, n0);
         n1 = __builtin_fmaf(v[i].y, a, n1);
         den = __builtin_fmaf(md[i].y, a, den);
+      }
+    }
+  } else {
+    for (int s0 = 0; s0 < NS; s0 += GRP) {  // slice 0 always holds a position
+      float mv[GRP];
+#pragma unroll
+      for (int i = 0; i < GRP; ++i) mv[i] = s0 + i < NS ? part[(s0 + i) * part_sz + D] : -INFINITY;
+#pragma unroll
+      for (int i = 0; i < GRP; ++i) mm = fmaxf(mm, mv[i]);
+    }
+    for (int s0 = 0; s0 < NS; s0 += GRP) {
+      float2 md[GRP], v[GRP];
+#pragma unroll
+      for (int i = 0; i < GRP; ++i) {
+        const bool ok = s0 + i < NS;  // uniform
+        md[i] = ok ? *reinterpret_cast<const float2*>(part + (s0 + i) * part_sz + D) : make_float2(0.0f, 0.0f);
+        v[i] = ok ? *reinterpret_cast<const float2*>(part + (s0 + i) * part_sz + d) : make_float2(0.0f, 0.0f);
+      }
+#pragma unroll
+      for (int i = 0; i < GRP; ++i) {
+        if (s0 + i < NS) {
+          const float a = attn_slice_weight(md[i].x, mm);
+          n0 = __builtin_fmaf(v[i].x, a, n0);
+          n1 = __builtin_fmaf(v[i].y, a, n1);
+          den = __builtin_fmaf(md[i].y, a, den);
+        }
       }
     }
   }

@@ -204,6 +204,59 @@ __device__ __forceinline__ uint32_t pack_low_bytes(uint32_t a, uint32_t b, uint3
   return __builtin_amdgcn_perm(cd, ab, 0x05040100u);             // {ab.b0, ab.b1, cd.b0, cd.b1}
 }
 
+// quant_codes with the N codes delivered packed, four to a dword (code i in byte i % 4 of out[i / 4]).  On the lean
+// path the rounding add writes its low byte -- which IS the code -- straight into its byte of the result
+// (v_add_f32 in its sub-dword-addressing form, destination byte selected, the other bytes kept), so rounding and
+// packing cost one operation per value instead of one and three quarters.  This part wants one instruction (or
+// one idle slot) between such a write and the next instruction that touches the same register; the compiler does
+// not see inside the statement, so the slots are written out: two dwords are filled alternately where there are
+// eight values, and a pause closes the sequence.
+template <int N, int STEPS = 2>
+__device__ __forceinline__ void quant_codes_packed(const float* a, float s, float rs, bool lean_ok, uint32_t* out) {
+  static_assert(N == 4 || N == 8, "one or two dwords of codes");
+  const float magic = 12582912.0f;  // 1.5 * 2^23
+  if (__builtin_expect(lean_ok, 1)) {
+    float q[N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      q[i] = a[i] * rs;
+      q[i] = __builtin_fmaf(__builtin_fmaf(-s, q[i], a[i]), rs, q[i]);
+      if constexpr (STEPS == 2) q[i] = __builtin_fmaf(__builtin_fmaf(-s, q[i], a[i]), rs, q[i]);
+    }
+    if constexpr (N == 8) {
+      uint32_t r0 = __float_as_uint(q[0] + magic), r1 = __float_as_uint(q[4] + magic);
+      asm("v_add_f32_sdwa %0, %2, %8 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD\n\t"
+          "v_add_f32_sdwa %1, %5, %8 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD\n\t"
+          "v_add_f32_sdwa %0, %3, %8 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD\n\t"
+          "v_add_f32_sdwa %1, %6, %8 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD\n\t"
+          "v_add_f32_sdwa %0, %4, %8 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD\n\t"
+          "v_add_f32_sdwa %1, %7, %8 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD\n\t"
+          "s_nop 0"
+          : "+v"(r0), "+v"(r1)
+          : "v"(q[1]), "v"(q[2]), "v"(q[3]), "v"(q[5]), "v"(q[6]), "v"(q[7]), "v"(magic));
+      out[0] = r0;
+      out[1] = r1;
+    } else {
+      uint32_t r0 = __float_as_uint(q[0] + magic);
+      asm("v_add_f32_sdwa %0, %1, %4 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD\n\t"
+          "s_nop 0\n\t"
+          "v_add_f32_sdwa %0, %2, %4 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD\n\t"
+          "s_nop 0\n\t"
+          "v_add_f32_sdwa %0, %3, %4 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD\n\t"
+          "s_nop 0"
+          : "+v"(r0)
+          : "v"(q[1]), "v"(q[2]), "v"(q[3]), "v"(magic));
+      out[0] = r0;
+    }
+  } else {
+    uint32_t c[N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) c[i] = quant_code_exact(a[i], s);
+#pragma unroll
+    for (int i = 0; i < N / 4; ++i) out[i] = pack_low_bytes(c[4 * i], c[4 * i + 1], c[4 * i + 2], c[4 * i + 3]);
+  }
+}
+
 // Raw buffer descriptor over [base, base + bytes): loads whose byte offset
 // falls outside return zero, which is how tile edges are handled without
 // branches.  0x00020000 is the gfx9 32-bit data-format dword.

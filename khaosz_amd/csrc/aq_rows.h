@@ -177,17 +177,14 @@ struct RowsToLds {
         const int v = i * 64 + lane;
         if (v < nvec) {
           float f[EPV];
-          uint32_t code[EPV];
+          uint32_t code[EPV / 4];
           values<NORM>(j, i, r, f);
-          quant_codes<EPV, STEPS>(f, rsc.s, rsc.rs, rsc.fast_ok, code);  // zero rows give zero codes
+          quant_codes_packed<EPV, STEPS>(f, rsc.s, rsc.rs, rsc.fast_ok, code);  // zero rows give zero codes
           uint8_t* dst = xs + m * pitch + v * EPV;
           if constexpr (BF16) {
-            uint2 o;
-            o.x = pack_low_bytes(code[0], code[1], code[2], code[3]);
-            o.y = pack_low_bytes(code[4], code[5], code[6], code[7]);
-            *reinterpret_cast<uint2*>(dst) = o;
+            *reinterpret_cast<uint2*>(dst) = make_uint2(code[0], code[1]);
           } else {
-            *reinterpret_cast<uint32_t*>(dst) = pack_low_bytes(code[0], code[1], code[2], code[3]);
+            *reinterpret_cast<uint32_t*>(dst) = code[0];
           }
         }
       }

@@ -15,16 +15,13 @@ template <bool BF16>
 __device__ __forceinline__ void quant_store(const uint4& v, float s, float rs, bool fast_ok, int8_t* dst) {
   constexpr int EPV = RowIn<BF16>::EPV;
   float f[EPV];
-  uint32_t c[EPV];
+  uint32_t c[EPV / 4];
   RowIn<BF16>::unpack(v, f);
-  quant_codes<EPV, quant_steps<BF16, false>()>(f, s, rs, fast_ok, c);
+  quant_codes_packed<EPV, quant_steps<BF16, false>()>(f, s, rs, fast_ok, c);
   if constexpr (BF16) {
-    uint2 o;
-    o.x = pack_low_bytes(c[0], c[1], c[2], c[3]);
-    o.y = pack_low_bytes(c[4], c[5], c[6], c[7]);
-    store_wt(reinterpret_cast<uint2*>(dst), o);
+    store_wt(reinterpret_cast<uint2*>(dst), make_uint2(c[0], c[1]));
   } else {
-    store_wt(reinterpret_cast<uint32_t*>(dst), pack_low_bytes(c[0], c[1], c[2], c[3]));
+    store_wt(reinterpret_cast<uint32_t*>(dst), c[0]);
   }
 }
 
@@ -234,16 +231,16 @@ __global__ __launch_bounds__(256) void rmsnorm_quant_kernel(const void* __restri
       const int v = i * 64 + lane;
       if (v < nvec) {
         float y[EPV];
-        uint32_t code[EPV];
+        uint32_t code[EPV / 4];
         normed(i, y);
-        quant_codes<EPV>(y, rsc.s, rsc.rs, rsc.fast_ok, code);
+        quant_codes_packed<EPV>(y, rsc.s, rsc.rs, rsc.fast_ok, code);
         if constexpr (BF16) {
           uint2 o;
-          o.x = pack_low_bytes(code[0], code[1], code[2], code[3]);
-          o.y = pack_low_bytes(code[4], code[5], code[6], code[7]);
+          o.x = code[0];
+          o.y = code[1];
           store_wt(reinterpret_cast<uint2*>(dst + (int64_t)v * EPV), o);
         } else {
-          store_wt(reinterpret_cast<uint32_t*>(dst + (int64_t)v * EPV), pack_low_bytes(code[0], code[1], code[2], code[3]));
+          store_wt(reinterpret_cast<uint32_t*>(dst + (int64_t)v * EPV), code[0]);
         }
       }
     }
@@ -341,20 +338,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void s
         const int v = i * 64 + lane;
         const uint32_t off = (uint32_t)v * 16u;
         float u[EPV], g[EPV], hh[EPV];
-        uint32_t code[EPV];
+        uint32_t code[EPV / 4];
         RowIn<BF16>::unpack(buffer_load_16(Ur, off), u);
         RowIn<BF16>::unpack(buffer_load_16(Gr, off), g);
 #pragma unroll
         for (int e = 0; e < EPV; ++e) hh[e] = swiglu_repro(u[e], g[e]);
-        quant_codes<EPV>(hh, rsc.s, rsc.rs, rsc.fast_ok, code);
+        quant_codes_packed<EPV>(hh, rsc.s, rsc.rs, rsc.fast_ok, code);
         if (v < nvec) {
           if constexpr (BF16) {
             uint2 o;
-            o.x = pack_low_bytes(code[0], code[1], code[2], code[3]);
-            o.y = pack_low_bytes(code[4], code[5], code[6], code[7]);
+            o.x = code[0];
+            o.y = code[1];
             store_wt(reinterpret_cast<uint2*>(dst + (int64_t)v * EPV), o);
           } else {
-            store_wt(reinterpret_cast<uint32_t*>(dst + (int64_t)v * EPV), pack_low_bytes(code[0], code[1], code[2], code[3]));
+            store_wt(reinterpret_cast<uint32_t*>(dst + (int64_t)v * EPV), code[0]);
           }
         }
       }
@@ -368,15 +365,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void s
     const __amdgpu_buffer_rsrc_t Qr = make_rsrc(dst, (uint32_t)F);
 #pragma unroll
     for (int i = 0; i < NC; ++i) {
-      uint32_t code[EPV];
-      quant_codes<EPV>(h[i], rsc.s, rsc.rs, rsc.fast_ok, code);
+      uint32_t code[EPV / 4];
+      quant_codes_packed<EPV>(h[i], rsc.s, rsc.rs, rsc.fast_ok, code);
       if constexpr (BF16) {
         typedef int v2i_t __attribute__((ext_vector_type(2)));
-        const v2i_t o = {(int)pack_low_bytes(code[0], code[1], code[2], code[3]),
-                         (int)pack_low_bytes(code[4], code[5], code[6], code[7])};
+        const v2i_t o = {(int)code[0],
+                         (int)code[1]};
         __builtin_amdgcn_raw_buffer_store_b64(o, Qr, lane * 8, i * 512, STORE_WT);
       } else {
-        __builtin_amdgcn_raw_buffer_store_b32((int)pack_low_bytes(code[0], code[1], code[2], code[3]), Qr, lane * 4,
+        __builtin_amdgcn_raw_buffer_store_b32((int)code[0], Qr, lane * 4,
                                               i * 256, STORE_WT);
       }
     }
@@ -417,15 +414,15 @@ __global__ __launch_bounds__(1024) void swiglu_quant_wg_kernel(const void* __res
   if (v == 0) scale[row] = rsc.s;
   if (v < nvec) {
     int8_t* dst = q + row * (int64_t)F;
-    uint32_t code[EPV];
-    quant_codes<EPV>(h, rsc.s, rsc.rs, rsc.fast_ok, code);
+    uint32_t code[EPV / 4];
+    quant_codes_packed<EPV>(h, rsc.s, rsc.rs, rsc.fast_ok, code);
     if constexpr (BF16) {
       uint2 o;
-      o.x = pack_low_bytes(code[0], code[1], code[2], code[3]);
-      o.y = pack_low_bytes(code[4], code[5], code[6], code[7]);
+      o.x = code[0];
+      o.y = code[1];
       store_wt(reinterpret_cast<uint2*>(dst + (int64_t)v * EPV), o);
     } else {
-      store_wt(reinterpret_cast<uint32_t*>(dst + (int64_t)v * EPV), pack_low_bytes(code[0], code[1], code[2], code[3]));
+      store_wt(reinterpret_cast<uint32_t*>(dst + (int64_t)v * EPV), code[0]);
     }
   }
 }

@@ -111,7 +111,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=1000)
     ap.add_argument("--workload", default="decode", choices=["decode", "prefill", "fp8", "block", "model"])
     ap.add_argument("--m", type=int, default=16, help="decode rows (1..16)")
-    ap.add_argument("--mnk", default=None, help="prefill workload only: M,N,K of the int8 Linear instead of configuration 3's "
+    ap.add_argument("--mnk", default=None, help="prefill and fp8 workloads only: M,N,K of the int8 Linear instead of configuration 3's "
                     "4096,2048,2048 (e.g. 8192,8192,8192 for a profile of the GEMM's steady state)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary workloads")
@@ -381,6 +381,9 @@ def bench_few_dozen_rows(torch, ops, args, dev):
 def bench_fp8(torch, ops, args, dev):
     M, K, N = 2048, 8192, 2048
     nbuf = 4
+    if getattr(args, "mnk", None) and args.workload == "fp8":
+        M, N, K = (int(v) for v in args.mnk.split(","))
+        nbuf = 4 if M * K <= (1 << 25) else 2
     weights = make_weights(torch, ops, N, K, nbuf, dev, seed=5, mode="fp8")
     g = torch.Generator(device=dev).manual_seed(6)
     xs = [torch.randn(M, K, generator=g, device=dev).to(torch.bfloat16) for _ in range(nbuf)]
@@ -430,7 +433,7 @@ def bench_fp8(torch, ops, args, dev):
         del wd
     t = flops / (ms * 1e-3) / 1e12
     tk = flops / (ms_k * 1e-3) / 1e12
-    traffic, traffic_src = measured_traffic("fp8")
+    traffic, traffic_src = measured_traffic("fp8") if (M, N, K) == (2048, 2048, 8192) else (None, "not measured for this shape")
     return {
         "workload": f"fp8_linear M={M} K={K} N={N} per-tensor e4m3 quantise + FP8 MFMA GEMM, bf16 out",
         "value": t, "unit": "TFLOP/s", "ms_per_step": ms, "flops_per_step": flops, "dtype": "fp8_e4m3",

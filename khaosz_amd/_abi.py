@@ -82,6 +82,7 @@ LAB_SYMBOLS = {
     "aq_lab_probe_empty": (_int, [_vp, _vp]),
     "aq_lab_probe_mfma_lds_issue": (_int, [_int, _int, _int, _vp, _vp, _vp]),
     "aq_lab_quant_tensor_fp8_onepass_spin": (_int, [_vp, _int, _i64, _vp, _vp, _vp, _sz, _int, _vp]),
+    "aq_lab_probe_swiglu_bf16": (_int, [_vp, _vp, _i64, _vp, _vp, _vp]),
     "aq_lab_set_gemv_timeline": (_int, [_vp]),
     "aq_lab_read_clock": (_int, [_vp]),
     "aq_lab_set_gemv_skip_weights": (_int, [_int]),

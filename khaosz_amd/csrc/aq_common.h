@@ -147,6 +147,18 @@ __device__ __forceinline__ float div_midrange(float n, float d) {
   return __builtin_fmaf(__builtin_fmaf(-d, q, n), y, q);
 }
 
+// The same quotient two operation slots cheaper, for ONE family of operands only: n = g and d = 1 + exp_repro(-g)
+// with g a bf16 number the test below lets through.  The quotient corrections use the hardware reciprocal as it
+// comes (no refinement of it).  For general operands that is only almost always the correctly rounded quotient; for
+// this family there are fewer than 65536 operand pairs, one per gate, and every one of them goes through the shipped
+// kernel against the CPU oracle's true divide in the tests (all bf16 gate patterns, bit for bit).
+__device__ __forceinline__ float div_bf16_gate(float n, float d) {
+  const float y = __builtin_amdgcn_rcpf(d);
+  float q = n * y;
+  q = __builtin_fmaf(__builtin_fmaf(-d, q, n), y, q);
+  return __builtin_fmaf(__builtin_fmaf(-d, q, n), y, q);
+}
+
 // The gates div_midrange may be used for: zero (0 / d = 0, with a sign that no code and no maximum depends on) or
 // 2^-62 <= |g| <= 80, so that 1 + exp(-g) < 2^116 and every intermediate of the short divide stays a normal
 // number.  Exact zeros must pass: rows of real bf16 activations hold a few per ten million values, and a row sent
@@ -192,12 +204,14 @@ __device__ __forceinline__ bool gates_midrange(const float* g) {
 // CLAMP = false drops the exponential's own argument clamp, the identity for such gates (|g| <= 80 < 87): one
 // operation less per product where the vector ALU is the bound (4096 x 5632: 27.9 -> 27.1 us); the one-row-per-
 // workgroup kernel, which is not, measured 0.2 us slower without it and keeps it.
-template <int N, bool CLAMP = true>
+// BF16_GATES: the gates are bf16 numbers, for which div_bf16_gate is certified.
+template <int N, bool CLAMP = true, bool BF16_GATES = false>
 __device__ __forceinline__ void swiglu_group_midrange(const float* u, const float* g, float* h) {
 #pragma unroll
   for (int i = 0; i < N; ++i) {
     if (i > 0 && (i & 3) == 0) __builtin_amdgcn_sched_barrier(0);
-    h[i] = __fmul_rn(u[i], div_midrange(g[i], __fadd_rn(1.0f, exp_repro<CLAMP>(-g[i]))));
+    const float d = __fadd_rn(1.0f, exp_repro<CLAMP>(-g[i]));
+    h[i] = __fmul_rn(u[i], BF16_GATES ? div_bf16_gate(g[i], d) : div_midrange(g[i], d));
   }
 }
 

@@ -31,6 +31,12 @@ int aq_lab_choose_gemm_tile(int64_t M, int64_t N, int compute_units);
  * first stage landed, [5] the first K step, [6] accumulator exchange + epilogue, [7] the whole tile. */
 int aq_lab_read_clock(long long *host8);
 
+/* The arithmetic of the row SwiGLU quantiser's mid-range path on single bf16 pairs: h[i] = up[i] * silu(gate[i])
+ * (fp32), and in_range[i] = 1 where the kernel's range test lets gate[i] take that path.  For the test that puts
+ * every bf16 gate pattern through it against the oracle. */
+int aq_lab_probe_swiglu_bf16(const uint16_t *up, const uint16_t *gate, int64_t n, float *h, uint8_t *in_range,
+                             void *stream);
+
 /* `workgroups` x 4 wavefronts each issue iters x 8 independent MFMAs.
  * kind 0 = i32_32x32x32_i8 (65536 ops each), 1 = i32_16x16x64_i8 (32768), 2 = f32_32x32x64 e4m3 (131072 flops).
  * data 0 = constant operands (no toggling: the clock stays at its maximum), 1 = random bytes, four operand

@@ -270,6 +270,31 @@ extern "C" int aq_lab_probe_read(const void* src, int64_t bytes, int loads_per_l
   }
 }
 
+namespace aq {
+// h[i] = up[i] * silu(gate[i]) for bf16 operands as the row kernel's mid-range path computes it (no clamp in the
+// exponential, the two-slot-shorter divide for bf16 gates), and whether the gate passes that path's range test.
+__global__ void probe_swiglu_bf16_kernel(const uint16_t* up, const uint16_t* gate, int64_t n, float* h, uint8_t* in_range) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const float u = __uint_as_float((uint32_t)up[i] << 16), g = __uint_as_float((uint32_t)gate[i] << 16);
+  float out;
+  swiglu_group_midrange<1, false, true>(&u, &g, &out);
+  h[i] = out;
+  GateRangeBf16 r;
+  r.add(make_uint4((uint32_t)gate[i] | ((uint32_t)gate[i] << 16), 0x3f803f80u, 0x3f803f80u, 0x3f803f80u));
+  in_range[i] = r.ok() ? 1 : 0;
+}
+}  // namespace aq
+
+extern "C" int aq_lab_probe_swiglu_bf16(const uint16_t* up, const uint16_t* gate, int64_t n, float* h, uint8_t* in_range,
+                                        void* stream) {
+  if (n < 0 || (n && (!up || !gate || !h || !in_range))) return AQ_E_NULL;
+  if (n == 0) return AQ_OK;
+  hipLaunchKernelGGL(aq::probe_swiglu_bf16_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), up, gate, n, h, in_range);
+  return (int)hipGetLastError();
+}
+
 extern "C" int aq_lab_probe_empty(int* sink, void* stream) {
   if (!sink) return AQ_E_NULL;
   hipLaunchKernelGGL(aq::probe_empty_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream), sink);

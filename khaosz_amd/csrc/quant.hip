@@ -307,7 +307,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void s
         range.add(cg[i]);
       else
         ok &= gates_midrange<EPV>(g);
-      swiglu_group_midrange<EPV, false>(u, g, h[i]);
+      swiglu_group_midrange<EPV, false, BF16>(u, g, h[i]);
       amax = fmaxf(amax, vec_amax<EPV>(h[i]));
       // h is wanted HERE: left to itself the compiler takes the range checks of all pairs (which need the gates only)
       // and the branch on them first, and requests each pair's up half inside the branch, one by one

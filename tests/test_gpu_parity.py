@@ -217,6 +217,75 @@ def test_swiglu_quant_divide_range_edges(oracle, M, F, dtype):
     assert bad.size == 0, f"first mismatches (row, col): {bad[:5].tolist()}"
 
 
+def _all_bf16_gates():
+    """every bf16 pattern that is a finite number, as uint16"""
+    pats = np.arange(65536, dtype=np.uint32)
+    finite = ((pats >> 7) & 0xff) != 0xff
+    return pats[finite].astype(np.uint16)
+
+
+def test_swiglu_short_divide_is_the_oracles_divide_for_every_bf16_gate(oracle):
+    """The row kernel's bf16 path divides g by 1 + exp(-g) with a sequence that is correctly rounded for this family
+    of operands only.  The family has one member per gate: every finite bf16 gate pattern goes through the same
+    arithmetic (lab probe: the header's functions, no clamp, short divide) against the oracle's product, which
+    uses the true divide -- all gates the kernel's range test admits must agree bit for bit, with up = 1 (the
+    quotient itself) and with other multipliers."""
+    from khaosz_amd import _abi
+    lab = _abi.load_lab()
+    gates = _all_bf16_gates()
+    n = gates.size
+    gd = torch.from_numpy(gates.view(np.int16)).to(DEV)
+    admitted = None
+    for up_val in (1.0, -1.0, 0.9921875, 3.140625, 2.0 ** -20):
+        up = torch.full((n,), up_val, dtype=torch.bfloat16)
+        ub = bf16_bits(up)
+        ud = torch.from_numpy(ub.view(np.int16)).to(DEV)
+        h = torch.empty(n, dtype=torch.float32, device=DEV)
+        ok = torch.empty(n, dtype=torch.uint8, device=DEV)
+        rc = lab.aq_lab_probe_swiglu_bf16(ud.data_ptr(), gd.data_ptr(), n, h.data_ptr(), ok.data_ptr(),
+                                          torch.cuda.current_stream().cuda_stream)
+        assert rc == 0
+        torch.cuda.synchronize()
+        ug = np.stack([ub, gates], axis=1).reshape(n, 2)          # rows of one product each: [up | gate]
+        _, _, want = oracle.c_swiglu_quant_i8(ug, bf16_bits=True, want_h=True)
+        got = to_np(h).view(np.uint32)
+        okn = to_np(ok).astype(bool)
+        admitted = okn
+        gf = (gates.astype(np.uint32) << 16).view(np.float32)
+        # the range test admits zero and 2^-62 <= |g| <= 80, nothing else
+        assert np.array_equal(okn, (gf == 0) | ((np.abs(gf) >= 2.0 ** -62) & (np.abs(gf) <= 80.0)))
+        w = want.reshape(n).view(np.uint32)
+        zero = gf == 0                                           # 0 / d: the sign of a zero is free
+        bad = np.flatnonzero(okn & ~zero & (got != w))
+        assert bad.size == 0, [(hex(int(gates[i])), hex(int(got[i])), hex(int(w[i]))) for i in bad[:5]]
+        assert np.all((got[zero] & 0x7fffffff) == 0)
+    assert admitted.sum() > 17000                                # two signs x 68 binades x 128 mantissas, and the zeros
+
+
+def test_swiglu_quant_kernel_scales_reveal_every_bf16_gates_quotient(oracle):
+    """The same certification through the SHIPPED kernel: a row whose only non-zero product is 1 * silu(g) has
+    amax = |silu(g)|, so its scale amax / 127 carries the quotient's bits (the map is one-to-one except where the
+    quotient's mantissa is above 1.984; a second row with up = 127/128 covers those).  Every admitted gate, both
+    multipliers, 5632-wide rows through the wavefront-per-row kernel."""
+    gates = _all_bf16_gates()
+    gf = (gates.astype(np.uint32) << 16).view(np.float32)
+    gates = gates[(np.abs(gf) >= 2.0 ** -62) & (np.abs(gf) <= 80.0)]
+    F = 5632
+    for up_val in (1.0, 0.9921875):
+        M = gates.size
+        ug = np.zeros((M, 2 * F), np.uint16)
+        col = (np.arange(M) * 37) % F
+        ug[np.arange(M), col] = bf16_bits(torch.tensor([up_val], dtype=torch.bfloat16))[0]
+        ug[np.arange(M), F + col] = gates
+        for lo in range(0, M, 4096):                             # (the oracle's turn takes most of the time)
+            part = np.ascontiguousarray(ug[lo:lo + 4096])
+            d = torch.from_numpy(part.view(np.int16)).to(DEV).view(torch.bfloat16)
+            q, s = ops.swiglu_quant_rowwise_i8(d)
+            qo, so = oracle.c_swiglu_quant_i8(part, bf16_bits=True)
+            assert np.array_equal(to_np(s).view(np.uint32), so.view(np.uint32)), (up_val, lo)
+            assert np.array_equal(to_np(q), qo), (up_val, lo)
+
+
 def test_swiglu_quant_tracks_the_unfused_flow():
     """Against silu, product and row quantiser as three launches (mlp.py:25-26 in bf16): the fused
     kernel keeps the product in fp32, so codes may differ by one step."""

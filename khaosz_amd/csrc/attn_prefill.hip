@@ -127,8 +127,31 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
       vro = paged_row(vr < T ? vr : T - 1);
     }
   };
+  // Direct kernel: K and V of this sequence and KV head behind buffer descriptors; a staging chunk's byte offset is
+  // a lane constant (computed once) plus the block's row distance -- one add per load where a 64-bit row product
+  // stood -- and rows past the sequence fall outside the descriptor and read as zero (they are masked anyway).
+  __amdgpu_buffer_rsrc_t Kd = make_rsrc(nullptr, 0), Vd = make_rsrc(nullptr, 0);
+  uint32_t koff[4] = {0, 0, 0, 0}, voff[4] = {0, 0, 0, 0};
+  uint32_t kblk = 0, vblk = 0;  // bytes between consecutive key blocks
+  if constexpr (!PAGED) {
+    Kd = make_rsrc(p.k + tok0 * p.k_stride + (int64_t)kvh * D, (uint32_t)(((int64_t)(S - 1) * p.k_stride + D) * 2));
+    Vd = make_rsrc(p.v + tok0 * p.v_stride + (int64_t)kvh * D, (uint32_t)(((int64_t)(S - 1) * p.v_stride + D) * 2));
+    kblk = (uint32_t)(PA_KB * p.k_stride * 2);
+    vblk = (uint32_t)(PA_KB * p.v_stride * 2);
+#pragma unroll
+    for (int c = 0; c < CPT; ++c) {
+      const int idx = c * 256 + tid, key = idx / (D / 8), ch = idx % (D / 8);
+      koff[c] = (uint32_t)(key * (int)p.k_stride + ch * 8) * 2u;
+      voff[c] = (uint32_t)(lane * (int)p.v_stride + (wave + 4 * c) * 8) * 2u;
+    }
+  }
   auto fetch1 = [&](int j, int c, uint4& kr_out, uint4& vr_out) __attribute__((always_inline)) {
     const int idx = c * 256 + tid, key = idx / (D / 8), ch = idx % (D / 8);
+    if constexpr (!PAGED) {
+      kr_out = buffer_load_16(Kd, koff[c] + (uint32_t)j * kblk);
+      vr_out = buffer_load_16(Vd, voff[c] + (uint32_t)j * vblk);
+      return;
+    }
     int kr = j * PA_KB + key;
     kr = kr < T ? kr : T - 1;  // past the last position: any valid row, masked by causality
     int vr = j * PA_KB + lane;
@@ -234,13 +257,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
     // Scores stay unscaled; the scale (> 0) is applied to the maximum and inside the exponent's fma.
     const bool diag = kb0 + PA_KB - 1 > qw0p;  // wavefront-uniform: some key of the block is ahead of some query
     float bm = -INFINITY;
+    if (diag) {  // a branch, not 32 compares and selects in every block: most blocks lie wholly behind the queries
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          if (kb0 + kt * 32 + 8 * (r / 4) + 4 * g + (r % 4) > qposp) s[kt][r] = -INFINITY;
+    }
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        if (diag && kb0 + kt * 32 + 8 * (r / 4) + 4 * g + (r % 4) > qposp) s[kt][r] = -INFINITY;
-        bm = fmaxf(bm, s[kt][r]);
-      }
+      for (int r = 0; r < 16; ++r) bm = fmaxf(bm, s[kt][r]);
     bm = fmaxf(bm, __shfl_xor(bm, 32, 64)) * p.scale_log2e;
     // The running maximum only has to bound the exponents, not equal the true maximum: it is raised (and the
     // accumulators rescaled) only when some query of the wavefront would otherwise see an exponent above 2^8;
@@ -327,6 +354,9 @@ extern "C" int aq_prefill_attn_causal(const void* q, int64_t q_stride, const voi
       (k_stride & 7) || (v_stride & 7))
     return AQ_E_ALIGN;
   if (S > (1 << 30) || Hq > 65535 || B > 65535 || ((S + aq::PA_QB - 1) / aq::PA_QB) * Hq * B > (int64_t)0x7fffffff)
+    return AQ_E_RANGE;
+  // 32-bit byte offsets inside one sequence's K and V (a key block past the end included)
+  if ((S + aq::PA_KB) * k_stride * 2 > (int64_t)0x7fffffff || (S + aq::PA_KB) * v_stride * 2 > (int64_t)0x7fffffff)
     return AQ_E_RANGE;
   aq::PrefillAttnArgs a{};
   a.q = static_cast<const uint16_t*>(q);

@@ -238,20 +238,40 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
     const int kb0 = j * PA_KB;
     if (kb0 > qw0p + 31) continue;  // wavefront-uniform: every key of the block is ahead of every query here
     // ---- scores, transposed: two tiles of 32 keys
+    // The K fragments are read two dimension steps ahead of the products that take them, and the two tiles'
+    // accumulation chains alternate: left to itself the compiler put every LDS read right in front of its MFMA
+    // (one LDS round trip per product, sixteen in a row) and ran the second tile's chain after the first's.
+    // Each chain still adds its steps in ascending order: same bits.
     pa_f32x16 s[2];
+    {
 #pragma unroll
-    for (int kt = 0; kt < 2; ++kt) {
-      pa_f32x16 c;
+      for (int r = 0; r < 16; ++r) s[0][r] = s[1][r] = 0.0f;
+      const uint16_t* k0 = &ks[col * KP + g * 8];
+      const uint16_t* k1 = k0 + 32 * KP;
+      constexpr int GRP = 2, NG = DSTEPS / GRP;
+      static_assert(DSTEPS % GRP == 0, "whole groups of dimension steps");
+      uint4 fa[2][GRP][2];
+      auto ldk = [&](int buf, int st0) __attribute__((always_inline)) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) c[r] = 0.0f;
-      const uint16_t* krow = &ks[(kt * 32 + col) * KP + g * 8];
+        for (int i = 0; i < GRP; ++i) {
+          fa[buf][i][0] = *reinterpret_cast<const uint4*>(k0 + (st0 + i) * 16);
+          fa[buf][i][1] = *reinterpret_cast<const uint4*>(k1 + (st0 + i) * 16);
+        }
+      };
+      ldk(0, 0);
+      if (NG > 1) ldk(1, GRP);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int st = 0; st < DSTEPS; ++st) {
-        const uint4 a = *reinterpret_cast<const uint4*>(krow + st * 16);
-        c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(pa_bf16x8, a), __builtin_bit_cast(pa_bf16x8, qf[st]),
-                                                   c, 0, 0, 0);
+      for (int gi = 0; gi < NG; ++gi) {
+#pragma unroll
+        for (int i = 0; i < GRP; ++i) {
+          const pa_bf16x8 qv = __builtin_bit_cast(pa_bf16x8, qf[gi * GRP + i]);
+          s[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(pa_bf16x8, fa[gi & 1][i][0]), qv, s[0], 0, 0, 0);
+          s[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(pa_bf16x8, fa[gi & 1][i][1]), qv, s[1], 0, 0, 0);
+        }
+        if (gi + 2 < NG) ldk(gi & 1, (gi + 2) * GRP);
+        __builtin_amdgcn_sched_barrier(0);
       }
-      s[kt] = c;
     }
     // ---- online softmax for this lane's query; register r of tile kt is key kb0 + 32 kt + 8 (r / 4) + 4 g + r % 4.
     // Scores stay unscaled; the scale (> 0) is applied to the maximum and inside the exponent's fma.
@@ -298,26 +318,38 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
     }
     l += ps;
     // ---- output, transposed: O^T[d, q] = alpha O^T + V^T P^T
+    if (raise) {  // one branch for all tiles (a branch per tile kept the tiles' products apart)
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      pa_f32x16 c = o[dt];
-      if (raise) {
+      for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) c[r] *= alpha;
-      }
-      const uint16_t* vrow = &vt[(dt * 32 + col) * VP + 4 * g];
+        for (int r = 0; r < 16; ++r) o[dt][r] *= alpha;
+    }
+    // V^T fragments of two dimension tiles at a time, all read before the pair's products, whose two chains
+    // alternate; each chain adds its four key groups in ascending order: same bits.
+    {
+      uint4 fv[DT][4];
+      auto ldv = [&](int dt) __attribute__((always_inline)) {
+        const uint16_t* vrow = &vt[(dt * 32 + col) * VP + 4 * g];
 #pragma unroll
-      for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2) {
-          // k slots of this lane group: keys 32 kt + 16 s2 + {4 g .. + 4, 8 + 4 g .. + 4}
-          const uint2 lo = *reinterpret_cast<const uint2*>(vrow + kt * 32 + s2 * 16);
-          const uint2 hi = *reinterpret_cast<const uint2*>(vrow + kt * 32 + s2 * 16 + 8);
-          const uint4 a = make_uint4(lo.x, lo.y, hi.x, hi.y);
-          c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(pa_bf16x8, a),
-                                                     __builtin_bit_cast(pa_bf16x8, pf[kt][s2]), c, 0, 0, 0);
+        for (int kk = 0; kk < 4; ++kk) {
+          // k slots of this lane group: keys 32 kt + 16 s2 + {4 g .. + 4, 8 + 4 g .. + 4}, kk = 2 kt + s2
+          const uint2 lo = *reinterpret_cast<const uint2*>(vrow + kk * 16);
+          const uint2 hi = *reinterpret_cast<const uint2*>(vrow + kk * 16 + 8);
+          fv[dt][kk] = make_uint4(lo.x, lo.y, hi.x, hi.y);
         }
-      o[dt] = c;
+      };
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) ldv(dt);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int d0 = 0; d0 < DT; d0 += 2) {
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) {
+          const pa_bf16x8 pv8 = __builtin_bit_cast(pa_bf16x8, pf[kk >> 1][kk & 1]);
+          o[d0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(pa_bf16x8, fv[d0][kk]), pv8, o[d0], 0, 0, 0);
+          o[d0 + 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(pa_bf16x8, fv[d0 + 1][kk]), pv8, o[d0 + 1], 0, 0, 0);
+        }
+      }
     }
   }
   // ---- normalise and store: register r of tile dt is dimension 32 dt + 8 (r / 4) + 4 g + r % 4 of query col

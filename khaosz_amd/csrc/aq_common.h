@@ -88,8 +88,27 @@ __device__ __forceinline__ uint32_t quant_code_exact(float a, float s) {
 // numbers with |value| <= maximum and s = fl(maximum / 127) in range -- 2.8e8
 // pairs, evaluated one by one on the CPU with the same IEEE operations
 // (oq_one_step_divide_mismatches in the oracle and the test that runs it).
+// With STEPS = 0, for the int8 codes of such rows: no correction at all, q0 = a * rs rounds to the same integer
+// as fl(a / s) for every value of the row, PROVIDED rs is fl(1 / s) moved by at most one unit in the last place
+// in a direction that depends on the 7 mantissa bits of the row maximum alone (reciprocal_for_bf16_rows below:
+// 104 of the 128 mantissas keep fl(1 / s), 18 take the next float up, 6 the next one down; which is which was found
+// by trying all three for every maximum, and the choice does not depend on the exponent).  The claim is evaluated
+// for every pair like the one above (oq_one_step_divide_mismatches with steps = -1, on the oracle's own copy of the
+// table) and on the shipped kernels over every value of rows with every mantissa.
 // `lean_ok` must be false for rows whose scale is outside [2^-64, 2^64], where
 // the residuals could leave the normal range; those rows take the full divide.
+//
+// Two bits per mantissa of the row maximum (mantissa m in bits 2 (m % 16) of word m / 16): 0 keep fl(1 / s), 1 one
+// unit up, 2 one unit down.
+__device__ __forceinline__ float reciprocal_for_bf16_rows(float amax, float s) {
+  const uint32_t m = (__float_as_uint(amax) >> 16) & 127u;
+  const uint32_t i = m >> 4;
+  const uint32_t w = (i & 4u) ? ((i & 2u) ? ((i & 1u) ? 0x00000105u : 0x40000004u) : ((i & 1u) ? 0x40014442u : 0x00000000u))
+                              : ((i & 2u) ? ((i & 1u) ? 0x10004480u : 0x80000000u) : ((i & 1u) ? 0x05015a02u : 0x00000000u));
+  const uint32_t adj = (w >> (2u * (m & 15u))) & 3u;
+  return __uint_as_float(__float_as_uint(__fdiv_rn(1.0f, s)) + (adj & 1u) - (adj >> 1));
+}
+
 template <int N, int STEPS = 2>
 __device__ __forceinline__ void quant_codes(const float* a, float s, float rs, bool lean_ok, uint32_t* out) {
   const float magic = 12582912.0f;  // 1.5 * 2^23
@@ -97,7 +116,7 @@ __device__ __forceinline__ void quant_codes(const float* a, float s, float rs, b
 #pragma unroll
     for (int i = 0; i < N; ++i) {
       float q = a[i] * rs;
-      q = __builtin_fmaf(__builtin_fmaf(-s, q, a[i]), rs, q);
+      if constexpr (STEPS >= 1) q = __builtin_fmaf(__builtin_fmaf(-s, q, a[i]), rs, q);
       if constexpr (STEPS == 2) q = __builtin_fmaf(__builtin_fmaf(-s, q, a[i]), rs, q);
       out[i] = __float_as_uint(q + magic);
     }
@@ -238,7 +257,7 @@ __device__ __forceinline__ void quant_codes_packed(const float* a, float s, floa
 #pragma unroll
     for (int i = 0; i < N; ++i) {
       q[i] = a[i] * rs;
-      q[i] = __builtin_fmaf(__builtin_fmaf(-s, q[i], a[i]), rs, q[i]);
+      if constexpr (STEPS >= 1) q[i] = __builtin_fmaf(__builtin_fmaf(-s, q[i], a[i]), rs, q[i]);
       if constexpr (STEPS == 2) q[i] = __builtin_fmaf(__builtin_fmaf(-s, q[i], a[i]), rs, q[i]);
     }
     if constexpr (N == 8) {

@@ -43,8 +43,9 @@ __device__ __forceinline__ float vec_amax(const float* f) {
 // Symmetric absmax scale of one row from its wavefront-wide maximum:
 // s = amax / 127 (1 for an all-zero row), rs = the reciprocal of s in the form
 // quant_codes<N, STEPS> expects (STEPS = 2: the once-refined hardware reciprocal;
-// STEPS = 1, rows of bf16 numbers: the correctly rounded one, a full divide once
-// per row), and whether s is in the range where the short sequence may be used.
+// STEPS = 1: the correctly rounded one, a full divide once per row; STEPS = 0,
+// rows of bf16 numbers: that one moved as the row maximum's mantissa asks), and
+// whether s is in the range where the short sequence may be used.
 struct RowScale {
   float s, rs;
   bool fast_ok;
@@ -54,7 +55,9 @@ __device__ __forceinline__ RowScale row_scale(float amax) {
   RowScale r;
   r.s = __fdiv_rn(amax, 127.0f);
   if (amax == 0.0f) r.s = 1.0f;
-  if constexpr (STEPS == 1) {
+  if constexpr (STEPS == 0) {
+    r.rs = reciprocal_for_bf16_rows(amax, r.s);
+  } else if constexpr (STEPS == 1) {
     r.rs = __fdiv_rn(1.0f, r.s);
   } else {
     const float y0 = __builtin_amdgcn_rcpf(r.s);
@@ -63,9 +66,9 @@ __device__ __forceinline__ RowScale row_scale(float amax) {
   r.fast_ok = r.s >= 5.421010862427522e-20f && r.s <= 1.8446744073709552e19f;  // [2^-64, 2^64]
   return r;
 }
-// correction steps for rows that are read as they are (bf16 numbers: one) or computed in fp32 (two)
+// correction steps for rows that are read as they are (bf16 numbers: none) or computed in fp32 (two)
 template <bool BF16, bool COMPUTED>
-constexpr int quant_steps() { return BF16 && !COMPUTED ? 1 : 2; }
+constexpr int quant_steps() { return BF16 && !COMPUTED ? 0 : 2; }
 
 // Sum across the wavefront in a fixed order: p[l] += p[l ^ 1], ^2, ^4, ^8, ^16, ^32, every add
 // rounded.  After the xor-1 and xor-2 steps a quad holds one value, after the half-row mirror a

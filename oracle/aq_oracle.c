@@ -645,7 +645,13 @@ void oq_quant_tensor_fp8_bf16(const uint16_t *x, int64_t numel, uint8_t *q, floa
  * whose codes differ (*pairs = the number evaluated).  divisor 127: code = clamp(rint(.), +-127); divisor 448:
  * code = e4m3fn(clamp(., +-448)) with the quotient given the sign of a (the kernel does that too: a zero residual
  * turns a quotient of -0 into +0).  steps = 0 evaluates q0 alone, which does differ: the check has teeth.
+ * steps = -1 (divisor 127) evaluates the int8 kernels' present form for bf16 rows: q0 alone, but with rs moved by
+ * one unit in the last place where the 7 mantissa bits of the maximum ask for it (the table below: 0 keep, 1 up,
+ * 2 down; two bits per mantissa, sixteen mantissas per word).
  */
+static const uint32_t oq_rs_adjust[8] = {0x00000000u, 0x05015a02u, 0x80000000u, 0x10004480u,
+                                         0x00000000u, 0x40014442u, 0x40000004u, 0x00000105u};
+
 int64_t oq_one_step_divide_mismatches(float divisor, int steps, uint32_t am_lo, uint32_t am_hi, int64_t *pairs) {
   int64_t bad = 0, n = 0;
   const int fp8 = divisor == 448.0f;
@@ -655,13 +661,20 @@ int64_t oq_one_step_divide_mismatches(float divisor, int steps, uint32_t am_lo, 
     const float amax = oq_bf16_to_f32((uint16_t)am);
     const float s = amax / divisor;
     if (!(s >= 5.421010862427522e-20f && s <= 1.8446744073709552e19f)) continue;
-    const float rs = 1.0f / s;
+    float rs = 1.0f / s;
+    if (steps < 0) {
+      const uint32_t m = am & 127u, adj = (oq_rs_adjust[m >> 4] >> (2u * (m & 15u))) & 3u;
+      uint32_t bits;
+      memcpy(&bits, &rs, 4);
+      bits += (adj & 1u) - (adj >> 1);
+      memcpy(&rs, &bits, 4);
+    }
     for (uint32_t ab = 0; ab <= am; ++ab) {
       for (int neg = 0; neg < 2; ++neg) {
         const float a = oq_bf16_to_f32((uint16_t)(ab | (neg ? 0x8000u : 0u)));
         const float q = a / s;
         const float q0 = a * rs;
-        float q1 = steps ? fmaf(fmaf(-s, q0, a), rs, q0) : q0;
+        float q1 = steps > 0 ? fmaf(fmaf(-s, q0, a), rs, q0) : q0;
         ++n;
         if (fp8) {
           q1 = copysignf(q1, a);

@@ -123,6 +123,60 @@ def test_quant_rowwise_scale_range_and_dense_ties(oracle, dtype):
             assert np.array_equal(to_np(y), want), f"rows {r0}.."
 
 
+def _rows_of_every_value_up_to(amax_bits: int, K: int) -> np.ndarray:
+    """bf16 bit patterns: rows of K values that begin with the maximum and together hold every bf16 number of
+    magnitude up to it, both signs (the last row is filled up with zeros)."""
+    mags = np.arange(amax_bits + 1, dtype=np.uint16)
+    vals = np.concatenate([mags, mags | np.uint16(0x8000)])
+    per = K - 1
+    n_rows = (vals.size + per - 1) // per
+    rows = np.zeros((n_rows, K), np.uint16)
+    rows[:, 0] = amax_bits
+    flat = np.zeros(n_rows * per, np.uint16)
+    flat[:vals.size] = vals
+    rows[:, 1:] = flat.reshape(n_rows, per)
+    return rows
+
+
+def test_bf16_rows_one_product_rounding_for_every_mantissa_of_the_maximum(oracle):
+    """Rows of bf16 numbers are rounded with one product, value times a reciprocal of the scale that is moved
+    by one unit in the last place for 24 of the 128 mantissas a row maximum can have.  Here: every mantissa, at
+    three exponents (the choice must not depend on it), rows that hold EVERY bf16 value up to the maximum --
+    through the row quantiser (rows of 8192 and of 2048 values: two kernels) against the oracle's divide."""
+    for K in (8192, 2048):
+        blocks = []
+        for exp_field in ([127, 90, 170] if K == 8192 else [127]):
+            for m in range(128):
+                blocks.append(_rows_of_every_value_up_to((exp_field << 7) | m, K))
+        bits = np.concatenate(blocks)
+        _say("every value of bf16 rows", K, bits.shape)
+        xd = torch.from_numpy(bits.view(np.int16)).to(DEV).view(torch.bfloat16)
+        q, s_ = ops.quant_rowwise_i8(xd)
+        qo, so = oracle.c_quant_rowwise_i8(bits, bf16_bits=True)
+        assert np.array_equal(to_np(s_).view(np.uint32), so.view(np.uint32))
+        bad = np.argwhere(to_np(q) != qo)
+        assert bad.size == 0, f"K={K}: first mismatches (row, col): {bad[:5].tolist()}"
+        del xd, q
+
+
+def test_bf16_rows_one_product_rounding_inside_the_decode_kernels(oracle):
+    """The same rows (every mantissa of the maximum, every value up to it) through the kernels that quantise
+    their rows themselves: 16 rows a call through the matrix-core GEMV, 8 and 3 through the dot-product one.
+    The weight is the identity, so the output is the codes times the row's scale, exactly."""
+    K = 2048
+    wq = torch.eye(K, dtype=torch.int8, device=DEV)
+    sw = torch.ones(K, device=DEV)
+    for m in range(128):
+        bits = _rows_of_every_value_up_to((127 << 7) | m, K)
+        qo, so = oracle.c_quant_rowwise_i8(bits, bf16_bits=True)
+        want = qo.astype(np.float32) * so[:, None]
+        xd = torch.from_numpy(bits.view(np.int16)).to(DEV).view(torch.bfloat16)
+        for rows in (16, 8, 3):
+            for r0 in range(0, xd.shape[0], rows):
+                y = ops.gemv_w8a8_decode(xd[r0:r0 + rows].contiguous(), wq, sw, None, out_dtype=torch.float32)
+                assert np.array_equal(to_np(y), want[r0:r0 + rows]), f"mantissa {m}, rows {r0}.. ({rows} a call)"
+
+
 @pytest.mark.parametrize("M,K", [(1, 16), (7, 48), (5, 1040), (64, 2048), (8, 5632), (130, 4096), (3, 12288)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_rmsnorm_quant_bit_exact(oracle, M, K, dtype):

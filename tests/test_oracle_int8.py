@@ -206,3 +206,20 @@ def test_one_correction_divide_gives_the_code_of_the_divide_for_every_pair_of_bf
     assert pairs > 5.5e8 and bad == 0
     bad0, _ = oracle.c_one_step_divide_mismatches(divisor, am_lo=0x3F80, am_hi=0x4000, steps=0)
     assert bad0 > 0
+
+
+def test_adjusted_reciprocal_product_gives_the_code_of_the_divide_for_every_pair_of_bf16_numbers(oracle):
+    """The int8 quantisers round rows of bf16 numbers with ONE product, value times a reciprocal of the scale
+    that is moved by one unit in the last place where the row maximum's mantissa asks for it.  Every pair
+    (row maximum, value), 5.6e8 of them: no code differs from the divide's.  The same product with the plain
+    reciprocal does differ (steps=0 above), and so does a table that moves nothing or moves the wrong way --
+    one binade of maxima under the plain reciprocal shows mismatches exactly where the table holds a move."""
+    bad, pairs = oracle.c_one_step_divide_mismatches(127.0, steps=-1)
+    assert pairs > 5.5e8 and bad == 0
+    # per mantissa: the plain reciprocal fails for the 24 mantissas whose entry is not 0, and only there
+    table = [0x00000000, 0x05015A02, 0x80000000, 0x10004480, 0x00000000, 0x40014442, 0x40000004, 0x00000105]
+    moved = {m for m in range(128) if (table[m >> 4] >> (2 * (m & 15))) & 3}
+    assert len(moved) == 24
+    failing = {m for m in range(128)
+               if oracle.c_one_step_divide_mismatches(127.0, am_lo=0x3F80 + m, am_hi=0x3F80 + m + 1, steps=0)[0]}
+    assert failing == moved

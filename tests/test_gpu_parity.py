@@ -218,7 +218,10 @@ def test_rmsnorm_quant_tracks_torch_rms_norm_then_quantise():
 
 
 @pytest.mark.parametrize("M,F", [(1, 16), (7, 48), (5, 1040), (64, 2048), (8, 5632), (130, 704), (1100, 1040), (4, 6912),
-                                 (1030, 6912), (3, 8192)])
+                                 (1030, 6912), (3, 8192),
+                                 # many long rows (the workgroup-per-row kernel at prefill sizes; ragged row ends,
+                                 # odd row counts)
+                                 (1031, 8192), (1101, 6160), (4099, 6912), (1029, 3600), (1500, 3344)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_swiglu_quant_bit_exact(oracle, M, F, dtype):
     if dtype == torch.float32 and F > 4096:
@@ -242,7 +245,7 @@ def test_swiglu_quant_bit_exact(oracle, M, F, dtype):
     assert bad.size == 0, f"first mismatches (row, col): {bad[:5].tolist()}"
 
 
-@pytest.mark.parametrize("M,F", [(40, 5632), (40, 1040), (1100, 704)])
+@pytest.mark.parametrize("M,F", [(40, 5632), (40, 1040), (1100, 704), (1100, 6912), (1100, 3600)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_swiglu_quant_divide_range_edges(oracle, M, F, dtype):
     """The kernels take a short divide for rows whose gates are zero or in 2^-62 .. 80 and the general one for the

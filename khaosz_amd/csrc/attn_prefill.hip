@@ -45,6 +45,7 @@ struct PrefillAttnArgs {
   const int64_t* table;  // [B, P] physical page ids, < 0: unmapped (zero keys and values)
   int64_t P, page, n_pages;
   int start, page_shift;
+  int paired;  // != 0: the second half of the workgroups takes the query blocks lightest first
 };
 
 typedef __bf16 pa_bf16x8 __attribute__((ext_vector_type(8)));
@@ -75,8 +76,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
   // first, then the block before it, ... -- the long workgroups start at once and the short ones fill in
   // behind them (in launch order the light blocks of head 0 would start first and the heavy ones of the last
   // heads would run alone at the end: 34 -> 28 us at 8 x 512, 339 -> 219 us at 4 x 2048 x 32 heads).
+  // When the whole launch is resident at once (two workgroups per compute unit), the second half of the
+  // numbering runs lightest first instead: the workgroup that joins a heavy one on its compute unit is then a
+  // light one, and every compute unit gets the same sum (8 x 512 x 16 heads: 22.4 -> 21.6 us; with more
+  // workgroups than slots the descending order is the better one, 4 x 2048 x 32 heads 186 against 194 us).
   const int nqb = (S + PA_QB - 1) / PA_QB, per = p.Hq * p.B;
-  const int q0 = (nqb - 1 - (int)blockIdx.x / per) * PA_QB, h = ((int)blockIdx.x % per) % p.Hq,
+  const int rank = (int)blockIdx.x / per, hrank = (nqb + 1) / 2;
+  const int qblk = (p.paired && rank >= hrank) ? rank - hrank : nqb - 1 - rank;
+  const int q0 = qblk * PA_QB, h = ((int)blockIdx.x % per) % p.Hq,
             b = ((int)blockIdx.x % per) / p.Hq;
   const int kvh = h / (p.Hq / p.Hkv);
   const int qw0 = q0 + wave * 32;          // first query row of this wavefront
@@ -404,6 +411,7 @@ extern "C" int aq_prefill_attn_causal(const void* q, int64_t q_stride, const voi
   a.Hkv = (int)Hkv;
   a.B = (int)B;
   const dim3 grid((unsigned)(((S + aq::PA_QB - 1) / aq::PA_QB) * Hq * B));
+  a.paired = grid.x <= 2u * (unsigned)aq::device_cus();
   hipStream_t st = static_cast<hipStream_t>(stream);
   const size_t lds = (size_t)(aq::PA_KB * (D + 8) + D * (aq::PA_KB + 4)) * sizeof(uint16_t);  // 34 KiB at most
   if (D == 128)
@@ -450,6 +458,7 @@ extern "C" int aq_prefill_attn_paged(const void* q, int64_t q_stride, const void
   a.Hkv = (int)Hkv;
   a.B = (int)B;
   const dim3 grid((unsigned)(((S + aq::PA_QB - 1) / aq::PA_QB) * Hq * B));
+  a.paired = grid.x <= 2u * (unsigned)aq::device_cus();
   hipStream_t st = static_cast<hipStream_t>(stream);
   const size_t lds = (size_t)(aq::PA_KB * (D + 8) + D * (aq::PA_KB + 4)) * sizeof(uint16_t);
   if (D == 128)

@@ -4,9 +4,9 @@ path can be measured end to end the way the reference measures itself
 token embedding, ``n_layers`` pre-norm blocks sharing one rotary table and one
 paged KV cache, a final RMSNorm and the vocabulary projection.
 
-Only what the benchmark's default configuration uses is here (grouped-query
-attention, SwiGLU MLP, no qk-norm, no gated attention, no MoE / MLA, optional
-tied embedding).  The attention mask follows ``process_attention_mask``
+Only what the benchmark's configurations use is here (grouped-query attention
+with its qk-norm and output-gate options, SwiGLU MLP, optional tied embedding;
+no MoE / MLA).  The attention mask follows ``process_attention_mask``
 (transformer.py:17-46) for the two cases the benchmark runs -- a prompt from
 position 0 (causal, no mask tensor) and one new token per sequence (a mask of
 zeros) -- without its device-to-host reads, so a step can be captured in a HIP

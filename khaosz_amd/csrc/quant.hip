@@ -256,20 +256,21 @@ __global__ __launch_bounds__(256) void rmsnorm_quant_kernel(const void* __restri
 // its NC vector pairs into h (fp32, kept in registers; the inputs die as it goes),
 // then reduces the absmax and rounds.
 //
-// The kernel is bound by its vector arithmetic (about 34 operations per element: the exponential's polynomial, a
-// correctly rounded divide, the two-correction rounding; 4096 x 5632 is 20 us of it at 2.4 GHz), so the work went
-// into keeping the vector ALUs fed and into the operation count:
+// The kernel is bound by its vector arithmetic (about 34 operations per element at first: the exponential's
+// polynomial, a correctly rounded divide, the two-correction rounding; 4096 x 5632 was 20 us of it at 2.4 GHz),
+// so the work went into keeping the vector ALUs fed and into the operation count:
 //  * every load of a row is requested up front, pair by pair (up vector, gate vector), and the arithmetic walks
 //    the pairs in that order, waiting for one pair at a time (loads return in request order).  A row's first pair
 //    arrives within a microsecond and the rest streams in behind the arithmetic.  (Left to itself the compiler
 //    waited for the whole row before the first operation; with only a few pairs requested ahead, a wavefront's
 //    time was the memory latency times its pairs.)
-//  * the divide is div_midrange (11 instead of 14 operation slots) whenever the row's gates allow it, which is
-//    tested on the raw bf16 pairs with packed 16-bit operations; a row with a gate outside is done again with
-//    the general divide, out of line.
+//  * the divide is div_midrange (11 instead of 14 operation slots; 9 for bf16 gates, div_bf16_gate) whenever the
+//    row's gates allow it, which is tested on the raw bf16 pairs with packed 16-bit operations; a row with a gate
+//    outside is done again with the general divide, out of line; the exponential goes without its argument clamp
+//    for such rows, and the rounding add packs its own byte (quant_codes_packed).
 //  * NC is the row's own number of vector pairs per lane (a pair past the row would cost its full arithmetic).
 // Four wavefronts fit a SIMD (128 registers: a row's h is 88 of them at F = 5632); the SIMD serves the oldest
-// first, so a compute unit's 16 rows finish one after the other, 4096 x 5632 bf16 in 28 us (before: 31.5).
+// first, so a compute unit's 16 rows finish one after the other, 4096 x 5632 bf16 in 26.2 us (at first: 31.5).
 template <bool BF16, int NC>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void swiglu_quant_kernel(
     const void* __restrict__ ug, int64_t M, int F, int64_t ld, int8_t* __restrict__ q, float* __restrict__ scale) {

@@ -155,7 +155,10 @@ struct EpiOperands {
 // MERGE > 0 (with FUSED): the rows are a decode step's attention output, combined here from the attention
 // kernel's partial results of up to MERGE slices (p.parts) -- the separate merge launch disappears.
 // FW: wavefronts per workgroup of a FUSED kernel (8, or 4 for short matrices).
-template <int MT, bool FUSED, int VPL, bool NORM = false, int MERGE = 0, int FW = GV_WAVES>
+// FK: K parts of a FUSED kernel (1; 4 for a short matrix with long rows, an MLP's down projection: every wavefront
+// still rounds a row, then FK wavefronts share a group of weight rows, so that the launch has a workgroup for
+// every compute unit where whole rows per wavefront would leave most of them without loads in flight).
+template <int MT, bool FUSED, int VPL, bool NORM = false, int MERGE = 0, int FW = GV_WAVES, int FK = 1>
 __global__ __launch_bounds__(GV_THREADS) void gemv_w8a8_kernel(GemvArgs p) {
   extern __shared__ __attribute__((aligned(16))) uint8_t xs[];  // [MT][K] activation codes, then [MT] scales
   const int tid = threadIdx.x, lane = tid & 63;
@@ -167,7 +170,7 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_w8a8_kernel(GemvArgs p) {
   // K parts: ksplit wavefronts share a group of GV_ROWS rows, wavefront kpart taking chunks kpart,
   // kpart + ksplit, ...; their sums meet in LDS (exact int32).  For short N and long K, where whole rows per
   // wavefront would leave most of the device without loads in flight.
-  const int ksplit = FUSED ? 1 : p.ksplit;
+  const int ksplit = FUSED ? FK : p.ksplit;
   const int kpart = wave % ksplit;
   const int n0 = __builtin_amdgcn_readfirstlane((blockIdx.x * (nwaves / ksplit) + wave / ksplit) * GV_ROWS);
 
@@ -367,20 +370,23 @@ static GemvShape gemv_shape(int N, int K, bool fused, int mt) {
   return sh;
 }
 
-template <int MT, bool FUSED, int VPL, bool NORM, int MERGE, int FW>
+template <int MT, bool FUSED, int VPL, bool NORM, int MERGE, int FW, int FK = 1>
 static int launch_gemv_fw(GemvArgs a, hipStream_t st) {
   GemvShape sh = gemv_shape(a.N, a.K, FUSED, MT);
-  if (FUSED) sh.waves = FW;
+  if (FUSED) {
+    sh.waves = FW;
+    sh.ksplit = FK;
+  }
   a.ksplit = sh.ksplit;
   const int rows_per_wg = GV_ROWS * (sh.waves / sh.ksplit);
   const unsigned grid = (unsigned)((a.N + rows_per_wg - 1) / rows_per_wg);
   const size_t lds = (size_t)MT * a.K + MT * sizeof(float) + (sh.ksplit > 1 ? (size_t)sh.waves * 64 * sizeof(int) : 0);
   if (lds > 64 * 1024) {  // beyond the default dynamic-LDS limit: opt this kernel in, once per device
     static LdsOptIn opted;
-    const int e = opted.ensure(reinterpret_cast<const void*>(&gemv_w8a8_kernel<MT, FUSED, VPL, NORM, MERGE, FW>));
+    const int e = opted.ensure(reinterpret_cast<const void*>(&gemv_w8a8_kernel<MT, FUSED, VPL, NORM, MERGE, FW, FK>));
     if (e) return e;
   }
-  hipLaunchKernelGGL((gemv_w8a8_kernel<MT, FUSED, VPL, NORM, MERGE, FW>), dim3(grid), dim3(sh.waves * 64), lds, st, a);
+  hipLaunchKernelGGL((gemv_w8a8_kernel<MT, FUSED, VPL, NORM, MERGE, FW, FK>), dim3(grid), dim3(sh.waves * 64), lds, st, a);
   return (int)hipGetLastError();
 }
 
@@ -1234,11 +1240,21 @@ static int gemv_dispatch_fused(const aq::GemvArgs& a, int mt, hipStream_t st) {
   if (aq::gemv_mfma_fq_ok(a.M, a.N, a.K, a.gamma != nullptr)) return aq::launch_gemv_mfma_fq(a, st);
   const int64_t vpl = (a.K / 8 + 63) / 64;  // 16-byte vectors per lane per bf16 row
   if (mt > 8 || vpl > 16) return -1;
-  // A short matrix with long rows (an MLP's down projection): the fused kernel cannot cut rows into K parts, so
-  // its N / 32 workgroups leave most compute units without loads in flight, and the separate row quantiser + the
-  // K-split GEMV on codes is faster (N = 2048, K = 5632, 8 rows: 11.0 against 9.1 us; K = 8192: 13.3 against 10.5;
-  // from N = 4096 on the one launch wins again).
-  if ((a.N + 31) / 32 * 4 <= aq::device_cus() && (a.K > 4096 || (a.M > 4 && a.K >= 4096))) return -1;
+  // A short matrix with long rows (an MLP's down projection): with whole rows per wavefront its N / 32 workgroups
+  // would leave most compute units without loads in flight (N = 2048, K = 5632, 8 rows: 11.0 us against 9.1 for
+  // the separate row quantiser + the K-split GEMV on codes).  The fused kernel with 4 K parts -- 8 weight rows per
+  // workgroup, every wavefront rounding one token row first -- is the fastest form: 8.6 -> 7.15 us for that shape,
+  // 8.0 -> 5.7 us for 4 rows of 6912 against 1536 weight rows, 7.0 -> 4.8 us for one row of 5632 (2 parts: 8.0,
+  // 8 parts: 12.1 us).  With the norm in front (rows stay short there) the two launches remain.
+  if ((a.N + 31) / 32 * 4 <= aq::device_cus() && (a.K > 4096 || (a.M > 4 && a.K >= 4096))) {
+    if (a.gamma) return -1;
+    switch (mt) {
+      case 1: return aq::launch_gemv_fw<1, true, 16, false, 0, aq::GV_WAVES, 4>(a, st);
+      case 2: return aq::launch_gemv_fw<2, true, 16, false, 0, aq::GV_WAVES, 4>(a, st);
+      case 4: return aq::launch_gemv_fw<4, true, 16, false, 0, aq::GV_WAVES, 4>(a, st);
+      default: return aq::launch_gemv_fw<8, true, 16, false, 0, aq::GV_WAVES, 4>(a, st);
+    }
+  }
   const bool small = vpl <= 4;
   if (a.gamma) {  // with the norm in front: short rows only (the gain's vectors stay in registers too)
     if (!small) return -1;
